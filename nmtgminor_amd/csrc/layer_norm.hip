@@ -1,0 +1,539 @@
+// LayerNorm forward / backward for gfx950.
+//
+// Stands in for fast_layer_norm_cuda.ln_fwd / ln_bwd of the reference
+// (onmt/modules/extensions/layer_norm/ln_api.cpp:80-249, kernels ln_fwd_kernels.cuh:7-108 and
+// ln_bwd_kernels.cuh:5-323). The design is not the reference's: there the hidden size is a
+// template constant and rows are spread over 32-lane warps with a per-size launcher registry;
+// here a row lives in the registers of WPR 64-lane wavefronts (VPL 16-byte vectors per lane),
+// any hidden size is accepted, statistics are two-pass in registers, and the gamma/beta
+// gradient is accumulated per lane over a block's rows and written as one partial row per block
+// which a second small kernel sums in a fixed order (deterministic).
+//
+// HBM traffic per row of H elements (the kernels are bandwidth bound):
+//   forward : read x, write z, +8 B (mu, rsigma)          -> 2 H elements
+//   backward: read dz, x, write dx, +8 B                  -> 3 H elements (+ the [n_part, H]
+//             fp32 partials once written and once read)
+#include "common.cuh"
+#include <algorithm>
+
+namespace nmtg {
+namespace {
+
+constexpr int LN_THREADS = 256;
+constexpr int LN_WAVES = LN_THREADS / kWave;
+
+template <typename T> struct ln_vec { static constexpr int EPV = 16 / sizeof(T); };
+
+// Sum over the WPR wavefronts that share a row. WPR == 1: wavefront butterfly only.
+template <int WPR>
+__device__ __forceinline__ float row_sum(float v, float* smem, int wave) {
+  v = wave_sum(v);
+  if constexpr (WPR > 1) {
+    __syncthreads();  // smem reuse guard
+    if ((threadIdx.x & (kWave - 1)) == 0) smem[wave] = v;
+    __syncthreads();
+    const int base = (wave / WPR) * WPR;
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < WPR; ++i) t += smem[base + i];
+    v = t;
+  }
+  return v;
+}
+
+template <int WPR>
+__device__ __forceinline__ void row_sum2(float& a, float& b, float* smem, int wave) {
+  wave_sum2(a, b);
+  if constexpr (WPR > 1) {
+    __syncthreads();
+    if ((threadIdx.x & (kWave - 1)) == 0) { smem[wave] = a; smem[LN_WAVES + wave] = b; }
+    __syncthreads();
+    const int base = (wave / WPR) * WPR;
+    float ta = 0.f, tb = 0.f;
+#pragma unroll
+    for (int i = 0; i < WPR; ++i) { ta += smem[base + i]; tb += smem[LN_WAVES + base + i]; }
+    a = ta; b = tb;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Forward: one row per WPR wavefronts, row held in registers.
+// ---------------------------------------------------------------------------------------------
+template <typename TI, typename TW, int VPL, int WPR>
+__global__ __launch_bounds__(LN_THREADS) void ln_fwd_kernel(
+    const TI* __restrict__ x, const TW* __restrict__ gamma, const TW* __restrict__ beta,
+    TW* __restrict__ z, float* __restrict__ mu, float* __restrict__ rsigma, int64_t rows, int hidden,
+    float eps) {
+  constexpr int EPV = ln_vec<TI>::EPV;
+  constexpr int RPB = LN_WAVES / WPR;  // rows per block per iteration
+  __shared__ float smem[2 * LN_WAVES];
+
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int sub = wave % WPR;  // which slice of the row this wavefront holds
+  const float rn = 1.f / static_cast<float>(hidden);
+  const int64_t groups = (rows + RPB - 1) / RPB;
+
+  for (int64_t g = blockIdx.x; g < groups; g += gridDim.x) {
+    const int64_t row = g * RPB + wave / WPR;
+    const bool row_ok = row < rows;
+    float xf[VPL][EPV];
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      const int col = ((sub * VPL + i) * kWave + lane) * EPV;
+      if (row_ok && col < hidden) {
+        load_pack<TI, EPV>(x + row * hidden + col, xf[i]);
+#pragma unroll
+        for (int j = 0; j < EPV; ++j) s += xf[i][j];
+      } else {
+#pragma unroll
+        for (int j = 0; j < EPV; ++j) xf[i][j] = 0.f;
+      }
+    }
+    const float mean = row_sum<WPR>(s, smem, wave) * rn;
+    float m2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      const int col = ((sub * VPL + i) * kWave + lane) * EPV;
+      if (col < hidden) {
+#pragma unroll
+        for (int j = 0; j < EPV; ++j) { const float d = xf[i][j] - mean; m2 += d * d; }
+      }
+    }
+    m2 = row_sum<WPR>(m2, smem, wave);
+    const float rs = rsqrtf(m2 * rn + eps);
+    if (row_ok && sub == 0 && lane == 0) { mu[row] = mean; rsigma[row] = rs; }
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      const int col = ((sub * VPL + i) * kWave + lane) * EPV;
+      if (row_ok && col < hidden) {
+        float gf[EPV], bf[EPV], zf[EPV];
+        load_pack<TW, EPV>(gamma + col, gf);
+        load_pack<TW, EPV>(beta + col, bf);
+#pragma unroll
+        for (int j = 0; j < EPV; ++j) zf[j] = gf[j] * (rs * (xf[i][j] - mean)) + bf[j];
+        store_pack<TW, EPV>(z + row * hidden + col, zf);
+      }
+    }
+  }
+}
+
+// Fallback for hidden sizes that are not a multiple of the vector width or exceed what the
+// register kernel holds: one block per row, three passes over the row (the re-reads hit cache).
+template <typename TI, typename TW>
+__global__ __launch_bounds__(LN_THREADS) void ln_fwd_generic_kernel(
+    const TI* __restrict__ x, const TW* __restrict__ gamma, const TW* __restrict__ beta,
+    TW* __restrict__ z, float* __restrict__ mu, float* __restrict__ rsigma, int64_t rows, int hidden,
+    float eps) {
+  __shared__ float smem[2 * LN_WAVES];
+  const int wave = threadIdx.x / kWave;
+  const float rn = 1.f / static_cast<float>(hidden);
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const TI* xr = x + row * hidden;
+    float s = 0.f;
+    for (int c = threadIdx.x; c < hidden; c += LN_THREADS) s += elem<TI>::to_float(xr[c]);
+    const float mean = row_sum<LN_WAVES>(s, smem, wave) * rn;
+    float m2 = 0.f;
+    for (int c = threadIdx.x; c < hidden; c += LN_THREADS) {
+      const float d = elem<TI>::to_float(xr[c]) - mean;
+      m2 += d * d;
+    }
+    m2 = row_sum<LN_WAVES>(m2, smem, wave);
+    const float rs = rsqrtf(m2 * rn + eps);
+    if (threadIdx.x == 0) { mu[row] = mean; rsigma[row] = rs; }
+    for (int c = threadIdx.x; c < hidden; c += LN_THREADS) {
+      const float y = rs * (elem<TI>::to_float(xr[c]) - mean);
+      z[row * hidden + c] =
+          elem<TW>::from_float(elem<TW>::to_float(gamma[c]) * y + elem<TW>::to_float(beta[c]));
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Backward. MEMEFF: x_or_z holds z and y is rebuilt as (z - beta) / gamma
+// (reference ln_bwd_kernels.cuh:91-110); otherwise y = rsigma * (x - mu).
+// Each lane keeps running sums of dz and dz*y for its own columns over all rows the block
+// visits; the block folds its wavefronts through LDS and writes one partial row.
+// ---------------------------------------------------------------------------------------------
+template <typename TI, typename TW, int VPL, int WPR, bool MEMEFF>
+__global__ __launch_bounds__(LN_THREADS) void ln_bwd_kernel(
+    const TW* __restrict__ dz, const TI* __restrict__ x_or_z, const float* __restrict__ mu,
+    const float* __restrict__ rsigma, const TW* __restrict__ gamma, const TW* __restrict__ beta,
+    TI* __restrict__ dx, float* __restrict__ dgamma_part, float* __restrict__ dbeta_part,
+    int64_t rows, int hidden) {
+  constexpr int EPV = ln_vec<TI>::EPV;
+  constexpr int RPB = LN_WAVES / WPR;
+  __shared__ float smem[2 * LN_WAVES];
+  extern __shared__ float fold[];  // [RPB-1][2][WPR*VPL*64*EPV] when RPB > 1
+
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const int sub = wave % WPR;
+  const float rn = 1.f / static_cast<float>(hidden);
+  const int64_t groups = (rows + RPB - 1) / RPB;
+
+  float gf[VPL][EPV], bf[VPL][EPV];
+  float dg_acc[VPL][EPV], db_acc[VPL][EPV];
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    const int col = ((sub * VPL + i) * kWave + lane) * EPV;
+    if (col < hidden) {
+      load_pack<TW, EPV>(gamma + col, gf[i]);
+      if constexpr (MEMEFF) load_pack<TW, EPV>(beta + col, bf[i]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < EPV; ++j) { gf[i][j] = 1.f; bf[i][j] = 0.f; }
+    }
+#pragma unroll
+    for (int j = 0; j < EPV; ++j) { dg_acc[i][j] = 0.f; db_acc[i][j] = 0.f; if (!MEMEFF) bf[i][j] = 0.f; }
+  }
+
+  for (int64_t g = blockIdx.x; g < groups; g += gridDim.x) {
+    const int64_t row = g * RPB + wave / WPR;
+    const bool row_ok = row < rows;
+    float dy[VPL][EPV], y[VPL][EPV];
+    float rs = 0.f, mean = 0.f;
+    if (row_ok) {
+      rs = rsigma[row];
+      if constexpr (!MEMEFF) mean = mu[row];
+    }
+    float sdy = 0.f, sdyy = 0.f;
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      const int col = ((sub * VPL + i) * kWave + lane) * EPV;
+      if (row_ok && col < hidden) {
+        float dzf[EPV], xf[EPV];
+        load_pack<TW, EPV>(dz + row * hidden + col, dzf);
+        load_pack<TI, EPV>(x_or_z + row * hidden + col, xf);
+#pragma unroll
+        for (int j = 0; j < EPV; ++j) {
+          float yv;
+          if constexpr (MEMEFF) yv = (xf[j] - bf[i][j]) / gf[i][j];
+          else yv = rs * (xf[j] - mean);
+          const float dyv = dzf[j] * gf[i][j];
+          sdy += dyv;
+          sdyy += dyv * yv;
+          dy[i][j] = dyv;
+          y[i][j] = yv;
+          dg_acc[i][j] += dzf[j] * yv;
+          db_acc[i][j] += dzf[j];
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < EPV; ++j) { dy[i][j] = 0.f; y[i][j] = 0.f; }
+      }
+    }
+    row_sum2<WPR>(sdy, sdyy, smem, wave);
+    const float mdy = sdy * rn, mdyy = sdyy * rn;
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      const int col = ((sub * VPL + i) * kWave + lane) * EPV;
+      if (row_ok && col < hidden) {
+        float dxf[EPV];
+#pragma unroll
+        for (int j = 0; j < EPV; ++j) dxf[j] = rs * (dy[i][j] - (mdyy * y[i][j] + mdy));
+        store_pack<TI, EPV>(dx + row * hidden + col, dxf);
+      }
+    }
+  }
+
+  // Fold the RPB row slots of the block (wavefronts that hold the same columns) in a fixed
+  // order, then write the block's partial row.
+  constexpr int SPAN = WPR * VPL * kWave * EPV;  // padded column span covered by the block
+  if constexpr (RPB > 1) {
+    const int slot = wave / WPR;
+    __syncthreads();
+    if (slot > 0) {
+#pragma unroll
+      for (int i = 0; i < VPL; ++i) {
+        const int pc = ((sub * VPL + i) * kWave + lane) * EPV;
+#pragma unroll
+        for (int j = 0; j < EPV; ++j) {
+          fold[((slot - 1) * 2 + 0) * SPAN + pc + j] = dg_acc[i][j];
+          fold[((slot - 1) * 2 + 1) * SPAN + pc + j] = db_acc[i][j];
+        }
+      }
+    }
+    __syncthreads();
+    if (slot == 0) {
+#pragma unroll
+      for (int i = 0; i < VPL; ++i) {
+        const int pc = ((sub * VPL + i) * kWave + lane) * EPV;
+#pragma unroll
+        for (int s = 0; s < RPB - 1; ++s) {
+#pragma unroll
+          for (int j = 0; j < EPV; ++j) {
+            dg_acc[i][j] += fold[(s * 2 + 0) * SPAN + pc + j];
+            db_acc[i][j] += fold[(s * 2 + 1) * SPAN + pc + j];
+          }
+        }
+      }
+    }
+  }
+  if (wave / WPR == 0) {
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      const int col = ((sub * VPL + i) * kWave + lane) * EPV;
+      if (col < hidden) {
+        store_pack<float, EPV>(dgamma_part + static_cast<int64_t>(blockIdx.x) * hidden + col, dg_acc[i]);
+        store_pack<float, EPV>(dbeta_part + static_cast<int64_t>(blockIdx.x) * hidden + col, db_acc[i]);
+      }
+    }
+  }
+}
+
+// Generic backward: one block per row slot, scalar columns, three passes; partial sums are kept
+// per thread for the columns c = threadIdx.x + k*LN_THREADS in the partial buffers themselves.
+template <typename TI, typename TW, bool MEMEFF>
+__global__ __launch_bounds__(LN_THREADS) void ln_bwd_generic_kernel(
+    const TW* __restrict__ dz, const TI* __restrict__ x_or_z, const float* __restrict__ mu,
+    const float* __restrict__ rsigma, const TW* __restrict__ gamma, const TW* __restrict__ beta,
+    TI* __restrict__ dx, float* __restrict__ dgamma_part, float* __restrict__ dbeta_part,
+    int64_t rows, int hidden) {
+  __shared__ float smem[2 * LN_WAVES];
+  const int wave = threadIdx.x / kWave;
+  const float rn = 1.f / static_cast<float>(hidden);
+  float* dgp = dgamma_part + static_cast<int64_t>(blockIdx.x) * hidden;
+  float* dbp = dbeta_part + static_cast<int64_t>(blockIdx.x) * hidden;
+  for (int c = threadIdx.x; c < hidden; c += LN_THREADS) { dgp[c] = 0.f; dbp[c] = 0.f; }
+  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
+    const float rs = rsigma[row];
+    const float mean = MEMEFF ? 0.f : mu[row];
+    float sdy = 0.f, sdyy = 0.f;
+    for (int c = threadIdx.x; c < hidden; c += LN_THREADS) {
+      const float gm = elem<TW>::to_float(gamma[c]);
+      const float xv = elem<TI>::to_float(x_or_z[row * hidden + c]);
+      const float yv = MEMEFF ? (xv - elem<TW>::to_float(beta[c])) / gm : rs * (xv - mean);
+      const float dzv = elem<TW>::to_float(dz[row * hidden + c]);
+      const float dyv = dzv * gm;
+      sdy += dyv;
+      sdyy += dyv * yv;
+      dgp[c] += dzv * yv;  // same thread owns column c in every row: no race
+      dbp[c] += dzv;
+    }
+    row_sum2<LN_WAVES>(sdy, sdyy, smem, wave);
+    const float mdy = sdy * rn, mdyy = sdyy * rn;
+    for (int c = threadIdx.x; c < hidden; c += LN_THREADS) {
+      const float gm = elem<TW>::to_float(gamma[c]);
+      const float xv = elem<TI>::to_float(x_or_z[row * hidden + c]);
+      const float yv = MEMEFF ? (xv - elem<TW>::to_float(beta[c])) / gm : rs * (xv - mean);
+      const float dyv = elem<TW>::to_float(dz[row * hidden + c]) * gm;
+      dx[row * hidden + c] = elem<TI>::from_float(rs * (dyv - (mdyy * yv + mdy)));
+    }
+  }
+}
+
+// Column sums of the [n_part, hidden] partials, in a fixed order. Block = 32 column lanes x 8
+// row groups; every thread walks its row group top to bottom, LDS folds the 8 groups in order.
+constexpr int FIN_COLS = 32, FIN_GROUPS = 8;
+template <typename TW>
+__global__ __launch_bounds__(FIN_COLS * FIN_GROUPS) void ln_bwd_finalize_kernel(
+    const float* __restrict__ dgamma_part, const float* __restrict__ dbeta_part,
+    TW* __restrict__ dgamma, TW* __restrict__ dbeta, int n_part, int hidden) {
+  __shared__ float red[FIN_GROUPS][FIN_COLS];
+  const float* src = blockIdx.y == 0 ? dgamma_part : dbeta_part;
+  TW* dst = blockIdx.y == 0 ? dgamma : dbeta;
+  const int cl = threadIdx.x % FIN_COLS, gr = threadIdx.x / FIN_COLS;
+  const int col = blockIdx.x * FIN_COLS + cl;
+  float s = 0.f;
+  if (col < hidden) {
+    const int per = (n_part + FIN_GROUPS - 1) / FIN_GROUPS;
+    const int lo = gr * per, hi = min(n_part, lo + per);
+    for (int p = lo; p < hi; ++p) s += src[static_cast<int64_t>(p) * hidden + col];
+  }
+  red[gr][cl] = s;
+  __syncthreads();
+  if (gr == 0 && col < hidden) {
+    float t = 0.f;
+#pragma unroll
+    for (int k = 0; k < FIN_GROUPS; ++k) t += red[k][cl];
+    dst[col] = elem<TW>::from_float(t);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Host-side shape planning.
+// ---------------------------------------------------------------------------------------------
+struct LnPlan {
+  bool vectorised;
+  int vpl, wpr;
+};
+
+template <typename TI>
+LnPlan ln_plan(int64_t hidden, int max_vpl) {
+  constexpr int EPV = ln_vec<TI>::EPV;
+  LnPlan p{false, 0, 0};
+  if (hidden % EPV != 0) return p;
+  const int64_t vecs = hidden / EPV;
+  for (int wpr = 1; wpr <= LN_WAVES; wpr *= 2) {
+    for (int vpl = 1; vpl <= max_vpl; vpl *= 2) {
+      if (static_cast<int64_t>(wpr) * vpl * kWave >= vecs) {
+        p.vectorised = true; p.vpl = vpl; p.wpr = wpr;
+        return p;
+      }
+    }
+  }
+  return p;
+}
+
+int ln_grid_limit() { return num_cus() * 8; }  // 8 blocks of 4 wavefronts per CU = full occupancy
+
+template <typename TI, typename TW>
+int ln_fwd_launch(const void* x, const void* gamma, const void* beta, void* z, float* mu,
+                  float* rsigma, int64_t rows, int64_t hidden, float eps, hipStream_t st) {
+  const bool al = aligned16(x) && aligned16(z) && aligned16(gamma) && aligned16(beta);
+  LnPlan p = al ? ln_plan<TI>(hidden, 8) : LnPlan{false, 0, 0};
+  auto X = static_cast<const TI*>(x);
+  auto G = static_cast<const TW*>(gamma);
+  auto B = static_cast<const TW*>(beta);
+  auto Z = static_cast<TW*>(z);
+  const int H = static_cast<int>(hidden);
+  if (!p.vectorised) {
+    const int grid = static_cast<int>(std::min<int64_t>(rows, ln_grid_limit()));
+    hipLaunchKernelGGL((ln_fwd_generic_kernel<TI, TW>), dim3(grid), dim3(LN_THREADS), 0, st, X, G, B,
+                       Z, mu, rsigma, rows, H, eps);
+    return 0;
+  }
+  const int rpb = LN_WAVES / p.wpr;
+  const int64_t groups = (rows + rpb - 1) / rpb;
+  const int grid = static_cast<int>(std::min<int64_t>(groups, ln_grid_limit()));
+#define LN_FWD_CASE(V, W)                                                                       \
+  if (p.vpl == V && p.wpr == W) {                                                               \
+    hipLaunchKernelGGL((ln_fwd_kernel<TI, TW, V, W>), dim3(grid), dim3(LN_THREADS), 0, st, X, G, \
+                       B, Z, mu, rsigma, rows, H, eps);                                         \
+    return 0;                                                                                   \
+  }
+  LN_FWD_CASE(1, 1) LN_FWD_CASE(2, 1) LN_FWD_CASE(4, 1) LN_FWD_CASE(8, 1)
+  LN_FWD_CASE(8, 2) LN_FWD_CASE(8, 4)
+#undef LN_FWD_CASE
+  return fail(NMTG_ERR_UNSUPPORTED, "ln_fwd: no kernel for plan vpl=%d wpr=%d", p.vpl, p.wpr);
+}
+
+constexpr int LN_BWD_MAX_VPL = 4;
+
+// One partial row per block: few enough blocks that the partials stay a small fraction of the
+// traffic, enough to keep every CU busy. Any n_part >= 1 is correct; this is the tuned choice.
+int64_t ln_bwd_parts_for(int64_t rows) {
+  const int64_t groups = (rows + LN_WAVES - 1) / LN_WAVES;
+  const int64_t cap = static_cast<int64_t>(num_cus()) * 2;
+  return std::max<int64_t>(1, std::min<int64_t>(groups, cap));
+}
+
+template <typename TI, typename TW>
+int ln_bwd_launch(const void* dz, const void* x_or_z, const float* mu, const float* rsigma,
+                  const void* gamma, const void* beta, void* dx, void* dgamma, void* dbeta,
+                  float* dgp, float* dbp, int64_t n_part, int64_t rows, int64_t hidden, bool memeff,
+                  hipStream_t st) {
+  auto DZ = static_cast<const TW*>(dz);
+  auto X = static_cast<const TI*>(x_or_z);
+  auto G = static_cast<const TW*>(gamma);
+  auto B = static_cast<const TW*>(beta);
+  auto DX = static_cast<TI*>(dx);
+  const int H = static_cast<int>(hidden);
+  const bool al = aligned16(dz) && aligned16(x_or_z) && aligned16(dx) && aligned16(gamma) &&
+                  (!memeff || aligned16(beta)) && aligned16(dgp) && aligned16(dbp);
+  LnPlan p = ln_plan<TI>(hidden, LN_BWD_MAX_VPL);
+  const int grid = static_cast<int>(n_part);
+  bool done = false;
+  if (p.vectorised && al) {
+    constexpr int EPV = ln_vec<TI>::EPV;
+    const int rpb = LN_WAVES / p.wpr;
+    const size_t fold_bytes =
+        rpb > 1 ? static_cast<size_t>(rpb - 1) * 2 * p.wpr * p.vpl * kWave * EPV * sizeof(float) : 0;
+#define LN_BWD_CASE(V, W)                                                                          \
+  if (!done && p.vpl == V && p.wpr == W) {                                                         \
+    if (memeff)                                                                                    \
+      hipLaunchKernelGGL((ln_bwd_kernel<TI, TW, V, W, true>), dim3(grid), dim3(LN_THREADS),        \
+                         fold_bytes, st, DZ, X, mu, rsigma, G, B, DX, dgp, dbp, rows, H);          \
+    else                                                                                           \
+      hipLaunchKernelGGL((ln_bwd_kernel<TI, TW, V, W, false>), dim3(grid), dim3(LN_THREADS),       \
+                         fold_bytes, st, DZ, X, mu, rsigma, G, B, DX, dgp, dbp, rows, H);          \
+    done = true;                                                                                   \
+  }
+    LN_BWD_CASE(1, 1) LN_BWD_CASE(2, 1) LN_BWD_CASE(4, 1) LN_BWD_CASE(4, 2) LN_BWD_CASE(4, 4)
+#undef LN_BWD_CASE
+  }
+  if (!done) {
+    if (memeff)
+      hipLaunchKernelGGL((ln_bwd_generic_kernel<TI, TW, true>), dim3(grid), dim3(LN_THREADS), 0, st,
+                         DZ, X, mu, rsigma, G, B, DX, dgp, dbp, rows, H);
+    else
+      hipLaunchKernelGGL((ln_bwd_generic_kernel<TI, TW, false>), dim3(grid), dim3(LN_THREADS), 0, st,
+                         DZ, X, mu, rsigma, G, B, DX, dgp, dbp, rows, H);
+  }
+  dim3 fgrid((H + FIN_COLS - 1) / FIN_COLS, 2);
+  hipLaunchKernelGGL((ln_bwd_finalize_kernel<TW>), fgrid, dim3(FIN_COLS * FIN_GROUPS), 0, st, dgp,
+                     dbp, static_cast<TW*>(dgamma), static_cast<TW*>(dbeta), static_cast<int>(n_part), H);
+  return 0;
+}
+
+// in/weight dtype pairs the reference registers (ln_fwd_cuda_kernel.cu:73-233): same type, or
+// 16-bit activations with fp32 weights.
+bool ln_pair_ok(int in_dtype, int w_dtype) {
+  return in_dtype == w_dtype || (w_dtype == NMTG_F32 && (in_dtype == NMTG_F16 || in_dtype == NMTG_BF16));
+}
+
+}  // namespace
+}  // namespace nmtg
+
+using namespace nmtg;
+
+extern "C" int nmtg_ln_fwd(const void* x, const void* gamma, const void* beta, void* z, float* mu,
+                           float* rsigma, int64_t rows, int64_t hidden, float eps, int in_dtype,
+                           int w_dtype, void* stream) {
+  NMTG_REQUIRE(x && gamma && beta && z && mu && rsigma, "ln_fwd: null pointer argument");
+  NMTG_REQUIRE(rows >= 0 && hidden > 0 && hidden <= (1 << 30), "ln_fwd: bad shape rows=%lld hidden=%lld",
+               (long long)rows, (long long)hidden);
+  NMTG_REQUIRE(eps >= 0.f, "ln_fwd: epsilon must be >= 0");
+  NMTG_REQUIRE(ln_pair_ok(in_dtype, w_dtype), "ln_fwd: unsupported dtype pair in=%d weight=%d", in_dtype, w_dtype);
+  if (rows == 0) return 0;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  int rc = 0;
+  if (in_dtype == w_dtype) {
+    NMTG_DISPATCH_DTYPE(in_dtype, T, rc = (ln_fwd_launch<T, T>(x, gamma, beta, z, mu, rsigma, rows, hidden, eps, st)));
+  } else if (in_dtype == NMTG_F16) {
+    rc = ln_fwd_launch<f16_t, float>(x, gamma, beta, z, mu, rsigma, rows, hidden, eps, st);
+  } else {
+    rc = ln_fwd_launch<bf16_t, float>(x, gamma, beta, z, mu, rsigma, rows, hidden, eps, st);
+  }
+  if (rc) return rc;
+  NMTG_CHECK_LAUNCH("ln_fwd");
+  return 0;
+}
+
+extern "C" int64_t nmtg_ln_bwd_parts(int64_t rows, int64_t hidden) {
+  if (rows <= 0 || hidden <= 0) return 1;
+  return ln_bwd_parts_for(rows);
+}
+
+extern "C" int nmtg_ln_bwd(const void* dz, const void* x_or_z, const float* mu, const float* rsigma,
+                           const void* gamma, const void* beta, void* dx, void* dgamma, void* dbeta,
+                           float* dgamma_part, float* dbeta_part, int64_t n_part, int64_t rows,
+                           int64_t hidden, int memory_efficient, int in_dtype, int w_dtype,
+                           void* stream) {
+  NMTG_REQUIRE(dz && x_or_z && rsigma && gamma && dx && dgamma && dbeta && dgamma_part && dbeta_part,
+               "ln_bwd: null pointer argument");
+  NMTG_REQUIRE(memory_efficient ? beta != nullptr : mu != nullptr,
+               "ln_bwd: %s is required", memory_efficient ? "beta (memory_efficient)" : "mu");
+  NMTG_REQUIRE(rows >= 0 && hidden > 0 && hidden <= (1 << 30), "ln_bwd: bad shape rows=%lld hidden=%lld",
+               (long long)rows, (long long)hidden);
+  NMTG_REQUIRE(ln_pair_ok(in_dtype, w_dtype), "ln_bwd: unsupported dtype pair in=%d weight=%d", in_dtype, w_dtype);
+  NMTG_REQUIRE(n_part >= 1 && n_part <= (1 << 20), "ln_bwd: n_part=%lld out of range", (long long)n_part);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  int rc = 0;
+  const bool me = memory_efficient != 0;
+  if (in_dtype == w_dtype) {
+    NMTG_DISPATCH_DTYPE(in_dtype, T, rc = (ln_bwd_launch<T, T>(dz, x_or_z, mu, rsigma, gamma, beta, dx, dgamma, dbeta,
+                                                               dgamma_part, dbeta_part, n_part, rows, hidden, me, st)));
+  } else if (in_dtype == NMTG_F16) {
+    rc = ln_bwd_launch<f16_t, float>(dz, x_or_z, mu, rsigma, gamma, beta, dx, dgamma, dbeta, dgamma_part,
+                                     dbeta_part, n_part, rows, hidden, me, st);
+  } else {
+    rc = ln_bwd_launch<bf16_t, float>(dz, x_or_z, mu, rsigma, gamma, beta, dx, dgamma, dbeta, dgamma_part,
+                                      dbeta_part, n_part, rows, hidden, me, st);
+  }
+  if (rc) return rc;
+  NMTG_CHECK_LAUNCH("ln_bwd");
+  return 0;
+}

@@ -1,0 +1,326 @@
+"""Pins the CPU oracle (oracle/) against PyTorch library routines, closed forms, invariants,
+brute-force loops and fp64 finite differences. All CPU; nothing here touches the HIP library.
+
+The reference tree stores no golden vectors for these ops (its tests draw random inputs and
+compare with PyTorch at run time), so the pins are the routines its fallback reduces to.
+"""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import attention, dropout_add, inputs, layer_norm, mlp, softmax_dropout, xentropy
+
+D = torch.float64
+
+
+# ------------------------------------------------------------------ LayerNorm
+@pytest.mark.parametrize("rows,hidden", [(7, 12), (33, 512), (5, 1000)])
+def test_ln_matches_library_and_autograd(rows, hidden):
+    d = inputs.layer_norm_inputs(rows, hidden, torch.float64, seed=3)
+    x = d["x"].clone().requires_grad_()
+    g = d["gamma"].clone().requires_grad_()
+    b = d["beta"].clone().requires_grad_()
+    z_lib = F.layer_norm(x, (hidden,), g, b, d["eps"])
+    z_lib.backward(d["dy"])
+    z, mu, rs = layer_norm.ln_fwd(d["x"], d["gamma"], d["beta"], d["eps"], D)
+    torch.testing.assert_close(z, z_lib.detach(), rtol=1e-12, atol=1e-12)
+    dx, dg, db = layer_norm.ln_bwd(d["dy"], d["x"], mu, rs, d["gamma"], D)
+    torch.testing.assert_close(dx, x.grad, rtol=1e-10, atol=1e-12)
+    torch.testing.assert_close(dg, g.grad, rtol=1e-10, atol=1e-12)
+    torch.testing.assert_close(db, b.grad, rtol=1e-10, atol=1e-12)
+    # memory-efficient backward (from z) equals the backward from x
+    dx2, dg2, db2 = layer_norm.ln_bwd_memory_efficient(d["dy"], z, rs, d["gamma"], d["beta"], D)
+    torch.testing.assert_close(dx2, dx, rtol=1e-9, atol=1e-11)
+    torch.testing.assert_close(dg2, dg, rtol=1e-9, atol=1e-11)
+
+
+def test_ln_invariants():
+    d = inputs.layer_norm_inputs(16, 64, torch.float64, seed=4)
+    ones, zeros = torch.ones(64, dtype=D), torch.zeros(64, dtype=D)
+    z, mu, rs = layer_norm.ln_fwd(d["x"], ones, zeros, 0.0, D)
+    assert z.mean(1).abs().max() < 1e-12                      # normalised rows have zero mean
+    torch.testing.assert_close((z * z).mean(1), torch.ones(16, dtype=D))  # ... and unit variance
+    torch.testing.assert_close(mu, d["x"].mean(1))
+    torch.testing.assert_close(rs, 1.0 / d["x"].var(1, unbiased=False).sqrt())
+    dx, _, _ = layer_norm.ln_bwd(d["dy"], d["x"], mu, rs, ones, D)
+    assert dx.sum(1).abs().max() < 1e-10                      # constant gamma: row sums of dx vanish
+    # shifting x by a row constant changes nothing
+    z2, _, _ = layer_norm.ln_fwd(d["x"] + 3.5, ones, zeros, 0.0, D)
+    torch.testing.assert_close(z2, z, rtol=1e-9, atol=1e-10)
+
+
+# ------------------------------------------------------------------ dropout-add
+def test_dropout_add_matches_autograd():
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(6, 10, generator=g, dtype=D, requires_grad=True)
+    r = torch.randn(6, 10, generator=g, dtype=D, requires_grad=True)
+    m = inputs.bernoulli_mask((6, 10), 0.7, g)
+    go = torch.randn(6, 10, generator=g, dtype=D)
+    out = dropout_add.dropout_add_fwd(x.detach(), r.detach(), m, 0.3, D)
+    ref = r + x * m.to(D) / 0.7
+    torch.testing.assert_close(out, ref.detach())
+    ref.backward(go)
+    dx, dr = dropout_add.dropout_add_bwd(go, m, 0.3, D)
+    torch.testing.assert_close(dx, x.grad)
+    torch.testing.assert_close(dr, r.grad)
+    torch.testing.assert_close(dropout_add.dropout_add_fwd(x.detach(), r.detach(), None, 0.0, D), (x + r).detach())
+    # all-ones mask at p -> 0 is the plain sum; all-zero mask leaves the residual
+    torch.testing.assert_close(dropout_add.dropout_add_fwd(x.detach(), r.detach(), torch.zeros_like(m), 0.3, D), r.detach())
+
+
+# ------------------------------------------------------------------ masked softmax + dropout
+def test_softmax_dropout_matches_library():
+    g = torch.Generator().manual_seed(6)
+    bh, tq, tk, heads = 6, 5, 9, 3
+    s = torch.randn(bh, tq, tk, generator=g, dtype=D)
+    pad = torch.zeros(2, tk, dtype=torch.bool)
+    pad[0, 6:] = True
+    pad[1, 3:] = True
+    sm_in = softmax_dropout.masked_scores(s, pad_mask=pad, heads=heads).requires_grad_()
+    m = inputs.bernoulli_mask((bh, tq, tk), 0.8, g)
+    lib = F.softmax(sm_in, dim=-1)
+    lib_dr = lib * m.to(D) / 0.8
+    sm, dr = softmax_dropout.softmax_dropout_fwd(sm_in.detach(), m, 0.2, D)
+    torch.testing.assert_close(sm, lib.detach())
+    torch.testing.assert_close(dr, lib_dr.detach())
+    go = torch.randn(bh, tq, tk, generator=g, dtype=D)
+    lib_dr.backward(go)
+    ds = softmax_dropout.softmax_dropout_bwd(go, sm, m, 0.2, D)
+    torch.testing.assert_close(ds, sm_in.grad)
+    # masked keys: exactly zero probability and gradient; rows sum to one
+    assert (sm.view(2, heads, tq, tk)[0, :, :, 6:] == 0).all() and (ds.view(2, heads, tq, tk)[1, :, :, 3:] == 0).all()
+    torch.testing.assert_close(sm.sum(-1), torch.ones(bh, tq, dtype=D))
+    assert ds.sum(-1).abs().max() < 1e-12
+
+
+def test_softmax_fully_masked_row_is_zero_and_time_mask():
+    s = torch.randn(2, 4, 4, dtype=D)
+    tm = torch.triu(torch.ones(4, 4), 1).bool()
+    sm, _ = softmax_dropout.softmax_dropout_fwd(softmax_dropout.masked_scores(s, time_mask=tm), None, 0.0, D)
+    assert (sm[:, 0, 1:] == 0).all() and torch.allclose(sm[:, 0, 0], torch.ones(2, dtype=D))
+    lib = F.softmax(s.masked_fill(tm, float("-inf")), -1)
+    torch.testing.assert_close(sm, lib)
+    allmask = torch.full((1, 2, 3), float("-inf"), dtype=D)
+    sm0, dr0 = softmax_dropout.softmax_dropout_fwd(allmask, None, 0.0, D)
+    assert (sm0 == 0).all() and (dr0 == 0).all()   # the library gives NaN here; the reference zeroes it
+
+
+# ------------------------------------------------------------------ xentropy
+@pytest.mark.parametrize("n,v,eps", [(9, 17, 0.1), (64, 1000, 0.0), (16, 4099, 0.3)])
+def test_xentropy_matches_library(n, v, eps):
+    d = inputs.xentropy_inputs(n, v, torch.float64, eps, padding_idx=1, pad_fraction=0.25, seed=7)
+    x = d["logits"].clone().requires_grad_()
+    lib = F.cross_entropy(x, d["labels"], ignore_index=1, reduction="none", label_smoothing=eps)
+    loss, lse = xentropy.xentropy_fwd(d["logits"], d["labels"], eps, 1, D)
+    torch.testing.assert_close(loss, lib.detach(), rtol=1e-11, atol=1e-12)
+    torch.testing.assert_close(lse, torch.logsumexp(d["logits"], 1))
+    gl = torch.rand(n, dtype=D) + 0.5
+    lib.backward(gl)
+    dx = xentropy.xentropy_bwd(gl, d["logits"], lse, d["labels"], eps, 1, D)
+    torch.testing.assert_close(dx, x.grad, rtol=1e-10, atol=1e-13)
+    pad = d["labels"] == 1
+    assert pad.any() and (loss[pad] == 0).all() and (dx[pad] == 0).all()      # exact zeros on padding
+    assert dx[~pad].sum(1).abs().max() < 1e-12                                # gradient rows sum to 0
+
+
+def test_xentropy_closed_forms():
+    # the two closed forms the reference's test states (extensions/xentropy/test_xentropy.py:44-62)
+    d = inputs.xentropy_inputs(12, 50, torch.float64, 0.1, padding_idx=0, pad_fraction=0.2, seed=8)
+    lp = F.log_softmax(d["logits"], -1)
+    ll = lp.gather(1, d["labels"].unsqueeze(1)).squeeze(1)
+    form = ((0.1 - 1.0) * ll - 0.1 * lp.mean(-1)).masked_fill(d["labels"] == 0, 0)
+    loss, _ = xentropy.xentropy_fwd(d["logits"], d["labels"], 0.1, 0, D)
+    torch.testing.assert_close(loss, form)
+    # eps = 0 reduces to lse - x_y; uniform logits give log V
+    loss0, lse0 = xentropy.xentropy_fwd(d["logits"], d["labels"], 0.0, -100, D)
+    torch.testing.assert_close(loss0, lse0 - d["logits"].gather(1, d["labels"].unsqueeze(1)).squeeze(1))
+    lu, _ = xentropy.xentropy_fwd(torch.zeros(3, 50, dtype=D), torch.tensor([4, 5, 6]), 0.1, -100, D)
+    torch.testing.assert_close(lu, torch.full((3,), math.log(50.0), dtype=D))
+
+
+# ------------------------------------------------------------------ MLP
+@pytest.mark.parametrize("act", ["relu", "gelu", "silu", "agelu", "none"])
+def test_mlp_matches_library_and_autograd(act):
+    d = inputs.mlp_inputs(24, 16, 40, torch.float64, p=0.2, seed=9, zero_bias=False)
+    x = d["x"].clone().requires_grad_()
+    ws = [d["w1"].clone().requires_grad_(), d["w2"].clone().requires_grad_()]
+    bs = [d["b1"].clone().requires_grad_(), d["b2"].clone().requires_grad_()]
+    h = F.linear(x, ws[0], bs[0])
+    lib_act = {"relu": F.relu, "gelu": F.gelu, "silu": F.silu, "none": lambda t: t,
+               "agelu": lambda t: F.gelu(t, approximate="tanh")}[act]
+    a = lib_act(h) * d["mask"].to(D) / 0.8
+    y_lib = F.linear(a, ws[1], bs[1])
+    y_lib.backward(d["dy"])
+    y, pre, post = mlp.mlp_fwd(d["x"], [d["w1"], d["w2"]], [d["b1"], d["b2"]], act, 0.2, [d["mask"]], D)
+    torch.testing.assert_close(y, y_lib.detach(), rtol=1e-11, atol=1e-12)
+    torch.testing.assert_close(pre[0], h.detach(), rtol=1e-12, atol=1e-12)
+    dx, dws, dbs = mlp.mlp_bwd(d["dy"], d["x"], [d["w1"], d["w2"]], pre, post, act, 0.2, [d["mask"]], D)
+    torch.testing.assert_close(dx, x.grad, rtol=1e-9, atol=1e-11)
+    for i in range(2):
+        torch.testing.assert_close(dws[i], ws[i].grad, rtol=1e-9, atol=1e-11)
+        torch.testing.assert_close(dbs[i], bs[i].grad, rtol=1e-9, atol=1e-11)
+
+
+def test_mlp_three_layers_and_activation_values():
+    g = torch.Generator().manual_seed(10)
+    x = torch.randn(5, 6, generator=g, dtype=D, requires_grad=True)
+    ws = [torch.randn(7, 6, generator=g, dtype=D), torch.randn(4, 7, generator=g, dtype=D), torch.randn(3, 4, generator=g, dtype=D)]
+    y_lib = F.linear(F.gelu(F.linear(F.gelu(F.linear(x, ws[0])), ws[1])), ws[2])
+    y, pre, post = mlp.mlp_fwd(x.detach(), ws, None, "gelu", 0.0, None, D)
+    torch.testing.assert_close(y, y_lib.detach())
+    dy = torch.randn(5, 3, generator=g, dtype=D)
+    y_lib.backward(dy)
+    dx, _, _ = mlp.mlp_bwd(dy, x.detach(), ws, pre, post, "gelu", 0.0, None, D)
+    torch.testing.assert_close(dx, x.grad)
+    # textbook values
+    t = torch.tensor([0.0, 1.0, -1.0], dtype=D)
+    torch.testing.assert_close(mlp.act_fwd(t, "gelu"), torch.tensor([0.0, 0.8413447460685429, -0.15865525393145707], dtype=D))
+    torch.testing.assert_close(mlp.act_fwd(t, "silu"), torch.tensor([0.0, 0.7310585786300049, -0.2689414213699951], dtype=D))
+
+
+# ------------------------------------------------------------------ attention
+def _deinterleave(w, heads, parts):
+    e3 = w.shape[0]
+    d = e3 // (heads * parts)
+    rest = w.shape[1:]
+    v = w.reshape(heads, parts, d, *rest)
+    return [v[:, i].reshape(heads * d, *rest) for i in range(parts)]
+
+
+def test_self_attention_matches_library_mha():
+    t, b, e, h = 7, 3, 16, 4
+    d = inputs.self_attn_inputs(t, b, e, h, torch.float64, p=0.0, seed=11, min_len=3, zero_bias=False)
+    out = attention.self_attn_fwd(d["x"], d["w_in"], d["w_out"], d["b_in"], d["b_out"], h, pad_mask=d["pad_mask"], ctype=D)
+    wq, wk, wv = _deinterleave(d["w_in"], h, 3)
+    bq, bk, bv = _deinterleave(d["b_in"], h, 3)
+    mha = torch.nn.MultiheadAttention(e, h, bias=True, dtype=D)
+    with torch.no_grad():
+        mha.in_proj_weight.copy_(torch.cat([wq, wk, wv]))
+        mha.in_proj_bias.copy_(torch.cat([bq, bk, bv]))
+        mha.out_proj.weight.copy_(d["w_out"])
+        mha.out_proj.bias.copy_(d["b_out"])
+    ref, attn = mha(d["x"], d["x"], d["x"], key_padding_mask=d["pad_mask"], need_weights=True, average_attn_weights=False)
+    torch.testing.assert_close(out["outputs"], ref.detach(), rtol=1e-10, atol=1e-11)
+    torch.testing.assert_close(out["softmax_results"].view(b, h, t, t), attn.detach(), rtol=1e-10, atol=1e-12)
+    # round trip of the weight interleave helper
+    torch.testing.assert_close(attention.interleave_qkv(wq, wk, wv, h), d["w_in"])
+
+
+def test_self_attention_causal_matches_sdpa_and_bruteforce():
+    t, b, e, h = 6, 2, 8, 2
+    d = inputs.self_attn_inputs(t, b, e, h, torch.float64, p=0.0, seed=12, causal=True, zero_bias=False)
+    out = attention.self_attn_fwd(d["x"], d["w_in"], d["w_out"], d["b_in"], d["b_out"], h, time_mask=d["time_mask"], ctype=D)
+    lin = out["input_lin_results"].view(t, b, h, 3, e // h)
+    q, k, v = [lin[:, :, :, i].permute(1, 2, 0, 3) for i in range(3)]   # [B,H,T,D]
+    sd = F.scaled_dot_product_attention(q, k, v, is_causal=True)
+    torch.testing.assert_close(out["matmul2_results"], sd.permute(2, 0, 1, 3).reshape(t, b, e), rtol=1e-10, atol=1e-12)
+    # brute force one (batch, head, query)
+    bi, hi, qi = 1, 1, 3
+    dd = e // h
+    acc = torch.zeros(dd, dtype=D)
+    ws = torch.tensor([math.exp(float(q[bi, hi, qi] @ k[bi, hi, j]) / math.sqrt(dd)) for j in range(qi + 1)], dtype=D)
+    for j in range(qi + 1):
+        acc += ws[j] / ws.sum() * v[bi, hi, j]
+    torch.testing.assert_close(out["matmul2_results"][qi, bi, hi * dd:(hi + 1) * dd], acc, rtol=1e-10, atol=1e-12)
+
+
+def _self_attn_autograd(d, h, pad=None, tm=None, p=0.0, dm=None):
+    """Independent autograd graph built from library ops on de-interleaved weights."""
+    t, b, e = d["x"].shape
+    dd = e // h
+    x = d["x"].clone().requires_grad_()
+    ps = [d[k].clone().requires_grad_() for k in ("w_in", "w_out", "b_in", "b_out")]
+    lin = F.linear(x, ps[0], ps[2]).view(t, b, h, 3, dd)
+    q, k, v = [lin[:, :, :, i].permute(1, 2, 0, 3) for i in range(3)]
+    s = q @ k.transpose(-1, -2) / math.sqrt(dd)
+    if pad is not None:
+        s = s.masked_fill(pad.view(b, 1, 1, t), float("-inf"))
+    if tm is not None:
+        s = s.masked_fill(tm.view(1, 1, t, t), float("-inf"))
+    pr = F.softmax(s, -1)
+    if dm is not None:
+        pr = pr * dm.view(b, h, t, t).to(D) / (1 - p)
+    ctx = (pr @ v).permute(2, 0, 1, 3).reshape(t, b, e)
+    out = F.linear(ctx, ps[1], ps[3])
+    out.backward(d["dout"])
+    return out.detach(), x.grad, [q_.grad for q_ in ps]
+
+
+@pytest.mark.parametrize("causal,p", [(False, 0.0), (False, 0.25), (True, 0.25)])
+def test_self_attention_backward_matches_autograd(causal, p):
+    t, b, e, h = 9, 3, 12, 3
+    d = inputs.self_attn_inputs(t, b, e, h, torch.float64, p=p, seed=13, min_len=4, causal=causal, zero_bias=False)
+    fwd = attention.self_attn_fwd(d["x"], d["w_in"], d["w_out"], d["b_in"], d["b_out"], h, d["pad_mask"], d["time_mask"],
+                                  p, d["dropout_mask"], D)
+    bwd = attention.self_attn_bwd(d["dout"], d["x"], d["w_in"], d["w_out"], h, fwd, p, d["dropout_mask"], D)
+    out, dx, (dwi, dwo, dbi, dbo) = _self_attn_autograd(d, h, d["pad_mask"], d["time_mask"], p, d["dropout_mask"])
+    torch.testing.assert_close(fwd["outputs"], out, rtol=1e-10, atol=1e-11)
+    for name, got, want in (("dx", bwd["dx"], dx), ("dw_in", bwd["dw_in"], dwi), ("dw_out", bwd["dw_out"], dwo),
+                            ("db_in", bwd["db_in"], dbi), ("db_out", bwd["db_out"], dbo)):
+        torch.testing.assert_close(got, want, rtol=1e-8, atol=1e-10, msg=lambda m, n=name: f"{n}: {m}")
+
+
+def test_encdec_attention_matches_library_and_autograd():
+    tq, tk, b, e, h = 5, 11, 2, 12, 3
+    dd = e // h
+    d = inputs.encdec_attn_inputs(tq, tk, b, e, h, torch.float64, p=0.2, seed=14, zero_bias=False)
+    fwd = attention.encdec_attn_fwd(d["x_q"], d["x_kv"], d["w_q"], d["w_kv"], d["w_out"], d["b_q"], d["b_kv"], d["b_out"],
+                                    h, d["pad_mask"], 0.2, d["dropout_mask"], D)
+    names = ("x_q", "x_kv", "w_q", "w_kv", "w_out", "b_q", "b_kv", "b_out")
+    leaf = {k: d[k].clone().requires_grad_() for k in names}
+    q = F.linear(leaf["x_q"], leaf["w_q"], leaf["b_q"]).view(tq, b, h, dd).permute(1, 2, 0, 3)
+    kv = F.linear(leaf["x_kv"], leaf["w_kv"], leaf["b_kv"]).view(tk, b, h, 2, dd)
+    k, v = kv[:, :, :, 0].permute(1, 2, 0, 3), kv[:, :, :, 1].permute(1, 2, 0, 3)
+    s = (q @ k.transpose(-1, -2) / math.sqrt(dd)).masked_fill(d["pad_mask"].view(b, 1, 1, tk), float("-inf"))
+    pr = F.softmax(s, -1) * d["dropout_mask"].view(b, h, tq, tk).to(D) / 0.8
+    out = F.linear((pr @ v).permute(2, 0, 1, 3).reshape(tq, b, e), leaf["w_out"], leaf["b_out"])
+    out.backward(d["dout"])
+    torch.testing.assert_close(fwd["outputs"], out.detach(), rtol=1e-10, atol=1e-11)
+    bwd = attention.encdec_attn_bwd(d["dout"], d["x_q"], d["x_kv"], d["w_q"], d["w_kv"], d["w_out"], h, fwd, 0.2,
+                                    d["dropout_mask"], D)
+    for k_, n in (("dx_q", "x_q"), ("dx_kv", "x_kv"), ("dw_q", "w_q"), ("dw_kv", "w_kv"), ("dw_out", "w_out"),
+                  ("db_q", "b_q"), ("db_kv", "b_kv"), ("db_out", "b_out")):
+        torch.testing.assert_close(bwd[k_], leaf[n].grad, rtol=1e-8, atol=1e-10, msg=lambda m, n=k_: f"{n}: {m}")
+    # p = 0 cross-check with the library's MultiheadAttention on de-interleaved weights
+    fwd0 = attention.encdec_attn_fwd(d["x_q"], d["x_kv"], d["w_q"], d["w_kv"], d["w_out"], d["b_q"], d["b_kv"], d["b_out"],
+                                     h, d["pad_mask"], 0.0, None, D)
+    wk, wv = _deinterleave(d["w_kv"], h, 2)
+    bk, bv = _deinterleave(d["b_kv"], h, 2)
+    mha = torch.nn.MultiheadAttention(e, h, bias=True, dtype=D)
+    with torch.no_grad():
+        mha.in_proj_weight.copy_(torch.cat([d["w_q"], wk, wv]))
+        mha.in_proj_bias.copy_(torch.cat([d["b_q"], bk, bv]))
+        mha.out_proj.weight.copy_(d["w_out"])
+        mha.out_proj.bias.copy_(d["b_out"])
+    ref, _ = mha(d["x_q"], d["x_kv"], d["x_kv"], key_padding_mask=d["pad_mask"])
+    torch.testing.assert_close(fwd0["outputs"], ref.detach(), rtol=1e-10, atol=1e-11)
+
+
+def test_attention_finite_differences():
+    # the reference validates its hand-written backward with fp64 gradcheck on tiny shapes
+    t, b, e, h = 4, 2, 8, 2
+    d = inputs.self_attn_inputs(t, b, e, h, torch.float64, p=0.0, seed=15, min_len=2, zero_bias=False)
+    fwd = attention.self_attn_fwd(d["x"], d["w_in"], d["w_out"], d["b_in"], d["b_out"], h, d["pad_mask"], ctype=D)
+    bwd = attention.self_attn_bwd(d["dout"], d["x"], d["w_in"], d["w_out"], h, fwd, ctype=D)
+    f = lambda x_: (attention.self_attn_fwd(x_, d["w_in"], d["w_out"], d["b_in"], d["b_out"], h, d["pad_mask"], ctype=D)["outputs"] * d["dout"]).sum()
+    eps = 1e-6
+    for idx in [(0, 0, 0), (2, 1, 5), (3, 0, 7)]:
+        xp, xm = d["x"].clone(), d["x"].clone()
+        xp[idx] += eps
+        xm[idx] -= eps
+        fd = (f(xp) - f(xm)) / (2 * eps)
+        assert abs(float(fd) - float(bwd["dx"][idx])) < 1e-6 * max(1.0, abs(float(fd)))
+
+
+def test_zipf_targets_and_masks_are_seeded():
+    a = inputs.xentropy_inputs(2000, 1000, with_logits=False, seed=1)
+    b = inputs.xentropy_inputs(2000, 1000, with_logits=False, seed=1)
+    assert torch.equal(a["labels"], b["labels"])
+    assert int((a["labels"] == 1).sum()) >= 200
+    assert a["labels"].min() >= 0 and a["labels"].max() < 1000
+    # heavy head: rank-0 id is the most frequent non-pad target
+    counts = torch.bincount(a["labels"], minlength=1000)
+    counts[1] = 0
+    assert int(counts.argmax()) == 0

@@ -1,0 +1,47 @@
+"""Comparison helpers shared by the parity tests.
+
+Tolerances (stated by the benchmark definition): fp32 1e-5 relative; fp16 / bf16 2e-2 relative
+and 1e-3 absolute; integer / index / zero-on-padding results bit-exact.
+"""
+import torch
+
+TOL = {
+    torch.float32: dict(rtol=1e-5, atol=1e-6),
+    torch.float16: dict(rtol=2e-2, atol=1e-3),
+    torch.bfloat16: dict(rtol=2e-2, atol=1e-3),
+}
+
+
+def assert_close(actual, expected, dtype, what="", rtol=None, atol=None, scale_atol=False):
+    """actual: tensor from the HIP path (any device / dtype); expected: oracle (CPU, fp32/fp64).
+
+    scale_atol: multiply the absolute tolerance by max|expected| — for reductions over thousands
+    of terms (weight / bias gradients) whose magnitude is far above 1.
+    """
+    tol = dict(TOL[dtype])
+    if rtol is not None:
+        tol["rtol"] = rtol
+    if atol is not None:
+        tol["atol"] = atol
+    a = actual.detach().to("cpu", torch.float64)
+    e = expected.detach().to("cpu", torch.float64)
+    assert a.shape == e.shape, f"{what}: shape {tuple(a.shape)} vs {tuple(e.shape)}"
+    at = tol["atol"]
+    if scale_atol:
+        at = at * max(1.0, float(e.abs().max()))
+    err = (a - e).abs()
+    bound = at + tol["rtol"] * e.abs()
+    bad = err > bound
+    if bad.any():
+        idx = torch.nonzero(bad)[0].tolist()
+        worst = float((err - bound).max())
+        raise AssertionError(
+            f"{what}: {int(bad.sum())}/{bad.numel()} elements out of tolerance "
+            f"(rtol={tol['rtol']}, atol={at}); first at {idx}: got {a[tuple(idx)].item()} "
+            f"want {e[tuple(idx)].item()}; worst excess {worst}")
+
+
+def rel_err(actual, expected):
+    a = actual.detach().to("cpu", torch.float64)
+    e = expected.detach().to("cpu", torch.float64)
+    return float((a - e).norm() / e.norm().clamp_min(1e-30))
