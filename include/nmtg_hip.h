@@ -74,6 +74,76 @@ int nmtg_ln_bwd(const void* dz, const void* x_or_z, const float* mu, const float
                 float* dgamma_part, float* dbeta_part, int64_t n_part, int64_t rows,
                 int64_t hidden, int memory_efficient, int in_dtype, int w_dtype, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Dropout + residual add (in place) and its backward.
+ * Reference: fused_dropout_add_cuda.forward(is_training, x, residual, p) -> (mask, out) and
+ *   .backward(grad, mask, p) -> dx,
+ *   onmt/modules/extensions/dropout_add/fused_dropout_add_cuda_kernel.cu:19-66 and :68-95.
+ *
+ * x <- residual + x * keep / (1 - p), n elements, in place in x (as the reference does).
+ * mask_mode: 0 = no dropout (x <- x + residual, mask untouched; the reference's eval / p == 0
+ *            branch), 1 = read the keep mask from `mask` (replay), 2 = draw the keep mask from
+ *            Philox4x32-10 keyed by (seed, offset, element index) and write it to `mask`.
+ * mask: n bytes, 1 = keep.
+ * ------------------------------------------------------------------------------------------ */
+int nmtg_dropout_add_fwd(void* x, const void* residual, uint8_t* mask, int64_t n, float p,
+                         int mask_mode, uint64_t seed, uint64_t offset, int dtype, void* stream);
+
+/* grad_x <- grad_out * mask / (1 - p); the residual's gradient is grad_out itself. */
+int nmtg_dropout_add_bwd(const void* grad_out, const uint8_t* mask, void* grad_x, int64_t n,
+                         float p, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Masked softmax over the last dimension with optional inverted dropout.
+ * Reference: the softmax stage of the fused attention, dispatch_softmax_dropout /
+ *   dispatch_softmax / dispatch_softmax_dropout_presampled
+ *   (onmt/modules/extensions/multihead_attn_blaslt/softmax_apex.h:443-486, :1263-1300, :874-912),
+ *   backward dispatch_softmax_dropout_backward_recompute / dispatch_softmax_backward_norecompute
+ *   (:4039-4075, :3467-3500); stand-alone callers use the module mask_softmax_dropout_cuda
+ *   (onmt/modules/optimized/attention_softmax.py:32-59).
+ *
+ * scores [rows, cols]; rows = batch * heads * q_len. key_mask (1 = masked key, may be NULL):
+ *   mask_kind 0 none, 1 key padding [batch, cols], 2 time mask [q_len, cols]. Scores may also
+ *   already hold -inf. A row with every key masked gives zeros.
+ * softmax_out (may be NULL) receives the probabilities before dropout, dropped_out the result.
+ * dropout_mode 0 none, 1 replay `dropout_mask` [rows, cols], 2 draw it from Philox and store it.
+ * Rows of up to 4096 keys (16-bit, cols % 8 == 0) / 2048 keys otherwise; the reference's limit is
+ *   2048 (softmax_apex.h:450-452).
+ * ------------------------------------------------------------------------------------------ */
+int nmtg_softmax_dropout_fwd(const void* scores, const uint8_t* key_mask, int mask_kind,
+                             void* softmax_out, void* dropped_out, uint8_t* dropout_mask,
+                             int dropout_mode, float p, uint64_t seed, uint64_t offset,
+                             int64_t rows, int64_t cols, int64_t q_len, int64_t heads, int dtype,
+                             void* stream);
+
+/* grad_scores = P * (g - sum_k P * g), g = dropout_mask * grad_dropped / (1 - p).
+ * saved holds the (masked) scores when saved_is_scores != 0 — P is recomputed, the reference's
+ * "backward_recompute" — or the probabilities P themselves. dropout_mode 0 or 1. */
+int nmtg_softmax_dropout_bwd(const void* grad_dropped, const void* saved, int saved_is_scores,
+                             const uint8_t* key_mask, int mask_kind, const uint8_t* dropout_mask,
+                             int dropout_mode, float p, void* grad_scores, int64_t rows,
+                             int64_t cols, int64_t q_len, int64_t heads, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Label-smoothed softmax cross-entropy.
+ * Reference: xentropy_cuda.forward(logits, labels, smoothing, half_to_float) ->
+ *   (losses, max_log_sum_exp) and .backward(grad_loss, logits, max_log_sum_exp, labels,
+ *   smoothing) -> grad_logits, onmt/modules/extensions/xentropy/interface.cpp:24-47,
+ *   xentropy_kernel.cu:571-718; the padding masked_fill_ of the Python wrapper
+ *   (onmt/modules/optimized/softmax_xentropy.py:10,24) is folded in through padding_idx
+ *   (pass a value no label takes, e.g. INT64_MIN, to switch it off).
+ *
+ * logits [rows, vocab] (fp32 / fp16 / bf16), labels int64 [rows]; losses, lse fp32 [rows];
+ * grad_loss fp32 [rows]; grad_logits [rows, vocab] in the logits dtype. fp32 accumulation.
+ * ------------------------------------------------------------------------------------------ */
+int nmtg_xentropy_fwd(const void* logits, const int64_t* labels, float* losses, float* lse,
+                      int64_t rows, int64_t vocab, float smoothing, int64_t padding_idx, int dtype,
+                      void* stream);
+
+int nmtg_xentropy_bwd(const float* grad_loss, const void* logits, const float* lse,
+                      const int64_t* labels, void* grad_logits, int64_t rows, int64_t vocab,
+                      float smoothing, int64_t padding_idx, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

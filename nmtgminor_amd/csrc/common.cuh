@@ -166,6 +166,98 @@ __device__ __forceinline__ void wave_sum2(float& a, float& b) {
   }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// Philox4x32-10 counter-based generator (Salmon et al., SC'11). One call turns a 128-bit
+// counter and a 64-bit key into four 32-bit words. Dropout draws u = (word >> 8) * 2^-24 in
+// [0, 1) and keeps an element when u < keep_probability.
+// ---------------------------------------------------------------------------------------------
+struct Philox {
+  uint32_t key0, key1;
+  __device__ __forceinline__ Philox(uint64_t seed) : key0(static_cast<uint32_t>(seed)), key1(static_cast<uint32_t>(seed >> 32)) {}
+  __device__ __forceinline__ uint4 operator()(uint64_t index, uint64_t offset) const {
+    uint32_t c0 = static_cast<uint32_t>(offset), c1 = static_cast<uint32_t>(offset >> 32);
+    uint32_t c2 = static_cast<uint32_t>(index), c3 = static_cast<uint32_t>(index >> 32);
+    uint32_t k0 = key0, k1 = key1;
+#pragma unroll
+    for (int r = 0; r < 10; ++r) {
+      const uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
+      const uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+      const uint32_t n0 = hi1 ^ c1 ^ k0, n2 = hi0 ^ c3 ^ k1;
+      c0 = n0; c1 = lo1; c2 = n2; c3 = lo0;
+      k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+    }
+    return make_uint4(c0, c1, c2, c3);
+  }
+};
+
+__device__ __forceinline__ float u01(uint32_t w) { return static_cast<float>(w >> 8) * (1.0f / 16777216.0f); }
+
+// Keep-decisions for N consecutive elements starting at linear element index `first` (first % 4
+// == 0 when N >= 4): element i uses word (i % 4) of the Philox block with index i / 4, so the
+// mask depends only on (seed, offset, element index), not on the launch shape.
+template <int N>
+__device__ __forceinline__ void philox_keep(const Philox& gen, uint64_t first, uint64_t offset, float keep_p,
+                                            uint8_t (&keep)[N]) {
+  if constexpr (N >= 4) {
+#pragma unroll
+    for (int b = 0; b < N / 4; ++b) {
+      const uint4 r = gen(first / 4 + b, offset);
+      keep[b * 4 + 0] = u01(r.x) < keep_p;
+      keep[b * 4 + 1] = u01(r.y) < keep_p;
+      keep[b * 4 + 2] = u01(r.z) < keep_p;
+      keep[b * 4 + 3] = u01(r.w) < keep_p;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const uint64_t e = first + i;
+      const uint4 r = gen(e / 4, offset);
+      const uint32_t w = (e & 3) == 0 ? r.x : (e & 3) == 1 ? r.y : (e & 3) == 2 ? r.z : r.w;
+      keep[i] = u01(w) < keep_p;
+    }
+  }
+}
+
+template <int N>
+__device__ __forceinline__ void load_bytes(const uint8_t* __restrict__ p, uint8_t (&out)[N]) {
+  if constexpr (N == 8) {
+    uint2 raw = *reinterpret_cast<const uint2*>(p);
+    const uint8_t* e = reinterpret_cast<const uint8_t*>(&raw);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) out[j] = e[j];
+  } else if constexpr (N == 4) {
+    uint32_t raw = *reinterpret_cast<const uint32_t*>(p);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) out[j] = (raw >> (8 * j)) & 0xffu;
+  } else if constexpr (N == 2) {
+    uint16_t raw = *reinterpret_cast<const uint16_t*>(p);
+    out[0] = raw & 0xffu; out[1] = raw >> 8;
+  } else {
+#pragma unroll
+    for (int j = 0; j < N; ++j) out[j] = p[j];
+  }
+}
+
+template <int N>
+__device__ __forceinline__ void store_bytes(uint8_t* __restrict__ p, const uint8_t (&in)[N]) {
+  if constexpr (N == 8) {
+    uint2 raw;
+    uint8_t* e = reinterpret_cast<uint8_t*>(&raw);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) e[j] = in[j];
+    *reinterpret_cast<uint2*>(p) = raw;
+  } else if constexpr (N == 4) {
+    uint32_t raw = in[0] | (in[1] << 8) | (in[2] << 16) | (static_cast<uint32_t>(in[3]) << 24);
+    *reinterpret_cast<uint32_t*>(p) = raw;
+  } else if constexpr (N == 2) {
+    *reinterpret_cast<uint16_t*>(p) = static_cast<uint16_t>(in[0] | (in[1] << 8));
+  } else {
+#pragma unroll
+    for (int j = 0; j < N; ++j) p[j] = in[j];
+  }
+}
+
 // Dispatch a runtime dtype code to a template parameter.
 #define NMTG_DISPATCH_DTYPE(code, T, ...)                                   \
   switch (code) {                                                           \

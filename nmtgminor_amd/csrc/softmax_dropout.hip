@@ -1,0 +1,291 @@
+// Masked row softmax with optional inverted dropout, and its backward, for gfx950.
+//
+// Stands in for the softmax stage of the reference's fused attention
+// (onmt/modules/extensions/multihead_attn_blaslt/softmax_apex.h: dispatch_softmax_dropout
+// :443-486, dispatch_softmax :1263-1300, dispatch_softmax_dropout_presampled :874-912,
+// dispatch_softmax_dropout_backward_recompute :4039-4075, dispatch_softmax_backward_norecompute
+// :3467-3500) and for the stand-alone module mask_softmax_dropout_cuda that
+// onmt/modules/optimized/attention_softmax.py:32-59 calls.
+//
+// One 64-lane wavefront owns one row of `cols` keys and keeps it in registers (VPL vectors of
+// EPV elements per lane), so every score is read once and every probability written once.
+// Masking can be fused: a key-padding mask [batch, cols] (row -> batch = row / (heads*q_len)) or
+// a time mask [q_len, cols] (row -> query = row % q_len); masked keys count as -inf. A row whose
+// keys are all masked yields zeros (the reference turns the NaN into 0, softmax_apex.h:209-211).
+// Dropout: keep mask of one byte per element, read (replay) or drawn from Philox and written.
+//
+// Bandwidth bound. Per element: forward reads the score (+1 B mask in replay mode), writes the
+// result (+1 B mask in RNG mode); backward reads grad, the saved scores or probabilities and the
+// mask byte, writes the score gradient.
+#include "common.cuh"
+
+namespace nmtg {
+namespace {
+
+constexpr int SM_THREADS = 256;
+constexpr int SM_WAVES = SM_THREADS / kWave;
+enum { SM_NO_DROPOUT = 0, SM_MASK_IN = 1, SM_MASK_RNG = 2 };
+enum { SM_NOMASK = 0, SM_PAD = 1, SM_TIME = 2 };
+
+struct SoftmaxArgs {
+  const void* in;          // fwd: scores; bwd: grad wrt the dropped probabilities
+  const void* saved;       // bwd: saved scores (recompute) or saved probabilities
+  void* out;               // fwd: dropped probabilities; bwd: grad wrt scores
+  void* out_softmax;       // fwd: optional pre-dropout probabilities
+  uint8_t* dmask;          // dropout keep mask
+  const uint8_t* kmask;    // key-padding or time mask (1 = masked)
+  int64_t rows;
+  int cols;
+  int q_len;               // queries per (batch, head)
+  int heads;
+  int kmask_kind;
+  int dropout_mode;
+  int from_scores;         // bwd: saved holds scores (1) or probabilities (0)
+  float keep_p, scale;
+  uint64_t seed, offset;
+};
+
+__device__ __forceinline__ const uint8_t* kmask_row(const SoftmaxArgs& a, int64_t row) {
+  if (a.kmask_kind == SM_PAD) return a.kmask + (row / (static_cast<int64_t>(a.heads) * a.q_len)) * a.cols;
+  if (a.kmask_kind == SM_TIME) return a.kmask + (row % a.q_len) * static_cast<int64_t>(a.cols);
+  return nullptr;
+}
+
+// Loads the row's scores into v (masked / out-of-range -> -inf), returns the normalised
+// probabilities in v and whether the row had any unmasked key.
+template <typename T, int EPV, int VPL>
+__device__ __forceinline__ void row_softmax(const T* __restrict__ src, const uint8_t* __restrict__ km, int cols,
+                                            int lane, float (&v)[VPL][EPV]) {
+  float mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    const int col = (i * kWave + lane) * EPV;
+    if (col < cols) {
+      load_pack<T, EPV>(src + col, v[i]);
+      if (km != nullptr) {
+        uint8_t mk[EPV];
+        load_bytes<EPV>(km + col, mk);
+#pragma unroll
+        for (int j = 0; j < EPV; ++j) if (mk[j]) v[i][j] = -INFINITY;
+      }
+#pragma unroll
+      for (int j = 0; j < EPV; ++j) mx = fmaxf(mx, v[i][j]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < EPV; ++j) v[i][j] = -INFINITY;
+    }
+  }
+  mx = wave_max(mx);
+  const float base = (mx == -INFINITY) ? 0.f : mx;
+  float sum = 0.f;
+  constexpr float LOG2E = 1.4426950408889634f;
+#pragma unroll
+  for (int i = 0; i < VPL; ++i)
+#pragma unroll
+    for (int j = 0; j < EPV; ++j) { v[i][j] = exp2f((v[i][j] - base) * LOG2E); sum += v[i][j]; }
+  sum = wave_sum(sum);
+  const float inv = sum > 0.f ? 1.f / sum : 0.f;
+#pragma unroll
+  for (int i = 0; i < VPL; ++i)
+#pragma unroll
+    for (int j = 0; j < EPV; ++j) v[i][j] *= inv;
+}
+
+template <typename T, int EPV, int VPL>
+__global__ __launch_bounds__(SM_THREADS) void softmax_fwd_kernel(SoftmaxArgs a) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * SM_WAVES + threadIdx.x / kWave;
+  if (row >= a.rows) return;
+  const int64_t base = row * a.cols;
+  float v[VPL][EPV];
+  row_softmax<T, EPV, VPL>(static_cast<const T*>(a.in) + base, kmask_row(a, row), a.cols, lane, v);
+  T* out = static_cast<T*>(a.out) + base;
+  T* out_sm = a.out_softmax ? static_cast<T*>(a.out_softmax) + base : nullptr;
+  const Philox gen(a.seed);
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    const int col = (i * kWave + lane) * EPV;
+    if (col < a.cols) {
+      if (out_sm) store_pack<T, EPV>(out_sm + col, v[i]);
+      if (a.dropout_mode != SM_NO_DROPOUT) {
+        uint8_t keep[EPV];
+        if (a.dropout_mode == SM_MASK_IN) {
+          load_bytes<EPV>(a.dmask + base + col, keep);
+        } else {
+          philox_keep<EPV>(gen, static_cast<uint64_t>(base + col), a.offset, a.keep_p, keep);
+          store_bytes<EPV>(a.dmask + base + col, keep);
+        }
+#pragma unroll
+        for (int j = 0; j < EPV; ++j) v[i][j] = keep[j] ? v[i][j] * a.scale : 0.f;
+      }
+      store_pack<T, EPV>(out + col, v[i]);
+    }
+  }
+}
+
+// dS = P * (g - sum_k P * g), g = keep * dP / (1 - p).
+template <typename T, int EPV, int VPL>
+__global__ __launch_bounds__(SM_THREADS) void softmax_bwd_kernel(SoftmaxArgs a) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * SM_WAVES + threadIdx.x / kWave;
+  if (row >= a.rows) return;
+  const int64_t base = row * a.cols;
+  float pr[VPL][EPV], g[VPL][EPV];
+  const T* saved = static_cast<const T*>(a.saved) + base;
+  if (a.from_scores) {
+    row_softmax<T, EPV, VPL>(saved, kmask_row(a, row), a.cols, lane, pr);
+  } else {
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      const int col = (i * kWave + lane) * EPV;
+      if (col < a.cols) load_pack<T, EPV>(saved + col, pr[i]);
+      else {
+#pragma unroll
+        for (int j = 0; j < EPV; ++j) pr[i][j] = 0.f;
+      }
+    }
+  }
+  const T* gin = static_cast<const T*>(a.in) + base;
+  float dot = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    const int col = (i * kWave + lane) * EPV;
+    if (col < a.cols) {
+      load_pack<T, EPV>(gin + col, g[i]);
+      if (a.dropout_mode != SM_NO_DROPOUT) {
+        uint8_t keep[EPV];
+        load_bytes<EPV>(a.dmask + base + col, keep);
+#pragma unroll
+        for (int j = 0; j < EPV; ++j) g[i][j] = keep[j] ? g[i][j] * a.scale : 0.f;
+      }
+#pragma unroll
+      for (int j = 0; j < EPV; ++j) dot += pr[i][j] * g[i][j];
+    } else {
+#pragma unroll
+      for (int j = 0; j < EPV; ++j) g[i][j] = 0.f;
+    }
+  }
+  dot = wave_sum(dot);
+  T* out = static_cast<T*>(a.out) + base;
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    const int col = (i * kWave + lane) * EPV;
+    if (col < a.cols) {
+#pragma unroll
+      for (int j = 0; j < EPV; ++j) g[i][j] = pr[i][j] * (g[i][j] - dot);
+      store_pack<T, EPV>(out + col, g[i]);
+    }
+  }
+}
+
+// Vector width: the widest of 16 / 8 / 4 / 2-byte accesses that every row start and the masks
+// allow, narrowed further for short rows so that all 64 lanes hold data.
+template <typename T>
+int pick_epv(const SoftmaxArgs& a, bool bwd) {
+  constexpr int WIDE = 16 / sizeof(T);
+  int epv = WIDE;
+  auto ok = [&](int e) {
+    if (a.cols % e) return false;
+    const uintptr_t bytes = static_cast<uintptr_t>(e) * sizeof(T);
+    auto al = [&](const void* p, uintptr_t b) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) % b) == 0; };
+    if (!al(a.in, bytes) || !al(a.out, bytes) || !al(a.saved, bytes) || !al(a.out_softmax, bytes)) return false;
+    if (!al(a.dmask, e) || !al(a.kmask, e)) return false;
+    (void)bwd;
+    return true;
+  };
+  while (epv > 1 && !ok(epv)) epv /= 2;
+  while (epv > 2 && a.cols < epv * kWave) epv /= 2;  // short rows: spread over more lanes
+  return epv;
+}
+
+template <typename T>
+int softmax_launch(const SoftmaxArgs& a, bool bwd, hipStream_t st) {
+  const int epv = pick_epv<T>(a, bwd);
+  const int vecs = (a.cols + epv - 1) / epv;
+  int vpl = 1;
+  while (vpl * kWave < vecs) vpl *= 2;
+  const unsigned grid = static_cast<unsigned>((a.rows + SM_WAVES - 1) / SM_WAVES);
+  bool done = false;
+#define SM_CASE(E, V)                                                                                     \
+  if (!done && epv == E && vpl == V) {                                                                    \
+    if (bwd) hipLaunchKernelGGL((softmax_bwd_kernel<T, E, V>), dim3(grid), dim3(SM_THREADS), 0, st, a);   \
+    else hipLaunchKernelGGL((softmax_fwd_kernel<T, E, V>), dim3(grid), dim3(SM_THREADS), 0, st, a);       \
+    done = true;                                                                                          \
+  }
+  if constexpr (sizeof(T) == 2) { SM_CASE(8, 1) SM_CASE(8, 2) SM_CASE(8, 4) SM_CASE(8, 8) }
+  SM_CASE(4, 1) SM_CASE(4, 2) SM_CASE(4, 4) SM_CASE(4, 8) SM_CASE(4, 16)
+  SM_CASE(2, 1) SM_CASE(2, 2) SM_CASE(2, 4) SM_CASE(2, 8) SM_CASE(2, 16)
+  SM_CASE(1, 1) SM_CASE(1, 2) SM_CASE(1, 4) SM_CASE(1, 8) SM_CASE(1, 16) SM_CASE(1, 32)
+#undef SM_CASE
+  if (!done)
+    return fail(NMTG_ERR_UNSUPPORTED,
+                "softmax: row length %d is beyond what one wavefront holds at vector width %d "
+                "(limit 4096 keys for aligned 16-bit rows, 2048 otherwise)", a.cols, epv);
+  return 0;
+}
+
+int check_common(const char* who, const SoftmaxArgs& a, float p) {
+  NMTG_REQUIRE(a.rows >= 0 && a.cols > 0, "%s: bad shape rows=%lld cols=%d", who, (long long)a.rows, a.cols);
+  NMTG_REQUIRE(a.dropout_mode >= SM_NO_DROPOUT && a.dropout_mode <= SM_MASK_RNG, "%s: bad dropout_mode", who);
+  NMTG_REQUIRE(a.kmask_kind >= SM_NOMASK && a.kmask_kind <= SM_TIME, "%s: bad mask_kind", who);
+  if (a.kmask_kind != SM_NOMASK) {
+    NMTG_REQUIRE(a.kmask != nullptr, "%s: mask_kind set but mask pointer is null", who);
+    NMTG_REQUIRE(a.q_len > 0 && a.heads > 0, "%s: q_len and heads must be positive with a mask", who);
+    NMTG_REQUIRE(a.rows % (static_cast<int64_t>(a.q_len) * (a.kmask_kind == SM_PAD ? a.heads : 1)) == 0,
+                 "%s: rows is not a multiple of %s", who, a.kmask_kind == SM_PAD ? "heads*q_len" : "q_len");
+  }
+  if (a.dropout_mode != SM_NO_DROPOUT) {
+    NMTG_REQUIRE(a.dmask != nullptr, "%s: dropout mask buffer required", who);
+    NMTG_REQUIRE(p >= 0.f && p < 1.f, "%s: dropout probability %f outside [0, 1)", who, p);
+  }
+  return 0;
+}
+
+}  // namespace
+}  // namespace nmtg
+
+using namespace nmtg;
+
+extern "C" int nmtg_softmax_dropout_fwd(const void* scores, const uint8_t* key_mask, int mask_kind, void* softmax_out,
+                                        void* dropped_out, uint8_t* dropout_mask, int dropout_mode, float p,
+                                        uint64_t seed, uint64_t offset, int64_t rows, int64_t cols, int64_t q_len,
+                                        int64_t heads, int dtype, void* stream) {
+  NMTG_REQUIRE(cols > 0 && cols <= (1 << 20) && q_len <= INT32_MAX && heads <= INT32_MAX,
+               "softmax_dropout_fwd: bad shape cols=%lld", (long long)cols);
+  SoftmaxArgs a{};
+  a.in = scores; a.out = dropped_out; a.out_softmax = softmax_out; a.dmask = dropout_mask; a.kmask = key_mask;
+  a.rows = rows; a.cols = static_cast<int>(cols); a.q_len = static_cast<int>(q_len); a.heads = static_cast<int>(heads);
+  a.kmask_kind = mask_kind; a.dropout_mode = dropout_mode;
+  a.keep_p = 1.f - p; a.scale = 1.f / (1.f - p); a.seed = seed; a.offset = offset;
+  if (int rc = check_common("softmax_dropout_fwd", a, p)) return rc;
+  if (rows == 0) return 0;
+  NMTG_REQUIRE(scores && dropped_out, "softmax_dropout_fwd: null pointer argument");
+  int rc = 0;
+  NMTG_DISPATCH_DTYPE(dtype, T, rc = softmax_launch<T>(a, false, static_cast<hipStream_t>(stream)));
+  if (rc) return rc;
+  NMTG_CHECK_LAUNCH("softmax_dropout_fwd");
+  return 0;
+}
+
+extern "C" int nmtg_softmax_dropout_bwd(const void* grad_dropped, const void* saved, int saved_is_scores,
+                                        const uint8_t* key_mask, int mask_kind, const uint8_t* dropout_mask,
+                                        int dropout_mode, float p, void* grad_scores, int64_t rows, int64_t cols,
+                                        int64_t q_len, int64_t heads, int dtype, void* stream) {
+  NMTG_REQUIRE(cols > 0 && cols <= (1 << 20) && q_len <= INT32_MAX && heads <= INT32_MAX,
+               "softmax_dropout_bwd: bad shape cols=%lld", (long long)cols);
+  NMTG_REQUIRE(dropout_mode != SM_MASK_RNG, "softmax_dropout_bwd: the backward replays a stored mask (mode 0 or 1)");
+  SoftmaxArgs a{};
+  a.in = grad_dropped; a.saved = saved; a.out = grad_scores; a.dmask = const_cast<uint8_t*>(dropout_mask);
+  a.kmask = key_mask; a.rows = rows; a.cols = static_cast<int>(cols); a.q_len = static_cast<int>(q_len);
+  a.heads = static_cast<int>(heads); a.kmask_kind = saved_is_scores ? mask_kind : SM_NOMASK;
+  a.dropout_mode = dropout_mode; a.from_scores = saved_is_scores ? 1 : 0;
+  a.keep_p = 1.f - p; a.scale = 1.f / (1.f - p);
+  if (int rc = check_common("softmax_dropout_bwd", a, p)) return rc;
+  if (rows == 0) return 0;
+  NMTG_REQUIRE(grad_dropped && saved && grad_scores, "softmax_dropout_bwd: null pointer argument");
+  int rc = 0;
+  NMTG_DISPATCH_DTYPE(dtype, T, rc = softmax_launch<T>(a, true, static_cast<hipStream_t>(stream)));
+  if (rc) return rc;
+  NMTG_CHECK_LAUNCH("softmax_dropout_bwd");
+  return 0;
+}

@@ -1,0 +1,224 @@
+// Label-smoothed softmax cross-entropy over large vocabularies, forward and backward, gfx950.
+//
+// Stands in for xentropy_cuda.forward / backward of the reference
+// (onmt/modules/extensions/xentropy/xentropy_kernel.cu:382-474 kernels, :571-718 host side,
+// interface.cpp:24-47) plus the padding handling its Python wrapper does afterwards with
+// masked_fill_ (onmt/modules/optimized/softmax_xentropy.py:10,24), which is fused here.
+//
+//   lse_i  = max_j x_ij + log sum_j exp(x_ij - max)
+//   loss_i = eps (lse_i - mean_j x_ij) + (1 - eps)(lse_i - x_{i,y_i});   0 if y_i == padding_idx
+//   dx_ij  = g_i (exp(x_ij - lse_i) - (1 - eps)[j == y_i] - eps / V);    0 if y_i == padding_idx
+//
+// One block per row. The forward makes ONE pass over the row (the reference makes two): every
+// lane keeps an online (max, sum-exp) pair plus the plain sum, merged across the block at the end.
+// Rows are not 16-byte aligned in general (V * sizeof(T) need not be a multiple of 16): each row is
+// split into a scalar head up to the first 16-byte boundary, a body of 16-byte vectors and a
+// scalar tail. All indexing is 64-bit (N * V exceeds 2^31 at the benchmark shape).
+//
+// Bandwidth bound: forward reads N*V elements once; backward reads them once and writes N*V
+// (rows whose label is the padding index are written as zeros without reading the logits).
+#include "common.cuh"
+
+namespace nmtg {
+namespace {
+
+constexpr int XE_THREADS = 1024;
+constexpr int XE_WAVES = XE_THREADS / kWave;
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float LN2 = 0.6931471805599453f;
+constexpr float NEG_BIG = -3.0e38f;
+
+struct Online {
+  float m, s;  // running max and sum of exp(x - m)
+};
+__device__ __forceinline__ Online merge(Online a, Online b) {
+  const float m = fmaxf(a.m, b.m);
+  Online r;
+  r.m = m;
+  r.s = a.s * exp2f((a.m - m) * LOG2E) + b.s * exp2f((b.m - m) * LOG2E);
+  return r;
+}
+
+template <int N>
+__device__ __forceinline__ void online_add(Online& st, float& sx, const float (&v)[N]) {
+  float cm = v[0];
+#pragma unroll
+  for (int j = 1; j < N; ++j) cm = fmaxf(cm, v[j]);
+  if (cm > st.m) {
+    st.s *= exp2f((st.m - cm) * LOG2E);
+    st.m = cm;
+  }
+  const float mb = st.m * LOG2E;
+  float acc = 0.f, sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < N; ++j) {
+    acc += exp2f(fmaf(v[j], LOG2E, -mb));
+    sum += v[j];
+  }
+  st.s += acc;
+  sx += sum;
+}
+
+template <typename T>
+__global__ __launch_bounds__(XE_THREADS) void xentropy_fwd_kernel(
+    const T* __restrict__ logits, const int64_t* __restrict__ labels, float* __restrict__ losses,
+    float* __restrict__ lse_out, int64_t vocab, float smoothing, int64_t padding_idx) {
+  constexpr int EPV = 16 / sizeof(T);
+  __shared__ float sm_m[XE_WAVES], sm_s[XE_WAVES], sm_x[XE_WAVES];
+  const int64_t row = blockIdx.x;
+  const T* x = logits + row * vocab;
+  const int tid = threadIdx.x;
+
+  const uintptr_t addr = reinterpret_cast<uintptr_t>(x);
+  int64_t head = static_cast<int64_t>(((16 - (addr & 15)) & 15) / sizeof(T));
+  if (head > vocab) head = vocab;
+  const int64_t nvec = (vocab - head) / EPV;
+  const int64_t tail0 = head + nvec * EPV;
+
+  Online st{NEG_BIG, 0.f};
+  float sx = 0.f;
+  if (tid < head) {
+    float v[1] = {elem<T>::to_float(x[tid])};
+    online_add<1>(st, sx, v);
+  }
+  const T* body = x + head;
+  int64_t i = tid;
+  // two vectors in flight per lane per trip
+  for (; i + XE_THREADS < nvec; i += 2 * XE_THREADS) {
+    float a[EPV], b[EPV];
+    load_pack<T, EPV>(body + i * EPV, a);
+    load_pack<T, EPV>(body + (i + XE_THREADS) * EPV, b);
+    online_add<EPV>(st, sx, a);
+    online_add<EPV>(st, sx, b);
+  }
+  if (i < nvec) {
+    float a[EPV];
+    load_pack<T, EPV>(body + i * EPV, a);
+    online_add<EPV>(st, sx, a);
+  }
+  if (tail0 + tid < vocab) {
+    float v[1] = {elem<T>::to_float(x[tail0 + tid])};
+    online_add<1>(st, sx, v);
+  }
+
+  // wavefront merge, then across the block's wavefronts
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) {
+    Online o{__shfl_xor(st.m, m, 64), __shfl_xor(st.s, m, 64)};
+    st = merge(st, o);
+    sx += __shfl_xor(sx, m, 64);
+  }
+  const int wave = tid / kWave, lane = tid & (kWave - 1);
+  if (lane == 0) { sm_m[wave] = st.m; sm_s[wave] = st.s; sm_x[wave] = sx; }
+  __syncthreads();
+  if (tid == 0) {
+    Online tot{sm_m[0], sm_s[0]};
+    float tx = sm_x[0];
+#pragma unroll
+    for (int w = 1; w < XE_WAVES; ++w) { tot = merge(tot, Online{sm_m[w], sm_s[w]}); tx += sm_x[w]; }
+    const float lse = tot.m + log2f(tot.s) * LN2;
+    const int64_t y = labels[row];
+    float loss = 0.f;
+    if (y != padding_idx) {
+      const float xy = (y >= 0 && y < vocab) ? elem<T>::to_float(x[y]) : 0.f;
+      loss = smoothing * (lse - tx / static_cast<float>(vocab)) + (1.f - smoothing) * (lse - xy);
+    }
+    losses[row] = loss;
+    lse_out[row] = lse;
+  }
+}
+
+template <typename T, bool VEC>
+__global__ __launch_bounds__(XE_THREADS) void xentropy_bwd_kernel(
+    const float* __restrict__ grad_loss, const T* __restrict__ logits, const float* __restrict__ lse_in,
+    const int64_t* __restrict__ labels, T* __restrict__ grad_logits, int64_t vocab, float smoothing,
+    int64_t padding_idx) {
+  constexpr int EPV = 16 / sizeof(T);
+  const int64_t row = blockIdx.x;
+  const T* x = logits + row * vocab;
+  T* dx = grad_logits + row * vocab;
+  const int tid = threadIdx.x;
+  const int64_t y = labels[row];
+  const float g = (y == padding_idx) ? 0.f : grad_loss[row];
+
+  const uintptr_t addr = reinterpret_cast<uintptr_t>(dx);
+  int64_t head = VEC ? static_cast<int64_t>(((16 - (addr & 15)) & 15) / sizeof(T)) : vocab;
+  if (head > vocab) head = vocab;
+  const int64_t nvec = (vocab - head) / EPV;
+  const int64_t tail0 = head + nvec * EPV;
+
+  if (y == padding_idx) {  // exact zeros, logits untouched
+    for (int64_t c = tid; c < head; c += XE_THREADS) dx[c] = elem<T>::from_float(0.f);
+    const float z[EPV] = {};
+    for (int64_t i = tid; i < nvec; i += XE_THREADS) store_pack<T, EPV>(dx + head + i * EPV, z);
+    for (int64_t c = tail0 + tid; c < vocab; c += XE_THREADS) dx[c] = elem<T>::from_float(0.f);
+    return;
+  }
+
+  const float nlse = -lse_in[row] * LOG2E;
+  const float sm = smoothing / static_cast<float>(vocab);
+  const float onem = 1.f - smoothing;
+  auto one = [&](int64_t c) {
+    float v = exp2f(fmaf(elem<T>::to_float(x[c]), LOG2E, nlse)) - sm;
+    if (c == y) v -= onem;
+    dx[c] = elem<T>::from_float(g * v);
+  };
+  for (int64_t c = tid; c < head; c += XE_THREADS) one(c);
+  for (int64_t i = tid; i < nvec; i += XE_THREADS) {
+    const int64_t c0 = head + i * EPV;
+    float v[EPV];
+    load_pack<T, EPV>(x + c0, v);
+#pragma unroll
+    for (int j = 0; j < EPV; ++j) v[j] = exp2f(fmaf(v[j], LOG2E, nlse)) - sm;
+    if (y >= c0 && y < c0 + EPV) {
+#pragma unroll
+      for (int j = 0; j < EPV; ++j) if (c0 + j == y) v[j] -= onem;
+    }
+#pragma unroll
+    for (int j = 0; j < EPV; ++j) v[j] *= g;
+    store_pack<T, EPV>(dx + c0, v);
+  }
+  for (int64_t c = tail0 + tid; c < vocab; c += XE_THREADS) one(c);
+}
+
+}  // namespace
+}  // namespace nmtg
+
+using namespace nmtg;
+
+extern "C" int nmtg_xentropy_fwd(const void* logits, const int64_t* labels, float* losses, float* lse, int64_t rows,
+                                 int64_t vocab, float smoothing, int64_t padding_idx, int dtype, void* stream) {
+  NMTG_REQUIRE(rows >= 0 && rows <= INT32_MAX, "xentropy_fwd: bad row count %lld", (long long)rows);
+  NMTG_REQUIRE(vocab > 0, "xentropy_fwd: number of classes must be positive");
+  if (rows == 0) return 0;
+  NMTG_REQUIRE(logits && labels && losses && lse, "xentropy_fwd: null pointer argument");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  NMTG_DISPATCH_DTYPE(dtype, T,
+                      hipLaunchKernelGGL((xentropy_fwd_kernel<T>), dim3(static_cast<unsigned>(rows)), dim3(XE_THREADS), 0,
+                                         st, static_cast<const T*>(logits), labels, losses, lse, vocab, smoothing,
+                                         padding_idx));
+  NMTG_CHECK_LAUNCH("xentropy_fwd");
+  return 0;
+}
+
+extern "C" int nmtg_xentropy_bwd(const float* grad_loss, const void* logits, const float* lse, const int64_t* labels,
+                                 void* grad_logits, int64_t rows, int64_t vocab, float smoothing, int64_t padding_idx,
+                                 int dtype, void* stream) {
+  NMTG_REQUIRE(rows >= 0 && rows <= INT32_MAX, "xentropy_bwd: bad row count %lld", (long long)rows);
+  NMTG_REQUIRE(vocab > 0, "xentropy_bwd: number of classes must be positive");
+  if (rows == 0) return 0;
+  NMTG_REQUIRE(grad_loss && logits && lse && labels && grad_logits, "xentropy_bwd: null pointer argument");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  // Vector accesses need the logits row and the gradient row to share their 16-byte phase.
+  const bool vec = ((reinterpret_cast<uintptr_t>(logits) ^ reinterpret_cast<uintptr_t>(grad_logits)) & 15u) == 0;
+  NMTG_DISPATCH_DTYPE(
+      dtype, T,
+      if (vec) hipLaunchKernelGGL((xentropy_bwd_kernel<T, true>), dim3(static_cast<unsigned>(rows)), dim3(XE_THREADS), 0, st,
+                                  grad_loss, static_cast<const T*>(logits), lse, labels, static_cast<T*>(grad_logits), vocab,
+                                  smoothing, padding_idx);
+      else hipLaunchKernelGGL((xentropy_bwd_kernel<T, false>), dim3(static_cast<unsigned>(rows)), dim3(XE_THREADS), 0, st,
+                              grad_loss, static_cast<const T*>(logits), lse, labels, static_cast<T*>(grad_logits), vocab,
+                              smoothing, padding_idx));
+  NMTG_CHECK_LAUNCH("xentropy_bwd");
+  return 0;
+}

@@ -1,0 +1,58 @@
+"""Stand-in for the reference module `xentropy_cuda`
+(onmt/modules/extensions/xentropy/interface.cpp:24-61): forward, backward, __version__.
+
+Both functions take one optional extra keyword, `padding_idx`: rows whose label equals it get a
+zero loss / zero gradient inside the kernel (the reference's Python wrapper does this afterwards
+with masked_fill_). Left at None the behaviour is the reference module's."""
+import torch
+
+from .. import _lib as L
+
+__version__ = "0.1"
+
+_NO_PAD = -(1 << 63)
+
+
+def _check(cond, msg):
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def forward(logits, labels, smoothing, half_to_float=False, *, padding_idx=None):
+    """-> [losses fp32 [N], max_log_sum_exp [N] (fp32 if half_to_float or fp32 logits)]."""
+    L.require_cuda(logits, labels)
+    if half_to_float:
+        _check(logits.dtype in (torch.float16, torch.bfloat16), "conversion is supported for Half type only")
+    _check(labels.dtype == torch.int64, "Label type should be CUDA Long")
+    _check(logits.dim() == 2, "Currently only 2 dim input supported")
+    _check(labels.dim() == 1, "Labels should be 1 dimensional")
+    _check(logits.size(0) == labels.size(0), "Input and label should have same number of examples")
+    _check(logits.numel() > 0, "Number of classes in input should not be 0")
+    logits = logits.contiguous()
+    labels = labels.contiguous()
+    n, v = logits.shape
+    losses = torch.empty(n, dtype=torch.float32, device=logits.device)
+    lse = torch.empty(n, dtype=torch.float32, device=logits.device)
+    L.call("nmtg_xentropy_fwd", L.ptr(logits), L.ptr(labels), L.ptr(losses), L.ptr(lse), L.i64(n), L.i64(v),
+           L.f32(smoothing), L.i64(_NO_PAD if padding_idx is None else padding_idx), L.i32(L.dtype_code(logits)),
+           L.stream_of(logits))
+    if not half_to_float and logits.dtype != torch.float32:
+        lse = lse.to(logits.dtype)
+    return [losses, lse]
+
+
+def backward(grad_loss, logits, max_log_sum_exp, labels, smoothing, *, padding_idx=None):
+    """-> grad_logits (logits dtype and shape)."""
+    L.require_cuda(grad_loss, logits, max_log_sum_exp, labels)
+    _check(labels.dtype == torch.int64, "Label type should be CUDA Long")
+    _check(logits.dim() == 2 and labels.dim() == 1 and logits.size(0) == labels.size(0), "shape mismatch")
+    _check(grad_loss.numel() == labels.numel() and max_log_sum_exp.numel() == labels.numel(), "shape mismatch")
+    logits = logits.contiguous()
+    grad_loss = grad_loss.contiguous().float()
+    lse = max_log_sum_exp.contiguous().float()
+    n, v = logits.shape
+    grad_logits = torch.empty_like(logits)
+    L.call("nmtg_xentropy_bwd", L.ptr(grad_loss), L.ptr(logits), L.ptr(lse), L.ptr(labels.contiguous()),
+           L.ptr(grad_logits), L.i64(n), L.i64(v), L.f32(smoothing),
+           L.i64(_NO_PAD if padding_idx is None else padding_idx), L.i32(L.dtype_code(logits)), L.stream_of(logits))
+    return grad_logits
