@@ -144,6 +144,64 @@ int nmtg_xentropy_bwd(const float* grad_loss, const void* logits, const float* l
                       const int64_t* labels, void* grad_logits, int64_t rows, int64_t vocab,
                       float smoothing, int64_t padding_idx, int dtype, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Strided-batched GEMM on the MFMA units (fp16 / bf16 in and out, fp32 accumulation), row-major:
+ *   C[b] = alpha * op(A[b]) * op(B[b]) (+ bias[n]),   op(A) is m x k, op(B) is k x n.
+ *   trans_a == 0: A stored [m, k] (lda >= k);  trans_a != 0: A stored [k, m] (lda >= m).
+ *   trans_b == 0: B stored [k, n] (ldb >= n);  trans_b != 0: B stored [n, k] (ldb >= k).
+ *   (trans_a, trans_b) = (0,1), (0,0), (1,0) are provided; these are the products the path uses.
+ * Reference: the cuBLAS / cuBLASLt calls behind the fused ops — mlp_gemm
+ *   (onmt/modules/extensions/mlp/mlp_gelu_cuda.cu:86-201), gemm_bias_lt
+ *   (multihead_attn_blaslt/gemm_blaslt.cuh:9-54) and the strided-batched wrapper
+ *   (multihead_attn_blaslt/strided_batched_gemm_blaslt.cuh:9-126); also linear_blaslt
+ *   (mlp_blaslt/linear.cpp:142-144).
+ * workspace (may be NULL): fp32 scratch of nmtg_gemm_workspace_bytes(m, n, k, batch) bytes; with
+ *   it a (1,0) product with a long reduction is split over the chip (deterministic reduction).
+ * ------------------------------------------------------------------------------------------ */
+int64_t nmtg_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k, int64_t batch);
+
+int nmtg_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alpha, const void* a,
+              int64_t lda, int64_t stride_a, const void* b, int64_t ldb, int64_t stride_b, void* c,
+              int64_t ldc, int64_t stride_c, int64_t batch, const void* bias, void* workspace,
+              int64_t workspace_bytes, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Fused MLP: y = W_n(... dropout(act(W_1 x + b_1)) ...) + b_n, nn.Linear weight layout [out, in].
+ * Reference: fused_mlp_gelu.forward / backward / backward_input_only
+ *   (onmt/modules/extensions/mlp/mlp_gelu.cpp:69-127, :129-194, :197-264), the relu / silu / agelu
+ *   siblings (mlp_relu.cpp:68-272, mlp_silu.cpp, mlp_agelu.cpp) and mlp_gelu_blaslt
+ *   (mlp_blaslt/mlp_gelu.cpp:75-242).
+ *
+ * x [batch, in_features]; weights[i] [out_features[i], in_i]; biases (array or NULL; entries may be
+ * NULL) [out_features[i]]; out [batch, out_features[n-1]].
+ * post_acts / pre_acts: the hidden layers' dropped activations / pre-activations, concatenated
+ *   layer after layer ([batch, out_features[0]], [batch, out_features[1]], ...) — the reference's
+ *   reserved_space / reserved_activations. pre_acts may be NULL (relu keeps only the output).
+ * mask: one byte per hidden activation in the same concatenated order, 1 = keep.
+ *   mask_mode 0 no dropout, 1 replay `mask`, 2 draw it from Philox (seed, offset) and store it.
+ * act: an nmtg_act code. dtype: NMTG_F16 or NMTG_BF16.
+ * ------------------------------------------------------------------------------------------ */
+int nmtg_mlp_fwd(int num_layers, const void* x, const void* const* weights,
+                 const void* const* biases, const int64_t* out_features, int64_t batch,
+                 int64_t in_features, void* out, void* post_acts, void* pre_acts, uint8_t* mask,
+                 int mask_mode, float p, uint64_t seed, uint64_t offset, int act, int dtype,
+                 void* stream);
+
+int64_t nmtg_mlp_bwd_workspace_bytes(int num_layers, const int64_t* out_features, int64_t batch,
+                                     int64_t in_features);
+
+/* grad_x may be NULL (the reference skips it when x does not require grad); grad_weights /
+ * grad_biases may be NULL or hold NULL entries (backward_input_only). mask NULL or p == 0: no
+ * dropout. With pre_acts == NULL and act == relu the gradient gate is taken from the dropped
+ * output (mlp_relu_cuda.cu:1174-1240). workspace: nmtg_mlp_bwd_workspace_bytes(...) bytes,
+ * 256-byte aligned. */
+int nmtg_mlp_bwd(int num_layers, const void* x, const void* const* weights,
+                 const int64_t* out_features, int64_t batch, int64_t in_features,
+                 const void* grad_out, const void* post_acts, const void* pre_acts,
+                 const uint8_t* mask, float p, int act, void* grad_x, void* const* grad_weights,
+                 void* const* grad_biases, void* workspace, int64_t workspace_bytes, int dtype,
+                 void* stream);
+
 #ifdef __cplusplus
 }
 #endif

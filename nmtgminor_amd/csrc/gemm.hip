@@ -1,0 +1,185 @@
+// Host side of the MFMA GEMM core: tile / split selection, alignment analysis, the column-sum
+// (bias gradient) helpers and the stand-alone C entry point nmtg_gemm.
+#include "gemm_inst.cuh"
+#include <algorithm>
+
+namespace nmtg {
+
+bool gemm_has(int layout, int tile, int epi) {
+  if (layout == LAYOUT_NT)
+    return (tile == TILE_L || tile == TILE_M) && (epi == EPI_PLAIN || epi == EPI_ACT_FWD || epi == EPI_SCORES);
+  if (layout == LAYOUT_NN) {
+    if (epi == EPI_PLAIN) return true;
+    return epi == EPI_ACT_BWD && (tile == TILE_L || tile == TILE_M);
+  }
+  if (layout == LAYOUT_TN) {
+    if (epi == EPI_PLAIN) return tile == TILE_M || tile == TILE_S;
+    return epi == EPI_SPLITK && (tile == TILE_L || tile == TILE_M);
+  }
+  return false;
+}
+
+namespace {
+
+int vec_of(const void* p, int64_t ld, int64_t batch_stride, int batch) {
+  const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+  auto ok = [&](int v) {
+    return a % (2 * v) == 0 && ld % v == 0 && (batch <= 1 || batch_stride % v == 0);
+  };
+  if (ok(8)) return 8;
+  if (ok(4)) return 4;
+  return 1;
+}
+
+int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+struct SplitPlan {
+  int tile, splits, k_per_split;
+};
+
+// Weight-gradient style products (small output, long reduction): spread the reduction over
+// enough blocks to occupy the chip; partial tiles go through an fp32 workspace.
+SplitPlan plan_splitk(int M, int N, int K, int batch) {
+  const int cus = num_cus();
+  SplitPlan p{TILE_M, 1, ceil_div(K, GEMM_BK) * GEMM_BK};
+  const int tiles_l = ceil_div(M, 256) * ceil_div(N, 256) * batch;
+  const int tiles_m = ceil_div(M, 128) * ceil_div(N, 128) * batch;
+  // prefer the large tile when it alone offers >= 1/8 of the chip (then <= 8-way split)
+  int tiles;
+  if (tiles_l * 8 >= cus) { p.tile = TILE_L; tiles = tiles_l; }
+  else { p.tile = TILE_M; tiles = tiles_m; }
+  int splits = std::max(1, (cus + tiles / 2) / tiles);
+  const int max_splits = std::max(1, K / (4 * GEMM_BK));  // at least 4 reduction steps per block
+  splits = std::min(splits, max_splits);
+  p.k_per_split = ceil_div(ceil_div(K, splits), GEMM_BK) * GEMM_BK;
+  p.splits = ceil_div(K, p.k_per_split);
+  return p;
+}
+
+size_t splitk_ws_bytes(const SplitPlan& p, int M, int N, int batch) {
+  int bm, bn;
+  tile_dims(p.tile, bm, bn);
+  const size_t area = static_cast<size_t>(ceil_div(M, bm)) * bm * ceil_div(N, bn) * bn;
+  return area * batch * p.splits * sizeof(float);
+}
+
+}  // namespace
+
+size_t gemm_splitk_workspace_bytes(int M, int N, int K, int batch) {
+  const SplitPlan p = plan_splitk(M, N, K, batch);
+  return splitk_ws_bytes(p, M, N, batch);
+}
+
+int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t workspace_bytes, hipStream_t st,
+             int* m_tiles_out) {
+  if (m_tiles_out) *m_tiles_out = 0;
+  if (a.M <= 0 || a.N <= 0 || a.batch <= 0) return 0;
+  if (a.K < 0) return fail(NMTG_ERR_INVALID, "gemm: negative K");
+  if (!a.A || !a.B || !a.C) return fail(NMTG_ERR_INVALID, "gemm: null operand pointer");
+  const bool a_kc = layout != LAYOUT_TN;
+  const bool b_kc = layout == LAYOUT_NT;
+  (void)a_kc; (void)b_kc;
+  a.a_vec = vec_of(a.A, a.lda, a.sA, a.batch);
+  a.b_vec = vec_of(a.B, a.ldb, a.sB, a.batch);
+  a.c_vec = vec_of(a.C, a.ldc, a.sC, a.batch);
+  if (a.aux_out) a.c_vec = std::min(a.c_vec, vec_of(a.aux_out, a.ldc, a.sC, a.batch));
+  if (a.aux_in) a.c_vec = std::min(a.c_vec, vec_of(a.aux_in, a.ld_aux, 0, 1));
+
+  int tile = -1;
+  a.splits = 1;
+  a.k_per_split = ceil_div(std::max(a.K, 1), GEMM_BK) * GEMM_BK;
+
+  if (layout == LAYOUT_TN && epi == EPI_PLAIN && workspace != nullptr) {
+    const SplitPlan p = plan_splitk(a.M, a.N, a.K, a.batch);
+    if (p.splits > 1 && splitk_ws_bytes(p, a.M, a.N, a.batch) <= workspace_bytes &&
+        (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0) {
+      epi = EPI_SPLITK;
+      tile = p.tile;
+      a.splits = p.splits;
+      a.k_per_split = p.k_per_split;
+      a.ws = static_cast<float*>(workspace);
+    }
+  }
+  if (tile < 0) {
+    const int cus = num_cus();
+    const int64_t cnt_l = static_cast<int64_t>(ceil_div(a.M, 256)) * ceil_div(a.N, 256) * a.batch;
+    if (a.N <= 64 && gemm_has(layout, TILE_S, epi)) tile = TILE_S;
+    else if (cnt_l * 4 >= cus * 3 && gemm_has(layout, TILE_L, epi)) tile = TILE_L;
+    else if (gemm_has(layout, TILE_M, epi)) tile = TILE_M;
+    else if (gemm_has(layout, TILE_L, epi)) tile = TILE_L;
+    else tile = TILE_S;
+  }
+  if (!gemm_has(layout, tile, epi))
+    return fail(NMTG_ERR_UNSUPPORTED, "gemm: layout %d has no kernel for epilogue %d", layout, epi);
+  int bm, bn;
+  tile_dims(tile, bm, bn);
+  a.m_tiles = ceil_div(a.M, bm);
+  a.n_tiles = ceil_div(a.N, bn);
+  if (m_tiles_out) *m_tiles_out = a.m_tiles;
+  if (static_cast<int64_t>(a.m_tiles) * a.n_tiles > 0x7fffffff || a.batch > 65535)
+    return fail(NMTG_ERR_UNSUPPORTED, "gemm: grid too large (tiles %d x %d, batch %d)", a.m_tiles, a.n_tiles, a.batch);
+  int rc;
+  if (layout == LAYOUT_NT) rc = gemm_launch_nt(dtype, tile, epi, a, st);
+  else if (layout == LAYOUT_NN) rc = gemm_launch_nn(dtype, tile, epi, a, st);
+  else rc = gemm_launch_tn(dtype, tile, epi, a, st);
+  if (rc) return rc;
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(NMTG_ERR_LAUNCH, "gemm: launch failed: %s", hipGetErrorString(e));
+  return 0;
+}
+
+int colsum_parts(int M) { return std::max(1, std::min(64, ceil_div(M, 128))); }
+
+int colsum_finish(int dtype, const float* part, int parts, int N, void* out, hipStream_t st) {
+  NMTG_DISPATCH_DTYPE(dtype, T,
+                      hipLaunchKernelGGL((colsum_final_kernel<T>), dim3(ceil_div(N, 256)), dim3(256), 0, st, part, parts, N,
+                                         static_cast<T*>(out)));
+  NMTG_CHECK_LAUNCH("colsum_finish");
+  return 0;
+}
+
+int colsum_run(int dtype, const void* X, int64_t ld, int M, int N, float* part, void* out, hipStream_t st) {
+  const int parts = colsum_parts(M);
+  const int rpb = ceil_div(M, parts);
+  NMTG_DISPATCH_DTYPE(dtype, T,
+                      hipLaunchKernelGGL((colsum_partial_kernel<T>), dim3(ceil_div(N, 64), parts), dim3(256), 0, st,
+                                         static_cast<const T*>(X), ld, M, N, rpb, part));
+  NMTG_CHECK_LAUNCH("colsum");
+  return colsum_finish(dtype, part, parts, N, out, st);
+}
+
+}  // namespace nmtg
+
+using namespace nmtg;
+
+extern "C" int64_t nmtg_gemm_workspace_bytes(int64_t m, int64_t n, int64_t k, int64_t batch) {
+  if (m <= 0 || n <= 0 || k <= 0 || batch <= 0 || m > INT32_MAX || n > INT32_MAX || k > INT32_MAX) return 0;
+  return static_cast<int64_t>(gemm_splitk_workspace_bytes(static_cast<int>(m), static_cast<int>(n), static_cast<int>(k),
+                                                          static_cast<int>(batch)));
+}
+
+extern "C" int nmtg_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alpha, const void* a, int64_t lda,
+                         int64_t stride_a, const void* b, int64_t ldb, int64_t stride_b, void* c, int64_t ldc,
+                         int64_t stride_c, int64_t batch, const void* bias, void* workspace, int64_t workspace_bytes,
+                         int dtype, void* stream) {
+  NMTG_REQUIRE(m >= 0 && n >= 0 && k >= 0 && batch >= 0 && m <= INT32_MAX && n <= INT32_MAX && k <= INT32_MAX &&
+                   batch <= 65535,
+               "gemm: bad shape m=%lld n=%lld k=%lld batch=%lld", (long long)m, (long long)n, (long long)k, (long long)batch);
+  int layout;
+  if (!trans_a && trans_b) layout = LAYOUT_NT;
+  else if (!trans_a && !trans_b) layout = LAYOUT_NN;
+  else if (trans_a && !trans_b) layout = LAYOUT_TN;
+  else return fail(NMTG_ERR_UNSUPPORTED, "gemm: A^T B^T is not provided (no caller on this path needs it)");
+  GemmArgs g{};
+  g.A = a; g.B = b; g.C = c;
+  g.lda = lda; g.ldb = ldb; g.ldc = ldc;
+  g.sA = stride_a; g.sB = stride_b; g.sC = stride_c;
+  g.M = static_cast<int>(m); g.N = static_cast<int>(n); g.K = static_cast<int>(k);
+  g.batch = static_cast<int>(batch);
+  g.alpha = alpha;
+  g.bias = bias;
+  // leading dimensions must cover the contiguous extent
+  NMTG_REQUIRE(lda >= (trans_a ? m : k) && ldb >= (trans_b ? k : n) && ldc >= n, "gemm: leading dimension too small");
+  return gemm_run(dtype, layout, EPI_PLAIN, g, workspace, static_cast<size_t>(std::max<int64_t>(0, workspace_bytes)),
+                  static_cast<hipStream_t>(stream));
+}

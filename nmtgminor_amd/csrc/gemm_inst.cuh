@@ -1,0 +1,58 @@
+// Per-layout instantiation units of the GEMM kernel (one translation unit per operand layout so
+// they compile in parallel). Tile configurations:
+//   L: 256x256 tile, 2x4 wavefronts (each 128x64), 512 threads  — large outputs
+//   M: 128x128 tile, 2x2 wavefronts (each 64x64),  256 threads  — outputs too small to fill the chip with L
+//   S: 256x64  tile, 4x1 wavefronts (each 64x64),  256 threads  — N <= 64 (per-head attention products)
+#pragma once
+#include "gemm.cuh"
+
+namespace nmtg {
+
+enum GemmTile { TILE_L = 0, TILE_M = 1, TILE_S = 2 };
+
+template <int TILE> struct tile_cfg;
+template <> struct tile_cfg<TILE_L> { static constexpr int BM = 256, BN = 256, WM = 2, WN = 4; };
+template <> struct tile_cfg<TILE_M> { static constexpr int BM = 128, BN = 128, WM = 2, WN = 2; };
+template <> struct tile_cfg<TILE_S> { static constexpr int BM = 256, BN = 64, WM = 4, WN = 1; };
+
+inline void tile_dims(int tile, int& bm, int& bn) {
+  if (tile == TILE_L) { bm = 256; bn = 256; }
+  else if (tile == TILE_M) { bm = 128; bn = 128; }
+  else { bm = 256; bn = 64; }
+}
+
+template <typename T, int TILE, bool A_KC, bool B_KC, int EPI>
+int gemm_launch_one(const GemmArgs& a, hipStream_t st) {
+  using C = tile_cfg<TILE>;
+  auto kern = gemm_kernel<T, C::BM, C::BN, C::WM, C::WN, A_KC, B_KC, EPI>;
+  constexpr int lds = gemm_lds_bytes<C::BM, C::BN>();
+  static bool attr_done = false;
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return fail(NMTG_ERR_LAUNCH, "gemm: cannot reserve %d bytes of LDS: %s", lds, hipGetErrorString(e));
+    attr_done = true;
+  }
+  dim3 grid(a.m_tiles * a.n_tiles, a.batch, a.splits);
+  hipLaunchKernelGGL(kern, grid, dim3(64 * C::WM * C::WN), lds, st, a);
+  return 0;
+}
+
+template <typename T, int TILE>
+int splitk_reduce_launch(const GemmArgs& a, hipStream_t st) {
+  using C = tile_cfg<TILE>;
+  constexpr int per_blk = C::WM * C::WN * (C::BM / C::WM / 32) * (C::BN / C::WN / 32) * 4 * 64;
+  const int64_t total = static_cast<int64_t>(a.batch) * a.m_tiles * a.n_tiles * per_blk;
+  hipLaunchKernelGGL((splitk_reduce_kernel<T, C::BM, C::BN, C::WM, C::WN>), dim3(static_cast<unsigned>((total + 255) / 256)),
+                     dim3(256), 0, st, a.ws, static_cast<T*>(a.C), a.ldc, a.M, a.N, a.m_tiles, a.n_tiles, a.batch, a.sC,
+                     a.splits, a.alpha, a.c_vec);
+  return 0;
+}
+
+// Defined in gemm_nt.hip / gemm_nn.hip / gemm_tn.hip. Return NMTG_ERR_UNSUPPORTED for a
+// (tile, epilogue) pair that is not instantiated.
+int gemm_launch_nt(int dtype, int tile, int epi, const GemmArgs& a, hipStream_t st);
+int gemm_launch_nn(int dtype, int tile, int epi, const GemmArgs& a, hipStream_t st);
+int gemm_launch_tn(int dtype, int tile, int epi, const GemmArgs& a, hipStream_t st);
+bool gemm_has(int layout, int tile, int epi);
+
+}  // namespace nmtg

@@ -482,9 +482,9 @@ using namespace nmtg;
 extern "C" int nmtg_ln_fwd(const void* x, const void* gamma, const void* beta, void* z, float* mu,
                            float* rsigma, int64_t rows, int64_t hidden, float eps, int in_dtype,
                            int w_dtype, void* stream) {
-  NMTG_REQUIRE(x && gamma && beta && z && mu && rsigma, "ln_fwd: null pointer argument");
   NMTG_REQUIRE(rows >= 0 && hidden > 0 && hidden <= (1 << 30), "ln_fwd: bad shape rows=%lld hidden=%lld",
                (long long)rows, (long long)hidden);
+  NMTG_REQUIRE(rows == 0 || (x && gamma && beta && z && mu && rsigma), "ln_fwd: null pointer argument");
   NMTG_REQUIRE(eps >= 0.f, "ln_fwd: epsilon must be >= 0");
   NMTG_REQUIRE(ln_pair_ok(in_dtype, w_dtype), "ln_fwd: unsupported dtype pair in=%d weight=%d", in_dtype, w_dtype);
   if (rows == 0) return 0;
@@ -512,9 +512,9 @@ extern "C" int nmtg_ln_bwd(const void* dz, const void* x_or_z, const float* mu, 
                            float* dgamma_part, float* dbeta_part, int64_t n_part, int64_t rows,
                            int64_t hidden, int memory_efficient, int in_dtype, int w_dtype,
                            void* stream) {
-  NMTG_REQUIRE(dz && x_or_z && rsigma && gamma && dx && dgamma && dbeta && dgamma_part && dbeta_part,
-               "ln_bwd: null pointer argument");
-  NMTG_REQUIRE(memory_efficient ? beta != nullptr : mu != nullptr,
+  NMTG_REQUIRE(gamma && dgamma && dbeta && dgamma_part && dbeta_part, "ln_bwd: null pointer argument");
+  NMTG_REQUIRE(rows == 0 || (dz && x_or_z && rsigma && dx), "ln_bwd: null pointer argument");
+  NMTG_REQUIRE(rows == 0 || (memory_efficient ? beta != nullptr : mu != nullptr),
                "ln_bwd: %s is required", memory_efficient ? "beta (memory_efficient)" : "mu");
   NMTG_REQUIRE(rows >= 0 && hidden > 0 && hidden <= (1 << 30), "ln_bwd: bad shape rows=%lld hidden=%lld",
                (long long)rows, (long long)hidden);

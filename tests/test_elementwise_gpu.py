@@ -88,7 +88,7 @@ def test_dropout_add_autograd_wrapper(dev):
 # ----------------------------------------------------------------------------- masked softmax
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("bh,tq,tk", [(8, 75, 56), (6, 5, 1), (4, 64, 512), (4, 17, 1500), (2, 128, 128),
-                                      (2, 9, 2048), (3, 7, 333), (2, 3, 4096)])
+                                      (2, 9, 2048), (4, 7, 333), (2, 3, 4096)])
 def test_softmax_dropout_fwd_bwd(dev, dtype, bh, tq, tk):
     if tk == 4096 and dtype == torch.float32:
         pytest.skip("4096 keys is the 16-bit limit")
@@ -194,8 +194,9 @@ def _xent_case(dev, n, v, dtype, eps, pad, seed=51, misalign=0):
     if big.any() and dtype != torch.float32:
         rel = ((dx.cpu().to(D) - dxo).abs() / dxo.abs())[big].max().item()
         assert rel < 2e-2, rel
-    rows = dx.cpu().to(D)[~padrows].sum(1).abs().max().item()
-    assert rows < (1e-5 if dtype == torch.float32 else 5e-2)                            # each row sums to ~0
+    if (~padrows).any():
+        rows = dx.cpu().to(D)[~padrows].sum(1).abs().max().item()
+        assert rows < (1e-5 if dtype == torch.float32 else 5e-2)                        # each row sums to ~0
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

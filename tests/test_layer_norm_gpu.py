@@ -59,7 +59,7 @@ def test_dtype_pairs(dev, dtype, wdtype, hidden):
     _run(130, hidden, dtype, wdtype, dev)
 
 
-@pytest.mark.parametrize("hidden", [1, 3, 100, 513, 1000, 20000])
+@pytest.mark.parametrize("hidden", [2, 3, 100, 513, 1000, 20000])
 def test_odd_hidden_sizes_take_the_generic_kernel(dev, hidden):
     _run(37, hidden, torch.float32, torch.float32, dev)
     _run(37, hidden, torch.bfloat16, torch.bfloat16, dev)
@@ -81,6 +81,8 @@ def test_empty_input(dev):
     g = torch.ones(512, device=dev)
     z, mu, rs = fast_layer_norm_cuda.ln_fwd(x, g, g, 1e-5)
     assert z.shape == (0, 512) and mu.numel() == 0
+    dx, dg, db, _, _ = fast_layer_norm_cuda.ln_bwd(x, x, mu, rs, g, None, False)
+    assert dx.shape == (0, 512) and (dg == 0).all() and (db == 0).all()
 
 
 def test_argument_errors_raise(dev):
