@@ -33,7 +33,7 @@ namespace nmtg {
 enum GemmEpi {
   EPI_PLAIN = 0,    // C = alpha*acc (+ bias[n])
   EPI_ACT_FWD = 1,  // h = acc + bias -> aux_out;  C = act(h) * keep * dscale
-  EPI_ACT_BWD = 2,  // C = acc * act'(aux_in) * keep * dscale;  colsum_part[m_tile][n] = sum_m C
+  EPI_ACT_BWD = 2,  // C = T(acc) * act'(aux_in) * dscale * keep (keep = 1 without a mask);  colsum_part[m_tile][n] = sum_m C
   EPI_SCORES = 3,   // C = alpha*acc, -inf where the key-padding / time mask is set
   EPI_SPLITK = 4    // fp32 partial tile -> workspace (reduced by splitk_reduce_kernel)
 };
@@ -428,14 +428,14 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const Gemm
           float h[8];
           load8(static_cast<const T*>(g.aux_in) + static_cast<int64_t>(m) * g.ld_aux + n, h);
 #pragma unroll
-          for (int k = 0; k < 8; ++k) v[k] *= act_grad(h[k], g.act);
+          for (int k = 0; k < 8; ++k) v[k] *= act_grad(h[k], g.act) * g.dscale;
           if (g.dmask != nullptr) {
             const uint8_t* mk = g.dmask + static_cast<int64_t>(m) * g.N + n;
             uint8_t keep[8];
             if (nvalid == 8 && (g.N & 7) == 0) load_bytes<8>(mk, keep);
             else for (int k = 0; k < 8; ++k) keep[k] = k < nvalid ? mk[k] : 0;
 #pragma unroll
-            for (int k = 0; k < 8; ++k) v[k] = keep[k] ? v[k] * g.dscale : 0.f;
+            for (int k = 0; k < 8; ++k) v[k] = keep[k] ? v[k] : 0.f;
           }
           // the bias gradient sums the values as stored (rounded to T), as the reference does
 #pragma unroll

@@ -191,10 +191,11 @@ extern "C" int nmtg_mlp_bwd(int num_layers, const void* x, const void* const* we
       g.aux_in = have_pre ? static_cast<const uint8_t*>(pre_acts) + offs[i - 1] * 2
                           : static_cast<const uint8_t*>(post_acts) + offs[i - 1] * 2;
       g.ld_aux = in_i;
+      g.dscale = 1.f;
       if (have_pre) {
         if (mask != nullptr && p > 0.f) { g.dmask = mask + offs[i - 1]; g.dscale = 1.f / (1.f - p); }
       } else if (p > 0.f) {
-        g.alpha = 1.f / (1.f - p);  // relu from the dropped output: a > 0 iff kept and h > 0
+        g.dscale = 1.f / (1.f - p);  // relu from the dropped output: a > 0 iff kept and h > 0
       }
       // one partial row per row tile of the GEMM
       g.colsum_part = (grad_biases && grad_biases[i - 1]) ? colsum_ws : nullptr;

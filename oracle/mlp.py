@@ -48,9 +48,16 @@ def act_bwd(h, act):
     raise ValueError(act)
 
 
-def mlp_fwd(x, weights, biases, act, p=0.0, masks=None, ctype=torch.float32):
+def _round(t, round_to):
+    """The fallback materialises its intermediate tensors in the working dtype (fp16 / bf16);
+    round_to reproduces those rounding points, the arithmetic in between stays in ctype."""
+    return t if round_to is None else t.to(round_to).to(t.dtype)
+
+
+def mlp_fwd(x, weights, biases, act, p=0.0, masks=None, ctype=torch.float32, round_to=None):
     """x [N, in]; weights[i] [out_i, in_i]; biases[i] [out_i] or None; masks[i] uint8 [N, out_i]
-    for every hidden layer (None / p == 0: no dropout).
+    for every hidden layer (None / p == 0: no dropout). round_to: dtype in which the fallback
+    stores the pre- and post-activations (None: keep full precision).
     -> (y, pre_acts [h_1..h_{n-1}], post_acts [a_1..a_{n-1}])."""
     a = x.to(ctype)
     n = len(weights)
@@ -61,15 +68,18 @@ def mlp_fwd(x, weights, biases, act, p=0.0, masks=None, ctype=torch.float32):
             h = h + biases[i].to(ctype)
         if i == n - 1:
             return h, pre, post
+        h = _round(h, round_to)
         pre.append(h)
         a = act_fwd(h, act)
         if masks is not None and p > 0.0:
             a = a * masks[i].to(ctype) / (1.0 - p)
+        a = _round(a, round_to)
         post.append(a)
 
 
-def mlp_bwd(dy, x, weights, pre, post, act, p=0.0, masks=None, ctype=torch.float32):
-    """-> (dx, [dW_1..dW_n], [db_1..db_n]) from the saved pre / post activations."""
+def mlp_bwd(dy, x, weights, pre, post, act, p=0.0, masks=None, ctype=torch.float32, round_to=None):
+    """-> (dx, [dW_1..dW_n], [db_1..db_n]) from the saved pre / post activations. round_to: dtype
+    in which the fallback stores the hidden-layer gradients."""
     n = len(weights)
     g = dy.to(ctype)
     dws, dbs = [None] * n, [None] * n
@@ -79,7 +89,9 @@ def mlp_bwd(dy, x, weights, pre, post, act, p=0.0, masks=None, ctype=torch.float
         dws[i] = g.t() @ inp
         g = g @ weights[i].to(ctype)
         if i > 0:
+            g = _round(g, round_to)
             g = g * act_bwd(pre[i - 1].to(ctype), act)
             if masks is not None and p > 0.0:
                 g = g * masks[i - 1].to(ctype) / (1.0 - p)
+            g = _round(g, round_to)
     return g, dws, dbs
