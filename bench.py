@@ -1,0 +1,345 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused transformer-layer ops on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME|all] [--no-cpu]
+
+A "step" is one forward+backward pass (forward only where the workload says so) of one op over
+one batch of seeded synthetic input already resident in HBM. The headline line is the fused-MLP
+workload (MFMA TFLOP/s); with `--workload all` (the default) the other benchmark workloads are
+measured too and reported under "others", each with its own roofline and CPU baseline.
+
+Timing: W warm-up steps, then exactly K steps replayed from a HIP graph of one step, bracketed by
+device synchronisation; per-kernel durations come from HIP events the library records around
+each launch (nmtg_trace_begin/end) in a separate eager pass, so they can be compared with a
+rocprofv3 kernel trace of the same command. The CPU baseline is the CPU oracle (oracle/, a
+restatement of the reference's PyTorch fallback) on the host cores, on a bounded sample.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published
+MFMA_PEAK_TFLOPS = 2500.0       # MI355X dense bf16 / fp16 MFMA, published
+
+
+def _sync():
+    torch.cuda.synchronize()
+
+
+class Workload:
+    name = ""
+    bound = "hbm"               # or "mfma"
+    dtype = "f32"
+    description = ""
+    data = "synthetic"
+
+    def setup(self, dev):
+        raise NotImplementedError
+
+    def step(self):
+        raise NotImplementedError
+
+    def work_per_step(self):    # bytes (hbm) or flops (mfma), algorithmic
+        raise NotImplementedError
+
+    def kernel_work(self):      # {kernel-name prefix: algorithmic work of ONE launch group per step}
+        return {}
+
+    def cpu_baseline(self):     # -> dict(value, unit, cores, kind, sample)
+        return None
+
+    @property
+    def unit(self):
+        return "GB/s" if self.bound == "hbm" else "TFLOP/s"
+
+    @property
+    def peak(self):
+        return HBM_PEAK_GBS if self.bound == "hbm" else MFMA_PEAK_TFLOPS
+
+    def rate(self, work, seconds):
+        return work / seconds / (1e9 if self.bound == "hbm" else 1e12)
+
+
+def _time_cpu(fn, reps=3):
+    fn()
+    ts = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t0)
+    ts.sort()
+    return ts[len(ts) // 2]
+
+
+class LayerNormWL(Workload):
+    name = "layer_norm"
+    bound = "hbm"
+    dtype = "f32"
+    description = "LayerNorm fwd+bwd fp32 [4096 x 512], eps 1e-5"
+
+    def setup(self, dev):
+        from oracle import inputs
+        from nmtgminor_amd.native import fast_layer_norm_cuda as ln
+        self.ln = ln
+        self.cpu = inputs.layer_norm_inputs()
+        d = self.cpu
+        self.x, self.g, self.b, self.dy = (d[k].to(dev) for k in ("x", "gamma", "beta", "dy"))
+        self.rows, self.h = self.x.shape
+
+    def step(self):
+        z, mu, rs = self.ln.ln_fwd(self.x, self.g, self.b, 1e-5)
+        return self.ln.ln_bwd(self.dy, self.x, mu, rs, self.g, None, False)
+
+    def _bytes(self):
+        t = self.rows * self.h * 4
+        fwd = 2 * t + 2 * self.h * 4 + 2 * self.rows * 4
+        bwd = 3 * t + 2 * self.rows * 4 + 3 * self.h * 4
+        return fwd, bwd
+
+    def work_per_step(self):
+        return sum(self._bytes())
+
+    def kernel_work(self):
+        fwd, bwd = self._bytes()
+        return {"ln_fwd": fwd, "ln_bwd": bwd}
+
+    def cpu_baseline(self):
+        from oracle import layer_norm as o
+        d = self.cpu
+
+        def run():
+            z, mu, rs = o.ln_fwd(d["x"], d["gamma"], d["beta"], d["eps"])
+            o.ln_bwd(d["dy"], d["x"], mu, rs, d["gamma"])
+        t = _time_cpu(run, 5)
+        return dict(value=self.work_per_step() / t / 1e9, unit="GB/s", cores=torch.get_num_threads(), kind="port",
+                    sample="full workload (4096 x 512 fp32 fwd+bwd), median of 5")
+
+
+class MlpWL(Workload):
+    name = "mlp"
+    bound = "mfma"
+    dtype = "f16"
+    description = "fused MLP fwd+bwd fp16: x [8192 x 512], 512->2048->512, gelu, dropout 0.1 (explicit mask)"
+
+    def setup(self, dev):
+        from oracle import inputs
+        from nmtgminor_amd.native import fused_mlp_gelu as m
+        self.m = m
+        self.cpu = inputs.mlp_inputs()
+        d = self.cpu
+        self.ins = [d[k].to(dev) for k in ("x", "w1", "w2", "b1", "b2")]
+        self.ins[0].requires_grad_()
+        self.mask = d["mask"].to(dev)
+        self.dy = d["dy"].to(dev)
+
+    def step(self):
+        out = self.m.forward(0.1, self.ins, self.mask)
+        return self.m.backward(0.1, self.dy, out, self.ins)
+
+    def work_per_step(self):
+        return 6 * 2.0 * 8192 * 512 * 2048
+
+    def kernel_work(self):
+        return {"gemm_": self.work_per_step()}
+
+    def cpu_baseline(self):
+        from oracle import mlp as o
+        d = self.cpu
+        ws, bs = [d["w1"].float(), d["w2"].float()], [d["b1"].float(), d["b2"].float()]
+        x, dy = d["x"].float(), d["dy"].float()
+
+        def run():
+            y, pre, post = o.mlp_fwd(x, ws, bs, "gelu", 0.1, [d["mask"]])
+            o.mlp_bwd(dy, x, ws, pre, post, "gelu", 0.1, [d["mask"]])
+        t = _time_cpu(run, 3)
+        return dict(value=self.work_per_step() / t / 1e12, unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
+                    sample="full workload in fp32 on the fp16-rounded values, median of 3")
+
+
+class XentropyWL(Workload):
+    name = "xentropy"
+    bound = "hbm"
+    dtype = "bf16"
+    description = ("label-smoothed cross-entropy fwd+bwd: bf16 logits [16384 x 250054], eps 0.1, "
+                   "10% padding (idx 1), fp32 accumulation")
+    data = "synthetic (logits drawn on the GPU by torch's Philox generator, seed 1005; targets from the seeded CPU generator)"
+    rows, vocab = 16384, 250054
+
+    def setup(self, dev):
+        from oracle import inputs
+        from nmtgminor_amd.native import xentropy_cuda as xe
+        self.xe = xe
+        d = inputs.xentropy_inputs(self.rows, self.vocab, with_logits=False)
+        self.labels_cpu = d["labels"]
+        self.labels = d["labels"].to(dev)
+        self.grad = d["grad_loss"].to(dev)
+        g = torch.Generator(device=dev)
+        g.manual_seed(1005)
+        self.logits = torch.empty(self.rows, self.vocab, dtype=torch.bfloat16, device=dev)
+        chunk = 1024
+        for r in range(0, self.rows, chunk):
+            self.logits[r:r + chunk] = (2.0 * torch.randn(chunk, self.vocab, generator=g, device=dev)).to(torch.bfloat16)
+        self.grad_logits = None
+
+    def step(self):
+        losses, lse = self.xe.forward(self.logits, self.labels, 0.1, True, padding_idx=1)
+        g = self.xe.backward(self.grad, self.logits, lse, self.labels, 0.1, padding_idx=1)
+        return losses, g
+
+    def _tensor_bytes(self):
+        return self.rows * self.vocab * 2
+
+    def work_per_step(self):
+        return 3 * self._tensor_bytes()
+
+    def kernel_work(self):
+        return {"xentropy_fwd": self._tensor_bytes(), "xentropy_bwd": 2 * self._tensor_bytes()}
+
+    def cpu_baseline(self):
+        from oracle import xentropy as o
+        n = 256
+        x = self.logits[:n].float().cpu()
+        y = self.labels_cpu[:n]
+        gl = torch.ones(n)
+
+        def run():
+            loss, lse = o.xentropy_fwd(x, y, 0.1, 1)
+            o.xentropy_bwd(gl, x, lse, y, 0.1, 1)
+        t = _time_cpu(run, 3)
+        return dict(value=3 * n * self.vocab * 2 / t / 1e9, unit="GB/s", cores=torch.get_num_threads(), kind="port",
+                    sample=f"first {n} of {self.rows} rows, fp32 on the bf16-rounded logits, algorithmic bf16 bytes / time, median of 3")
+
+
+WORKLOADS = {w.name: w for w in (LayerNormWL, MlpWL, XentropyWL)}
+try:
+    from _bench_attention import ATTENTION_WORKLOADS   # added with the attention ops
+    WORKLOADS.update(ATTENTION_WORKLOADS)
+except ImportError:
+    pass
+PRIMARY = "mlp"
+
+
+def measure(w, dev, steps, warmup, do_cpu, trace_steps):
+    from nmtgminor_amd import _lib
+    w.setup(dev)
+    for _ in range(max(1, warmup)):
+        w.step()
+    _sync()
+    # one step captured into a HIP graph, replayed K times
+    graph = None
+    try:
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            w.step()
+            _sync()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=s):
+                w.step()
+        _sync()
+        graph.replay()
+        _sync()
+    except Exception as e:  # pragma: no cover - falls back to eager launches
+        sys.stderr.write(f"[bench] {w.name}: graph capture failed ({e}); timing eager launches\n")
+        graph = None
+    _sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        if graph is not None:
+            graph.replay()
+        else:
+            w.step()
+    _sync()
+    wall = time.perf_counter() - t0
+    per_step = wall / steps
+    # per-kernel durations (HIP events around every launch, eager pass)
+    _lib.trace_begin()
+    for _ in range(trace_steps):
+        w.step()
+    _sync()
+    tr = _lib.trace_end()
+    kernels = []
+    for name, (cnt, ms) in sorted(tr.items(), key=lambda kv: -kv[1][1]):
+        kernels.append(dict(name=name, launches_per_step=cnt / trace_steps, avg_us=ms / cnt * 1e3,
+                            us_per_step=ms / trace_steps * 1e3))
+    roof = None
+    best = None
+    for prefix, work in w.kernel_work().items():
+        sel = [k for k in kernels if k["name"].startswith(prefix)]
+        if not sel:
+            continue
+        us = sum(k["us_per_step"] for k in sel)
+        if best is None or us > best[0]:
+            best = (us, prefix, work, sel)
+    if best is not None:
+        us, prefix, work, sel = best
+        achieved = w.rate(work, us * 1e-6)
+        launches = sum(k["launches_per_step"] for k in sel)
+        roof = dict(bound=w.bound, achieved=round(achieved, 3), peak=w.peak, unit=w.unit, frac=round(achieved / w.peak, 4),
+                    traffic=None, kernel=(prefix + "*" if prefix.endswith("_") else prefix), launches_per_step=launches,
+                    avg_launch_us=round(us / launches, 3), work_per_step=work)
+    res = dict(workload=w.name, description=w.description, metric="achieved HBM GB/s" if w.bound == "hbm" else "MFMA TFLOP/s",
+               value=round(w.rate(w.work_per_step(), per_step), 3), unit=w.unit, ms_per_step=round(per_step * 1e3, 5),
+               frac_of_peak=round(w.rate(w.work_per_step(), per_step) / w.peak, 4), dtype=w.dtype, data=w.data,
+               timed="hip graph replay" if graph is not None else "eager launches", roofline=roof,
+               kernels=[dict(name=k["name"], launches_per_step=k["launches_per_step"], avg_us=round(k["avg_us"], 3))
+                        for k in kernels])
+    res["cpu_baseline"] = w.cpu_baseline() if do_cpu else None
+    if res["cpu_baseline"]:
+        res["cpu_baseline"]["value"] = round(res["cpu_baseline"]["value"], 4)
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="all", help="one of %s, or all" % ", ".join(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--trace-steps", type=int, default=10)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.stderr.write("bench.py measures one GPU: this build has no multi-GPU path (each op is independent per "
+                         "token row / per (batch, head); see DESIGN.md for how it would shard). Run with --gpus 1.\n")
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        sys.stderr.write("bench.py needs a GPU (MI355X); the ops have no CPU path.\n")
+        sys.exit(2)
+    torch.set_num_threads(os.cpu_count() or 1)
+    dev = torch.device("cuda:0")
+    names = list(WORKLOADS) if args.workload == "all" else [args.workload]
+    if PRIMARY in names:                     # headline first
+        names.remove(PRIMARY)
+        names.insert(0, PRIMARY)
+    results = []
+    for n in names:
+        w = WORKLOADS[n]()
+        steps = args.steps if w.name != "xentropy" else max(3, min(args.steps, 10))
+        results.append(measure(w, dev, steps, args.warmup, not args.no_cpu, min(args.trace_steps, steps)))
+        results[-1]["steps"] = steps
+        del w
+        torch.cuda.empty_cache()
+    head = results[0]
+    line = {
+        "metric": "MFMA TFLOP/s (fused MLP fwd+bwd)" if head["workload"] == "mlp" else head["metric"] + f" ({head['workload']})",
+        "value": head["value"], "unit": head["unit"], "n_gpus": 1, "steps": head["steps"], "warmup": args.warmup,
+        "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": head["dtype"], "data": head["data"],
+        "config": {"workload": head["description"], "timed": head["timed"]},
+        "roofline": head["roofline"], "cpu_baseline": head["cpu_baseline"], "kernels": head["kernels"],
+        "others": results[1:],
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

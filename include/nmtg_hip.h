@@ -202,6 +202,17 @@ int nmtg_mlp_bwd(int num_layers, const void* x, const void* const* weights,
                  void* const* grad_biases, void* workspace, int64_t workspace_bytes, int dtype,
                  void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Per-kernel timing for benchmarks (no counterpart in the reference, whose tests time whole ops
+ * with CUDA events, e.g. onmt/modules/test_layer_norm.py:14-31). Between nmtg_trace_begin() and
+ * nmtg_trace_end() every kernel the library enqueues is bracketed by two HIP events on its
+ * stream. nmtg_trace_end waits for them and writes lines "name launches total_ms\n" into `out`
+ * (NUL-terminated, truncated to `capacity`); it returns the full text length. Not for use while
+ * a stream is being captured into a graph. Process-wide switch.
+ * ------------------------------------------------------------------------------------------ */
+int nmtg_trace_begin(void);
+int64_t nmtg_trace_end(char* out, int64_t capacity);
+
 #ifdef __cplusplus
 }
 #endif

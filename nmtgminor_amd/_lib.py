@@ -54,7 +54,7 @@ def load():
         lib.nmtg_version.restype = ctypes.c_int
         for name in header_functions():
             fn = getattr(lib, name)  # AttributeError here = header / library mismatch
-            if name.endswith("_parts") or name.endswith("_bytes"):
+            if name.endswith("_parts") or name.endswith("_bytes") or name == "nmtg_trace_end":
                 fn.restype = ctypes.c_int64
         _lib = lib
     return _lib
@@ -106,3 +106,18 @@ def call(name, *args):
     """Call entry point `name` with already-wrapped ctypes arguments and raise on error."""
     fn = getattr(load(), name)
     check(fn(*args), name)
+
+
+def trace_begin():
+    check(load().nmtg_trace_begin(), "nmtg_trace_begin")
+
+
+def trace_end():
+    """-> {kernel name: (launches, total milliseconds)} since trace_begin()."""
+    buf = ctypes.create_string_buffer(1 << 16)
+    load().nmtg_trace_end(buf, ctypes.c_int64(len(buf)))
+    out = {}
+    for line in buf.value.decode().splitlines():
+        name, count, ms = line.split()
+        out[name] = (int(count), float(ms))
+    return out

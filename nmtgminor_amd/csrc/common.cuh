@@ -10,6 +10,7 @@
 #include <cstdarg>
 
 #include "../../include/nmtg_hip.h"
+#include "trace.cuh"
 
 namespace nmtg {
 

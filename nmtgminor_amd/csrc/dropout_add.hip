@@ -85,6 +85,7 @@ int dropout_add_fwd_launch(void* x, const void* residual, uint8_t* mask, int64_t
   T* X = static_cast<T*>(x);
   const T* R = static_cast<const T*>(residual);
   constexpr int WIDE = 16 / sizeof(T);
+  TraceScope trace("dropout_add_fwd", st);
   const bool wide = aligned16(x) && aligned16(residual) && (mode == DA_EVAL || aligned8(mask));
 #define DA_LAUNCH(EPV, MODE)                                                                         \
   {                                                                                                  \
@@ -111,6 +112,7 @@ int masked_scale_launch(const void* g, const uint8_t* mask, void* dx, int64_t n,
   const float scale = 1.f / (1.f - p);
   constexpr int WIDE = 16 / sizeof(T);
   const bool wide = aligned16(g) && aligned16(dx) && aligned8(mask);
+  TraceScope trace("dropout_add_bwd", st);
   if (wide) {
     const int64_t per_block = static_cast<int64_t>(DA_THREADS) * WIDE;
     hipLaunchKernelGGL((masked_scale_kernel<T, WIDE>), dim3(static_cast<unsigned>((n + per_block - 1) / per_block)),

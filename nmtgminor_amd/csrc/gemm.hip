@@ -131,6 +131,7 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
 int colsum_parts(int M) { return std::max(1, std::min(64, ceil_div(M, 128))); }
 
 int colsum_finish(int dtype, const float* part, int parts, int N, void* out, hipStream_t st) {
+  TraceScope trace("colsum_final", st);
   NMTG_DISPATCH_DTYPE(dtype, T,
                       hipLaunchKernelGGL((colsum_final_kernel<T>), dim3(ceil_div(N, 256)), dim3(256), 0, st, part, parts, N,
                                          static_cast<T*>(out)));
@@ -141,9 +142,12 @@ int colsum_finish(int dtype, const float* part, int parts, int N, void* out, hip
 int colsum_run(int dtype, const void* X, int64_t ld, int M, int N, float* part, void* out, hipStream_t st) {
   const int parts = colsum_parts(M);
   const int rpb = ceil_div(M, parts);
+  {
+  TraceScope trace("colsum_partial", st);
   NMTG_DISPATCH_DTYPE(dtype, T,
                       hipLaunchKernelGGL((colsum_partial_kernel<T>), dim3(ceil_div(N, 64), parts), dim3(256), 0, st,
                                          static_cast<const T*>(X), ld, M, N, rpb, part));
+  }
   NMTG_CHECK_LAUNCH("colsum");
   return colsum_finish(dtype, part, parts, N, out, st);
 }

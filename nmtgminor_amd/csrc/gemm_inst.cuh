@@ -5,6 +5,7 @@
 //   S: 256x64  tile, 4x1 wavefronts (each 64x64),  256 threads  — N <= 64 (per-head attention products)
 #pragma once
 #include "gemm.cuh"
+#include <string>
 
 namespace nmtg {
 
@@ -33,6 +34,11 @@ int gemm_launch_one(const GemmArgs& a, hipStream_t st) {
     attr_done = true;
   }
   dim3 grid(a.m_tiles * a.n_tiles, a.batch, a.splits);
+  static const std::string name = std::string("gemm_") + (A_KC ? (B_KC ? "nt" : "nn") : "tn") + "_" +
+                                  (TILE == TILE_L ? "256x256" : TILE == TILE_M ? "128x128" : "256x64") + "_" +
+                                  (EPI == EPI_PLAIN ? "plain" : EPI == EPI_ACT_FWD ? "actfwd" : EPI == EPI_ACT_BWD ? "actbwd"
+                                   : EPI == EPI_SCORES ? "scores" : "splitk");
+  TraceScope trace(name.c_str(), st);
   hipLaunchKernelGGL(kern, grid, dim3(64 * C::WM * C::WN), lds, st, a);
   return 0;
 }
@@ -42,6 +48,7 @@ int splitk_reduce_launch(const GemmArgs& a, hipStream_t st) {
   using C = tile_cfg<TILE>;
   constexpr int per_blk = C::WM * C::WN * (C::BM / C::WM / 32) * (C::BN / C::WN / 32) * 4 * 64;
   const int64_t total = static_cast<int64_t>(a.batch) * a.m_tiles * a.n_tiles * per_blk;
+  TraceScope trace("splitk_reduce", st);
   hipLaunchKernelGGL((splitk_reduce_kernel<T, C::BM, C::BN, C::WM, C::WN>), dim3(static_cast<unsigned>((total + 255) / 256)),
                      dim3(256), 0, st, a.ws, static_cast<T*>(a.C), a.ldc, a.M, a.N, a.m_tiles, a.n_tiles, a.batch, a.sC,
                      a.splits, a.alpha, a.c_vec);

@@ -389,6 +389,7 @@ int ln_fwd_launch(const void* x, const void* gamma, const void* beta, void* z, f
   auto B = static_cast<const TW*>(beta);
   auto Z = static_cast<TW*>(z);
   const int H = static_cast<int>(hidden);
+  TraceScope trace("ln_fwd", st);
   if (!p.vectorised) {
     const int grid = static_cast<int>(std::min<int64_t>(rows, ln_grid_limit()));
     hipLaunchKernelGGL((ln_fwd_generic_kernel<TI, TW>), dim3(grid), dim3(LN_THREADS), 0, st, X, G, B,
@@ -436,6 +437,8 @@ int ln_bwd_launch(const void* dz, const void* x_or_z, const float* mu, const flo
   LnPlan p = ln_plan<TI>(hidden, LN_BWD_MAX_VPL);
   const int grid = static_cast<int>(n_part);
   bool done = false;
+  {
+  TraceScope trace("ln_bwd", st);
   if (p.vectorised && al) {
     constexpr int EPV = ln_vec<TI>::EPV;
     const int rpb = LN_WAVES / p.wpr;
@@ -462,6 +465,8 @@ int ln_bwd_launch(const void* dz, const void* x_or_z, const float* mu, const flo
       hipLaunchKernelGGL((ln_bwd_generic_kernel<TI, TW, false>), dim3(grid), dim3(LN_THREADS), 0, st,
                          DZ, X, mu, rsigma, G, B, DX, dgp, dbp, rows, H);
   }
+  }
+  TraceScope trace("ln_bwd_finalize", st);
   dim3 fgrid((H + FIN_COLS - 1) / FIN_COLS, 2);
   hipLaunchKernelGGL((ln_bwd_finalize_kernel<TW>), fgrid, dim3(FIN_COLS * FIN_GROUPS), 0, st, dgp,
                      dbp, static_cast<TW*>(dgamma), static_cast<TW*>(dbeta), static_cast<int>(n_part), H);

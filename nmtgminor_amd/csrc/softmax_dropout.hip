@@ -206,6 +206,7 @@ int softmax_launch(const SoftmaxArgs& a, bool bwd, hipStream_t st) {
   while (vpl * kWave < vecs) vpl *= 2;
   const unsigned grid = static_cast<unsigned>((a.rows + SM_WAVES - 1) / SM_WAVES);
   bool done = false;
+  TraceScope trace(bwd ? "softmax_dropout_bwd" : "softmax_dropout_fwd", st);
 #define SM_CASE(E, V)                                                                                     \
   if (!done && epv == E && vpl == V) {                                                                    \
     if (bwd) hipLaunchKernelGGL((softmax_bwd_kernel<T, E, V>), dim3(grid), dim3(SM_THREADS), 0, st, a);   \

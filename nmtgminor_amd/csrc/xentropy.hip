@@ -193,6 +193,7 @@ extern "C" int nmtg_xentropy_fwd(const void* logits, const int64_t* labels, floa
   if (rows == 0) return 0;
   NMTG_REQUIRE(logits && labels && losses && lse, "xentropy_fwd: null pointer argument");
   hipStream_t st = static_cast<hipStream_t>(stream);
+  TraceScope trace("xentropy_fwd", st);
   NMTG_DISPATCH_DTYPE(dtype, T,
                       hipLaunchKernelGGL((xentropy_fwd_kernel<T>), dim3(static_cast<unsigned>(rows)), dim3(XE_THREADS), 0,
                                          st, static_cast<const T*>(logits), labels, losses, lse, vocab, smoothing,
@@ -211,6 +212,7 @@ extern "C" int nmtg_xentropy_bwd(const float* grad_loss, const void* logits, con
   hipStream_t st = static_cast<hipStream_t>(stream);
   // Vector accesses need the logits row and the gradient row to share their 16-byte phase.
   const bool vec = ((reinterpret_cast<uintptr_t>(logits) ^ reinterpret_cast<uintptr_t>(grad_logits)) & 15u) == 0;
+  TraceScope trace("xentropy_bwd", st);
   NMTG_DISPATCH_DTYPE(
       dtype, T,
       if (vec) hipLaunchKernelGGL((xentropy_bwd_kernel<T, true>), dim3(static_cast<unsigned>(rows)), dim3(XE_THREADS), 0, st,
