@@ -203,6 +203,72 @@ int nmtg_mlp_bwd(int num_layers, const void* x, const void* const* weights,
                  void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Self-attention (time-first activations, per-head interleaved q/k/v).
+ * Reference: self_multihead_attn_blaslt.forward / backward / forward_compact / backward_compact
+ *   (onmt/modules/extensions/multihead_attn_blaslt/self_multihead_attn.cpp:95-132, :162-212,
+ *   :135-160, :215-240; device side self_multihead_attn_cuda.cu:40-243, :413-742).
+ *
+ * x [T, B, E]; w_in [3E, E] with rows ordered (head, {q,k,v}, head_dim); w_out [E, E]; biases may
+ * be NULL. lin [T, B, 3E] (= [T, B*H, 3, D]) is the input projection: written when x / w_in are
+ * given, read when both are NULL (the "compact" form, projections done by the caller).
+ * mask (1 = masked): mask_kind 0 none, 1 key padding [B, T], 2 time mask [T, T].
+ * scores [B*H, T, T]: scaled, masked (-inf) pre-softmax scores; softmax_out (may be NULL) the
+ * probabilities before dropout; dropped the probabilities after dropout (what multiplies v).
+ * dropout_mode 0 none, 1 replay dropout_mask [B*H, T, T], 2 draw it (Philox) and store it.
+ * ctx [T, B, E]; out [T, B, E] (NULL together with w_out in the compact form).
+ * dtype NMTG_F16 or NMTG_BF16 (the reference is fp16 only); T <= 4096.
+ * ------------------------------------------------------------------------------------------ */
+int nmtg_self_attn_fwd(const void* x, const void* w_in, const void* w_out, const void* b_in,
+                       const void* b_out, const uint8_t* mask, int mask_kind, void* lin,
+                       void* scores, void* softmax_out, void* dropped, uint8_t* dropout_mask,
+                       int dropout_mode, float p, uint64_t seed, uint64_t offset, void* ctx,
+                       void* out, int64_t t, int64_t b, int64_t e, int heads, int dtype,
+                       void* stream);
+
+int64_t nmtg_self_attn_bwd_workspace_bytes(int64_t t, int64_t b, int64_t e, int heads);
+
+/* grad_out [T, B, E]: gradient of `out`, or of `ctx` in the compact form (w_out == NULL; then
+ * ctx, x, w_in may be NULL and only grad_lin is produced). Any of grad_x, grad_w_*, grad_b_* may
+ * be NULL to skip it. grad_lin (may be NULL): receives the gradient of `lin`, [T, B, 3E].
+ * dropout_mask NULL or p == 0: no dropout was applied. The probabilities are recomputed from
+ * `scores`. workspace: nmtg_self_attn_bwd_workspace_bytes bytes, 256-byte aligned. */
+int nmtg_self_attn_bwd(const void* grad_out, const void* ctx, const void* dropped,
+                       const void* scores, const void* lin, const void* x, const void* w_in,
+                       const void* w_out, const uint8_t* dropout_mask, float p, void* grad_x,
+                       void* grad_w_in, void* grad_w_out, void* grad_b_in, void* grad_b_out,
+                       void* grad_lin, void* workspace, int64_t workspace_bytes, int64_t t,
+                       int64_t b, int64_t e, int heads, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Encoder-decoder attention.
+ * Reference: encdec_multihead_attn_bias_blaslt.forward / backward / forward_compact /
+ *   backward_compact (multihead_attn_blaslt/encdec_multihead_attn_bias.cpp:124-173, :203-267,
+ *   :175-201, :269-308; device side encdec_multihead_attn_bias_cuda.cu:40-273, :1089-1472).
+ *
+ * x_q [Tq, B, E], x_kv [Tk, B, E]; w_q [E, E]; w_kv [2E, E] with rows ordered (head, {k,v},
+ * head_dim); q_lin [Tq, B, E], kv_lin [Tk, B, 2E] written (or read, when the matching input and
+ * weight are NULL). pad_mask [B, Tk] (1 = masked) or NULL. Other arguments as for self-attention;
+ * scores / dropped are [B*H, Tq, Tk]; Tk <= 4096.
+ * ------------------------------------------------------------------------------------------ */
+int nmtg_encdec_attn_fwd(const void* x_q, const void* x_kv, const void* w_q, const void* w_kv,
+                         const void* w_out, const void* b_q, const void* b_kv, const void* b_out,
+                         const uint8_t* pad_mask, void* q_lin, void* kv_lin, void* scores,
+                         void* softmax_out, void* dropped, uint8_t* dropout_mask, int dropout_mode,
+                         float p, uint64_t seed, uint64_t offset, void* ctx, void* out, int64_t tq,
+                         int64_t tk, int64_t b, int64_t e, int heads, int dtype, void* stream);
+
+int64_t nmtg_encdec_attn_bwd_workspace_bytes(int64_t tq, int64_t tk, int64_t b, int64_t e, int heads);
+
+int nmtg_encdec_attn_bwd(const void* grad_out, const void* ctx, const void* dropped,
+                         const void* scores, const void* q_lin, const void* kv_lin,
+                         const void* x_q, const void* x_kv, const void* w_q, const void* w_kv,
+                         const void* w_out, const uint8_t* dropout_mask, float p, void* grad_x_q,
+                         void* grad_x_kv, void* grad_w_q, void* grad_w_kv, void* grad_w_out,
+                         void* grad_b_q, void* grad_b_kv, void* grad_b_out, void* grad_q_lin,
+                         void* grad_kv_lin, void* workspace, int64_t workspace_bytes, int64_t tq,
+                         int64_t tk, int64_t b, int64_t e, int heads, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Per-kernel timing for benchmarks (no counterpart in the reference, whose tests time whole ops
  * with CUDA events, e.g. onmt/modules/test_layer_norm.py:14-31). Between nmtg_trace_begin() and
  * nmtg_trace_end() every kernel the library enqueues is bracketed by two HIP events on its

@@ -1,0 +1,56 @@
+"""Shared plumbing of the attention stand-in modules."""
+import ctypes
+
+import torch
+
+from .. import _lib as L
+from .._rng import philox_seed_offset
+
+
+def check(cond, msg):
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def check_half(*tensors):
+    for t in tensors:
+        if t is not None:
+            check(t.dtype in (torch.float16, torch.bfloat16), "Only HALF / BFLOAT16 is supported")
+    dts = {t.dtype for t in tensors if t is not None}
+    check(len(dts) <= 1, "all tensors must share one dtype")
+
+
+def mask_arg(mask, use_time_mask, batch, len_q, len_k):
+    """Reference mask conventions: time mask [len_q, len_k]; key padding [B, len_k] or
+    [B, 1, 1, len_k] (onmt/modules/optimized/self_attention_func.py:90-99). -> (uint8 tensor, kind)"""
+    if mask is None or mask.numel() == 0:
+        return None, 0
+    if use_time_mask:
+        check(mask.numel() == len_q * len_k, "time mask must be [len_q, len_k]")
+        return mask.reshape(len_q, len_k).to(torch.uint8).contiguous(), 2
+    check(mask.numel() == batch * len_k, "key padding mask must be [batch, len_k]")
+    return mask.reshape(batch, len_k).to(torch.uint8).contiguous(), 1
+
+
+def dropout_args(is_training, p, shape, device, dropout_mask):
+    """-> (mask tensor, mode, seed, offset)"""
+    if is_training and p > 0.0:
+        if dropout_mask is not None:
+            n = 1
+            for s in shape:
+                n *= s
+            check(dropout_mask.dtype == torch.uint8 and dropout_mask.numel() == n, "dropout mask must be uint8 [B*H, Tq, Tk]")
+            return dropout_mask.contiguous().view(shape), 1, 0, 0
+        m = torch.empty(shape, dtype=torch.uint8, device=device)
+        n = m.numel()
+        seed, offset = philox_seed_offset(device, n)
+        return m, 2, seed, offset
+    return torch.empty(0, dtype=torch.uint8, device=device), 0, 0, 0
+
+
+def u64(v):
+    return ctypes.c_uint64(v)
+
+
+def workspace(nbytes, device):
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)

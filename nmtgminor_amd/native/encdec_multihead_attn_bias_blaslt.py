@@ -1,0 +1,145 @@
+"""Stand-in for the reference module `encdec_multihead_attn_bias_blaslt`
+(onmt/modules/extensions/multihead_attn_blaslt/encdec_multihead_attn_bias.cpp:124-475): forward,
+backward, forward_compact, backward_compact, backward_recompute; plus backward_input_only of the
+older `encdec_multihead_attn_bias_cuda` (multihead_attn/encdec_multihead_attn_bias.cpp:308-310).
+
+Extras: any bias may be None (Whisper's key projection has none); fp16 and bf16; `forward` /
+`forward_compact` take an optional keyword `dropout_mask` to replay an explicit keep-mask."""
+import torch
+
+from .. import _lib as L
+from . import _attn_common as A
+
+
+def _shapes(q3, kv3, heads, kv_last):
+    A.check(q3.dim() == 3 and kv3.dim() == 3, "expected 3D tensor")
+    tq, b, e = q3.shape
+    tk = kv3.shape[0]
+    A.check(kv3.shape[1] == b and kv3.shape[2] == e * kv_last and e % heads == 0, "query / key-value shapes do not match")
+    return tq, tk, b, e
+
+
+def _fwd(is_training, heads, x_q, x_kv, w_q, w_kv, w_out, b_q, b_kv, b_out, q_lin, kv_lin, pad_mask, p, dropout_mask,
+         tq, tk, b, e, dev, dt):
+    km, kind = A.mask_arg(pad_mask, False, b, tq, tk)
+    bh = b * heads
+    if q_lin is None:
+        q_lin = torch.empty(tq, b, e, dtype=dt, device=dev)
+    if kv_lin is None:
+        kv_lin = torch.empty(tk, b, 2 * e, dtype=dt, device=dev)
+    scores = torch.empty(bh, tq, tk, dtype=dt, device=dev)
+    dropped = torch.empty(bh, tq, tk, dtype=dt, device=dev)
+    ctx = torch.empty(tq, b, e, dtype=dt, device=dev)
+    out = torch.empty(tq, b, e, dtype=dt, device=dev) if w_out is not None else None
+    dmask, mode, seed, offset = A.dropout_args(is_training, p, (bh, tq, tk), dev, dropout_mask)
+    L.call("nmtg_encdec_attn_fwd", L.ptr(x_q), L.ptr(x_kv), L.ptr(w_q), L.ptr(w_kv), L.ptr(w_out), L.ptr(b_q), L.ptr(b_kv),
+           L.ptr(b_out), L.ptr(km), L.ptr(q_lin), L.ptr(kv_lin), L.ptr(scores), L.ptr(None), L.ptr(dropped),
+           L.ptr(dmask if mode else None), L.i32(mode), L.f32(p), A.u64(seed), A.u64(offset), L.ptr(ctx), L.ptr(out),
+           L.i64(tq), L.i64(tk), L.i64(b), L.i64(e), L.i32(heads), L.i32(L.dtype_code(ctx)), L.stream_of(ctx))
+    return q_lin, kv_lin, scores, dropped, dmask, ctx, out
+
+
+def forward(is_training, heads, inputs_q, inputs_kv, input_weights_q, input_weights_kv, output_weights, input_biases_q,
+            input_biases_kv, output_biases, pad_mask, dropout_prob, *, dropout_mask=None):
+    """-> [input_lin_q_results, input_lin_kv_results, attn_scores, dropout_results, dropout_mask,
+    matmul2_results, outputs]"""
+    tensors = (inputs_q, inputs_kv, input_weights_q, input_weights_kv, output_weights, input_biases_q, input_biases_kv,
+               output_biases)
+    L.require_cuda(*tensors, pad_mask, dropout_mask)
+    A.check_half(*tensors)
+    tq, tk, b, e = _shapes(inputs_q, inputs_kv, heads, 1)
+    A.check(input_weights_q.shape == (e, e) and input_weights_kv.shape == (2 * e, e) and output_weights.shape == (e, e),
+            "weight shapes do not match the inputs")
+    c = lambda z: z.contiguous() if z is not None else None
+    return list(_fwd(is_training, heads, c(inputs_q), c(inputs_kv), c(input_weights_q), c(input_weights_kv),
+                     c(output_weights), c(input_biases_q), c(input_biases_kv), c(output_biases), None, None, pad_mask,
+                     dropout_prob, dropout_mask, tq, tk, b, e, inputs_q.device, inputs_q.dtype))
+
+
+def forward_compact(is_training, heads, input_lin_q_results, input_lin_kv_results, pad_mask, dropout_prob, *,
+                    dropout_mask=None):
+    """-> [attn_scores, dropout_results, dropout_mask, matmul2_results]"""
+    L.require_cuda(input_lin_q_results, input_lin_kv_results, pad_mask, dropout_mask)
+    A.check_half(input_lin_q_results, input_lin_kv_results)
+    tq, tk, b, e = _shapes(input_lin_q_results, input_lin_kv_results, heads, 2)
+    r = _fwd(is_training, heads, None, None, None, None, None, None, None, None, input_lin_q_results.contiguous(),
+             input_lin_kv_results.contiguous(), pad_mask, dropout_prob, dropout_mask, tq, tk, b, e,
+             input_lin_q_results.device, input_lin_q_results.dtype)
+    return [r[2], r[3], r[4], r[5]]
+
+
+def _bwd(heads, output_grads, matmul2_results, dropout_results, attn_scores, q_lin, kv_lin, inputs_q, inputs_kv, w_q, w_kv,
+         w_out, dropout_mask, p, want_weights=True, want_biases=True):
+    L.require_cuda(output_grads, dropout_results, attn_scores, q_lin, kv_lin, inputs_q, inputs_kv, w_q, w_kv, w_out)
+    A.check_half(output_grads, dropout_results, attn_scores, q_lin, kv_lin, inputs_q, inputs_kv, w_q, w_kv, w_out)
+    tq, tk, b, e = _shapes(q_lin, kv_lin, heads, 2)
+    dev, dt = output_grads.device, output_grads.dtype
+    g = output_grads.contiguous()
+    use_mask = dropout_mask is not None and dropout_mask.numel() > 0 and p > 0.0
+    compact = w_out is None
+    n = {k: None for k in ("dxq", "dxkv", "dwq", "dwkv", "dwo", "dbq", "dbkv", "dbo", "dq", "dkv")}
+    if compact:
+        n["dq"] = torch.empty(tq, b, e, dtype=dt, device=dev)
+        n["dkv"] = torch.empty(tk, b, 2 * e, dtype=dt, device=dev)
+    else:
+        n["dxq"] = torch.empty(tq, b, e, dtype=dt, device=dev)
+        n["dxkv"] = torch.empty(tk, b, e, dtype=dt, device=dev)
+        if want_weights:
+            n["dwq"] = torch.empty(e, e, dtype=dt, device=dev)
+            n["dwkv"] = torch.empty(2 * e, e, dtype=dt, device=dev)
+            n["dwo"] = torch.empty(e, e, dtype=dt, device=dev)
+            if want_biases:
+                n["dbq"] = torch.empty(e, dtype=dt, device=dev)
+                n["dbkv"] = torch.empty(2 * e, dtype=dt, device=dev)
+                n["dbo"] = torch.empty(e, dtype=dt, device=dev)
+    ws_bytes = L.load().nmtg_encdec_attn_bwd_workspace_bytes(L.i64(tq), L.i64(tk), L.i64(b), L.i64(e), L.i32(heads))
+    ws = A.workspace(ws_bytes, dev)
+    c = lambda z: z.contiguous() if z is not None else None
+    L.call("nmtg_encdec_attn_bwd", L.ptr(g), L.ptr(c(matmul2_results)), L.ptr(c(dropout_results)), L.ptr(c(attn_scores)),
+           L.ptr(c(q_lin)), L.ptr(c(kv_lin)), L.ptr(c(inputs_q)), L.ptr(c(inputs_kv)), L.ptr(c(w_q)), L.ptr(c(w_kv)),
+           L.ptr(c(w_out)), L.ptr(c(dropout_mask) if use_mask else None), L.f32(p), L.ptr(n["dxq"]), L.ptr(n["dxkv"]),
+           L.ptr(n["dwq"]), L.ptr(n["dwkv"]), L.ptr(n["dwo"]), L.ptr(n["dbq"]), L.ptr(n["dbkv"]), L.ptr(n["dbo"]),
+           L.ptr(n["dq"]), L.ptr(n["dkv"]), L.ptr(ws), L.i64(ws.numel()), L.i64(tq), L.i64(tk), L.i64(b), L.i64(e),
+           L.i32(heads), L.i32(L.dtype_code(g)), L.stream_of(g))
+    return n
+
+
+def backward(heads, output_grads, matmul2_results, dropout_results, attn_scores, input_lin_q_results,
+             input_lin_kv_results, inputs_q, inputs_kv, input_weights_q, input_weights_kv, output_weights, dropout_mask,
+             dropout_prob):
+    """-> [input_q_grads, input_kv_grads, input_weight_q_grads, input_weight_kv_grads,
+    output_weight_grads, input_bias_q_grads, input_bias_kv_grads, output_bias_grads]"""
+    n = _bwd(heads, output_grads, matmul2_results, dropout_results, attn_scores, input_lin_q_results, input_lin_kv_results,
+             inputs_q, inputs_kv, input_weights_q, input_weights_kv, output_weights, dropout_mask, dropout_prob)
+    return [n[k] for k in ("dxq", "dxkv", "dwq", "dwkv", "dwo", "dbq", "dbkv", "dbo")]
+
+
+def backward_input_only(heads, output_grads, matmul2_results, dropout_results, attn_scores, input_lin_q_results,
+                        input_lin_kv_results, inputs_q, inputs_kv, input_weights_q, input_weights_kv, output_weights,
+                        dropout_mask, dropout_prob):
+    """-> [input_q_grads, input_kv_grads]"""
+    n = _bwd(heads, output_grads, matmul2_results, dropout_results, attn_scores, input_lin_q_results, input_lin_kv_results,
+             inputs_q, inputs_kv, input_weights_q, input_weights_kv, output_weights, dropout_mask, dropout_prob,
+             want_weights=False)
+    return [n["dxq"], n["dxkv"]]
+
+
+def backward_compact(heads, output_lin_grads, dropout_results, attn_scores, input_lin_q_results, input_lin_kv_results,
+                     dropout_mask, dropout_prob):
+    """-> [input_lin_q_grads, input_lin_kv_grads]"""
+    n = _bwd(heads, output_lin_grads, None, dropout_results, attn_scores, input_lin_q_results, input_lin_kv_results, None,
+             None, None, None, None, dropout_mask, dropout_prob)
+    return [n["dq"], n["dkv"]]
+
+
+def backward_recompute(heads, output_grads, inputs_q, inputs_kv, input_weights_q, input_weights_kv, input_biases_q,
+                       input_biases_kv, output_weights, dropout_mask, pad_mask, dropout_prob):
+    """Re-runs the forward from the inputs and the stored dropout mask, then the backward. The
+    output bias does not enter any gradient, so it is not an argument (as in the reference)."""
+    training = dropout_mask is not None and dropout_mask.numel() > 0 and dropout_prob > 0.0
+    q_lin, kv_lin, scores, dropped, dmask, ctx, _ = forward(training, heads, inputs_q, inputs_kv, input_weights_q,
+                                                            input_weights_kv, output_weights, input_biases_q,
+                                                            input_biases_kv, None, pad_mask, dropout_prob,
+                                                            dropout_mask=dropout_mask if training else None)
+    return backward(heads, output_grads, ctx, dropped, scores, q_lin, kv_lin, inputs_q, inputs_kv, input_weights_q,
+                    input_weights_kv, output_weights, dmask, dropout_prob)

@@ -1,0 +1,198 @@
+"""Self / encoder-decoder attention parity: HIP (through the C ABI) vs the CPU oracle on identical
+seeded inputs, dropout via a replayed mask or p = 0.
+
+Follows the reference's attention tests: the same function evaluated on the fused path and on
+the PyTorch path with random key-padding or triu time masks, outputs and every gradient compared
+(onmt/modules/optimized/test_encdec_attention_func.py:93-181 — Tq=64, Tk=512, B=64, E=1024, H=16;
+test_self_attention_func.py:38-68 — T=512, B=64), tolerance 1e-2 / 1e-3 there, 2e-2 / 1e-3 here.
+"""
+import pytest
+import torch
+
+from nmtgminor_amd.modules.encdec_attention import EncdecMultiheadAttn
+from nmtgminor_amd.modules.encdec_attention_func_bias import encdec_attn_bias_compact_func, encdec_attn_bias_func
+from nmtgminor_amd.modules.self_attention import SelfMultiheadAttn
+from nmtgminor_amd.modules.self_attention_func import self_attn_compact_func, self_attn_func
+from nmtgminor_amd.native import encdec_multihead_attn_bias_blaslt as ed_native, self_multihead_attn_blaslt as sa_native
+from oracle import attention as oat, inputs
+from util import assert_close
+
+pytestmark = pytest.mark.gpu
+D = torch.float64
+
+
+def _self_case(dev, t, b, e, h, dtype, p, causal=False, zero_bias=False, seed=71, recompute=False):
+    d = inputs.self_attn_inputs(t, b, e, h, dtype, p=p, seed=seed, causal=causal, zero_bias=zero_bias)
+    fwd = oat.self_attn_fwd(d["x"], d["w_in"], d["w_out"], d["b_in"], d["b_out"], h, d["pad_mask"], d["time_mask"], p,
+                            d["dropout_mask"], D, round_to=dtype)
+    bwd = oat.self_attn_bwd(d["dout"], d["x"], d["w_in"], d["w_out"], h, fwd, p, d["dropout_mask"], D, round_to=dtype)
+    leaves = [d[k].to(dev).requires_grad_() for k in ("x", "w_in", "w_out", "b_in", "b_out")]
+    mask = (d["time_mask"] if causal else d["pad_mask"]).to(dev)
+    dm = d["dropout_mask"].to(dev) if p > 0 else None
+    out, cov = self_attn_func(causal, True, h, leaves[0], leaves[1], leaves[2], leaves[3], leaves[4], mask, p, False, None,
+                              False, None, True, True, recompute, dm)
+    out.backward(d["dout"].to(dev))
+    assert_close(out, fwd["outputs"], dtype, "outputs")
+    assert_close(cov, fwd["dropout_results"], dtype, "dropout_results")
+    # masked keys carry exactly zero probability
+    covc = cov.float().cpu().view(b, h, t, t)
+    if causal:
+        assert (covc[:, :, torch.triu(torch.ones(t, t), 1).bool()] == 0).all()
+    else:
+        assert (covc.permute(0, 3, 1, 2)[d["pad_mask"]] == 0).all()
+    assert_close(leaves[0].grad, bwd["dx"], dtype, "dx", scale_atol=True)
+    assert_close(leaves[1].grad, bwd["dw_in"], dtype, "dW_in", scale_atol=True)
+    assert_close(leaves[2].grad, bwd["dw_out"], dtype, "dW_out", scale_atol=True)
+    assert_close(leaves[3].grad, bwd["db_in"], dtype, "db_in", scale_atol=True)
+    assert_close(leaves[4].grad, bwd["db_out"], dtype, "db_out", scale_atol=True)
+    return d, fwd, bwd
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("t,b,e,h,p", [(64, 4, 256, 4, 0.0), (128, 3, 512, 8, 0.1), (200, 2, 256, 4, 0.25), (33, 2, 128, 2, 0.1)])
+def test_self_attention_key_padding(dev, dtype, t, b, e, h, p):
+    _self_case(dev, t, b, e, h, dtype, p)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_self_attention_causal_and_recompute(dev, dtype):
+    _self_case(dev, 128, 4, 512, 8, dtype, 0.1, causal=True)
+    _self_case(dev, 96, 2, 256, 4, dtype, 0.2, recompute=True)
+
+
+def test_self_attention_intermediates_and_native_contract(dev):
+    dtype = torch.bfloat16
+    t, b, e, h = 64, 2, 256, 4
+    d = inputs.self_attn_inputs(t, b, e, h, dtype, p=0.1, seed=72, zero_bias=False)
+    fwd = oat.self_attn_fwd(d["x"], d["w_in"], d["w_out"], d["b_in"], d["b_out"], h, d["pad_mask"], None, 0.1,
+                            d["dropout_mask"], D, round_to=dtype)
+    g = lambda k: d[k].to(dev)
+    lin, scores, dropped, dmask, ctx, out = sa_native.forward(False, True, h, g("x"), g("w_in"), g("w_out"), g("b_in"),
+                                                              g("b_out"), g("pad_mask"), 0.1, dropout_mask=g("dropout_mask"))
+    assert lin.shape == (t, b, 3 * e) and scores.shape == (b * h, t, t) and ctx.shape == (t, b, e)
+    assert_close(lin, fwd["input_lin_results"], dtype, "input_lin_results")
+    sc, so = scores.float().cpu(), fwd["attn_scores"].float()
+    assert torch.equal(torch.isinf(sc), torch.isinf(so))                       # -inf exactly on the masked keys
+    fin = ~torch.isinf(so)
+    assert_close(sc[fin], so[fin], dtype, "attn_scores")
+    assert_close(ctx, fwd["matmul2_results"], dtype, "matmul2_results")
+    assert torch.equal(dmask.cpu(), d["dropout_mask"])
+    # compact form: projections outside
+    scores2, dropped2, _, ctx2 = sa_native.forward_compact(False, True, h, lin, g("pad_mask"), 0.1, dropout_mask=g("dropout_mask"))
+    assert torch.equal(ctx2, ctx) and torch.equal(dropped2, dropped)
+    dctx = torch.randn(t, b, e, generator=torch.Generator().manual_seed(1)).to(dtype)
+    (dlin,) = sa_native.backward_compact(False, h, dctx.to(dev), dropped, scores, lin, dmask, 0.1)
+    q, k, v = [fwd["input_lin_results"].to(D).view(t, b * h, 3, e // h)[:, :, i] for i in range(3)]
+    dq, dk, dv = oat._core_bwd(dctx.to(D).view(t, b * h, e // h), q, k, v, fwd["softmax_results"], fwd["dropout_results"],
+                               0.1, d["dropout_mask"], D, round_to=dtype)
+    assert_close(dlin, torch.stack([dq, dk, dv], 2).reshape(t, b, 3 * e), dtype, "compact dlin", scale_atol=True)
+
+
+def test_self_attention_rng_dropout_eval_and_no_bias(dev):
+    dtype = torch.float16
+    t, b, e, h = 64, 2, 128, 4
+    d = inputs.self_attn_inputs(t, b, e, h, dtype, p=0.0, seed=73, zero_bias=False)
+    g = lambda k: d[k].to(dev)
+    # biases None (Whisper-style projections without bias)
+    fwd = oat.self_attn_fwd(d["x"], d["w_in"], d["w_out"], None, None, h, d["pad_mask"], None, 0.0, None, D, round_to=dtype)
+    out, cov = self_attn_func(False, False, h, g("x"), g("w_in"), g("w_out"), None, None, g("pad_mask"), 0.3, False, None,
+                              False, None, True, True, False)
+    assert_close(out, fwd["outputs"], dtype, "eval, no bias")              # eval: dropout not applied
+    torch.cuda.manual_seed(11)
+    r = sa_native.forward(False, True, h, g("x"), g("w_in"), g("w_out"), None, None, g("pad_mask"), 0.3)
+    dmask = r[3]
+    assert dmask.shape == (b * h, t, t) and abs(dmask.float().mean().item() - 0.7) < 0.02
+    fwd2 = oat.self_attn_fwd(d["x"], d["w_in"], d["w_out"], None, None, h, d["pad_mask"], None, 0.3, dmask.cpu(), D, round_to=dtype)
+    assert_close(r[5], fwd2["outputs"], dtype, "rng dropout outputs")
+    with pytest.raises(NotImplementedError):
+        self_attn_func(False, False, h, g("x"), g("w_in"), g("w_out"), None, None, None, 0.0, True, None, False, None, True, True, False)
+    with pytest.raises(RuntimeError):
+        sa_native.forward(False, False, h, g("x").float(), g("w_in").float(), g("w_out").float(), None, None, None, 0.0)
+
+
+def _encdec_case(dev, tq, tk, b, e, h, dtype, p, zero_bias=False, biases=True, seed=74):
+    d = inputs.encdec_attn_inputs(tq, tk, b, e, h, dtype, p=p, seed=seed, zero_bias=zero_bias)
+    if not biases:
+        d["b_q"] = d["b_kv"] = d["b_out"] = None
+    fwd = oat.encdec_attn_fwd(d["x_q"], d["x_kv"], d["w_q"], d["w_kv"], d["w_out"], d["b_q"], d["b_kv"], d["b_out"], h,
+                              d["pad_mask"], p, d["dropout_mask"], D, round_to=dtype)
+    bwd = oat.encdec_attn_bwd(d["dout"], d["x_q"], d["x_kv"], d["w_q"], d["w_kv"], d["w_out"], h, fwd, p, d["dropout_mask"],
+                              D, round_to=dtype)
+    names = ("x_q", "x_kv", "w_q", "w_kv", "w_out", "b_q", "b_kv", "b_out")
+    leaf = {k: (d[k].to(dev).requires_grad_() if d[k] is not None else None) for k in names}
+    dm = d["dropout_mask"].to(dev) if p > 0 else None
+    out, cov = encdec_attn_bias_func(False, True, h, leaf["x_q"], leaf["x_kv"], leaf["w_q"], leaf["w_kv"], leaf["w_out"],
+                                     leaf["b_q"], leaf["b_kv"], leaf["b_out"], d["pad_mask"].to(dev), p, False, None, False,
+                                     None, None, True, True, dm)
+    out.backward(d["dout"].to(dev))
+    assert_close(out, fwd["outputs"], dtype, "outputs")
+    assert_close(cov, fwd["dropout_results"], dtype, "dropout_results")
+    assert (cov.float().cpu().view(b, h, tq, tk).permute(0, 3, 1, 2)[d["pad_mask"]] == 0).all()
+    for key, n in (("dx_q", "x_q"), ("dx_kv", "x_kv"), ("dw_q", "w_q"), ("dw_kv", "w_kv"), ("dw_out", "w_out"),
+                   ("db_q", "b_q"), ("db_kv", "b_kv"), ("db_out", "b_out")):
+        if leaf[n] is not None:
+            assert_close(leaf[n].grad, bwd[key], dtype, key, scale_atol=True)
+    return d, fwd, leaf
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("tq,tk,b,e,h,p", [(64, 512, 4, 256, 4, 0.0), (32, 1500, 2, 256, 4, 0.1), (17, 100, 3, 128, 2, 0.2)])
+def test_encdec_attention(dev, dtype, tq, tk, b, e, h, p):
+    _encdec_case(dev, tq, tk, b, e, h, dtype, p)
+
+
+def test_encdec_attention_without_biases_and_compact(dev):
+    dtype = torch.bfloat16
+    d, fwd, leaf = _encdec_case(dev, 48, 300, 2, 256, 4, dtype, 0.1, biases=False)
+    r = ed_native.forward(True, 4, leaf["x_q"].detach(), leaf["x_kv"].detach(), leaf["w_q"].detach(), leaf["w_kv"].detach(),
+                          leaf["w_out"].detach(), None, None, None, d["pad_mask"].to(dev), 0.1,
+                          dropout_mask=d["dropout_mask"].to(dev))
+    q_lin, kv_lin, scores, dropped, dmask, ctx, out = r
+    assert q_lin.shape == (48, 2, 256) and kv_lin.shape == (300, 2, 512) and scores.shape == (8, 48, 300)
+    assert_close(kv_lin, fwd["input_lin_kv_results"], dtype, "kv_lin")
+    ctx2, cov2 = encdec_attn_bias_compact_func(False, True, 4, q_lin, kv_lin, d["pad_mask"].to(dev), 0.1, False, None, False,
+                                               None, None, True, True, d["dropout_mask"].to(dev))
+    assert torch.equal(ctx2, ctx) and torch.equal(cov2, dropped)
+    dq, dkv = ed_native.backward_compact(4, d["dout"].to(dev), dropped, scores, q_lin, kv_lin, dmask, 0.1)
+    assert dq.shape == q_lin.shape and dkv.shape == kv_lin.shape and torch.isfinite(dq.float()).all()
+
+
+def test_modules_state_dict_names_and_forward(dev):
+    sa = SelfMultiheadAttn(256, 4, dropout=0.0).to(dev).half()
+    assert sorted(sa.state_dict()) == ["in_proj_bias", "in_proj_weight", "out_proj_bias", "out_proj_weight"]
+    x = torch.randn(40, 3, 256, device=dev).half()
+    pad = torch.zeros(3, 40, dtype=torch.bool, device=dev)
+    pad[1, 30:] = True
+    y, cov = sa(x, None, key_padding_mask=pad)
+    ref = oat.self_attn_fwd(x.cpu(), sa.in_proj_weight.detach().cpu(), sa.out_proj_weight.detach().cpu(),
+                            sa.in_proj_bias.detach().cpu(), sa.out_proj_bias.detach().cpu(), 4, pad.cpu(), None, 0.0, None, D,
+                            round_to=torch.float16)
+    assert_close(y, ref["outputs"], torch.float16, "module outputs")
+    y2, _ = sa(x, None, attn_mask=torch.triu(torch.ones(40, 40, device=dev), 1).bool())
+    assert y2.shape == x.shape
+    ed = EncdecMultiheadAttn(4, 256).to(dev).half()
+    assert sorted(ed.state_dict()) == ["in_proj_weight_kv", "in_proj_weight_q", "out_proj_weight"]
+    mem = torch.randn(70, 3, 256, device=dev).half()
+    o, c = ed(x, mem, mem, attn_mask=torch.zeros(3, 70, dtype=torch.bool, device=dev))
+    assert o.shape == x.shape and c.shape == (12, 40, 70)
+
+
+def test_feed_forward_module(dev):
+    from nmtgminor_amd.modules.feed_forward import PositionWiseFeedForward
+    from oracle import mlp as omlp
+    ff = PositionWiseFeedForward(128, 512, dropout=0.1, activation="gelu").to(dev).half().eval()
+    assert sorted(ff.state_dict()) == ["in_proj_bias", "in_proj_weight", "out_proj_bias", "out_proj_weight"]
+    x = torch.randn(20, 4, 128, device=dev).half()
+    y = ff(x)
+    w = [ff.in_proj_weight.detach().cpu(), ff.out_proj_weight.detach().cpu()]
+    bb = [ff.in_proj_bias.detach().cpu(), ff.out_proj_bias.detach().cpu()]
+    yo, _, _ = omlp.mlp_fwd(x.cpu().view(80, 128), w, bb, "gelu", 0.0, None, D, round_to=torch.float16)
+    assert_close(y.view(80, 128), yo, torch.float16, "feed-forward eval")
+    ffr = PositionWiseFeedForward(128, 512, dropout=0.0, activation="relu", dropout_residual=True, res_dropout=0.0).to(dev).half()
+    yr = ffr(x.clone())
+    w = [ffr.in_proj_weight.detach().cpu(), ffr.out_proj_weight.detach().cpu()]
+    bb = [ffr.in_proj_bias.detach().cpu(), ffr.out_proj_bias.detach().cpu()]
+    yo, _, _ = omlp.mlp_fwd(x.cpu().view(80, 128), w, bb, "relu", 0.0, None, D, round_to=torch.float16)
+    assert_close(yr.view(80, 128), yo.to(torch.float16).to(D) + x.cpu().view(80, 128).to(D), torch.float16, "residual")
+    with pytest.raises(NotImplementedError):
+        PositionWiseFeedForward(128, 512, glu=True)
