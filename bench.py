@@ -218,12 +218,107 @@ class XentropyWL(Workload):
                     sample=f"first {n} of {self.rows} rows, fp32 on the bf16-rounded logits, algorithmic bf16 bytes / time, median of 3")
 
 
-WORKLOADS = {w.name: w for w in (LayerNormWL, MlpWL, XentropyWL)}
-try:
-    from _bench_attention import ATTENTION_WORKLOADS   # added with the attention ops
-    WORKLOADS.update(ATTENTION_WORKLOADS)
-except ImportError:
-    pass
+class SelfAttnWL(Workload):
+    name = "self_attn"
+    bound = "mfma"
+    dtype = "bf16"
+    description = ("encoder self-attention fwd+bwd bf16: T=512, B=32, E=1024, 16 heads, key-padding lengths U[256,512], "
+                   "softmax dropout 0.1 (explicit mask)")
+    T, B, E, H = 512, 32, 1024, 16
+
+    def setup(self, dev):
+        from oracle import inputs
+        from nmtgminor_amd.native import self_multihead_attn_blaslt as m
+        self.m = m
+        d = inputs.self_attn_inputs(self.T, self.B, self.E, self.H)
+        self.cpu = d
+        g = lambda k: d[k].to(dev)
+        self.x, self.w_in, self.w_out, self.b_in, self.b_out = g("x"), g("w_in"), g("w_out"), g("b_in"), g("b_out")
+        self.pad, self.dm, self.dout = g("pad_mask"), g("dropout_mask"), g("dout")
+
+    def step(self):
+        lin, scores, dropped, dmask, ctx, out = self.m.forward(False, True, self.H, self.x, self.w_in, self.w_out, self.b_in,
+                                                               self.b_out, self.pad, 0.1, dropout_mask=self.dm)
+        return self.m.backward(False, self.H, self.dout, ctx, dropped, scores, lin, self.x, self.w_in, self.w_out, dmask, 0.1)
+
+    def _flops_fwd(self):
+        t, b, e, h = self.T, self.B, self.E, self.H
+        tok = t * b
+        return 2.0 * tok * e * 3 * e + 2 * (2.0 * b * h * t * t * (e // h)) + 2.0 * tok * e * e
+
+    def work_per_step(self):
+        return 3 * self._flops_fwd()
+
+    def kernel_work(self):
+        return {"gemm_": self.work_per_step()}
+
+    def cpu_baseline(self):
+        from oracle import attention as o
+        d = self.cpu
+        nb = 2                                                   # batch columns are independent
+        sl = lambda z: z[:, :nb].float()
+        x, dout = sl(d["x"]), sl(d["dout"])
+        w_in, w_out, b_in, b_out = (d[k].float() for k in ("w_in", "w_out", "b_in", "b_out"))
+        pad, dm = d["pad_mask"][:nb], d["dropout_mask"][:nb * self.H]
+
+        def run():
+            f = o.self_attn_fwd(x, w_in, w_out, b_in, b_out, self.H, pad, None, 0.1, dm)
+            o.self_attn_bwd(dout, x, w_in, w_out, self.H, f, 0.1, dm)
+        t = _time_cpu(run, 3)
+        return dict(value=self.work_per_step() * nb / self.B / t / 1e12, unit="TFLOP/s", cores=torch.get_num_threads(),
+                    kind="port", sample=f"{nb} of {self.B} batch columns (independent), fp32 on the bf16-rounded values, median of 3")
+
+
+class EncdecAttnWL(Workload):
+    name = "encdec_attn"
+    bound = "mfma"
+    dtype = "bf16"
+    description = ("decoder layer attention fwd bf16: cross-attention Tq=128 over Tk=1500 (B=16, E=1024, 16 heads, key lengths "
+                   "U[750,1500]) + causal self-attention T=128; eval (no dropout)")
+    TQ, TK, B, E, H = 128, 1500, 16, 1024, 16
+
+    def setup(self, dev):
+        from oracle import inputs
+        from nmtgminor_amd.native import encdec_multihead_attn_bias_blaslt as m, self_multihead_attn_blaslt as sm
+        self.m, self.sm = m, sm
+        d = inputs.encdec_attn_inputs(self.TQ, self.TK, self.B, self.E, self.H)
+        s = inputs.self_attn_inputs(self.TQ, self.B, self.E, self.H, p=0.0, seed=1004, causal=True)
+        self.cpu, self.cpu_self = d, s
+        self.a = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in d.items()}
+        self.s = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in s.items()}
+
+    def step(self):
+        s, a = self.s, self.a
+        r1 = self.sm.forward(True, False, self.H, s["x"], s["w_in"], s["w_out"], s["b_in"], s["b_out"], s["time_mask"], 0.0)
+        r2 = self.m.forward(False, self.H, a["x_q"], a["x_kv"], a["w_q"], a["w_kv"], a["w_out"], a["b_q"], a["b_kv"],
+                            a["b_out"], a["pad_mask"], 0.0)
+        return r1[-1], r2[-1]
+
+    def work_per_step(self):
+        tq, tk, b, e, h = self.TQ, self.TK, self.B, self.E, self.H
+        d = e // h
+        cross = 2.0 * tq * b * e * e + 2.0 * tk * b * e * 2 * e + 2 * (2.0 * b * h * tq * tk * d) + 2.0 * tq * b * e * e
+        self_ = 2.0 * tq * b * e * 3 * e + 2 * (2.0 * b * h * tq * tq * d) + 2.0 * tq * b * e * e
+        return cross + self_
+
+    def kernel_work(self):
+        return {"gemm_": self.work_per_step()}
+
+    def cpu_baseline(self):
+        from oracle import attention as o
+        d, s = self.cpu, self.cpu_self
+        f = lambda z: z.float() if z is not None and z.is_floating_point() else z
+
+        def run():
+            o.self_attn_fwd(f(s["x"]), f(s["w_in"]), f(s["w_out"]), f(s["b_in"]), f(s["b_out"]), self.H, None, s["time_mask"])
+            o.encdec_attn_fwd(f(d["x_q"]), f(d["x_kv"]), f(d["w_q"]), f(d["w_kv"]), f(d["w_out"]), f(d["b_q"]), f(d["b_kv"]),
+                              f(d["b_out"]), self.H, d["pad_mask"])
+        t = _time_cpu(run, 3)
+        return dict(value=self.work_per_step() / t / 1e12, unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
+                    sample="full workload in fp32 on the bf16-rounded values, median of 3")
+
+
+WORKLOADS = {w.name: w for w in (LayerNormWL, MlpWL, SelfAttnWL, EncdecAttnWL, XentropyWL)}
 PRIMARY = "mlp"
 
 
