@@ -67,13 +67,11 @@ template <> struct elem<bf16_t> {
   static __device__ __forceinline__ float to_float(bf16_t v) {
     return __uint_as_float(static_cast<uint32_t>(v.bits) << 16);
   }
-  // round-to-nearest-even, NaN kept quiet
+  // round-to-nearest-even in hardware (v_cvt_pk_bf16_f32 on gfx950)
   static __device__ __forceinline__ bf16_t from_float(float v) {
-    uint32_t u = __float_as_uint(v);
+    const __bf16 b = static_cast<__bf16>(v);
     bf16_t r;
-    if ((u & 0x7fffffffu) > 0x7f800000u) { r.bits = static_cast<uint16_t>((u >> 16) | 0x40u); return r; }
-    u += 0x7fffu + ((u >> 16) & 1u);
-    r.bits = static_cast<uint16_t>(u >> 16);
+    r.bits = __builtin_bit_cast(uint16_t, b);
     return r;
   }
 };

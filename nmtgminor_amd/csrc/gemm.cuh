@@ -27,6 +27,7 @@
 //     round-robin) works on a contiguous run of tiles and re-uses A / B through its own L2.
 #pragma once
 #include "common.cuh"
+#include <type_traits>
 
 namespace nmtg {
 
@@ -48,7 +49,7 @@ struct GemmArgs {
   int batch;
   int splits, k_per_split;
   float alpha;
-  int a_vec, b_vec, c_vec;  // widest legal vector (in elements: 8, 4 or 1) on each side
+  int vec;                  // widest access (elements: 8, 4 or 1) every operand and extent allows
   const void* bias;
   void* aux_out;
   const void* aux_in;
@@ -63,7 +64,16 @@ struct GemmArgs {
   int kmask_kind, heads;
   float* ws;
   int m_tiles, n_tiles;
+#ifdef NMTG_GEMM_PROF
+  long long* prof;          // per-block phase timestamps (tuning builds only)
+#endif
 };
+
+#ifdef NMTG_GEMM_PROF
+#define NMTG_PROF_MARK(i) do { if (g.prof != nullptr && threadIdx.x == 0) g.prof[(static_cast<long long>(blockIdx.y) * gridDim.x + blockIdx.x) * 8 + (i)] = clock64(); } while (0)
+#else
+#define NMTG_PROF_MARK(i) do { } while (0)
+#endif
 
 template <typename T> struct mfma;
 typedef float acc16_t __attribute__((ext_vector_type(16)));
@@ -85,114 +95,230 @@ constexpr int GEMM_BK = 64;
 __device__ __forceinline__ int lds_swz(int row) { return (row ^ (row >> 3)) & 7; }
 
 // Activation and derivative (fp32 math). Codes are nmtg_act.
-__device__ __forceinline__ float act_apply(float h, int act) {
+//
+// The exact-erf gelu is the hot one (it runs on every hidden activation inside the GEMM
+// epilogue), so the normal CDF uses the rational approximation 7.1.26 of Abramowitz & Stegun,
+//   erfc(z) = (a1 t + a2 t^2 + a3 t^3 + a4 t^4 + a5 t^5) exp(-z^2),  t = 1 / (1 + p z),  z >= 0,
+// absolute error < 1.5e-7 (fp32 rounding level, far inside the 16-bit output precision), at
+// about a third of the instructions of erff(); Phi and the density share the one exponential.
+struct NormalCdfPdf { float cdf, pdf; };
+__device__ __forceinline__ NormalCdfPdf normal_cdf_pdf(float h) {
+  const float z = fabsf(h) * 0.70710678118654752f;
+  const float t = __frcp_rn(fmaf(0.3275911f, z, 1.f));
+  // coefficients pre-multiplied by 1/2: half_erfc = 0.5 * erfc(z)
+  float poly = fmaf(0.5f * 1.061405429f, t, 0.5f * -1.453152027f);
+  poly = fmaf(poly, t, 0.5f * 1.421413741f);
+  poly = fmaf(poly, t, 0.5f * -0.284496736f);
+  poly = fmaf(poly, t, 0.5f * 0.254829592f);
+  const float e = exp2f(h * h * -0.72134752044448170f);  // exp(-h^2 / 2)
+  const float half_erfc = poly * t * e;
+  NormalCdfPdf r;
+  r.cdf = h >= 0.f ? 1.f - half_erfc : half_erfc;
+  r.pdf = 0.3989422804014327f * e;
+  return r;
+}
+
+template <int ACT>
+__device__ __forceinline__ float act_apply(float h) {
+  if constexpr (ACT == NMTG_ACT_RELU) return fmaxf(h, 0.f);
+  else if constexpr (ACT == NMTG_ACT_GELU) return h * normal_cdf_pdf(h).cdf;
+  else if constexpr (ACT == NMTG_ACT_SILU) return h * __frcp_rn(1.f + exp2f(h * -1.4426950408889634f));
+  else if constexpr (ACT == NMTG_ACT_AGELU) {
+    // 0.5 h (1 + tanh u) = h * sigmoid(2u)
+    const float u2 = 1.5957691216057308f * (h + 0.044715f * h * h * h);
+    return h * __frcp_rn(1.f + exp2f(u2 * -1.4426950408889634f));
+  } else return h;
+}
+template <int ACT>
+__device__ __forceinline__ float act_grad(float h) {
+  if constexpr (ACT == NMTG_ACT_RELU) return h > 0.f ? 1.f : 0.f;
+  else if constexpr (ACT == NMTG_ACT_GELU) {
+    const NormalCdfPdf n = normal_cdf_pdf(h);
+    return fmaf(h, n.pdf, n.cdf);
+  } else if constexpr (ACT == NMTG_ACT_SILU) {
+    const float s = __frcp_rn(1.f + exp2f(h * -1.4426950408889634f));
+    return s * (1.f + h * (1.f - s));
+  } else if constexpr (ACT == NMTG_ACT_AGELU) {
+    // d/dh [h s(2u)] = s + h s (1 - s) 2u',  u' = k (1 + 3 c h^2)
+    const float u2 = 1.5957691216057308f * (h + 0.044715f * h * h * h);
+    const float sg = __frcp_rn(1.f + exp2f(u2 * -1.4426950408889634f));
+    return sg + h * sg * (1.f - sg) * 1.5957691216057308f * (1.f + 0.134145f * h * h);
+  } else return 1.f;
+}
+
+// Calls f(std::integral_constant<int, ACT>) for the runtime activation code: one uniform branch
+// outside the element loops instead of a switch per element.
+template <typename F>
+__device__ __forceinline__ void dispatch_act(int act, F&& f) {
   switch (act) {
-    case NMTG_ACT_RELU: return fmaxf(h, 0.f);
-    case NMTG_ACT_GELU: return 0.5f * h * (1.f + erff(h * 0.70710678118654752f));
-    case NMTG_ACT_SILU: return h / (1.f + __expf(-h));
-    case NMTG_ACT_AGELU: {
-      const float u = 0.7978845608028654f * (h + 0.044715f * h * h * h);
-      return 0.5f * h * (1.f + tanhf(u));
-    }
-    default: return h;
+    case NMTG_ACT_RELU: f(std::integral_constant<int, NMTG_ACT_RELU>{}); break;
+    case NMTG_ACT_GELU: f(std::integral_constant<int, NMTG_ACT_GELU>{}); break;
+    case NMTG_ACT_SILU: f(std::integral_constant<int, NMTG_ACT_SILU>{}); break;
+    case NMTG_ACT_AGELU: f(std::integral_constant<int, NMTG_ACT_AGELU>{}); break;
+    default: f(std::integral_constant<int, NMTG_ACT_NONE>{}); break;
   }
 }
-__device__ __forceinline__ float act_grad(float h, int act) {
-  switch (act) {
-    case NMTG_ACT_RELU: return h > 0.f ? 1.f : 0.f;
-    case NMTG_ACT_GELU: {
-      const float cdf = 0.5f * (1.f + erff(h * 0.70710678118654752f));
-      const float pdf = 0.3989422804014327f * __expf(-0.5f * h * h);
-      return cdf + h * pdf;
-    }
-    case NMTG_ACT_SILU: {
-      const float s = 1.f / (1.f + __expf(-h));
-      return s * (1.f + h * (1.f - s));
-    }
-    case NMTG_ACT_AGELU: {
-      const float k = 0.7978845608028654f;
-      const float t = tanhf(k * (h + 0.044715f * h * h * h));
-      return 0.5f * (1.f + t) + 0.5f * h * (1.f - t * t) * k * (1.f + 0.134145f * h * h);
-    }
-    default: return 1.f;
+
+// ---------------------------------------------------------------------------------------------
+// Vector-width-templated, branch-free global accesses. VEC (8, 4 or 1 elements) is the widest
+// access every operand of the call allows; a group of 8 elements moves as 8/VEC accesses, each
+// with its own validity bit. Out-of-range loads read a clamped (always mapped) address and are
+// zeroed by a select, so the loads of a tile are straight-line code the compiler can issue back
+// to back.
+// ---------------------------------------------------------------------------------------------
+template <int VEC> struct raw_vec;
+template <> struct raw_vec<8> { typedef uint4 type; };
+template <> struct raw_vec<4> { typedef uint2 type; };
+template <> struct raw_vec<1> { typedef uint16_t type; };
+
+// Loads elements [0, 8) at p (element e valid iff e < nvalid, nvalid a multiple of VEC or >= 8);
+// `safe` is any mapped address of the same alignment class.
+template <int VEC, bool ZERO = true>
+__device__ __forceinline__ uint4 load8(const uint16_t* __restrict__ p, const uint16_t* __restrict__ safe, int nvalid) {
+  typedef typename raw_vec<VEC>::type R;
+  union { uint4 v; R r[8 / VEC]; } u;
+#pragma unroll
+  for (int h = 0; h < 8 / VEC; ++h) {
+    const bool ok = h * VEC < nvalid;
+    R val = *reinterpret_cast<const R*>(ok ? p + h * VEC : safe);
+    if (ZERO && !ok) val = R{};
+    u.r[h] = val;
   }
+  return u.v;
+}
+
+template <int VEC>
+__device__ __forceinline__ void store8(uint16_t* __restrict__ p, const uint4& v, int nvalid) {
+  typedef typename raw_vec<VEC>::type R;
+  union { uint4 v; R r[8 / VEC]; } u;
+  u.v = v;
+#pragma unroll
+  for (int h = 0; h < 8 / VEC; ++h)
+    if (h * VEC < nvalid) *reinterpret_cast<R*>(p + h * VEC) = u.r[h];
+}
+
+template <int VEC>
+__device__ __forceinline__ uint2 load8_bytes(const uint8_t* __restrict__ p, const uint8_t* __restrict__ safe, int nvalid) {
+  if constexpr (VEC == 8) {
+    const bool ok = nvalid > 0;
+    uint2 v = *reinterpret_cast<const uint2*>(ok ? p : safe);
+    if (!ok) v = make_uint2(0, 0);
+    return v;
+  } else if constexpr (VEC == 4) {
+    uint2 v;
+    const bool ok0 = nvalid > 0, ok1 = nvalid > 4;
+    v.x = *reinterpret_cast<const uint32_t*>(ok0 ? p : safe);
+    v.y = *reinterpret_cast<const uint32_t*>(ok1 ? p + 4 : safe);
+    if (!ok0) v.x = 0;
+    if (!ok1) v.y = 0;
+    return v;
+  } else {
+    uint32_t w[2] = {0, 0};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const bool ok = e < nvalid;
+      uint32_t b = *(ok ? p + e : safe);
+      if (!ok) b = 0;
+      w[e >> 2] |= b << (8 * (e & 3));
+    }
+    return make_uint2(w[0], w[1]);
+  }
+}
+
+template <int VEC>
+__device__ __forceinline__ void store8_bytes(uint8_t* __restrict__ p, uint2 v, int nvalid) {
+  if constexpr (VEC == 8) {
+    if (nvalid > 0) *reinterpret_cast<uint2*>(p) = v;
+  } else if constexpr (VEC == 4) {
+    if (nvalid > 0) *reinterpret_cast<uint32_t*>(p) = v.x;
+    if (nvalid > 4) *reinterpret_cast<uint32_t*>(p + 4) = v.y;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      if (e < nvalid) p[e] = static_cast<uint8_t>(((e < 4 ? v.x : v.y) >> (8 * (e & 3))) & 0xffu);
+  }
+}
+
+__device__ __forceinline__ uint8_t byte_of(uint2 v, int e) { return ((e < 4 ? v.x : v.y) >> (8 * (e & 3))) & 0xffu; }
+
+template <typename T>
+__device__ __forceinline__ void unpack8(const uint4& raw, float (&v)[8]) {
+  const T* e = reinterpret_cast<const T*>(&raw);
+#pragma unroll
+  for (int k = 0; k < 8; ++k) v[k] = elem<T>::to_float(e[k]);
+}
+template <typename T>
+__device__ __forceinline__ uint4 pack8(const float (&v)[8]) {
+  uint4 raw;
+  T* e = reinterpret_cast<T*>(&raw);
+#pragma unroll
+  for (int k = 0; k < 8; ++k) e[k] = elem<T>::from_float(v[k]);
+  return raw;
 }
 
 // ---------------------------------------------------------------------------------------------
 // Global -> register -> LDS staging of one operand tile [ROWS][64 k].
 // ---------------------------------------------------------------------------------------------
-template <typename T, int ROWS, int NT, bool KC>
+template <typename T, int ROWS, int NT, bool KC, int VEC>
 struct TileStage {
   static constexpr int UNITS = KC ? ROWS * 8 : ROWS * 2;  // 16-byte chunks (KC) or 4k x 8row blocks (MC)
   static constexpr int PER = (UNITS + NT - 1) / NT;
   static constexpr int NREG = KC ? PER : PER * 4;
+  static constexpr int RG8 = ROWS / 64 > 0 ? ROWS / 64 : 1;
+  // With 16-byte accesses a register is wholly valid or wholly out of range: the loads leave
+  // out-of-range registers unzeroed and remember them in `valid`; store() zeroes them. That keeps
+  // every use of a loaded value (and so the wait for it) behind the MFMA work of the step.
+  static constexpr bool DEFER = VEC == 8;
   uint4 regs[NREG];
+  uint32_t valid;
 
   // base: operand pointer for this batch; rows_total / row0: extent and tile origin in the row
   // index; k0: first k of this step; kend: one past the last valid k.
   __device__ __forceinline__ void load(const T* __restrict__ base, int64_t ld, int rows_total, int row0, int k0,
-                                       int kend, int vec, int tid) {
+                                       int kend, int tid) {
+    const uint16_t* b16 = reinterpret_cast<const uint16_t*>(base);
+    valid = 0;
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int q = tid + i * NT;
       if constexpr (KC) {
-        uint4 v = make_uint4(0, 0, 0, 0);
         const int row = q >> 3, c = q & 7;
         const int grow = row0 + row, gk = k0 + c * 8;
-        if (q < UNITS && grow < rows_total && gk < kend) {
-          const T* p = base + static_cast<int64_t>(grow) * ld + gk;
-          if (vec == 8 && gk + 8 <= kend) {
-            v = *reinterpret_cast<const uint4*>(p);
-          } else if (vec >= 4 && gk + 8 <= kend) {
-            const uint2 lo = *reinterpret_cast<const uint2*>(p), hi = *reinterpret_cast<const uint2*>(p + 4);
-            v = make_uint4(lo.x, lo.y, hi.x, hi.y);
-          } else {
-            uint16_t e[8];
-#pragma unroll
-            for (int j = 0; j < 8; ++j) e[j] = (gk + j < kend) ? reinterpret_cast<const uint16_t*>(p)[j] : 0;
-            v = make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16));
-          }
-        }
-        regs[i] = v;
+        const bool ok = (UNITS % NT == 0 || q < UNITS) && grow < rows_total;
+        const int nvalid = ok ? kend - gk : 0;
+        regs[i] = load8<VEC, !DEFER>(b16 + static_cast<int64_t>(ok ? grow : 0) * ld + (nvalid > 0 ? gk : 0), b16, nvalid);
+        if (nvalid > 0) valid |= 1u << i;
       } else {
-        constexpr int RG8 = ROWS / 64 > 0 ? ROWS / 64 : 1;
         const int rg_lo = q & 7, kq_lo = (q >> 3) & 1, rest = q >> 4;
         const int rg = rg_lo + 8 * (rest % RG8), kq = kq_lo + 2 * (rest / RG8);
         const int grow = row0 + rg * 8;
+        const bool qok = (UNITS % NT == 0 || q < UNITS);
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) {
-          uint4 v = make_uint4(0, 0, 0, 0);
           const int gk = k0 + kq * 4 + kk;
-          if (q < UNITS && gk < kend && grow < rows_total) {
-            const T* p = base + static_cast<int64_t>(gk) * ld + grow;
-            if (vec == 8 && grow + 8 <= rows_total) {
-              v = *reinterpret_cast<const uint4*>(p);
-            } else if (vec >= 4 && grow + 8 <= rows_total) {
-              const uint2 lo = *reinterpret_cast<const uint2*>(p), hi = *reinterpret_cast<const uint2*>(p + 4);
-              v = make_uint4(lo.x, lo.y, hi.x, hi.y);
-            } else {
-              uint16_t e[8];
-#pragma unroll
-              for (int j = 0; j < 8; ++j) e[j] = (grow + j < rows_total) ? reinterpret_cast<const uint16_t*>(p)[j] : 0;
-              v = make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16));
-            }
-          }
-          regs[i * 4 + kk] = v;
+          const bool ok = qok && gk < kend;
+          const int nvalid = ok ? rows_total - grow : 0;
+          regs[i * 4 + kk] = load8<VEC, !DEFER>(b16 + static_cast<int64_t>(ok ? gk : 0) * ld + (nvalid > 0 ? grow : 0), b16, nvalid);
+          if (nvalid > 0) valid |= 1u << (i * 4 + kk);
         }
       }
     }
   }
 
-  __device__ __forceinline__ void store(T* __restrict__ buf, int tid) const {
+  __device__ __forceinline__ void store(T* __restrict__ buf, int tid) {
+    if constexpr (DEFER) {
+#pragma unroll
+      for (int r = 0; r < NREG; ++r)
+        if (!((valid >> r) & 1u)) regs[r] = make_uint4(0, 0, 0, 0);
+    }
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int q = tid + i * NT;
-      if (q >= UNITS) continue;
+      if (UNITS % NT != 0 && q >= UNITS) continue;
       if constexpr (KC) {
         const int row = q >> 3, c = q & 7;
         *reinterpret_cast<uint4*>(buf + row * GEMM_BK + ((c ^ lds_swz(row)) * 8)) = regs[i];
       } else {
-        constexpr int RG8 = ROWS / 64 > 0 ? ROWS / 64 : 1;
         const int rg_lo = q & 7, kq_lo = (q >> 3) & 1, rest = q >> 4;
         const int rg = rg_lo + 8 * (rest % RG8), kq = kq_lo + 2 * (rest / RG8);
         const uint32_t* w0 = reinterpret_cast<const uint32_t*>(&regs[i * 4 + 0]);
@@ -224,7 +350,7 @@ constexpr int gemm_lds_bytes() {
   return main_loop > c_tile ? main_loop : c_tile;
 }
 
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC, int EPI>
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC, int EPI, int VEC>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const GemmArgs g) {
   constexpr int NT = 64 * WAVES_M * WAVES_N;
   constexpr int BK = GEMM_BK;
@@ -238,11 +364,18 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const Gemm
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm0 = (wave / WAVES_N) * WTM, wn0 = (wave % WAVES_N) * WTN;
 
-  // tile coordinates, XCD-aware
+  // Tile coordinates. Consecutive block ids go round-robin to the 8 XCDs (each with its own L2), so
+  // block ids are first regrouped to give every XCD a contiguous run of the tile order, and the
+  // tile order itself walks groups of GM tile rows column by column: the ~32 tiles an XCD runs at
+  // once then form a GM x 32/GM patch and share their A / B panels through that XCD's L2.
   int bid = blockIdx.x;
   const int ntile = g.m_tiles * g.n_tiles;
   if ((ntile & 7) == 0) bid = (bid & 7) * (ntile >> 3) + (bid >> 3);
-  const int tile_m = bid / g.n_tiles, tile_n = bid % g.n_tiles;
+  constexpr int GM = 4;
+  const int in_group = GM * g.n_tiles;
+  const int first_m = (bid / in_group) * GM;
+  const int gsize = min(g.m_tiles - first_m, GM);
+  const int tile_m = first_m + (bid % in_group) % gsize, tile_n = (bid % in_group) / gsize;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int bz = blockIdx.y, split = blockIdx.z;
 
@@ -260,22 +393,39 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const Gemm
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  TileStage<T, BM, NT, A_KC> stA;
-  TileStage<T, BN, NT, B_KC> stB;
+  TileStage<T, BM, NT, A_KC, VEC> stA;
+  TileStage<T, BN, NT, B_KC, VEC> stB;
 
+  NMTG_PROF_MARK(0);
   if (nk > 0) {
-    stA.load(A, g.lda, g.M, m0, kbeg, kend, g.a_vec, tid);
-    stB.load(B, g.ldb, g.N, n0, kbeg, kend, g.b_vec, tid);
+    stA.load(A, g.lda, g.M, m0, kbeg, kend, tid);
+    stB.load(B, g.ldb, g.N, n0, kbeg, kend, tid);
     stA.store(sA, tid);
     stB.store(sB, tid);
   }
   __syncthreads();
 
+  NMTG_PROF_MARK(1);
+  // per-lane LDS offsets of the MFMA fragments (elements), constant over the K loop
+  int offA[TM][2], offB[TN][2];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int row = wm0 + i * 32 + (lane & 31);
+    offA[i][0] = row * BK;
+    offA[i][1] = lds_swz(row);
+  }
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int row = wn0 + j * 32 + (lane & 31);
+    offB[j][0] = row * BK;
+    offB[j][1] = lds_swz(row);
+  }
+
   for (int kt = 0; kt < nk; ++kt) {
     const int cur = kt & 1;
     if (kt + 1 < nk) {
-      stA.load(A, g.lda, g.M, m0, kbeg + (kt + 1) * BK, kend, g.a_vec, tid);
-      stB.load(B, g.ldb, g.N, n0, kbeg + (kt + 1) * BK, kend, g.b_vec, tid);
+      stA.load(A, g.lda, g.M, m0, kbeg + (kt + 1) * BK, kend, tid);
+      stB.load(B, g.ldb, g.N, n0, kbeg + (kt + 1) * BK, kend, tid);
     }
     const T* cA = sA + cur * BM * BK;
     const T* cB = sB + cur * BN * BK;
@@ -284,15 +434,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const Gemm
       uint4 fm[TM], fn[TN];
       const int c = kk * 2 + (lane >> 5);
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const int row = wm0 + i * 32 + (lane & 31);
-        fm[i] = *reinterpret_cast<const uint4*>(cA + row * BK + ((c ^ lds_swz(row)) * 8));
-      }
+      for (int i = 0; i < TM; ++i) fm[i] = *reinterpret_cast<const uint4*>(cA + offA[i][0] + ((c ^ offA[i][1]) * 8));
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int row = wn0 + j * 32 + (lane & 31);
-        fn[j] = *reinterpret_cast<const uint4*>(cB + row * BK + ((c ^ lds_swz(row)) * 8));
-      }
+      for (int j = 0; j < TN; ++j) fn[j] = *reinterpret_cast<const uint4*>(cB + offB[j][0] + ((c ^ offB[j][1]) * 8));
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -305,6 +449,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const Gemm
     __syncthreads();
   }
 
+  NMTG_PROF_MARK(2);
   // Lane (l) register r of tile (i, j) holds C[m][n] with
   //   m = m0 + wm0 + 32 i + (l & 31),   n = n0 + wn0 + 32 j + 8 (r / 4) + 4 (l >> 5) + (r % 4).
   if constexpr (EPI == EPI_SPLITK) {
@@ -332,9 +477,17 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const Gemm
         const int nl = wn0 + j * 32 + q * 8 + (lane >> 5) * 4;
         float bv[4] = {0.f, 0.f, 0.f, 0.f};
         if (EPI != EPI_ACT_BWD && bias != nullptr) {
+          // clamped, branch-free loads (columns past N are never stored)
+          const int nn = n0 + nl;
+          if constexpr (VEC >= 4) {
+            const uint2 raw = *reinterpret_cast<const uint2*>(bias + (nn < g.N ? nn : 0));
+            const T* e4 = reinterpret_cast<const T*>(&raw);
 #pragma unroll
-          for (int e = 0; e < 4; ++e)
-            if (n0 + nl + e < g.N) bv[e] = elem<T>::to_float(bias[n0 + nl + e]);
+            for (int e = 0; e < 4; ++e) bv[e] = elem<T>::to_float(e4[e]);
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) bv[e] = elem<T>::to_float(bias[min(nn + e, g.N - 1)]);
+          }
         }
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
@@ -347,111 +500,120 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const Gemm
       }
     }
     __syncthreads();
+    NMTG_PROF_MARK(3);
 
     // ---- phase 2: row-contiguous 8-element chunks, coalesced global traffic ----
     constexpr int CPR = BN / 8;        // chunks per tile row
     constexpr int RPP = NT / CPR;      // rows per pass
-    static_assert(NT % CPR == 0 && BM % RPP == 0, "epilogue mapping");
+    constexpr int PASSES = BM / RPP;
+    constexpr int GRP = PASSES < 8 ? PASSES : 8;   // passes whose side loads are issued together
+    static_assert(NT % CPR == 0 && BM % RPP == 0 && PASSES % GRP == 0, "epilogue mapping");
     const int cc = tid % CPR, r_in = tid / CPR;
     const int n = n0 + cc * 8;
-    T* C = static_cast<T*>(g.C) + static_cast<int64_t>(bz) * g.sC;
+    const int ncols = g.N - n;         // valid columns of this lane's chunk (<= 0: none)
+    uint16_t* C = reinterpret_cast<uint16_t*>(g.C) + static_cast<int64_t>(bz) * g.sC;
+    uint16_t* AUX = reinterpret_cast<uint16_t*>(g.aux_out);
+    if (AUX != nullptr) AUX += static_cast<int64_t>(bz) * g.sC;
+    const uint16_t* HIN = reinterpret_cast<const uint16_t*>(g.aux_in);
     float csum[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    const int nvalid = min(8, g.N - n);
+    const bool use_dmask = (EPI == EPI_ACT_FWD || EPI == EPI_ACT_BWD) && g.dmask != nullptr;
+    const bool dmask_in = use_dmask && !(EPI == EPI_ACT_FWD && g.rng);
+    const bool tmask = EPI == EPI_SCORES && g.kmask_kind == 2;
+    uint2 padm = make_uint2(0, 0);
+    if (EPI == EPI_SCORES && g.kmask_kind == 1)
+      padm = load8_bytes<VEC>(g.kmask + static_cast<int64_t>(bz / g.heads) * g.N + n, g.kmask, ncols);
 
-    auto store8 = [&](T* dst, const float (&v)[8]) {
-      if (nvalid == 8 && g.c_vec == 8) {
-        store_pack<T, 8>(dst, v);
-      } else if (nvalid == 8 && g.c_vec >= 4) {
-        const float lo[4] = {v[0], v[1], v[2], v[3]}, hi[4] = {v[4], v[5], v[6], v[7]};
-        store_pack<T, 4>(dst, lo);
-        store_pack<T, 4>(dst + 4, hi);
-      } else {
-        for (int e = 0; e < nvalid; ++e) dst[e] = elem<T>::from_float(v[e]);
+    auto phase2 = [&](auto act_tag) {
+    constexpr int ACT = decltype(act_tag)::value;
+    for (int p0 = 0; p0 < PASSES; p0 += GRP) {
+      // side inputs of GRP passes first (independent loads in flight together), then the math and stores
+      uint4 hraw[GRP];
+      uint2 mraw[GRP];
+#pragma unroll
+      for (int u = 0; u < GRP; ++u) {
+        const int m = m0 + (p0 + u) * RPP + r_in;
+        const int nv = m < g.M ? ncols : 0;
+        if constexpr (EPI == EPI_ACT_BWD)
+          hraw[u] = load8<VEC>(HIN + static_cast<int64_t>(m < g.M ? m : 0) * g.ld_aux + (nv > 0 ? n : 0), HIN, nv);
+        if (dmask_in) mraw[u] = load8_bytes<VEC>(g.dmask + static_cast<int64_t>(m < g.M ? m : 0) * g.N + (nv > 0 ? n : 0), g.dmask, nv);
+        else if (tmask) mraw[u] = load8_bytes<VEC>(g.kmask + static_cast<int64_t>(m < g.M ? m : 0) * g.N + (nv > 0 ? n : 0), g.kmask, nv);
+        else mraw[u] = make_uint2(0x01010101u, 0x01010101u);
       }
-    };
-    auto load8 = [&](const T* src, float (&v)[8]) {
-      if (nvalid == 8 && g.c_vec == 8) {
-        load_pack<T, 8>(src, v);
-      } else {
-        for (int e = 0; e < 8; ++e) v[e] = e < nvalid ? elem<T>::to_float(src[e]) : 0.f;
-      }
-    };
-
-    if (nvalid > 0) {
-#pragma unroll 4
-      for (int p = 0; p < BM / RPP; ++p) {
-        const int ml = p * RPP + r_in;
+#pragma unroll
+      for (int u = 0; u < GRP; ++u) {
+        const int ml = (p0 + u) * RPP + r_in;
         const int m = m0 + ml;
-        if (m >= g.M) break;
+        const int nv = m < g.M ? ncols : 0;
         float v[8];
         {
           const uint2* s = reinterpret_cast<const uint2*>(sC + ml * PITCH + cc * 16);
           const uint2 lo = s[0], hi = s[1];
-          const uint4 raw = make_uint4(lo.x, lo.y, hi.x, hi.y);
-          const T* e = reinterpret_cast<const T*>(&raw);
-#pragma unroll
-          for (int k = 0; k < 8; ++k) v[k] = elem<T>::to_float(e[k]);
+          unpack8<T>(make_uint4(lo.x, lo.y, hi.x, hi.y), v);
         }
         const int64_t off = static_cast<int64_t>(m) * g.ldc + n;
         if constexpr (EPI == EPI_PLAIN) {
-          store8(C + off, v);
+          store8<VEC>(C + off, pack8<T>(v), nv);
         } else if constexpr (EPI == EPI_ACT_FWD) {
-          if (g.aux_out != nullptr) store8(static_cast<T*>(g.aux_out) + static_cast<int64_t>(bz) * g.sC + off, v);
+          if (AUX != nullptr) store8<VEC>(AUX + off, pack8<T>(v), nv);
           float a[8];
 #pragma unroll
-          for (int k = 0; k < 8; ++k) a[k] = act_apply(v[k], g.act);
-          if (g.dmask != nullptr) {
-            uint8_t* mk = const_cast<uint8_t*>(g.dmask) + static_cast<int64_t>(m) * g.N + n;
-            uint8_t keep[8];
+          for (int k = 0; k < 8; ++k) a[k] = act_apply<ACT>(v[k]);
+          if (use_dmask) {
+            uint2 keep = mraw[u];
             if (g.rng) {
+              uint8_t kb[8];
               const uint64_t first = static_cast<uint64_t>(m) * g.N + n;
               if ((g.N & 3) == 0) {
-                philox_keep<8>(Philox(g.seed), first, g.offset, g.keep_p, keep);
+                philox_keep<8>(Philox(g.seed), first, g.offset, g.keep_p, kb);
               } else {
+#pragma unroll
                 for (int k = 0; k < 8; ++k) {
                   uint8_t one[1];
                   philox_keep<1>(Philox(g.seed), first + k, g.offset, g.keep_p, one);
-                  keep[k] = one[0];
+                  kb[k] = one[0];
                 }
               }
-              if (nvalid == 8 && (g.N & 7) == 0) store_bytes<8>(mk, keep);
-              else for (int k = 0; k < nvalid; ++k) mk[k] = keep[k];
-            } else {
-              if (nvalid == 8 && (g.N & 7) == 0) load_bytes<8>(mk, keep);
-              else for (int k = 0; k < 8; ++k) keep[k] = k < nvalid ? mk[k] : 0;
+              keep.x = kb[0] | (kb[1] << 8) | (kb[2] << 16) | (static_cast<uint32_t>(kb[3]) << 24);
+              keep.y = kb[4] | (kb[5] << 8) | (kb[6] << 16) | (static_cast<uint32_t>(kb[7]) << 24);
+              store8_bytes<VEC>(const_cast<uint8_t*>(g.dmask) + static_cast<int64_t>(m) * g.N + n, keep, nv);
             }
 #pragma unroll
-            for (int k = 0; k < 8; ++k) a[k] = keep[k] ? a[k] * g.dscale : 0.f;
+            for (int k = 0; k < 8; ++k) a[k] = byte_of(keep, k) ? a[k] * g.dscale : 0.f;
           }
-          store8(C + off, a);
+          store8<VEC>(C + off, pack8<T>(a), nv);
         } else if constexpr (EPI == EPI_ACT_BWD) {
           float h[8];
-          load8(static_cast<const T*>(g.aux_in) + static_cast<int64_t>(m) * g.ld_aux + n, h);
+          unpack8<T>(hraw[u], h);
 #pragma unroll
-          for (int k = 0; k < 8; ++k) v[k] *= act_grad(h[k], g.act) * g.dscale;
-          if (g.dmask != nullptr) {
-            const uint8_t* mk = g.dmask + static_cast<int64_t>(m) * g.N + n;
-            uint8_t keep[8];
-            if (nvalid == 8 && (g.N & 7) == 0) load_bytes<8>(mk, keep);
-            else for (int k = 0; k < 8; ++k) keep[k] = k < nvalid ? mk[k] : 0;
+          for (int k = 0; k < 8; ++k) v[k] *= act_grad<ACT>(h[k]) * g.dscale;
+          if (use_dmask) {
 #pragma unroll
-            for (int k = 0; k < 8; ++k) v[k] = keep[k] ? v[k] : 0.f;
+            for (int k = 0; k < 8; ++k) v[k] = byte_of(mraw[u], k) ? v[k] : 0.f;
           }
           // the bias gradient sums the values as stored (rounded to T), as the reference does
+          const uint4 packed = pack8<T>(v);
+          float r[8];
+          unpack8<T>(packed, r);
+          if (nv > 0) {
 #pragma unroll
-          for (int k = 0; k < 8; ++k) { v[k] = elem<T>::to_float(elem<T>::from_float(v[k])); csum[k] += v[k]; }
-          store8(C + off, v);
+            for (int k = 0; k < 8; ++k) csum[k] += (k < nv) ? r[k] : 0.f;
+          }
+          store8<VEC>(C + off, packed, nv);
         } else if constexpr (EPI == EPI_SCORES) {
           if (g.kmask_kind != 0) {
-            const uint8_t* mk = g.kmask_kind == 1 ? g.kmask + static_cast<int64_t>(bz / g.heads) * g.N + n
-                                                  : g.kmask + static_cast<int64_t>(m) * g.N + n;
-            for (int k = 0; k < nvalid; ++k) if (mk[k]) v[k] = -INFINITY;
+            const uint2 mk = g.kmask_kind == 1 ? padm : mraw[u];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) if (byte_of(mk, k)) v[k] = -INFINITY;
           }
-          store8(C + off, v);
+          store8<VEC>(C + off, pack8<T>(v), nv);
         }
       }
     }
+    };
+    if constexpr (EPI == EPI_ACT_FWD || EPI == EPI_ACT_BWD) dispatch_act(g.act, phase2);
+    else phase2(std::integral_constant<int, NMTG_ACT_NONE>{});
 
+    NMTG_PROF_MARK(4);
     if constexpr (EPI == EPI_ACT_BWD) {
       if (g.colsum_part != nullptr) {
         __syncthreads();
@@ -508,43 +670,58 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
 }
 
 // Column sums of a row-major [M, N] matrix: partial[mb][n] over row blocks (fp32), fixed order.
-template <typename T>
+// Block = 32 column lanes (8 columns each = one 16-byte load for 16-bit T) x 8 row lanes.
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void colsum_partial_kernel(const T* __restrict__ X, int64_t ld, int M, int N,
                                                              int rows_per_block, float* __restrict__ part) {
-  // thread -> 2 adjacent columns x (256/32 = 8) row lanes
-  __shared__ float red[8][64];
+  constexpr int CPT = VEC ? 8 : 1;
+  __shared__ float red[8][32 * CPT + 1];
   const int cl = threadIdx.x & 31, rl = threadIdx.x >> 5;
-  const int n = blockIdx.x * 64 + cl * 2;
+  const int n = (blockIdx.x * 32 + cl) * CPT;
   const int r0 = blockIdx.y * rows_per_block;
   const int r1 = min(M, r0 + rows_per_block);
-  float s0 = 0.f, s1 = 0.f;
+  float s[CPT];
+#pragma unroll
+  for (int j = 0; j < CPT; ++j) s[j] = 0.f;
   if (n < N) {
+#pragma unroll 4
     for (int r = r0 + rl; r < r1; r += 8) {
-      const T* p = X + static_cast<int64_t>(r) * ld + n;
-      s0 += elem<T>::to_float(p[0]);
-      if (n + 1 < N) s1 += elem<T>::to_float(p[1]);
+      float v[CPT];
+      load_pack<T, CPT>(X + static_cast<int64_t>(r) * ld + n, v);
+#pragma unroll
+      for (int j = 0; j < CPT; ++j) s[j] += v[j];
     }
   }
-  red[rl][cl * 2] = s0;
-  red[rl][cl * 2 + 1] = s1;
-  __syncthreads();
-  if (threadIdx.x < 64) {
-    float s = 0.f;
 #pragma unroll
-    for (int k = 0; k < 8; ++k) s += red[k][threadIdx.x];
-    const int col = blockIdx.x * 64 + threadIdx.x;
-    if (col < N) part[static_cast<int64_t>(blockIdx.y) * N + col] = s;
+  for (int j = 0; j < CPT; ++j) red[rl][cl * CPT + j] = s[j];
+  __syncthreads();
+  for (int c = threadIdx.x; c < 32 * CPT; c += 256) {
+    const int col = blockIdx.x * 32 * CPT + c;
+    if (col < N) {
+      float t = 0.f;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) t += red[k][c];
+      part[static_cast<int64_t>(blockIdx.y) * N + col] = t;
+    }
   }
 }
 
-// out[n] = T(sum_p part[p][n]) in order p = 0..parts-1.
+// out[n] = T(sum_p part[p][n]) in order p = 0..parts-1; 8 partial rows in flight per thread.
 template <typename T>
 __global__ __launch_bounds__(256) void colsum_final_kernel(const float* __restrict__ part, int parts, int N,
                                                            T* __restrict__ out) {
   const int n = blockIdx.x * 256 + threadIdx.x;
   if (n >= N) return;
   float s = 0.f;
-  for (int p = 0; p < parts; ++p) s += part[static_cast<int64_t>(p) * N + n];
+  int p = 0;
+  for (; p + 8 <= parts; p += 8) {
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = part[static_cast<int64_t>(p + j) * N + n];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s += v[j];
+  }
+  for (; p < parts; ++p) s += part[static_cast<int64_t>(p) * N + n];
   out[n] = elem<T>::from_float(s);
 }
 

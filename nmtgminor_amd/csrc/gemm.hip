@@ -2,6 +2,7 @@
 // (bias gradient) helpers and the stand-alone C entry point nmtg_gemm.
 #include "gemm_inst.cuh"
 #include <algorithm>
+#include <cstdlib>
 
 namespace nmtg {
 
@@ -78,12 +79,27 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
   if (!a.A || !a.B || !a.C) return fail(NMTG_ERR_INVALID, "gemm: null operand pointer");
   const bool a_kc = layout != LAYOUT_TN;
   const bool b_kc = layout == LAYOUT_NT;
-  (void)a_kc; (void)b_kc;
-  a.a_vec = vec_of(a.A, a.lda, a.sA, a.batch);
-  a.b_vec = vec_of(a.B, a.ldb, a.sB, a.batch);
-  a.c_vec = vec_of(a.C, a.ldc, a.sC, a.batch);
-  if (a.aux_out) a.c_vec = std::min(a.c_vec, vec_of(a.aux_out, a.ldc, a.sC, a.batch));
-  if (a.aux_in) a.c_vec = std::min(a.c_vec, vec_of(a.aux_in, a.ld_aux, 0, 1));
+  // widest access every pointer, pitch and extent of this call allows (8, 4 or 1 elements)
+  int vec = 8;
+  auto narrow = [&](const void* p, int64_t ld, int64_t stride, int batch, int64_t extent) {
+    int v = vec_of(p, ld, stride, batch);
+    while (v > 1 && extent % v != 0) v = v == 8 ? 4 : 1;
+    vec = std::min(vec, v);
+  };
+  narrow(a.A, a.lda, a.sA, a.batch, a_kc ? a.K : a.M);
+  narrow(a.B, a.ldb, a.sB, a.batch, b_kc ? a.K : a.N);
+  narrow(a.C, a.ldc, a.sC, a.batch, a.N);
+  if (a.aux_out) narrow(a.aux_out, a.ldc, a.sC, a.batch, a.N);
+  if (a.bias) narrow(a.bias, 8, 0, 1, a.N);
+  if (a.aux_in) narrow(a.aux_in, a.ld_aux, 0, 1, a.N);
+  auto narrow_bytes = [&](const uint8_t* p) {   // byte masks addressed as row * N + n
+    int v = 8;
+    while (v > 1 && (reinterpret_cast<uintptr_t>(p) % v != 0 || a.N % v != 0)) v = v == 8 ? 4 : 1;
+    vec = std::min(vec, v);
+  };
+  if (a.dmask) narrow_bytes(a.dmask);
+  if (a.kmask && a.kmask_kind != 0) narrow_bytes(a.kmask);
+  a.vec = vec;
 
   int tile = -1;
   a.splits = 1;
@@ -91,7 +107,7 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
 
   if (layout == LAYOUT_TN && epi == EPI_PLAIN && workspace != nullptr) {
     const SplitPlan p = plan_splitk(a.M, a.N, a.K, a.batch);
-    if (p.splits > 1 && splitk_ws_bytes(p, a.M, a.N, a.batch) <= workspace_bytes &&
+    if (p.splits > 1 && (p.tile != TILE_L || vec == 8) && splitk_ws_bytes(p, a.M, a.N, a.batch) <= workspace_bytes &&
         (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0) {
       epi = EPI_SPLITK;
       tile = p.tile;
@@ -100,13 +116,17 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
       a.ws = static_cast<float*>(workspace);
     }
   }
+  // NMTG_GEMM_TILE=0|1|2 (256x256 | 128x128 | 256x64) overrides the tile choice: a tuning aid.
+  static const int forced_tile = [] { const char* e = getenv("NMTG_GEMM_TILE"); return e ? atoi(e) : -1; }();
+  if (tile < 0 && forced_tile >= 0 && gemm_has(layout, forced_tile, epi) && (forced_tile != TILE_L || vec == 8)) tile = forced_tile;
   if (tile < 0) {
     const int cus = num_cus();
     const int64_t cnt_l = static_cast<int64_t>(ceil_div(a.M, 256)) * ceil_div(a.N, 256) * a.batch;
+    const bool l_ok = vec == 8 && gemm_has(layout, TILE_L, epi);
     if (a.N <= 64 && gemm_has(layout, TILE_S, epi)) tile = TILE_S;
-    else if (cnt_l * 4 >= cus * 3 && gemm_has(layout, TILE_L, epi)) tile = TILE_L;
+    else if (cnt_l * 4 >= cus * 3 && l_ok) tile = TILE_L;
     else if (gemm_has(layout, TILE_M, epi)) tile = TILE_M;
-    else if (gemm_has(layout, TILE_L, epi)) tile = TILE_L;
+    else if (l_ok) tile = TILE_L;
     else tile = TILE_S;
   }
   if (!gemm_has(layout, tile, epi))
@@ -143,10 +163,17 @@ int colsum_run(int dtype, const void* X, int64_t ld, int M, int N, float* part, 
   const int parts = colsum_parts(M);
   const int rpb = ceil_div(M, parts);
   {
-  TraceScope trace("colsum_partial", st);
-  NMTG_DISPATCH_DTYPE(dtype, T,
-                      hipLaunchKernelGGL((colsum_partial_kernel<T>), dim3(ceil_div(N, 64), parts), dim3(256), 0, st,
-                                         static_cast<const T*>(X), ld, M, N, rpb, part));
+    TraceScope trace("colsum_partial", st);
+    const bool vec = dtype != NMTG_F32 && aligned16(X) && ld % 8 == 0 && N % 8 == 0;
+    if (vec) {
+      NMTG_DISPATCH_DTYPE(dtype, T,
+                          hipLaunchKernelGGL((colsum_partial_kernel<T, true>), dim3(ceil_div(N, 256), parts), dim3(256), 0, st,
+                                             static_cast<const T*>(X), ld, M, N, rpb, part));
+    } else {
+      NMTG_DISPATCH_DTYPE(dtype, T,
+                          hipLaunchKernelGGL((colsum_partial_kernel<T, false>), dim3(ceil_div(N, 32), parts), dim3(256), 0, st,
+                                             static_cast<const T*>(X), ld, M, N, rpb, part));
+    }
   }
   NMTG_CHECK_LAUNCH("colsum");
   return colsum_finish(dtype, part, parts, N, out, st);

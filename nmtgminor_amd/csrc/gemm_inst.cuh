@@ -22,10 +22,10 @@ inline void tile_dims(int tile, int& bm, int& bn) {
   else { bm = 256; bn = 64; }
 }
 
-template <typename T, int TILE, bool A_KC, bool B_KC, int EPI>
-int gemm_launch_one(const GemmArgs& a, hipStream_t st) {
+template <typename T, int TILE, bool A_KC, bool B_KC, int EPI, int VEC>
+int gemm_launch_vec(const GemmArgs& a, hipStream_t st) {
   using C = tile_cfg<TILE>;
-  auto kern = gemm_kernel<T, C::BM, C::BN, C::WM, C::WN, A_KC, B_KC, EPI>;
+  auto kern = gemm_kernel<T, C::BM, C::BN, C::WM, C::WN, A_KC, B_KC, EPI, VEC>;
   constexpr int lds = gemm_lds_bytes<C::BM, C::BN>();
   static bool attr_done = false;
   if (!attr_done) {
@@ -37,10 +37,22 @@ int gemm_launch_one(const GemmArgs& a, hipStream_t st) {
   static const std::string name = std::string("gemm_") + (A_KC ? (B_KC ? "nt" : "nn") : "tn") + "_" +
                                   (TILE == TILE_L ? "256x256" : TILE == TILE_M ? "128x128" : "256x64") + "_" +
                                   (EPI == EPI_PLAIN ? "plain" : EPI == EPI_ACT_FWD ? "actfwd" : EPI == EPI_ACT_BWD ? "actbwd"
-                                   : EPI == EPI_SCORES ? "scores" : "splitk");
+                                   : EPI == EPI_SCORES ? "scores" : "splitk") + (VEC == 8 ? "" : VEC == 4 ? "_v4" : "_v1");
   TraceScope trace(name.c_str(), st);
   hipLaunchKernelGGL(kern, grid, dim3(64 * C::WM * C::WN), lds, st, a);
   return 0;
+}
+
+// The 256x256 tile exists for 16-byte accesses only; narrower calls are routed to the smaller tiles.
+template <typename T, int TILE, bool A_KC, bool B_KC, int EPI>
+int gemm_launch_one(const GemmArgs& a, hipStream_t st) {
+  if (a.vec == 8) return gemm_launch_vec<T, TILE, A_KC, B_KC, EPI, 8>(a, st);
+  if constexpr (TILE != TILE_L) {
+    if (a.vec == 4) return gemm_launch_vec<T, TILE, A_KC, B_KC, EPI, 4>(a, st);
+    return gemm_launch_vec<T, TILE, A_KC, B_KC, EPI, 1>(a, st);
+  } else {
+    return fail(NMTG_ERR_UNSUPPORTED, "gemm: the 256x256 tile needs 16-byte aligned operands");
+  }
 }
 
 template <typename T, int TILE>
@@ -51,7 +63,7 @@ int splitk_reduce_launch(const GemmArgs& a, hipStream_t st) {
   TraceScope trace("splitk_reduce", st);
   hipLaunchKernelGGL((splitk_reduce_kernel<T, C::BM, C::BN, C::WM, C::WN>), dim3(static_cast<unsigned>((total + 255) / 256)),
                      dim3(256), 0, st, a.ws, static_cast<T*>(a.C), a.ldc, a.M, a.N, a.m_tiles, a.n_tiles, a.batch, a.sC,
-                     a.splits, a.alpha, a.c_vec);
+                     a.splits, a.alpha, a.vec);
   return 0;
 }
 

@@ -324,31 +324,42 @@ __global__ __launch_bounds__(LN_THREADS) void ln_bwd_generic_kernel(
   }
 }
 
-// Column sums of the [n_part, hidden] partials, in a fixed order. Block = 32 column lanes x 8
-// row groups; every thread walks its row group top to bottom, LDS folds the 8 groups in order.
-constexpr int FIN_COLS = 32, FIN_GROUPS = 8;
-template <typename TW>
-__global__ __launch_bounds__(FIN_COLS * FIN_GROUPS) void ln_bwd_finalize_kernel(
+// Column sums of the [n_part, hidden] partials, in a fixed order. Block = FIN_CL column lanes
+// (CPT columns each) x FIN_GR row groups; a thread walks rows gr, gr + FIN_GR, ... with several
+// independent loads in flight, LDS folds the FIN_GR groups in order.
+constexpr int FIN_CL = 32, FIN_GR = 32;
+template <typename TW, int CPT>
+__global__ __launch_bounds__(FIN_CL * FIN_GR) void ln_bwd_finalize_kernel(
     const float* __restrict__ dgamma_part, const float* __restrict__ dbeta_part,
     TW* __restrict__ dgamma, TW* __restrict__ dbeta, int n_part, int hidden) {
-  __shared__ float red[FIN_GROUPS][FIN_COLS];
+  __shared__ float red[FIN_GR][FIN_CL * CPT + 1];
   const float* src = blockIdx.y == 0 ? dgamma_part : dbeta_part;
   TW* dst = blockIdx.y == 0 ? dgamma : dbeta;
-  const int cl = threadIdx.x % FIN_COLS, gr = threadIdx.x / FIN_COLS;
-  const int col = blockIdx.x * FIN_COLS + cl;
-  float s = 0.f;
-  if (col < hidden) {
-    const int per = (n_part + FIN_GROUPS - 1) / FIN_GROUPS;
-    const int lo = gr * per, hi = min(n_part, lo + per);
-    for (int p = lo; p < hi; ++p) s += src[static_cast<int64_t>(p) * hidden + col];
-  }
-  red[gr][cl] = s;
-  __syncthreads();
-  if (gr == 0 && col < hidden) {
-    float t = 0.f;
+  const int cl = threadIdx.x % FIN_CL, gr = threadIdx.x / FIN_CL;
+  const int col = (blockIdx.x * FIN_CL + cl) * CPT;
+  float s[CPT];
 #pragma unroll
-    for (int k = 0; k < FIN_GROUPS; ++k) t += red[k][cl];
-    dst[col] = elem<TW>::from_float(t);
+  for (int j = 0; j < CPT; ++j) s[j] = 0.f;
+  if (col < hidden) {
+#pragma unroll 4
+    for (int p = gr; p < n_part; p += FIN_GR) {
+      float v[CPT];
+      load_pack<float, CPT>(src + static_cast<int64_t>(p) * hidden + col, v);
+#pragma unroll
+      for (int j = 0; j < CPT; ++j) s[j] += v[j];
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < CPT; ++j) red[gr][cl * CPT + j] = s[j];
+  __syncthreads();
+  for (int c = threadIdx.x; c < FIN_CL * CPT; c += FIN_CL * FIN_GR) {
+    const int out_col = blockIdx.x * FIN_CL * CPT + c;
+    if (out_col < hidden) {
+      float t = 0.f;
+#pragma unroll
+      for (int k = 0; k < FIN_GR; ++k) t += red[k][c];
+      dst[out_col] = elem<TW>::from_float(t);
+    }
   }
 }
 
@@ -467,9 +478,15 @@ int ln_bwd_launch(const void* dz, const void* x_or_z, const float* mu, const flo
   }
   }
   TraceScope trace("ln_bwd_finalize", st);
-  dim3 fgrid((H + FIN_COLS - 1) / FIN_COLS, 2);
-  hipLaunchKernelGGL((ln_bwd_finalize_kernel<TW>), fgrid, dim3(FIN_COLS * FIN_GROUPS), 0, st, dgp,
-                     dbp, static_cast<TW*>(dgamma), static_cast<TW*>(dbeta), static_cast<int>(n_part), H);
+  if (H % 4 == 0 && aligned16(dgp) && aligned16(dbp)) {
+    dim3 fgrid((H + FIN_CL * 4 - 1) / (FIN_CL * 4), 2);
+    hipLaunchKernelGGL((ln_bwd_finalize_kernel<TW, 4>), fgrid, dim3(FIN_CL * FIN_GR), 0, st, dgp, dbp,
+                       static_cast<TW*>(dgamma), static_cast<TW*>(dbeta), static_cast<int>(n_part), H);
+  } else {
+    dim3 fgrid((H + FIN_CL - 1) / FIN_CL, 2);
+    hipLaunchKernelGGL((ln_bwd_finalize_kernel<TW, 1>), fgrid, dim3(FIN_CL * FIN_GR), 0, st, dgp, dbp,
+                       static_cast<TW*>(dgamma), static_cast<TW*>(dbeta), static_cast<int>(n_part), H);
+  }
   return 0;
 }
 
