@@ -131,6 +131,9 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
   }
   if (!gemm_has(layout, tile, epi))
     return fail(NMTG_ERR_UNSUPPORTED, "gemm: layout %d has no kernel for epilogue %d", layout, epi);
+  // direct-to-LDS operand loads need whole 64-k steps (k_per_split is a multiple of 64 already)
+  static const bool dma_off = getenv("NMTG_GEMM_NO_DMA") != nullptr;
+  a.dma = (!dma_off && a.K > 0 && a.K % GEMM_BK == 0) ? 1 : 0;
   int bm, bn;
   tile_dims(tile, bm, bn);
   a.m_tiles = ceil_div(a.M, bm);

@@ -22,10 +22,10 @@ inline void tile_dims(int tile, int& bm, int& bn) {
   else { bm = 256; bn = 64; }
 }
 
-template <typename T, int TILE, bool A_KC, bool B_KC, int EPI, int VEC>
+template <typename T, int TILE, bool A_KC, bool B_KC, int EPI, int VEC, bool DMA = false>
 int gemm_launch_vec(const GemmArgs& a, hipStream_t st) {
   using C = tile_cfg<TILE>;
-  auto kern = gemm_kernel<T, C::BM, C::BN, C::WM, C::WN, A_KC, B_KC, EPI, VEC>;
+  auto kern = gemm_kernel<T, C::BM, C::BN, C::WM, C::WN, A_KC, B_KC, EPI, VEC, DMA>;
   constexpr int lds = gemm_lds_bytes<C::BM, C::BN>();
   static bool attr_done = false;
   if (!attr_done) {
@@ -37,7 +37,8 @@ int gemm_launch_vec(const GemmArgs& a, hipStream_t st) {
   static const std::string name = std::string("gemm_") + (A_KC ? (B_KC ? "nt" : "nn") : "tn") + "_" +
                                   (TILE == TILE_L ? "256x256" : TILE == TILE_M ? "128x128" : "256x64") + "_" +
                                   (EPI == EPI_PLAIN ? "plain" : EPI == EPI_ACT_FWD ? "actfwd" : EPI == EPI_ACT_BWD ? "actbwd"
-                                   : EPI == EPI_SCORES ? "scores" : "splitk") + (VEC == 8 ? "" : VEC == 4 ? "_v4" : "_v1");
+                                   : EPI == EPI_SCORES ? "scores" : "splitk") + (VEC == 8 ? "" : VEC == 4 ? "_v4" : "_v1") +
+                                  (DMA ? "_dma" : "");
   TraceScope trace(name.c_str(), st);
   hipLaunchKernelGGL(kern, grid, dim3(64 * C::WM * C::WN), lds, st, a);
   return 0;
@@ -46,6 +47,9 @@ int gemm_launch_vec(const GemmArgs& a, hipStream_t st) {
 // The 256x256 tile exists for 16-byte accesses only; narrower calls are routed to the smaller tiles.
 template <typename T, int TILE, bool A_KC, bool B_KC, int EPI>
 int gemm_launch_one(const GemmArgs& a, hipStream_t st) {
+  if constexpr (A_KC || B_KC) {
+    if (a.vec == 8 && a.dma) return gemm_launch_vec<T, TILE, A_KC, B_KC, EPI, 8, true>(a, st);
+  }
   if (a.vec == 8) return gemm_launch_vec<T, TILE, A_KC, B_KC, EPI, 8>(a, st);
   if constexpr (TILE != TILE_L) {
     if (a.vec == 4) return gemm_launch_vec<T, TILE, A_KC, B_KC, EPI, 4>(a, st);
