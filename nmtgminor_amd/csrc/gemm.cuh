@@ -583,16 +583,18 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const Gemm
         const int m = m0 + ml;
         const int nv = m < g.M ? ncols : 0;
         float v[8];
+        uint4 raw;
         {
           const uint2* s = reinterpret_cast<const uint2*>(sC + ml * PITCH + cc * 16);
           const uint2 lo = s[0], hi = s[1];
-          unpack8<T>(make_uint4(lo.x, lo.y, hi.x, hi.y), v);
+          raw = make_uint4(lo.x, lo.y, hi.x, hi.y);
+          unpack8<T>(raw, v);
         }
         const int64_t off = static_cast<int64_t>(m) * g.ldc + n;
         if constexpr (EPI == EPI_PLAIN) {
-          store8<VEC>(C + off, pack8<T>(v), nv);
+          store8<VEC>(C + off, raw, nv);
         } else if constexpr (EPI == EPI_ACT_FWD) {
-          if (AUX != nullptr) store8<VEC>(AUX + off, pack8<T>(v), nv);
+          if (AUX != nullptr) store8<VEC>(AUX + off, raw, nv);
           float a[8];
 #pragma unroll
           for (int k = 0; k < 8; ++k) a[k] = act_apply<ACT>(v[k]);
@@ -615,19 +617,16 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const Gemm
               keep.y = kb[4] | (kb[5] << 8) | (kb[6] << 16) | (static_cast<uint32_t>(kb[7]) << 24);
               store8_bytes<VEC>(const_cast<uint8_t*>(g.dmask) + static_cast<int64_t>(m) * g.N + n, keep, nv);
             }
+            // keep bytes are 0 / 1: scale = float(byte) * 1/(1-p)
 #pragma unroll
-            for (int k = 0; k < 8; ++k) a[k] = byte_of(keep, k) ? a[k] * g.dscale : 0.f;
+            for (int k = 0; k < 8; ++k) a[k] *= static_cast<float>(byte_of(keep, k)) * g.dscale;
           }
           store8<VEC>(C + off, pack8<T>(a), nv);
         } else if constexpr (EPI == EPI_ACT_BWD) {
           float h[8];
           unpack8<T>(hraw[u], h);
 #pragma unroll
-          for (int k = 0; k < 8; ++k) v[k] *= act_grad<ACT>(h[k]) * g.dscale;
-          if (use_dmask) {
-#pragma unroll
-            for (int k = 0; k < 8; ++k) v[k] = byte_of(mraw[u], k) ? v[k] : 0.f;
-          }
+          for (int k = 0; k < 8; ++k) v[k] *= act_grad<ACT>(h[k]) * (static_cast<float>(byte_of(mraw[u], k)) * g.dscale);
           // the bias gradient sums the values as stored (rounded to T), as the reference does
           const uint4 packed = pack8<T>(v);
           float r[8];
