@@ -51,6 +51,7 @@ struct GemmArgs {
   float alpha;
   int vec;                  // widest access (elements: 8, 4 or 1) every operand and extent allows
   int dma;                  // every 64-k step of every split is full: direct-to-LDS loads allowed
+  int ring;                 // the call meets the requirements of the slot-ring kernel (gemm_ring.cuh)
   const void* bias;
   void* aux_out;
   const void* aux_in;
@@ -102,16 +103,21 @@ __device__ __forceinline__ int lds_swz(int row) { return (row ^ (row >> 3)) & 7;
 //   erfc(z) = (a1 t + a2 t^2 + a3 t^3 + a4 t^4 + a5 t^5) exp(-z^2),  t = 1 / (1 + p z),  z >= 0,
 // absolute error < 1.5e-7 (fp32 rounding level, far inside the 16-bit output precision), at
 // about a third of the instructions of erff(); Phi and the density share the one exponential.
+// Single-instruction reciprocal and 2^x (v_rcp_f32 / v_exp_f32, 1 ulp): the library forms expand to a
+// ten-instruction IEEE division and a range-checked exponential, which dominated the epilogue.
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
 struct NormalCdfPdf { float cdf, pdf; };
 __device__ __forceinline__ NormalCdfPdf normal_cdf_pdf(float h) {
   const float z = fabsf(h) * 0.70710678118654752f;
-  const float t = __frcp_rn(fmaf(0.3275911f, z, 1.f));
+  const float t = fast_rcp(fmaf(0.3275911f, z, 1.f));
   // coefficients pre-multiplied by 1/2: half_erfc = 0.5 * erfc(z)
   float poly = fmaf(0.5f * 1.061405429f, t, 0.5f * -1.453152027f);
   poly = fmaf(poly, t, 0.5f * 1.421413741f);
   poly = fmaf(poly, t, 0.5f * -0.284496736f);
   poly = fmaf(poly, t, 0.5f * 0.254829592f);
-  const float e = exp2f(h * h * -0.72134752044448170f);  // exp(-h^2 / 2)
+  const float e = fast_exp2(h * h * -0.72134752044448170f);  // exp(-h^2 / 2)
   const float half_erfc = poly * t * e;
   NormalCdfPdf r;
   r.cdf = h >= 0.f ? 1.f - half_erfc : half_erfc;
@@ -123,11 +129,11 @@ template <int ACT>
 __device__ __forceinline__ float act_apply(float h) {
   if constexpr (ACT == NMTG_ACT_RELU) return fmaxf(h, 0.f);
   else if constexpr (ACT == NMTG_ACT_GELU) return h * normal_cdf_pdf(h).cdf;
-  else if constexpr (ACT == NMTG_ACT_SILU) return h * __frcp_rn(1.f + exp2f(h * -1.4426950408889634f));
+  else if constexpr (ACT == NMTG_ACT_SILU) return h * fast_rcp(1.f + fast_exp2(h * -1.4426950408889634f));
   else if constexpr (ACT == NMTG_ACT_AGELU) {
     // 0.5 h (1 + tanh u) = h * sigmoid(2u)
     const float u2 = 1.5957691216057308f * (h + 0.044715f * h * h * h);
-    return h * __frcp_rn(1.f + exp2f(u2 * -1.4426950408889634f));
+    return h * fast_rcp(1.f + fast_exp2(u2 * -1.4426950408889634f));
   } else return h;
 }
 template <int ACT>
@@ -137,12 +143,12 @@ __device__ __forceinline__ float act_grad(float h) {
     const NormalCdfPdf n = normal_cdf_pdf(h);
     return fmaf(h, n.pdf, n.cdf);
   } else if constexpr (ACT == NMTG_ACT_SILU) {
-    const float s = __frcp_rn(1.f + exp2f(h * -1.4426950408889634f));
+    const float s = fast_rcp(1.f + fast_exp2(h * -1.4426950408889634f));
     return s * (1.f + h * (1.f - s));
   } else if constexpr (ACT == NMTG_ACT_AGELU) {
     // d/dh [h s(2u)] = s + h s (1 - s) 2u',  u' = k (1 + 3 c h^2)
     const float u2 = 1.5957691216057308f * (h + 0.044715f * h * h * h);
-    const float sg = __frcp_rn(1.f + exp2f(u2 * -1.4426950408889634f));
+    const float sg = fast_rcp(1.f + fast_exp2(u2 * -1.4426950408889634f));
     return sg + h * sg * (1.f - sg) * 1.5957691216057308f * (1.f + 0.134145f * h * h);
   } else return 1.f;
 }
@@ -370,124 +376,18 @@ __device__ __forceinline__ void dma_tile(const T* __restrict__ base, int64_t ld,
 __device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0f70); }  // vmcnt(0)
 
 // ---------------------------------------------------------------------------------------------
-// The kernel.
+// Epilogue shared by the GEMM kernels: accumulators -> (bias, activation, masks, ...) -> global.
 // ---------------------------------------------------------------------------------------------
-template <int BM, int BN>
-constexpr int gemm_lds_bytes() {
-  constexpr int main_loop = 2 * (BM + BN) * GEMM_BK * 2;
-  constexpr int c_tile = BM * (BN * 2 + 8);
-  return main_loop > c_tile ? main_loop : c_tile;
-}
-
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC, int EPI, int VEC, bool DMA = false>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const GemmArgs g) {
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int EPI, int VEC>
+__device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, acc16_t (&acc)[BM / WAVES_M / 32][BN / WAVES_N / 32],
+                                              uint8_t* lds_raw, int tile_m, int tile_n, int bz, int split) {
   constexpr int NT = 64 * WAVES_M * WAVES_N;
-  constexpr int BK = GEMM_BK;
   constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
   constexpr int TM = WTM / 32, TN = WTN / 32;
-  static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA tile");
-  extern __shared__ __align__(16) uint8_t lds_raw[];
-  T* sA = reinterpret_cast<T*>(lds_raw);
-  T* sB = sA + 2 * BM * BK;
-
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm0 = (wave / WAVES_N) * WTM, wn0 = (wave % WAVES_N) * WTN;
-
-  // Tile coordinates. Consecutive block ids go round-robin to the 8 XCDs (each with its own L2), so
-  // block ids are first regrouped to give every XCD a contiguous run of the tile order, and the
-  // tile order itself walks groups of GM tile rows column by column: the ~32 tiles an XCD runs at
-  // once then form a GM x 32/GM patch and share their A / B panels through that XCD's L2.
-  int bid = blockIdx.x;
-  const int ntile = g.m_tiles * g.n_tiles;
-  if ((ntile & 7) == 0) bid = (bid & 7) * (ntile >> 3) + (bid >> 3);
-  constexpr int GM = 4;
-  const int in_group = GM * g.n_tiles;
-  const int first_m = (bid / in_group) * GM;
-  const int gsize = min(g.m_tiles - first_m, GM);
-  const int tile_m = first_m + (bid % in_group) % gsize, tile_n = (bid % in_group) / gsize;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
-  const int bz = blockIdx.y, split = blockIdx.z;
-
-  const T* A = static_cast<const T*>(g.A) + static_cast<int64_t>(bz) * g.sA;
-  const T* B = static_cast<const T*>(g.B) + static_cast<int64_t>(bz) * g.sB;
-  const int kbeg = split * g.k_per_split;
-  const int kend = min(g.K, kbeg + g.k_per_split);
-  const int nk = (kend - kbeg + BK - 1) / BK;
-
-  acc16_t acc[TM][TN];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-  TileStage<T, BM, NT, A_KC, VEC> stA;
-  TileStage<T, BN, NT, B_KC, VEC> stB;
-
-  // DMA: reduction-contiguous operands go global -> LDS directly (whole 64-k steps only; the host
-  // selects this variant when every step of every split is full).
-  constexpr bool DMA_A = DMA && A_KC && VEC == 8, DMA_B = DMA && B_KC && VEC == 8;
-  NMTG_PROF_MARK(0);
-  if (nk > 0) {
-    if constexpr (DMA_A) dma_tile<T, BM, NT>(A, g.lda, g.M, m0, kbeg, sA, tid);
-    else stA.load(A, g.lda, g.M, m0, kbeg, kend, tid);
-    if constexpr (DMA_B) dma_tile<T, BN, NT>(B, g.ldb, g.N, n0, kbeg, sB, tid);
-    else stB.load(B, g.ldb, g.N, n0, kbeg, kend, tid);
-    if constexpr (!DMA_A) stA.store(sA, tid);
-    if constexpr (!DMA_B) stB.store(sB, tid);
-    if constexpr (DMA_A || DMA_B) wait_vmem_all();
-  }
-  __syncthreads();
-
-  NMTG_PROF_MARK(1);
-  // per-lane LDS offsets of the MFMA fragments (elements), constant over the K loop
-  int offA[TM][2], offB[TN][2];
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-    const int row = wm0 + i * 32 + (lane & 31);
-    offA[i][0] = row * BK;
-    offA[i][1] = lds_swz(row);
-  }
-#pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    const int row = wn0 + j * 32 + (lane & 31);
-    offB[j][0] = row * BK;
-    offB[j][1] = lds_swz(row);
-  }
-
-  for (int kt = 0; kt < nk; ++kt) {
-    const int cur = kt & 1;
-    if (kt + 1 < nk) {
-      if constexpr (DMA_A) dma_tile<T, BM, NT>(A, g.lda, g.M, m0, kbeg + (kt + 1) * BK, sA + (cur ^ 1) * BM * BK, tid);
-      else stA.load(A, g.lda, g.M, m0, kbeg + (kt + 1) * BK, kend, tid);
-      if constexpr (DMA_B) dma_tile<T, BN, NT>(B, g.ldb, g.N, n0, kbeg + (kt + 1) * BK, sB + (cur ^ 1) * BN * BK, tid);
-      else stB.load(B, g.ldb, g.N, n0, kbeg + (kt + 1) * BK, kend, tid);
-    }
-    const T* cA = sA + cur * BM * BK;
-    const T* cB = sB + cur * BN * BK;
-#pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-      uint4 fm[TM], fn[TN];
-      const int c = kk * 2 + (lane >> 5);
-#pragma unroll
-      for (int i = 0; i < TM; ++i) fm[i] = *reinterpret_cast<const uint4*>(cA + offA[i][0] + ((c ^ offA[i][1]) * 8));
-#pragma unroll
-      for (int j = 0; j < TN; ++j) fn[j] = *reinterpret_cast<const uint4*>(cB + offB[j][0] + ((c ^ offB[j][1]) * 8));
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) mfma<T>::run(fn[j], fm[i], acc[i][j]);
-    }
-    if (kt + 1 < nk) {
-      if constexpr (!DMA_A) stA.store(sA + (cur ^ 1) * BM * BK, tid);
-      if constexpr (!DMA_B) stB.store(sB + (cur ^ 1) * BN * BK, tid);
-      if constexpr (DMA_A || DMA_B) wait_vmem_all();
-    }
-    __syncthreads();
-  }
-
-  NMTG_PROF_MARK(2);
+  const int ntile = g.m_tiles * g.n_tiles;
   // Lane (l) register r of tile (i, j) holds C[m][n] with
   //   m = m0 + wm0 + 32 i + (l & 31),   n = n0 + wn0 + 32 j + 8 (r / 4) + 4 (l >> 5) + (r % 4).
   if constexpr (EPI == EPI_SPLITK) {
@@ -666,6 +566,128 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const Gemm
       }
     }
   }
+}
+
+// ---------------------------------------------------------------------------------------------
+// The kernel.
+// ---------------------------------------------------------------------------------------------
+template <int BM, int BN>
+constexpr int gemm_lds_bytes() {
+  constexpr int main_loop = 2 * (BM + BN) * GEMM_BK * 2;
+  constexpr int c_tile = BM * (BN * 2 + 8);
+  return main_loop > c_tile ? main_loop : c_tile;
+}
+
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC, int EPI, int VEC, bool DMA = false>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const GemmArgs g) {
+  constexpr int NT = 64 * WAVES_M * WAVES_N;
+  constexpr int BK = GEMM_BK;
+  constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA tile");
+  extern __shared__ __align__(16) uint8_t lds_raw[];
+  T* sA = reinterpret_cast<T*>(lds_raw);
+  T* sB = sA + 2 * BM * BK;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm0 = (wave / WAVES_N) * WTM, wn0 = (wave % WAVES_N) * WTN;
+
+  // Tile coordinates. Consecutive block ids go round-robin to the 8 XCDs (each with its own L2), so
+  // block ids are first regrouped to give every XCD a contiguous run of the tile order, and the
+  // tile order itself walks groups of GM tile rows column by column: the ~32 tiles an XCD runs at
+  // once then form a GM x 32/GM patch and share their A / B panels through that XCD's L2.
+  int bid = blockIdx.x;
+  const int ntile = g.m_tiles * g.n_tiles;
+  if ((ntile & 7) == 0) bid = (bid & 7) * (ntile >> 3) + (bid >> 3);
+  constexpr int GM = 4;
+  const int in_group = GM * g.n_tiles;
+  const int first_m = (bid / in_group) * GM;
+  const int gsize = min(g.m_tiles - first_m, GM);
+  const int tile_m = first_m + (bid % in_group) % gsize, tile_n = (bid % in_group) / gsize;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int bz = blockIdx.y, split = blockIdx.z;
+
+  const T* A = static_cast<const T*>(g.A) + static_cast<int64_t>(bz) * g.sA;
+  const T* B = static_cast<const T*>(g.B) + static_cast<int64_t>(bz) * g.sB;
+  const int kbeg = split * g.k_per_split;
+  const int kend = min(g.K, kbeg + g.k_per_split);
+  const int nk = (kend - kbeg + BK - 1) / BK;
+
+  acc16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  TileStage<T, BM, NT, A_KC, VEC> stA;
+  TileStage<T, BN, NT, B_KC, VEC> stB;
+
+  // DMA: reduction-contiguous operands go global -> LDS directly (whole 64-k steps only; the host
+  // selects this variant when every step of every split is full).
+  constexpr bool DMA_A = DMA && A_KC && VEC == 8, DMA_B = DMA && B_KC && VEC == 8;
+  NMTG_PROF_MARK(0);
+  if (nk > 0) {
+    if constexpr (DMA_A) dma_tile<T, BM, NT>(A, g.lda, g.M, m0, kbeg, sA, tid);
+    else stA.load(A, g.lda, g.M, m0, kbeg, kend, tid);
+    if constexpr (DMA_B) dma_tile<T, BN, NT>(B, g.ldb, g.N, n0, kbeg, sB, tid);
+    else stB.load(B, g.ldb, g.N, n0, kbeg, kend, tid);
+    if constexpr (!DMA_A) stA.store(sA, tid);
+    if constexpr (!DMA_B) stB.store(sB, tid);
+    if constexpr (DMA_A || DMA_B) wait_vmem_all();
+  }
+  __syncthreads();
+
+  NMTG_PROF_MARK(1);
+  // per-lane LDS offsets of the MFMA fragments (elements), constant over the K loop
+  int offA[TM][2], offB[TN][2];
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int row = wm0 + i * 32 + (lane & 31);
+    offA[i][0] = row * BK;
+    offA[i][1] = lds_swz(row);
+  }
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int row = wn0 + j * 32 + (lane & 31);
+    offB[j][0] = row * BK;
+    offB[j][1] = lds_swz(row);
+  }
+
+  for (int kt = 0; kt < nk; ++kt) {
+    const int cur = kt & 1;
+    if (kt + 1 < nk) {
+      if constexpr (DMA_A) dma_tile<T, BM, NT>(A, g.lda, g.M, m0, kbeg + (kt + 1) * BK, sA + (cur ^ 1) * BM * BK, tid);
+      else stA.load(A, g.lda, g.M, m0, kbeg + (kt + 1) * BK, kend, tid);
+      if constexpr (DMA_B) dma_tile<T, BN, NT>(B, g.ldb, g.N, n0, kbeg + (kt + 1) * BK, sB + (cur ^ 1) * BN * BK, tid);
+      else stB.load(B, g.ldb, g.N, n0, kbeg + (kt + 1) * BK, kend, tid);
+    }
+    const T* cA = sA + cur * BM * BK;
+    const T* cB = sB + cur * BN * BK;
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; ++kk) {
+      uint4 fm[TM], fn[TN];
+      const int c = kk * 2 + (lane >> 5);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) fm[i] = *reinterpret_cast<const uint4*>(cA + offA[i][0] + ((c ^ offA[i][1]) * 8));
+#pragma unroll
+      for (int j = 0; j < TN; ++j) fn[j] = *reinterpret_cast<const uint4*>(cB + offB[j][0] + ((c ^ offB[j][1]) * 8));
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) mfma<T>::run(fn[j], fm[i], acc[i][j]);
+    }
+    if (kt + 1 < nk) {
+      if constexpr (!DMA_A) stA.store(sA + (cur ^ 1) * BM * BK, tid);
+      if constexpr (!DMA_B) stB.store(sB + (cur ^ 1) * BN * BK, tid);
+      if constexpr (DMA_A || DMA_B) wait_vmem_all();
+    }
+    __syncthreads();
+  }
+
+  NMTG_PROF_MARK(2);
+  gemm_epilogue<T, BM, BN, WAVES_M, WAVES_N, EPI, VEC>(g, acc, lds_raw, tile_m, tile_n, bz, split);
 }
 
 // Sums the split-K partials (in the accumulator layout written above), scales, converts to T and

@@ -134,6 +134,11 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
   // direct-to-LDS operand loads need whole 64-k steps (k_per_split is a multiple of 64 already)
   static const bool dma_off = getenv("NMTG_GEMM_NO_DMA") != nullptr;
   a.dma = (!dma_off && a.K > 0 && a.K % GEMM_BK == 0) ? 1 : 0;
+  // the slot-ring kernel addresses each operand with 32-bit lane offsets
+  static const bool ring_off = getenv("NMTG_GEMM_NO_RING") != nullptr;
+  const int64_t a_bytes = static_cast<int64_t>(a_kc ? a.M : a.K) * a.lda * 2;
+  const int64_t b_bytes = static_cast<int64_t>(b_kc ? a.N : a.K) * a.ldb * 2;
+  a.ring = (!ring_off && a.dma && vec == 8 && tile != TILE_S && a_bytes < (int64_t{1} << 32) && b_bytes < (int64_t{1} << 32)) ? 1 : 0;
   int bm, bn;
   tile_dims(tile, bm, bn);
   a.m_tiles = ceil_div(a.M, bm);

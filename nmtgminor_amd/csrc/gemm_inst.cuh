@@ -5,6 +5,7 @@
 //   S: 256x64  tile, 4x1 wavefronts (each 64x64),  256 threads  — N <= 64 (per-head attention products)
 #pragma once
 #include "gemm.cuh"
+#include "gemm_ring.cuh"
 #include <string>
 
 namespace nmtg {
@@ -44,10 +45,40 @@ int gemm_launch_vec(const GemmArgs& a, hipStream_t st) {
   return 0;
 }
 
+
+// Slot-ring kernel (gemm_ring.cuh): the 256x256 tile owns the whole LDS (10 slots), the 128x128
+// tile takes 5 slots so that two blocks share a CU and one block's epilogue overlaps the other's
+// main loop.
+template <int TILE> struct ring_slots { static constexpr int value = TILE == TILE_L ? 10 : 5; };
+
+template <typename T, int TILE, bool A_KC, bool B_KC, int EPI>
+int gemm_launch_ring(const GemmArgs& a, hipStream_t st) {
+  using C = tile_cfg<TILE>;
+  constexpr int RING = ring_slots<TILE>::value;
+  auto kern = gemm_ring_kernel<T, C::BM, C::BN, C::WM, C::WN, A_KC, B_KC, EPI, RING>;
+  constexpr int lds = gemm_ring_lds_bytes<C::BM, C::BN, RING>();
+  static bool attr_done = false;
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return fail(NMTG_ERR_LAUNCH, "gemm: cannot reserve %d bytes of LDS: %s", lds, hipGetErrorString(e));
+    attr_done = true;
+  }
+  dim3 grid(a.m_tiles * a.n_tiles, a.batch, a.splits);
+  static const std::string name = std::string("gemm_") + (A_KC ? (B_KC ? "nt" : "nn") : "tn") + "_" +
+                                  (TILE == TILE_L ? "256x256" : "128x128") + "_" +
+                                  (EPI == EPI_PLAIN ? "plain" : EPI == EPI_ACT_FWD ? "actfwd" : EPI == EPI_ACT_BWD ? "actbwd"
+                                   : EPI == EPI_SCORES ? "scores" : "splitk") + "_ring";
+  TraceScope trace(name.c_str(), st);
+  hipLaunchKernelGGL(kern, grid, dim3(64 * C::WM * C::WN), lds, st, a);
+  return 0;
+}
+
 // The 256x256 tile exists for 16-byte accesses only; narrower calls are routed to the smaller tiles.
 template <typename T, int TILE, bool A_KC, bool B_KC, int EPI>
 int gemm_launch_one(const GemmArgs& a, hipStream_t st) {
-  if constexpr (A_KC || B_KC) {
+  if constexpr (TILE != TILE_S) {
+    if (a.vec == 8 && a.ring) return gemm_launch_ring<T, TILE, A_KC, B_KC, EPI>(a, st);
+  } else if constexpr (A_KC || B_KC) {
     if (a.vec == 8 && a.dma) return gemm_launch_vec<T, TILE, A_KC, B_KC, EPI, 8, true>(a, st);
   }
   if (a.vec == 8) return gemm_launch_vec<T, TILE, A_KC, B_KC, EPI, 8>(a, st);
