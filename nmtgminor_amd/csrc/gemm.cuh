@@ -204,20 +204,20 @@ __device__ __forceinline__ void store8(uint16_t* __restrict__ p, const uint4& v,
     if (h * VEC < nvalid) *reinterpret_cast<R*>(p + h * VEC) = u.r[h];
 }
 
-template <int VEC>
+template <int VEC, bool ZERO = true>
 __device__ __forceinline__ uint2 load8_bytes(const uint8_t* __restrict__ p, const uint8_t* __restrict__ safe, int nvalid) {
   if constexpr (VEC == 8) {
     const bool ok = nvalid > 0;
     uint2 v = *reinterpret_cast<const uint2*>(ok ? p : safe);
-    if (!ok) v = make_uint2(0, 0);
+    if (ZERO && !ok) v = make_uint2(0, 0);
     return v;
   } else if constexpr (VEC == 4) {
     uint2 v;
     const bool ok0 = nvalid > 0, ok1 = nvalid > 4;
     v.x = *reinterpret_cast<const uint32_t*>(ok0 ? p : safe);
     v.y = *reinterpret_cast<const uint32_t*>(ok1 ? p + 4 : safe);
-    if (!ok0) v.x = 0;
-    if (!ok1) v.y = 0;
+    if (ZERO && !ok0) v.x = 0;
+    if (ZERO && !ok1) v.y = 0;
     return v;
   } else {
     uint32_t w[2] = {0, 0};
@@ -408,31 +408,56 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, acc16_t (&acc)[
     constexpr int PITCH = BN * 2 + 8;  // bytes
     uint8_t* sC = lds_raw;
     const T* bias = static_cast<const T*>(g.bias);
+    // bias values of this lane's columns, loaded together ahead of the conversion loop (one
+    // uniform branch around all of them: loads inside per-iteration branches wait one by one)
+    float bv[TN][4][4];
+    if (EPI != EPI_ACT_BWD && bias != nullptr) {
+      if constexpr (VEC >= 4) {
+        uint2 braw[TN][4];
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int nn = n0 + wn0 + j * 32 + q * 8 + (lane >> 5) * 4;
+            braw[j][q] = *reinterpret_cast<const uint2*>(bias + (nn < g.N ? nn : 0));  // columns past N are never stored
+          }
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const T* e4 = reinterpret_cast<const T*>(&braw[j][q]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) bv[j][q][e] = elem<T>::to_float(e4[e]);
+          }
+      } else {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int nn = n0 + wn0 + j * 32 + q * 8 + (lane >> 5) * 4;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) bv[j][q][e] = elem<T>::to_float(bias[min(nn + e, g.N - 1)]);
+          }
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) bv[j][q][e] = 0.f;
+    }
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int nl = wn0 + j * 32 + q * 8 + (lane >> 5) * 4;
-        float bv[4] = {0.f, 0.f, 0.f, 0.f};
-        if (EPI != EPI_ACT_BWD && bias != nullptr) {
-          // clamped, branch-free loads (columns past N are never stored)
-          const int nn = n0 + nl;
-          if constexpr (VEC >= 4) {
-            const uint2 raw = *reinterpret_cast<const uint2*>(bias + (nn < g.N ? nn : 0));
-            const T* e4 = reinterpret_cast<const T*>(&raw);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) bv[e] = elem<T>::to_float(e4[e]);
-          } else {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) bv[e] = elem<T>::to_float(bias[min(nn + e, g.N - 1)]);
-          }
-        }
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
           const int ml = wm0 + i * 32 + (lane & 31);
           float v[4];
 #pragma unroll
-          for (int e = 0; e < 4; ++e) v[e] = acc[i][j][q * 4 + e] * g.alpha + bv[e];
+          for (int e = 0; e < 4; ++e) v[e] = acc[i][j][q * 4 + e] * g.alpha + bv[j][q][e];
           store_pack<T, 4>(reinterpret_cast<T*>(sC + ml * PITCH + nl * 2), v);
         }
       }
@@ -457,6 +482,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, acc16_t (&acc)[
     const bool use_dmask = (EPI == EPI_ACT_FWD || EPI == EPI_ACT_BWD) && g.dmask != nullptr;
     const bool dmask_in = use_dmask && !(EPI == EPI_ACT_FWD && g.rng);
     const bool tmask = EPI == EPI_SCORES && g.kmask_kind == 2;
+    const uint8_t* side_mask = dmask_in ? g.dmask : tmask ? g.kmask : nullptr;   // [M, N] byte mask read per chunk
     uint2 padm = make_uint2(0, 0);
     if (EPI == EPI_SCORES && g.kmask_kind == 1)
       padm = load8_bytes<VEC>(g.kmask + static_cast<int64_t>(bz / g.heads) * g.N + n, g.kmask, ncols);
@@ -467,15 +493,28 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, acc16_t (&acc)[
       // side inputs of GRP passes first (independent loads in flight together), then the math and stores
       uint4 hraw[GRP];
       uint2 mraw[GRP];
+      // Values of out-of-range chunks are never stored, so with 16-byte accesses the loads skip the
+      // zeroing select (it would make each load wait for its own data); the mask branch encloses
+      // the whole group so that its loads stay in one basic block.
+      constexpr bool ZSIDE = VEC != 8;
+      if constexpr (EPI == EPI_ACT_BWD) {
 #pragma unroll
-      for (int u = 0; u < GRP; ++u) {
-        const int m = m0 + (p0 + u) * RPP + r_in;
-        const int nv = m < g.M ? ncols : 0;
-        if constexpr (EPI == EPI_ACT_BWD)
-          hraw[u] = load8<VEC>(HIN + static_cast<int64_t>(m < g.M ? m : 0) * g.ld_aux + (nv > 0 ? n : 0), HIN, nv);
-        if (dmask_in) mraw[u] = load8_bytes<VEC>(g.dmask + static_cast<int64_t>(m < g.M ? m : 0) * g.N + (nv > 0 ? n : 0), g.dmask, nv);
-        else if (tmask) mraw[u] = load8_bytes<VEC>(g.kmask + static_cast<int64_t>(m < g.M ? m : 0) * g.N + (nv > 0 ? n : 0), g.kmask, nv);
-        else mraw[u] = make_uint2(0x01010101u, 0x01010101u);
+        for (int u = 0; u < GRP; ++u) {
+          const int m = m0 + (p0 + u) * RPP + r_in;
+          const int nv = m < g.M ? ncols : 0;
+          hraw[u] = load8<VEC, ZSIDE>(HIN + static_cast<int64_t>(m < g.M ? m : 0) * g.ld_aux + (nv > 0 ? n : 0), HIN, nv);
+        }
+      }
+      if (side_mask != nullptr) {
+#pragma unroll
+        for (int u = 0; u < GRP; ++u) {
+          const int m = m0 + (p0 + u) * RPP + r_in;
+          const int nv = m < g.M ? ncols : 0;
+          mraw[u] = load8_bytes<VEC, ZSIDE>(side_mask + static_cast<int64_t>(m < g.M ? m : 0) * g.N + (nv > 0 ? n : 0), side_mask, nv);
+        }
+      } else {
+#pragma unroll
+        for (int u = 0; u < GRP; ++u) mraw[u] = make_uint2(0x01010101u, 0x01010101u);
       }
 #pragma unroll
       for (int u = 0; u < GRP; ++u) {

@@ -191,6 +191,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_ring_kernel(const
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
+  NMTG_PROF_MARK(0);
   // ---- prologue: fill the ring ----
   static_for<0, RING>([&](auto tt) {
     constexpr int t = decltype(tt)::value;
@@ -200,6 +201,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_ring_kernel(const
   if (nk > 0) wait_vmcnt_upto<(RING - SPS) * IPS, IPS>((min(RING, total) - SPS) * IPS);
   ring_barrier();
 
+  NMTG_PROF_MARK(1);
   int pos_r = 0, pos_w = 0;
   const char* a_cur = a_base - step_a;  // stage s - 1 at the top of iteration s
   const char* b_cur = b_base - step_b;
@@ -268,6 +270,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_ring_kernel(const
     ring_barrier();
   }
 
+  NMTG_PROF_MARK(2);
   gemm_epilogue<T, BM, BN, WAVES_M, WAVES_N, EPI, 8>(g, acc, lds_raw, tile_m, tile_n, bz, split);
 }
 
