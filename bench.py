@@ -318,8 +318,43 @@ class EncdecAttnWL(Workload):
                     sample="full workload in fp32 on the bf16-rounded values, median of 3")
 
 
+
+class CopyWL(Workload):
+    """Plain device copy of a known size: the calibration target for the rocprofv3 FETCH_SIZE /
+    WRITE_SIZE counters (not part of `--workload all`)."""
+    name = "copy"
+    bound = "hbm"
+    dtype = "f32"
+    description = "torch copy of 1 GiB fp32 (1 GiB read + 1 GiB written): counter calibration"
+
+    def setup(self, dev):
+        n = 1 << 28
+        self.src = torch.ones(n, dtype=torch.float32, device=dev)
+        self.dst = torch.empty_like(self.src)
+
+    def step(self):
+        self.dst.copy_(self.src)
+        return self.dst
+
+    def work_per_step(self):
+        return 2 * self.src.numel() * 4
+
+
 WORKLOADS = {w.name: w for w in (LayerNormWL, MlpWL, SelfAttnWL, EncdecAttnWL, XentropyWL)}
+EXTRA_WORKLOADS = {CopyWL.name: CopyWL}
 PRIMARY = "mlp"
+
+
+def _measured_traffic():
+    """HBM bytes per step of each workload's dominant kernel group, measured offline with rocprofv3
+    --pmc FETCH_SIZE / WRITE_SIZE (counters cannot be read from inside this process); the file
+    holds the figures and the commands that produced them."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get("bytes_per_step", {})
+    except (OSError, ValueError):
+        return {}
 
 
 def measure(w, dev, steps, warmup, do_cpu, trace_steps):
@@ -367,6 +402,7 @@ def measure(w, dev, steps, warmup, do_cpu, trace_steps):
                             us_per_step=ms / trace_steps * 1e3))
     roof = None
     best = None
+    traffic_table = _measured_traffic().get(w.name, {})
     for prefix, work in w.kernel_work().items():
         sel = [k for k in kernels if k["name"].startswith(prefix)]
         if not sel:
@@ -379,7 +415,7 @@ def measure(w, dev, steps, warmup, do_cpu, trace_steps):
         achieved = w.rate(work, us * 1e-6)
         launches = sum(k["launches_per_step"] for k in sel)
         roof = dict(bound=w.bound, achieved=round(achieved, 3), peak=w.peak, unit=w.unit, frac=round(achieved / w.peak, 4),
-                    traffic=None, kernel=(prefix + "*" if prefix.endswith("_") else prefix), launches_per_step=launches,
+                    traffic=traffic_table.get(prefix), kernel=(prefix + "*" if prefix.endswith("_") else prefix), launches_per_step=launches,
                     avg_launch_us=round(us / launches, 3), work_per_step=work)
     res = dict(workload=w.name, description=w.description, metric="achieved HBM GB/s" if w.bound == "hbm" else "MFMA TFLOP/s",
                value=round(w.rate(w.work_per_step(), per_step), 3), unit=w.unit, ms_per_step=round(per_step * 1e3, 5),
@@ -412,12 +448,13 @@ def main():
     torch.set_num_threads(os.cpu_count() or 1)
     dev = torch.device("cuda:0")
     names = list(WORKLOADS) if args.workload == "all" else [args.workload]
+    table = dict(WORKLOADS, **EXTRA_WORKLOADS)
     if PRIMARY in names:                     # headline first
         names.remove(PRIMARY)
         names.insert(0, PRIMARY)
     results = []
     for n in names:
-        w = WORKLOADS[n]()
+        w = table[n]()
         steps = args.steps if w.name != "xentropy" else max(3, min(args.steps, 10))
         results.append(measure(w, dev, steps, args.warmup, not args.no_cpu, min(args.trace_steps, steps)))
         results[-1]["steps"] = steps

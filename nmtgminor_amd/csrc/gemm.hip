@@ -146,6 +146,8 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
   if (m_tiles_out) *m_tiles_out = a.m_tiles;
   if (static_cast<int64_t>(a.m_tiles) * a.n_tiles > 0x7fffffff || a.batch > 65535)
     return fail(NMTG_ERR_UNSUPPORTED, "gemm: grid too large (tiles %d x %d, batch %d)", a.m_tiles, a.n_tiles, a.batch);
+  if (epi == EPI_SPLITK && a.ws == nullptr)
+    return fail(NMTG_ERR_INVALID, "gemm: the split-K epilogue needs a workspace");
   int rc;
   if (layout == LAYOUT_NT) rc = gemm_launch_nt(dtype, tile, epi, a, st);
   else if (layout == LAYOUT_NN) rc = gemm_launch_nn(dtype, tile, epi, a, st);
