@@ -17,7 +17,9 @@ F.scaled_dot_product_attention, nn.MultiheadAttention after de-interleaving the 
 autograd), against closed forms and invariants, by brute-force Python loops on tiny shapes and
 by fp64 finite differences (torch.autograd.gradcheck, the reference's own method for its
 hand-written backward, onmt/modules/optimized/self_attention_func.py:955-967). The reference
-tree holds no stored golden vectors for these ops; tests/golden/ holds small fixtures written
-from this oracle so that a change in the arithmetic of either side is noticed.
+tree holds no stored golden vectors for these ops; tests/golden/ holds small fixtures written by
+tests/golden/make_fixtures.py from PyTorch's library routines and autograd (not from this
+package), against which tests/test_golden_cpu.py checks every function here, including the
+fallback's 16-bit rounding points (round_to=).
 """
 from . import attention, dropout_add, inputs, layer_norm, mlp, softmax_dropout, xentropy  # noqa: F401
