@@ -1,0 +1,100 @@
+"""Hazard check of the slot-ring schedule of the GEMM main loop (nmtgminor_amd/csrc/gemm_ring.cuh).
+
+A small event model of one wavefront replays the kernel's issue / wait / barrier / read sequence
+with the kernel's own bookkeeping formulas (ring positions, number of transfers allowed to stay in
+flight at each wait) and checks the three properties the loop relies on, for every ring size,
+stage size and step count the templates admit:
+  1. a slot is read only after its transfers were covered by a vmcnt wait that precedes the last
+     barrier (transfers of a wavefront complete in issue order, `s_waitcnt vmcnt(n)` leaves at most
+     the newest n outstanding; every wavefront runs the same sequence, so "covered before the
+     barrier" for one holds for all);
+  2. a ring position is overwritten only when the slot it held belongs to a stage every wavefront
+     has finished reading (a barrier lies between the last read and the issue);
+  3. the position arithmetic finds slot s * SPS + j of stage s where the kernel looks for it.
+"""
+import itertools
+
+import pytest
+
+
+def simulate(ring, sa, sb, ips, nk):
+    sps = sa + sb
+    assert ring >= 2 * sps
+    total = nk * sps
+    issued = []            # transfer ids in issue order: (slot number, instruction)
+    content = [None] * ring  # slot number held (or being filled) at each ring position
+    covered = set()        # slots whose transfers a wait has covered
+    visible = set()        # ... and a barrier has followed
+
+    def issue(q, pos, reading_stage):
+        old = content[pos]
+        if old is not None:
+            # property 2: the slot being overwritten was consumed in an iteration that a barrier has closed
+            assert old // sps < reading_stage, (ring, sps, nk, q, pos, old, reading_stage)
+        content[pos] = q
+        for i in range(ips):
+            issued.append((q, i))
+
+    def wait(n, max_n):
+        k = min(n, max_n)
+        assert k >= 0 and k % ips == 0
+        done = issued if k == 0 else issued[:-k]
+        for q, _ in done:
+            covered.add(q)
+
+    def barrier():
+        visible.update(covered)
+
+    # prologue
+    for t in range(ring):
+        if t // sps < nk:
+            issue(t, t, reading_stage=0)
+    if nk > 0:
+        wait((min(ring, total) - sps) * ips, (ring - sps) * ips)
+    barrier()
+    pos_r = pos_w = 0
+    for s in range(nk):
+        if s >= 1:
+            for t in range(sps):
+                d = (ring + t) // sps
+                q = ring + (s - 1) * sps + t
+                assert q // sps == s - 1 + d and q % sps == (ring + t) % sps     # the kernel's compile-time (j, d)
+                if s - 1 + d < nk:
+                    issue(q, pos_w, reading_stage=s)
+                pos_w = 0 if pos_w + 1 == ring else pos_w + 1
+        for j in range(sps):           # every operand slot of stage s is read by some wavefront
+            p = pos_r + j
+            if p >= ring:
+                p -= ring
+            q = s * sps + j
+            assert content[p] == q, (ring, sps, nk, s, j, p, content[p])          # property 3
+            assert q in visible, (ring, sps, nk, s, j)                             # property 1
+        pos_r += sps
+        if pos_r >= ring:
+            pos_r -= ring
+        if s + 1 < nk:
+            n_issued = min(ring + s * sps, total)
+            assert n_issued * ips == len(issued)
+            wait((n_issued - (s + 2) * sps) * ips, (ring - 2 * sps) * ips)
+        barrier()
+    return len(issued)
+
+
+CONFIGS = [(ring, sa, sb, ips) for ring, (sa, sb), ips in itertools.product((4, 5, 6, 8, 10), ((1, 1), (2, 1), (2, 2)), (2, 4))
+           if ring >= 2 * (sa + sb)]
+
+
+@pytest.mark.parametrize("ring,sa,sb,ips", CONFIGS)
+def test_ring_schedule_has_no_hazard(ring, sa, sb, ips):
+    for nk in range(0, 70):
+        n = simulate(ring, sa, sb, ips, nk)
+        assert n == nk * (sa + sb) * ips          # every slot of every stage is issued exactly once
+
+
+def test_shipped_configurations_are_covered():
+    # 256x256 tile: 2 + 2 slots per stage, 10-slot ring, 8 wavefronts -> 2 transfers per wavefront and slot;
+    # 128x128 tile: 1 + 1 slots, 5-slot ring, 4 wavefronts -> 4 transfers
+    assert (10, 2, 2, 2) in CONFIGS and (5, 1, 1, 4) in CONFIGS
+    # vmcnt is a 6-bit counter: the deepest wait the kernel can ask for must fit
+    for ring, sa, sb, ips in ((10, 2, 2, 2), (5, 1, 1, 4)):
+        assert (ring - (sa + sb)) * ips < 64
