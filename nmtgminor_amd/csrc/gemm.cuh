@@ -757,7 +757,15 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
   const int64_t per_split = static_cast<int64_t>(batch) * m_tiles * n_tiles * PER_BLK;
   float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
   const float4* w = reinterpret_cast<const float4*>(ws) + idx;
-  for (int sp = 0; sp < splits; ++sp) {
+  int sp = 0;
+  for (; sp + 4 <= splits; sp += 4) {   // four partials in flight, summed in split order
+    float4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] = w[(sp + u) * per_split];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) { s.x += v[u].x; s.y += v[u].y; s.z += v[u].z; s.w += v[u].w; }
+  }
+  for (; sp < splits; ++sp) {
     const float4 v = w[sp * per_split];
     s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
   }
@@ -782,8 +790,36 @@ __global__ __launch_bounds__(256) void colsum_partial_kernel(const T* __restrict
 #pragma unroll
   for (int j = 0; j < CPT; ++j) s[j] = 0.f;
   if (n < N) {
-#pragma unroll 4
-    for (int r = r0 + rl; r < r1; r += 8) {
+    // Latency-bound (few blocks, short rows): 16 rows are loaded before any is added (two loops on
+    // purpose, see ln_bwd_finalize_kernel); the sum order is unchanged.
+    constexpr int BATCH = 16;
+    int r = r0 + rl;
+    for (; r + (BATCH - 1) * 8 < r1; r += BATCH * 8) {
+      // raw words first, conversion only in the adding loop (a conversion is a use of the load)
+      constexpr int NV = (CPT * sizeof(T)) / 16;   // 16-byte vectors per access; 0 in the scalar form
+      if constexpr (NV > 0) {
+        uint4 raw[BATCH][NV];
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u)
+#pragma unroll
+          for (int i = 0; i < NV; ++i)
+            raw[u][i] = reinterpret_cast<const uint4*>(X + static_cast<int64_t>(r + u * 8) * ld + n)[i];
+        __builtin_amdgcn_sched_barrier(0);   // keep every load ahead of the first add
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) {
+          const T* e = reinterpret_cast<const T*>(raw[u]);
+#pragma unroll
+          for (int j = 0; j < CPT; ++j) s[j] += elem<T>::to_float(e[j]);
+        }
+      } else {
+        T raw[BATCH];
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) raw[u] = X[static_cast<int64_t>(r + u * 8) * ld + n];
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) s[0] += elem<T>::to_float(raw[u]);
+      }
+    }
+    for (; r < r1; r += 8) {
       float v[CPT];
       load_pack<T, CPT>(X + static_cast<int64_t>(r) * ld + n, v);
 #pragma unroll
@@ -812,6 +848,14 @@ __global__ __launch_bounds__(256) void colsum_final_kernel(const float* __restri
   if (n >= N) return;
   float s = 0.f;
   int p = 0;
+  // a few blocks of dependent-latency work: 32, then 8 partial rows in flight per thread
+  for (; p + 32 <= parts; p += 32) {
+    float v[32];
+#pragma unroll
+    for (int j = 0; j < 32; ++j) v[j] = part[static_cast<int64_t>(p + j) * N + n];
+#pragma unroll
+    for (int j = 0; j < 32; ++j) s += v[j];
+  }
   for (; p + 8 <= parts; p += 8) {
     float v[8];
 #pragma unroll

@@ -341,8 +341,22 @@ __global__ __launch_bounds__(FIN_CL * FIN_GR) void ln_bwd_finalize_kernel(
 #pragma unroll
   for (int j = 0; j < CPT; ++j) s[j] = 0.f;
   if (col < hidden) {
-#pragma unroll 4
-    for (int p = gr; p < n_part; p += FIN_GR) {
+    // The kernel is a handful of blocks, so what it costs is global-load latency: 16 partial rows
+    // are loaded before any of them is added (written as two loops on purpose: with the load and
+    // the add in one loop body the compiler waits for each load in turn). Sum order unchanged.
+    constexpr int BATCH = 16;
+    int p = gr;
+    for (; p + (BATCH - 1) * FIN_GR < n_part; p += BATCH * FIN_GR) {
+      float v[BATCH][CPT];
+#pragma unroll
+      for (int u = 0; u < BATCH; ++u) load_pack<float, CPT>(src + static_cast<int64_t>(p + u * FIN_GR) * hidden + col, v[u]);
+      __builtin_amdgcn_sched_barrier(0);   // keep every load ahead of the first add
+#pragma unroll
+      for (int u = 0; u < BATCH; ++u)
+#pragma unroll
+        for (int j = 0; j < CPT; ++j) s[j] += v[u][j];
+    }
+    for (; p < n_part; p += FIN_GR) {
       float v[CPT];
       load_pack<float, CPT>(src + static_cast<int64_t>(p) * hidden + col, v);
 #pragma unroll
