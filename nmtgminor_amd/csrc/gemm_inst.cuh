@@ -49,7 +49,7 @@ int gemm_launch_vec(const GemmArgs& a, hipStream_t st) {
 // Slot-ring kernel (gemm_ring.cuh): the 256x256 tile owns the whole LDS (10 slots), the 128x128
 // tile takes 5 slots so that two blocks share a CU and one block's epilogue overlaps the other's
 // main loop.
-template <int TILE> struct ring_slots { static constexpr int value = TILE == TILE_L ? 10 : 5; };
+template <int TILE> struct ring_slots { static constexpr int value = TILE == TILE_M ? 5 : 10; };
 
 template <typename T, int TILE, bool A_KC, bool B_KC, int EPI>
 int gemm_launch_ring(const GemmArgs& a, hipStream_t st) {
@@ -65,7 +65,7 @@ int gemm_launch_ring(const GemmArgs& a, hipStream_t st) {
   }
   dim3 grid(a.m_tiles * a.n_tiles, a.batch, a.splits);
   static const std::string name = std::string("gemm_") + (A_KC ? (B_KC ? "nt" : "nn") : "tn") + "_" +
-                                  (TILE == TILE_L ? "256x256" : "128x128") + "_" +
+                                  (TILE == TILE_L ? "256x256" : TILE == TILE_M ? "128x128" : "256x64") + "_" +
                                   (EPI == EPI_PLAIN ? "plain" : EPI == EPI_ACT_FWD ? "actfwd" : EPI == EPI_ACT_BWD ? "actbwd"
                                    : EPI == EPI_SCORES ? "scores" : "splitk") + "_ring";
   TraceScope trace(name.c_str(), st);
@@ -76,9 +76,8 @@ int gemm_launch_ring(const GemmArgs& a, hipStream_t st) {
 // The 256x256 tile exists for 16-byte accesses only; narrower calls are routed to the smaller tiles.
 template <typename T, int TILE, bool A_KC, bool B_KC, int EPI>
 int gemm_launch_one(const GemmArgs& a, hipStream_t st) {
-  if constexpr (TILE != TILE_S) {
-    if (a.vec == 8 && a.ring) return gemm_launch_ring<T, TILE, A_KC, B_KC, EPI>(a, st);
-  } else if constexpr (A_KC || B_KC) {
+  if (a.vec == 8 && a.ring) return gemm_launch_ring<T, TILE, A_KC, B_KC, EPI>(a, st);
+  if constexpr (TILE == TILE_S && (A_KC || B_KC)) {
     if (a.vec == 8 && a.dma) return gemm_launch_vec<T, TILE, A_KC, B_KC, EPI, 8, true>(a, st);
   }
   if (a.vec == 8) return gemm_launch_vec<T, TILE, A_KC, B_KC, EPI, 8>(a, st);

@@ -88,9 +88,11 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_ring_kernel(const
   constexpr int NT = 64 * WAVES_M * WAVES_N, NW = NT / 64;
   constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
   constexpr int TM = WTM / 32, TN = WTN / 32;
-  constexpr int SA = BM / 128, SB = BN / 128, SPS = SA + SB;
+  constexpr int SA = BM / 128, SB = (BN + 127) / 128, SPS = SA + SB;
   constexpr int IPS = 16 / NW;  // transfers per wavefront per slot
-  static_assert(BM % 128 == 0 && BN % 128 == 0, "block tile is a whole number of slots");
+  // BN = 64 (the per-head products) fills a whole B slot too: its upper 64 rows hold clamped duplicates no
+  // fragment reads, which keeps the transfer count per slot uniform for the vmcnt bookkeeping.
+  static_assert(BM % 128 == 0 && (BN % 128 == 0 || BN == 64), "block tile is a whole number of slots (or a 64-row B tile)");
   static_assert(WTM % 32 == 0 && WTN % 32 == 0 && 128 % WTM == 0 && 128 % WTN == 0, "a wave tile lies inside one slot");
   static_assert(16 % NW == 0, "slots are dealt evenly to the wavefronts");
   static_assert(RING >= 2 * SPS, "the ring must hold the stage being read and the next one");
