@@ -17,6 +17,7 @@
 // masked_fill pass over the [B*H, Tq, Tk] tensor); bias gradients are column-sum kernels with a
 // fixed reduction order; weight gradients split the token dimension over the chip.
 #include "gemm.cuh"
+#include <cstdlib>
 #include <algorithm>
 
 // implemented in softmax_dropout.hip
@@ -55,10 +56,30 @@ int core_fwd(const Core& c, Strided q, Strided k, Strided v, const uint8_t* mask
   g.C = scores; g.ldc = c.tk; g.sC = static_cast<int64_t>(c.tq) * c.tk;
   g.M = c.tq; g.N = c.tk; g.K = c.d; g.batch = c.bh; g.alpha = c.scale;
   g.kmask = mask; g.kmask_kind = mask_kind; g.heads = c.heads;
-  if (int rc = gemm_run(c.dtype, LAYOUT_NT, EPI_SCORES, g, nullptr, 0, c.st)) return rc;
-  if (int rc = nmtg_softmax_dropout_fwd(scores, nullptr, 0, softmax_out, dropped, dmask, dropout_mode, p, seed, offset,
-                                        static_cast<int64_t>(c.bh) * c.tq, c.tk, c.tq, c.heads, c.dtype, c.st))
-    return rc;
+  // NMTG_ATTN_FUSED=1: scores, softmax and dropout in one kernel (rows of up to 512 keys). Compiled in but not
+  // yet through the GPU test-suite, hence opt-in; read per call so that a test can switch it.
+  int fused = 0;
+  if (getenv("NMTG_ATTN_FUSED") != nullptr) {
+    GemmArgs f = g;
+    f.out2 = dropped;
+    f.aux_out = softmax_out;
+    if (dropout_mode != 0) {
+      f.dmask = dmask;
+      f.rng = dropout_mode == 2;
+      f.keep_p = 1.f - p;
+      f.dscale = 1.f / (1.f - p);
+      f.seed = seed;
+      f.offset = offset;
+    }
+    fused = gemm_scores_softmax_try(c.dtype, f, c.st);
+    if (fused < 0) return fused;
+  }
+  if (!fused) {
+    if (int rc = gemm_run(c.dtype, LAYOUT_NT, EPI_SCORES, g, nullptr, 0, c.st)) return rc;
+    if (int rc = nmtg_softmax_dropout_fwd(scores, nullptr, 0, softmax_out, dropped, dmask, dropout_mode, p, seed, offset,
+                                          static_cast<int64_t>(c.bh) * c.tq, c.tk, c.tq, c.heads, c.dtype, c.st))
+      return rc;
+  }
   GemmArgs h{};
   h.A = dropped; h.lda = c.tk; h.sA = static_cast<int64_t>(c.tq) * c.tk;
   h.B = v.p; h.ldb = v.ld; h.sB = v.stride;

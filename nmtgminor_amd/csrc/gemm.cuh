@@ -36,7 +36,11 @@ enum GemmEpi {
   EPI_ACT_FWD = 1,  // h = acc + bias -> aux_out;  C = act(h) * keep * dscale
   EPI_ACT_BWD = 2,  // C = T(acc) * act'(aux_in) * dscale * keep (keep = 1 without a mask);  colsum_part[m_tile][n] = sum_m C
   EPI_SCORES = 3,   // C = alpha*acc, -inf where the key-padding / time mask is set
-  EPI_SPLITK = 4    // fp32 partial tile -> workspace (reduced by splitk_reduce_kernel)
+  EPI_SPLITK = 4,   // fp32 partial tile -> workspace (reduced by splitk_reduce_kernel)
+  // C = alpha*acc with the mask as -inf (as EPI_SCORES), then the row softmax of the stored (rounded) scores and
+  // dropout in the same pass: aux_out = softmax (optional), out2 = dropped probabilities. The block tile spans
+  // the whole row (N <= BN), one wavefront normalises one row.
+  EPI_SCORES_SOFTMAX = 5
 };
 
 struct GemmArgs {
@@ -54,6 +58,7 @@ struct GemmArgs {
   int ring;                 // the call meets the requirements of the slot-ring kernel (gemm_ring.cuh)
   const void* bias;
   void* aux_out;
+  void* out2;               // EPI_SCORES_SOFTMAX: dropped probabilities, laid out like C
   const void* aux_in;
   int64_t ld_aux;
   const uint8_t* dmask;     // dropout keep mask [M, N] dense; read, or written when rng != 0
@@ -487,6 +492,91 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, acc16_t (&acc)[
     if (EPI == EPI_SCORES && g.kmask_kind == 1)
       padm = load8_bytes<VEC>(g.kmask + static_cast<int64_t>(bz / g.heads) * g.N + n, g.kmask, ncols);
 
+    if constexpr (EPI == EPI_SCORES_SOFTMAX) {
+      // One wavefront per row: lane cc holds the row's elements 8 cc .. 8 cc + 7.
+      static_assert(CPR == 64 && VEC == 8, "the row tile is 512 columns wide and moves 16-byte chunks");
+      uint16_t* OUT2 = reinterpret_cast<uint16_t*>(g.out2) + static_cast<int64_t>(bz) * g.sC;
+      const bool time_mask = g.kmask_kind == 2;
+      const bool drop = g.dmask != nullptr;
+      const bool replay = drop && !g.rng;
+      uint2 padm2 = make_uint2(0, 0);
+      if (g.kmask_kind == 1) padm2 = load8_bytes<VEC>(g.kmask + static_cast<int64_t>(bz / g.heads) * g.N + n, g.kmask, ncols);
+      constexpr float LOG2E = 1.4426950408889634f;
+      const Philox gen(g.seed);
+      for (int p0 = 0; p0 < PASSES; p0 += GRP) {
+        uint2 traw[GRP], draw[GRP];
+        if (time_mask) {
+#pragma unroll
+          for (int u = 0; u < GRP; ++u) {
+            const int m = m0 + (p0 + u) * RPP + r_in;
+            const int nv = m < g.M ? ncols : 0;
+            traw[u] = load8_bytes<VEC, false>(g.kmask + static_cast<int64_t>(m < g.M ? m : 0) * g.N + (nv > 0 ? n : 0), g.kmask, nv);
+          }
+        } else {
+#pragma unroll
+          for (int u = 0; u < GRP; ++u) traw[u] = padm2;
+        }
+        if (replay) {
+#pragma unroll
+          for (int u = 0; u < GRP; ++u) {
+            const int m = m0 + (p0 + u) * RPP + r_in;
+            const int nv = m < g.M ? ncols : 0;
+            const int64_t row = static_cast<int64_t>(bz) * g.M + (m < g.M ? m : 0);
+            draw[u] = load8_bytes<VEC, false>(g.dmask + row * g.N + (nv > 0 ? n : 0), g.dmask, nv);
+          }
+        } else {
+#pragma unroll
+          for (int u = 0; u < GRP; ++u) draw[u] = make_uint2(0x01010101u, 0x01010101u);
+        }
+#pragma unroll
+        for (int u = 0; u < GRP; ++u) {
+          const int ml = (p0 + u) * RPP + r_in;
+          const int m = m0 + ml;
+          const int nv = m < g.M ? ncols : 0;
+          float v[8];
+          {
+            const uint2* sp = reinterpret_cast<const uint2*>(sC + ml * PITCH + cc * 16);
+            const uint2 lo = sp[0], hi = sp[1];
+            unpack8<T>(make_uint4(lo.x, lo.y, hi.x, hi.y), v);
+          }
+          // masked keys and the columns past N count as -inf
+#pragma unroll
+          for (int k = 0; k < 8; ++k)
+            if (byte_of(traw[u], k) || ncols <= 0) v[k] = -INFINITY;
+          const int64_t off = static_cast<int64_t>(m) * g.ldc + n;
+          store8<VEC>(C + off, pack8<T>(v), nv);
+          float mx = v[0];
+#pragma unroll
+          for (int k = 1; k < 8; ++k) mx = fmaxf(mx, v[k]);
+          mx = wave_max(mx);
+          const float base = (mx == -INFINITY) ? 0.f : mx;   // a row without any key gives zeros
+          float sum = 0.f;
+#pragma unroll
+          for (int k = 0; k < 8; ++k) { v[k] = exp2f((v[k] - base) * LOG2E); sum += v[k]; }
+          sum = wave_sum(sum);
+          const float inv = sum > 0.f ? 1.f / sum : 0.f;
+#pragma unroll
+          for (int k = 0; k < 8; ++k) v[k] *= inv;
+          if (AUX != nullptr) store8<VEC>(AUX + off, pack8<T>(v), nv);
+          if (drop) {
+            uint2 keep = draw[u];
+            if (g.rng) {
+              uint8_t kb[8];
+              const uint64_t first = (static_cast<uint64_t>(bz) * g.M + m) * g.N + n;
+              philox_keep<8>(gen, first, g.offset, g.keep_p, kb);
+              keep.x = kb[0] | (kb[1] << 8) | (kb[2] << 16) | (static_cast<uint32_t>(kb[3]) << 24);
+              keep.y = kb[4] | (kb[5] << 8) | (kb[6] << 16) | (static_cast<uint32_t>(kb[7]) << 24);
+              store8_bytes<VEC>(const_cast<uint8_t*>(g.dmask) + first, keep, nv);
+            }
+#pragma unroll
+            for (int k = 0; k < 8; ++k) v[k] = byte_of(keep, k) ? v[k] * g.dscale : 0.f;
+          }
+          store8<VEC>(OUT2 + off, pack8<T>(v), nv);
+        }
+      }
+      return;
+    }
+
     auto phase2 = [&](auto act_tag) {
     constexpr int ACT = decltype(act_tag)::value;
     for (int p0 = 0; p0 < PASSES; p0 += GRP) {
@@ -880,6 +970,12 @@ size_t gemm_splitk_workspace_bytes(int M, int N, int K, int batch);
 // used (= rows of colsum_part written by EPI_ACT_BWD).
 int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t workspace_bytes, hipStream_t st,
              int* m_tiles_out = nullptr);
+
+// Fused Q K^T -> mask -> softmax -> dropout (EPI_SCORES_SOFTMAX) for rows of at most 512 keys. `a` is filled as
+// for EPI_SCORES plus out2 (dropped probabilities), aux_out (softmax, optional), dmask / rng / keep_p / dscale /
+// seed / offset. Returns 1 if the kernel was launched, 0 if the call does not qualify (the caller then runs the
+// scores GEMM and the softmax kernel), or a negative nmtg_status.
+int gemm_scores_softmax_try(int dtype, GemmArgs a, hipStream_t st);
 
 // bias-gradient style column sums: out[n] = sum_m X[m][n]; part is fp32 scratch of
 // colsum_parts(M) * N floats.

@@ -140,7 +140,7 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
   const int64_t b_bytes = static_cast<int64_t>(b_kc ? a.N : a.K) * a.ldb * 2;
   // The 256x64 tile runs the ring loop only on request (NMTG_GEMM_RING_S=1): that instantiation has not been
   // through the GPU test-suite yet.
-  static const bool ring_s = getenv("NMTG_GEMM_RING_S") != nullptr;
+  const bool ring_s = getenv("NMTG_GEMM_RING_S") != nullptr;   // read per call so that a test can switch it
   a.ring = (!ring_off && a.dma && vec == 8 && (tile != TILE_S || ring_s) && a_bytes < (int64_t{1} << 32) &&
             b_bytes < (int64_t{1} << 32)) ? 1 : 0;
   int bm, bn;
@@ -160,6 +160,30 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(NMTG_ERR_LAUNCH, "gemm: launch failed: %s", hipGetErrorString(e));
   return 0;
+}
+
+int gemm_scores_softmax_try(int dtype, GemmArgs a, hipStream_t st) {
+  if (a.M <= 0 || a.N <= 0 || a.batch <= 0) return 0;
+  if (dtype != NMTG_F16 && dtype != NMTG_BF16) return 0;
+  if (a.N > 512 || a.N % 8 != 0 || a.K <= 0 || a.K % 8 != 0 || a.batch > 65535 || !a.out2) return 0;
+  auto ok16 = [](const void* p, int64_t ld, int64_t stride, int batch) { return vec_of(p, ld, stride, batch) == 8; };
+  if (!ok16(a.A, a.lda, a.sA, a.batch) || !ok16(a.B, a.ldb, a.sB, a.batch) || !ok16(a.C, a.ldc, a.sC, a.batch) ||
+      !ok16(a.out2, a.ldc, a.sC, a.batch) || (a.aux_out && !ok16(a.aux_out, a.ldc, a.sC, a.batch)))
+    return 0;
+  auto ok8 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 8 == 0; };
+  if ((a.dmask && !ok8(a.dmask)) || (a.kmask && a.kmask_kind != 0 && !ok8(a.kmask))) return 0;
+  a.vec = 8;
+  a.dma = 0;
+  a.ring = 0;
+  a.splits = 1;
+  a.k_per_split = ceil_div(a.K, GEMM_BK) * GEMM_BK;
+  a.m_tiles = ceil_div(a.M, 128);
+  a.n_tiles = 1;
+  if (static_cast<int64_t>(a.m_tiles) > 0x7fffffff) return 0;
+  if (int rc = gemm_launch_nt(dtype, TILE_R, EPI_SCORES_SOFTMAX, a, st)) return rc;
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(NMTG_ERR_LAUNCH, "gemm: launch failed: %s", hipGetErrorString(e));
+  return 1;
 }
 
 int colsum_parts(int M) { return std::max(1, std::min(64, ceil_div(M, 128))); }

@@ -3,6 +3,7 @@
 //   L: 256x256 tile, 2x4 wavefronts (each 128x64), 512 threads  — large outputs
 //   M: 128x128 tile, 2x2 wavefronts (each 64x64),  256 threads  — outputs too small to fill the chip with L
 //   S: 256x64  tile, 4x1 wavefronts (each 64x64),  256 threads  — N <= 64 (per-head attention products)
+//   R: 128x512 tile, 4x2 wavefronts (each 32x256), 512 threads  — whole score rows (fused softmax epilogue only)
 #pragma once
 #include "gemm.cuh"
 #include "gemm_ring.cuh"
@@ -10,16 +11,18 @@
 
 namespace nmtg {
 
-enum GemmTile { TILE_L = 0, TILE_M = 1, TILE_S = 2 };
+enum GemmTile { TILE_L = 0, TILE_M = 1, TILE_S = 2, TILE_R = 3 };
 
 template <int TILE> struct tile_cfg;
 template <> struct tile_cfg<TILE_L> { static constexpr int BM = 256, BN = 256, WM = 2, WN = 4; };
 template <> struct tile_cfg<TILE_M> { static constexpr int BM = 128, BN = 128, WM = 2, WN = 2; };
 template <> struct tile_cfg<TILE_S> { static constexpr int BM = 256, BN = 64, WM = 4, WN = 1; };
+template <> struct tile_cfg<TILE_R> { static constexpr int BM = 128, BN = 512, WM = 4, WN = 2; };
 
 inline void tile_dims(int tile, int& bm, int& bn) {
   if (tile == TILE_L) { bm = 256; bn = 256; }
   else if (tile == TILE_M) { bm = 128; bn = 128; }
+  else if (tile == TILE_R) { bm = 128; bn = 512; }
   else { bm = 256; bn = 64; }
 }
 
@@ -36,9 +39,10 @@ int gemm_launch_vec(const GemmArgs& a, hipStream_t st) {
   }
   dim3 grid(a.m_tiles * a.n_tiles, a.batch, a.splits);
   static const std::string name = std::string("gemm_") + (A_KC ? (B_KC ? "nt" : "nn") : "tn") + "_" +
-                                  (TILE == TILE_L ? "256x256" : TILE == TILE_M ? "128x128" : "256x64") + "_" +
+                                  (TILE == TILE_L ? "256x256" : TILE == TILE_M ? "128x128" : TILE == TILE_R ? "128x512" : "256x64") + "_" +
                                   (EPI == EPI_PLAIN ? "plain" : EPI == EPI_ACT_FWD ? "actfwd" : EPI == EPI_ACT_BWD ? "actbwd"
-                                   : EPI == EPI_SCORES ? "scores" : "splitk") + (VEC == 8 ? "" : VEC == 4 ? "_v4" : "_v1") +
+                                   : EPI == EPI_SCORES ? "scores" : EPI == EPI_SCORES_SOFTMAX ? "scores_softmax" : "splitk") +
+                                  (VEC == 8 ? "" : VEC == 4 ? "_v4" : "_v1") +
                                   (DMA ? "_dma" : "");
   TraceScope trace(name.c_str(), st);
   hipLaunchKernelGGL(kern, grid, dim3(64 * C::WM * C::WN), lds, st, a);

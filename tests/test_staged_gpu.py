@@ -1,0 +1,99 @@
+"""Kernel variants that are compiled into the library but switched off by default because they have
+not been through the GPU test-suite yet:
+
+  NMTG_GEMM_RING_S=1   the slot-ring main loop for the 256x64 tile (per-head products P V, dS K, Pd^T dC, dS^T Q)
+  NMTG_ATTN_FUSED=1    Q K^T -> mask -> softmax -> dropout in one kernel (rows of up to 512 keys)
+
+The library reads both switches on every call, so each test runs the default path and the staged
+path in one process and compares them (and the staged path with the CPU oracle). The tests only run
+when NMTG_TEST_STAGED=1 is set; once they have passed on the GPU the switches can become defaults.
+"""
+import os
+
+import pytest
+import torch
+
+from nmtgminor_amd.native import self_multihead_attn_blaslt as sa_native
+from nmtgminor_amd.native.linear_gemm import gemm
+from oracle import attention as oat, inputs
+from util import assert_close
+
+pytestmark = [pytest.mark.gpu,
+              pytest.mark.skipif(os.environ.get("NMTG_TEST_STAGED") != "1",
+                                 reason="staged kernel variants: set NMTG_TEST_STAGED=1 to validate them")]
+D = torch.float64
+
+
+class switch:
+    def __init__(self, name):
+        self.name = name
+
+    def __enter__(self):
+        os.environ[self.name] = "1"
+
+    def __exit__(self, *exc):
+        os.environ.pop(self.name, None)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("batch,m,n,k", [(8, 512, 64, 512), (3, 300, 64, 192), (2, 256, 64, 64), (5, 77, 64, 128)])
+def test_ring_256x64_matches_two_buffer_loop(dev, dtype, batch, m, n, k):
+    g = torch.Generator().manual_seed(91)
+    a = torch.randn(batch, m, k, generator=g).to(dtype).to(dev)
+    b_kn = torch.randn(batch, k, n, generator=g).to(dtype).to(dev)        # NN: P V, dS K
+    a_km = torch.randn(batch, k, m, generator=g).to(dtype).to(dev)        # TN: Pd^T dC, dS^T Q
+    ref_nn = gemm(a, b_kn)
+    ref_tn = gemm(a_km, b_kn, trans_a=True, split_k=False)
+    with switch("NMTG_GEMM_RING_S"):
+        got_nn = gemm(a, b_kn)
+        got_tn = gemm(a_km, b_kn, trans_a=True, split_k=False)
+    # same products in the same order: identical bits
+    assert torch.equal(got_nn, ref_nn)
+    assert torch.equal(got_tn, ref_tn)
+    want = (a.double().cpu() @ b_kn.double().cpu())
+    assert_close(got_nn, want, dtype, "nn", scale_atol=True)
+
+
+def _self_fwd(dev, d, h, p, fused):
+    g = lambda k: d[k].to(dev) if d[k] is not None else None
+    dm = g("dropout_mask") if p > 0 else None
+    mask = g("time_mask") if d["time_mask"] is not None else g("pad_mask")
+    args = (d["time_mask"] is not None, True, h, g("x"), g("w_in"), g("w_out"), g("b_in"), g("b_out"), mask, p)
+    if fused:
+        with switch("NMTG_ATTN_FUSED"):
+            return sa_native.forward(*args, dropout_mask=dm)
+    return sa_native.forward(*args, dropout_mask=dm)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("t,b,e,h,p,causal", [(512, 2, 256, 4, 0.1, False), (128, 3, 512, 8, 0.0, False),
+                                              (200, 2, 256, 4, 0.25, False), (96, 2, 128, 2, 0.1, True),
+                                              (40, 2, 128, 2, 0.1, False)])
+def test_fused_scores_softmax_matches_two_kernel_path(dev, dtype, t, b, e, h, p, causal):
+    d = inputs.self_attn_inputs(t, b, e, h, dtype, p=p, seed=92, causal=causal, zero_bias=False)
+    lin0, sc0, dr0, dm0, ctx0, out0 = _self_fwd(dev, d, h, p, fused=False)
+    lin1, sc1, dr1, dm1, ctx1, out1 = _self_fwd(dev, d, h, p, fused=True)
+    assert torch.equal(lin0, lin1)
+    assert torch.equal(sc0, sc1)                         # scores: same product, same rounding, same -inf pattern
+    assert_close(dr1.float(), dr0.float().cpu(), dtype, "dropped vs two-kernel path")
+    assert torch.equal(dr1 == 0, dr0 == 0)               # masked keys and dropped units: zeros in the same places
+    fwd = oat.self_attn_fwd(d["x"], d["w_in"], d["w_out"], d["b_in"], d["b_out"], h, d["pad_mask"], d["time_mask"], p,
+                            d["dropout_mask"] if p > 0 else None, D, round_to=dtype)
+    assert_close(dr1, fwd["dropout_results"], dtype, "dropped vs oracle")
+    assert_close(out1, fwd["outputs"], dtype, "outputs vs oracle")
+
+
+def test_fused_scores_softmax_rng_mask_is_the_same_stream(dev):
+    # Philox keep-mask keyed by (seed, offset, element index): both paths must draw the same mask
+    dtype = torch.bfloat16
+    t, b, e, h = 64, 2, 128, 2
+    d = inputs.self_attn_inputs(t, b, e, h, dtype, p=0.0, seed=93, zero_bias=False)
+    g = lambda k: d[k].to(dev)
+    args = (False, True, h, g("x"), g("w_in"), g("w_out"), g("b_in"), g("b_out"), g("pad_mask"), 0.3)
+    torch.cuda.manual_seed(17)
+    r0 = sa_native.forward(*args)
+    torch.cuda.manual_seed(17)
+    with switch("NMTG_ATTN_FUSED"):
+        r1 = sa_native.forward(*args)
+    assert torch.equal(r0[3], r1[3])
+    assert_close(r1[2].float(), r0[2].float().cpu(), dtype, "dropped (rng)")
