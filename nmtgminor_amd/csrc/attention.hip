@@ -102,18 +102,30 @@ int core_bwd(const Core& c, Strided q, Strided k, Strided v, Strided dctx, const
     g.M = c.tk; g.N = c.d; g.K = c.tq; g.batch = c.bh; g.alpha = 1.f;
     if (int rc = gemm_run(c.dtype, LAYOUT_TN, EPI_PLAIN, g, nullptr, 0, c.st)) return rc;
   }
-  {  // dP [tq, tk] = dctx [tq, d] v^T
+  const bool drop = dmask != nullptr && p > 0.f;
+  {  // dP [tq, tk] = dctx [tq, d] v^T, then dS = softmax'(scores; g) in place
     GemmArgs g{};
     g.A = dctx.p; g.lda = dctx.ld; g.sA = dctx.stride;
     g.B = v.p; g.ldb = v.ld; g.sB = v.stride;
     g.C = ds_buf; g.ldc = c.tk; g.sC = tt;
     g.M = c.tq; g.N = c.tk; g.K = c.d; g.batch = c.bh; g.alpha = 1.f;
-    if (int rc = gemm_run(c.dtype, LAYOUT_NT, EPI_PLAIN, g, nullptr, 0, c.st)) return rc;
+    int fused = 0;
+    if (getenv("NMTG_ATTN_FUSED") != nullptr) {   // staged one-kernel form, see core_fwd
+      GemmArgs f = g;
+      f.aux_in = scores;
+      f.dmask = drop ? dmask : nullptr;
+      f.dscale = drop ? 1.f / (1.f - p) : 1.f;
+      fused = gemm_dsoftmax_try(c.dtype, f, c.st);
+      if (fused < 0) return fused;
+    }
+    if (!fused) {
+      if (int rc = gemm_run(c.dtype, LAYOUT_NT, EPI_PLAIN, g, nullptr, 0, c.st)) return rc;
+      if (int rc = nmtg_softmax_dropout_bwd(ds_buf, scores, 1, nullptr, 0, drop ? dmask : nullptr, drop ? 1 : 0,
+                                            drop ? p : 0.f, ds_buf, static_cast<int64_t>(c.bh) * c.tq, c.tk, c.tq, c.heads,
+                                            c.dtype, c.st))
+        return rc;
+    }
   }
-  const bool drop = dmask != nullptr && p > 0.f;
-  if (int rc = nmtg_softmax_dropout_bwd(ds_buf, scores, 1, nullptr, 0, drop ? dmask : nullptr, drop ? 1 : 0, drop ? p : 0.f,
-                                        ds_buf, static_cast<int64_t>(c.bh) * c.tq, c.tk, c.tq, c.heads, c.dtype, c.st))
-    return rc;
   {  // dq [tq, d] = scale dS [tq, tk] k [tk, d]
     GemmArgs g{};
     g.A = ds_buf; g.lda = c.tk; g.sA = tt;

@@ -40,7 +40,11 @@ enum GemmEpi {
   // C = alpha*acc with the mask as -inf (as EPI_SCORES), then the row softmax of the stored (rounded) scores and
   // dropout in the same pass: aux_out = softmax (optional), out2 = dropped probabilities. The block tile spans
   // the whole row (N <= BN), one wavefront normalises one row.
-  EPI_SCORES_SOFTMAX = 5
+  EPI_SCORES_SOFTMAX = 5,
+  // Backward counterpart on the same whole-row tile: acc = dP (gradient of the dropped probabilities, rounded to
+  // T as the two-kernel path stores it); P is recomputed from the saved scores (aux_in, laid out like C) and
+  // C = P * (g - sum_k P g), g = keep * dP / (1 - p).
+  EPI_DSOFTMAX = 6
 };
 
 struct GemmArgs {
@@ -577,6 +581,71 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, acc16_t (&acc)[
       return;
     }
 
+    if constexpr (EPI == EPI_DSOFTMAX) {
+      static_assert(CPR == 64 && VEC == 8, "the row tile is 512 columns wide and moves 16-byte chunks");
+      const uint16_t* SC = reinterpret_cast<const uint16_t*>(g.aux_in) + static_cast<int64_t>(bz) * g.sC;
+      const bool drop = g.dmask != nullptr;
+      constexpr float LOG2E = 1.4426950408889634f;
+      for (int p0 = 0; p0 < PASSES; p0 += GRP) {
+        uint4 sraw[GRP];
+        uint2 draw[GRP];
+#pragma unroll
+        for (int u = 0; u < GRP; ++u) {
+          const int m = m0 + (p0 + u) * RPP + r_in;
+          const int nv = m < g.M ? ncols : 0;
+          sraw[u] = load8<VEC, false>(SC + static_cast<int64_t>(m < g.M ? m : 0) * g.ldc + (nv > 0 ? n : 0), SC, nv);
+        }
+        if (drop) {
+#pragma unroll
+          for (int u = 0; u < GRP; ++u) {
+            const int m = m0 + (p0 + u) * RPP + r_in;
+            const int nv = m < g.M ? ncols : 0;
+            const int64_t row = static_cast<int64_t>(bz) * g.M + (m < g.M ? m : 0);
+            draw[u] = load8_bytes<VEC, false>(g.dmask + row * g.N + (nv > 0 ? n : 0), g.dmask, nv);
+          }
+        } else {
+#pragma unroll
+          for (int u = 0; u < GRP; ++u) draw[u] = make_uint2(0x01010101u, 0x01010101u);
+        }
+#pragma unroll
+        for (int u = 0; u < GRP; ++u) {
+          const int ml = (p0 + u) * RPP + r_in;
+          const int m = m0 + ml;
+          const int nv = m < g.M ? ncols : 0;
+          float gr[8], pr[8];
+          {
+            const uint2* sp = reinterpret_cast<const uint2*>(sC + ml * PITCH + cc * 16);
+            const uint2 lo = sp[0], hi = sp[1];
+            unpack8<T>(make_uint4(lo.x, lo.y, hi.x, hi.y), gr);
+          }
+          unpack8<T>(sraw[u], pr);
+#pragma unroll
+          for (int k = 0; k < 8; ++k) {
+            if (ncols <= 0) { pr[k] = -INFINITY; gr[k] = 0.f; }            // columns past N
+            else gr[k] = byte_of(draw[u], k) ? gr[k] * g.dscale : 0.f;      // g = keep * dP / (1 - p)
+          }
+          float mx = pr[0];
+#pragma unroll
+          for (int k = 1; k < 8; ++k) mx = fmaxf(mx, pr[k]);
+          mx = wave_max(mx);
+          const float base = (mx == -INFINITY) ? 0.f : mx;
+          float sum = 0.f;
+#pragma unroll
+          for (int k = 0; k < 8; ++k) { pr[k] = exp2f((pr[k] - base) * LOG2E); sum += pr[k]; }
+          sum = wave_sum(sum);
+          const float inv = sum > 0.f ? 1.f / sum : 0.f;
+          float dot = 0.f;
+#pragma unroll
+          for (int k = 0; k < 8; ++k) { pr[k] *= inv; dot += pr[k] * gr[k]; }
+          dot = wave_sum(dot);
+#pragma unroll
+          for (int k = 0; k < 8; ++k) gr[k] = pr[k] * (gr[k] - dot);
+          store8<VEC>(C + static_cast<int64_t>(m) * g.ldc + n, pack8<T>(gr), nv);
+        }
+      }
+      return;
+    }
+
     auto phase2 = [&](auto act_tag) {
     constexpr int ACT = decltype(act_tag)::value;
     for (int p0 = 0; p0 < PASSES; p0 += GRP) {
@@ -976,6 +1045,9 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
 // seed / offset. Returns 1 if the kernel was launched, 0 if the call does not qualify (the caller then runs the
 // scores GEMM and the softmax kernel), or a negative nmtg_status.
 int gemm_scores_softmax_try(int dtype, GemmArgs a, hipStream_t st);
+// Backward counterpart (EPI_DSOFTMAX): A = dctx, B = v, aux_in = saved scores, dmask / dscale for a replayed
+// dropout mask, C = gradient of the scores. Same return convention.
+int gemm_dsoftmax_try(int dtype, GemmArgs a, hipStream_t st);
 
 // bias-gradient style column sums: out[n] = sum_m X[m][n]; part is fp32 scratch of
 // colsum_parts(M) * N floats.

@@ -162,13 +162,15 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
   return 0;
 }
 
-int gemm_scores_softmax_try(int dtype, GemmArgs a, hipStream_t st) {
+namespace {
+// Shared eligibility test and launch of the whole-row tile (128 x 512, N <= 512): 16-byte accesses everywhere.
+int row_tile_try(int dtype, int epi, GemmArgs a, const void* extra_like_c, hipStream_t st) {
   if (a.M <= 0 || a.N <= 0 || a.batch <= 0) return 0;
   if (dtype != NMTG_F16 && dtype != NMTG_BF16) return 0;
-  if (a.N > 512 || a.N % 8 != 0 || a.K <= 0 || a.K % 8 != 0 || a.batch > 65535 || !a.out2) return 0;
+  if (a.N > 512 || a.N % 8 != 0 || a.K <= 0 || a.K % 8 != 0 || a.batch > 65535 || !extra_like_c) return 0;
   auto ok16 = [](const void* p, int64_t ld, int64_t stride, int batch) { return vec_of(p, ld, stride, batch) == 8; };
   if (!ok16(a.A, a.lda, a.sA, a.batch) || !ok16(a.B, a.ldb, a.sB, a.batch) || !ok16(a.C, a.ldc, a.sC, a.batch) ||
-      !ok16(a.out2, a.ldc, a.sC, a.batch) || (a.aux_out && !ok16(a.aux_out, a.ldc, a.sC, a.batch)))
+      !ok16(extra_like_c, a.ldc, a.sC, a.batch) || (a.aux_out && !ok16(a.aux_out, a.ldc, a.sC, a.batch)))
     return 0;
   auto ok8 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 8 == 0; };
   if ((a.dmask && !ok8(a.dmask)) || (a.kmask && a.kmask_kind != 0 && !ok8(a.kmask))) return 0;
@@ -179,11 +181,23 @@ int gemm_scores_softmax_try(int dtype, GemmArgs a, hipStream_t st) {
   a.k_per_split = ceil_div(a.K, GEMM_BK) * GEMM_BK;
   a.m_tiles = ceil_div(a.M, 128);
   a.n_tiles = 1;
-  if (static_cast<int64_t>(a.m_tiles) > 0x7fffffff) return 0;
-  if (int rc = gemm_launch_nt(dtype, TILE_R, EPI_SCORES_SOFTMAX, a, st)) return rc;
+  if (int rc = gemm_launch_nt(dtype, TILE_R, epi, a, st)) return rc;
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(NMTG_ERR_LAUNCH, "gemm: launch failed: %s", hipGetErrorString(e));
   return 1;
+}
+}  // namespace
+
+int gemm_scores_softmax_try(int dtype, GemmArgs a, hipStream_t st) {
+  return row_tile_try(dtype, EPI_SCORES_SOFTMAX, a, a.out2, st);
+}
+
+int gemm_dsoftmax_try(int dtype, GemmArgs a, hipStream_t st) {
+  a.bias = nullptr;
+  a.aux_out = nullptr;
+  a.kmask = nullptr;
+  a.kmask_kind = 0;
+  return row_tile_try(dtype, EPI_DSOFTMAX, a, a.aux_in, st);
 }
 
 int colsum_parts(int M) { return std::max(1, std::min(64, ceil_div(M, 128))); }

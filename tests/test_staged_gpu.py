@@ -97,3 +97,24 @@ def test_fused_scores_softmax_rng_mask_is_the_same_stream(dev):
         r1 = sa_native.forward(*args)
     assert torch.equal(r0[3], r1[3])
     assert_close(r1[2].float(), r0[2].float().cpu(), dtype, "dropped (rng)")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("t,b,e,h,p,causal", [(512, 2, 256, 4, 0.1, False), (200, 2, 256, 4, 0.25, False),
+                                              (96, 2, 128, 2, 0.0, True), (40, 2, 128, 2, 0.1, False)])
+def test_fused_softmax_backward_matches_two_kernel_path(dev, dtype, t, b, e, h, p, causal):
+    d = inputs.self_attn_inputs(t, b, e, h, dtype, p=p, seed=94, causal=causal, zero_bias=False)
+    lin, scores, dropped, dmask, ctx, out = _self_fwd(dev, d, h, p, fused=False)
+    g = lambda k: d[k].to(dev)
+    args = (causal, h, g("dout"), ctx, dropped, scores, lin, g("x"), g("w_in"), g("w_out"), dmask, p)
+    ref = sa_native.backward(*args)
+    with switch("NMTG_ATTN_FUSED"):
+        got = sa_native.backward(*args)
+    fwd = oat.self_attn_fwd(d["x"], d["w_in"], d["w_out"], d["b_in"], d["b_out"], h, d["pad_mask"], d["time_mask"], p,
+                            d["dropout_mask"] if p > 0 else None, D, round_to=dtype)
+    bwd = oat.self_attn_bwd(d["dout"], d["x"], d["w_in"], d["w_out"], h, fwd, p, d["dropout_mask"] if p > 0 else None, D,
+                            round_to=dtype)
+    for name, a_, r_, o_ in zip(("dx", "dw_in", "dw_out", "db_in", "db_out"), got, ref,
+                                (bwd["dx"], bwd["dw_in"], bwd["dw_out"], bwd["db_in"], bwd["db_out"])):
+        assert_close(a_, r_.float().cpu(), dtype, name + " vs two-kernel path", scale_atol=True)
+        assert_close(a_, o_, dtype, name + " vs oracle", scale_atol=True)
