@@ -3,6 +3,7 @@
 #include "trace.cuh"
 #include <cstring>
 #include <algorithm>
+#include <atomic>
 #include <map>
 #include <mutex>
 #include <vector>
@@ -16,14 +17,14 @@ struct Record {
 };
 
 std::mutex g_mu;
-bool g_on = false;
+std::atomic<bool> g_on{false};   // read without the lock on every launch
 std::vector<Record> g_records;        // records in use since trace_begin
 std::vector<Record> g_pool;           // events kept for reuse
 constexpr size_t MAX_RECORDS = 1 << 16;
 
 }  // namespace
 
-bool trace_on() { return g_on; }
+bool trace_on() { return g_on.load(std::memory_order_relaxed); }
 
 void trace_open(const char* name, hipStream_t st, int* slot) {
   std::lock_guard<std::mutex> lk(g_mu);
