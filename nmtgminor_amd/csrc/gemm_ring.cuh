@@ -50,6 +50,9 @@ __device__ __forceinline__ void static_for(F&& f) {
 }
 
 // One transfer: lane l copies the 16 bytes at sbase + voff(l) to LDS address lds_addr + 16 l.
+// M0 carries the LDS address. The compiler warns that M0 is a reserved register it will not save
+// around the statement; that is what is wanted: on gfx9 it only ever writes M0 immediately before
+// an instruction of its own that reads it, never keeps a value in it across other code.
 __device__ __forceinline__ void dma16(uint32_t voff, const void* sbase, uint32_t lds_addr) {
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                :
