@@ -496,7 +496,13 @@ def main():
     for n in names:
         w = table[n]()
         steps = args.steps if w.name != "xentropy" else max(3, min(args.steps, 10))
-        results.append(measure(w, dev, steps, args.warmup, not args.no_cpu, min(args.trace_steps, steps)))
+        try:
+            results.append(measure(w, dev, steps, args.warmup, not args.no_cpu, min(args.trace_steps, steps)))
+        except Exception as e:
+            if n == names[0]:
+                raise                    # no headline without the first workload
+            sys.stderr.write(f"[bench] workload {n} failed: {e}\n")
+            results.append(dict(workload=n, error=str(e)))
         results[-1]["steps"] = steps
         del w
         torch.cuda.empty_cache()
