@@ -81,6 +81,30 @@ template <typename T, int N> struct alignas(sizeof(T) * N >= 16 ? 16 : sizeof(T)
   T v[N];
 };
 
+// Load without conversion / conversion without load: a kernel that wants several loads in flight issues all its
+// load_raw calls first and converts afterwards (a conversion is a use of the loaded registers, and the compiler
+// waits for a load at its first use).
+template <typename T, int N>
+__device__ __forceinline__ pack<T, N> load_raw(const T* __restrict__ p) {
+  return *reinterpret_cast<const pack<T, N>*>(p);
+}
+// Pins a loaded pack in registers at this point of the program: the compiler may otherwise sink a load into the
+// branch that holds its only use, where it waits for it alone.
+template <typename T, int N>
+__device__ __forceinline__ void pin_raw(pack<T, N>& r) {
+  static_assert(sizeof(pack<T, N>) % 4 == 0, "whole 32-bit words");
+  uint32_t w[sizeof(pack<T, N>) / 4];
+  __builtin_memcpy(w, &r, sizeof(w));
+#pragma unroll
+  for (int k = 0; k < static_cast<int>(sizeof(w) / 4); ++k) asm volatile("" : "+v"(w[k]));
+  __builtin_memcpy(&r, w, sizeof(w));
+}
+template <typename T, int N>
+__device__ __forceinline__ void unpack_raw(const pack<T, N>& r, float (&out)[N]) {
+#pragma unroll
+  for (int j = 0; j < N; ++j) out[j] = elem<T>::to_float(r.v[j]);
+}
+
 template <typename T, int N>
 __device__ __forceinline__ void load_pack(const T* __restrict__ p, float (&out)[N]) {
   constexpr int BYTES = sizeof(T) * N;

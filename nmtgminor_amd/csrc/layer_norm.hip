@@ -74,16 +74,36 @@ __global__ __launch_bounds__(LN_THREADS) void ln_fwd_kernel(
   const float rn = 1.f / static_cast<float>(hidden);
   const int64_t groups = (rows + RPB - 1) / RPB;
 
+  // Loads are issued unconditionally from clamped (always mapped) addresses and ahead of any use: a load inside a
+  // branch waits for its own data before the next one is issued, which made a row cost four memory latencies.
+  pack<TW, EPV> gr[VPL], br[VPL];
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    const int col = ((sub * VPL + i) * kWave + lane) * EPV;
+    const int cc = col < hidden ? col : 0;
+    gr[i] = load_raw<TW, EPV>(gamma + cc);
+    br[i] = load_raw<TW, EPV>(beta + cc);
+  }
+
   for (int64_t g = blockIdx.x; g < groups; g += gridDim.x) {
     const int64_t row = g * RPB + wave / WPR;
     const bool row_ok = row < rows;
+    const int64_t rowc = row_ok ? row : 0;
+    pack<TI, EPV> xr[VPL];
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      const int col = ((sub * VPL + i) * kWave + lane) * EPV;
+      xr[i] = load_raw<TI, EPV>(x + rowc * hidden + (col < hidden ? col : 0));
+    }
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) pin_raw(xr[i]);
     float xf[VPL][EPV];
     float s = 0.f;
 #pragma unroll
     for (int i = 0; i < VPL; ++i) {
       const int col = ((sub * VPL + i) * kWave + lane) * EPV;
       if (row_ok && col < hidden) {
-        load_pack<TI, EPV>(x + row * hidden + col, xf[i]);
+        unpack_raw<TI, EPV>(xr[i], xf[i]);
 #pragma unroll
         for (int j = 0; j < EPV; ++j) s += xf[i][j];
       } else {
@@ -109,8 +129,8 @@ __global__ __launch_bounds__(LN_THREADS) void ln_fwd_kernel(
       const int col = ((sub * VPL + i) * kWave + lane) * EPV;
       if (row_ok && col < hidden) {
         float gf[EPV], bf[EPV], zf[EPV];
-        load_pack<TW, EPV>(gamma + col, gf);
-        load_pack<TW, EPV>(beta + col, bf);
+        unpack_raw<TW, EPV>(gr[i], gf);
+        unpack_raw<TW, EPV>(br[i], bf);
 #pragma unroll
         for (int j = 0; j < EPV; ++j) zf[j] = gf[j] * (rs * (xf[i][j] - mean)) + bf[j];
         store_pack<TW, EPV>(z + row * hidden + col, zf);
@@ -193,19 +213,30 @@ __global__ __launch_bounds__(LN_THREADS) void ln_bwd_kernel(
     const int64_t row = g * RPB + wave / WPR;
     const bool row_ok = row < rows;
     float dy[VPL][EPV], y[VPL][EPV];
-    float rs = 0.f, mean = 0.f;
-    if (row_ok) {
-      rs = rsigma[row];
-      if constexpr (!MEMEFF) mean = mu[row];
+    // every load of the row first, from clamped addresses (see ln_fwd_kernel)
+    const int64_t rowc = row_ok ? row : 0;
+    float rs = rsigma[rowc], mean = 0.f;
+    if constexpr (!MEMEFF) mean = mu[rowc];
+    pack<TW, EPV> dzr[VPL];
+    pack<TI, EPV> xr[VPL];
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      const int col = ((sub * VPL + i) * kWave + lane) * EPV;
+      const int cc = col < hidden ? col : 0;
+      dzr[i] = load_raw<TW, EPV>(dz + rowc * hidden + cc);
+      xr[i] = load_raw<TI, EPV>(x_or_z + rowc * hidden + cc);
     }
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) { pin_raw(dzr[i]); pin_raw(xr[i]); }
+    if (!row_ok) { rs = 0.f; mean = 0.f; }
     float sdy = 0.f, sdyy = 0.f;
 #pragma unroll
     for (int i = 0; i < VPL; ++i) {
       const int col = ((sub * VPL + i) * kWave + lane) * EPV;
       if (row_ok && col < hidden) {
         float dzf[EPV], xf[EPV];
-        load_pack<TW, EPV>(dz + row * hidden + col, dzf);
-        load_pack<TI, EPV>(x_or_z + row * hidden + col, xf);
+        unpack_raw<TW, EPV>(dzr[i], dzf);
+        unpack_raw<TI, EPV>(xr[i], xf);
 #pragma unroll
         for (int j = 0; j < EPV; ++j) {
           float yv;
