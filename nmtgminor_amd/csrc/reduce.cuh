@@ -1,0 +1,153 @@
+// Small fixed-order reduction kernels that follow a GEMM: the sum over split-K partials and the column sums behind
+// every bias gradient. They are latency-bound (a few blocks, short dependent chains), so each keeps a batch of loads
+// in flight before the first add. Hosts: reduce.hip (column sums), gemm_inst.cuh (split-K).
+#pragma once
+#include "common.cuh"
+
+namespace nmtg {
+
+// Sums the split-K partials (in the accumulator layout the GEMM kernels' split-K epilogue writes, gemm.cuh), scales, converts to T and
+// writes row-major C; fixed summation order.
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, T* __restrict__ C, int64_t ldc,
+                                                            int M, int N, int m_tiles, int n_tiles, int batch,
+                                                            int64_t sC, int splits, float alpha, int c_vec) {
+  constexpr int NW = WAVES_M * WAVES_N;
+  constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int PER_BLK = NW * TM * TN * 4 * 64;  // float4 slots per tile
+  const int64_t total = static_cast<int64_t>(batch) * m_tiles * n_tiles * PER_BLK;
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int lane = idx & 63;
+  int64_t t = idx >> 6;
+  const int q = t & 3; t >>= 2;
+  const int j = t % TN; t /= TN;
+  const int i = t % TM; t /= TM;
+  const int wave = t % NW; t /= NW;
+  const int tile = t % (m_tiles * n_tiles);
+  const int bz = t / (m_tiles * n_tiles);
+  const int tile_m = tile / n_tiles, tile_n = tile % n_tiles;
+  const int m = tile_m * BM + (wave / WAVES_N) * WTM + i * 32 + (lane & 31);
+  const int n = tile_n * BN + (wave % WAVES_N) * WTN + j * 32 + q * 8 + (lane >> 5) * 4;
+  if (m >= M || n >= N) return;
+  const int64_t per_split = static_cast<int64_t>(batch) * m_tiles * n_tiles * PER_BLK;
+  float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+  const float4* w = reinterpret_cast<const float4*>(ws) + idx;
+  int sp = 0;
+  for (; sp + 4 <= splits; sp += 4) {   // four partials in flight, summed in split order
+    float4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] = w[(sp + u) * per_split];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) { s.x += v[u].x; s.y += v[u].y; s.z += v[u].z; s.w += v[u].w; }
+  }
+  for (; sp < splits; ++sp) {
+    const float4 v = w[sp * per_split];
+    s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+  }
+  const float v[4] = {s.x * alpha, s.y * alpha, s.z * alpha, s.w * alpha};
+  T* dst = C + static_cast<int64_t>(bz) * sC + static_cast<int64_t>(m) * ldc + n;
+  if (n + 4 <= N && c_vec >= 4) store_pack<T, 4>(dst, v);
+  else for (int e = 0; e < 4 && n + e < N; ++e) dst[e] = elem<T>::from_float(v[e]);
+}
+
+// Column sums of a row-major [M, N] matrix: partial[mb][n] over row blocks (fp32), fixed order.
+// Block = 32 column lanes (8 columns each = one 16-byte load for 16-bit T) x 8 row lanes.
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void colsum_partial_kernel(const T* __restrict__ X, int64_t ld, int M, int N,
+                                                             int rows_per_block, float* __restrict__ part) {
+  constexpr int CPT = VEC ? 8 : 1;
+  __shared__ float red[8][32 * CPT + 1];
+  const int cl = threadIdx.x & 31, rl = threadIdx.x >> 5;
+  const int n = (blockIdx.x * 32 + cl) * CPT;
+  const int r0 = blockIdx.y * rows_per_block;
+  const int r1 = min(M, r0 + rows_per_block);
+  float s[CPT];
+#pragma unroll
+  for (int j = 0; j < CPT; ++j) s[j] = 0.f;
+  if (n < N) {
+    // Latency-bound (few blocks, short rows): 16 rows are loaded before any is added (two loops on
+    // purpose, see ln_bwd_finalize_kernel); the sum order is unchanged.
+    constexpr int BATCH = 16;
+    int r = r0 + rl;
+    for (; r + (BATCH - 1) * 8 < r1; r += BATCH * 8) {
+      // raw words first, conversion only in the adding loop (a conversion is a use of the load)
+      constexpr int NV = (CPT * sizeof(T)) / 16;   // 16-byte vectors per access; 0 in the scalar form
+      if constexpr (NV > 0) {
+        uint4 raw[BATCH][NV];
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u)
+#pragma unroll
+          for (int i = 0; i < NV; ++i)
+            raw[u][i] = reinterpret_cast<const uint4*>(X + static_cast<int64_t>(r + u * 8) * ld + n)[i];
+        __builtin_amdgcn_sched_barrier(0);   // keep every load ahead of the first add
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) {
+          const T* e = reinterpret_cast<const T*>(raw[u]);
+#pragma unroll
+          for (int j = 0; j < CPT; ++j) s[j] += elem<T>::to_float(e[j]);
+        }
+      } else {
+        T raw[BATCH];
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) raw[u] = X[static_cast<int64_t>(r + u * 8) * ld + n];
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) s[0] += elem<T>::to_float(raw[u]);
+      }
+    }
+    for (; r < r1; r += 8) {
+      float v[CPT];
+      load_pack<T, CPT>(X + static_cast<int64_t>(r) * ld + n, v);
+#pragma unroll
+      for (int j = 0; j < CPT; ++j) s[j] += v[j];
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < CPT; ++j) red[rl][cl * CPT + j] = s[j];
+  __syncthreads();
+  for (int c = threadIdx.x; c < 32 * CPT; c += 256) {
+    const int col = blockIdx.x * 32 * CPT + c;
+    if (col < N) {
+      float t = 0.f;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) t += red[k][c];
+      part[static_cast<int64_t>(blockIdx.y) * N + col] = t;
+    }
+  }
+}
+
+// out[n] = T(sum_p part[p][n]) in order p = 0..parts-1; 8 partial rows in flight per thread.
+template <typename T>
+__global__ __launch_bounds__(256) void colsum_final_kernel(const float* __restrict__ part, int parts, int N,
+                                                           T* __restrict__ out) {
+  const int n = blockIdx.x * 256 + threadIdx.x;
+  if (n >= N) return;
+  float s = 0.f;
+  int p = 0;
+  // a few blocks of dependent-latency work: 32, then 8 partial rows in flight per thread
+  for (; p + 32 <= parts; p += 32) {
+    float v[32];
+#pragma unroll
+    for (int j = 0; j < 32; ++j) v[j] = part[static_cast<int64_t>(p + j) * N + n];
+#pragma unroll
+    for (int j = 0; j < 32; ++j) s += v[j];
+  }
+  for (; p + 8 <= parts; p += 8) {
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = part[static_cast<int64_t>(p + j) * N + n];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s += v[j];
+  }
+  for (; p < parts; ++p) s += part[static_cast<int64_t>(p) * N + n];
+  out[n] = elem<T>::from_float(s);
+}
+
+// bias-gradient style column sums: out[n] = sum_m X[m][n]; part is fp32 scratch of
+// colsum_parts(M) * N floats.
+int colsum_parts(int M);
+int colsum_run(int dtype, const void* X, int64_t ld, int M, int N, float* part, void* out, hipStream_t st);
+int colsum_finish(int dtype, const float* part, int parts, int N, void* out, hipStream_t st);
+
+}  // namespace nmtg

@@ -1,0 +1,111 @@
+"""Builds tests/hostsim/_build/libnmtg_hostsim.so: the library's elementwise kernel sources (LayerNorm, softmax +
+dropout, dropout + add, cross-entropy, the column-sum and split-K reductions) compiled as plain C++ for the CPU and run lane by lane by hostsim.cpp.
+
+The kernel sources are used as they are, apart from three textual substitutions that C++ needs:
+    extern __shared__ T name[];   ->  T* name = (T*) the simulator's dynamic-LDS block
+    __shared__                    ->  static            (blocks run one after the other, so one copy is per block)
+    "+v" asm register constraint  ->  "+r"              (an empty asm statement that only pins a value)
+and the path of the public header. The result exports the same extern "C" entry points as libnmtg_hip.so for those
+operators, plus hostsim_* hooks (stubs.cpp) for the reductions that have no entry point of their own, and takes host
+pointers. Test infrastructure: python tests/hostsim/build.py
+"""
+import os
+import re
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+CSRC = os.path.join(ROOT, "nmtgminor_amd", "csrc")
+BUILD = os.path.join(HERE, "_build")
+CXX = os.environ.get("HOSTSIM_CXX", "/opt/rocm/lib/llvm/bin/clang++")
+# HOSTSIM_SANITIZE=1: AddressSanitizer build (host code only). The kernels' loads and stores are then checked against
+# the bounds of the tensors they are handed, when the process runs with the sanitizer's runtime preloaded:
+#   HOSTSIM_SANITIZE=1 LD_PRELOAD=$(clang++ -print-file-name=libclang_rt.asan-x86_64.so) \
+#   ASAN_OPTIONS=detect_leaks=0:detect_stack_use_after_return=0 python -m pytest tests/test_hostsim_cpu.py
+SANITIZE = os.environ.get("HOSTSIM_SANITIZE") == "1"
+LIB = os.path.join(BUILD, "libnmtg_hostsim_asan.so" if SANITIZE else "libnmtg_hostsim.so")
+
+KERNEL_SOURCES = ["api.hip", "layer_norm.hip", "softmax_dropout.hip", "dropout_add.hip", "xentropy.hip", "reduce.hip"]
+HEADERS = ["common.cuh", "trace.cuh", "reduce.cuh"]
+OWN_SOURCES = ["hostsim.cpp", "stubs.cpp"]
+
+
+def transform(text):
+    text = re.sub(r"extern\s+__shared__\s+([A-Za-z_][\w:]*)\s+(\w+)\s*\[\s*\]\s*;",
+                  r"\1* \2 = reinterpret_cast<\1*>(::hostsim::dynamic_lds);", text)
+    text = re.sub(r"\b__shared__\b", "static", text)
+    text = text.replace('"+v"', '"+r"')
+    text = text.replace('"../../include/nmtg_hip.h"', '"%s"' % os.path.join(ROOT, "include", "nmtg_hip.h"))
+    return text
+
+
+def sources():
+    out = [os.path.join(CSRC, n) for n in KERNEL_SOURCES + HEADERS if os.path.exists(os.path.join(CSRC, n))]
+    out += [os.path.join(HERE, n) for n in OWN_SOURCES]
+    out += [os.path.join(HERE, "shim", "hip", n) for n in os.listdir(os.path.join(HERE, "shim", "hip"))]
+    out.append(os.path.abspath(__file__))
+    return out
+
+
+def stale():
+    if not os.path.exists(LIB):
+        return True
+    built = os.path.getmtime(LIB)
+    return any(os.path.getmtime(s) > built for s in sources())
+
+
+def available():
+    return os.path.exists(CXX)
+
+
+def build(verbose=False):
+    os.makedirs(BUILD, exist_ok=True)
+    units = []
+    for name in KERNEL_SOURCES + HEADERS:
+        src = os.path.join(CSRC, name)
+        if not os.path.exists(src):
+            continue
+        dst = os.path.join(BUILD, name if name.endswith(".cuh") else name.replace(".hip", ".cpp"))
+        with open(src) as f:
+            text = '#line 1 "%s"\n' % src + transform(f.read())
+        with open(dst, "w") as f:
+            f.write(text)
+        if not name.endswith(".cuh"):
+            units.append(dst)
+    units += [os.path.join(HERE, n) for n in OWN_SOURCES]
+    flags = ["-x", "c++", "-std=c++17", "-O1", "-g", "-fPIC", "-fno-strict-aliasing", "-Wno-unknown-pragmas",
+             "-Wno-pass-failed", "-Wno-unused-command-line-argument", "-I" + os.path.join(HERE, "shim"), "-I" + BUILD]
+    link = []
+    if SANITIZE:
+        # host code only: there is no device code in this build at all (-x c++)
+        flags += ["-fsanitize=address", "-fno-gpu-sanitize", "-shared-libasan", "-fno-omit-frame-pointer"]
+        link = ["-fsanitize=address", "-fno-gpu-sanitize", "-shared-libasan"]
+    objs = []
+    procs = []
+    for u in units:
+        obj = os.path.join(BUILD, os.path.basename(u) + (".asan.o" if SANITIZE else ".o"))
+        objs.append(obj)
+        procs.append((u, subprocess.Popen([CXX] + flags + ["-c", u, "-o", obj], stdout=subprocess.PIPE,
+                                          stderr=subprocess.STDOUT, text=True)))
+    failed = False
+    for u, p in procs:
+        out, _ = p.communicate()
+        if p.returncode != 0 or verbose:
+            sys.stderr.write(out)
+        failed |= p.returncode != 0
+    if failed:
+        raise RuntimeError("hostsim: compilation failed")
+    subprocess.check_call([CXX, "-shared", "-o", LIB] + link + objs)
+    return LIB
+
+
+def ensure():
+    """Path of an up-to-date library (built on demand)."""
+    if stale():
+        build()
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

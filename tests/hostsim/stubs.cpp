@@ -1,0 +1,37 @@
+// Pieces of the library that the CPU build does not take from the kernel sources (per-kernel event tracing is off),
+// and C hooks for the reduction kernels, which the real library only reaches from inside its GEMM-based operators.
+#include "reduce.cuh"
+
+namespace nmtg {
+bool trace_on() { return false; }
+void trace_open(const char*, hipStream_t, int*) {}
+void trace_close(hipStream_t, int) {}
+}  // namespace nmtg
+
+using namespace nmtg;
+
+extern "C" int hostsim_colsum_parts(int M) { return colsum_parts(M); }
+
+extern "C" int hostsim_colsum(int dtype, const void* X, int64_t ld, int M, int N, float* part, void* out) {
+  return colsum_run(dtype, X, ld, M, N, part, out, nullptr);
+}
+
+// Split-K reduction for the 128x128 tile (2 x 2 wavefronts) and the 256x256 tile (2 x 4), launched as gemm_inst.cuh does.
+template <typename T, int BM, int BN, int WM, int WN>
+static int splitk(const float* ws, void* C, int64_t ldc, int M, int N, int m_tiles, int n_tiles, int batch, int64_t sC,
+                  int splits, float alpha, int c_vec) {
+  constexpr int per_blk = WM * WN * (BM / WM / 32) * (BN / WN / 32) * 4 * 64;
+  const int64_t total = static_cast<int64_t>(batch) * m_tiles * n_tiles * per_blk;
+  hipLaunchKernelGGL((splitk_reduce_kernel<T, BM, BN, WM, WN>), dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0,
+                     nullptr, ws, static_cast<T*>(C), ldc, M, N, m_tiles, n_tiles, batch, sC, splits, alpha, c_vec);
+  return 0;
+}
+
+extern "C" int hostsim_splitk_reduce(int dtype, int tile, const float* ws, void* C, int64_t ldc, int M, int N, int m_tiles,
+                                     int n_tiles, int batch, int64_t sC, int splits, float alpha, int c_vec) {
+  if (tile == 1) {
+    NMTG_DISPATCH_DTYPE(dtype, T, return (splitk<T, 128, 128, 2, 2>(ws, C, ldc, M, N, m_tiles, n_tiles, batch, sC, splits, alpha, c_vec)));
+  }
+  NMTG_DISPATCH_DTYPE(dtype, T, return (splitk<T, 256, 256, 2, 4>(ws, C, ldc, M, N, m_tiles, n_tiles, batch, sC, splits, alpha, c_vec)));
+  return -1;
+}
