@@ -26,13 +26,31 @@ CXX = os.environ.get("HOSTSIM_CXX", "/opt/rocm/lib/llvm/bin/clang++")
 SANITIZE = os.environ.get("HOSTSIM_SANITIZE") == "1"
 LIB = os.path.join(BUILD, "libnmtg_hostsim_asan.so" if SANITIZE else "libnmtg_hostsim.so")
 
-KERNEL_SOURCES = ["api.hip", "layer_norm.hip", "softmax_dropout.hip", "dropout_add.hip", "xentropy.hip", "reduce.hip"]
-HEADERS = ["common.cuh", "trace.cuh", "reduce.cuh"]
+KERNEL_SOURCES = ["api.hip", "layer_norm.hip", "softmax_dropout.hip", "dropout_add.hip", "xentropy.hip", "reduce.hip",
+                  "gemm.hip", "gemm_nt.hip", "gemm_nn.hip", "gemm_tn.hip", "mlp.hip", "attention.hip"]
+HEADERS = ["common.cuh", "trace.cuh", "reduce.cuh", "gemm.cuh", "gemm_ring.cuh", "gemm_inst.cuh"]
 OWN_SOURCES = ["hostsim.cpp", "stubs.cpp"]
 
 
+# Inline assembly cannot be compiled for the host. Every statement is listed here with what it does, and a statement
+# that is not listed stops the build.
+ASM_REWRITES = [
+    # one 1 KB global -> LDS transfer: lane l copies 16 bytes from sbase + voff to LDS address lds_addr + 16 l
+    (r'asm volatile\("s_mov_b32 m0, %2\\n\\ts_nop 0\\n\\tglobal_load_lds_dwordx4 %0, %1"\s*:\s*:\s*"v"\(voff\), "s"\(sbase\), '
+     r'"s"\(lds_addr\)\s*:\s*"memory", "m0"\);',
+     "::hostsim::dma_issue(static_cast<const char*>(sbase) + voff, lds_addr + 16 * ::hostsim::lane_id(), 16);"),
+    # LDS reads done, then the workgroup barrier
+    (r'asm volatile\("s_waitcnt lgkmcnt\(0\)\\n\\ts_barrier" ::: "memory"\);', "::hostsim::sync_block();"),
+]
+
+
 def transform(text):
-    text = re.sub(r"extern\s+__shared__\s+([A-Za-z_][\w:]*)\s+(\w+)\s*\[\s*\]\s*;",
+    for pattern, replacement in ASM_REWRITES:
+        text = re.sub(pattern, lambda m: replacement, text)
+    left = [m.group(0) for m in re.finditer(r'asm volatile\("[^"]+"', text)]
+    if left:
+        raise RuntimeError("hostsim: inline assembly without a host translation: %s" % left[0])
+    text = re.sub(r"extern\s+__shared__\s+(?:__align__\(\d+\)\s+)?([A-Za-z_][\w:]*)\s+(\w+)\s*\[\s*\]\s*;",
                   r"\1* \2 = reinterpret_cast<\1*>(::hostsim::dynamic_lds);", text)
     text = re.sub(r"\b__shared__\b", "static", text)
     text = text.replace('"+v"', '"+r"')
@@ -74,7 +92,7 @@ def build(verbose=False):
         if not name.endswith(".cuh"):
             units.append(dst)
     units += [os.path.join(HERE, n) for n in OWN_SOURCES]
-    flags = ["-x", "c++", "-std=c++17", "-O1", "-g", "-fPIC", "-fno-strict-aliasing", "-Wno-unknown-pragmas",
+    flags = ["-x", "c++", "-std=c++17", "-O1", "-gline-tables-only", "-fPIC", "-fno-strict-aliasing", "-Wno-unknown-pragmas",
              "-Wno-pass-failed", "-Wno-unused-command-line-argument", "-I" + os.path.join(HERE, "shim"), "-I" + BUILD]
     link = []
     if SANITIZE:

@@ -1,16 +1,57 @@
 // CPU execution of HIP kernels compiled as plain C++ (see shim/hip/hip_runtime.h): blocks run one after the other,
-// every thread of a block is a fiber (ucontext), and fibers meet at wavefront shuffles and block barriers exactly as
-// 64-lane wavefronts do. One OS thread runs everything, so runs are deterministic. Checks that hardware does not make:
-//   - a shuffle reached by only part of a wavefront, or with different lane masks, aborts with a message;
+// every thread of a block is a fiber (ucontext), and fibers meet at wavefront-wide operations (shuffles, MFMA, LDS
+// transpose reads) and block barriers exactly as 64-lane wavefronts do. One OS thread runs everything, so runs are
+// deterministic. Checks that hardware does not make:
+//   - a wavefront-wide operation reached by only part of a wavefront, or by lanes that disagree on the operation,
+//     aborts with a message;
 //   - a block barrier that some live wavefront never reaches while others wait aborts with a message.
+// Direct global -> LDS transfers are asynchronous on the hardware. HOSTSIM_DMA picks one of the two extreme timings:
+//   late  (default)  a transfer lands only when its lane executes the vmcnt wait that covers it: a missing or too
+//                    weak wait leaves stale (poisoned) LDS behind the reads that needed it;
+//   early            a transfer lands the moment it is issued: a slot that is refilled before every wavefront has
+//                    finished reading it corrupts those reads (the scheduler runs wavefront 0 as far as it can go,
+//                    then wavefront 1, ..., so later wavefronts are the slow readers).
+// Dynamic LDS is filled with 0xFF bytes (NaN in every float format used) at the start of every block.
 // Test infrastructure only.
 #include <hip/hip_runtime.h>
 
 #include <sys/mman.h>
 #include <ucontext.h>
 
+// Switching fibers with swapcontext costs two system calls (the signal mask). The plain x86-64 build switches with
+// a dozen instructions instead; the AddressSanitizer build keeps swapcontext, which the sanitizer knows how to follow.
+#if defined(__x86_64__) && !defined(__SANITIZE_ADDRESS__) && !(defined(__has_feature) && __has_feature(address_sanitizer))
+#define HOSTSIM_FAST_SWITCH 1
+extern "C" void hostsim_switch(void** save_sp, void* load_sp);
+asm(R"(
+    .text
+    .globl hostsim_switch
+    .type hostsim_switch,@function
+hostsim_switch:
+    pushq %rbp
+    pushq %rbx
+    pushq %r12
+    pushq %r13
+    pushq %r14
+    pushq %r15
+    movq %rsp, (%rdi)
+    movq %rsi, %rsp
+    popq %r15
+    popq %r14
+    popq %r13
+    popq %r12
+    popq %rbx
+    popq %rbp
+    ret
+    .size hostsim_switch,.-hostsim_switch
+)");
+#else
+#define HOSTSIM_FAST_SWITCH 0
+#endif
+
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <vector>
 
 hostsim::Index threadIdx, blockIdx;
@@ -26,18 +67,30 @@ constexpr int WAVE = 64;
 constexpr size_t STACK_BYTES = 256 << 10;
 constexpr size_t LDS_BYTES = 160 << 10;
 
-enum State { RUNNABLE, AT_SHUFFLE, AT_BARRIER, DONE };
+enum State { RUNNABLE, AT_COLLECTIVE, AT_BARRIER, DONE };
+
+struct Transfer {
+  const void* src;
+  uint32_t lds_offset;
+  int bytes;
+};
 
 struct Fiber {
   ucontext_t ctx;
+  void* sp;      // saved stack pointer (fast switch)
   State state;
-  uint64_t bits;
-  int mask;
+  Resolver resolver;
+  void* payload;
+  std::vector<Transfer> pending;   // issued, not yet landed, oldest first
 };
+
+bool dma_early = false;
+size_t lds_in_use = 0;
 
 Fiber fibers[MAX_THREADS];
 unsigned char* stacks = nullptr;
 ucontext_t scheduler;
+void* scheduler_sp = nullptr;
 int current = -1;
 const std::function<void()>* kernel_body = nullptr;
 dim3 cur_block_dim;
@@ -47,33 +100,56 @@ dim3 cur_block_dim;
   std::abort();
 }
 
+void yield() {
+#if HOSTSIM_FAST_SWITCH
+  hostsim_switch(&fibers[current].sp, scheduler_sp);
+#else
+  swapcontext(&fibers[current].ctx, &scheduler);
+#endif
+}
+
 void fiber_main() {
   (*kernel_body)();
   fibers[current].state = DONE;
-  swapcontext(&fibers[current].ctx, &scheduler);
+  yield();
   die("resumed a finished fiber");
 }
-
-void yield() { swapcontext(&fibers[current].ctx, &scheduler); }
 
 void resume(int t) {
   current = t;
   threadIdx.x = t % cur_block_dim.x;
   threadIdx.y = (t / cur_block_dim.x) % cur_block_dim.y;
   threadIdx.z = t / (cur_block_dim.x * cur_block_dim.y);
+#if HOSTSIM_FAST_SWITCH
+  hostsim_switch(&scheduler_sp, fibers[t].sp);
+#else
   swapcontext(&scheduler, &fibers[t].ctx);
+#endif
 }
 
 void run_block(int nthreads) {
   for (int t = 0; t < nthreads; ++t) {
     Fiber& f = fibers[t];
+#if HOSTSIM_FAST_SWITCH
+    // initial frame: six callee-saved registers, then the address `ret` jumps to; fiber_main must find the stack as
+    // after a call (16-byte aligned before the return address was pushed)
+    void** top = reinterpret_cast<void**>(stacks + static_cast<size_t>(t + 1) * STACK_BYTES);
+    top -= 2;                                            // keeps (top of frame + 8) 16-byte aligned
+    *--top = nullptr;                                    // slot a caller's return address would occupy
+    *--top = reinterpret_cast<void*>(&fiber_main);
+    for (int r = 0; r < 6; ++r) *--top = nullptr;
+    f.sp = top;
+#else
     getcontext(&f.ctx);
     f.ctx.uc_stack.ss_sp = stacks + static_cast<size_t>(t) * STACK_BYTES;
     f.ctx.uc_stack.ss_size = STACK_BYTES;
     f.ctx.uc_link = nullptr;
     makecontext(&f.ctx, fiber_main, 0);
+#endif
     f.state = RUNNABLE;
+    f.pending.clear();
   }
+  std::memset(dynamic_lds, 0xff, lds_in_use);
   const int waves = (nthreads + WAVE - 1) / WAVE;
   for (;;) {
     for (int w = 0; w < waves; ++w) {
@@ -81,26 +157,18 @@ void run_block(int nthreads) {
       for (;;) {
         for (int t = lo; t < hi; ++t)
           if (fibers[t].state == RUNNABLE) resume(t);
-        int at_shuffle = 0, live = 0;
-        for (int t = lo; t < hi; ++t) {
-          live += fibers[t].state != DONE;
-          at_shuffle += fibers[t].state == AT_SHUFFLE;
-        }
-        if (at_shuffle == 0) break;             // wavefront finished or waits at the block barrier
+        int arrived = 0;
+        for (int t = lo; t < hi; ++t) arrived += fibers[t].state == AT_COLLECTIVE;
+        if (arrived == 0) break;                // wavefront finished or waits at the block barrier
         current = lo;
-        if (at_shuffle != hi - lo) die("wavefront shuffle reached by only some of the lanes");
-        uint64_t in[WAVE];
-        const int mask = fibers[lo].mask;
+        if (arrived != hi - lo) die("wavefront-wide operation reached by only some of the lanes");
+        void* payloads[WAVE];
         for (int t = lo; t < hi; ++t) {
-          if (fibers[t].mask != mask) die("lanes of one wavefront shuffle with different masks");
-          in[t - lo] = fibers[t].bits;
+          if (fibers[t].resolver != fibers[lo].resolver) die("lanes of one wavefront are at different wavefront-wide operations");
+          payloads[t - lo] = fibers[t].payload;
         }
-        for (int t = lo; t < hi; ++t) {
-          const int src = (t - lo) ^ mask;
-          fibers[t].bits = src < hi - lo ? in[src] : in[t - lo];
-          fibers[t].state = RUNNABLE;
-        }
-        (void)live;
+        fibers[lo].resolver(payloads, hi - lo);
+        for (int t = lo; t < hi; ++t) fibers[t].state = RUNNABLE;
       }
     }
     int done = 0, waiting = 0;
@@ -118,13 +186,58 @@ void run_block(int nthreads) {
 }
 }  // namespace
 
-uint64_t shfl_xor_bits(uint64_t bits, int mask) {
+void wave_collective(Resolver resolver, void* payload) {
   Fiber& f = fibers[current];
-  f.bits = bits;
-  f.mask = mask;
-  f.state = AT_SHUFFLE;
+  f.resolver = resolver;
+  f.payload = payload;
+  f.state = AT_COLLECTIVE;
   yield();
-  return fibers[current].bits;
+}
+
+void fail(const char* what) { die(what); }
+
+unsigned lane_id() { return static_cast<unsigned>(current) & (WAVE - 1); }
+
+namespace {
+struct Shuffle { uint64_t bits; int mask; };
+void resolve_shuffle(void** payloads, int lanes) {
+  uint64_t in[WAVE];
+  const int mask = static_cast<Shuffle*>(payloads[0])->mask;
+  for (int l = 0; l < lanes; ++l) {
+    if (static_cast<Shuffle*>(payloads[l])->mask != mask) die("lanes of one wavefront shuffle with different masks");
+    in[l] = static_cast<Shuffle*>(payloads[l])->bits;
+  }
+  for (int l = 0; l < lanes; ++l) static_cast<Shuffle*>(payloads[l])->bits = (l ^ mask) < lanes ? in[l ^ mask] : in[l];
+}
+
+void land(const Transfer& t) {
+  if (static_cast<size_t>(t.lds_offset) + t.bytes > lds_in_use) die("global -> LDS transfer outside the block's LDS allocation");
+  std::memcpy(dynamic_lds + t.lds_offset, t.src, t.bytes);
+}
+}  // namespace
+
+uint64_t shfl_xor_bits(uint64_t bits, int mask) {
+  Shuffle s{bits, mask};
+  wave_collective(resolve_shuffle, &s);
+  return s.bits;
+}
+
+void dma_issue(const void* src, uint32_t lds_offset, int bytes) {
+  const Transfer t{src, lds_offset, bytes};
+  if (dma_early) land(t);
+  else fibers[current].pending.push_back(t);
+}
+
+void dma_wait(int may_stay_outstanding) {
+  std::vector<Transfer>& q = fibers[current].pending;
+  const int n = static_cast<int>(q.size()) - may_stay_outstanding;
+  if (n <= 0) return;
+  for (int i = 0; i < n; ++i) land(q[i]);
+  q.erase(q.begin(), q.begin() + n);
+}
+
+uint32_t lds_offset_of(uint32_t low_address_bits) {
+  return low_address_bits - static_cast<uint32_t>(reinterpret_cast<uintptr_t>(dynamic_lds));
 }
 
 void sync_block() {
@@ -149,6 +262,9 @@ void launch(dim3 grid, dim3 block, size_t dynamic_lds_bytes, const std::function
     stacks = static_cast<unsigned char*>(p);
     dynamic_lds = stacks + MAX_THREADS * STACK_BYTES;
   }
+  const char* mode = std::getenv("HOSTSIM_DMA");
+  dma_early = mode != nullptr && std::strcmp(mode, "early") == 0;
+  lds_in_use = dynamic_lds_bytes;
   kernel_body = &body;
   cur_block_dim = block;
   blockDim = block;

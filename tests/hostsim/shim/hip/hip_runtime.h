@@ -8,6 +8,8 @@
 #include <cstring>
 #include <functional>
 
+#include "hip_fp16.h"
+
 #define __global__
 #define __device__
 #define __host__
@@ -35,13 +37,24 @@ typedef void* hipStream_t;
 typedef int hipError_t;
 enum { hipSuccess = 0 };
 enum hipDeviceAttribute_t { hipDeviceAttributeMultiprocessorCount = 1 };
+enum hipFuncAttribute { hipFuncAttributeMaxDynamicSharedMemorySize = 8 };
 
 namespace hostsim {
 struct Index { unsigned x, y, z; };
 // block-by-block, lane-by-lane execution of `body` (the kernel call with its arguments bound)
 void launch(dim3 grid, dim3 block, size_t dynamic_lds_bytes, const std::function<void()>& body);
+// Wavefront-wide operation: every lane of the wavefront calls this with the same resolver; once all have arrived the
+// resolver runs once over the lanes' payloads (payloads[l] belongs to lane l), then every lane continues.
+typedef void (*Resolver)(void** payloads, int lanes);
+void wave_collective(Resolver resolver, void* payload);
+[[noreturn]] void fail(const char* what);
+unsigned lane_id();
 uint64_t shfl_xor_bits(uint64_t bits, int mask);
 void sync_block();
+// direct global -> LDS transfers (asynchronous; see hostsim.cpp for the two timing models)
+void dma_issue(const void* src, uint32_t lds_offset, int bytes);
+void dma_wait(int may_stay_outstanding);
+uint32_t lds_offset_of(uint32_t low_address_bits);   // LDS byte offset from the low 32 bits of a pointer into LDS
 int compute_units();     // HOSTSIM_CUS (default 4): small, so that grid-stride loops take several trips
 extern unsigned char* dynamic_lds;   // at least dynamic_lds_bytes of the current launch
 }  // namespace hostsim
@@ -53,6 +66,8 @@ static inline hipError_t hipGetLastError() { return hipSuccess; }
 static inline const char* hipGetErrorString(hipError_t) { return "host simulation"; }
 static inline hipError_t hipGetDevice(int* dev) { *dev = 0; return hipSuccess; }
 static inline hipError_t hipDeviceGetAttribute(int* v, hipDeviceAttribute_t, int) { *v = hostsim::compute_units(); return hipSuccess; }
+
+static inline hipError_t hipFuncSetAttribute(const void*, hipFuncAttribute, int) { return hipSuccess; }
 
 #define hipLaunchKernelGGL(kernel, grid, block, lds, stream, ...) \
   ::hostsim::launch((grid), (block), (lds), [=]() { kernel(__VA_ARGS__); })
@@ -77,3 +92,113 @@ static inline float rsqrtf(float v) { return 1.0f / std::sqrt(v); }
 static inline float __builtin_amdgcn_exp2f(float v) { return std::exp2(v); }
 static inline float __builtin_amdgcn_rcpf(float v) { return 1.0f / v; }
 static inline void __builtin_amdgcn_sched_barrier(int) {}
+
+// ---------------------------------------------------------------------------------------------------------------
+// gfx950 instructions the GEMM kernels use, by their compiler-builtin names (unknown to an x86 compiler, so free).
+// ---------------------------------------------------------------------------------------------------------------
+static inline uint32_t __builtin_amdgcn_readfirstlane(uint32_t v) { return v; }   // only used on wavefront-uniform values
+static inline int __builtin_amdgcn_readfirstlane(int v) { return v; }
+
+// v_perm_b32: byte i of the result is byte sel[i] of the eight bytes {src1 (0..3), src0 (4..7)}; 0x0c selects 0x00
+static inline uint32_t __builtin_amdgcn_perm(uint32_t src0, uint32_t src1, uint32_t sel) {
+  const uint64_t both = (static_cast<uint64_t>(src0) << 32) | src1;
+  uint32_t out = 0;
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t s = (sel >> (8 * i)) & 0xffu;
+    uint32_t byte;
+    if (s < 8) byte = static_cast<uint32_t>(both >> (8 * s)) & 0xffu;
+    else if (s == 0x0c) byte = 0;
+    else hostsim::fail("v_perm_b32 selector outside the forms this stand-in implements");
+    out |= byte << (8 * i);
+  }
+  return out;
+}
+
+// s_waitcnt: only the vmcnt field matters here (bits 3:0 and 15:14 of the gfx9 encoding)
+static inline void __builtin_amdgcn_s_waitcnt(int imm) { hostsim::dma_wait((imm & 15) | (((imm >> 14) & 3) << 4)); }
+
+// global_load_lds_dwordx4 through the compiler builtin: lane l moves `bytes` from its own global address to LDS address
+// (wavefront-uniform base) + l * bytes
+static inline void __builtin_amdgcn_global_load_lds(const __attribute__((address_space(1))) void* src,
+                                                    __attribute__((address_space(3))) void* lds_base, int bytes, int offset, int) {
+  const uint32_t low = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds_base)) + static_cast<uint32_t>(offset);
+  hostsim::dma_issue(reinterpret_cast<const void*>(reinterpret_cast<uintptr_t>(src)), hostsim::lds_offset_of(low) + hostsim::lane_id() * bytes, bytes);
+}
+
+// ds_read_b64_tr_b16: within a group of 16 lanes, lane i receives element (i & 3) of the four 16-bit elements that
+// lane 4 e + (i >> 2) addressed, for e = 0..3
+typedef short hostsim_short4 __attribute__((ext_vector_type(4)));
+namespace hostsim {
+struct TrRead { const unsigned char* addr; short out[4]; };
+static inline void resolve_tr_read(void** payloads, int lanes) {
+  if (lanes != 64) fail("LDS transpose read in a partial wavefront");
+  short raw[64][4];
+  for (int l = 0; l < 64; ++l) std::memcpy(raw[l], static_cast<TrRead*>(payloads[l])->addr, 8);
+  for (int l = 0; l < 64; ++l) {
+    const int blk = l & ~15, i = l & 15;
+    for (int e = 0; e < 4; ++e) static_cast<TrRead*>(payloads[l])->out[e] = raw[blk + 4 * e + (i >> 2)][i & 3];
+  }
+}
+}  // namespace hostsim
+static inline hostsim_short4 __builtin_amdgcn_ds_read_tr16_b64_v4i16(__attribute__((address_space(3))) hostsim_short4* p) {
+  hostsim::TrRead r;
+  r.addr = reinterpret_cast<const unsigned char*>(reinterpret_cast<uintptr_t>(p));
+  hostsim::wave_collective(hostsim::resolve_tr_read, &r);
+  return hostsim_short4{r.out[0], r.out[1], r.out[2], r.out[3]};
+}
+
+// v_mfma_f32_32x32x16_{f16,bf16}: D[i][j] = C[i][j] + sum_k A[i][k] B[k][j], 32 x 32 x 16. Lane l holds
+// A[l & 31][8 (l >> 5) + t] and B[8 (l >> 5) + t][l & 31] for t = 0..7, and D[8 (r / 4) + 4 (l >> 5) + r % 4][l & 31]
+// in accumulator register r = 0..15.
+typedef float hostsim_float16 __attribute__((ext_vector_type(16)));
+namespace hostsim {
+struct Mfma { const uint16_t* a; const uint16_t* b; float* c; };
+template <bool BF16>
+static inline float widen(uint16_t bits) {
+  if (BF16) { const uint32_t u = static_cast<uint32_t>(bits) << 16; float f; std::memcpy(&f, &u, 4); return f; }
+  return __half2float(__ushort_as_half(bits));
+}
+template <bool BF16>
+static inline void resolve_mfma(void** payloads, int lanes) {
+  if (lanes != 64) fail("MFMA in a partial wavefront");
+  float A[32][16], B[16][32];
+  for (int l = 0; l < 64; ++l) {
+    const Mfma* m = static_cast<const Mfma*>(payloads[l]);
+    for (int t = 0; t < 8; ++t) {
+      A[l & 31][8 * (l >> 5) + t] = widen<BF16>(m->a[t]);
+      B[8 * (l >> 5) + t][l & 31] = widen<BF16>(m->b[t]);
+    }
+  }
+  for (int l = 0; l < 64; ++l) {
+    float* c = static_cast<Mfma*>(payloads[l])->c;
+    const int j = l & 31;
+    for (int r = 0; r < 16; ++r) {
+      const int i = 8 * (r / 4) + 4 * (l >> 5) + r % 4;
+      float s = c[r];
+      for (int k = 0; k < 16; ++k) s += A[i][k] * B[k][j];
+      c[r] = s;
+    }
+  }
+}
+template <bool BF16, typename V>
+static inline hostsim_float16 mfma(V a, V b, hostsim_float16 c) {
+  uint16_t av[8], bv[8];
+  float cv[16];
+  std::memcpy(av, &a, 16);
+  std::memcpy(bv, &b, 16);
+  std::memcpy(cv, &c, 64);
+  Mfma m{av, bv, cv};
+  wave_collective(resolve_mfma<BF16>, &m);
+  hostsim_float16 d;
+  std::memcpy(&d, cv, 64);
+  return d;
+}
+}  // namespace hostsim
+typedef _Float16 hostsim_half8 __attribute__((ext_vector_type(8)));
+typedef __bf16 hostsim_bf16x8 __attribute__((ext_vector_type(8)));
+static inline hostsim_float16 __builtin_amdgcn_mfma_f32_32x32x16_f16(hostsim_half8 a, hostsim_half8 b, hostsim_float16 c, int, int, int) {
+  return hostsim::mfma<false>(a, b, c);
+}
+static inline hostsim_float16 __builtin_amdgcn_mfma_f32_32x32x16_bf16(hostsim_bf16x8 a, hostsim_bf16x8 b, hostsim_float16 c, int, int, int) {
+  return hostsim::mfma<true>(a, b, c);
+}

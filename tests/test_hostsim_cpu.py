@@ -1,19 +1,19 @@
-"""The elementwise kernels' own source, executed on the CPU.
+"""The kernels' own source, executed on the CPU.
 
-tests/hostsim compiles layer_norm.hip, softmax_dropout.hip, dropout_add.hip and xentropy.hip (with the library's
-plumbing in api.hip) as plain C++ against a small stand-in for the HIP headers and runs every kernel lane by lane:
-one fiber per thread, 64-lane wavefronts that meet at shuffles, block barriers, blocks one after the other. The
-resulting library exports the same extern "C" entry points as libnmtg_hip.so, so the checks below are the GPU
-tests' own functions (tests/test_layer_norm_gpu.py, tests/test_elementwise_gpu.py) called with host tensors, at
-sizes a CPU finishes in seconds. The compute-unit count the launch code sees is set small, so grid-stride loops make
-several trips and partial last groups occur.
+tests/hostsim compiles the library's .hip sources as plain C++ against a small stand-in for the HIP headers and runs
+every kernel lane by lane: one fiber per thread, 64-lane wavefronts that meet at shuffles, MFMA instructions and LDS
+transpose reads, block barriers, blocks one after the other; the asynchronous global -> LDS transfers of the GEMM
+loops land either as late or as early as the kernel's own waits allow (HOSTSIM_DMA). The resulting library exports
+the same extern "C" entry points as libnmtg_hip.so, so the checks below are the GPU tests' own functions
+(tests/test_*_gpu.py) called with host tensors, at sizes a CPU finishes in seconds.
 
-What this covers: indexing, masking, clamping, reduction trees, launch arithmetic, the C entry points' argument
-checks. What it cannot cover: memory ordering, occupancy, anything about timing, and the GEMM / attention / MLP
-kernels (MFMA, LDS transfers), which only run on the GPU.
+What this covers: indexing, masking, clamping, LDS layouts and fragment reads, reduction trees, launch arithmetic,
+tile selection, workspace use, the waits that order LDS transfers against their reads, the C entry points' argument
+checks, and (in the sanitizer run at the end) that no kernel touches memory outside the tensors it was handed.
+What it cannot cover: real memory ordering and caches, occupancy, register pressure, anything about speed. A GPU
+run of the same tests remains the proof; this run keeps mistakes of the first kind from ever reaching the GPU.
 """
 import ctypes
-import itertools
 import os
 import subprocess
 import sys
@@ -21,58 +21,58 @@ import sys
 import pytest
 import torch
 
-from nmtgminor_amd import _lib, _rng
+from nmtgminor_amd import _rng
 
 sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "hostsim"))
-import build as hostsim_build  # noqa: E402
+import harness  # noqa: E402
+from harness import hostsim_build  # noqa: E402
 
+import test_attention_gpu as tat  # noqa: E402
 import test_elementwise_gpu as tel  # noqa: E402
+import test_gemm_gpu as tg  # noqa: E402
 import test_layer_norm_gpu as tln  # noqa: E402
+import test_mlp_gpu as tm  # noqa: E402
+import test_staged_gpu as tst  # noqa: E402
+import test_zz_golden_gpu as tgold  # noqa: E402
 
 pytestmark = pytest.mark.skipif(not hostsim_build.available(), reason="no host C++ compiler with __bf16 (ROCm clang++)")
 CPU = torch.device("cpu")
 F32, F16, BF16 = torch.float32, torch.float16, torch.bfloat16
+SANITIZER_RUN = os.environ.get("HOSTSIM_SANITIZE") == "1"
+# the sanitizer build is several times slower: it repeats every check except the ones marked long
+long_case = pytest.mark.skipif(SANITIZER_RUN, reason="left out of the sanitizer run for time")
 
 
 @pytest.fixture(scope="session")
 def hostsim_lib():
-    lib = ctypes.CDLL(hostsim_build.ensure())
-    lib.nmtg_last_error.restype = ctypes.c_char_p
-    lib.nmtg_version.restype = ctypes.c_int
-    lib.nmtg_ln_bwd_parts.restype = ctypes.c_int64
-    return lib
+    return harness.library()
 
 
 @pytest.fixture(autouse=True)
 def on_the_cpu(hostsim_lib, monkeypatch):
-    counter = itertools.count()
-    monkeypatch.setattr(_lib, "_lib", hostsim_lib)                    # what _lib.load() hands out
-    monkeypatch.setattr(_lib, "require_cuda", lambda *t: None)
-    monkeypatch.setattr(_lib, "stream_of", lambda t: ctypes.c_void_p(0))
+    harness.install(monkeypatch.setattr)
+    # elementwise kernels: few compute units, so that grid-stride loops make several trips and last groups are partial
     monkeypatch.setenv("HOSTSIM_CUS", "2")
-
-    # `t.to(device)` hands back a copy on the GPU box; on the CPU it would alias `t`, and the in-place operators
-    # would then change the inputs the oracle is given afterwards
-    plain_to = torch.Tensor.to
-
-    def copying_to(self, *a, **k):
-        out = plain_to(self, *a, **k)
-        if a and isinstance(a[0], torch.device) and out.data_ptr() == self.data_ptr() and out.numel() > 0:
-            out = out.clone()
-        return out
-    monkeypatch.setattr(torch.Tensor, "to", copying_to)
-
-    def seed_offset(dev, n):                                          # one Philox stream, advancing like the GPU one
-        return 1234, 4 * next(counter)
-    for name, mod in list(sys.modules.items()):
-        if name.startswith("nmtgminor_amd") and hasattr(mod, "philox_seed_offset"):
-            monkeypatch.setattr(mod, "philox_seed_offset", seed_offset)
+    monkeypatch.delenv("HOSTSIM_DMA", raising=False)
 
 
-def test_only_the_simulated_operators_are_exported(hostsim_lib):
+@pytest.fixture
+def mi355x(monkeypatch):
+    """GEMM-based operators: the tile and split-K choices depend on the compute-unit count, so show them the real one."""
+    monkeypatch.setenv("HOSTSIM_CUS", "256")
+
+
+@pytest.fixture(params=["late", "early"])
+def dma(request, monkeypatch):
+    monkeypatch.setenv("HOSTSIM_DMA", request.param)
+    return request.param
+
+
+def test_every_entry_point_but_the_event_tracing_is_exported(hostsim_lib):
+    from nmtgminor_amd import _lib
     assert hostsim_lib.nmtg_version() == 100
-    with pytest.raises(AttributeError):
-        hostsim_lib.nmtg_gemm
+    missing = [n for n in _lib.header_functions() if not hasattr(hostsim_lib, n)]
+    assert missing == ["nmtg_trace_begin", "nmtg_trace_end"]          # HIP events: nothing to simulate
 
 
 # ----------------------------------------------------------------------------- LayerNorm
@@ -225,6 +225,125 @@ def test_split_k_reduction(hostsim_lib, dtype, tile, m, n, batch, splits, c_vec)
         want[bz[ok], row[ok], col[ok] + e] = summed[ok, e]
     assert torch.equal(c.double(), want.to(dtype).double())
     assert (want[:, :, :n] != 777.0).all()                      # every element of C has exactly one slot
+
+
+# ----------------------------------------------------------------------------- GEMM core
+@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 64), (128, 128, 128), (300, 200, 72), (1, 8, 8), (257, 129, 1000), (64, 1504, 64),
+                                   pytest.param(512, 2048, 512, marks=long_case), pytest.param(1024, 64, 512, marks=long_case)])
+@pytest.mark.parametrize("layout", ["nt", "nn", "tn"])
+def test_gemm_layouts(mi355x, dtype, m, n, k, layout):
+    tg.test_gemm_layouts(CPU, dtype, m, n, k, layout)
+
+
+@pytest.mark.parametrize("layout", ["nt", "nn", "tn"])
+@pytest.mark.parametrize("m,n,k", [(300, 520, 448), (700, 130, 256)])
+def test_gemm_ring_under_both_transfer_timings(mi355x, dma, layout, m, n, k):
+    # K of several 64-steps: the ring wraps around, slots are refilled while later wavefronts still read
+    tg.test_gemm_layouts(CPU, BF16, m, n, k, layout)
+
+
+@long_case
+@pytest.mark.parametrize("dtype", [F16, BF16])
+def test_gemm_unaligned_extents(mi355x, dtype):
+    tg.test_gemm_unaligned_extents(CPU, dtype)
+
+
+def test_gemm_bias_and_batched_strided_views(mi355x):
+    tg.test_gemm_bias_and_batched_strided_views(CPU)
+
+
+@long_case
+def test_gemm_split_k(mi355x, hostsim_lib):
+    # reduction-heavy dW-shaped product: the call splits K and reduces the partials in a fixed order
+    m, n, k = 256, 128, 4096
+    assert hostsim_lib.nmtg_gemm_workspace_bytes(ctypes.c_int64(m), ctypes.c_int64(n), ctypes.c_int64(k), ctypes.c_int64(1)) > 0
+    a, b = tg._mk((k, m), CPU, F16, 11), tg._mk((k, n), CPU, F16, 12)
+    c1, c2 = tg.gemm(a, b, True, False), tg.gemm(a, b, True, False)
+    assert torch.equal(c1, c2)
+    tg.assert_close(c1, tg._ref(a, b, True, False), F16, "split-k", scale_atol=True)
+    tg.assert_close(tg.gemm(a, b, True, False, split_k=False), tg._ref(a, b, True, False), F16, "no split", scale_atol=True)
+
+
+# ----------------------------------------------------------------------------- fused MLP
+@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("act", ["gelu", "relu", "silu", "agelu"])
+@pytest.mark.parametrize("tokens,dm,di,p", [(72, 96, 200, 0.5), pytest.param(256, 128, 256, 0.0, marks=long_case)])
+def test_mlp_autograd_function(mi355x, dtype, act, tokens, dm, di, p):
+    tm.test_mlp_autograd_function(CPU, dtype, act, tokens, dm, di, p)
+
+
+@long_case
+def test_mlp_recompute_input_only_three_layers_rng(mi355x):
+    tm.test_mlp_recompute_and_input_only(CPU)
+    tm.test_mlp_three_layers_and_rng_mask(CPU)
+
+
+# ----------------------------------------------------------------------------- attention
+@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("t,b,e,h,p", [pytest.param(64, 4, 256, 4, 0.0, marks=long_case), (33, 2, 128, 2, 0.1),
+                                       pytest.param(200, 2, 256, 4, 0.25, marks=long_case)])
+def test_self_attention_key_padding(mi355x, dtype, t, b, e, h, p):
+    tat.test_self_attention_key_padding(CPU, dtype, t, b, e, h, p)
+
+
+def test_self_attention_contract_rng_eval_no_bias(mi355x):
+    tat.test_self_attention_intermediates_and_native_contract(CPU)
+    tat.test_self_attention_rng_dropout_eval_and_no_bias(CPU)
+
+
+@long_case
+def test_self_attention_causal_and_recompute(mi355x):
+    tat.test_self_attention_causal_and_recompute(CPU, BF16)
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("tq,tk,b,e,h,p", [(17, 100, 3, 128, 2, 0.2), pytest.param(32, 1500, 2, 256, 4, 0.1, marks=long_case)])
+def test_encdec_attention(mi355x, dtype, tq, tk, b, e, h, p):
+    tat.test_encdec_attention(CPU, dtype, tq, tk, b, e, h, p)
+
+
+@long_case
+def test_encdec_attention_without_biases_compact_and_modules(mi355x):
+    tat.test_encdec_attention_without_biases_and_compact(CPU)
+    tat.test_modules_state_dict_names_and_forward(CPU)
+    tat.test_feed_forward_module(CPU)
+
+
+# ----------------------------------------------------------------------------- variants that are switched off by default
+@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("batch,m,n,k", [(3, 300, 64, 192), (2, 256, 64, 64), (5, 77, 64, 128)])
+def test_ring_loop_of_the_256x64_tile(mi355x, dma, dtype, batch, m, n, k):
+    tst.test_ring_256x64_matches_two_buffer_loop(CPU, dtype, batch, m, n, k)
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("t,b,e,h,p,causal", [pytest.param(200, 2, 256, 4, 0.25, False, marks=long_case), (96, 2, 128, 2, 0.1, True),
+                                              (40, 2, 128, 2, 0.1, False), pytest.param(512, 2, 256, 4, 0.1, False, marks=long_case)])
+def test_fused_scores_softmax(mi355x, dtype, t, b, e, h, p, causal):
+    tst.test_fused_scores_softmax_matches_two_kernel_path(CPU, dtype, t, b, e, h, p, causal)
+
+
+def test_fused_scores_softmax_draws_the_same_dropout_mask(mi355x):
+    tst.test_fused_scores_softmax_rng_mask_is_the_same_stream(CPU)
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("t,b,e,h,p,causal", [(96, 2, 128, 2, 0.0, True), (40, 2, 128, 2, 0.1, False),
+                                              pytest.param(200, 2, 256, 4, 0.25, False, marks=long_case)])
+def test_fused_softmax_backward(mi355x, dtype, t, b, e, h, p, causal):
+    tst.test_fused_softmax_backward_matches_two_kernel_path(CPU, dtype, t, b, e, h, p, causal)
+
+
+# ----------------------------------------------------------------------------- committed fixtures
+@pytest.mark.parametrize("name", [n for n in dir(tgold) if n.startswith("test_") and n != "test_mlp_fixture"])
+def test_golden_fixtures(mi355x, name):
+    getattr(tgold, name)(CPU)
+
+
+@pytest.mark.parametrize("act", ["gelu", "relu", "silu", "agelu"])
+def test_golden_mlp_fixture(mi355x, act):
+    tgold.test_mlp_fixture(CPU, act)
 
 
 # ----------------------------------------------------------------------------- the same checks, bounds-checked
