@@ -16,7 +16,7 @@ import torch
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, HERE)
-import build as hostsim_build  # noqa: E402
+import hostsim_build  # noqa: E402
 
 from nmtgminor_amd import _lib  # noqa: E402
 

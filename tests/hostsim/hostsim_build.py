@@ -7,7 +7,7 @@ The kernel sources are used as they are, apart from three textual substitutions 
     "+v" asm register constraint  ->  "+r"              (an empty asm statement that only pins a value)
 and the path of the public header. The result exports the same extern "C" entry points as libnmtg_hip.so for those
 operators, plus hostsim_* hooks (stubs.cpp) for the reductions that have no entry point of their own, and takes host
-pointers. Test infrastructure: python tests/hostsim/build.py
+pointers. Test infrastructure: python tests/hostsim/hostsim_build.py
 """
 import os
 import re
