@@ -319,6 +319,111 @@ class EncdecAttnWL(Workload):
 
 
 
+class SoftmaxDropoutWL(Workload):
+    name = "softmax_dropout"
+    bound = "hbm"
+    dtype = "bf16"
+    description = ("masked softmax + dropout as its own op, fwd + recomputing bwd, bf16 scores [512 x 512 x 512] "
+                   "(32 sentences x 16 heads), key-padding mask, dropout 0.1 (explicit mask)")
+    HEADS, BATCH, T = 16, 32, 512
+
+    def setup(self, dev):
+        from oracle import inputs
+        from nmtgminor_amd.native import mask_softmax_dropout_cuda as sm
+        self.sm = sm
+        g = torch.Generator().manual_seed(1003)
+        self.heads, b, t = self.HEADS, self.BATCH, self.T
+        bh = b * self.heads
+        self.cpu_scores = (torch.randn(bh, t, t, generator=g) * 3).to(torch.bfloat16)
+        self.cpu_pad, _ = inputs.lengths_mask(b, t, t // 2, t, g)
+        self.cpu_dm = inputs.bernoulli_mask((bh, t, t), 0.9, g)
+        self.cpu_go = torch.randn(bh, t, t, generator=g).to(torch.bfloat16)
+        self.s, self.pad, self.dm, self.go = (v.to(dev) for v in (self.cpu_scores, self.cpu_pad, self.cpu_dm, self.cpu_go))
+        self.n = self.s.numel()
+
+    def step(self):
+        _, _, dropped = self.sm.forward(True, self.heads, self.s, 0.1, pad_mask=self.pad, dropout_mask=self.dm,
+                                        want_softmax=False)
+        ds = self.sm.backward_recompute(self.heads, self.go, None, self.s, self.dm, 0.1, pad_mask=self.pad)
+        return dropped, ds
+
+    def _bytes(self):
+        # fwd: scores read, dropped probabilities written, dropout mask read; bwd: gradient and scores read, mask read,
+        # gradient of the scores written (the key-padding mask is 16 KB)
+        return 5 * self.n, 7 * self.n
+
+    def work_per_step(self):
+        return sum(self._bytes())
+
+    def kernel_work(self):
+        fwd, bwd = self._bytes()
+        return {"softmax_dropout_fwd": fwd, "softmax_dropout_bwd": bwd}
+
+    def cpu_baseline(self):
+        from oracle import softmax_dropout as o
+        rows = self.heads                           # the 16 heads of the first sentence, of 512 (sentence, head) slices
+        s, dm, go = self.cpu_scores[:rows], self.cpu_dm[:rows], self.cpu_go[:rows]
+        pad = self.cpu_pad[:1]
+
+        def run():
+            masked = o.masked_scores(s.float(), pad_mask=pad, heads=rows)
+            sm_, _ = o.softmax_dropout_fwd(masked, dm, 0.1)
+            o.softmax_dropout_bwd(go, sm_, dm, 0.1)
+        t = _time_cpu(run, 3)
+        return dict(value=self.work_per_step() * rows / self.s.shape[0] / t / 1e9, unit="GB/s", cores=torch.get_num_threads(),
+                    kind="port", sample="the first sentence (16 of the 512 [512 x 512] slices), fwd+bwd, median of 3")
+
+
+class DropoutAddWL(Workload):
+    name = "dropout_add"
+    bound = "hbm"
+    dtype = "bf16"
+    description = "dropout + residual add fwd+bwd bf16 [512 x 32 x 1024], dropout 0.1 (explicit mask), in place"
+    SHAPE = (512, 32, 1024)
+
+    def setup(self, dev):
+        from oracle import inputs
+        from nmtgminor_amd.native import fused_dropout_add_cuda as da
+        self.da = da
+        g = torch.Generator().manual_seed(1006)
+        shape = self.SHAPE
+        self.cpu_x = torch.randn(shape, generator=g).to(torch.bfloat16)
+        self.cpu_r = torch.randn(shape, generator=g).to(torch.bfloat16)
+        self.cpu_m = inputs.bernoulli_mask(shape, 0.9, g)
+        self.cpu_g = torch.randn(shape, generator=g).to(torch.bfloat16)
+        self.x0, self.r, self.m, self.g = (v.to(dev) for v in (self.cpu_x, self.cpu_r, self.cpu_m, self.cpu_g))
+        self.x = self.x0.clone()
+        self.n = self.x.numel()
+
+    def step(self):
+        # in place, as the reference: x <- dropout(x) + residual. The buffer is reused from step to step; its values
+        # stay finite (a random walk of unit steps over the run) and do not influence the time.
+        mask, out = self.da.forward(True, self.x, self.r, 0.1, self.m)
+        dx = self.da.backward(self.g, mask, 0.1)
+        return out, dx
+
+    def _bytes(self):
+        return 7 * self.n, 5 * self.n     # fwd: x, residual read + x written (2 B each) + mask; bwd: g read, dx written + mask
+
+    def work_per_step(self):
+        return sum(self._bytes())
+
+    def kernel_work(self):
+        fwd, bwd = self._bytes()
+        return {"dropout_add_fwd": fwd, "dropout_add_bwd": bwd}
+
+    def cpu_baseline(self):
+        from oracle import dropout_add as o
+        x, r, m, g = self.cpu_x, self.cpu_r, self.cpu_m, self.cpu_g
+
+        def run():
+            o.dropout_add_fwd(x, r, m, 0.1)
+            o.dropout_add_bwd(g, m, 0.1)
+        t = _time_cpu(run, 3)
+        return dict(value=self.work_per_step() / t / 1e9, unit="GB/s", cores=torch.get_num_threads(), kind="port",
+                    sample="full workload ([512 x 32 x 1024] bf16 fwd+bwd), median of 3")
+
+
 class CopyWL(Workload):
     """Plain device copy of a known size: the calibration target for the rocprofv3 FETCH_SIZE /
     WRITE_SIZE counters (not part of `--workload all`)."""
@@ -340,7 +445,7 @@ class CopyWL(Workload):
         return 2 * self.src.numel() * 4
 
 
-WORKLOADS = {w.name: w for w in (LayerNormWL, MlpWL, SelfAttnWL, EncdecAttnWL, XentropyWL)}
+WORKLOADS = {w.name: w for w in (LayerNormWL, MlpWL, SelfAttnWL, EncdecAttnWL, SoftmaxDropoutWL, DropoutAddWL, XentropyWL)}
 EXTRA_WORKLOADS = {CopyWL.name: CopyWL}
 PRIMARY = "mlp"
 
