@@ -31,6 +31,7 @@ import test_attention_gpu as tat  # noqa: E402
 import test_elementwise_gpu as tel  # noqa: E402
 import test_gemm_gpu as tg  # noqa: E402
 import test_layer_norm_gpu as tln  # noqa: E402
+import test_layers_gpu as tla  # noqa: E402
 import test_mlp_gpu as tm  # noqa: E402
 import test_staged_gpu as tst  # noqa: E402
 import test_zz_golden_gpu as tgold  # noqa: E402
@@ -308,6 +309,29 @@ def test_encdec_attention_without_biases_compact_and_modules(mi355x):
     tat.test_encdec_attention_without_biases_and_compact(CPU)
     tat.test_modules_state_dict_names_and_forward(CPU)
     tat.test_feed_forward_module(CPU)
+
+
+# ----------------------------------------------------------------------------- layer glue
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_pre_post_processing(mi355x, dtype):
+    tla.test_pre_post_processing_sequences(CPU, dtype)
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("macaron,training", [(False, False), (False, True), (True, True)])
+def test_encoder_layer(mi355x, dtype, macaron, training):
+    tla.test_encoder_layer_matches_the_oracle(CPU, dtype, macaron, training)
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("ignore_source", [False, True])
+def test_decoder_layer(mi355x, dtype, ignore_source):
+    tla.test_decoder_layer_matches_the_oracle(CPU, dtype, ignore_source)
+
+
+def test_layers_stochastic_depth_dropout_and_options(mi355x):
+    tla.test_encoder_layer_stochastic_depth(CPU)
+    tla.test_layers_with_dropout_and_unsupported_options(CPU)
 
 
 # ----------------------------------------------------------------------------- variants that are switched off by default

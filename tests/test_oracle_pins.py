@@ -10,7 +10,7 @@ import pytest
 import torch
 import torch.nn.functional as F
 
-from oracle import attention, dropout_add, inputs, layer_norm, mlp, softmax_dropout, xentropy
+from oracle import attention, dropout_add, inputs, layer_norm, mlp, softmax_dropout, transformer_layers, xentropy
 
 D = torch.float64
 
@@ -312,6 +312,88 @@ def test_attention_finite_differences():
         xm[idx] -= eps
         fd = (f(xp) - f(xm)) / (2 * eps)
         assert abs(float(fd) - float(bwd["dx"][idx])) < 1e-6 * max(1.0, abs(float(fd)))
+
+
+def _layer_params_from_torch(layer, heads, decoder):
+    """nn.Transformer{En,De}coderLayer weights under the reference's key names and layouts."""
+    sd = {k: v.detach() for k, v in layer.state_dict().items()}
+    e = sd["norm1.weight"].numel()
+    p = {}
+
+    def ln(dst, src):
+        p[dst + ".layer_norm.function.weight"], p[dst + ".layer_norm.function.bias"] = sd[src + ".weight"], sd[src + ".bias"]
+
+    def self_attn(dst, src):
+        w, b = sd[src + ".in_proj_weight"], sd[src + ".in_proj_bias"]
+        p[dst + ".in_proj_weight"] = attention.interleave_qkv(w[:e], w[e:2 * e], w[2 * e:], heads)
+        p[dst + ".in_proj_bias"] = attention.interleave_qkv(b[:e], b[e:2 * e], b[2 * e:], heads)
+        p[dst + ".out_proj_weight"], p[dst + ".out_proj_bias"] = sd[src + ".out_proj.weight"], sd[src + ".out_proj.bias"]
+
+    ln("preprocess_attn", "norm1")
+    self_attn("multihead_tgt" if decoder else "multihead", "self_attn")
+    if decoder:
+        ln("preprocess_src_attn", "norm2")
+        w, b = sd["multihead_attn.in_proj_weight"], sd["multihead_attn.in_proj_bias"]
+        p["multihead_src.in_proj_weight_q"], p["multihead_src.in_proj_bias_q"] = w[:e], b[:e]
+        p["multihead_src.in_proj_weight_kv"] = attention.interleave_kv(w[e:2 * e], w[2 * e:], heads)
+        p["multihead_src.in_proj_bias_kv"] = attention.interleave_kv(b[e:2 * e], b[2 * e:], heads)
+        p["multihead_src.out_proj_weight"], p["multihead_src.out_proj_bias"] = sd["multihead_attn.out_proj.weight"], sd["multihead_attn.out_proj.bias"]
+    ln("preprocess_ffn", "norm3" if decoder else "norm2")
+    p["feedforward.in_proj_weight"], p["feedforward.in_proj_bias"] = sd["linear1.weight"], sd["linear1.bias"]
+    p["feedforward.out_proj_weight"], p["feedforward.out_proj_bias"] = sd["linear2.weight"], sd["linear2.bias"]
+    return p
+
+
+def test_layer_oracle_matches_torch_modules():
+    # pre-norm residual blocks: the composition is PyTorch's own norm_first Transformer layer
+    t, tk, b, e, h, inner = 9, 11, 3, 16, 4, 40
+    g = torch.Generator().manual_seed(71)
+    x = torch.randn(t, b, e, generator=g, dtype=D)
+    ctxt = torch.randn(tk, b, e, generator=g, dtype=D)
+    pad, _ = inputs.lengths_mask(b, t, 4, t, g)
+    src_pad, _ = inputs.lengths_mask(b, tk, 5, tk, g)
+    causal = torch.triu(torch.ones(t, t), 1).bool()
+    torch.manual_seed(72)
+    enc = torch.nn.TransformerEncoderLayer(e, h, inner, dropout=0.0, activation="gelu", norm_first=True, dtype=D)
+    dec = torch.nn.TransformerDecoderLayer(e, h, inner, dropout=0.0, activation="gelu", norm_first=True, dtype=D)
+    for m in list(enc.modules()) + list(dec.modules()):          # biases and LayerNorm affines away from 0 / 1
+        for name, prm in m.named_parameters(recurse=False):
+            if prm.dim() == 1:
+                prm.data.add_(0.1 * torch.randn(prm.shape, generator=g, dtype=D))
+    want = enc(x, src_key_padding_mask=pad)
+    got = transformer_layers.encoder_layer(x, _layer_params_from_torch(enc, h, False), h, pad, act="gelu")
+    torch.testing.assert_close(got, want.detach(), rtol=1e-10, atol=1e-10)
+    want = dec(x, ctxt, tgt_mask=causal, memory_key_padding_mask=src_pad)
+    got, cov = transformer_layers.decoder_layer(x, ctxt, _layer_params_from_torch(dec, h, True), h, causal, src_pad, act="gelu")
+    torch.testing.assert_close(got, want.detach(), rtol=1e-10, atol=1e-10)
+    assert cov.shape == (b * h, t, tk) and torch.allclose(cov.sum(-1), torch.ones(b * h, t, dtype=D))
+    # the scale factors: macaron halves both feed-forward blocks, a surviving layer is scaled by 1 / (1 - death_rate)
+    p = _layer_params_from_torch(enc, h, False)
+    base = transformer_layers.encoder_layer(x, p, h, pad, act="gelu")
+    scaled = transformer_layers.encoder_layer(x, p, h, pad, act="gelu", death_rate=0.5, training=True)
+    assert not torch.allclose(base, scaled)
+    assert torch.allclose(transformer_layers.encoder_layer(x, p, h, pad, act="gelu", death_rate=0.5, training=False), base)
+    # death_rate = 0.5 doubles each residual branch: check against the hand composition on the first branch only
+    zero_ffn = dict(p)
+    zero_ffn["feedforward.out_proj_weight"] = torch.zeros_like(p["feedforward.out_proj_weight"])
+    zero_ffn["feedforward.out_proj_bias"] = torch.zeros_like(p["feedforward.out_proj_bias"])
+    a1 = transformer_layers.encoder_layer(x, zero_ffn, h, pad, act="gelu") - x
+    a2 = transformer_layers.encoder_layer(x, zero_ffn, h, pad, act="gelu", death_rate=0.5, training=True) - x
+    torch.testing.assert_close(a2, 2 * a1, rtol=1e-10, atol=1e-12)
+    # macaron: with the macaron block a copy of the feed-forward block and the attention silenced,
+    # y = x + 0.5 F(x) followed by + 0.5 F(.) again
+    mac = dict(zero_ffn)
+    for k in list(p):
+        if k.startswith("feedforward."):
+            mac[k] = p[k]
+            mac[k.replace("feedforward.", "mcr_feedforward.")] = p[k]
+        if k.startswith("preprocess_ffn."):
+            mac[k.replace("preprocess_ffn.", "preprocess_mcr_ffn.")] = p[k]
+    mac["multihead.out_proj_weight"] = torch.zeros_like(p["multihead.out_proj_weight"])
+    mac["multihead.out_proj_bias"] = torch.zeros_like(p["multihead.out_proj_bias"])
+    half = lambda z: z + 0.5 * (transformer_layers.encoder_layer(z, dict(mac, **{"multihead.out_proj_weight": mac["multihead.out_proj_weight"]}), h, pad, act="gelu", macaron=False) - z)
+    got = transformer_layers.encoder_layer(x, mac, h, pad, act="gelu", macaron=True)
+    torch.testing.assert_close(got, half(half(x)), rtol=1e-10, atol=1e-12)
 
 
 def test_zipf_targets_and_masks_are_seeded():
