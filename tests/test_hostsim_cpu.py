@@ -31,7 +31,7 @@ import test_attention_gpu as tat  # noqa: E402
 import test_elementwise_gpu as tel  # noqa: E402
 import test_gemm_gpu as tg  # noqa: E402
 import test_layer_norm_gpu as tln  # noqa: E402
-import test_layers_gpu as tla  # noqa: E402
+import test_zy_layers_gpu as tla  # noqa: E402
 import test_mlp_gpu as tm  # noqa: E402
 import test_staged_gpu as tst  # noqa: E402
 import test_zz_golden_gpu as tgold  # noqa: E402

@@ -169,7 +169,7 @@ def test_decoder_layer_matches_the_oracle(dev, dtype, ignore_source):
         assert not any(n.startswith("multihead_src") or n.startswith("preprocess_src_attn") for n in layer.state_dict())
     else:
         layer_close(cin.grad, c64.grad, dtype, "decoder dcontext")
-        assert_close(coverage, cov.detach(), dtype, "coverage")
+        assert_close(coverage, cov.detach(), dtype, "coverage", atol=4e-3)   # probabilities behind three rounded operators
     for name, prm in layer.named_parameters():
         layer_close(prm.grad, p64r[name].grad, dtype, "d " + name)
 
