@@ -67,6 +67,9 @@ static inline const char* hipGetErrorString(hipError_t) { return "host simulatio
 static inline hipError_t hipGetDevice(int* dev) { *dev = 0; return hipSuccess; }
 static inline hipError_t hipDeviceGetAttribute(int* v, hipDeviceAttribute_t, int) { *v = hostsim::compute_units(); return hipSuccess; }
 
+#define HIP_SYMBOL(x) x
+template <typename T>
+static inline hipError_t hipGetSymbolAddress(void** p, const T& symbol) { *p = const_cast<void*>(static_cast<const void*>(&symbol)); return hipSuccess; }
 static inline hipError_t hipFuncSetAttribute(const void*, hipFuncAttribute, int) { return hipSuccess; }
 
 #define hipLaunchKernelGGL(kernel, grid, block, lds, stream, ...) \
