@@ -71,6 +71,7 @@ struct GemmArgs {
   int rng;                  // ACT_FWD: draw the keep mask from Philox and store it to dmask
   uint64_t seed, offset;
   int act;
+  int act_lut;              // gelu / gelu' through the LDS table (ring kernels only; set by the host on request)
   float* colsum_part;
   const uint8_t* kmask;
   int kmask_kind, heads;
@@ -135,10 +136,40 @@ __device__ __forceinline__ NormalCdfPdf normal_cdf_pdf(float h) {
   return r;
 }
 
+// gelu through a table. The activation epilogues are VALU-bound (about 30 instruction slots per element, two of
+// them quarter-rate transcendentals), so Phi(h) and gelu'(h) can instead be read from a 513-entry table over
+// [-6, 6] that the block builds in LDS with the exact formula: one fused multiply-add for the table coordinate, a
+// clamp, a fraction, one 8-byte LDS read of (value, difference to the next entry) and one fused multiply-add.
+// Linear interpolation error: step^2 / 8 * max|f''| = 1.7e-5 for Phi, 4e-5 for gelu' (the 16-bit tolerances are
+// 1e-3). Outside [-6, 6] the end values (1e-9 / 1 - 1e-9) are used.
+constexpr int NMTG_ACT_GELU_LUT = 100;      // internal activation code: gelu evaluated through the table
+constexpr int ACT_LUT_N = 512;
+constexpr float ACT_LUT_R = 6.f;
+constexpr int ACT_LUT_BYTES = (ACT_LUT_N + 1) * 8;
+
+template <bool GRAD>
+__device__ __forceinline__ void act_lut_fill(float2* tab, int tid, int nthreads) {
+  constexpr float STEP = 2.f * ACT_LUT_R / ACT_LUT_N;
+  for (int t = tid; t <= ACT_LUT_N; t += nthreads) {
+    const float x0 = -ACT_LUT_R + STEP * static_cast<float>(t);
+    const NormalCdfPdf a = normal_cdf_pdf(x0), b = normal_cdf_pdf(x0 + STEP);
+    const float f0 = GRAD ? fmaf(x0, a.pdf, a.cdf) : a.cdf;
+    const float f1 = GRAD ? fmaf(x0 + STEP, b.pdf, b.cdf) : b.cdf;
+    tab[t] = make_float2(f0, f1 - f0);
+  }
+}
+__device__ __forceinline__ float act_lut_eval(const float2* tab, float h) {
+  float u = fmaf(h, ACT_LUT_N / (2.f * ACT_LUT_R), 0.5f * ACT_LUT_N);
+  u = __builtin_amdgcn_fmed3f(u, 0.f, static_cast<float>(ACT_LUT_N));
+  const float2 e = tab[static_cast<int>(u)];
+  return fmaf(__builtin_amdgcn_fractf(u), e.y, e.x);
+}
+
 template <int ACT>
-__device__ __forceinline__ float act_apply(float h) {
+__device__ __forceinline__ float act_apply(float h, const float2* tab) {
   if constexpr (ACT == NMTG_ACT_RELU) return fmaxf(h, 0.f);
   else if constexpr (ACT == NMTG_ACT_GELU) return h * normal_cdf_pdf(h).cdf;
+  else if constexpr (ACT == NMTG_ACT_GELU_LUT) return h * act_lut_eval(tab, h);
   else if constexpr (ACT == NMTG_ACT_SILU) return h * fast_rcp(1.f + fast_exp2(h * -1.4426950408889634f));
   else if constexpr (ACT == NMTG_ACT_AGELU) {
     // 0.5 h (1 + tanh u) = h * sigmoid(2u)
@@ -147,11 +178,13 @@ __device__ __forceinline__ float act_apply(float h) {
   } else return h;
 }
 template <int ACT>
-__device__ __forceinline__ float act_grad(float h) {
+__device__ __forceinline__ float act_grad(float h, const float2* tab) {
   if constexpr (ACT == NMTG_ACT_RELU) return h > 0.f ? 1.f : 0.f;
   else if constexpr (ACT == NMTG_ACT_GELU) {
     const NormalCdfPdf n = normal_cdf_pdf(h);
     return fmaf(h, n.pdf, n.cdf);
+  } else if constexpr (ACT == NMTG_ACT_GELU_LUT) {
+    return act_lut_eval(tab, h);
   } else if constexpr (ACT == NMTG_ACT_SILU) {
     const float s = fast_rcp(1.f + fast_exp2(h * -1.4426950408889634f));
     return s * (1.f + h * (1.f - s));
@@ -165,8 +198,14 @@ __device__ __forceinline__ float act_grad(float h) {
 
 // Calls f(std::integral_constant<int, ACT>) for the runtime activation code: one uniform branch
 // outside the element loops instead of a switch per element.
-template <typename F>
-__device__ __forceinline__ void dispatch_act(int act, F&& f) {
+template <bool LUT_OK, typename F>
+__device__ __forceinline__ void dispatch_act(int act, int lut, F&& f) {
+  if constexpr (LUT_OK) {
+    if (lut && act == NMTG_ACT_GELU) {
+      f(std::integral_constant<int, NMTG_ACT_GELU_LUT>{});
+      return;
+    }
+  }
   switch (act) {
     case NMTG_ACT_RELU: f(std::integral_constant<int, NMTG_ACT_RELU>{}); break;
     case NMTG_ACT_GELU: f(std::integral_constant<int, NMTG_ACT_GELU>{}); break;
@@ -388,7 +427,7 @@ __device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0
 // ---------------------------------------------------------------------------------------------
 // Epilogue shared by the GEMM kernels: accumulators -> (bias, activation, masks, ...) -> global.
 // ---------------------------------------------------------------------------------------------
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int EPI, int VEC>
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int EPI, int VEC, bool LUT_OK = false>
 __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, acc16_t (&acc)[BM / WAVES_M / 32][BN / WAVES_N / 32],
                                               uint8_t* lds_raw, int tile_m, int tile_n, int bz, int split) {
   constexpr int NT = 64 * WAVES_M * WAVES_N;
@@ -471,6 +510,11 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, acc16_t (&acc)[
           store_pack<T, 4>(reinterpret_cast<T*>(sC + ml * PITCH + nl * 2), v);
         }
       }
+    }
+    // activation table behind the staged tile (LUT_OK: the kernel's LDS allocation has the room)
+    const float2* act_tab = reinterpret_cast<const float2*>(sC + ((BM * PITCH + 15) & ~15));
+    if constexpr (LUT_OK && (EPI == EPI_ACT_FWD || EPI == EPI_ACT_BWD)) {
+      if (g.act_lut && g.act == NMTG_ACT_GELU) act_lut_fill<EPI == EPI_ACT_BWD>(const_cast<float2*>(act_tab), tid, NT);
     }
     __syncthreads();
     NMTG_PROF_MARK(3);
@@ -696,7 +740,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, acc16_t (&acc)[
           if (AUX != nullptr) store8<VEC>(AUX + off, raw, nv);
           float a[8];
 #pragma unroll
-          for (int k = 0; k < 8; ++k) a[k] = act_apply<ACT>(v[k]);
+          for (int k = 0; k < 8; ++k) a[k] = act_apply<ACT>(v[k], act_tab);
           if (use_dmask) {
             uint2 keep = mraw[u];
             if (g.rng) {
@@ -725,7 +769,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, acc16_t (&acc)[
           float h[8];
           unpack8<T>(hraw[u], h);
 #pragma unroll
-          for (int k = 0; k < 8; ++k) v[k] *= act_grad<ACT>(h[k]) * (static_cast<float>(byte_of(mraw[u], k)) * g.dscale);
+          for (int k = 0; k < 8; ++k) v[k] *= act_grad<ACT>(h[k], act_tab) * (static_cast<float>(byte_of(mraw[u], k)) * g.dscale);
           // the bias gradient sums the values as stored (rounded to T), as the reference does
           const uint4 packed = pack8<T>(v);
           float r[8];
@@ -746,7 +790,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, acc16_t (&acc)[
       }
     }
     };
-    if constexpr (EPI == EPI_ACT_FWD || EPI == EPI_ACT_BWD) dispatch_act(g.act, phase2);
+    if constexpr (EPI == EPI_ACT_FWD || EPI == EPI_ACT_BWD) dispatch_act<LUT_OK>(g.act, g.act_lut, phase2);
     else phase2(std::integral_constant<int, NMTG_ACT_NONE>{});
 
     NMTG_PROF_MARK(4);

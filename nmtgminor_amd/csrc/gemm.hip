@@ -143,6 +143,9 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
   const bool ring_s = getenv("NMTG_GEMM_RING_S") != nullptr;   // read per call so that a test can switch it
   a.ring = (!ring_off && a.dma && vec == 8 && (tile != TILE_S || ring_s) && a_bytes < (int64_t{1} << 32) &&
             b_bytes < (int64_t{1} << 32)) ? 1 : 0;
+  // gelu through the LDS table: switched on per call by NMTG_GELU_LUT=1 (ring kernels only, they have the LDS room);
+  // off by default until it has been through the GPU test-suite and measured
+  a.act_lut = (a.ring && (epi == EPI_ACT_FWD || epi == EPI_ACT_BWD) && getenv("NMTG_GELU_LUT") != nullptr) ? 1 : 0;
   int bm, bn;
   tile_dims(tile, bm, bn);
   a.m_tiles = ceil_div(a.M, bm);

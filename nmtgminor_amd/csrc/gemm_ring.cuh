@@ -82,7 +82,7 @@ __device__ __forceinline__ void ring_barrier() { asm volatile("s_waitcnt lgkmcnt
 template <int BM, int BN, int RING>
 constexpr int gemm_ring_lds_bytes() {
   constexpr int main_loop = RING * RING_SLOT_BYTES;
-  constexpr int c_tile = BM * (BN * 2 + 8);
+  constexpr int c_tile = ((BM * (BN * 2 + 8) + 15) & ~15) + ACT_LUT_BYTES;   // staged output tile + activation table
   return main_loop > c_tile ? main_loop : c_tile;
 }
 
@@ -276,7 +276,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_ring_kernel(const
   }
 
   NMTG_PROF_MARK(2);
-  gemm_epilogue<T, BM, BN, WAVES_M, WAVES_N, EPI, 8>(g, acc, lds_raw, tile_m, tile_n, bz, split);
+  gemm_epilogue<T, BM, BN, WAVES_M, WAVES_N, EPI, 8, true>(g, acc, lds_raw, tile_m, tile_n, bz, split);
 }
 
 }  // namespace nmtg

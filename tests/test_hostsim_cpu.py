@@ -359,6 +359,12 @@ def test_fused_softmax_backward(mi355x, dtype, t, b, e, h, p, causal):
     tst.test_fused_softmax_backward_matches_two_kernel_path(CPU, dtype, t, b, e, h, p, causal)
 
 
+@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("tokens,dm,di,p", [(256, 128, 256, 0.1), pytest.param(300, 192, 448, 0.0, marks=long_case)])
+def test_table_gelu(mi355x, dtype, tokens, dm, di, p):
+    tst.test_table_gelu_matches_the_formula(CPU, dtype, tokens, dm, di, p)
+
+
 # ----------------------------------------------------------------------------- committed fixtures
 @pytest.mark.parametrize("name", [n for n in dir(tgold) if n.startswith("test_") and n != "test_mlp_fixture"])
 def test_golden_fixtures(mi355x, name):

@@ -3,6 +3,7 @@ not been through the GPU test-suite yet:
 
   NMTG_GEMM_RING_S=1   the slot-ring main loop for the 256x64 tile (per-head products P V, dS K, Pd^T dC, dS^T Q)
   NMTG_ATTN_FUSED=1    Q K^T -> mask -> softmax -> dropout in one kernel (rows of up to 512 keys)
+  NMTG_GELU_LUT=1      gelu and its derivative in the MLP epilogues read from a 513-entry table in LDS
 
 The library reads both switches on every call, so each test runs the default path and the staged
 path in one process and compares them (and the staged path with the CPU oracle). The tests only run
@@ -13,9 +14,9 @@ import os
 import pytest
 import torch
 
-from nmtgminor_amd.native import self_multihead_attn_blaslt as sa_native
+from nmtgminor_amd.native import fused_mlp_gelu, self_multihead_attn_blaslt as sa_native
 from nmtgminor_amd.native.linear_gemm import gemm
-from oracle import attention as oat, inputs
+from oracle import attention as oat, inputs, mlp as omlp
 from util import assert_close
 
 pytestmark = [pytest.mark.gpu,
@@ -118,3 +119,41 @@ def test_fused_softmax_backward_matches_two_kernel_path(dev, dtype, t, b, e, h, 
                                 (bwd["dx"], bwd["dw_in"], bwd["dw_out"], bwd["db_in"], bwd["db_out"])):
         assert_close(a_, r_.float().cpu(), dtype, name + " vs two-kernel path", scale_atol=True)
         assert_close(a_, o_, dtype, name + " vs oracle", scale_atol=True)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("tokens,dm,di,p", [(256, 128, 256, 0.1), (300, 192, 448, 0.0), (128, 512, 2048, 0.2)])
+def test_table_gelu_matches_the_formula(dev, dtype, tokens, dm, di, p):
+    # wide pre-activations (|h| up to ~8): both ends of the table and the clamp beyond them are used
+    d = inputs.mlp_inputs(tokens, dm, di, dtype, p=p, seed=95, zero_bias=False)
+    d["x"] = (d["x"].float() * 4).to(dtype)
+    ins = [d[k].to(dev) for k in ("x", "w1", "w2", "b1", "b2")]
+    ins[0].requires_grad_()                                      # asks the backward for dx
+    mask = d["mask"].to(dev) if p > 0 else None
+    dy = d["dy"].to(dev)
+    ref = fused_mlp_gelu.forward(p, ins, mask)
+    gref = fused_mlp_gelu.backward(p, dy, ref, ins)
+    with switch("NMTG_GELU_LUT"):
+        got = fused_mlp_gelu.forward(p, ins, mask)
+        ggot = fused_mlp_gelu.backward(p, dy, ref, ins)          # same saved tensors: only the derivative differs
+    assert torch.equal(got[2], ref[2])                           # pre-activations do not involve the activation
+    pre = ref[2].float()
+    assert pre.abs().max() > 6.5 and (pre.abs() < 0.05).any()
+    # Phi from the table is within 2e-5 of the formula, a twentieth of an fp16 ulp and less of a bf16 ulp: after
+    # rounding most elements are identical and the rest one ulp apart (so the table is in use, and accurate)
+    same = (got[1] == ref[1]).float().mean().item()
+    assert (0.75 if dtype == torch.float16 else 0.9) < same < 1.0, same
+    ulp = 2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7      # largest relative size of one unit in the last place
+    assert_close(got[1], ref[1].float().cpu(), dtype, "post-activations: table vs formula", rtol=1.05 * ulp, atol=3e-5)
+    # downstream of the activations: sums of slightly different rounded terms, themselves rounded once more
+    assert_close(got[0], ref[0].float().cpu(), dtype, "y: table vs formula", rtol=2.1 * ulp, atol=1e-3, scale_atol=True)
+    for name, a_, r_ in zip(("dx", "dw1", "dw2", "db1", "db2"), ggot, gref):
+        assert_close(a_, r_.float().cpu(), dtype, name + ": table vs formula", rtol=2.1 * ulp, atol=2e-3, scale_atol=True)
+    ws, bs = [d["w1"], d["w2"]], [d["b1"], d["b2"]]
+    masks = [d["mask"]] if p > 0 else None
+    y, pre_o, post_o = omlp.mlp_fwd(d["x"], ws, bs, "gelu", p, masks, D, round_to=dtype)
+    gx, gws, gbs = omlp.mlp_bwd(d["dy"], d["x"], ws, pre_o, post_o, "gelu", p, masks, D, round_to=dtype)
+    assert_close(got[0], y, dtype, "y vs oracle", scale_atol=True)
+    assert_close(ggot[0], gx, dtype, "dx vs oracle", scale_atol=True)
+    assert_close(ggot[1], gws[0], dtype, "dW1 vs oracle", scale_atol=True)
+    assert_close(ggot[3], gbs[0], dtype, "db1 vs oracle", scale_atol=True)
