@@ -245,6 +245,49 @@ void sync_block() {
   yield();
 }
 
+
+// ---- wavefront-wide instructions (declared in the stand-in header; here so that they are compiled with optimisation
+// while the kernel sources themselves are not) ----
+void resolve_tr_read(void** payloads, int lanes) {
+  if (lanes != 64) fail("LDS transpose read in a partial wavefront");
+  short raw[64][4];
+  for (int l = 0; l < 64; ++l) std::memcpy(raw[l], static_cast<TrRead*>(payloads[l])->addr, 8);
+  for (int l = 0; l < 64; ++l) {
+    const int blk = l & ~15, i = l & 15;
+    for (int e = 0; e < 4; ++e) static_cast<TrRead*>(payloads[l])->out[e] = raw[blk + 4 * e + (i >> 2)][i & 3];
+  }
+}
+
+template <bool BF16>
+static inline float widen(uint16_t bits) {
+  if (BF16) { const uint32_t u = static_cast<uint32_t>(bits) << 16; float f; std::memcpy(&f, &u, 4); return f; }
+  return __half2float(__ushort_as_half(bits));
+}
+template <bool BF16>
+static void resolve_mfma(void** payloads, int lanes) {
+  if (lanes != 64) fail("MFMA in a partial wavefront");
+  float A[32][16], B[16][32];
+  for (int l = 0; l < 64; ++l) {
+    const Mfma* m = static_cast<const Mfma*>(payloads[l]);
+    for (int t = 0; t < 8; ++t) {
+      A[l & 31][8 * (l >> 5) + t] = widen<BF16>(m->a[t]);
+      B[8 * (l >> 5) + t][l & 31] = widen<BF16>(m->b[t]);
+    }
+  }
+  for (int l = 0; l < 64; ++l) {
+    float* c = static_cast<Mfma*>(payloads[l])->c;
+    const int j = l & 31;
+    for (int r = 0; r < 16; ++r) {
+      const int i = 8 * (r / 4) + 4 * (l >> 5) + r % 4;
+      float s = c[r];
+      for (int k = 0; k < 16; ++k) s += A[i][k] * B[k][j];
+      c[r] = s;
+    }
+  }
+}
+void resolve_mfma_f16(void** payloads, int lanes) { resolve_mfma<false>(payloads, lanes); }
+void resolve_mfma_bf16(void** payloads, int lanes) { resolve_mfma<true>(payloads, lanes); }
+
 int compute_units() {
   const char* e = std::getenv("HOSTSIM_CUS");
   const int n = e ? std::atoi(e) : 4;

@@ -24,6 +24,10 @@ CXX = os.environ.get("HOSTSIM_CXX", "/opt/rocm/lib/llvm/bin/clang++")
 #   HOSTSIM_SANITIZE=1 LD_PRELOAD=$(clang++ -print-file-name=libclang_rt.asan-x86_64.so) \
 #   ASAN_OPTIONS=detect_leaks=0:detect_stack_use_after_return=0 python -m pytest tests/test_hostsim_cpu.py
 SANITIZE = os.environ.get("HOSTSIM_SANITIZE") == "1"
+# The kernel sources are compiled without optimisation: their epilogues unroll into functions of 10^5 instructions that
+# take a minute each to optimise and run no faster for it (the time goes into fiber switches and the MFMA arithmetic,
+# which live in hostsim.cpp and are optimised).
+OPT = os.environ.get("HOSTSIM_OPT", "-O0")
 LIB = os.path.join(BUILD, "libnmtg_hostsim_asan.so" if SANITIZE else "libnmtg_hostsim.so")
 
 KERNEL_SOURCES = ["api.hip", "layer_norm.hip", "softmax_dropout.hip", "dropout_add.hip", "xentropy.hip", "reduce.hip",
@@ -92,7 +96,7 @@ def build(verbose=False):
         if not name.endswith(".cuh"):
             units.append(dst)
     units += [os.path.join(HERE, n) for n in OWN_SOURCES]
-    flags = ["-x", "c++", "-std=c++17", "-O1", "-gline-tables-only", "-fPIC", "-fno-strict-aliasing", "-Wno-unknown-pragmas",
+    flags = ["-x", "c++", "-std=c++17", OPT, "-gline-tables-only", "-fPIC", "-fno-strict-aliasing", "-Wno-unknown-pragmas",
              "-Wno-pass-failed", "-Wno-unused-command-line-argument", "-I" + os.path.join(HERE, "shim"), "-I" + BUILD]
     link = []
     if SANITIZE:
@@ -104,7 +108,8 @@ def build(verbose=False):
     for u in units:
         obj = os.path.join(BUILD, os.path.basename(u) + (".asan.o" if SANITIZE else ".o"))
         objs.append(obj)
-        procs.append((u, subprocess.Popen([CXX] + flags + ["-c", u, "-o", obj], stdout=subprocess.PIPE,
+        opt = ["-O2"] if os.path.dirname(u) == HERE else []
+        procs.append((u, subprocess.Popen([CXX] + flags + opt + ["-c", u, "-o", obj], stdout=subprocess.PIPE,
                                           stderr=subprocess.STDOUT, text=True)))
     failed = False
     for u, p in procs:
@@ -126,4 +131,7 @@ def ensure():
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
+    if "--if-stale" in sys.argv:
+        print(ensure())
+    else:
+        print(build(verbose=True))

@@ -135,15 +135,7 @@ static inline void __builtin_amdgcn_global_load_lds(const __attribute__((address
 typedef short hostsim_short4 __attribute__((ext_vector_type(4)));
 namespace hostsim {
 struct TrRead { const unsigned char* addr; short out[4]; };
-static inline void resolve_tr_read(void** payloads, int lanes) {
-  if (lanes != 64) fail("LDS transpose read in a partial wavefront");
-  short raw[64][4];
-  for (int l = 0; l < 64; ++l) std::memcpy(raw[l], static_cast<TrRead*>(payloads[l])->addr, 8);
-  for (int l = 0; l < 64; ++l) {
-    const int blk = l & ~15, i = l & 15;
-    for (int e = 0; e < 4; ++e) static_cast<TrRead*>(payloads[l])->out[e] = raw[blk + 4 * e + (i >> 2)][i & 3];
-  }
-}
+void resolve_tr_read(void** payloads, int lanes);
 }  // namespace hostsim
 static inline hostsim_short4 __builtin_amdgcn_ds_read_tr16_b64_v4i16(__attribute__((address_space(3))) hostsim_short4* p) {
   hostsim::TrRead r;
@@ -158,33 +150,8 @@ static inline hostsim_short4 __builtin_amdgcn_ds_read_tr16_b64_v4i16(__attribute
 typedef float hostsim_float16 __attribute__((ext_vector_type(16)));
 namespace hostsim {
 struct Mfma { const uint16_t* a; const uint16_t* b; float* c; };
-template <bool BF16>
-static inline float widen(uint16_t bits) {
-  if (BF16) { const uint32_t u = static_cast<uint32_t>(bits) << 16; float f; std::memcpy(&f, &u, 4); return f; }
-  return __half2float(__ushort_as_half(bits));
-}
-template <bool BF16>
-static inline void resolve_mfma(void** payloads, int lanes) {
-  if (lanes != 64) fail("MFMA in a partial wavefront");
-  float A[32][16], B[16][32];
-  for (int l = 0; l < 64; ++l) {
-    const Mfma* m = static_cast<const Mfma*>(payloads[l]);
-    for (int t = 0; t < 8; ++t) {
-      A[l & 31][8 * (l >> 5) + t] = widen<BF16>(m->a[t]);
-      B[8 * (l >> 5) + t][l & 31] = widen<BF16>(m->b[t]);
-    }
-  }
-  for (int l = 0; l < 64; ++l) {
-    float* c = static_cast<Mfma*>(payloads[l])->c;
-    const int j = l & 31;
-    for (int r = 0; r < 16; ++r) {
-      const int i = 8 * (r / 4) + 4 * (l >> 5) + r % 4;
-      float s = c[r];
-      for (int k = 0; k < 16; ++k) s += A[i][k] * B[k][j];
-      c[r] = s;
-    }
-  }
-}
+void resolve_mfma_f16(void** payloads, int lanes);
+void resolve_mfma_bf16(void** payloads, int lanes);
 template <bool BF16, typename V>
 static inline hostsim_float16 mfma(V a, V b, hostsim_float16 c) {
   uint16_t av[8], bv[8];
@@ -193,7 +160,7 @@ static inline hostsim_float16 mfma(V a, V b, hostsim_float16 c) {
   std::memcpy(bv, &b, 16);
   std::memcpy(cv, &c, 64);
   Mfma m{av, bv, cv};
-  wave_collective(resolve_mfma<BF16>, &m);
+  wave_collective(BF16 ? resolve_mfma_bf16 : resolve_mfma_f16, &m);
   hostsim_float16 d;
   std::memcpy(&d, cv, 64);
   return d;

@@ -42,11 +42,21 @@ F32, F16, BF16 = torch.float32, torch.float16, torch.bfloat16
 SANITIZER_RUN = os.environ.get("HOSTSIM_SANITIZE") == "1"
 # the sanitizer build is several times slower: it repeats every check except the ones marked long
 long_case = pytest.mark.skipif(SANITIZER_RUN, reason="left out of the sanitizer run for time")
+HALVES = [BF16] if SANITIZER_RUN else [F16, BF16]          # the two 16-bit types share every index computation
+
+
+_sanitizer_build = {}
 
 
 @pytest.fixture(scope="session")
 def hostsim_lib():
-    return harness.library()
+    lib = harness.library()
+    # the sanitizer variant is needed by the last test of this file: compile it meanwhile
+    if not SANITIZER_RUN and "proc" not in _sanitizer_build:
+        env = dict(os.environ, HOSTSIM_SANITIZE="1")
+        _sanitizer_build["proc"] = subprocess.Popen([sys.executable, os.path.join(harness.HERE, "hostsim_build.py"), "--if-stale"],
+                                                    env=env, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+    return lib
 
 
 @pytest.fixture(autouse=True)
@@ -163,6 +173,7 @@ def test_xentropy_misaligned_base(misalign):
     tel._xent_case(CPU, 9, 1001, BF16, 0.1, pad=0, misalign=misalign)
 
 
+@long_case
 def test_xentropy_no_smoothing_module_and_autograd():
     tel.test_xentropy_no_smoothing_and_module_parity(CPU)
     tel.test_xentropy_autograd_function(CPU)
@@ -229,7 +240,7 @@ def test_split_k_reduction(hostsim_lib, dtype, tile, m, n, batch, splits, c_vec)
 
 
 # ----------------------------------------------------------------------------- GEMM core
-@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("dtype", HALVES)
 @pytest.mark.parametrize("m,n,k", [(256, 256, 64), (128, 128, 128), (300, 200, 72), (1, 8, 8), (257, 129, 1000), (64, 1504, 64),
                                    pytest.param(512, 2048, 512, marks=long_case), pytest.param(1024, 64, 512, marks=long_case)])
 @pytest.mark.parametrize("layout", ["nt", "nn", "tn"])
@@ -245,7 +256,7 @@ def test_gemm_ring_under_both_transfer_timings(mi355x, dma, layout, m, n, k):
 
 
 @long_case
-@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("dtype", HALVES)
 def test_gemm_unaligned_extents(mi355x, dtype):
     tg.test_gemm_unaligned_extents(CPU, dtype)
 
@@ -267,7 +278,7 @@ def test_gemm_split_k(mi355x, hostsim_lib):
 
 
 # ----------------------------------------------------------------------------- fused MLP
-@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("dtype", HALVES)
 @pytest.mark.parametrize("act", ["gelu", "relu", "silu", "agelu"])
 @pytest.mark.parametrize("tokens,dm,di,p", [(72, 96, 200, 0.5), pytest.param(256, 128, 256, 0.0, marks=long_case)])
 def test_mlp_autograd_function(mi355x, dtype, act, tokens, dm, di, p):
@@ -281,13 +292,14 @@ def test_mlp_recompute_input_only_three_layers_rng(mi355x):
 
 
 # ----------------------------------------------------------------------------- attention
-@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("dtype", HALVES)
 @pytest.mark.parametrize("t,b,e,h,p", [pytest.param(64, 4, 256, 4, 0.0, marks=long_case), (33, 2, 128, 2, 0.1),
                                        pytest.param(200, 2, 256, 4, 0.25, marks=long_case)])
 def test_self_attention_key_padding(mi355x, dtype, t, b, e, h, p):
     tat.test_self_attention_key_padding(CPU, dtype, t, b, e, h, p)
 
 
+@long_case
 def test_self_attention_contract_rng_eval_no_bias(mi355x):
     tat.test_self_attention_intermediates_and_native_contract(CPU)
     tat.test_self_attention_rng_dropout_eval_and_no_bias(CPU)
@@ -298,7 +310,7 @@ def test_self_attention_causal_and_recompute(mi355x):
     tat.test_self_attention_causal_and_recompute(CPU, BF16)
 
 
-@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("dtype", HALVES)
 @pytest.mark.parametrize("tq,tk,b,e,h,p", [(17, 100, 3, 128, 2, 0.2), pytest.param(32, 1500, 2, 256, 4, 0.1, marks=long_case)])
 def test_encdec_attention(mi355x, dtype, tq, tk, b, e, h, p):
     tat.test_encdec_attention(CPU, dtype, tq, tk, b, e, h, p)
@@ -317,31 +329,33 @@ def test_pre_post_processing(mi355x, dtype):
     tla.test_pre_post_processing_sequences(CPU, dtype)
 
 
-@pytest.mark.parametrize("dtype", [F16, BF16])
-@pytest.mark.parametrize("macaron,training", [(False, False), (False, True), (True, True)])
+@pytest.mark.parametrize("dtype", HALVES)
+@pytest.mark.parametrize("macaron,training", [pytest.param(False, False, marks=long_case), pytest.param(False, True, marks=long_case),
+                                              (True, True)])
 def test_encoder_layer(mi355x, dtype, macaron, training):
     tla.test_encoder_layer_matches_the_oracle(CPU, dtype, macaron, training)
 
 
-@pytest.mark.parametrize("dtype", [F16, BF16])
-@pytest.mark.parametrize("ignore_source", [False, True])
+@pytest.mark.parametrize("dtype", HALVES)
+@pytest.mark.parametrize("ignore_source", [False, pytest.param(True, marks=long_case)])
 def test_decoder_layer(mi355x, dtype, ignore_source):
     tla.test_decoder_layer_matches_the_oracle(CPU, dtype, ignore_source)
 
 
+@long_case
 def test_layers_stochastic_depth_dropout_and_options(mi355x):
     tla.test_encoder_layer_stochastic_depth(CPU)
     tla.test_layers_with_dropout_and_unsupported_options(CPU)
 
 
 # ----------------------------------------------------------------------------- variants that are switched off by default
-@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("dtype", HALVES)
 @pytest.mark.parametrize("batch,m,n,k", [(3, 300, 64, 192), (2, 256, 64, 64), (5, 77, 64, 128)])
 def test_ring_loop_of_the_256x64_tile(mi355x, dma, dtype, batch, m, n, k):
     tst.test_ring_256x64_matches_two_buffer_loop(CPU, dtype, batch, m, n, k)
 
 
-@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("dtype", HALVES)
 @pytest.mark.parametrize("t,b,e,h,p,causal", [pytest.param(200, 2, 256, 4, 0.25, False, marks=long_case), (96, 2, 128, 2, 0.1, True),
                                               (40, 2, 128, 2, 0.1, False), pytest.param(512, 2, 256, 4, 0.1, False, marks=long_case)])
 def test_fused_scores_softmax(mi355x, dtype, t, b, e, h, p, causal):
@@ -352,14 +366,14 @@ def test_fused_scores_softmax_draws_the_same_dropout_mask(mi355x):
     tst.test_fused_scores_softmax_rng_mask_is_the_same_stream(CPU)
 
 
-@pytest.mark.parametrize("dtype", [F16, BF16])
-@pytest.mark.parametrize("t,b,e,h,p,causal", [(96, 2, 128, 2, 0.0, True), (40, 2, 128, 2, 0.1, False),
+@pytest.mark.parametrize("dtype", HALVES)
+@pytest.mark.parametrize("t,b,e,h,p,causal", [pytest.param(96, 2, 128, 2, 0.0, True, marks=long_case), (40, 2, 128, 2, 0.1, False),
                                               pytest.param(200, 2, 256, 4, 0.25, False, marks=long_case)])
 def test_fused_softmax_backward(mi355x, dtype, t, b, e, h, p, causal):
     tst.test_fused_softmax_backward_matches_two_kernel_path(CPU, dtype, t, b, e, h, p, causal)
 
 
-@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("dtype", HALVES)
 @pytest.mark.parametrize("tokens,dm,di,p", [(256, 128, 256, 0.1), pytest.param(300, 192, 448, 0.0, marks=long_case)])
 def test_table_gelu(mi355x, dtype, tokens, dm, di, p):
     tst.test_table_gelu_matches_the_formula(CPU, dtype, tokens, dm, di, p)
@@ -394,6 +408,8 @@ def test_every_check_again_under_address_sanitizer():
                              text=True).stdout.strip()
     if not os.path.isabs(runtime) or not os.path.exists(runtime):
         pytest.skip("no AddressSanitizer runtime beside the compiler")
+    if "proc" in _sanitizer_build:
+        _sanitizer_build["proc"].wait()
     env = dict(os.environ, HOSTSIM_SANITIZE="1", LD_PRELOAD=runtime,
                ASAN_OPTIONS="detect_leaks=0:detect_stack_use_after_return=0")
     run = subprocess.run([sys.executable, "-m", "pytest", os.path.abspath(__file__), "-x", "-q", "-p", "no:cacheprovider"],
