@@ -137,13 +137,15 @@ __device__ __forceinline__ NormalCdfPdf normal_cdf_pdf(float h) {
 }
 
 // gelu through a table. The activation epilogues are VALU-bound (about 30 instruction slots per element, two of
-// them quarter-rate transcendentals), so Phi(h) and gelu'(h) can instead be read from a 513-entry table over
-// [-6, 6] that the block builds in LDS with the exact formula: one fused multiply-add for the table coordinate, a
-// clamp, a fraction, one 8-byte LDS read of (value, difference to the next entry) and one fused multiply-add.
-// Linear interpolation error: step^2 / 8 * max|f''| = 1.7e-5 for Phi, 4e-5 for gelu' (the 16-bit tolerances are
-// 1e-3). Outside [-6, 6] the end values (1e-9 / 1 - 1e-9) are used.
+// them quarter-rate transcendentals), so Phi(h) and gelu'(h) can instead be read from a 2049-entry table over
+// [-6, 6] (16 KB) that the block builds in LDS with the exact formula: one fused multiply-add for the table
+// coordinate, a clamp, a fraction, one 8-byte LDS read of (value, difference to the next entry) and one fused
+// multiply-add. Linear interpolation error: step^2 / 8 * max|f''| = 1.0e-6 for Phi, 2.6e-6 for gelu': a rounded
+// 16-bit result differs from the formula's in about one element in a thousand, by one unit in the last place.
+// (A 513-entry table, error 1.7e-5, flipped enough bf16 roundings to push the second layer's output past the
+// absolute tolerance on a few elements in 10^5 at the benchmark shape.) Outside [-6, 6] the end values are used.
 constexpr int NMTG_ACT_GELU_LUT = 100;      // internal activation code: gelu evaluated through the table
-constexpr int ACT_LUT_N = 512;
+constexpr int ACT_LUT_N = 2048;
 constexpr float ACT_LUT_R = 6.f;
 constexpr int ACT_LUT_BYTES = (ACT_LUT_N + 1) * 8;
 

@@ -3,7 +3,8 @@
 Mirrors EncdecAttnBiasFunc / encdec_attn_bias_func and the compact variant of the reference
 (onmt/modules/optimized/encdec_attention_func_bias.py:41-668, :687-1011): the same 20 positional
 arguments and 20 gradient slots; biases may be None (the reference then leaves its fused path,
-:69-73; here the fused path takes them). Rotary encoding and incremental decoding raise. A 21st
+:69-73; here the fused path takes them). Rotary encoding raises; incremental decoding (inference with a cache
+dict) runs in nmtgminor_amd/modules/incremental.py. A 21st
 optional argument replays an explicit dropout keep-mask."""
 import torch
 
@@ -61,6 +62,15 @@ class EncdecAttnBiasFunc(torch.autograd.Function):
 def encdec_attn_bias_func(*args):
     args = cast_if_autocast_enabled(*args)
     with no_autocast():
+        if len(args) > 14 and args[13]:               # incremental decoding: encoder keys / values come from the cache
+            from .incremental import encdec_attn_step
+            (_, _, heads, inputs_q, inputs_kv, w_q, w_kv, w_out, b_q, b_kv, b_out, mask, _, _, cache, rotary) = args[:16]
+            if rotary:
+                raise NotImplementedError("encdec_attn_bias_func: rotary position encoding has no HIP kernel")
+            if cache is None:
+                raise RuntimeError("encdec_attn_bias_func: incremental decoding needs an incremental_cache dict")
+            outputs, probs = encdec_attn_step(heads, inputs_q, inputs_kv, w_q, w_kv, w_out, b_q, b_kv, b_out, mask, cache)
+            return (outputs, probs) if args[19] else (outputs,)
         return EncdecAttnBiasFunc.apply(*args)
 
 

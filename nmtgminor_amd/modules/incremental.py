@@ -1,0 +1,79 @@
+"""Incremental (step by step) decoding for the two attention operators, on the HIP kernels.
+
+What the reference does in the `incremental` branches of its attention functions
+(onmt/modules/optimized/self_attention_func.py:162-174, encdec_attention_func_bias.py:181-213), with the same
+cache entries so that the reference's beam search can reorder them (every entry is time-first [T, B, E] and is
+re-indexed along dimension 1):
+    self-attention     cache['k'], cache['v']      keys / values of all positions decoded so far (grow by one row)
+    cross-attention    cache['c_k'], cache['c_v']  keys / values of the encoder states (computed at the first step)
+Inference only (no autograd graph, no dropout). The projections are GEMM calls of the library, the attention core is
+the compact cross-attention entry point (queries and a [Tk, B*H, 2, D] key/value block come in, the context goes
+out); the cache bookkeeping (slices, concatenation, the interleave of keys and values) is tensor movement on the
+device, exactly the reference's. A later step may carry one new position only: with more than one, the new
+positions would need a causal mask among themselves, which the cross-attention core does not take.
+"""
+import torch
+
+from ..native import encdec_multihead_attn_bias_blaslt as ed_native
+from ..native.linear_gemm import gemm
+
+
+def _project(x, weight, bias):
+    t, b, e = x.shape
+    return gemm(x.reshape(t * b, e), weight, False, True, bias=bias).view(t, b, weight.shape[0])
+
+
+def _core(heads, q_lin, keys, values, pad_mask):
+    """q_lin [Tq, B, E]; keys, values [Tk, B, E] -> (context [Tq, B, E], probabilities [B*H, Tq, Tk])."""
+    tk, b, e = keys.shape
+    d = e // heads
+    kv = torch.stack([keys.view(tk, b * heads, d), values.view(tk, b * heads, d)], dim=-2).view(tk, b, 2 * e)
+    scores, probs, _, context = ed_native.forward_compact(False, heads, q_lin.contiguous(), kv, pad_mask, 0.0)
+    return context, probs
+
+
+@torch.no_grad()
+def self_attn_step(heads, inputs, input_weights, output_weights, input_biases, output_biases, mask, cache):
+    """inputs [T_new, B, E]: all positions at the first call (no 'k' in the cache; `mask` is then the usual time mask
+    [T, T]), one new position afterwards. -> (outputs [T_new, B, E], probabilities [B*H, T_new, T_total])."""
+    t_new, b, e = inputs.shape
+    d = e // heads
+    lin = _project(inputs, input_weights, input_biases).view(t_new, b * heads, 3, d)
+    queries = lin[:, :, 0, :].reshape(t_new, b, e)
+    keys = lin[:, :, 1, :].reshape(t_new, b, e)
+    values = lin[:, :, 2, :].reshape(t_new, b, e)
+    first = not ("k" in cache and "v" in cache)
+    if not first:
+        if t_new != 1:
+            raise NotImplementedError("incremental self-attention: one new position per step once the cache is filled")
+        keys = torch.cat([cache["k"], keys], dim=0)
+        values = torch.cat([cache["v"], values], dim=0)
+    cache["k"], cache["v"] = keys, values
+    if first and t_new > 1:
+        # a prefix of several positions: the full-sequence kernel with its time mask, fed with the same projection
+        from ..native import self_multihead_attn_blaslt as sa_native
+        if mask is None:
+            mask = torch.triu(torch.ones(t_new, t_new, dtype=torch.bool, device=inputs.device), 1)
+        _, probs, _, context = sa_native.forward_compact(True, False, heads, lin.view(t_new, b, 3 * e), mask.to(torch.bool), 0.0)
+    else:
+        context, probs = _core(heads, queries, keys, values, None)
+    return _project(context, output_weights, output_biases), probs
+
+
+@torch.no_grad()
+def encdec_attn_step(heads, inputs_q, inputs_kv, input_weights_q, input_weights_kv, output_weights, input_bias_q,
+                     input_bias_kv, output_bias, mask, cache):
+    """inputs_q [Tq, B, E]; inputs_kv [Tk, B, E] is read at the first call only. mask: key padding [B, Tk]."""
+    tq, b, e = inputs_q.shape
+    d = e // heads
+    if "c_k" in cache and "c_v" in cache:
+        keys, values = cache["c_k"], cache["c_v"]
+    else:
+        tk = inputs_kv.shape[0]
+        kv = _project(inputs_kv, input_weights_kv, input_bias_kv).view(tk, b * heads, 2, d)
+        keys = kv[:, :, 0, :].reshape(tk, b, e)
+        values = kv[:, :, 1, :].reshape(tk, b, e)
+        cache["c_k"], cache["c_v"] = keys, values
+    q_lin = _project(inputs_q, input_weights_q, input_bias_q)
+    context, probs = _core(heads, q_lin, keys, values, mask)
+    return _project(context, output_weights, output_bias), probs

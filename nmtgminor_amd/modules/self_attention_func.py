@@ -3,8 +3,9 @@
 Mirrors SelfAttnFunc / self_attn_func and SelfAttnCompactFunc / self_attn_compact_func of the
 reference (onmt/modules/optimized/self_attention_func.py:50-520, :523-837): the same 17
 positional arguments and 17 gradient slots. Every call takes the fused path (fp16 or bf16, biases
-optional, T <= 4096); what the HIP path does not cover (rotary position encoding, incremental
-decoding) raises instead of falling back. As in the reference's fused branch the result is always
+optional, T <= 4096); what the HIP path does not cover (rotary position encoding) raises instead of
+falling back. Incremental decoding (inference, `incremental=True` with a cache dict) runs in
+nmtgminor_amd/modules/incremental.py. As in the reference's fused branch the result is always
 the pair (outputs, dropout_results). An 18th optional argument replays an explicit dropout
 keep-mask."""
 import torch
@@ -73,6 +74,14 @@ class SelfAttnFunc(torch.autograd.Function):
 def self_attn_func(*args):
     args = cast_if_autocast_enabled(*args)
     with no_autocast():
+        if len(args) > 13 and args[12]:               # incremental decoding: cache in, one more position out
+            from .incremental import self_attn_step
+            (use_time_mask, is_training, heads, inputs, w_in, w_out, b_in, b_out, mask, p, rotary, pos_emb, _, cache) = args[:14]
+            if rotary:
+                raise NotImplementedError("self_attn_func: rotary position encoding has no HIP kernel")
+            if cache is None:
+                raise RuntimeError("self_attn_func: incremental decoding needs an incremental_cache dict")
+            return self_attn_step(heads, inputs, w_in, w_out, b_in, b_out, mask if use_time_mask else None, cache)
         return SelfAttnFunc.apply(*args)
 
 

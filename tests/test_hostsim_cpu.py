@@ -31,6 +31,7 @@ import test_attention_gpu as tat  # noqa: E402
 import test_elementwise_gpu as tel  # noqa: E402
 import test_gemm_gpu as tg  # noqa: E402
 import test_layer_norm_gpu as tln  # noqa: E402
+import test_zx_incremental_gpu as tinc  # noqa: E402
 import test_zy_layers_gpu as tla  # noqa: E402
 import test_mlp_gpu as tm  # noqa: E402
 import test_staged_gpu as tst  # noqa: E402
@@ -346,6 +347,19 @@ def test_decoder_layer(mi355x, dtype, ignore_source):
 def test_layers_stochastic_depth_dropout_and_options(mi355x):
     tla.test_encoder_layer_stochastic_depth(CPU)
     tla.test_layers_with_dropout_and_unsupported_options(CPU)
+
+
+# ----------------------------------------------------------------------------- incremental decoding
+@pytest.mark.parametrize("dtype", HALVES)
+def test_incremental_decoding(mi355x, dtype):
+    tinc.test_self_attention_step_by_step(CPU, dtype, 3)
+    tinc.test_cross_attention_with_cached_encoder_states(CPU, dtype)
+
+
+@long_case
+def test_incremental_decoder_layer_with_beam_reordering(mi355x):
+    tinc.test_self_attention_step_by_step(CPU, F16, 1)
+    tinc.test_decoder_layer_step_by_step_with_beam_reordering(CPU)
 
 
 # ----------------------------------------------------------------------------- variants that are switched off by default

@@ -3,7 +3,7 @@ not been through the GPU test-suite yet:
 
   NMTG_GEMM_RING_S=1   the slot-ring main loop for the 256x64 tile (per-head products P V, dS K, Pd^T dC, dS^T Q)
   NMTG_ATTN_FUSED=1    Q K^T -> mask -> softmax -> dropout in one kernel (rows of up to 512 keys)
-  NMTG_GELU_LUT=1      gelu and its derivative in the MLP epilogues read from a 513-entry table in LDS
+  NMTG_GELU_LUT=1      gelu and its derivative in the MLP epilogues read from a 2049-entry table in LDS
 
 The library reads both switches on every call, so each test runs the default path and the staged
 path in one process and compares them (and the staged path with the CPU oracle). The tests only run
@@ -139,10 +139,10 @@ def test_table_gelu_matches_the_formula(dev, dtype, tokens, dm, di, p):
     assert torch.equal(got[2], ref[2])                           # pre-activations do not involve the activation
     pre = ref[2].float()
     assert pre.abs().max() > 6.5 and (pre.abs() < 0.05).any()
-    # Phi from the table is within 2e-5 of the formula, a twentieth of an fp16 ulp and less of a bf16 ulp: after
-    # rounding most elements are identical and the rest one ulp apart (so the table is in use, and accurate)
+    # Phi from the table is within 1e-6 of the formula: after rounding nearly all elements are identical and the rest
+    # one ulp apart (so the table is in use, and accurate)
     same = (got[1] == ref[1]).float().mean().item()
-    assert (0.75 if dtype == torch.float16 else 0.9) < same < 1.0, same
+    assert 0.95 < same < 1.0, same    # the differing ones sit in the negative tail, where gelu itself is below 1e-2
     ulp = 2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7      # largest relative size of one unit in the last place
     assert_close(got[1], ref[1].float().cpu(), dtype, "post-activations: table vs formula", rtol=1.05 * ulp, atol=3e-5)
     # downstream of the activations: sums of slightly different rounded terms, themselves rounded once more

@@ -1,0 +1,118 @@
+"""Incremental decoding (one position per step, keys / values cached) against the full-sequence operators.
+
+Decoding position by position with the cache must reproduce, row by row, what the same module computes for the whole
+sequence under a causal mask: the property the reference's translator relies on
+(onmt/modules/optimized/self_attention_func.py:162-174, encdec_attention_func_bias.py:181-213). The cache entries
+('k', 'v', 'c_k', 'c_v': time-first [T, B, E]) can be re-indexed along the batch dimension between steps, as beam
+search does.
+"""
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from nmtgminor_amd.modules.encdec_attention import EncdecMultiheadAttn
+from nmtgminor_amd.modules.self_attention import SelfMultiheadAttn
+from nmtgminor_amd.modules.transformer_layers import DecoderLayer
+from oracle import inputs
+from util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def _randomise(module, seed):
+    g = torch.Generator().manual_seed(seed)
+    with torch.no_grad():
+        for p in module.parameters():
+            p.add_((0.1 if p.dim() == 1 else 0.02) * torch.randn(p.shape, generator=g))
+    return module
+
+
+def close(a, b, dtype, what):
+    # the same products, accumulated by different kernels (a [1, T] row instead of a [T, T] tile)
+    assert_close(a, b.float().cpu(), dtype, what, rtol=2e-2, atol=4e-3 if dtype == torch.float16 else 3e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("prefix", [1, 3])
+def test_self_attention_step_by_step(dev, dtype, prefix):
+    t, b, e, h = 11, 3, 128, 4
+    attn = _randomise(SelfMultiheadAttn(e, h, 0.1), 91).to(dev).to(dtype).eval()
+    x = torch.randn(t, b, e, generator=torch.Generator().manual_seed(92)).to(dtype).to(dev)
+    causal = torch.triu(torch.ones(t, t, device=dev), 1).bool()
+    with torch.no_grad():
+        full, _ = attn(x, None, None, causal)
+    cache = {}
+    rows = []
+    with torch.no_grad():
+        out, cov = attn(x[:prefix], None, None, causal[:prefix, :prefix], incremental=True, incremental_cache=cache)
+        rows.append(out)
+        assert cov.shape == (b * h, prefix, prefix)
+        for i in range(prefix, t):
+            out, cov = attn(x[i:i + 1], None, None, causal[i:i + 1, :i + 1], incremental=True, incremental_cache=cache)
+            rows.append(out)
+            assert cache["k"].shape == (i + 1, b, e) and cache["v"].shape == (i + 1, b, e)
+            assert cov.shape == (b * h, 1, i + 1)
+            assert_close(cov.float().sum(-1), torch.ones(b * h, 1), dtype, "probabilities sum to one", atol=2e-2)
+    close(torch.cat(rows), full, dtype, "stepwise self-attention")
+    with pytest.raises(NotImplementedError):
+        attn(x[:2], None, None, None, incremental=True, incremental_cache=cache)       # two positions onto a filled cache
+    with pytest.raises(RuntimeError):
+        attn(x[:1], None, None, None, incremental=True, incremental_cache=None)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_cross_attention_with_cached_encoder_states(dev, dtype):
+    tq, tk, b, e, h = 7, 37, 3, 128, 4
+    g = torch.Generator().manual_seed(93)
+    attn = _randomise(EncdecMultiheadAttn(h, e, 0.1), 94).to(dev).to(dtype).eval()
+    q = torch.randn(tq, b, e, generator=g).to(dtype).to(dev)
+    ctxt = torch.randn(tk, b, e, generator=g).to(dtype).to(dev)
+    pad, _ = inputs.lengths_mask(b, tk, tk // 2, tk, g)
+    pad = pad.to(dev)
+    with torch.no_grad():
+        full, full_cov = attn(q, ctxt, ctxt, pad)
+        cache = {}
+        rows = []
+        for i in range(tq):
+            # after the first step the encoder states are not read again
+            kv = ctxt if i == 0 else torch.full_like(ctxt, float("nan"))
+            out, cov = attn(q[i:i + 1], kv, kv, pad, incremental=True, incremental_cache=cache)
+            rows.append(out)
+            close(cov, full_cov[:, i:i + 1], dtype, "stepwise coverage")
+        assert cache["c_k"].shape == (tk, b, e) and cache["c_v"].shape == (tk, b, e)
+    close(torch.cat(rows), full, dtype, "stepwise cross-attention")
+
+
+def test_decoder_layer_step_by_step_with_beam_reordering(dev):
+    dtype = torch.bfloat16
+    opt = SimpleNamespace(model_size=128, inner_size=256, n_heads=4, dropout=0.1, attn_dropout=0.1, variational_dropout=False,
+                          macaron=False, rezero=False, ffn_activation="gelu", ffn_glu=False, fast_self_attention=True,
+                          fast_xattention=True, fast_feed_forward=True, ignore_source=False)
+    tq, tk, b = 6, 20, 4
+    g = torch.Generator().manual_seed(95)
+    layer = _randomise(DecoderLayer(opt), 96).to(dev).to(dtype).eval()
+    x = torch.randn(tq, b, 128, generator=g).to(dtype).to(dev)
+    ctxt = torch.randn(tk, b, 128, generator=g).to(dtype).to(dev)
+    src_pad, _ = inputs.lengths_mask(b, tk, tk // 2, tk, g)
+    src_pad = src_pad.to(dev)
+    causal = torch.triu(torch.ones(tq, tq, device=dev), 1).bool()
+    perm = torch.tensor([2, 0, 3, 1], device=dev)
+    with torch.no_grad():
+        full, _, _ = layer(x, ctxt, causal, src_pad)
+        # the hypotheses are re-ordered after step 2: from then on batch entry j continues hypothesis perm[j]
+        x_after = x[:, perm]
+        full_after, _, _ = layer(torch.cat([x[:3][:, perm], x_after[3:]]), ctxt[:, perm], causal, src_pad[perm])
+        cache = None
+        rows = []
+        for i in range(tq):
+            if i == 3:
+                for key in cache:
+                    cache[key] = cache[key].index_select(1, perm)
+            cur_x = x[i:i + 1] if i < 3 else x_after[i:i + 1]
+            cur_ctxt, cur_pad = (ctxt, src_pad) if i < 3 else (ctxt[:, perm], src_pad[perm])
+            out, _, cache = layer(cur_x, cur_ctxt, causal[i:i + 1, :i + 1], cur_pad, incremental=True, incremental_cache=cache)
+            rows.append(out)
+        assert sorted(cache) == ["c_k", "c_v", "k", "v"]
+    close(torch.cat(rows[:3]), full[:3], dtype, "steps before the re-ordering")
+    close(torch.cat(rows[3:]), full_after[3:], dtype, "steps after the re-ordering")
