@@ -617,7 +617,8 @@ def main():
         "value": head["value"], "unit": head["unit"], "n_gpus": 1, "steps": head["steps"], "warmup": args.warmup,
         "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": head["dtype"], "data": head["data"],
-        "config": {"workload": head["description"], "timed": head["timed"]},
+        "config": {"workload": head["description"], "timed": head["timed"],
+                   "switches": {k: v for k, v in sorted(os.environ.items()) if k.startswith("NMTG_")}},
         "roofline": head["roofline"], "cpu_baseline": head["cpu_baseline"], "kernels": head["kernels"],
         "others": results[1:],
     }
