@@ -5,10 +5,15 @@ older `encdec_multihead_attn_bias_cuda` (multihead_attn/encdec_multihead_attn_bi
 
 Extras: any bias may be None (Whisper's key projection has none); fp16 and bf16; `forward` /
 `forward_compact` take an optional keyword `dropout_mask` to replay an explicit keep-mask."""
+import os
+
 import torch
 
 from .. import _lib as L
 from . import _attn_common as A
+from .linear_gemm import gemm
+
+KEY_BLOCK = 64      # the GEMM main loops move whole 64-element steps of the reduction dimension with 16-byte accesses
 
 
 def _shapes(q3, kv3, heads, kv_last):
@@ -39,6 +44,31 @@ def _fwd(is_training, heads, x_q, x_kv, w_q, w_kv, w_out, b_q, b_kv, b_out, q_li
     return q_lin, kv_lin, scores, dropped, dmask, ctx, out
 
 
+def _fwd_padded_keys(heads, x_q, x_kv, w_q, w_kv, w_out, b_q, b_kv, b_out, pad_mask, tq, tk, b, e):
+    """Inference forward for a key length that is not a multiple of 64 (Whisper's 1500 encoder frames): the projected
+    keys / values are written into a buffer of tk_pad = ceil(tk / 64) * 64 rows whose extra rows are zero and masked,
+    so that the score / probability rows are 16-byte aligned and the per-head products run their fast main loops
+    (with tk = 1500 every row of those tensors starts on an 8-byte boundary only, and the products over the keys end
+    in a partial step). Masked keys have probability exactly 0, so the results for the real keys are the same numbers;
+    the returned key/value projection, scores and probabilities are views of the padded buffers, cut back to tk."""
+    dev, dt = x_q.device, x_q.dtype
+    tk_pad = (tk + KEY_BLOCK - 1) // KEY_BLOCK * KEY_BLOCK
+    kv_lin = torch.empty(tk_pad, b, 2 * e, dtype=dt, device=dev)
+    kv_lin[tk:].zero_()
+    gemm(x_kv.view(tk * b, e), w_kv, False, True, bias=b_kv, out=kv_lin[:tk].view(tk * b, 2 * e))
+    q_lin = gemm(x_q.view(tq * b, e), w_q, False, True, bias=b_q).view(tq, b, e)
+    mask = torch.ones(b, tk_pad, dtype=torch.uint8, device=dev)
+    if pad_mask is not None and pad_mask.numel() > 0:
+        mask[:, :tk] = pad_mask.reshape(b, tk).to(torch.uint8)
+    else:
+        mask[:, :tk] = 0
+    r = _fwd(False, heads, None, None, None, None, None, None, None, None, q_lin, kv_lin, mask, 0.0, None, tq, tk_pad, b, e,
+             dev, dt)
+    scores, dropped, dmask, ctx = r[2], r[3], r[4], r[5]
+    out = gemm(ctx.view(tq * b, e), w_out, False, True, bias=b_out).view(tq, b, e)
+    return [q_lin, kv_lin[:tk], scores[:, :, :tk], dropped[:, :, :tk], dmask, ctx, out]
+
+
 def forward(is_training, heads, inputs_q, inputs_kv, input_weights_q, input_weights_kv, output_weights, input_biases_q,
             input_biases_kv, output_biases, pad_mask, dropout_prob, *, dropout_mask=None):
     """-> [input_lin_q_results, input_lin_kv_results, attn_scores, dropout_results, dropout_mask,
@@ -51,6 +81,10 @@ def forward(is_training, heads, inputs_q, inputs_kv, input_weights_q, input_weig
     A.check(input_weights_q.shape == (e, e) and input_weights_kv.shape == (2 * e, e) and output_weights.shape == (e, e),
             "weight shapes do not match the inputs")
     c = lambda z: z.contiguous() if z is not None else None
+    # switched on by NMTG_ATTN_PAD_KEYS=1 until it has been through the GPU test-suite and measured
+    if not is_training and tk % KEY_BLOCK != 0 and os.environ.get("NMTG_ATTN_PAD_KEYS") == "1":
+        return _fwd_padded_keys(heads, c(inputs_q), c(inputs_kv), c(input_weights_q), c(input_weights_kv), c(output_weights),
+                                c(input_biases_q), c(input_biases_kv), c(output_biases), pad_mask, tq, tk, b, e)
     return list(_fwd(is_training, heads, c(inputs_q), c(inputs_kv), c(input_weights_q), c(input_weights_kv),
                      c(output_weights), c(input_biases_q), c(input_biases_kv), c(output_biases), None, None, pad_mask,
                      dropout_prob, dropout_mask, tq, tk, b, e, inputs_q.device, inputs_q.dtype))
@@ -94,10 +128,14 @@ def _bwd(heads, output_grads, matmul2_results, dropout_results, attn_scores, q_l
                 n["dbo"] = torch.empty(e, dtype=dt, device=dev)
     ws_bytes = L.load().nmtg_encdec_attn_bwd_workspace_bytes(L.i64(tq), L.i64(tk), L.i64(b), L.i64(e), L.i32(heads))
     ws = A.workspace(ws_bytes, dev)
+    # contiguous copies (if any) are bound to names: a temporary would be freed before the kernels read it
     c = lambda z: z.contiguous() if z is not None else None
-    L.call("nmtg_encdec_attn_bwd", L.ptr(g), L.ptr(c(matmul2_results)), L.ptr(c(dropout_results)), L.ptr(c(attn_scores)),
-           L.ptr(c(q_lin)), L.ptr(c(kv_lin)), L.ptr(c(inputs_q)), L.ptr(c(inputs_kv)), L.ptr(c(w_q)), L.ptr(c(w_kv)),
-           L.ptr(c(w_out)), L.ptr(c(dropout_mask) if use_mask else None), L.f32(p), L.ptr(n["dxq"]), L.ptr(n["dxkv"]),
+    (matmul2_results, dropout_results, attn_scores, q_lin, kv_lin, inputs_q, inputs_kv, w_q, w_kv, w_out) = map(
+        c, (matmul2_results, dropout_results, attn_scores, q_lin, kv_lin, inputs_q, inputs_kv, w_q, w_kv, w_out))
+    dropout_mask = c(dropout_mask) if use_mask else None
+    L.call("nmtg_encdec_attn_bwd", L.ptr(g), L.ptr(matmul2_results), L.ptr(dropout_results), L.ptr(attn_scores),
+           L.ptr(q_lin), L.ptr(kv_lin), L.ptr(inputs_q), L.ptr(inputs_kv), L.ptr(w_q), L.ptr(w_kv),
+           L.ptr(w_out), L.ptr(dropout_mask), L.f32(p), L.ptr(n["dxq"]), L.ptr(n["dxkv"]),
            L.ptr(n["dwq"]), L.ptr(n["dwkv"]), L.ptr(n["dwo"]), L.ptr(n["dbq"]), L.ptr(n["dbkv"]), L.ptr(n["dbo"]),
            L.ptr(n["dq"]), L.ptr(n["dkv"]), L.ptr(ws), L.i64(ws.numel()), L.i64(tq), L.i64(tk), L.i64(b), L.i64(e),
            L.i32(heads), L.i32(L.dtype_code(g)), L.stream_of(g))

@@ -47,6 +47,7 @@ def backward(output_grads, dropout_add_mask, dropout_prob):
     _check(dropout_add_mask.dtype == torch.uint8 and dropout_add_mask.numel() == output_grads.numel(),
            "fused_dropout_add: mask must be uint8 with the gradient's size")
     dx = torch.empty_like(output_grads)
-    L.call("nmtg_dropout_add_bwd", L.ptr(output_grads), L.ptr(dropout_add_mask.contiguous()), L.ptr(dx),
+    dropout_add_mask = dropout_add_mask.contiguous()      # bound to a name: a temporary would be freed before the kernel reads it
+    L.call("nmtg_dropout_add_bwd", L.ptr(output_grads), L.ptr(dropout_add_mask), L.ptr(dx),
            L.i64(output_grads.numel()), L.f32(dropout_prob), L.i32(L.dtype_code(output_grads)), L.stream_of(output_grads))
     return dx

@@ -92,10 +92,14 @@ def _bwd(heads, output_grads, matmul2_results, dropout_results, attn_scores, inp
             db_out = torch.empty(e, dtype=dt, device=dev)
     ws_bytes = L.load().nmtg_self_attn_bwd_workspace_bytes(L.i64(t), L.i64(b), L.i64(e), L.i32(heads))
     ws = A.workspace(ws_bytes, dev)
+    # contiguous copies (if any) are bound to names: a temporary would be freed before the kernels read it
     c = lambda z: z.contiguous() if z is not None else None
-    L.call("nmtg_self_attn_bwd", L.ptr(g), L.ptr(c(matmul2_results)), L.ptr(c(dropout_results)), L.ptr(c(attn_scores)),
-           L.ptr(c(input_lin_results)), L.ptr(c(inputs)), L.ptr(c(input_weights)), L.ptr(c(output_weights)),
-           L.ptr(c(dropout_mask) if use_mask else None), L.f32(dropout_prob), L.ptr(dx), L.ptr(dw_in), L.ptr(dw_out),
+    (matmul2_results, dropout_results, attn_scores, input_lin_results, inputs, input_weights, output_weights) = map(
+        c, (matmul2_results, dropout_results, attn_scores, input_lin_results, inputs, input_weights, output_weights))
+    dropout_mask = c(dropout_mask) if use_mask else None
+    L.call("nmtg_self_attn_bwd", L.ptr(g), L.ptr(matmul2_results), L.ptr(dropout_results), L.ptr(attn_scores),
+           L.ptr(input_lin_results), L.ptr(inputs), L.ptr(input_weights), L.ptr(output_weights),
+           L.ptr(dropout_mask), L.f32(dropout_prob), L.ptr(dx), L.ptr(dw_in), L.ptr(dw_out),
            L.ptr(db_in), L.ptr(db_out), L.ptr(dlin), L.ptr(ws), L.i64(ws.numel()), L.i64(t), L.i64(b), L.i64(e),
            L.i32(heads), L.i32(L.dtype_code(g)), L.stream_of(g))
     return dx, dw_in, dw_out, db_in, db_out, dlin

@@ -52,7 +52,8 @@ def backward(grad_loss, logits, max_log_sum_exp, labels, smoothing, *, padding_i
     lse = max_log_sum_exp.contiguous().float()
     n, v = logits.shape
     grad_logits = torch.empty_like(logits)
-    L.call("nmtg_xentropy_bwd", L.ptr(grad_loss), L.ptr(logits), L.ptr(lse), L.ptr(labels.contiguous()),
+    labels = labels.contiguous()                          # bound to a name: a temporary would be freed before the kernel reads it
+    L.call("nmtg_xentropy_bwd", L.ptr(grad_loss), L.ptr(logits), L.ptr(lse), L.ptr(labels),
            L.ptr(grad_logits), L.i64(n), L.i64(v), L.f32(smoothing),
            L.i64(_NO_PAD if padding_idx is None else padding_idx), L.i32(L.dtype_code(logits)), L.stream_of(logits))
     return grad_logits

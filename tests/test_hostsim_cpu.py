@@ -393,6 +393,14 @@ def test_table_gelu(mi355x, dtype, tokens, dm, di, p):
     tst.test_table_gelu_matches_the_formula(CPU, dtype, tokens, dm, di, p)
 
 
+@pytest.mark.parametrize("dtype", HALVES)
+@pytest.mark.parametrize("tq,tk,b,e,h,masked", [(17, 100, 3, 128, 2, True), (8, 70, 2, 128, 2, False),
+                                                pytest.param(32, 1500, 2, 256, 4, True, marks=long_case)])
+def test_padded_keys(mi355x, dtype, tq, tk, b, e, h, masked):
+    # also the regression test for saved tensors that reach the backward as non-contiguous views
+    tst.test_padded_keys_give_the_same_cross_attention(CPU, dtype, tq, tk, b, e, h, masked)
+
+
 # ----------------------------------------------------------------------------- committed fixtures
 @pytest.mark.parametrize("name", [n for n in dir(tgold) if n.startswith("test_") and n != "test_mlp_fixture"])
 def test_golden_fixtures(mi355x, name):

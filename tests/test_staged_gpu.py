@@ -3,6 +3,8 @@ not been through the GPU test-suite yet:
 
   NMTG_GEMM_RING_S=1   the slot-ring main loop for the 256x64 tile (per-head products P V, dS K, Pd^T dC, dS^T Q)
   NMTG_ATTN_FUSED=1    Q K^T -> mask -> softmax -> dropout in one kernel (rows of up to 512 keys)
+  NMTG_ATTN_PAD_KEYS=1 inference cross-attention with a key length that is not a multiple of 64: keys / values padded
+                       with masked zero rows so that every tensor of the middle section is 16-byte aligned
   NMTG_GELU_LUT=1      gelu and its derivative in the MLP epilogues read from a 2049-entry table in LDS
 
 The library reads both switches on every call, so each test runs the default path and the staged
@@ -14,7 +16,7 @@ import os
 import pytest
 import torch
 
-from nmtgminor_amd.native import fused_mlp_gelu, self_multihead_attn_blaslt as sa_native
+from nmtgminor_amd.native import encdec_multihead_attn_bias_blaslt as ed_native, fused_mlp_gelu, self_multihead_attn_blaslt as sa_native
 from nmtgminor_amd.native.linear_gemm import gemm
 from oracle import attention as oat, inputs, mlp as omlp
 from util import assert_close
@@ -157,3 +159,39 @@ def test_table_gelu_matches_the_formula(dev, dtype, tokens, dm, di, p):
     assert_close(ggot[0], gx, dtype, "dx vs oracle", scale_atol=True)
     assert_close(ggot[1], gws[0], dtype, "dW1 vs oracle", scale_atol=True)
     assert_close(ggot[3], gbs[0], dtype, "db1 vs oracle", scale_atol=True)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("tq,tk,b,e,h,masked", [(17, 100, 3, 128, 2, True), (32, 1500, 2, 256, 4, True), (8, 70, 2, 128, 2, False)])
+def test_padded_keys_give_the_same_cross_attention(dev, dtype, tq, tk, b, e, h, masked):
+    d = inputs.encdec_attn_inputs(tq, tk, b, e, h, dtype, p=0.0, seed=96, zero_bias=False)
+    g = lambda k: d[k].to(dev) if d[k] is not None else None
+    pad = g("pad_mask") if masked else None
+    args = (False, h, g("x_q"), g("x_kv"), g("w_q"), g("w_kv"), g("w_out"), g("b_q"), g("b_kv"), g("b_out"), pad, 0.0)
+    ref = ed_native.forward(*args)
+    with switch("NMTG_ATTN_PAD_KEYS"):
+        got = ed_native.forward(*args)
+    names = ("q_lin", "kv_lin", "scores", "dropped", "dropout_mask", "context", "outputs")
+    assert got[2].shape == ref[2].shape == (b * h, tq, tk) and not got[2].is_contiguous()      # views of the padded rows
+    ulp = 2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7
+    for name, a_, r_ in zip(names, got, ref):
+        if name == "dropout_mask":
+            continue
+        if name in ("q_lin", "kv_lin", "scores"):
+            assert torch.equal(a_, r_), name         # the same products in the same order
+        else:
+            # masked keys carry probability exactly 0 and the padded value rows are 0; the softmax kernel sums a
+            # 1536-wide row with another lane assignment than a 1500-wide one, so a last bit may differ
+            assert_close(a_, r_.float().cpu(), dtype, name, rtol=2.1 * ulp, atol=1e-4)
+            assert torch.equal(a_ == 0, r_ == 0), name
+    fwd = oat.encdec_attn_fwd(d["x_q"], d["x_kv"], d["w_q"], d["w_kv"], d["w_out"], d["b_q"], d["b_kv"], d["b_out"], h,
+                              d["pad_mask"] if masked else None, 0.0, None, D, round_to=dtype)
+    assert_close(got[6], fwd["outputs"], dtype, "outputs vs oracle")
+    assert_close(got[3], fwd["dropout_results"], dtype, "probabilities vs oracle")
+    # the backward accepts the views (it copies them into the layout its kernels read)
+    grads = ed_native.backward(h, g("dout"), got[5], got[3], got[2], got[0], got[1], g("x_q"), g("x_kv"), g("w_q"), g("w_kv"),
+                               g("w_out"), None, 0.0)
+    want = ed_native.backward(h, g("dout"), ref[5], ref[3], ref[2], ref[0], ref[1], g("x_q"), g("x_kv"), g("w_q"), g("w_kv"),
+                              g("w_out"), None, 0.0)
+    for a_, r_ in zip(grads, want):
+        assert_close(a_, r_.float().cpu(), dtype, "gradients from the views", rtol=4 * ulp, atol=2e-3, scale_atol=True)
