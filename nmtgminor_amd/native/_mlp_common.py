@@ -101,9 +101,13 @@ def backward(act, p, grad_o, post, pre, mask, inputs, input_only=False, need_dx=
     ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
     use_mask = mask is not None and mask.numel() > 0 and p > 0.0
     have_pre = pre is not None and pre.numel() > 0
+    # the saved buffers are read as dense arrays: a strided view is copied (and the copy bound to a name, so that it
+    # lives until the kernels have been queued)
+    post = post.contiguous() if post is not None and post.numel() else None
+    pre = pre.contiguous() if have_pre else None
+    mask = mask.contiguous() if use_mask else None
     L.call("nmtg_mlp_bwd", L.i32(n), L.ptr(x2), _ptr_array(weights), of, L.i64(batch), L.i64(in_f), L.ptr(g2),
-           L.ptr(post if post is not None and post.numel() else None), L.ptr(pre if have_pre else None),
-           L.ptr(mask if use_mask else None), L.f32(p), L.i32(L.ACT_CODES[act]), L.ptr(dx), _ptr_array(dws),
+           L.ptr(post), L.ptr(pre), L.ptr(mask), L.f32(p), L.i32(L.ACT_CODES[act]), L.ptr(dx), _ptr_array(dws),
            _ptr_array(dbs), L.ptr(ws), L.i64(ws.numel()), L.i32(L.dtype_code(x)), L.stream_of(x))
     dx_out = dx.view(x.shape) if dx is not None else None
     if input_only:
