@@ -119,6 +119,11 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
   // NMTG_GEMM_TILE=0|1|2 (256x256 | 128x128 | 256x64) overrides the tile choice: a tuning aid.
   static const int forced_tile = [] { const char* e = getenv("NMTG_GEMM_TILE"); return e ? atoi(e) : -1; }();
   if (tile < 0 && forced_tile >= 0 && gemm_has(layout, forced_tile, epi) && (forced_tile != TILE_L || vec == 8)) tile = forced_tile;
+  // NMTG_GEMM_ACT_TILE=1 (read per call): the activation epilogues take the 128x128 tile, of which two blocks share a
+  // CU, so that one block's (VALU-bound) epilogue overlaps the other's main loop. Off until measured.
+  if (tile < 0 && (epi == EPI_ACT_FWD || epi == EPI_ACT_BWD) && gemm_has(layout, TILE_M, epi) &&
+      getenv("NMTG_GEMM_ACT_TILE") != nullptr)
+    tile = TILE_M;
   if (tile < 0) {
     const int cus = num_cus();
     const int64_t cnt_l = static_cast<int64_t>(ceil_div(a.M, 256)) * ceil_div(a.N, 256) * a.batch;

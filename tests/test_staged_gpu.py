@@ -5,6 +5,7 @@ not been through the GPU test-suite yet:
   NMTG_ATTN_FUSED=1    Q K^T -> mask -> softmax -> dropout in one kernel (rows of up to 512 keys)
   NMTG_ATTN_PAD_KEYS=1 inference cross-attention with a key length that is not a multiple of 64: keys / values padded
                        with masked zero rows so that every tensor of the middle section is 16-byte aligned
+  NMTG_GEMM_ACT_TILE=1 the activation epilogues of the MLP on the 128x128 tile (two blocks per CU) instead of 256x256
   NMTG_GELU_LUT=1      gelu and its derivative in the MLP epilogues read from a 2049-entry table in LDS
 
 The library reads both switches on every call, so each test runs the default path and the staged
@@ -195,3 +196,34 @@ def test_padded_keys_give_the_same_cross_attention(dev, dtype, tq, tk, b, e, h, 
                               g("w_out"), None, 0.0)
     for a_, r_ in zip(grads, want):
         assert_close(a_, r_.float().cpu(), dtype, "gradients from the views", rtol=4 * ulp, atol=2e-3, scale_atol=True)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("act", ["gelu", "relu"])
+def test_activation_epilogues_on_the_small_tile(dev, dtype, act):
+    # a shape whose activation GEMMs take the 256x256 tile by default: 16 x 12 tiles of 256 x 256 >= 3/4 of the 256 CUs
+    from nmtgminor_amd.native import fused_mlp_relu
+    tokens, dm, di, p = 4096, 128, 3072, 0.1
+    d = inputs.mlp_inputs(tokens, dm, di, dtype, p=p, seed=97, zero_bias=False)
+    ins = [d[k].to(dev) for k in ("x", "w1", "w2", "b1", "b2")]
+    ins[0].requires_grad_()
+    mask, dy = d["mask"].to(dev), d["dy"].to(dev)
+    if act == "gelu":
+        fwd = lambda: fused_mlp_gelu.forward(p, ins, mask)
+        bwd = lambda out: fused_mlp_gelu.backward(p, dy, out, ins)
+    else:
+        fwd = lambda: fused_mlp_relu.forward(p, True, ins, mask)
+        bwd = lambda out: fused_mlp_relu.backward(p, dy, out, ins)
+    ref = fwd()
+    gref = bwd(ref)
+    with switch("NMTG_GEMM_ACT_TILE"):
+        got = fwd()
+        ggot = bwd(ref)
+    # another blocking of the same products: every element is the same sum in the same order ...
+    for a_, r_ in zip(list(got) + list(ggot[:3]), list(ref) + list(gref[:3])):
+        if a_ is not None and a_.numel():
+            assert torch.equal(a_, r_)
+    # ... except the first layer's bias gradient, whose partial sums are taken per row tile (128 instead of 256 rows)
+    ulp = 2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7
+    for a_, r_ in zip(ggot[3:], gref[3:]):
+        assert_close(a_, r_.float().cpu(), dtype, "bias gradients", rtol=1.05 * ulp, atol=1e-4)
