@@ -72,6 +72,8 @@ struct GemmArgs {
   uint64_t seed, offset;
   int act;
   int act_lut;              // gelu / gelu' through the LDS table (ring kernels only; set by the host on request)
+  int defer_reduce;         // host only: a split-K call leaves its reduction to the caller (who queues it in a ReduceTail)
+  int tile_used;            // host only, filled by gemm_run: the tile the call ran with
   float* colsum_part;
   const uint8_t* kmask;
   int kmask_kind, heads;
@@ -947,7 +949,9 @@ size_t gemm_splitk_workspace_bytes(int M, int N, int K, int batch);
 // may split K. Returns 0 or a negative nmtg_status; *m_tiles_out receives the number of row tiles
 // used (= rows of colsum_part written by EPI_ACT_BWD).
 int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t workspace_bytes, hipStream_t st,
-             int* m_tiles_out = nullptr);
+             int* m_tiles_out = nullptr, GemmArgs* planned_out = nullptr);
+// planned_out (optional) receives the arguments as launched (splits, tiles, vec, ws, tile_used): with a.defer_reduce
+// set and planned_out->splits > 1 the caller owes the reduction of the partials (tail_add_splitk).
 
 // Fused Q K^T -> mask -> softmax -> dropout (EPI_SCORES_SOFTMAX) for rows of at most 512 keys. `a` is filled as
 // for EPI_SCORES plus out2 (dropped probabilities), aux_out (softmax, optional), dmask / rng / keep_p / dscale /

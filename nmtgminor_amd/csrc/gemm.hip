@@ -72,7 +72,7 @@ size_t gemm_splitk_workspace_bytes(int M, int N, int K, int batch) {
 }
 
 int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t workspace_bytes, hipStream_t st,
-             int* m_tiles_out) {
+             int* m_tiles_out, GemmArgs* planned_out) {
   if (m_tiles_out) *m_tiles_out = 0;
   if (a.M <= 0 || a.N <= 0 || a.batch <= 0) return 0;
   if (a.K < 0) return fail(NMTG_ERR_INVALID, "gemm: negative K");
@@ -160,6 +160,9 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
     return fail(NMTG_ERR_UNSUPPORTED, "gemm: grid too large (tiles %d x %d, batch %d)", a.m_tiles, a.n_tiles, a.batch);
   if (epi == EPI_SPLITK && a.ws == nullptr)
     return fail(NMTG_ERR_INVALID, "gemm: the split-K epilogue needs a workspace");
+  a.tile_used = tile;
+  if (epi != EPI_SPLITK) a.defer_reduce = 0;
+  if (planned_out) *planned_out = a;
   int rc;
   if (layout == LAYOUT_NT) rc = gemm_launch_nt(dtype, tile, epi, a, st);
   else if (layout == LAYOUT_NN) rc = gemm_launch_nn(dtype, tile, epi, a, st);

@@ -11,13 +11,7 @@
 
 namespace nmtg {
 
-enum GemmTile { TILE_L = 0, TILE_M = 1, TILE_S = 2, TILE_R = 3 };
-
-template <int TILE> struct tile_cfg;
-template <> struct tile_cfg<TILE_L> { static constexpr int BM = 256, BN = 256, WM = 2, WN = 4; };
-template <> struct tile_cfg<TILE_M> { static constexpr int BM = 128, BN = 128, WM = 2, WN = 2; };
-template <> struct tile_cfg<TILE_S> { static constexpr int BM = 256, BN = 64, WM = 4, WN = 1; };
-template <> struct tile_cfg<TILE_R> { static constexpr int BM = 128, BN = 512, WM = 4, WN = 2; };
+// GemmTile and tile_cfg<TILE> (block tile and wavefront grid of each tile) live in reduce.cuh: the reduction kernels need them too.
 
 inline void tile_dims(int tile, int& bm, int& bn) {
   if (tile == TILE_L) { bm = 256; bn = 256; }

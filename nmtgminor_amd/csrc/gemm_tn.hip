@@ -7,8 +7,8 @@ template <typename T> static int run(int tile, int epi, const GemmArgs& a, hipSt
   CASE(TILE_M, EPI_PLAIN) CASE(TILE_S, EPI_PLAIN)
   if (epi == EPI_SPLITK) {
     int rc = NMTG_ERR_UNSUPPORTED;
-    if (tile == TILE_L) { rc = gemm_launch_one<T, TILE_L, false, false, EPI_SPLITK>(a, st); if (!rc) rc = splitk_reduce_launch<T, TILE_L>(a, st); return rc; }
-    if (tile == TILE_M) { rc = gemm_launch_one<T, TILE_M, false, false, EPI_SPLITK>(a, st); if (!rc) rc = splitk_reduce_launch<T, TILE_M>(a, st); return rc; }
+    if (tile == TILE_L) { rc = gemm_launch_one<T, TILE_L, false, false, EPI_SPLITK>(a, st); if (!rc && !a.defer_reduce) rc = splitk_reduce_launch<T, TILE_L>(a, st); return rc; }
+    if (tile == TILE_M) { rc = gemm_launch_one<T, TILE_M, false, false, EPI_SPLITK>(a, st); if (!rc && !a.defer_reduce) rc = splitk_reduce_launch<T, TILE_M>(a, st); return rc; }
   }
   return fail(NMTG_ERR_UNSUPPORTED, "gemm TN: no kernel for tile %d epilogue %d", tile, epi);
 }

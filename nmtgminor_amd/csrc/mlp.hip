@@ -16,6 +16,7 @@
 // tensors; here those tensors cross HBM once per direction.
 #include "gemm.cuh"
 #include <algorithm>
+#include <cstdlib>
 #include <vector>
 
 namespace nmtg {
@@ -27,13 +28,16 @@ size_t align_up(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
 
 struct BwdPlan {
   size_t dh_bytes;       // one dh buffer [batch, max hidden] (two are used, ping-pong)
-  size_t colsum_bytes;   // fp32 partials for bias gradients
+  size_t colsum_bytes;   // fp32 partials for one layer's bias gradient
   size_t splitk_bytes;   // largest weight-gradient split-K workspace
-  size_t total() const { return 2 * dh_bytes + colsum_bytes + splitk_bytes; }
+  int layers;
+  // one column-sum and one split-K region per layer: with the reductions deferred to one launch at the end
+  // (NMTG_MLP_TAIL) every layer's partials stay alive until then
+  size_t total() const { return 2 * dh_bytes + layers * (colsum_bytes + splitk_bytes); }
 };
 
 BwdPlan plan_bwd(int num_layers, const int64_t* out_features, int64_t batch, int64_t in_features) {
-  BwdPlan p{0, 0, 0};
+  BwdPlan p{0, 0, 0, num_layers};
   int64_t max_hidden = 0, max_out = 0;
   for (int i = 0; i < num_layers; ++i) {
     if (i < num_layers - 1) max_hidden = std::max(max_hidden, out_features[i]);
@@ -146,8 +150,16 @@ extern "C" int nmtg_mlp_bwd(int num_layers, const void* x, const void* const* we
   NMTG_REQUIRE(batch == 0 || (x && grad_out), "mlp_bwd: null pointer argument");
   uint8_t* wsb = static_cast<uint8_t*>(workspace);
   void* dh[2] = {wsb, wsb + plan.dh_bytes};
-  float* colsum_ws = reinterpret_cast<float*>(wsb + 2 * plan.dh_bytes);
-  void* splitk_ws = wsb + 2 * plan.dh_bytes + plan.colsum_bytes;
+  // NMTG_MLP_TAIL=1 (read per call; off until validated on the GPU and measured): the split-K reductions and the final
+  // bias-gradient sums of all layers run as one launch at the end instead of two launches per layer
+  const bool tail_mode = getenv("NMTG_MLP_TAIL") != nullptr;
+  ReduceTail tail;
+  auto colsum_region = [&](int layer) {
+    return reinterpret_cast<float*>(wsb + 2 * plan.dh_bytes + (tail_mode ? layer : 0) * plan.colsum_bytes);
+  };
+  auto splitk_region = [&](int layer) {
+    return static_cast<void*>(wsb + 2 * plan.dh_bytes + plan.layers * plan.colsum_bytes + (tail_mode ? layer : 0) * plan.splitk_bytes);
+  };
 
   // element offsets of each hidden layer inside the concatenated buffers
   int64_t offs[MAX_LAYERS] = {0};
@@ -161,10 +173,22 @@ extern "C" int nmtg_mlp_bwd(int num_layers, const void* x, const void* const* we
     const int64_t in_i = i == 0 ? in_features : out_features[i - 1];
     const void* input_i = i == 0 ? x : static_cast<const uint8_t*>(post_acts) + offs[i - 1] * 2;
     int rc;
-    // bias gradient
+    // bias gradient (its partial rows: written by the data-gradient GEMM of the layer above, or by a kernel of its own)
+    float* colsum_ws = colsum_region(i);
     if (grad_biases && grad_biases[i]) {
-      if (bias_from_parts) rc = colsum_finish(dtype, colsum_ws, parts_rows, static_cast<int>(out_i), grad_biases[i], st);
-      else rc = colsum_run(dtype, g_cur, out_i, static_cast<int>(batch), static_cast<int>(out_i), colsum_ws, grad_biases[i], st);
+      if (tail_mode && !tail.full()) {
+        int parts = parts_rows;
+        rc = 0;
+        if (!bias_from_parts) {
+          parts = colsum_parts(static_cast<int>(batch));
+          rc = colsum_partial_run(dtype, g_cur, out_i, static_cast<int>(batch), static_cast<int>(out_i), colsum_ws, st);
+        }
+        if (!rc) rc = tail_add_colsum(tail, colsum_ws, parts, static_cast<int>(out_i), grad_biases[i]);
+      } else if (bias_from_parts) {
+        rc = colsum_finish(dtype, colsum_ws, parts_rows, static_cast<int>(out_i), grad_biases[i], st);
+      } else {
+        rc = colsum_run(dtype, g_cur, out_i, static_cast<int>(batch), static_cast<int>(out_i), colsum_ws, grad_biases[i], st);
+      }
       if (rc) return rc;
     }
     // weight gradient: dW_i [out_i, in_i] = g^T input
@@ -175,7 +199,12 @@ extern "C" int nmtg_mlp_bwd(int num_layers, const void* x, const void* const* we
       g.C = grad_weights[i]; g.ldc = in_i;
       g.M = static_cast<int>(out_i); g.N = static_cast<int>(in_i); g.K = static_cast<int>(batch);
       g.batch = 1; g.alpha = 1.f;
-      rc = gemm_run(dtype, LAYOUT_TN, EPI_PLAIN, g, splitk_ws, plan.splitk_bytes, st);
+      g.defer_reduce = (tail_mode && !tail.full()) ? 1 : 0;
+      GemmArgs planned{};
+      rc = gemm_run(dtype, LAYOUT_TN, EPI_PLAIN, g, splitk_region(i), plan.splitk_bytes, st, nullptr, &planned);
+      if (!rc && planned.defer_reduce && planned.splits > 1)
+        rc = tail_add_splitk(tail, planned.tile_used, planned.ws, planned.C, planned.ldc, planned.M, planned.N, planned.m_tiles,
+                             planned.n_tiles, planned.batch, planned.sC, planned.splits, planned.alpha, planned.vec);
       if (rc) return rc;
     }
     // data gradient
@@ -198,7 +227,7 @@ extern "C" int nmtg_mlp_bwd(int num_layers, const void* x, const void* const* we
         g.dscale = 1.f / (1.f - p);  // relu from the dropped output: a > 0 iff kept and h > 0
       }
       // one partial row per row tile of the GEMM
-      g.colsum_part = (grad_biases && grad_biases[i - 1]) ? colsum_ws : nullptr;
+      g.colsum_part = (grad_biases && grad_biases[i - 1]) ? colsum_region(i - 1) : nullptr;
       rc = gemm_run(dtype, LAYOUT_NN, EPI_ACT_BWD, g, nullptr, 0, st, &parts_rows);
       if (rc) return rc;
       bias_from_parts = g.colsum_part != nullptr;
@@ -214,5 +243,5 @@ extern "C" int nmtg_mlp_bwd(int num_layers, const void* x, const void* const* we
       if (rc) return rc;
     }
   }
-  return 0;
+  return tail_launch(tail, dtype, st);
 }

@@ -9,15 +9,14 @@ namespace nmtg {
 // Sums the split-K partials (in the accumulator layout the GEMM kernels' split-K epilogue writes, gemm.cuh), scales, converts to T and
 // writes row-major C; fixed summation order.
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N>
-__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, T* __restrict__ C, int64_t ldc,
-                                                            int M, int N, int m_tiles, int n_tiles, int batch,
-                                                            int64_t sC, int splits, float alpha, int c_vec) {
+__device__ __forceinline__ void splitk_reduce_slot(int64_t idx, const float* __restrict__ ws, T* __restrict__ C, int64_t ldc,
+                                                   int M, int N, int m_tiles, int n_tiles, int batch, int64_t sC, int splits,
+                                                   float alpha, int c_vec) {
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
   constexpr int TM = WTM / 32, TN = WTN / 32;
   constexpr int PER_BLK = NW * TM * TN * 4 * 64;  // float4 slots per tile
   const int64_t total = static_cast<int64_t>(batch) * m_tiles * n_tiles * PER_BLK;
-  const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
   if (idx >= total) return;
   const int lane = idx & 63;
   int64_t t = idx >> 6;
@@ -50,6 +49,14 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
   T* dst = C + static_cast<int64_t>(bz) * sC + static_cast<int64_t>(m) * ldc + n;
   if (n + 4 <= N && c_vec >= 4) store_pack<T, 4>(dst, v);
   else for (int e = 0; e < 4 && n + e < N; ++e) dst[e] = elem<T>::from_float(v[e]);
+}
+
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, T* __restrict__ C, int64_t ldc,
+                                                            int M, int N, int m_tiles, int n_tiles, int batch,
+                                                            int64_t sC, int splits, float alpha, int c_vec) {
+  splitk_reduce_slot<T, BM, BN, WAVES_M, WAVES_N>(static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x, ws, C, ldc, M, N, m_tiles,
+                                                  n_tiles, batch, sC, splits, alpha, c_vec);
 }
 
 // Column sums of a row-major [M, N] matrix: partial[mb][n] over row blocks (fp32), fixed order.
@@ -119,9 +126,7 @@ __global__ __launch_bounds__(256) void colsum_partial_kernel(const T* __restrict
 
 // out[n] = T(sum_p part[p][n]) in order p = 0..parts-1; 8 partial rows in flight per thread.
 template <typename T>
-__global__ __launch_bounds__(256) void colsum_final_kernel(const float* __restrict__ part, int parts, int N,
-                                                           T* __restrict__ out) {
-  const int n = blockIdx.x * 256 + threadIdx.x;
+__device__ __forceinline__ void colsum_final_column(int n, const float* __restrict__ part, int parts, int N, T* __restrict__ out) {
   if (n >= N) return;
   float s = 0.f;
   int p = 0;
@@ -143,6 +148,75 @@ __global__ __launch_bounds__(256) void colsum_final_kernel(const float* __restri
   for (; p < parts; ++p) s += part[static_cast<int64_t>(p) * N + n];
   out[n] = elem<T>::from_float(s);
 }
+
+template <typename T>
+__global__ __launch_bounds__(256) void colsum_final_kernel(const float* __restrict__ part, int parts, int N,
+                                                           T* __restrict__ out) {
+  colsum_final_column<T>(blockIdx.x * 256 + threadIdx.x, part, parts, N, out);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Several of the reductions above in one launch: an operator that ends in a handful of them (the MLP backward: two
+// split-K reductions and two bias-gradient sums) queues them as jobs and runs one kernel at its end instead of
+// four launches of a few microseconds each. A block finds its job from the block ranges (uniform per block) and
+// then does exactly what the stand-alone kernel's block would have done: results are bit-identical.
+// ---------------------------------------------------------------------------------------------
+enum GemmTile { TILE_L = 0, TILE_M = 1, TILE_S = 2, TILE_R = 3 };
+
+template <int TILE> struct tile_cfg;
+template <> struct tile_cfg<TILE_L> { static constexpr int BM = 256, BN = 256, WM = 2, WN = 4; };
+template <> struct tile_cfg<TILE_M> { static constexpr int BM = 128, BN = 128, WM = 2, WN = 2; };
+template <> struct tile_cfg<TILE_S> { static constexpr int BM = 256, BN = 64, WM = 4, WN = 1; };
+template <> struct tile_cfg<TILE_R> { static constexpr int BM = 128, BN = 512, WM = 4, WN = 2; };
+
+enum TailKind { TAIL_SPLITK_M = 1, TAIL_SPLITK_L = 2, TAIL_COLSUM = 3 };
+struct TailJob {
+  int kind;
+  int first_block;       // the job's blocks are [first_block, next job's first_block)
+  const float* src;      // split-K partials / column-sum partial rows
+  void* dst;
+  int64_t ldc, sC;
+  int M, N, m_tiles, n_tiles, batch, splits, c_vec, parts;
+  float alpha;
+};
+constexpr int TAIL_MAX_JOBS = 8;
+struct TailArgs {
+  int njobs;
+  TailJob job[TAIL_MAX_JOBS];
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void reduce_tail_kernel(const TailArgs a) {
+  int j = 0;
+  while (j + 1 < a.njobs && static_cast<int>(blockIdx.x) >= a.job[j + 1].first_block) ++j;
+  const TailJob& t = a.job[j];
+  const int64_t local = static_cast<int64_t>(blockIdx.x - t.first_block) * 256 + threadIdx.x;
+  if (t.kind == TAIL_SPLITK_M) {
+    using C = tile_cfg<TILE_M>;
+    splitk_reduce_slot<T, C::BM, C::BN, C::WM, C::WN>(local, t.src, static_cast<T*>(t.dst), t.ldc, t.M, t.N, t.m_tiles, t.n_tiles,
+                                                      t.batch, t.sC, t.splits, t.alpha, t.c_vec);
+  } else if (t.kind == TAIL_SPLITK_L) {
+    using C = tile_cfg<TILE_L>;
+    splitk_reduce_slot<T, C::BM, C::BN, C::WM, C::WN>(local, t.src, static_cast<T*>(t.dst), t.ldc, t.M, t.N, t.m_tiles, t.n_tiles,
+                                                      t.batch, t.sC, t.splits, t.alpha, t.c_vec);
+  } else if (t.kind == TAIL_COLSUM) {
+    colsum_final_column<T>(static_cast<int>(local), t.src, t.parts, t.N, static_cast<T*>(t.dst));
+  }
+}
+
+// Host side (reduce.hip): a list of jobs of one dtype, launched once.
+struct ReduceTail {
+  TailArgs args;
+  int blocks;
+  ReduceTail() : blocks(0) { args.njobs = 0; }
+  bool full() const { return args.njobs >= TAIL_MAX_JOBS; }
+};
+int tail_add_splitk(ReduceTail& t, int tile, const float* ws, void* C, int64_t ldc, int M, int N, int m_tiles, int n_tiles,
+                    int batch, int64_t sC, int splits, float alpha, int c_vec);
+int tail_add_colsum(ReduceTail& t, const float* part, int parts, int N, void* out);
+int tail_launch(const ReduceTail& t, int dtype, hipStream_t st);
+// the partial phase of colsum_run alone (its final sum is then queued with tail_add_colsum)
+int colsum_partial_run(int dtype, const void* X, int64_t ld, int M, int N, float* part, hipStream_t st);
 
 // bias-gradient style column sums: out[n] = sum_m X[m][n]; part is fp32 scratch of
 // colsum_parts(M) * N floats.

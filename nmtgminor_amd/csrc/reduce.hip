@@ -18,7 +18,7 @@ int colsum_finish(int dtype, const float* part, int parts, int N, void* out, hip
   return 0;
 }
 
-int colsum_run(int dtype, const void* X, int64_t ld, int M, int N, float* part, void* out, hipStream_t st) {
+int colsum_partial_run(int dtype, const void* X, int64_t ld, int M, int N, float* part, hipStream_t st) {
   const int parts = colsum_parts(M);
   const int rpb = ceil_div(M, parts);
   {
@@ -35,7 +35,51 @@ int colsum_run(int dtype, const void* X, int64_t ld, int M, int N, float* part, 
     }
   }
   NMTG_CHECK_LAUNCH("colsum");
-  return colsum_finish(dtype, part, parts, N, out, st);
+  return 0;
+}
+
+int colsum_run(int dtype, const void* X, int64_t ld, int M, int N, float* part, void* out, hipStream_t st) {
+  if (int rc = colsum_partial_run(dtype, X, ld, M, N, part, st)) return rc;
+  return colsum_finish(dtype, part, colsum_parts(M), N, out, st);
+}
+
+// ---- several reductions in one launch ----
+int tail_add_splitk(ReduceTail& t, int tile, const float* ws, void* C, int64_t ldc, int M, int N, int m_tiles, int n_tiles,
+                    int batch, int64_t sC, int splits, float alpha, int c_vec) {
+  if (t.full() || (tile != TILE_M && tile != TILE_L)) return fail(NMTG_ERR_UNSUPPORTED, "reduce tail: cannot queue this split-K job");
+  const int bm = tile == TILE_M ? 128 : 256;
+  const int64_t slots = static_cast<int64_t>(batch) * m_tiles * n_tiles * (static_cast<int64_t>(bm) * bm / 4);   // one float4 slot per 4 outputs
+  const int64_t blocks = (slots + 255) / 256;
+  if (blocks <= 0 || t.blocks + blocks > 0x7fffffff) return fail(NMTG_ERR_UNSUPPORTED, "reduce tail: grid too large");
+  TailJob& j = t.args.job[t.args.njobs++];
+  j = TailJob{};
+  j.kind = tile == TILE_M ? TAIL_SPLITK_M : TAIL_SPLITK_L;
+  j.first_block = t.blocks;
+  j.src = ws; j.dst = C; j.ldc = ldc; j.sC = sC;
+  j.M = M; j.N = N; j.m_tiles = m_tiles; j.n_tiles = n_tiles; j.batch = batch; j.splits = splits; j.c_vec = c_vec;
+  j.alpha = alpha;
+  t.blocks += static_cast<int>(blocks);
+  return 0;
+}
+
+int tail_add_colsum(ReduceTail& t, const float* part, int parts, int N, void* out) {
+  if (t.full()) return fail(NMTG_ERR_UNSUPPORTED, "reduce tail: too many jobs");
+  TailJob& j = t.args.job[t.args.njobs++];
+  j = TailJob{};
+  j.kind = TAIL_COLSUM;
+  j.first_block = t.blocks;
+  j.src = part; j.dst = out; j.parts = parts; j.N = N;
+  t.blocks += ceil_div(N, 256);
+  return 0;
+}
+
+int tail_launch(const ReduceTail& t, int dtype, hipStream_t st) {
+  if (t.args.njobs == 0 || t.blocks == 0) return 0;
+  TraceScope trace("reduce_tail", st);
+  NMTG_DISPATCH_DTYPE(dtype, T,
+                      hipLaunchKernelGGL((reduce_tail_kernel<T>), dim3(static_cast<unsigned>(t.blocks)), dim3(256), 0, st, t.args));
+  NMTG_CHECK_LAUNCH("reduce_tail");
+  return 0;
 }
 
 }  // namespace nmtg

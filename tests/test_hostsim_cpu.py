@@ -408,6 +408,17 @@ def test_padded_keys(mi355x, dtype, tq, tk, b, e, h, masked):
     tst.test_padded_keys_give_the_same_cross_attention(CPU, dtype, tq, tk, b, e, h, masked)
 
 
+@pytest.mark.parametrize("dtype", HALVES)
+@pytest.mark.parametrize("tokens,dm,di", [(4096, 128, 256), pytest.param(1000, 192, 448, marks=long_case)])
+def test_mlp_backward_with_one_reduction_launch(mi355x, dtype, tokens, dm, di):
+    tst.test_mlp_backward_with_one_reduction_launch(CPU, dtype, tokens, dm, di)
+
+
+@long_case
+def test_three_layer_mlp_backward_with_one_reduction_launch(mi355x):
+    tst.test_three_layer_mlp_backward_with_one_reduction_launch(CPU)
+
+
 # ----------------------------------------------------------------------------- committed fixtures
 @pytest.mark.parametrize("name", [n for n in dir(tgold) if n.startswith("test_") and n != "test_mlp_fixture"])
 def test_golden_fixtures(mi355x, name):

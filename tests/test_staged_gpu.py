@@ -6,6 +6,7 @@ not been through the GPU test-suite yet:
   NMTG_ATTN_PAD_KEYS=1 inference cross-attention with a key length that is not a multiple of 64: keys / values padded
                        with masked zero rows so that every tensor of the middle section is 16-byte aligned
   NMTG_GEMM_ACT_TILE=1 the activation epilogues of the MLP on the 128x128 tile (two blocks per CU) instead of 256x256
+  NMTG_MLP_TAIL=1      the MLP backward's split-K reductions and bias-gradient sums as one launch at its end
   NMTG_GELU_LUT=1      gelu and its derivative in the MLP epilogues read from a 2049-entry table in LDS
 
 The library reads both switches on every call, so each test runs the default path and the staged
@@ -227,3 +228,40 @@ def test_activation_epilogues_on_the_small_tile(dev, dtype, act):
     ulp = 2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7
     for a_, r_ in zip(ggot[3:], gref[3:]):
         assert_close(a_, r_.float().cpu(), dtype, "bias gradients", rtol=1.05 * ulp, atol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("tokens,dm,di", [(4096, 128, 256), (1000, 192, 448), (8192, 512, 2048)])
+def test_mlp_backward_with_one_reduction_launch(dev, dtype, tokens, dm, di):
+    # NMTG_MLP_TAIL=1: split-K reductions and bias-gradient sums of all layers in one launch at the end
+    p = 0.1
+    d = inputs.mlp_inputs(tokens, dm, di, dtype, p=p, seed=98, zero_bias=False)
+    ins = [d[k].to(dev) for k in ("x", "w1", "w2", "b1", "b2")]
+    ins[0].requires_grad_()
+    mask, dy = d["mask"].to(dev), d["dy"].to(dev)
+    out = fused_mlp_gelu.forward(p, ins, mask)
+    want = fused_mlp_gelu.backward(p, dy, out, ins)
+    with switch("NMTG_MLP_TAIL"):
+        got = fused_mlp_gelu.backward(p, dy, out, ins)
+        only_dx = fused_mlp_gelu.backward_input_only(p, dy, out, ins)
+    for a_, r_ in zip(got, want):
+        assert torch.equal(a_, r_)                   # the same blocks do the same sums, only launched together
+    assert torch.equal(only_dx[0], want[0])
+
+
+def test_three_layer_mlp_backward_with_one_reduction_launch(dev):
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(99)
+    tokens, sizes = 2048, (96, 320, 160, 64)
+    x = torch.randn(tokens, sizes[0], generator=g).to(dtype).to(dev).requires_grad_()
+    ws = [(0.05 * torch.randn(sizes[i + 1], sizes[i], generator=g)).to(dtype).to(dev) for i in range(3)]
+    bs = [(0.1 * torch.randn(sizes[i + 1], generator=g)).to(dtype).to(dev) for i in range(3)]
+    dy = torch.randn(tokens, sizes[-1], generator=g).to(dtype).to(dev)
+    ins = [x] + ws + bs
+    out = fused_mlp_gelu.forward(0.0, ins)
+    want = fused_mlp_gelu.backward(0.0, dy, out, ins)
+    with switch("NMTG_MLP_TAIL"):
+        got = fused_mlp_gelu.backward(0.0, dy, out, ins)
+    assert len(got) == 7
+    for a_, r_ in zip(got, want):
+        assert torch.equal(a_, r_)
