@@ -582,6 +582,10 @@ def main():
     ap.add_argument("--workload", default="all", help="one of %s, or all" % ", ".join(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--trace-steps", type=int, default=10)
+    ap.add_argument("--variants", default="",
+                    help="semicolon-separated sets of per-call library switches to time after the default configuration, "
+                         "e.g. 'NMTG_GELU_LUT;NMTG_GELU_LUT+NMTG_GEMM_ACT_TILE'. Each set is exported as NAME=1 for one "
+                         "extra measurement of every selected workload (no CPU baseline); results go to 'variants'.")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.stderr.write("bench.py measures one GPU: this build has no multi-GPU path (each op is independent per "
@@ -611,6 +615,30 @@ def main():
         results[-1]["steps"] = steps
         del w
         torch.cuda.empty_cache()
+    # per-call switches of the library (staged kernel variants): the same workloads again under each requested set
+    variants = []
+    for spec in [v.strip() for v in args.variants.split(";") if v.strip()]:
+        switches = [n.strip() for n in spec.split("+") if n.strip()]
+        saved = {n: os.environ.get(n) for n in switches}
+        os.environ.update({n: "1" for n in switches})
+        try:
+            for n in names:
+                w = table[n]()
+                steps = args.steps if w.name != "xentropy" else max(3, min(args.steps, 10))
+                try:
+                    r = measure(w, dev, steps, args.warmup, False, min(args.trace_steps, steps))
+                    variants.append(dict(switches=switches, workload=n, value=r["value"], unit=r["unit"], ms_per_step=r["ms_per_step"],
+                                         kernels=r["kernels"]))
+                except Exception as e:
+                    variants.append(dict(switches=switches, workload=n, error=str(e)))
+                del w
+                torch.cuda.empty_cache()
+        finally:
+            for n, v in saved.items():
+                if v is None:
+                    os.environ.pop(n, None)
+                else:
+                    os.environ[n] = v
     head = results[0]
     line = {
         "metric": "MFMA TFLOP/s (fused MLP fwd+bwd)" if head["workload"] == "mlp" else head["metric"] + f" ({head['workload']})",
@@ -622,6 +650,8 @@ def main():
         "roofline": head["roofline"], "cpu_baseline": head["cpu_baseline"], "kernels": head["kernels"],
         "others": results[1:],
     }
+    if variants:
+        line["variants"] = variants
     print(json.dumps(line))
 
 
