@@ -52,7 +52,7 @@ class PositionWiseFeedForward(nn.Module):
     def forward(self, input, *args, **kwargs):
         seq_len, bsz, hidden_size = input.shape
         dropout = self.dropout if self.training else 0.0
-        hidden = self.fused_function(dropout, recompute, input.reshape(seq_len * bsz, -1), self.in_proj_weight,
+        hidden = self.fused_function(dropout, recompute, input.reshape(seq_len * bsz, hidden_size), self.in_proj_weight,
                                      self.out_proj_weight, self.in_proj_bias, self.out_proj_bias)
         hidden = hidden.view(seq_len, bsz, hidden_size)
         if self.dropout_residual:

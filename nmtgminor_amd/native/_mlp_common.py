@@ -69,6 +69,8 @@ def forward(act, p, inputs, mask=None, save_pre=True):
     else:
         mask = torch.empty(0, dtype=torch.uint8, device=dev)
         mode = 0
+    if batch == 0:          # nothing to compute (an empty shard): the buffers above are already the result
+        return out, post, pre, mask
     of = (ctypes.c_int64 * n)(*outs)
     L.call("nmtg_mlp_fwd", L.i32(n), L.ptr(x2), _ptr_array(weights), _ptr_array(biases), of, L.i64(batch), L.i64(in_f),
            L.ptr(out), L.ptr(post if hidden else None), L.ptr(pre if (save_pre and hidden) else None),
@@ -96,6 +98,12 @@ def backward(act, p, grad_o, post, pre, mask, inputs, input_only=False, need_dx=
     else:
         dws = [torch.empty_like(w) for w in weights]
         dbs = [torch.empty(o, dtype=x.dtype, device=dev) if b is not None else None for o, b in zip(outs, biases)]
+    if batch == 0:          # an empty batch contributes zero gradients
+        for t in dws + dbs:
+            if t is not None:
+                t.zero_()
+        dx_empty = dx.view(x.shape) if dx is not None else None
+        return [dx_empty] if input_only else [dx_empty] + dws + dbs
     of = (ctypes.c_int64 * n)(*outs)
     ws_bytes = int(L.load().nmtg_mlp_bwd_workspace_bytes(L.i32(n), of, L.i64(batch), L.i64(in_f)))
     ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)

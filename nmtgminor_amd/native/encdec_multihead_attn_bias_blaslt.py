@@ -37,6 +37,8 @@ def _fwd(is_training, heads, x_q, x_kv, w_q, w_kv, w_out, b_q, b_kv, b_out, q_li
     ctx = torch.empty(tq, b, e, dtype=dt, device=dev)
     out = torch.empty(tq, b, e, dtype=dt, device=dev) if w_out is not None else None
     dmask, mode, seed, offset = A.dropout_args(is_training, p, (bh, tq, tk), dev, dropout_mask)
+    if tq == 0 or b == 0:       # an empty batch / no query position: the (empty) buffers are the result
+        return q_lin, kv_lin, scores, dropped, dmask, ctx, out
     L.call("nmtg_encdec_attn_fwd", L.ptr(x_q), L.ptr(x_kv), L.ptr(w_q), L.ptr(w_kv), L.ptr(w_out), L.ptr(b_q), L.ptr(b_kv),
            L.ptr(b_out), L.ptr(km), L.ptr(q_lin), L.ptr(kv_lin), L.ptr(scores), L.ptr(None), L.ptr(dropped),
            L.ptr(dmask if mode else None), L.i32(mode), L.f32(p), A.u64(seed), A.u64(offset), L.ptr(ctx), L.ptr(out),
@@ -126,6 +128,11 @@ def _bwd(heads, output_grads, matmul2_results, dropout_results, attn_scores, q_l
                 n["dbq"] = torch.empty(e, dtype=dt, device=dev)
                 n["dbkv"] = torch.empty(2 * e, dtype=dt, device=dev)
                 n["dbo"] = torch.empty(e, dtype=dt, device=dev)
+    if tq == 0 or b == 0:       # an empty batch / no query position contributes zero gradients
+        for z in n.values():
+            if z is not None:
+                z.zero_()
+        return n
     ws_bytes = L.load().nmtg_encdec_attn_bwd_workspace_bytes(L.i64(tq), L.i64(tk), L.i64(b), L.i64(e), L.i32(heads))
     ws = A.workspace(ws_bytes, dev)
     # contiguous copies (if any) are bound to names: a temporary would be freed before the kernels read it

@@ -29,6 +29,11 @@ def gemm(a, b, trans_a=False, trans_b=False, alpha=1.0, bias=None, out=None, spl
     if out is None:
         out = torch.empty(batch, m, n, dtype=a3.dtype, device=a3.device)
     o3 = out if out.dim() == 3 else out.unsqueeze(0)
+    if k == 0 and o3.numel() > 0:          # an empty sum: alpha * 0 (+ bias)
+        o3.zero_()
+        if bias is not None:
+            o3.add_(bias)
+        return out if a.dim() == 3 else o3[0]
     ws = None
     ws_bytes = 0
     if split_k and trans_a and not trans_b:

@@ -39,6 +39,8 @@ def forward(use_time_mask, is_training, heads, inputs, input_weights, output_wei
     ctx = torch.empty(t, b, e, dtype=dt, device=dev)
     out = torch.empty(t, b, e, dtype=dt, device=dev)
     dmask, mode, seed, offset = A.dropout_args(is_training, dropout_prob, (bh, t, t), dev, dropout_mask)
+    if t == 0 or b == 0:        # an empty batch: the (empty) buffers are the result
+        return [lin, scores, dropped, dmask, ctx, out]
     L.call("nmtg_self_attn_fwd", L.ptr(x), L.ptr(w_in), L.ptr(w_out), L.ptr(b_in), L.ptr(b_out), L.ptr(km), L.i32(kind),
            L.ptr(lin), L.ptr(scores), L.ptr(None), L.ptr(dropped), L.ptr(dmask if mode else None), L.i32(mode),
            L.f32(dropout_prob), A.u64(seed), A.u64(offset), L.ptr(ctx), L.ptr(out), L.i64(t), L.i64(b), L.i64(e),
@@ -90,6 +92,11 @@ def _bwd(heads, output_grads, matmul2_results, dropout_results, attn_scores, inp
         if want_weights and want_biases:
             db_in = torch.empty(3 * e, dtype=dt, device=dev)
             db_out = torch.empty(e, dtype=dt, device=dev)
+    if t == 0 or b == 0:        # an empty batch contributes zero gradients
+        for z in (dx, dw_in, dw_out, db_in, db_out, dlin):
+            if z is not None:
+                z.zero_()
+        return dx, dw_in, dw_out, db_in, db_out, dlin
     ws_bytes = L.load().nmtg_self_attn_bwd_workspace_bytes(L.i64(t), L.i64(b), L.i64(e), L.i32(heads))
     ws = A.workspace(ws_bytes, dev)
     # contiguous copies (if any) are bound to names: a temporary would be freed before the kernels read it

@@ -47,6 +47,7 @@ def backward(grad_loss, logits, max_log_sum_exp, labels, smoothing, *, padding_i
     _check(labels.dtype == torch.int64, "Label type should be CUDA Long")
     _check(logits.dim() == 2 and labels.dim() == 1 and logits.size(0) == labels.size(0), "shape mismatch")
     _check(grad_loss.numel() == labels.numel() and max_log_sum_exp.numel() == labels.numel(), "shape mismatch")
+    _check(logits.numel() > 0, "Number of classes in input should not be 0")      # as the reference (xentropy_kernel.cu:659)
     logits = logits.contiguous()
     grad_loss = grad_loss.contiguous().float()
     lse = max_log_sum_exp.contiguous().float()

@@ -31,6 +31,7 @@ import test_attention_gpu as tat  # noqa: E402
 import test_elementwise_gpu as tel  # noqa: E402
 import test_gemm_gpu as tg  # noqa: E402
 import test_layer_norm_gpu as tln  # noqa: E402
+import test_zv_empty_inputs_gpu as temp  # noqa: E402
 import test_zw_strided_inputs_gpu as tstr  # noqa: E402
 import test_zx_incremental_gpu as tinc  # noqa: E402
 import test_zy_layers_gpu as tla  # noqa: E402
@@ -348,6 +349,12 @@ def test_decoder_layer(mi355x, dtype, ignore_source):
 def test_layers_stochastic_depth_dropout_and_options(mi355x):
     tla.test_encoder_layer_stochastic_depth(CPU)
     tla.test_layers_with_dropout_and_unsupported_options(CPU)
+
+
+# ----------------------------------------------------------------------------- empty inputs
+@pytest.mark.parametrize("name", [n for n in dir(temp) if n.startswith("test_")])
+def test_empty_inputs(mi355x, name):
+    getattr(temp, name)(CPU)
 
 
 # ----------------------------------------------------------------------------- strided arguments
