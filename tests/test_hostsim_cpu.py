@@ -31,6 +31,7 @@ import test_attention_gpu as tat  # noqa: E402
 import test_elementwise_gpu as tel  # noqa: E402
 import test_gemm_gpu as tg  # noqa: E402
 import test_layer_norm_gpu as tln  # noqa: E402
+import test_zu_random_shapes_gpu as trnd  # noqa: E402
 import test_zv_empty_inputs_gpu as temp  # noqa: E402
 import test_zw_strided_inputs_gpu as tstr  # noqa: E402
 import test_zx_incremental_gpu as tinc  # noqa: E402
@@ -349,6 +350,12 @@ def test_decoder_layer(mi355x, dtype, ignore_source):
 def test_layers_stochastic_depth_dropout_and_options(mi355x):
     tla.test_encoder_layer_stochastic_depth(CPU)
     tla.test_layers_with_dropout_and_unsupported_options(CPU)
+
+
+# ----------------------------------------------------------------------------- randomly drawn shapes
+@pytest.mark.parametrize("seed", trnd.SEEDS[:16] if SANITIZER_RUN else trnd.SEEDS)
+def test_random_shapes(mi355x, seed):
+    trnd.test_random_shape(CPU, seed)
 
 
 # ----------------------------------------------------------------------------- empty inputs
