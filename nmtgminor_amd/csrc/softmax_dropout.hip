@@ -82,7 +82,7 @@ __device__ __forceinline__ void row_softmax(const T* __restrict__ src, const uin
 #pragma unroll
   for (int i = 0; i < VPL; ++i)
 #pragma unroll
-    for (int j = 0; j < EPV; ++j) { v[i][j] = exp2f((v[i][j] - base) * LOG2E); sum += v[i][j]; }
+    for (int j = 0; j < EPV; ++j) { v[i][j] = __builtin_amdgcn_exp2f((v[i][j] - base) * LOG2E); sum += v[i][j]; }   // argument <= 0
   sum = wave_sum(sum);
   const float inv = sum > 0.f ? 1.f / sum : 0.f;
 #pragma unroll

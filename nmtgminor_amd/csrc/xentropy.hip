@@ -162,7 +162,7 @@ __global__ __launch_bounds__(XE_THREADS) void xentropy_bwd_kernel(
   const float sm = smoothing / static_cast<float>(vocab);
   const float onem = 1.f - smoothing;
   auto one = [&](int64_t c) {
-    float v = exp2f(fmaf(elem<T>::to_float(x[c]), LOG2E, nlse)) - sm;
+    float v = __builtin_amdgcn_exp2f(fmaf(elem<T>::to_float(x[c]), LOG2E, nlse)) - sm;
     if (c == y) v -= onem;
     dx[c] = elem<T>::from_float(g * v);
   };
@@ -172,7 +172,9 @@ __global__ __launch_bounds__(XE_THREADS) void xentropy_bwd_kernel(
     float v[EPV];
     load_pack<T, EPV>(x + c0, v);
 #pragma unroll
-    for (int j = 0; j < EPV; ++j) v[j] = exp2f(fmaf(v[j], LOG2E, nlse)) - sm;
+    // the bare v_exp_f32: its argument is x - lse <= 0, and a probability below 2^-126 may as well be 0 (the library
+    // exp2f spends four more instructions per element on keeping it a denormal; this kernel is close to VALU-bound)
+    for (int j = 0; j < EPV; ++j) v[j] = __builtin_amdgcn_exp2f(fmaf(v[j], LOG2E, nlse)) - sm;
     if (y >= c0 && y < c0 + EPV) {
 #pragma unroll
       for (int j = 0; j < EPV; ++j) if (c0 + j == y) v[j] -= onem;

@@ -104,7 +104,7 @@ def _softmax(rnd, seed, dev):
 
 
 def _layer_norm(rnd, seed, dev):
-    rows, hid = rnd.choice([1, 2, 7, 64, 257]), rnd.choice([2, 8, 64, 100, 512, 768, 1000, 1024, 4096, 5000])
+    rows, hid = rnd.choice([1, 2, 7, 64, 257]), rnd.choice([8, 24, 64, 100, 512, 768, 1000, 1024, 4096, 5000])
     d, wd = rnd.choice([(F32, F32), (BF16, BF16), (F16, F32)])
     rnd.case = f"layer norm rows {rows} hidden {hid} {d}/{wd}"
     x = inputs.layer_norm_inputs(rows, hid, d, wd, seed=seed)
