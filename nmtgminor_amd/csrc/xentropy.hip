@@ -24,6 +24,9 @@ namespace {
 
 constexpr int XE_THREADS = 1024;
 constexpr int XE_WAVES = XE_THREADS / kWave;
+// 16-byte loads a lane keeps in flight in the streaming loops: one load per trip leaves 16 bytes per lane in flight,
+// which at two 1024-thread blocks per CU (32 KB) is less than the memory latency needs at full bandwidth
+constexpr int XE_INFLIGHT = 4;
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
 constexpr float NEG_BIG = -3.0e38f;
@@ -86,15 +89,22 @@ __global__ __launch_bounds__(XE_THREADS) void xentropy_fwd_kernel(
   }
   const T* body = x + head;
   int64_t i = tid;
-  // two vectors in flight per lane per trip
-  for (; i + XE_THREADS < nvec; i += 2 * XE_THREADS) {
-    float a[EPV], b[EPV];
-    load_pack<T, EPV>(body + i * EPV, a);
-    load_pack<T, EPV>(body + (i + XE_THREADS) * EPV, b);
-    online_add<EPV>(st, sx, a);
-    online_add<EPV>(st, sx, b);
+  // XE_INFLIGHT vectors in flight per lane per trip: all loads are issued (and pinned) before the first is used; the
+  // vectors are consumed in the same order as one at a time
+  for (; i + (XE_INFLIGHT - 1) * XE_THREADS < nvec; i += XE_INFLIGHT * XE_THREADS) {
+    pack<T, EPV> raw[XE_INFLIGHT];
+#pragma unroll
+    for (int u = 0; u < XE_INFLIGHT; ++u) raw[u] = load_raw<T, EPV>(body + (i + u * XE_THREADS) * EPV);
+#pragma unroll
+    for (int u = 0; u < XE_INFLIGHT; ++u) pin_raw(raw[u]);
+#pragma unroll
+    for (int u = 0; u < XE_INFLIGHT; ++u) {
+      float a[EPV];
+      unpack_raw<T, EPV>(raw[u], a);
+      online_add<EPV>(st, sx, a);
+    }
   }
-  if (i < nvec) {
+  for (; i < nvec; i += XE_THREADS) {
     float a[EPV];
     load_pack<T, EPV>(body + i * EPV, a);
     online_add<EPV>(st, sx, a);
@@ -167,13 +177,11 @@ __global__ __launch_bounds__(XE_THREADS) void xentropy_bwd_kernel(
     dx[c] = elem<T>::from_float(g * v);
   };
   for (int64_t c = tid; c < head; c += XE_THREADS) one(c);
-  for (int64_t i = tid; i < nvec; i += XE_THREADS) {
-    const int64_t c0 = head + i * EPV;
-    float v[EPV];
-    load_pack<T, EPV>(x + c0, v);
-#pragma unroll
+  // one vector of the row: v holds the logits on entry
+  auto finish = [&](int64_t c0, float (&v)[EPV]) {
     // the bare v_exp_f32: its argument is x - lse <= 0, and a probability below 2^-126 may as well be 0 (the library
     // exp2f spends four more instructions per element on keeping it a denormal; this kernel is close to VALU-bound)
+#pragma unroll
     for (int j = 0; j < EPV; ++j) v[j] = __builtin_amdgcn_exp2f(fmaf(v[j], LOG2E, nlse)) - sm;
     if (y >= c0 && y < c0 + EPV) {
 #pragma unroll
@@ -182,6 +190,27 @@ __global__ __launch_bounds__(XE_THREADS) void xentropy_bwd_kernel(
 #pragma unroll
     for (int j = 0; j < EPV; ++j) v[j] *= g;
     store_pack<T, EPV>(dx + c0, v);
+  };
+  int64_t i = tid;
+  // XE_INFLIGHT loads in flight per lane per trip (see the forward kernel)
+  for (; i + (XE_INFLIGHT - 1) * XE_THREADS < nvec; i += XE_INFLIGHT * XE_THREADS) {
+    pack<T, EPV> raw[XE_INFLIGHT];
+#pragma unroll
+    for (int u = 0; u < XE_INFLIGHT; ++u) raw[u] = load_raw<T, EPV>(x + head + (i + u * XE_THREADS) * EPV);
+#pragma unroll
+    for (int u = 0; u < XE_INFLIGHT; ++u) pin_raw(raw[u]);
+#pragma unroll
+    for (int u = 0; u < XE_INFLIGHT; ++u) {
+      float v[EPV];
+      unpack_raw<T, EPV>(raw[u], v);
+      finish(head + (i + u * XE_THREADS) * EPV, v);
+    }
+  }
+  for (; i < nvec; i += XE_THREADS) {
+    const int64_t c0 = head + i * EPV;
+    float v[EPV];
+    load_pack<T, EPV>(x + c0, v);
+    finish(c0, v);
   }
   for (int64_t c = tail0 + tid; c < vocab; c += XE_THREADS) one(c);
 }
