@@ -92,12 +92,12 @@ __device__ __forceinline__ pack<T, N> load_raw(const T* __restrict__ p) {
 // branch that holds its only use, where it waits for it alone.
 template <typename T, int N>
 __device__ __forceinline__ void pin_raw(pack<T, N>& r) {
-  static_assert(sizeof(pack<T, N>) % 4 == 0, "whole 32-bit words");
-  uint32_t w[sizeof(pack<T, N>) / 4];
-  __builtin_memcpy(w, &r, sizeof(w));
+  constexpr int WORDS = (sizeof(pack<T, N>) + 3) / 4;       // a pack narrower than a word is pinned in one word
+  uint32_t w[WORDS] = {};
+  __builtin_memcpy(w, &r, sizeof(r));
 #pragma unroll
-  for (int k = 0; k < static_cast<int>(sizeof(w) / 4); ++k) asm volatile("" : "+v"(w[k]));
-  __builtin_memcpy(&r, w, sizeof(w));
+  for (int k = 0; k < WORDS; ++k) asm volatile("" : "+v"(w[k]));
+  __builtin_memcpy(&r, w, sizeof(r));
 }
 template <typename T, int N>
 __device__ __forceinline__ void unpack_raw(const pack<T, N>& r, float (&out)[N]) {

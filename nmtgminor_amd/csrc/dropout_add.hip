@@ -24,16 +24,22 @@ __global__ __launch_bounds__(DA_THREADS) void dropout_add_fwd_kernel(
   const int64_t first = (static_cast<int64_t>(blockIdx.x) * DA_THREADS + threadIdx.x) * EPV;
   if (first >= n) return;
   if (first + EPV <= n) {
+    // all loads are issued before the first conversion, so the lane waits for memory once
+    pack<T, EPV> rawx = load_raw<T, EPV>(x + first), rawr = load_raw<T, EPV>(residual + first);
+    pack<uint8_t, EPV> rawm = {};
+    if constexpr (MODE == DA_MASK_IN) rawm = load_raw<uint8_t, EPV>(mask + first);
+    pin_raw(rawx); pin_raw(rawr); pin_raw(rawm);
     float xv[EPV], rv[EPV];
-    load_pack<T, EPV>(x + first, xv);
-    load_pack<T, EPV>(residual + first, rv);
+    unpack_raw<T, EPV>(rawx, xv);
+    unpack_raw<T, EPV>(rawr, rv);
     if constexpr (MODE == DA_EVAL) {
 #pragma unroll
       for (int j = 0; j < EPV; ++j) xv[j] += rv[j];
     } else {
       uint8_t keep[EPV];
       if constexpr (MODE == DA_MASK_IN) {
-        load_bytes<EPV>(mask + first, keep);
+#pragma unroll
+        for (int j = 0; j < EPV; ++j) keep[j] = rawm.v[j];
       } else {
         philox_keep<EPV>(Philox(seed), static_cast<uint64_t>(first), offset, keep_p, keep);
         store_bytes<EPV>(mask + first, keep);

@@ -51,22 +51,41 @@ __device__ __forceinline__ const uint8_t* kmask_row(const SoftmaxArgs& a, int64_
   return nullptr;
 }
 
-// Loads the row's scores into v (masked / out-of-range -> -inf), returns the normalised
-// probabilities in v and whether the row had any unmasked key.
+// Every kernel below issues all of a row's loads (scores, key mask, dropout mask, gradient) before it uses any of
+// them, so that a wavefront waits for memory once per row instead of once per load: with one row per wavefront
+// these kernels are bound by that latency, not by bandwidth. Lanes beyond the row's end load from column 0 and
+// discard the value.
+template <int EPV>
+__device__ __forceinline__ int row_col(int i, int lane) { return (i * kWave + lane) * EPV; }
+
 template <typename T, int EPV, int VPL>
-__device__ __forceinline__ void row_softmax(const T* __restrict__ src, const uint8_t* __restrict__ km, int cols,
-                                            int lane, float (&v)[VPL][EPV]) {
+__device__ __forceinline__ void row_load(const T* __restrict__ src, int cols, int lane, pack<T, EPV> (&r)[VPL]) {
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    const int col = row_col<EPV>(i, lane);
+    r[i] = load_raw<T, EPV>(src + (col < cols ? col : 0));
+  }
+}
+template <typename T, int EPV, int VPL>
+__device__ __forceinline__ void row_pin(pack<T, EPV> (&r)[VPL]) {
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) pin_raw(r[i]);
+}
+
+// Turns the row's loaded scores into normalised probabilities in v (masked / out-of-range -> -inf before the
+// maximum; a row with every key masked gives zeros).
+template <typename T, int EPV, int VPL>
+__device__ __forceinline__ void row_softmax(const pack<T, EPV> (&rx)[VPL], const pack<uint8_t, EPV> (&rk)[VPL],
+                                            bool masked, int cols, int lane, float (&v)[VPL][EPV]) {
   float mx = -INFINITY;
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
-    const int col = (i * kWave + lane) * EPV;
+    const int col = row_col<EPV>(i, lane);
     if (col < cols) {
-      load_pack<T, EPV>(src + col, v[i]);
-      if (km != nullptr) {
-        uint8_t mk[EPV];
-        load_bytes<EPV>(km + col, mk);
+      unpack_raw<T, EPV>(rx[i], v[i]);
+      if (masked) {
 #pragma unroll
-        for (int j = 0; j < EPV; ++j) if (mk[j]) v[i][j] = -INFINITY;
+        for (int j = 0; j < EPV; ++j) if (rk[i].v[j]) v[i][j] = -INFINITY;
       }
 #pragma unroll
       for (int j = 0; j < EPV; ++j) mx = fmaxf(mx, v[i][j]);
@@ -97,20 +116,29 @@ __global__ __launch_bounds__(SM_THREADS) void softmax_fwd_kernel(SoftmaxArgs a) 
   const int64_t row = static_cast<int64_t>(blockIdx.x) * SM_WAVES + threadIdx.x / kWave;
   if (row >= a.rows) return;
   const int64_t base = row * a.cols;
+  const uint8_t* km = kmask_row(a, row);
+  const bool mask_in = a.dropout_mode == SM_MASK_IN;
+  pack<T, EPV> rx[VPL];
+  pack<uint8_t, EPV> rk[VPL] = {}, rd[VPL] = {};
+  row_load<T, EPV, VPL>(static_cast<const T*>(a.in) + base, a.cols, lane, rx);
+  if (km != nullptr) row_load<uint8_t, EPV, VPL>(km, a.cols, lane, rk);
+  if (mask_in) row_load<uint8_t, EPV, VPL>(a.dmask + base, a.cols, lane, rd);
+  row_pin(rx); row_pin(rk); row_pin(rd);
   float v[VPL][EPV];
-  row_softmax<T, EPV, VPL>(static_cast<const T*>(a.in) + base, kmask_row(a, row), a.cols, lane, v);
+  row_softmax<T, EPV, VPL>(rx, rk, km != nullptr, a.cols, lane, v);
   T* out = static_cast<T*>(a.out) + base;
   T* out_sm = a.out_softmax ? static_cast<T*>(a.out_softmax) + base : nullptr;
   const Philox gen(a.seed);
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
-    const int col = (i * kWave + lane) * EPV;
+    const int col = row_col<EPV>(i, lane);
     if (col < a.cols) {
       if (out_sm) store_pack<T, EPV>(out_sm + col, v[i]);
       if (a.dropout_mode != SM_NO_DROPOUT) {
         uint8_t keep[EPV];
-        if (a.dropout_mode == SM_MASK_IN) {
-          load_bytes<EPV>(a.dmask + base + col, keep);
+        if (mask_in) {
+#pragma unroll
+          for (int j = 0; j < EPV; ++j) keep[j] = rd[i].v[j];
         } else {
           philox_keep<EPV>(gen, static_cast<uint64_t>(base + col), a.offset, a.keep_p, keep);
           store_bytes<EPV>(a.dmask + base + col, keep);
@@ -130,33 +158,36 @@ __global__ __launch_bounds__(SM_THREADS) void softmax_bwd_kernel(SoftmaxArgs a) 
   const int64_t row = static_cast<int64_t>(blockIdx.x) * SM_WAVES + threadIdx.x / kWave;
   if (row >= a.rows) return;
   const int64_t base = row * a.cols;
+  const uint8_t* km = a.from_scores ? kmask_row(a, row) : nullptr;
+  const bool dropped = a.dropout_mode != SM_NO_DROPOUT;
+  pack<T, EPV> rs[VPL], rg[VPL];
+  pack<uint8_t, EPV> rk[VPL] = {}, rd[VPL] = {};
+  row_load<T, EPV, VPL>(static_cast<const T*>(a.saved) + base, a.cols, lane, rs);
+  row_load<T, EPV, VPL>(static_cast<const T*>(a.in) + base, a.cols, lane, rg);
+  if (km != nullptr) row_load<uint8_t, EPV, VPL>(km, a.cols, lane, rk);
+  if (dropped) row_load<uint8_t, EPV, VPL>(a.dmask + base, a.cols, lane, rd);
+  row_pin(rs); row_pin(rg); row_pin(rk); row_pin(rd);
   float pr[VPL][EPV], g[VPL][EPV];
-  const T* saved = static_cast<const T*>(a.saved) + base;
   if (a.from_scores) {
-    row_softmax<T, EPV, VPL>(saved, kmask_row(a, row), a.cols, lane, pr);
+    row_softmax<T, EPV, VPL>(rs, rk, km != nullptr, a.cols, lane, pr);
   } else {
 #pragma unroll
     for (int i = 0; i < VPL; ++i) {
-      const int col = (i * kWave + lane) * EPV;
-      if (col < a.cols) load_pack<T, EPV>(saved + col, pr[i]);
+      if (row_col<EPV>(i, lane) < a.cols) unpack_raw<T, EPV>(rs[i], pr[i]);
       else {
 #pragma unroll
         for (int j = 0; j < EPV; ++j) pr[i][j] = 0.f;
       }
     }
   }
-  const T* gin = static_cast<const T*>(a.in) + base;
   float dot = 0.f;
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
-    const int col = (i * kWave + lane) * EPV;
-    if (col < a.cols) {
-      load_pack<T, EPV>(gin + col, g[i]);
-      if (a.dropout_mode != SM_NO_DROPOUT) {
-        uint8_t keep[EPV];
-        load_bytes<EPV>(a.dmask + base + col, keep);
+    if (row_col<EPV>(i, lane) < a.cols) {
+      unpack_raw<T, EPV>(rg[i], g[i]);
+      if (dropped) {
 #pragma unroll
-        for (int j = 0; j < EPV; ++j) g[i][j] = keep[j] ? g[i][j] * a.scale : 0.f;
+        for (int j = 0; j < EPV; ++j) g[i][j] = rd[i].v[j] ? g[i][j] * a.scale : 0.f;
       }
 #pragma unroll
       for (int j = 0; j < EPV; ++j) dot += pr[i][j] * g[i][j];
@@ -169,7 +200,7 @@ __global__ __launch_bounds__(SM_THREADS) void softmax_bwd_kernel(SoftmaxArgs a) 
   T* out = static_cast<T*>(a.out) + base;
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
-    const int col = (i * kWave + lane) * EPV;
+    const int col = row_col<EPV>(i, lane);
     if (col < a.cols) {
 #pragma unroll
       for (int j = 0; j < EPV; ++j) g[i][j] = pr[i][j] * (g[i][j] - dot);
