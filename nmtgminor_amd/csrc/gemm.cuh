@@ -605,7 +605,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, acc16_t (&acc)[
           const float base = (mx == -INFINITY) ? 0.f : mx;   // a row without any key gives zeros
           float sum = 0.f;
 #pragma unroll
-          for (int k = 0; k < 8; ++k) { v[k] = exp2f((v[k] - base) * LOG2E); sum += v[k]; }
+          for (int k = 0; k < 8; ++k) { v[k] = fast_exp2((v[k] - base) * LOG2E); sum += v[k]; }
           sum = wave_sum(sum);
           const float inv = sum > 0.f ? 1.f / sum : 0.f;
 #pragma unroll
@@ -680,7 +680,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, acc16_t (&acc)[
           const float base = (mx == -INFINITY) ? 0.f : mx;
           float sum = 0.f;
 #pragma unroll
-          for (int k = 0; k < 8; ++k) { pr[k] = exp2f((pr[k] - base) * LOG2E); sum += pr[k]; }
+          for (int k = 0; k < 8; ++k) { pr[k] = fast_exp2((pr[k] - base) * LOG2E); sum += pr[k]; }
           sum = wave_sum(sum);
           const float inv = sum > 0.f ? 1.f / sum : 0.f;
           float dot = 0.f;
