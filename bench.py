@@ -424,6 +424,55 @@ class DropoutAddWL(Workload):
                     sample="full workload ([512 x 32 x 1024] bf16 fwd+bwd), median of 3")
 
 
+class GeneratorLossWL(Workload):
+    name = "generator_loss"
+    bound = "mfma"
+    dtype = "bf16"
+    description = ("output projection + label-smoothed cross-entropy fwd+bwd in chunks of 4096 rows (no [N, V] logits tensor): "
+                   "bf16 states [16384 x 1024], vocabulary 250054, eps 0.1, 10% padding (idx 1)")
+    ROWS, MODEL, VOCAB, CHUNK = 16384, 1024, 250054, 4096
+
+    def setup(self, dev):
+        from oracle import inputs
+        from nmtgminor_amd.modules.generator_loss import LinearSoftmaxCrossEntropy
+        self.fn = LinearSoftmaxCrossEntropy
+        n, e, v = self.ROWS, self.MODEL, self.VOCAB
+        d = inputs.xentropy_inputs(n, v, with_logits=False)
+        self.labels_cpu = d["labels"]
+        self.labels, self.grad = d["labels"].to(dev), d["grad_loss"].to(dev)
+        g = torch.Generator(device=dev)
+        g.manual_seed(1006)
+        self.h = torch.randn(n, e, generator=g, device=dev).to(torch.bfloat16).requires_grad_()
+        self.w = (torch.randn(v, e, generator=g, device=dev) / e ** 0.5).to(torch.bfloat16).requires_grad_()
+
+    def step(self):
+        self.h.grad = self.w.grad = None
+        losses = self.fn.apply(self.h, self.w, None, self.labels, 0.1, 1, self.CHUNK)
+        losses.backward(self.grad)
+        return losses, self.h.grad, self.w.grad
+
+    def work_per_step(self):
+        # the projection in the forward, again in the backward, and the two gradient contractions
+        return 4 * 2.0 * self.ROWS * self.MODEL * self.VOCAB
+
+    def kernel_work(self):
+        return {"gemm_": self.work_per_step()}
+
+    def cpu_baseline(self):
+        from oracle import generator_loss as o
+        n = 128
+        h, w = self.h[:n].detach().float().cpu(), self.w.detach().float().cpu()
+        y, gl = self.labels_cpu[:n], torch.ones(n)
+
+        def run():
+            o.generator_loss_fwd(h, w, None, y, 0.1, 1)
+            o.generator_loss_bwd(gl, h, w, None, y, 0.1, 1)
+        t = _time_cpu(run, 3)
+        # the oracle's backward recomputes the projection as the chunked operator does: 4 products of n x E x V
+        return dict(value=4 * 2.0 * n * self.MODEL * self.VOCAB / t / 1e12, unit="TFLOP/s", cores=torch.get_num_threads(),
+                    kind="port", sample=f"first {n} of {self.ROWS} rows against the full vocabulary, fp32, median of 3")
+
+
 class CopyWL(Workload):
     """Plain device copy of a known size: the calibration target for the rocprofv3 FETCH_SIZE /
     WRITE_SIZE counters (not part of `--workload all`)."""
@@ -445,7 +494,8 @@ class CopyWL(Workload):
         return 2 * self.src.numel() * 4
 
 
-WORKLOADS = {w.name: w for w in (LayerNormWL, MlpWL, SelfAttnWL, EncdecAttnWL, SoftmaxDropoutWL, DropoutAddWL, XentropyWL)}
+WORKLOADS = {w.name: w for w in (LayerNormWL, MlpWL, SelfAttnWL, EncdecAttnWL, SoftmaxDropoutWL, DropoutAddWL, XentropyWL,
+                                    GeneratorLossWL)}
 EXTRA_WORKLOADS = {CopyWL.name: CopyWL}
 PRIMARY = "mlp"
 
@@ -604,7 +654,7 @@ def main():
     results = []
     for n in names:
         w = table[n]()
-        steps = args.steps if w.name != "xentropy" else max(3, min(args.steps, 10))
+        steps = args.steps if w.name not in ("xentropy", "generator_loss") else max(3, min(args.steps, 10))
         try:
             results.append(measure(w, dev, steps, args.warmup, not args.no_cpu, min(args.trace_steps, steps)))
         except Exception as e:
@@ -624,7 +674,7 @@ def main():
         try:
             for n in names:
                 w = table[n]()
-                steps = args.steps if w.name != "xentropy" else max(3, min(args.steps, 10))
+                steps = args.steps if w.name not in ("xentropy", "generator_loss") else max(3, min(args.steps, 10))
                 try:
                     r = measure(w, dev, steps, args.warmup, False, min(args.trace_steps, steps))
                     variants.append(dict(switches=switches, workload=n, value=r["value"], unit=r["unit"], ms_per_step=r["ms_per_step"],

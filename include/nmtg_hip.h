@@ -133,16 +133,19 @@ int nmtg_softmax_dropout_bwd(const void* grad_dropped, const void* saved, int sa
  *   (onmt/modules/optimized/softmax_xentropy.py:10,24) is folded in through padding_idx
  *   (pass a value no label takes, e.g. INT64_MIN, to switch it off).
  *
- * logits [rows, vocab] (fp32 / fp16 / bf16), labels int64 [rows]; losses, lse fp32 [rows];
- * grad_loss fp32 [rows]; grad_logits [rows, vocab] in the logits dtype. fp32 accumulation.
+ * logits [rows, vocab] (fp32 / fp16 / bf16) with row pitch ld_logits >= vocab elements (the
+ * reference's tensors are dense: ld_logits = vocab), labels int64 [rows]; losses, lse fp32 [rows];
+ * grad_loss fp32 [rows]; grad_logits [rows, vocab] in the logits dtype with row pitch ld_grad;
+ * elements between vocab and the pitch are neither read nor written. fp32 accumulation.
  * ------------------------------------------------------------------------------------------ */
 int nmtg_xentropy_fwd(const void* logits, const int64_t* labels, float* losses, float* lse,
-                      int64_t rows, int64_t vocab, float smoothing, int64_t padding_idx, int dtype,
-                      void* stream);
+                      int64_t rows, int64_t vocab, int64_t ld_logits, float smoothing,
+                      int64_t padding_idx, int dtype, void* stream);
 
 int nmtg_xentropy_bwd(const float* grad_loss, const void* logits, const float* lse,
                       const int64_t* labels, void* grad_logits, int64_t rows, int64_t vocab,
-                      float smoothing, int64_t padding_idx, int dtype, void* stream);
+                      int64_t ld_logits, int64_t ld_grad, float smoothing, int64_t padding_idx,
+                      int dtype, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Strided-batched GEMM on the MFMA units (fp16 / bf16 in and out, fp32 accumulation), row-major:

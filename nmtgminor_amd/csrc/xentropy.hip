@@ -68,11 +68,11 @@ __device__ __forceinline__ void online_add(Online& st, float& sx, const float (&
 template <typename T>
 __global__ __launch_bounds__(XE_THREADS) void xentropy_fwd_kernel(
     const T* __restrict__ logits, const int64_t* __restrict__ labels, float* __restrict__ losses,
-    float* __restrict__ lse_out, int64_t vocab, float smoothing, int64_t padding_idx) {
+    float* __restrict__ lse_out, int64_t vocab, int64_t ld, float smoothing, int64_t padding_idx) {
   constexpr int EPV = 16 / sizeof(T);
   __shared__ float sm_m[XE_WAVES], sm_s[XE_WAVES], sm_x[XE_WAVES];
   const int64_t row = blockIdx.x;
-  const T* x = logits + row * vocab;
+  const T* x = logits + row * ld;
   const int tid = threadIdx.x;
 
   const uintptr_t addr = reinterpret_cast<uintptr_t>(x);
@@ -144,12 +144,12 @@ __global__ __launch_bounds__(XE_THREADS) void xentropy_fwd_kernel(
 template <typename T, bool VEC>
 __global__ __launch_bounds__(XE_THREADS) void xentropy_bwd_kernel(
     const float* __restrict__ grad_loss, const T* __restrict__ logits, const float* __restrict__ lse_in,
-    const int64_t* __restrict__ labels, T* __restrict__ grad_logits, int64_t vocab, float smoothing,
-    int64_t padding_idx) {
+    const int64_t* __restrict__ labels, T* __restrict__ grad_logits, int64_t vocab, int64_t ld, int64_t ld_grad,
+    float smoothing, int64_t padding_idx) {
   constexpr int EPV = 16 / sizeof(T);
   const int64_t row = blockIdx.x;
-  const T* x = logits + row * vocab;
-  T* dx = grad_logits + row * vocab;
+  const T* x = logits + row * ld;
+  T* dx = grad_logits + row * ld_grad;
   const int tid = threadIdx.x;
   const int64_t y = labels[row];
   const float g = (y == padding_idx) ? 0.f : grad_loss[row];
@@ -221,40 +221,48 @@ __global__ __launch_bounds__(XE_THREADS) void xentropy_bwd_kernel(
 using namespace nmtg;
 
 extern "C" int nmtg_xentropy_fwd(const void* logits, const int64_t* labels, float* losses, float* lse, int64_t rows,
-                                 int64_t vocab, float smoothing, int64_t padding_idx, int dtype, void* stream) {
+                                 int64_t vocab, int64_t ld_logits, float smoothing, int64_t padding_idx, int dtype,
+                                 void* stream) {
   NMTG_REQUIRE(rows >= 0 && rows <= INT32_MAX, "xentropy_fwd: bad row count %lld", (long long)rows);
   NMTG_REQUIRE(vocab > 0, "xentropy_fwd: number of classes must be positive");
+  NMTG_REQUIRE(ld_logits >= vocab, "xentropy_fwd: row pitch %lld is below the number of classes %lld",
+               (long long)ld_logits, (long long)vocab);
   if (rows == 0) return 0;
   NMTG_REQUIRE(logits && labels && losses && lse, "xentropy_fwd: null pointer argument");
   hipStream_t st = static_cast<hipStream_t>(stream);
   TraceScope trace("xentropy_fwd", st);
   NMTG_DISPATCH_DTYPE(dtype, T,
                       hipLaunchKernelGGL((xentropy_fwd_kernel<T>), dim3(static_cast<unsigned>(rows)), dim3(XE_THREADS), 0,
-                                         st, static_cast<const T*>(logits), labels, losses, lse, vocab, smoothing,
-                                         padding_idx));
+                                         st, static_cast<const T*>(logits), labels, losses, lse, vocab, ld_logits,
+                                         smoothing, padding_idx));
   NMTG_CHECK_LAUNCH("xentropy_fwd");
   return 0;
 }
 
 extern "C" int nmtg_xentropy_bwd(const float* grad_loss, const void* logits, const float* lse, const int64_t* labels,
-                                 void* grad_logits, int64_t rows, int64_t vocab, float smoothing, int64_t padding_idx,
-                                 int dtype, void* stream) {
+                                 void* grad_logits, int64_t rows, int64_t vocab, int64_t ld_logits, int64_t ld_grad,
+                                 float smoothing, int64_t padding_idx, int dtype, void* stream) {
   NMTG_REQUIRE(rows >= 0 && rows <= INT32_MAX, "xentropy_bwd: bad row count %lld", (long long)rows);
   NMTG_REQUIRE(vocab > 0, "xentropy_bwd: number of classes must be positive");
+  NMTG_REQUIRE(ld_logits >= vocab && ld_grad >= vocab, "xentropy_bwd: a row pitch (%lld, %lld) is below the number of classes %lld",
+               (long long)ld_logits, (long long)ld_grad, (long long)vocab);
   if (rows == 0) return 0;
   NMTG_REQUIRE(grad_loss && logits && lse && labels && grad_logits, "xentropy_bwd: null pointer argument");
   hipStream_t st = static_cast<hipStream_t>(stream);
-  // Vector accesses need the logits row and the gradient row to share their 16-byte phase.
-  const bool vec = ((reinterpret_cast<uintptr_t>(logits) ^ reinterpret_cast<uintptr_t>(grad_logits)) & 15u) == 0;
+  // Vector accesses need every logits row and its gradient row to share their 16-byte phase: the two bases do, and the
+  // two pitches differ by a multiple of 16 bytes.
+  const int64_t esize = dtype == NMTG_F32 ? 4 : 2;
+  const bool vec = ((reinterpret_cast<uintptr_t>(logits) ^ reinterpret_cast<uintptr_t>(grad_logits)) & 15u) == 0 &&
+                   ((ld_logits - ld_grad) * esize) % 16 == 0;
   TraceScope trace("xentropy_bwd", st);
   NMTG_DISPATCH_DTYPE(
       dtype, T,
       if (vec) hipLaunchKernelGGL((xentropy_bwd_kernel<T, true>), dim3(static_cast<unsigned>(rows)), dim3(XE_THREADS), 0, st,
                                   grad_loss, static_cast<const T*>(logits), lse, labels, static_cast<T*>(grad_logits), vocab,
-                                  smoothing, padding_idx);
+                                  ld_logits, ld_grad, smoothing, padding_idx);
       else hipLaunchKernelGGL((xentropy_bwd_kernel<T, false>), dim3(static_cast<unsigned>(rows)), dim3(XE_THREADS), 0, st,
                               grad_loss, static_cast<const T*>(logits), lse, labels, static_cast<T*>(grad_logits), vocab,
-                              smoothing, padding_idx));
+                              ld_logits, ld_grad, smoothing, padding_idx));
   NMTG_CHECK_LAUNCH("xentropy_bwd");
   return 0;
 }

@@ -1,0 +1,174 @@
+"""Output projection + label-smoothed cross-entropy without the [N, V] logits tensor.
+
+The reference projects the decoder states to the vocabulary (Generator.forward,
+onmt/modules/base_seq2seq.py:26-47) and hands the whole logits tensor to the loss
+(CrossEntropyLossBase._compute_loss, onmt/modules/loss.py:60-109, which calls
+SoftmaxCrossEntropyLoss.apply(logits, labels, smoothing, padding_idx, half_to_float)). At a vocabulary of 250 054 and
+16 384 target positions that tensor and its gradient are 8.2 GB each. Here the same two kernels (the MFMA projection and
+the cross-entropy) run over `chunk_rows` positions at a time: the forward keeps only the per-row losses and
+log-sum-exp, the backward recomputes each chunk's logits, turns them into their gradient and contracts that at once
+with the weight (gradient of the states) and with the states (weight gradient, accumulated over the chunks in fp32).
+Per-row results are those of the unchunked pair of operators; arbitrary per-row upstream gradients (loss weights) are
+supported because nothing of the backward is precomputed in the forward.
+
+The chunk buffers have a row pitch of the vocabulary rounded up to 64 elements, so that the projection's stores and the
+two contractions that read the logits gradient move 16 bytes per access whatever the vocabulary size (250 054 is not a
+multiple of 4); the cross-entropy kernels read and write the first V elements of each pitched row in place.
+
+Beyond the kernels this module only slices, accumulates the weight gradient (`add_` in fp32) and sums the bias
+gradient (`sum`); those are device-side PyTorch calls on already computed chunks.
+"""
+import torch
+import torch.nn as nn
+
+from ..native import linear_gemm, xentropy_cuda
+
+DEFAULT_CHUNK_ROWS = 4096
+
+
+def _check(cond, msg):
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _check_inputs(hidden, weight, bias, labels, chunk_rows):
+    _check(hidden.dim() == 2 and weight.dim() == 2, "hidden must be [N, E] and weight [V, E]")
+    _check(hidden.size(1) == weight.size(1), "hidden and weight disagree on the model dimension")
+    _check(hidden.dtype in (torch.float16, torch.bfloat16) and weight.dtype == hidden.dtype,
+           "fp16 or bf16 states and weights of one dtype required")
+    _check(bias is None or (bias.dim() == 1 and bias.size(0) == weight.size(0) and bias.dtype == hidden.dtype),
+           "bias must be [V] in the dtype of the weights")
+    _check(labels.dim() == 1 and labels.size(0) == hidden.size(0), "one label per row required")
+    _check(labels.dtype == torch.int64, "Label type should be CUDA Long")
+    _check(int(chunk_rows) > 0, "chunk_rows must be positive")
+
+
+def _chunks(n, chunk_rows):
+    return [(r0, min(n, r0 + chunk_rows)) for r0 in range(0, n, chunk_rows)]
+
+
+def _chunk_buffer(rows, v, like):
+    """[rows, v] view of a buffer whose row pitch is v rounded up to 64 elements."""
+    pitch = (v + 63) // 64 * 64
+    return torch.empty(rows, pitch, dtype=like.dtype, device=like.device)[:, :v]
+
+
+def _logits(hidden, weight, bias, r0, r1, buf):
+    return linear_gemm.gemm(hidden[r0:r1], weight, trans_b=True, bias=bias, out=buf[:r1 - r0])
+
+
+class LinearSoftmaxCrossEntropy(torch.autograd.Function):
+    """apply(hidden [N, E], weight [V, E], bias [V] | None, labels [N], smoothing=0.0, padding_idx=-100,
+    chunk_rows=4096) -> losses fp32 [N] (zeros where labels == padding_idx): what
+    SoftmaxCrossEntropyLoss.apply(F.linear(hidden, weight, bias), labels, smoothing, padding_idx, True) returns."""
+
+    @staticmethod
+    def forward(ctx, hidden, weight, bias, labels, smoothing=0.0, padding_idx=-100, chunk_rows=DEFAULT_CHUNK_ROWS):
+        _check_inputs(hidden, weight, bias, labels, chunk_rows)
+        hidden, weight, labels = hidden.contiguous(), weight.contiguous(), labels.contiguous()
+        bias = bias.contiguous() if bias is not None else None
+        n, v = hidden.size(0), weight.size(0)
+        losses = torch.empty(n, dtype=torch.float32, device=hidden.device)
+        lse = torch.empty(n, dtype=torch.float32, device=hidden.device)
+        if n > 0:
+            _check(v > 0, "Number of classes in input should not be 0")
+            buf = _chunk_buffer(min(n, chunk_rows), v, hidden)
+            for r0, r1 in _chunks(n, chunk_rows):
+                z = _logits(hidden, weight, bias, r0, r1, buf)
+                part, m = xentropy_cuda.forward(z, labels[r0:r1], smoothing, True, padding_idx=padding_idx)
+                losses[r0:r1] = part
+                lse[r0:r1] = m
+        ctx.save_for_backward(hidden, weight, bias, labels, lse)
+        ctx.smoothing, ctx.padding_idx, ctx.chunk_rows = smoothing, padding_idx, chunk_rows
+        return losses
+
+    @staticmethod
+    def backward(ctx, grad_loss):
+        hidden, weight, bias, labels, lse = ctx.saved_tensors
+        need_h, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        need_b = bias is not None and ctx.needs_input_grad[2]
+        n, v = hidden.size(0), weight.size(0)
+        grad_loss = grad_loss.contiguous().float()
+        dh = torch.empty_like(hidden) if need_h else None
+        dw = torch.zeros(weight.shape, dtype=torch.float32, device=weight.device) if need_w else None
+        db = torch.zeros(v, dtype=torch.float32, device=weight.device) if need_b else None
+        if n > 0 and (need_h or need_w or need_b):
+            buf = _chunk_buffer(min(n, ctx.chunk_rows), v, hidden)
+            gbuf = _chunk_buffer(min(n, ctx.chunk_rows), v, hidden)
+            for r0, r1 in _chunks(n, ctx.chunk_rows):
+                z = _logits(hidden, weight, bias, r0, r1, buf)                       # the forward's logits again
+                dz = xentropy_cuda.backward(grad_loss[r0:r1], z, lse[r0:r1], labels[r0:r1], ctx.smoothing,
+                                            padding_idx=ctx.padding_idx, out=gbuf[:r1 - r0])
+                if need_h:
+                    linear_gemm.gemm(dz, weight, out=dh[r0:r1])                      # [n, V] x [V, E]
+                if need_w:
+                    dw.add_(linear_gemm.gemm(dz, hidden[r0:r1], trans_a=True))       # [V, n] x [n, E]
+                if need_b:
+                    db.add_(dz.sum(dim=0, dtype=torch.float32))
+        return (dh, dw.to(weight.dtype) if need_w else None, db.to(bias.dtype) if need_b else None,
+                None, None, None, None)
+
+
+def linear_cross_entropy_eval(hidden, weight, bias, labels, padding_idx=-100, chunk_rows=DEFAULT_CHUNK_ROWS):
+    """No-gradient pass for validation: -> (losses fp32 [N] without smoothing, argmax int64 [N]); the reference's
+    eval branch takes the argmax of the unnormalised logits (onmt/modules/loss.py:293-299)."""
+    _check_inputs(hidden, weight, bias, labels, chunk_rows)
+    with torch.no_grad():
+        hidden, weight, labels = hidden.contiguous(), weight.contiguous(), labels.contiguous()
+        bias = bias.contiguous() if bias is not None else None
+        n, v = hidden.size(0), weight.size(0)
+        losses = torch.empty(n, dtype=torch.float32, device=hidden.device)
+        preds = torch.empty(n, dtype=torch.int64, device=hidden.device)
+        if n > 0:
+            _check(v > 0, "Number of classes in input should not be 0")
+            buf = _chunk_buffer(min(n, chunk_rows), v, hidden)
+            for r0, r1 in _chunks(n, chunk_rows):
+                z = _logits(hidden, weight, bias, r0, r1, buf)
+                losses[r0:r1] = xentropy_cuda.forward(z, labels[r0:r1], 0.0, True, padding_idx=padding_idx)[0]
+                preds[r0:r1] = torch.argmax(z, dim=1)
+    return losses, preds
+
+
+class GeneratorLoss(nn.Module):
+    """The reference's Generator (its parameter is `linear`, so checkpoints map key by key) and the fast branch of
+    CrossEntropyLossBase._compute_loss in one module.
+
+    forward(hidden [..., E], targets [...], loss_weights=None, loss_constraint=0, sum_loss=True, eval=False)
+    -> dict(loss, data, correct, total). `loss` is sum_i w_i (loss_i - loss_constraint) (or the per-row tensor when
+    sum_loss is False); `data` is the unweighted, unconstrained sum as a Python float (per-row tensor when sum_loss is
+    False), as the reference reports it; label smoothing applies in training mode only. Rows whose target is the
+    padding index contribute zero loss and zero gradient (the reference drops them with index_select first);
+    `total` counts the others and `correct` (eval=True only) how many of those the argmax hits."""
+
+    def __init__(self, hidden_size, output_size, label_smoothing=0.0, padding_idx=0, bias=True,
+                 chunk_rows=DEFAULT_CHUNK_ROWS):
+        super().__init__()
+        self.linear = nn.Linear(hidden_size, output_size, bias=bias)
+        stdv = 1.0 / hidden_size ** 0.5
+        nn.init.uniform_(self.linear.weight, -stdv, stdv)
+        if bias:
+            nn.init.zeros_(self.linear.bias)
+        self.hidden_size, self.output_size = hidden_size, output_size
+        self.label_smoothing, self.padding_idx, self.chunk_rows = label_smoothing, padding_idx, chunk_rows
+
+    def forward(self, hidden, targets, loss_weights=None, loss_constraint=0, sum_loss=True, eval=False):
+        h = hidden.reshape(-1, hidden.size(-1))
+        y = targets.reshape(-1)
+        correct, total = 0, 0
+        if eval:
+            rows, preds = linear_cross_entropy_eval(h, self.linear.weight, self.linear.bias, y, self.padding_idx,
+                                                    self.chunk_rows)
+            real = y != self.padding_idx
+            correct, total = int(((preds == y) & real).sum().item()), int(real.sum().item())
+        else:
+            smoothing = self.label_smoothing if self.training else 0.0
+            rows = LinearSoftmaxCrossEntropy.apply(h, self.linear.weight, self.linear.bias, y, smoothing,
+                                                   self.padding_idx, self.chunk_rows)
+        data = rows.detach().sum().item() if sum_loss else rows.detach()
+        # the constraint is subtracted on real rows only: padded rows are not part of the reference's batch
+        loss = rows - loss_constraint * (y != self.padding_idx).to(rows.dtype) if loss_constraint else rows
+        if loss_weights is not None:
+            loss = loss * loss_weights.reshape(-1).to(loss.dtype)
+        if sum_loss:
+            loss = loss.sum()
+        return dict(loss=loss, data=data, correct=correct, total=total)

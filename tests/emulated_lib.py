@@ -127,18 +127,18 @@ def softmax_bwd(grad, saved, is_scores, key_mask, kind, dmask, dmode, p, gs, row
     put(T(gs, shape, DT[v(dt)]), osd.softmax_dropout_bwd(G, SV, dm, v(p) if dm is not None else 0.0, D))
 
 
-def xent_fwd(logits, labels, losses, lse, rows, vocab, smoothing, pad, dt, st):
+def xent_fwd(logits, labels, losses, lse, rows, vocab, ld, smoothing, pad, dt, st):
     n, vv = v(rows), v(vocab)
-    lo, ls = oxe.xentropy_fwd(T(logits, (n, vv), DT[v(dt)]), T(labels, (n,), torch.int64), v(smoothing), v(pad), D)
+    lo, ls = oxe.xentropy_fwd(T(logits, (n, v(ld)), DT[v(dt)])[:, :vv], T(labels, (n,), torch.int64), v(smoothing), v(pad), D)
     put(T(losses, (n,), torch.float32), lo)
     put(T(lse, (n,), torch.float32), ls)
 
 
-def xent_bwd(gl, logits, lse, labels, gout, rows, vocab, smoothing, pad, dt, st):
+def xent_bwd(gl, logits, lse, labels, gout, rows, vocab, ld, ldg, smoothing, pad, dt, st):
     n, vv = v(rows), v(vocab)
-    g = oxe.xentropy_bwd(T(gl, (n,), torch.float32), T(logits, (n, vv), DT[v(dt)]), T(lse, (n,), torch.float32).to(D),
+    g = oxe.xentropy_bwd(T(gl, (n,), torch.float32), T(logits, (n, v(ld)), DT[v(dt)])[:, :vv], T(lse, (n,), torch.float32).to(D),
                          T(labels, (n,), torch.int64), v(smoothing), v(pad), D)
-    put(T(gout, (n, vv), DT[v(dt)]), g)
+    put(T(gout, (n, v(ldg)), DT[v(dt)])[:, :vv], g)
 
 
 def _ptrs(arr, n):

@@ -39,6 +39,7 @@ import test_zy_layers_gpu as tla  # noqa: E402
 import test_mlp_gpu as tm  # noqa: E402
 import test_staged_gpu as tst  # noqa: E402
 import test_zz_golden_gpu as tgold  # noqa: E402
+import test_zzb_generator_loss_gpu as tgen  # noqa: E402
 
 pytestmark = pytest.mark.skipif(not hostsim_build.available(), reason="no host C++ compiler with __bf16 (ROCm clang++)")
 CPU = torch.device("cpu")
@@ -365,9 +366,15 @@ def test_empty_inputs(mi355x, name):
 
 
 # ----------------------------------------------------------------------------- strided arguments
-@pytest.mark.parametrize("name", [n for n in dir(tstr) if n.startswith("test_")])
+@pytest.mark.parametrize("name", [n for n in dir(tstr) if n.startswith("test_") and "row_pitched" not in n])
 def test_strided_arguments(mi355x, name):
     getattr(tstr, name)(CPU)
+
+
+@pytest.mark.parametrize("dtype", [F16, torch.float32])
+@pytest.mark.parametrize("v,pitch,gpitch", [(1000, 1024, 1024), (517, 520, 576), (250, 251, 250)])
+def test_cross_entropy_on_row_pitched_logits(mi355x, dtype, v, pitch, gpitch):
+    tstr.test_cross_entropy_reads_and_writes_row_pitched_logits_in_place(CPU, dtype, v, pitch, gpitch)
 
 
 # ----------------------------------------------------------------------------- incremental decoding
@@ -381,6 +388,21 @@ def test_incremental_decoding(mi355x, dtype):
 def test_incremental_decoder_layer_with_beam_reordering(mi355x):
     tinc.test_self_attention_step_by_step(CPU, F16, 1)
     tinc.test_decoder_layer_step_by_step_with_beam_reordering(CPU)
+
+
+# ----------------------------------------------------------------------------- projection + loss in row chunks
+@pytest.mark.parametrize("dtype", HALVES)
+def test_chunked_projection_loss(mi355x, dtype):
+    tgen.test_chunked_projection_loss_matches_oracle_and_unchunked_operators(CPU, dtype, 80, 64, 1000, 32, True, 0.1)
+    tgen.test_chunked_projection_loss_matches_oracle_and_unchunked_operators(CPU, dtype, 33, 64, 2048, 8, True, 0.3)
+
+
+def test_chunked_projection_loss_module_and_validation(mi355x):
+    tgen.test_chunked_projection_loss_matches_oracle_and_unchunked_operators(CPU, F16, 64, 128, 517, 64, False, 0.0)
+    tgen.test_per_row_weights_and_no_gradient_for_frozen_weights(CPU)
+    tgen.test_validation_pass_counts_correct_predictions(CPU)
+    tgen.test_module_matches_the_reference_loss_assembly(CPU)
+    tgen.test_argument_checks_and_empty_batch(CPU)
 
 
 # ----------------------------------------------------------------------------- variants that are switched off by default

@@ -10,7 +10,8 @@ import pytest
 import torch
 import torch.nn.functional as F
 
-from oracle import attention, dropout_add, inputs, layer_norm, mlp, softmax_dropout, transformer_layers, xentropy
+from oracle import (attention, dropout_add, generator_loss, inputs, layer_norm, mlp, softmax_dropout, transformer_layers,
+                    xentropy)
 
 D = torch.float64
 
@@ -138,6 +139,44 @@ def test_xentropy_closed_forms():
     torch.testing.assert_close(loss0, lse0 - d["logits"].gather(1, d["labels"].unsqueeze(1)).squeeze(1))
     lu, _ = xentropy.xentropy_fwd(torch.zeros(3, 50, dtype=D), torch.tensor([4, 5, 6]), 0.1, -100, D)
     torch.testing.assert_close(lu, torch.full((3,), math.log(50.0), dtype=D))
+
+
+@pytest.mark.parametrize("bias", [True, False])
+def test_generator_loss_matches_library_and_autograd(bias):
+    # projection + loss against F.linear -> F.cross_entropy and autograd through both
+    g = torch.Generator().manual_seed(77)
+    n, e, v, eps, pad = 23, 12, 41, 0.1, 3
+    h = torch.randn(n, e, dtype=D, generator=g).requires_grad_()
+    w = (torch.randn(v, e, dtype=D, generator=g) * 0.3).requires_grad_()
+    b = (torch.randn(v, dtype=D, generator=g) * 0.1).requires_grad_() if bias else None
+    y = torch.randint(0, v, (n,), generator=g)
+    y[::5] = pad
+    gl = torch.rand(n, dtype=D, generator=g) + 0.5
+    z = F.linear(h, w, b)
+    lib = F.cross_entropy(z, y, ignore_index=pad, reduction="none", label_smoothing=eps)
+    lib.backward(gl)
+    loss, lse, am = generator_loss.generator_loss_fwd(h.detach(), w.detach(), None if b is None else b.detach(), y, eps, pad, D, D)
+    torch.testing.assert_close(loss, lib.detach(), rtol=1e-11, atol=1e-12)
+    torch.testing.assert_close(lse, torch.logsumexp(z.detach(), 1))
+    assert torch.equal(am, z.detach().argmax(1))
+    dh, dw, db = generator_loss.generator_loss_bwd(gl, h.detach(), w.detach(), None if b is None else b.detach(), y, eps, pad, D, D)
+    torch.testing.assert_close(dh, h.grad, rtol=1e-10, atol=1e-13)
+    torch.testing.assert_close(dw, w.grad, rtol=1e-10, atol=1e-13)
+    if bias:
+        torch.testing.assert_close(db, b.grad, rtol=1e-10, atol=1e-13)
+        assert abs(float(db.sum())) < 1e-12                   # every gradient row of the logits sums to zero
+    else:
+        assert db is None
+    assert (loss[y == pad] == 0).all() and (dh[y == pad] == 0).all()
+
+
+def test_generator_loss_rounds_the_logits_where_the_reference_stores_them():
+    g = torch.Generator().manual_seed(78)
+    h, w = torch.randn(8, 16, generator=g).bfloat16(), torch.randn(30, 16, generator=g).bfloat16()
+    y = torch.randint(0, 30, (8,), generator=g)
+    loss, _, _ = generator_loss.generator_loss_fwd(h, w, None, y, 0.0, -100, torch.bfloat16)
+    z = (h.float() @ w.float().t()).bfloat16()
+    torch.testing.assert_close(loss, F.cross_entropy(z.float(), y, reduction="none"))
 
 
 # ------------------------------------------------------------------ MLP

@@ -86,6 +86,32 @@ def test_mlp_and_cross_entropy_take_strided_tensors(dev):
     assert torch.equal(got, want)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("v,pitch,gpitch", [(1000, 1024, 1024), (517, 520, 576), (250, 251, 250)])
+def test_cross_entropy_reads_and_writes_row_pitched_logits_in_place(dev, dtype, v, pitch, gpitch):
+    # rows of `v` classes inside wider buffers: nothing is copied, and nothing beyond a row's classes is touched
+    x = inputs.xentropy_inputs(12, v, dtype, 0.1, 1, 0.25, seed=6)
+    big = torch.full((12, pitch), float("nan"), dtype=dtype, device=dev)
+    view = big[:, :v]
+    view.copy_(x["logits"])
+    labels, gl = x["labels"].to(dev), x["grad_loss"].to(dev)
+    widen = dtype != torch.float32
+    ref = xentropy_cuda.forward(x["logits"].to(dev), labels, 0.1, widen, padding_idx=1)
+    got = xentropy_cuda.forward(view, labels, 0.1, widen, padding_idx=1)
+    # the reduction order within a row depends on where its 16-byte boundaries fall: equal to rounding
+    for a, b in zip(got, ref):
+        torch.testing.assert_close(a, b, rtol=1e-5, atol=1e-5)
+    pad = x["labels"] == 1
+    assert pad.any() and (got[0].cpu()[pad] == 0).all()
+    want = xentropy_cuda.backward(gl, x["logits"].to(dev), ref[1], labels, 0.1, padding_idx=1)
+    gbig = torch.full((12, gpitch), 7.0, dtype=dtype, device=dev)
+    out = xentropy_cuda.backward(gl, view, ref[1], labels, 0.1, padding_idx=1, out=gbig[:, :v])
+    assert out.data_ptr() == gbig.data_ptr() and torch.equal(out, want)                 # elementwise: bit for bit
+    assert (gbig[:, v:] == 7.0).all() and (gbig.cpu()[pad][:, :v] == 0).all()
+    with pytest.raises(RuntimeError):
+        xentropy_cuda.backward(gl, view, ref[1], labels, 0.1, padding_idx=1, out=gbig[:, :v - 1])
+
+
 def test_operators_that_work_in_place_or_on_rows_refuse_strided_tensors(dev):
     x = strided(torch.randn(8, 64), dev)
     w = torch.ones(64, device=dev)
