@@ -137,6 +137,10 @@ int nmtg_softmax_dropout_bwd(const void* grad_dropped, const void* saved, int sa
  * reference's tensors are dense: ld_logits = vocab), labels int64 [rows]; losses, lse fp32 [rows];
  * grad_loss fp32 [rows]; grad_logits [rows, vocab] in the logits dtype with row pitch ld_grad;
  * elements between vocab and the pitch are neither read nor written. fp32 accumulation.
+ * The backward is elementwise once lse is known, so it also works on a slice of the classes:
+ * the `vocab` columns handed in are classes [class_offset, class_offset + vocab) of
+ * total_classes (labels stay global; smoothing spreads over total_classes). The whole row:
+ * class_offset = 0, total_classes = vocab.
  * ------------------------------------------------------------------------------------------ */
 int nmtg_xentropy_fwd(const void* logits, const int64_t* labels, float* losses, float* lse,
                       int64_t rows, int64_t vocab, int64_t ld_logits, float smoothing,
@@ -144,8 +148,9 @@ int nmtg_xentropy_fwd(const void* logits, const int64_t* labels, float* losses, 
 
 int nmtg_xentropy_bwd(const float* grad_loss, const void* logits, const float* lse,
                       const int64_t* labels, void* grad_logits, int64_t rows, int64_t vocab,
-                      int64_t ld_logits, int64_t ld_grad, float smoothing, int64_t padding_idx,
-                      int dtype, void* stream);
+                      int64_t ld_logits, int64_t ld_grad, int64_t class_offset,
+                      int64_t total_classes, float smoothing, int64_t padding_idx, int dtype,
+                      void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Strided-batched GEMM on the MFMA units (fp16 / bf16 in and out, fp32 accumulation), row-major:

@@ -145,14 +145,17 @@ template <typename T, bool VEC>
 __global__ __launch_bounds__(XE_THREADS) void xentropy_bwd_kernel(
     const float* __restrict__ grad_loss, const T* __restrict__ logits, const float* __restrict__ lse_in,
     const int64_t* __restrict__ labels, T* __restrict__ grad_logits, int64_t vocab, int64_t ld, int64_t ld_grad,
-    float smoothing, int64_t padding_idx) {
+    int64_t class_offset, int64_t total_classes, float smoothing, int64_t padding_idx) {
   constexpr int EPV = 16 / sizeof(T);
   const int64_t row = blockIdx.x;
   const T* x = logits + row * ld;
   T* dx = grad_logits + row * ld_grad;
   const int tid = threadIdx.x;
-  const int64_t y = labels[row];
-  const float g = (y == padding_idx) ? 0.f : grad_loss[row];
+  // the row holds classes [class_offset, class_offset + vocab) of total_classes: y is the label's position in the row
+  // (outside [0, vocab) if the label belongs to another slice)
+  const bool padded = labels[row] == padding_idx;
+  const int64_t y = labels[row] - class_offset;
+  const float g = padded ? 0.f : grad_loss[row];
 
   const uintptr_t addr = reinterpret_cast<uintptr_t>(dx);
   int64_t head = VEC ? static_cast<int64_t>(((16 - (addr & 15)) & 15) / sizeof(T)) : vocab;
@@ -160,7 +163,7 @@ __global__ __launch_bounds__(XE_THREADS) void xentropy_bwd_kernel(
   const int64_t nvec = (vocab - head) / EPV;
   const int64_t tail0 = head + nvec * EPV;
 
-  if (y == padding_idx) {  // exact zeros, logits untouched
+  if (padded) {  // exact zeros, logits untouched
     for (int64_t c = tid; c < head; c += XE_THREADS) dx[c] = elem<T>::from_float(0.f);
     const float z[EPV] = {};
     for (int64_t i = tid; i < nvec; i += XE_THREADS) store_pack<T, EPV>(dx + head + i * EPV, z);
@@ -169,7 +172,7 @@ __global__ __launch_bounds__(XE_THREADS) void xentropy_bwd_kernel(
   }
 
   const float nlse = -lse_in[row] * LOG2E;
-  const float sm = smoothing / static_cast<float>(vocab);
+  const float sm = smoothing / static_cast<float>(total_classes);
   const float onem = 1.f - smoothing;
   auto one = [&](int64_t c) {
     float v = __builtin_amdgcn_exp2f(fmaf(elem<T>::to_float(x[c]), LOG2E, nlse)) - sm;
@@ -241,11 +244,15 @@ extern "C" int nmtg_xentropy_fwd(const void* logits, const int64_t* labels, floa
 
 extern "C" int nmtg_xentropy_bwd(const float* grad_loss, const void* logits, const float* lse, const int64_t* labels,
                                  void* grad_logits, int64_t rows, int64_t vocab, int64_t ld_logits, int64_t ld_grad,
-                                 float smoothing, int64_t padding_idx, int dtype, void* stream) {
+                                 int64_t class_offset, int64_t total_classes, float smoothing, int64_t padding_idx,
+                                 int dtype, void* stream) {
   NMTG_REQUIRE(rows >= 0 && rows <= INT32_MAX, "xentropy_bwd: bad row count %lld", (long long)rows);
   NMTG_REQUIRE(vocab > 0, "xentropy_bwd: number of classes must be positive");
   NMTG_REQUIRE(ld_logits >= vocab && ld_grad >= vocab, "xentropy_bwd: a row pitch (%lld, %lld) is below the number of classes %lld",
                (long long)ld_logits, (long long)ld_grad, (long long)vocab);
+  NMTG_REQUIRE(class_offset >= 0 && total_classes >= class_offset + vocab,
+               "xentropy_bwd: classes [%lld, %lld) do not lie within %lld classes", (long long)class_offset,
+               (long long)(class_offset + vocab), (long long)total_classes);
   if (rows == 0) return 0;
   NMTG_REQUIRE(grad_loss && logits && lse && labels && grad_logits, "xentropy_bwd: null pointer argument");
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -259,10 +266,10 @@ extern "C" int nmtg_xentropy_bwd(const float* grad_loss, const void* logits, con
       dtype, T,
       if (vec) hipLaunchKernelGGL((xentropy_bwd_kernel<T, true>), dim3(static_cast<unsigned>(rows)), dim3(XE_THREADS), 0, st,
                                   grad_loss, static_cast<const T*>(logits), lse, labels, static_cast<T*>(grad_logits), vocab,
-                                  ld_logits, ld_grad, smoothing, padding_idx);
+                                  ld_logits, ld_grad, class_offset, total_classes, smoothing, padding_idx);
       else hipLaunchKernelGGL((xentropy_bwd_kernel<T, false>), dim3(static_cast<unsigned>(rows)), dim3(XE_THREADS), 0, st,
                               grad_loss, static_cast<const T*>(logits), lse, labels, static_cast<T*>(grad_logits), vocab,
-                              ld_logits, ld_grad, smoothing, padding_idx));
+                              ld_logits, ld_grad, class_offset, total_classes, smoothing, padding_idx));
   NMTG_CHECK_LAUNCH("xentropy_bwd");
   return 0;
 }

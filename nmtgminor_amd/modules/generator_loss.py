@@ -5,18 +5,20 @@ onmt/modules/base_seq2seq.py:26-47) and hands the whole logits tensor to the los
 (CrossEntropyLossBase._compute_loss, onmt/modules/loss.py:60-109, which calls
 SoftmaxCrossEntropyLoss.apply(logits, labels, smoothing, padding_idx, half_to_float)). At a vocabulary of 250 054 and
 16 384 target positions that tensor and its gradient are 8.2 GB each. Here the same two kernels (the MFMA projection and
-the cross-entropy) run over `chunk_rows` positions at a time: the forward keeps only the per-row losses and
-log-sum-exp, the backward recomputes each chunk's logits, turns them into their gradient and contracts that at once
-with the weight (gradient of the states) and with the states (weight gradient, accumulated over the chunks in fp32).
-Per-row results are those of the unchunked pair of operators; arbitrary per-row upstream gradients (loss weights) are
-supported because nothing of the backward is precomputed in the forward.
+the cross-entropy) run over pieces of it. The forward walks the rows `chunk_rows` at a time (a row's log-sum-exp needs
+the whole row) and keeps only the per-row losses and log-sum-exp. The backward is elementwise once the log-sum-exp is
+known, so it walks the vocabulary in column slices over all rows: it recomputes a slice's logits, turns them into
+their gradient and contracts that at once with the states (the slice's weight gradient: complete, written once) and
+with the slice's weights (gradient of the states, [N, E], summed over the slices in fp32). Per-row results are those of
+the unchunked pair of operators to rounding; arbitrary per-row upstream gradients (loss weights) are supported because
+nothing of the backward is precomputed in the forward.
 
 The chunk buffers have a row pitch of the vocabulary rounded up to 64 elements, so that the projection's stores and the
 two contractions that read the logits gradient move 16 bytes per access whatever the vocabulary size (250 054 is not a
 multiple of 4); the cross-entropy kernels read and write the first V elements of each pitched row in place.
 
-Beyond the kernels this module only slices, accumulates the weight gradient (`add_` in fp32) and sums the bias
-gradient (`sum`); those are device-side PyTorch calls on already computed chunks.
+Beyond the kernels this module only slices, sums the per-slice gradients of the states (`add_` in fp32, [N, E]) and
+the bias gradient (`sum` over a slice's rows); those are device-side PyTorch calls on already computed pieces.
 """
 import torch
 import torch.nn as nn
@@ -51,6 +53,12 @@ def _chunk_buffer(rows, v, like):
     """[rows, v] view of a buffer whose row pitch is v rounded up to 64 elements."""
     pitch = (v + 63) // 64 * 64
     return torch.empty(rows, pitch, dtype=like.dtype, device=like.device)[:, :v]
+
+
+def _slice_columns(n, v, chunk_rows):
+    """Columns per vocabulary slice of the backward: a [n, columns] buffer as large as the forward's [chunk_rows, v]
+    one, in whole groups of 64 columns."""
+    return max(64, (min(n, chunk_rows) * ((v + 63) // 64 * 64) // n) // 64 * 64)
 
 
 def _logits(hidden, weight, bias, r0, r1, buf):
@@ -89,24 +97,43 @@ class LinearSoftmaxCrossEntropy(torch.autograd.Function):
         need_b = bias is not None and ctx.needs_input_grad[2]
         n, v = hidden.size(0), weight.size(0)
         grad_loss = grad_loss.contiguous().float()
-        dh = torch.empty_like(hidden) if need_h else None
-        dw = torch.zeros(weight.shape, dtype=torch.float32, device=weight.device) if need_w else None
-        db = torch.zeros(v, dtype=torch.float32, device=weight.device) if need_b else None
+        dh = dw = db = None
+        if need_w:
+            dw = torch.empty_like(weight) if n > 0 else torch.zeros_like(weight)
+        if need_b:
+            db = torch.empty_like(bias) if n > 0 else torch.zeros_like(bias)
+        if need_h:
+            dh = torch.empty_like(hidden)
         if n > 0 and (need_h or need_w or need_b):
-            buf = _chunk_buffer(min(n, ctx.chunk_rows), v, hidden)
-            gbuf = _chunk_buffer(min(n, ctx.chunk_rows), v, hidden)
-            for r0, r1 in _chunks(n, ctx.chunk_rows):
-                z = _logits(hidden, weight, bias, r0, r1, buf)                       # the forward's logits again
-                dz = xentropy_cuda.backward(grad_loss[r0:r1], z, lse[r0:r1], labels[r0:r1], ctx.smoothing,
-                                            padding_idx=ctx.padding_idx, out=gbuf[:r1 - r0])
-                if need_h:
-                    linear_gemm.gemm(dz, weight, out=dh[r0:r1])                      # [n, V] x [V, E]
+            # Given the log-sum-exp of each row the logits gradient is elementwise, so the backward walks the
+            # vocabulary in slices of whole columns: a slice's weight and bias gradients are complete (contracted over
+            # all rows at once, written once) and only the small [N, E] gradient of the states is summed over slices.
+            cols = _slice_columns(n, v, ctx.chunk_rows)
+            buf = _chunk_buffer(n, min(v, cols), hidden)
+            gbuf = _chunk_buffer(n, min(v, cols), hidden)
+            dh32 = None
+            for c0 in range(0, v, cols):
+                c1 = min(v, c0 + cols)
+                w_c = weight[c0:c1]
+                z = linear_gemm.gemm(hidden, w_c, trans_b=True, bias=None if bias is None else bias[c0:c1],
+                                     out=buf[:, :c1 - c0])                           # the forward's logits again
+                dz = xentropy_cuda.backward(grad_loss, z, lse, labels, ctx.smoothing, padding_idx=ctx.padding_idx,
+                                            out=gbuf[:, :c1 - c0], class_offset=c0, total_classes=v)
                 if need_w:
-                    dw.add_(linear_gemm.gemm(dz, hidden[r0:r1], trans_a=True))       # [V, n] x [n, E]
+                    linear_gemm.gemm(dz, hidden, trans_a=True, out=dw[c0:c1])        # [V_c, N] x [N, E]
                 if need_b:
-                    db.add_(dz.sum(dim=0, dtype=torch.float32))
-        return (dh, dw.to(weight.dtype) if need_w else None, db.to(bias.dtype) if need_b else None,
-                None, None, None, None)
+                    db[c0:c1] = dz.sum(dim=0, dtype=torch.float32)
+                if need_h:
+                    part = linear_gemm.gemm(dz, w_c)                                 # [N, V_c] x [V_c, E]
+                    if c0 == 0 and c1 == v:
+                        dh = part
+                    elif dh32 is None:
+                        dh32 = part.float()
+                    else:
+                        dh32.add_(part)
+            if need_h and dh32 is not None:
+                dh.copy_(dh32)
+        return dh, dw, db, None, None, None, None
 
 
 def linear_cross_entropy_eval(hidden, weight, bias, labels, padding_idx=-100, chunk_rows=DEFAULT_CHUNK_ROWS):

@@ -51,8 +51,11 @@ def forward(logits, labels, smoothing, half_to_float=False, *, padding_idx=None)
     return [losses, lse]
 
 
-def backward(grad_loss, logits, max_log_sum_exp, labels, smoothing, *, padding_idx=None, out=None):
-    """-> grad_logits (logits dtype and shape); written into `out` when given."""
+def backward(grad_loss, logits, max_log_sum_exp, labels, smoothing, *, padding_idx=None, out=None, class_offset=0,
+             total_classes=None):
+    """-> grad_logits (logits dtype and shape); written into `out` when given. With `class_offset` / `total_classes`
+    the columns of `logits` are the slice [class_offset, class_offset + logits.size(1)) of that many classes (the
+    backward is elementwise given the log-sum-exp of the whole row); labels stay global."""
     L.require_cuda(grad_loss, logits, max_log_sum_exp, labels)
     _check(labels.dtype == torch.int64, "Label type should be CUDA Long")
     _check(logits.dim() == 2 and labels.dim() == 1 and logits.size(0) == labels.size(0), "shape mismatch")
@@ -71,6 +74,7 @@ def backward(grad_loss, logits, max_log_sum_exp, labels, smoothing, *, padding_i
         grad_logits = out
     labels = labels.contiguous()                          # bound to a name: a temporary would be freed before the kernel reads it
     L.call("nmtg_xentropy_bwd", L.ptr(grad_loss), L.ptr(logits), L.ptr(lse), L.ptr(labels),
-           L.ptr(grad_logits), L.i64(n), L.i64(v), L.i64(logits.stride(0)), L.i64(grad_logits.stride(0)), L.f32(smoothing),
+           L.ptr(grad_logits), L.i64(n), L.i64(v), L.i64(logits.stride(0)), L.i64(grad_logits.stride(0)),
+           L.i64(class_offset), L.i64(v if total_classes is None else total_classes), L.f32(smoothing),
            L.i64(_NO_PAD if padding_idx is None else padding_idx), L.i32(L.dtype_code(logits)), L.stream_of(logits))
     return grad_logits

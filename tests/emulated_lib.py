@@ -134,11 +134,14 @@ def xent_fwd(logits, labels, losses, lse, rows, vocab, ld, smoothing, pad, dt, s
     put(T(lse, (n,), torch.float32), ls)
 
 
-def xent_bwd(gl, logits, lse, labels, gout, rows, vocab, ld, ldg, smoothing, pad, dt, st):
-    n, vv = v(rows), v(vocab)
-    g = oxe.xentropy_bwd(T(gl, (n,), torch.float32), T(logits, (n, v(ld)), DT[v(dt)])[:, :vv], T(lse, (n,), torch.float32).to(D),
+def xent_bwd(gl, logits, lse, labels, gout, rows, vocab, ld, ldg, c0, total, smoothing, pad, dt, st):
+    n, vv, c0, total = v(rows), v(vocab), v(c0), v(total)
+    # a slice of the classes: embed it in a row of `total` classes (the other columns do not influence the slice)
+    z = torch.zeros(n, total, dtype=D)
+    z[:, c0:c0 + vv] = T(logits, (n, v(ld)), DT[v(dt)])[:, :vv].to(D)
+    g = oxe.xentropy_bwd(T(gl, (n,), torch.float32), z, T(lse, (n,), torch.float32).to(D),
                          T(labels, (n,), torch.int64), v(smoothing), v(pad), D)
-    put(T(gout, (n, v(ldg)), DT[v(dt)])[:, :vv], g)
+    put(T(gout, (n, v(ldg)), DT[v(dt)])[:, :vv], g[:, c0:c0 + vv])
 
 
 def _ptrs(arr, n):

@@ -398,9 +398,14 @@ def test_empty_inputs(mi355x, name):
 
 
 # ----------------------------------------------------------------------------- strided arguments
-@pytest.mark.parametrize("name", [n for n in dir(tstr) if n.startswith("test_") and "row_pitched" not in n])
+@pytest.mark.parametrize("name", [n for n in dir(tstr) if n.startswith("test_") and "row_pitched" not in n and "slice_of" not in n])
 def test_strided_arguments(mi355x, name):
     getattr(tstr, name)(CPU)
+
+
+@pytest.mark.parametrize("dtype", [BF16, torch.float32])
+def test_cross_entropy_backward_on_a_slice_of_the_classes(mi355x, dtype):
+    tstr.test_cross_entropy_backward_on_a_slice_of_the_classes(CPU, dtype)
 
 
 @pytest.mark.parametrize("dtype", [F16, torch.float32])

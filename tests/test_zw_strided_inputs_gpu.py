@@ -112,6 +112,21 @@ def test_cross_entropy_reads_and_writes_row_pitched_logits_in_place(dev, dtype, 
         xentropy_cuda.backward(gl, view, ref[1], labels, 0.1, padding_idx=1, out=gbig[:, :v - 1])
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_cross_entropy_backward_on_a_slice_of_the_classes(dev, dtype):
+    # given the log-sum-exp of the whole row the backward is elementwise: any column slice gives the full result's columns
+    v = 1000
+    x = inputs.xentropy_inputs(10, v, dtype, 0.1, 1, 0.2, seed=8)
+    logits, labels, gl = x["logits"].to(dev), x["labels"].to(dev), x["grad_loss"].to(dev)
+    _, lse = xentropy_cuda.forward(logits, labels, 0.1, dtype != torch.float32, padding_idx=1)
+    want = xentropy_cuda.backward(gl, logits, lse, labels, 0.1, padding_idx=1)
+    for c0, c1 in ((0, 384), (384, 768), (768, 1000), (123, 130)):
+        got = xentropy_cuda.backward(gl, logits[:, c0:c1], lse, labels, 0.1, padding_idx=1, class_offset=c0, total_classes=v)
+        assert got.shape == (10, c1 - c0) and torch.equal(got, want[:, c0:c1]), (c0, c1)
+    with pytest.raises(RuntimeError):
+        xentropy_cuda.backward(gl, logits[:, 900:], lse, labels, 0.1, padding_idx=1, class_offset=950, total_classes=v)
+
+
 def test_operators_that_work_in_place_or_on_rows_refuse_strided_tensors(dev):
     x = strided(torch.randn(8, 64), dev)
     w = torch.ones(64, device=dev)
