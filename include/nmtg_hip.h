@@ -277,6 +277,50 @@ int nmtg_encdec_attn_bwd(const void* grad_out, const void* ctx, const void* drop
                          int64_t tk, int64_t b, int64_t e, int heads, int dtype, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Column sums of a row-major matrix: out[c] = sum_r x[r * ld + c], fp32 accumulation in a fixed
+ * order (partial sums per block of rows, then one sum over the partials), result in the dtype
+ * of x. The bias gradients of the reference's linear layers: torch.sum(grads, 0)
+ * (onmt/modules/optimized/relative_self_attention_func.py:562-563, :715) and the bias gradient
+ * of linear_blaslt.backward (onmt/modules/extensions/mlp_blaslt/linear.cpp:59-104).
+ * workspace: fp32 scratch of nmtg_colsum_workspace_bytes(rows, cols) bytes. rows, cols < 2^31.
+ * ------------------------------------------------------------------------------------------ */
+int64_t nmtg_colsum_workspace_bytes(int64_t rows, int64_t cols);
+
+int nmtg_colsum(const void* x, int64_t rows, int64_t cols, int64_t ld, void* out, void* workspace,
+                int64_t workspace_bytes, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Elementwise pieces of self-attention with relative position encodings (Transformer-XL form).
+ * Reference: RelativeShift.forward / backward and the bias additions and the sum of the two score
+ *   terms in RelativeSelfAttnFunc (onmt/modules/optimized/relative_self_attention_func.py:26-76,
+ *   :210-217, :246-253, :621-630); the products around them are nmtg_gemm calls.
+ *
+ * nmtg_rel_query_bias: rw_q[r][d] = q[r * ld_q + d] + r_w_bias[(r % heads) * head_dim + d] and
+ *   rr_q likewise with r_r_bias, for r < rows (rows = len_q * batch * heads: the queries as they
+ *   lie inside the in-projection output, ld_q = 3 * head_dim there), d < head_dim. rw_q, rr_q
+ *   dense [rows, head_dim]. The sums are rounded once to the dtype, as an elementwise add does.
+ *
+ * nmtg_rel_shift_add: scores[b][i][j] += shift(bd)[b][i][j] for j < len_k, in place, where
+ *   shift views bd[b] (dense [len_q, len_r], len_r >= len_k) with a zero column in front as
+ *   [len_r + 1, len_q], drops the first row and reads the rest as [len_q, len_r]: with
+ *   p = i * len_r + j + len_q, i2 = p / (len_r + 1), c = p % (len_r + 1) the value is 0 if c == 0
+ *   and bd[b][i2][c - 1] otherwise.
+ *
+ * nmtg_rel_shift_bwd: the adjoint, grad_bd[b][i2][c - 1] = grad_scores[b][i][j] at the same
+ *   correspondence (0 where j >= len_k or where p < len_q); grad_bd dense [batch, len_q, len_r].
+ * dtype: NMTG_F16, NMTG_BF16 or NMTG_F32.
+ * ------------------------------------------------------------------------------------------ */
+int nmtg_rel_query_bias(const void* q, int64_t ld_q, const void* r_w_bias, const void* r_r_bias,
+                        void* rw_q, void* rr_q, int64_t rows, int64_t heads, int64_t head_dim,
+                        int dtype, void* stream);
+
+int nmtg_rel_shift_add(void* scores, const void* bd, int64_t batch, int64_t len_q, int64_t len_k,
+                       int64_t len_r, int dtype, void* stream);
+
+int nmtg_rel_shift_bwd(const void* grad_scores, void* grad_bd, int64_t batch, int64_t len_q,
+                       int64_t len_k, int64_t len_r, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Per-kernel timing for benchmarks (no counterpart in the reference, whose tests time whole ops
  * with CUDA events, e.g. onmt/modules/test_layer_norm.py:14-31). Between nmtg_trace_begin() and
  * nmtg_trace_end() every kernel the library enqueues is bracketed by two HIP events on its

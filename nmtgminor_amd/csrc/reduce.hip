@@ -83,3 +83,25 @@ int tail_launch(const ReduceTail& t, int dtype, hipStream_t st) {
 }
 
 }  // namespace nmtg
+
+using namespace nmtg;
+
+extern "C" int64_t nmtg_colsum_workspace_bytes(int64_t rows, int64_t cols) {
+  if (rows <= 0 || cols <= 0 || rows > INT32_MAX || cols > INT32_MAX) return 0;
+  return static_cast<int64_t>(colsum_parts(static_cast<int>(rows))) * cols * static_cast<int64_t>(sizeof(float));
+}
+
+extern "C" int nmtg_colsum(const void* x, int64_t rows, int64_t cols, int64_t ld, void* out, void* workspace,
+                           int64_t workspace_bytes, int dtype, void* stream) {
+  NMTG_REQUIRE(rows > 0 && rows <= INT32_MAX && cols >= 0 && cols <= INT32_MAX,
+               "colsum: bad sizes (rows %lld, columns %lld); a sum over no rows is the caller's zero fill", (long long)rows,
+               (long long)cols);
+  NMTG_REQUIRE(ld >= cols, "colsum: row pitch %lld below the number of columns %lld", (long long)ld, (long long)cols);
+  if (cols == 0) return 0;
+  NMTG_REQUIRE(x && out, "colsum: null pointer argument");
+  NMTG_REQUIRE(workspace && workspace_bytes >= nmtg_colsum_workspace_bytes(rows, cols),
+               "colsum: workspace of %lld bytes, need %lld", (long long)workspace_bytes,
+               (long long)nmtg_colsum_workspace_bytes(rows, cols));
+  return colsum_run(dtype, x, ld, static_cast<int>(rows), static_cast<int>(cols), static_cast<float*>(workspace), out,
+                    static_cast<hipStream_t>(stream));
+}

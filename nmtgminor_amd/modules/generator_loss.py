@@ -17,8 +17,8 @@ The chunk buffers have a row pitch of the vocabulary rounded up to 64 elements, 
 two contractions that read the logits gradient move 16 bytes per access whatever the vocabulary size (250 054 is not a
 multiple of 4); the cross-entropy kernels read and write the first V elements of each pitched row in place.
 
-Beyond the kernels this module only slices, sums the per-slice gradients of the states (`add_` in fp32, [N, E]) and
-the bias gradient (`sum` over a slice's rows); those are device-side PyTorch calls on already computed pieces.
+Beyond the kernels (projection, cross-entropy, column sums for the bias gradient) this module only slices and sums the
+per-slice gradients of the states (`add_` in fp32, [N, E]): a device-side PyTorch call on already computed pieces.
 """
 import torch
 import torch.nn as nn
@@ -122,7 +122,10 @@ class LinearSoftmaxCrossEntropy(torch.autograd.Function):
                 if need_w:
                     linear_gemm.gemm(dz, hidden, trans_a=True, out=dw[c0:c1])        # [V_c, N] x [N, E]
                 if need_b:
-                    db[c0:c1] = dz.sum(dim=0, dtype=torch.float32)
+                    if db.dtype == dz.dtype:
+                        linear_gemm.colsum(dz, out=db[c0:c1])                        # fixed-order fp32 column sums
+                    else:
+                        db[c0:c1] = linear_gemm.colsum(dz)
                 if need_h:
                     part = linear_gemm.gemm(dz, w_c)                                 # [N, V_c] x [V_c, E]
                     if c0 == 0 and c1 == v:

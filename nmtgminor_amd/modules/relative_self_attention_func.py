@@ -1,0 +1,163 @@
+"""Self-attention with relative position encodings (Transformer-XL form) on the HIP kernels.
+
+Mirrors RelativeShift, RelativeSelfAttnFunc and relative_self_attn_func of the reference
+(onmt/modules/optimized/relative_self_attention_func.py:26-76, :79-726, :738-766): the same 21 positional arguments and
+21 gradient slots. Every product is an MFMA GEMM (nmtg_gemm through native/linear_gemm.py and native/linear_blaslt.py),
+the additions of r_w_bias / r_r_bias, the relative shift with the sum of the two score terms and the shift's adjoint are
+the kernels of native/relative_position.py, softmax + dropout is the fused kernel of the other attention ops (mask fused,
+probabilities recomputed from the saved scores in the backward) and the bias gradients are column-sum kernels. What is
+left to PyTorch: views, allocation, and one elementwise add that joins the two query-gradient terms.
+
+Covered: sinusoidal positions projected by pos_weights (learnable_pos=False), key-padding or time mask, training and
+inference, fp16 / bf16. Not covered, and raising instead of falling back: learnable position embeddings, incremental
+decoding. `recompute` is accepted and gives the same numbers; the intermediate tensors are kept either way. A 22nd
+optional argument replays an explicit dropout keep-mask."""
+import torch
+
+from ..native import linear_blaslt, linear_gemm, mask_softmax_dropout_cuda as softmax_native, relative_position
+from ._autocast import cast_if_autocast_enabled, no_autocast
+
+
+class RelativeShift(object):
+    """x [B, len_q, len_r]: zero column in front, read as [B, len_r + 1, len_q], first row dropped
+    (relative_self_attention_func.py:26-76). Only the batch-first form exists, as in the reference."""
+
+    @staticmethod
+    def forward(x, batch_first, emb_last):
+        assert len(x.shape) == 3, "Input must have 3 dimensions B x len_q x len_r or len_q x len_r x demb!"
+        assert (batch_first or emb_last) and not (batch_first and emb_last), \
+            "Batch first and Embedding last must be mutually exclusive"
+        if not batch_first:
+            raise NotImplementedError
+        x = x.contiguous()
+        return relative_position.shift_add_(torch.zeros_like(x), x)
+
+    @staticmethod
+    def backward(grad_x, batch_first, emb_last):
+        if not batch_first:
+            raise NotImplementedError
+        return relative_position.shift_backward(grad_x, grad_x.size(2))
+
+
+def _mask_kwargs(mask, use_time_mask):
+    if mask is None:
+        return {}
+    if use_time_mask:
+        assert mask.dim() == 2, "Timing mask is not 2D!"
+        return dict(time_mask=mask)
+    return dict(pad_mask=mask)
+
+
+class RelativeSelfAttnFunc(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, inputs, pos, use_time_mask, is_training, heads, input_weights, output_weights, pos_weights,
+                input_biases, output_biases, pos_biases, r_w_bias, r_r_bias, mask, dropout_prob, incremental,
+                incremental_cache, low_precision, learnable_pos, return_coverage, recompute, dropout_mask=None):
+        if learnable_pos:
+            raise NotImplementedError("relative_self_attn_func: learnable position embeddings have no HIP path")
+        if incremental:
+            raise NotImplementedError("relative_self_attn_func: incremental decoding has no HIP path")
+        inputs = inputs.contiguous()
+        len_q, bsz, embed = inputs.shape
+        head_dim = embed // heads
+        scale = head_dim ** -0.5
+        if pos.size(1) == 1:
+            pos = pos.repeat(1, bsz, 1)          # one position projection per batch column, as the reference lays it out
+        pos = pos.contiguous()
+        len_r = pos.size(0)
+        if len_r < len_q:
+            raise RuntimeError("relative_self_attn_func: %d relative positions for %d keys" % (len_r, len_q))
+        mask_kw = _mask_kwargs(mask, use_time_mask)
+
+        lin = linear_blaslt.forward(inputs, input_weights, input_biases)                  # [T, B, 3E]
+        pos_lin = linear_blaslt.forward(pos, pos_weights, pos_biases)                     # [R, B, E]
+        lin4 = lin.view(len_q, bsz * heads, 3, head_dim)
+        queries, keys, values = lin4[:, :, 0, :], lin4[:, :, 1, :], lin4[:, :, 2, :]
+        r_head_k = pos_lin.view(len_r, bsz * heads, head_dim)
+        rw_head_q, rr_head_q = relative_position.query_bias(queries, r_w_bias, r_r_bias, heads)
+
+        # AC = (q + r_w_bias) k^T, BD = shift((q + r_r_bias) r_k^T), both scaled by the GEMM
+        scores = linear_gemm.gemm(rw_head_q.transpose(0, 1), keys.transpose(0, 1), trans_b=True, alpha=scale)
+        matmul_bd = linear_gemm.gemm(rr_head_q.transpose(0, 1), r_head_k.transpose(0, 1), trans_b=True, alpha=scale)
+        relative_position.shift_add_(scores, matmul_bd)                                   # [B*H, T, T]
+        del matmul_bd
+
+        dmask, _, dropped = softmax_native.forward(is_training, heads, scores, dropout_prob, dropout_mask=dropout_mask,
+                                                   want_softmax=False, **mask_kw)
+        matmul2_results = torch.empty(len_q, bsz * heads, head_dim, dtype=inputs.dtype, device=inputs.device)
+        linear_gemm.gemm(dropped, values.transpose(0, 1), out=matmul2_results.transpose(0, 1))
+        matmul2_results = matmul2_results.view(len_q, bsz, embed)
+        outputs = linear_blaslt.forward(matmul2_results, output_weights, output_biases)
+
+        ctx.heads, ctx.p, ctx.scale = heads, dropout_prob if is_training else 0.0, scale
+        ctx.use_time_mask, ctx.return_coverage = use_time_mask, return_coverage
+        ctx.save_for_backward(inputs, pos, input_weights, output_weights, pos_weights, lin, pos_lin, rw_head_q, rr_head_q,
+                              scores, dropped, dmask, matmul2_results, mask)
+        if return_coverage:
+            ctx.mark_non_differentiable(dropped)
+            return outputs, dropped
+        return outputs
+
+    @staticmethod
+    def backward(ctx, *output_grads):
+        (inputs, pos, input_weights, output_weights, pos_weights, lin, pos_lin, rw_head_q, rr_head_q, scores, dropped,
+         dmask, matmul2_results, mask) = ctx.saved_tensors
+        heads, p, scale = ctx.heads, ctx.p, ctx.scale
+        output_grads = output_grads[0].contiguous()
+        len_q, bsz, embed = inputs.shape
+        head_dim = embed // heads
+        len_r = pos.size(0)
+        lin4 = lin.view(len_q, bsz * heads, 3, head_dim)
+        keys, values = lin4[:, :, 1, :], lin4[:, :, 2, :]
+        r_head_k = pos_lin.view(len_r, bsz * heads, head_dim)
+
+        output_lin_grads, output_weight_grads, output_bias_grads = \
+            linear_blaslt.backward(matmul2_results, output_weights, output_grads, True)
+        output_lin_grads = output_lin_grads.view(len_q, bsz * heads, head_dim).transpose(0, 1)      # [B*H, T, D]
+
+        lin_grads = torch.empty_like(lin4)
+        queries_grads, keys_grads, values_grads = lin_grads[:, :, 0, :], lin_grads[:, :, 1, :], lin_grads[:, :, 2, :]
+        matmul2_dgrad1 = linear_gemm.gemm(output_lin_grads, values.transpose(0, 1), trans_b=True)  # [B*H, T, T]
+        linear_gemm.gemm(dropped, output_lin_grads, trans_a=True, out=values_grads.transpose(0, 1))
+        # dropout and softmax backward in one kernel, probabilities recomputed from the saved scores (mask fused)
+        score_grads = softmax_native.backward_recompute(heads, matmul2_dgrad1, None, scores, dmask, p,
+                                                        **_mask_kwargs(mask, ctx.use_time_mask))
+        del matmul2_dgrad1
+
+        # the score gradient flows to both terms: AC directly, BD through the adjoint of the shift
+        queries_grads_ac = torch.empty(len_q, bsz * heads, head_dim, dtype=lin.dtype, device=lin.device)
+        linear_gemm.gemm(score_grads, keys.transpose(0, 1), alpha=scale, out=queries_grads_ac.transpose(0, 1))
+        linear_gemm.gemm(score_grads, rw_head_q.transpose(0, 1), trans_a=True, alpha=scale, out=keys_grads.transpose(0, 1))
+        r_w_bias_grads = linear_gemm.colsum(queries_grads_ac.view(len_q * bsz, embed)).view(heads, head_dim)
+
+        matmul_bd_grads = relative_position.shift_backward(score_grads, len_r)                     # [B*H, T, R]
+        del score_grads
+        queries_grads_bd = torch.empty_like(queries_grads_ac)
+        linear_gemm.gemm(matmul_bd_grads, r_head_k.transpose(0, 1), alpha=scale, out=queries_grads_bd.transpose(0, 1))
+        r_head_k_grad = torch.empty(len_r, bsz * heads, head_dim, dtype=lin.dtype, device=lin.device)
+        linear_gemm.gemm(matmul_bd_grads, rr_head_q.transpose(0, 1), trans_a=True, alpha=scale,
+                         out=r_head_k_grad.transpose(0, 1))
+        r_r_bias_grads = linear_gemm.colsum(queries_grads_bd.view(len_q * bsz, embed)).view(heads, head_dim)
+        torch.add(queries_grads_ac, queries_grads_bd, out=queries_grads)
+
+        _, pos_weight_grads, pos_bias_grads = linear_blaslt.backward(pos, pos_weights, r_head_k_grad.view(len_r, bsz, embed),
+                                                                     False)
+        input_grads, input_weight_grads, input_bias_grads = \
+            linear_blaslt.backward(inputs, input_weights, lin_grads.view(len_q, bsz, 3 * embed), True)
+        return (input_grads, None, None, None, None, input_weight_grads, output_weight_grads, pos_weight_grads,
+                input_bias_grads, output_bias_grads, pos_bias_grads, r_w_bias_grads, r_r_bias_grads,
+                None, None, None, None, None, None, None, None, None)
+
+
+def relative_self_attn_func(input, pos, use_mask, is_training, num_heads, in_proj_weight, out_proj_weight,
+                            pos_proj_weight, in_proj_bias, out_proj_bias, pos_proj_bias, r_w_bias, r_r_bias, mask, dropout,
+                            incremental, incremental_cache, low_precision, learnable_pos, return_coverage, recompute,
+                            dropout_mask=None):
+    (input, pos, in_proj_weight, out_proj_weight, pos_proj_weight, in_proj_bias, out_proj_bias, pos_proj_bias, r_w_bias,
+     r_r_bias) = cast_if_autocast_enabled(input, pos, in_proj_weight, out_proj_weight, pos_proj_weight, in_proj_bias,
+                                          out_proj_bias, pos_proj_bias, r_w_bias, r_r_bias)
+    with no_autocast():
+        return RelativeSelfAttnFunc.apply(input, pos, use_mask, is_training, num_heads, in_proj_weight, out_proj_weight,
+                                          pos_proj_weight, in_proj_bias, out_proj_bias, pos_proj_bias, r_w_bias, r_r_bias,
+                                          mask, dropout, incremental, incremental_cache, low_precision, learnable_pos,
+                                          return_coverage, recompute, dropout_mask)

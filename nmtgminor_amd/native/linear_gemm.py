@@ -45,3 +45,25 @@ def gemm(a, b, trans_a=False, trans_b=False, alpha=1.0, bias=None, out=None, spl
            L.ptr(o3), L.i64(o3.stride(1)), L.i64(o3.stride(0)), L.i64(batch), L.ptr(bias), L.ptr(ws), L.i64(ws_bytes),
            L.i32(L.dtype_code(a3)), L.stream_of(a3))
     return out if a.dim() == 3 else o3[0]
+
+
+def colsum(x, out=None):
+    """x [rows, cols] (row-major, innermost stride 1, any row pitch) -> sum over the rows, [cols] in x's dtype, fp32
+    accumulation in a fixed order (the reference's torch.sum(grads, 0) behind every bias gradient)."""
+    L.require_cuda(x, out)
+    if x.dim() != 2 or (x.size(1) > 1 and x.stride(1) != 1):
+        raise RuntimeError("colsum: a [rows, cols] matrix with unit innermost stride required")
+    rows, cols = x.shape
+    if out is None:
+        out = torch.empty(cols, dtype=x.dtype, device=x.device)
+    elif out.shape != (cols,) or out.dtype != x.dtype or not out.is_contiguous():
+        raise RuntimeError("colsum: out must be a contiguous [cols] tensor of the input dtype")
+    if rows == 0:
+        return out.zero_()
+    if cols == 0:
+        return out
+    ws_bytes = int(L.load().nmtg_colsum_workspace_bytes(L.i64(rows), L.i64(cols)))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+    L.call("nmtg_colsum", L.ptr(x), L.i64(rows), L.i64(cols), L.i64(x.stride(0) if rows > 1 else max(cols, x.stride(0))),
+           L.ptr(out), L.ptr(ws), L.i64(ws_bytes), L.i32(L.dtype_code(x)), L.stream_of(x))
+    return out

@@ -95,6 +95,22 @@ def self_attn_inputs(t=512, batch=32, d_model=1024, heads=16, dtype=torch.bfloat
     return d
 
 
+def rel_self_attn_inputs(t=64, batch=2, d_model=256, heads=4, dtype=torch.bfloat16, p=0.1, seed=1006, len_r=None,
+                         pos_batch=1, causal=False):
+    """Self-attention with relative positions: the self-attention inputs plus sinusoid-sized position states
+    pos ~ N(0,1) [R, 1 or B, E] (R >= T), W_pos [E, E] xavier-uniform, b_pos and r_w_bias, r_r_bias [H, D] ~ 0.1 N(0,1)."""
+    d = self_attn_inputs(t, batch, d_model, heads, dtype, p, seed, zero_bias=False, causal=causal)
+    g = _gen(seed + 7919)
+    e = d_model
+    r = t if len_r is None else len_r
+    d["pos"] = torch.randn(r, pos_batch, e, generator=g).to(dtype)
+    d["w_pos"] = xavier_uniform((e, e), g).to(dtype)
+    d["b_pos"] = (0.1 * torch.randn(e, generator=g)).to(dtype)
+    d["r_w_bias"] = (0.1 * torch.randn(heads, e // heads, generator=g)).to(dtype)
+    d["r_r_bias"] = (0.1 * torch.randn(heads, e // heads, generator=g)).to(dtype)
+    return d
+
+
 def encdec_attn_inputs(tq=128, tk=1500, batch=16, d_model=1024, heads=16, dtype=torch.bfloat16, p=0.0,
                        seed=1004, zero_bias=True):
     """Workload 4: encoder states [Tk,B,E], decoder states [Tq,B,E] ~ N(0,1); W_q [E,E],

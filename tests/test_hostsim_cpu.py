@@ -41,6 +41,7 @@ import test_mlp_gpu as tm  # noqa: E402
 import test_staged_gpu as tst  # noqa: E402
 import test_zz_golden_gpu as tgold  # noqa: E402
 import test_zzb_generator_loss_gpu as tgen  # noqa: E402
+import test_zzc_relative_attention_gpu as trel  # noqa: E402
 
 pytestmark = pytest.mark.skipif(not hostsim_build.available(), reason="no host C++ compiler with __bf16 (ROCm clang++)")
 CPU = torch.device("cpu")
@@ -443,6 +444,37 @@ def test_chunked_projection_loss_module_and_validation(mi355x):
     tgen.test_validation_pass_counts_correct_predictions(CPU)
     tgen.test_module_matches_the_reference_loss_assembly(CPU)
     tgen.test_argument_checks_and_empty_batch(CPU)
+
+
+# ----------------------------------------------------------------------------- relative-position self-attention
+@pytest.mark.parametrize("dtype", [BF16, F16, F32])
+@pytest.mark.parametrize("b,tq,tk,r", [(3, 16, 16, 16), (2, 9, 9, 13), (1, 40, 40, 48), (2, 7, 5, 8), (1, 1, 1, 1)])
+def test_relative_shift_kernels(mi355x, dtype, b, tq, tk, r):
+    trel.test_shift_add_and_its_adjoint_move_values_exactly(CPU, dtype, b, tq, tk, r)
+
+
+def test_relative_position_elementwise_kernels_and_linear_layer(mi355x):
+    trel.test_shift_refuses_fewer_positions_than_keys(CPU)
+    for t, b, h, d in ((5, 2, 4, 64), (3, 1, 3, 20), (4, 2, 2, 7)):
+        for dtype in (BF16, F32):
+            trel.test_query_bias_adds_per_head_biases_to_queries_inside_the_projection(CPU, dtype, t, b, h, d)
+    for rows, cols, pitch in ((300, 64, 64), (129, 40, 48), (5, 7, 7), (1000, 520, 1024), (1, 16, 16)):
+        for dtype in (BF16, F16, F32):
+            trel.test_column_sums(CPU, dtype, rows, cols, pitch)
+    trel.test_linear_layer_and_its_three_gradients(CPU, BF16)
+
+
+@pytest.mark.parametrize("dtype", HALVES)
+@pytest.mark.parametrize("t,b,e,h,len_r,pos_batch,causal,p", [
+    (64, 2, 256, 4, None, 1, False, 0.1), pytest.param(48, 3, 128, 2, 80, 1, False, 0.0, marks=long_case),
+    (40, 2, 128, 4, None, 2, True, 0.25), (33, 1, 192, 3, 37, 1, False, 0.1)])
+def test_relative_attention(mi355x, dtype, t, b, e, h, len_r, pos_batch, causal, p):
+    trel.test_relative_attention_matches_oracle(CPU, dtype, t, b, e, h, len_r, pos_batch, causal, p)
+
+
+def test_relative_attention_module_and_inference(mi355x):
+    trel.test_inference_returns_probabilities_and_single_output_form(CPU)
+    trel.test_module_has_the_reference_parameters_and_runs(CPU)
 
 
 # ----------------------------------------------------------------------------- variants that are switched off by default

@@ -10,8 +10,8 @@ import pytest
 import torch
 import torch.nn.functional as F
 
-from oracle import (attention, dropout_add, generator_loss, inputs, layer_norm, mlp, softmax_dropout, transformer_layers,
-                    xentropy)
+from oracle import (attention, dropout_add, generator_loss, inputs, layer_norm, mlp, relative_attention, softmax_dropout,
+                    transformer_layers, xentropy)
 
 D = torch.float64
 
@@ -351,6 +351,87 @@ def test_attention_finite_differences():
         xm[idx] -= eps
         fd = (f(xp) - f(xm)) / (2 * eps)
         assert abs(float(fd) - float(bwd["dx"][idx])) < 1e-6 * max(1.0, abs(float(fd)))
+
+
+# ------------------------------------------------------------------ relative-position self-attention
+@pytest.mark.parametrize("b,tq,r", [(2, 5, 5), (1, 4, 9), (3, 7, 8), (1, 1, 1)])
+def test_relative_shift_index_arithmetic_and_adjoint(b, tq, r):
+    g = torch.Generator().manual_seed(tq * 31 + r)
+    x = torch.randn(b, tq, r, generator=g, dtype=D)
+    got = relative_attention.relative_shift(x)
+    want = torch.zeros_like(x)
+    for n in range(b):                       # the closed form of the pad / view / drop / view sequence, element by element
+        for i in range(tq):
+            for j in range(r):
+                p = i * r + j + tq
+                i2, c = divmod(p, r + 1)
+                want[n, i, j] = 0.0 if c == 0 else x[n, i2, c - 1]
+    assert torch.equal(got, want)
+    # the adjoint: <shift(x), y> == <x, shift_bwd(y)>, and autograd of the forward agrees
+    y = torch.randn(b, tq, r, generator=g, dtype=D)
+    back = relative_attention.relative_shift_bwd(y)
+    torch.testing.assert_close((got * y).sum(), (x * back).sum(), rtol=1e-12, atol=1e-12)
+    xa = x.clone().requires_grad_()
+    relative_attention.relative_shift(xa).backward(y)
+    assert torch.equal(back, xa.grad)
+
+
+def test_relative_shift_aligns_distances_on_and_below_the_diagonal():
+    # what the shift is for (Transformer-XL): with R = T positions ordered from distance T-1 down to 0, the score of
+    # query i against key j <= i is the one computed against the position of distance i - j
+    t = 6
+    x = torch.arange(2 * t * t, dtype=D).view(2, t, t)
+    got = relative_attention.relative_shift(x)
+    for i in range(t):
+        for j in range(i + 1):
+            assert torch.equal(got[:, i, j], x[:, i, t - 1 - (i - j)])
+        if i + 1 < t:
+            assert (got[:, i, i + 1] == 0).all()          # the padded zero lands just above the diagonal
+
+
+def _rel_direct(d, h):
+    """Per-element Transformer-XL definition under a causal mask (only j <= i is looked at)."""
+    x, pos = d["x"].to(D), d["pos"].to(D)
+    t, b, e = x.shape
+    dh = e // h
+    lin = (x.reshape(t * b, e) @ d["w_in"].to(D).t() + d["b_in"].to(D)).view(t, b, h, 3, dh)
+    rk = (pos[:, 0] @ d["w_pos"].to(D).t() + d["b_pos"].to(D)).view(-1, h, dh)        # [R, H, D], R == T
+    u, vb = d["r_w_bias"].to(D), d["r_r_bias"].to(D)
+    out = torch.zeros(t, b, e, dtype=D)
+    for n in range(b):
+        for hh in range(h):
+            q, k, v = lin[:, n, hh, 0], lin[:, n, hh, 1], lin[:, n, hh, 2]
+            for i in range(t):
+                s = torch.stack([((q[i] + u[hh]) @ k[j] + (q[i] + vb[hh]) @ rk[t - 1 - (i - j), hh]) * dh ** -0.5
+                                 for j in range(i + 1)])
+                out[i, n, hh * dh:(hh + 1) * dh] = torch.softmax(s, 0) @ v[:i + 1]
+    return (out.reshape(t * b, e) @ d["w_out"].to(D).t() + d["b_out"].to(D)).view(t, b, e)
+
+
+def test_relative_attention_forward_matches_the_per_element_definition():
+    d = inputs.rel_self_attn_inputs(7, 2, 24, 3, torch.float64, p=0.0, seed=5, causal=True)
+    f = relative_attention.rel_self_attn_fwd(d["x"], d["pos"], d["w_in"], d["w_out"], d["w_pos"], d["b_in"], d["b_out"],
+                                             d["b_pos"], d["r_w_bias"], d["r_r_bias"], 3, None, d["time_mask"], 0.0, None, D)
+    torch.testing.assert_close(f["outputs"], _rel_direct(d, 3), rtol=1e-10, atol=1e-10)
+
+
+@pytest.mark.parametrize("causal,p,len_r,pos_batch", [(False, 0.0, None, 1), (False, 0.25, 13, 1), (True, 0.25, None, 2)])
+def test_relative_attention_backward_matches_autograd(causal, p, len_r, pos_batch):
+    h = 2
+    d = inputs.rel_self_attn_inputs(9, 2, 16, h, torch.float64, p=p, seed=6, len_r=len_r, pos_batch=pos_batch, causal=causal)
+    names = ("x", "pos", "w_in", "w_out", "w_pos", "b_in", "b_out", "b_pos", "r_w_bias", "r_r_bias")
+    leaves = {k: d[k].clone().requires_grad_() for k in names}
+    fa = relative_attention.rel_self_attn_fwd(*(leaves[k] for k in names), h, d["pad_mask"], d["time_mask"], p,
+                                              d["dropout_mask"], D)
+    fa["outputs"].backward(d["dout"])
+    f = relative_attention.rel_self_attn_fwd(*(d[k] for k in names), h, d["pad_mask"], d["time_mask"], p, d["dropout_mask"], D)
+    g = relative_attention.rel_self_attn_bwd(d["dout"], d["x"], d["pos"], d["w_in"], d["w_out"], d["w_pos"], h, f, p,
+                                             d["dropout_mask"], D)
+    for k, gk in (("x", "dx"), ("w_in", "dw_in"), ("w_out", "dw_out"), ("w_pos", "dw_pos"), ("b_in", "db_in"),
+                  ("b_out", "db_out"), ("b_pos", "db_pos"), ("r_w_bias", "dr_w_bias"), ("r_r_bias", "dr_r_bias")):
+        torch.testing.assert_close(g[gk], leaves[k].grad, rtol=1e-9, atol=1e-10, msg=lambda m, k=k: f"{k}: {m}")
+    if pos_batch == 1:            # the position states are shared over the batch: their gradient sums over it
+        assert leaves["pos"].grad.shape == d["pos"].shape
 
 
 def _layer_params_from_torch(layer, heads, decoder):

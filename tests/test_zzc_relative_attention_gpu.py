@@ -1,0 +1,169 @@
+"""Self-attention with relative position encodings against the fp32 oracle (oracle/relative_attention.py), and its
+elementwise kernels (bias additions, relative shift, the shift's adjoint, column sums) bit for bit against index
+arithmetic on the CPU.
+
+What the reference computes here: RelativeShift and RelativeSelfAttnFunc
+(onmt/modules/optimized/relative_self_attention_func.py:26-76, :79-726). The shift moves values without arithmetic, so
+it is compared exactly; the attention results to the 16-bit tolerance of the other attention tests.
+"""
+import pytest
+import torch
+
+from nmtgminor_amd.modules.relative_self_attention import RelativeSelfMultiheadAttn
+from nmtgminor_amd.modules.relative_self_attention_func import RelativeShift, relative_self_attn_func
+from nmtgminor_amd.native import linear_blaslt, linear_gemm, relative_position
+from oracle import inputs, relative_attention as orel
+from util import assert_close
+
+pytestmark = pytest.mark.gpu
+D = torch.float64
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("b,tq,tk,r", [(3, 16, 16, 16), (2, 9, 9, 13), (1, 40, 40, 48), (2, 7, 5, 8), (1, 1, 1, 1)])
+def test_shift_add_and_its_adjoint_move_values_exactly(dev, dtype, b, tq, tk, r):
+    g = torch.Generator().manual_seed(b * 100 + tq + r)
+    ac = torch.randint(-8, 9, (b, tq, tk), generator=g).to(dtype)          # small integers: the sum is exact in every dtype
+    bd = torch.randint(-8, 9, (b, tq, r), generator=g).to(dtype)
+    got = relative_position.shift_add_(ac.clone().to(dev), bd.to(dev))
+    want = ac.to(D) + orel.relative_shift(bd.to(D))[:, :, :tk]
+    assert torch.equal(got.cpu().to(D), want)
+    gs = torch.randint(-8, 9, (b, tq, tk), generator=g).to(dtype)
+    back = relative_position.shift_backward(gs.to(dev), r)
+    full = torch.cat([gs.to(D), torch.zeros(b, tq, r - tk, dtype=D)], dim=-1)
+    assert back.shape == (b, tq, r) and torch.equal(back.cpu().to(D), orel.relative_shift_bwd(full))
+    if tk == r:                                                              # the class the reference exposes
+        assert torch.equal(RelativeShift.forward(bd.to(dev), True, False).cpu().to(D), orel.relative_shift(bd.to(D)))
+        assert torch.equal(RelativeShift.backward(gs.to(dev), True, False).cpu().to(D), orel.relative_shift_bwd(gs.to(D)))
+
+
+def test_shift_refuses_fewer_positions_than_keys(dev):
+    with pytest.raises(RuntimeError):
+        relative_position.shift_add_(torch.zeros(1, 4, 8, dtype=torch.bfloat16, device=dev),
+                                     torch.zeros(1, 4, 6, dtype=torch.bfloat16, device=dev))
+    with pytest.raises(RuntimeError):
+        relative_position.shift_backward(torch.zeros(1, 4, 8, dtype=torch.bfloat16, device=dev), 6)
+    with pytest.raises(NotImplementedError):
+        RelativeShift.forward(torch.zeros(4, 8, 2, dtype=torch.bfloat16, device=dev), False, True)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("t,b,h,d", [(5, 2, 4, 64), (3, 1, 3, 20), (4, 2, 2, 7)])
+def test_query_bias_adds_per_head_biases_to_queries_inside_the_projection(dev, dtype, t, b, h, d):
+    g = torch.Generator().manual_seed(t + d)
+    lin = torch.randn(t, b * h, 3, d, generator=g).to(dtype)
+    u, w = torch.randn(h, d, generator=g).to(dtype), torch.randn(h, d, generator=g).to(dtype)
+    rw, rr = relative_position.query_bias(lin.to(dev)[:, :, 0, :], u.to(dev), w.to(dev), h)
+    q = lin[:, :, 0, :].reshape(t, b, h, d)
+    assert torch.equal(rw.cpu(), (q + u).reshape(t, b * h, d)) and torch.equal(rr.cpu(), (q + w).reshape(t, b * h, d))
+    with pytest.raises(RuntimeError):
+        relative_position.query_bias(lin.to(dev)[:, :, 0, :], u.to(dev)[:, :d - 1], w.to(dev), h)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("rows,cols,pitch", [(300, 64, 64), (129, 40, 48), (5, 7, 7), (1000, 520, 1024), (1, 16, 16)])
+def test_column_sums(dev, dtype, rows, cols, pitch):
+    g = torch.Generator().manual_seed(rows + cols)
+    x = torch.randn(rows, pitch, generator=g).to(dtype)
+    got = linear_gemm.colsum(x.to(dev)[:, :cols])
+    assert got.dtype == dtype and got.shape == (cols,)
+    assert_close(got, x[:, :cols].to(D).sum(0), dtype, "column sums", scale_atol=True)
+    assert torch.equal(linear_gemm.colsum(x.to(dev)[:0, :cols]).cpu(), torch.zeros(cols, dtype=dtype))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_linear_layer_and_its_three_gradients(dev, dtype):
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(6, 5, 64, generator=g).to(dtype)
+    w = (torch.randn(96, 64, generator=g) / 8).to(dtype)
+    b = torch.randn(96, generator=g).to(dtype)
+    gy = torch.randn(6, 5, 96, generator=g).to(dtype)
+    y = linear_blaslt.forward(x.to(dev), w.to(dev), b.to(dev))
+    assert y.shape == (6, 5, 96)
+    assert_close(y, x.to(D) @ w.to(D).t() + b.to(D), dtype, "linear forward")
+    dx, dw, db = linear_blaslt.backward(x.to(dev), w.to(dev), gy.to(dev), True)
+    assert_close(dx, gy.to(D) @ w.to(D), dtype, "linear grad input")
+    assert_close(dw, gy.to(D).reshape(30, 96).t() @ x.to(D).reshape(30, 64), dtype, "linear grad weight", scale_atol=True)
+    assert_close(db, gy.to(D).reshape(30, 96).sum(0), dtype, "linear grad bias", scale_atol=True)
+    assert linear_blaslt.backward(x.to(dev), w.to(dev), gy.to(dev), False)[0] is None
+
+
+NAMES = ("x", "pos", "w_in", "w_out", "w_pos", "b_in", "b_out", "b_pos", "r_w_bias", "r_r_bias")
+GRADS = (("x", "dx"), ("w_in", "dw_in"), ("w_out", "dw_out"), ("w_pos", "dw_pos"), ("b_in", "db_in"), ("b_out", "db_out"),
+         ("b_pos", "db_pos"), ("r_w_bias", "dr_w_bias"), ("r_r_bias", "dr_r_bias"))
+
+
+def _run(dev, d, heads, training, use_time_mask, p, return_coverage=True):
+    t = {k: d[k].to(dev).requires_grad_() for k in NAMES}
+    mask = d["time_mask"] if use_time_mask else d["pad_mask"]
+    dm = d["dropout_mask"].to(dev) if (training and p > 0) else None
+    res = relative_self_attn_func(t["x"], t["pos"], use_time_mask, training, heads, t["w_in"], t["w_out"], t["w_pos"],
+                                  t["b_in"], t["b_out"], t["b_pos"], t["r_w_bias"], t["r_r_bias"],
+                                  None if mask is None else mask.to(dev), p, False, None, False, False, return_coverage, False,
+                                  dm)
+    return t, res
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("t,b,e,h,len_r,pos_batch,causal,p", [
+    (64, 2, 256, 4, None, 1, False, 0.1),      # encoder form: key padding, positions shared over the batch
+    (48, 3, 128, 2, 80, 1, False, 0.0),        # more positions than keys (bidirectional 2T-1 style table), no dropout
+    (40, 2, 128, 4, None, 2, True, 0.25),      # decoder form: time mask, positions per batch column
+    (33, 1, 192, 3, 37, 1, False, 0.1),        # odd lengths: the unvectorised shift kernels, head_dim 64
+])
+def test_relative_attention_matches_oracle(dev, dtype, t, b, e, h, len_r, pos_batch, causal, p):
+    d = inputs.rel_self_attn_inputs(t, b, e, h, dtype, p=p, seed=200 + t, len_r=len_r, pos_batch=pos_batch, causal=causal)
+    leaves, (out, cov) = _run(dev, d, h, True, causal, p)
+    out.backward(d["dout"].to(dev))
+    f = orel.rel_self_attn_fwd(*(d[k] for k in NAMES), h, d["pad_mask"], d["time_mask"], p, d["dropout_mask"], D, round_to=dtype)
+    g = orel.rel_self_attn_bwd(d["dout"], d["x"], d["pos"], d["w_in"], d["w_out"], d["w_pos"], h, f, p, d["dropout_mask"], D,
+                               round_to=dtype)
+    # the scores are rounded three times here (AC, BD, their sum) against once in plain self-attention, so a probability
+    # moves by a 16-bit ulp of its score more often than there; for outputs that cancel to near zero (|out| ~ 1e-2 where the
+    # terms are ~ 1) the absolute tolerance is 2e-3 instead of 1e-3, the relative one stays 2e-2
+    assert_close(out, f["outputs"], dtype, "outputs", atol=2e-3)
+    assert_close(cov, f["dropout_results"], dtype, "coverage (dropped probabilities)")
+    masked = (d["time_mask"].unsqueeze(0).expand(b * h, t, t) if causal
+              else d["pad_mask"].view(b, 1, 1, t).expand(b, h, t, t).reshape(b * h, t, t))
+    assert (cov.cpu()[masked] == 0).all()                                   # masked keys: probability exactly zero
+    for name, key in GRADS:
+        assert_close(leaves[name].grad, g[key], dtype, "grad " + name, scale_atol=name != "x")
+    assert leaves["pos"].grad is None                                       # the reference returns no gradient for pos
+
+
+def test_inference_returns_probabilities_and_single_output_form(dev):
+    dtype, h = torch.bfloat16, 4
+    d = inputs.rel_self_attn_inputs(32, 2, 128, h, dtype, p=0.3, seed=9)
+    f = orel.rel_self_attn_fwd(*(d[k] for k in NAMES), h, d["pad_mask"], None, 0.0, None, D, round_to=dtype)
+    with torch.no_grad():
+        _, (out, cov) = _run(dev, d, h, False, False, 0.3)
+        _, only = _run(dev, d, h, False, False, 0.3, return_coverage=False)
+    assert_close(out, f["outputs"], dtype, "inference outputs")
+    assert_close(cov, f["softmax_results"], dtype, "inference coverage")
+    assert torch.is_tensor(only) and torch.equal(only, out)
+
+
+def test_module_has_the_reference_parameters_and_runs(dev):
+    torch.manual_seed(4)
+    m = RelativeSelfMultiheadAttn(128, 4, dropout=0.0).to(dev).to(torch.bfloat16)
+    shapes = {k: tuple(v.shape) for k, v in m.named_parameters()}
+    assert shapes == {"in_proj_weight": (384, 128), "out_proj_weight": (128, 128), "pos_proj_weight": (128, 128),
+                      "pos_proj_bias": (128,), "in_proj_bias": (384,), "out_proj_bias": (128,), "r_w_bias": (4, 32),
+                      "r_r_bias": (4, 32)}
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(24, 2, 128, generator=g).to(torch.bfloat16)
+    pos = torch.randn(24, 1, 128, generator=g).to(torch.bfloat16)
+    pad = torch.zeros(2, 24, dtype=torch.bool)
+    pad[1, 17:] = True
+    out, cov = m(x.to(dev), pos.to(dev), key_padding_mask=pad.t().unsqueeze(0).to(dev))        # the reference's [1, T, B] form
+    P = {k: v.detach().cpu() for k, v in m.named_parameters()}
+    f = orel.rel_self_attn_fwd(x, pos, P["in_proj_weight"], P["out_proj_weight"], P["pos_proj_weight"], P["in_proj_bias"],
+                               P["out_proj_bias"], P["pos_proj_bias"], P["r_w_bias"], P["r_r_bias"], 4, pad, None, 0.0, None, D,
+                               round_to=torch.bfloat16)
+    assert_close(out, f["outputs"], torch.bfloat16, "module outputs")
+    out.float().sum().backward()
+    assert all(p.grad is not None for p in m.parameters())
+    with pytest.raises(NotImplementedError):
+        RelativeSelfMultiheadAttn(128, 4, learnable_pos=True, max_pos=8)
+    with pytest.raises(NotImplementedError):
+        m(x.to(dev), pos.to(dev), incremental=True, incremental_cache={})
