@@ -8,6 +8,7 @@ The expected values come from PyTorch's own CPU library routines and autograd in
 F.silu, F.gelu(approximate="tanh")) on small seeded inputs — the routines the reference's
 PyTorch fallback itself calls (onmt/modules/layer_norm.py:29-33, onmt/modules/mlp/mlp.py:14-42,
 onmt/modules/optimized/self_attention_func.py:141-287, encdec_attention_func_bias.py:141-351,
+relative_self_attention_func.py:128-345 with the relative shift written as an explicit gather,
 onmt/modules/optimized/softmax_xentropy.py). Neither oracle/ nor the HIP library is imported here,
 so the fixtures are independent of both; tests/test_golden_cpu.py checks the oracle against them
 and tests/test_zz_golden_gpu.py the HIP path.
@@ -213,7 +214,52 @@ def encdec_attention():
          pad_mask=pad.to(torch.uint8), heads=h, softmax_results=sm, matmul2_results=ctx.reshape(tq, b, e), outputs=out)
 
 
+def relative_attention():
+    """Self-attention with relative positions. The shift is a gather over an index table built element by element from
+    its closed form (output (i, j) reads padded element i R + j + T of the zero-fronted [T, R + 1] matrix), not the
+    reference's pad / view sequence."""
+    g = gen(108)
+    t, r, b, e, h, p = 9, 12, 2, 64, 2, 0.25
+    d = e // h
+    mk = lambda *s, scale=1.0: rnd16(scale * torch.randn(*s, generator=g, dtype=D))
+    x0, pos0 = mk(t, b, e), mk(r, 1, e)
+    w_in0, w_out0, w_pos0 = mk(3 * e, e, scale=1 / math.sqrt(e)), mk(e, e, scale=1 / math.sqrt(e)), mk(e, e, scale=1 / math.sqrt(e))
+    b_in0, b_out0, b_pos0 = mk(3 * e, scale=0.1), mk(e, scale=0.1), mk(e, scale=0.1)
+    u0, v0 = mk(h, d, scale=0.1), mk(h, d, scale=0.1)
+    lengths = torch.tensor([9, 6])
+    pad = torch.arange(t).unsqueeze(0) >= lengths.unsqueeze(1)
+    dm = (torch.rand(b * h, t, t, generator=g) < 1 - p).to(torch.uint8)
+    dout = mk(t, b, e)
+    leaves = [z.clone().requires_grad_() for z in (x0, w_in0, w_out0, w_pos0, b_in0, b_out0, b_pos0, u0, v0)]
+    x, w_in, w_out, w_pos, b_in, b_out, b_pos, u, v = leaves
+    lin = rb(F.linear(x, w_in, b_in)).view(t, b * h, 3, d)
+    q, k, val = lin[:, :, 0, :], lin[:, :, 1, :], lin[:, :, 2, :]
+    r_k = rb(F.linear(pos0.expand(r, b, e), w_pos, b_pos)).view(r, b * h, d)
+    rw_q = rb(q.view(t, b, h, d) + u).view(t, b * h, d)
+    rr_q = rb(q.view(t, b, h, d) + v).view(t, b * h, d)
+    ac = rb(torch.matmul(rw_q.transpose(0, 1), k.transpose(0, 1).transpose(1, 2)) / math.sqrt(d))
+    bd = rb(torch.matmul(rr_q.transpose(0, 1), r_k.transpose(0, 1).transpose(1, 2)) / math.sqrt(d))       # [B*H, T, R]
+    src = torch.zeros(t, t, dtype=torch.long)            # index into the flattened zero-fronted [T, R + 1] matrix
+    for i in range(t):
+        for j in range(t):
+            src[i, j] = i * r + j + t
+    padded = torch.cat([bd.new_zeros(b * h, t, 1), bd], dim=2).reshape(b * h, t * (r + 1))
+    shifted = padded.gather(1, src.view(1, t * t).expand(b * h, t * t)).view(b * h, t, t)
+    scores = rb(ac + shifted)
+    scores = scores.view(b, h, t, t).masked_fill(pad.view(b, 1, 1, t), float("-inf")).view(b * h, t, t)
+    sm = F.softmax(scores, -1)
+    dropped = rb(sm * dm.to(D) / (1 - p))
+    ctx = rb(torch.matmul(dropped, val.transpose(0, 1)).transpose(0, 1))
+    out = F.linear(ctx.reshape(t, b, e), w_out, b_out)
+    out.backward(dout)
+    save("relative_attention", f32=True, x=x0, pos=pos0, w_in=w_in0, w_out=w_out0, w_pos=w_pos0, b_in=b_in0, b_out=b_out0,
+         b_pos=b_pos0, r_w_bias=u0, r_r_bias=v0, pad_mask=pad.to(torch.uint8), dropout_mask=dm, p=p, heads=h, dout=dout,
+         softmax_results=sm, dropout_results=dropped, matmul2_results=ctx.reshape(t, b, e), outputs=out, dx=x.grad,
+         dw_in=w_in.grad, dw_out=w_out.grad, dw_pos=w_pos.grad, db_in=b_in.grad, db_out=b_out.grad, db_pos=b_pos.grad,
+         dr_w_bias=u.grad, dr_r_bias=v.grad)
+
+
 if __name__ == "__main__":
     torch.set_num_threads(1)
-    for f in (layer_norm, dropout_add, softmax_dropout, xentropy, mlp, self_attention, encdec_attention):
+    for f in (layer_norm, dropout_add, softmax_dropout, xentropy, mlp, self_attention, encdec_attention, relative_attention):
         f()

@@ -9,7 +9,7 @@ import os
 import numpy as np
 import torch
 
-from oracle import attention, dropout_add, layer_norm, mlp, softmax_dropout, xentropy
+from oracle import attention, dropout_add, layer_norm, mlp, relative_attention, softmax_dropout, xentropy
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 D = torch.float64
@@ -105,3 +105,17 @@ def test_encdec_attention_fixture():
                                     f["pad_mask"].bool(), 0.0, None, D, round_to=BF)
     for k in ("softmax_results", "matmul2_results", "outputs"):
         close(fwd[k], f[k], k, **F32)
+
+
+def test_relative_attention_fixture():
+    f = load("relative_attention")
+    p, h = float(f["p"]), int(f["heads"])
+    names = ("x", "pos", "w_in", "w_out", "w_pos", "b_in", "b_out", "b_pos", "r_w_bias", "r_r_bias")
+    fwd = relative_attention.rel_self_attn_fwd(*(f[k] for k in names), h, f["pad_mask"].bool(), None, p, f["dropout_mask"], D,
+                                               round_to=BF)
+    for k in ("softmax_results", "dropout_results", "matmul2_results", "outputs"):
+        close(fwd[k], f[k], k, **F32)
+    bwd = relative_attention.rel_self_attn_bwd(f["dout"], f["x"], f["pos"], f["w_in"], f["w_out"], f["w_pos"], h, fwd, p,
+                                               f["dropout_mask"], D, round_to=BF)
+    for k in ("dx", "dw_in", "dw_out", "dw_pos", "db_in", "db_out", "db_pos", "dr_w_bias", "dr_r_bias"):
+        close(bwd[k], f[k], k, **F32)

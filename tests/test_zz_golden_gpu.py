@@ -14,6 +14,7 @@ import torch
 
 from nmtgminor_amd.modules import mlp as mmlp
 from nmtgminor_amd.modules.encdec_attention_func_bias import encdec_attn_bias_func
+from nmtgminor_amd.modules.relative_self_attention_func import relative_self_attn_func
 from nmtgminor_amd.modules.self_attention_func import self_attn_func
 from nmtgminor_amd.native import (fast_layer_norm_cuda, fused_dropout_add_cuda, fused_mlp_gelu, mask_softmax_dropout_cuda,
                                   self_multihead_attn_blaslt as sa_native, xentropy_cuda)
@@ -130,3 +131,19 @@ def test_encdec_attention_fixture(dev):
                                      None)
     assert_close(out, f["outputs"], BF, "outputs")
     assert_close(cov, f["softmax_results"], BF, "softmax_results")
+
+
+def test_relative_attention_fixture(dev):
+    f = load("relative_attention")
+    p, h = float(f["p"]), int(f["heads"])
+    names = ("x", "pos", "w_in", "w_out", "w_pos", "b_in", "b_out", "b_pos", "r_w_bias", "r_r_bias")
+    t = {k: f[k].to(BF).to(dev).requires_grad_() for k in names}
+    out, cov = relative_self_attn_func(t["x"], t["pos"], False, True, h, t["w_in"], t["w_out"], t["w_pos"], t["b_in"],
+                                       t["b_out"], t["b_pos"], t["r_w_bias"], t["r_r_bias"], f["pad_mask"].bool().to(dev), p,
+                                       False, None, False, False, True, False, f["dropout_mask"].to(dev))
+    out.backward(f["dout"].to(BF).to(dev))
+    assert_close(out, f["outputs"], BF, "outputs", atol=2e-3)      # scores rounded three times (AC, BD, sum): see the op's test
+    assert_close(cov, f["dropout_results"], BF, "dropout_results")
+    for k, gk in (("x", "dx"), ("w_in", "dw_in"), ("w_out", "dw_out"), ("w_pos", "dw_pos"), ("b_in", "db_in"),
+                  ("b_out", "db_out"), ("b_pos", "db_pos"), ("r_w_bias", "dr_w_bias"), ("r_r_bias", "dr_r_bias")):
+        assert_close(t[k].grad, f[gk], BF, gk, scale_atol=True)
