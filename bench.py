@@ -269,6 +269,62 @@ class SelfAttnWL(Workload):
                     kind="port", sample=f"{nb} of {self.B} batch columns (independent), fp32 on the bf16-rounded values, median of 3")
 
 
+class RelSelfAttnWL(Workload):
+    name = "rel_self_attn"
+    bound = "mfma"
+    dtype = "bf16"
+    description = ("self-attention with relative positions fwd+bwd bf16 (speech-encoder form): T=512, B=32, E=1024, 16 heads, "
+                   "R=512 positions shared over the batch, key-padding lengths U[256,512], softmax dropout 0.1 (explicit mask)")
+    T, B, E, H = 512, 32, 1024, 16
+    NAMES = ("x", "pos", "w_in", "w_out", "w_pos", "b_in", "b_out", "b_pos", "r_w_bias", "r_r_bias")
+
+    def setup(self, dev):
+        from oracle import inputs
+        from nmtgminor_amd.modules.relative_self_attention_func import relative_self_attn_func
+        self.fn = relative_self_attn_func
+        d = inputs.rel_self_attn_inputs(self.T, self.B, self.E, self.H, torch.bfloat16, p=0.1, seed=1006)
+        self.cpu = d
+        self.t = {k: d[k].to(dev).requires_grad_(k != "pos") for k in self.NAMES}
+        self.pad, self.dm, self.dout = d["pad_mask"].to(dev), d["dropout_mask"].to(dev), d["dout"].to(dev)
+
+    def step(self):
+        t = self.t
+        for v in t.values():
+            v.grad = None
+        out = self.fn(t["x"], t["pos"], False, True, self.H, t["w_in"], t["w_out"], t["w_pos"], t["b_in"], t["b_out"],
+                      t["b_pos"], t["r_w_bias"], t["r_r_bias"], self.pad, 0.1, False, None, False, False, False, False, self.dm)
+        out.backward(self.dout)
+        return t["x"].grad
+
+    def _flops_fwd(self):
+        t, b, e, h = self.T, self.B, self.E, self.H
+        tok = t * b
+        # in-projection, position projection (per batch column, as the reference lays it out), AC, BD, P V, out-projection
+        return 2.0 * tok * e * 3 * e + 2.0 * tok * e * e + 3 * (2.0 * b * h * t * t * (e // h)) + 2.0 * tok * e * e
+
+    def work_per_step(self):
+        # backward: two products per forward product, except the position projection (weight gradient only)
+        return 3 * self._flops_fwd() - 2.0 * self.T * self.B * self.E * self.E
+
+    def kernel_work(self):
+        return {"gemm_": self.work_per_step()}
+
+    def cpu_baseline(self):
+        from oracle import relative_attention as o
+        d = self.cpu
+        nb = 2                                                   # batch columns are independent
+        a = {k: d[k].float() for k in self.NAMES}
+        a["x"] = a["x"][:, :nb]
+        dout, pad, dm = d["dout"][:, :nb].float(), d["pad_mask"][:nb], d["dropout_mask"][:nb * self.H]
+
+        def run():
+            f = o.rel_self_attn_fwd(*(a[k] for k in self.NAMES), self.H, pad, None, 0.1, dm)
+            o.rel_self_attn_bwd(dout, a["x"], a["pos"], a["w_in"], a["w_out"], a["w_pos"], self.H, f, 0.1, dm)
+        t = _time_cpu(run, 3)
+        return dict(value=self.work_per_step() * nb / self.B / t / 1e12, unit="TFLOP/s", cores=torch.get_num_threads(),
+                    kind="port", sample=f"{nb} of {self.B} batch columns (independent), fp32 on the bf16-rounded values, median of 3")
+
+
 class EncdecAttnWL(Workload):
     name = "encdec_attn"
     bound = "mfma"
@@ -495,7 +551,7 @@ class CopyWL(Workload):
 
 
 WORKLOADS = {w.name: w for w in (LayerNormWL, MlpWL, SelfAttnWL, EncdecAttnWL, SoftmaxDropoutWL, DropoutAddWL, XentropyWL,
-                                    GeneratorLossWL)}
+                                    GeneratorLossWL, RelSelfAttnWL)}
 EXTRA_WORKLOADS = {CopyWL.name: CopyWL}
 PRIMARY = "mlp"
 
@@ -624,14 +680,74 @@ def measure(w, dev, steps, warmup, do_cpu, trace_steps):
     return res
 
 
+RESULT_TAG = "NMTG_BENCH_RESULT "
+
+
+def _run_workloads(names, args, dev, emit):
+    """Measures the named workloads one after the other in this process. emit: print each result as soon as it exists
+    (tagged line on stdout), so that a parent process keeps what was measured if a later workload ends the process."""
+    table = dict(WORKLOADS, **EXTRA_WORKLOADS)
+    results = []
+    for n in names:
+        w = table[n]()
+        steps = args.steps if w.name not in ("xentropy", "generator_loss") else max(3, min(args.steps, 10))
+        try:
+            results.append(measure(w, dev, steps, args.warmup, not args.no_cpu, min(args.trace_steps, steps)))
+        except Exception as e:
+            if n == names[0] and not emit:
+                raise                    # no headline without the first workload
+            sys.stderr.write(f"[bench] workload {n} failed: {e}\n")
+            results.append(dict(workload=n, error=str(e)))
+        results[-1]["steps"] = steps
+        if emit:
+            print(RESULT_TAG + json.dumps(results[-1]), flush=True)
+        del w
+        torch.cuda.empty_cache()
+    return results
+
+
+def _in_child(names, args, limit_s):
+    """Runs `bench.py --in-process --emit-results` on the named workloads as a child process and collects the results it
+    printed. A workload the child did not get to (it ended early, or ran into the time limit) is reported as an error
+    entry, so one workload cannot take the others' measurements with it."""
+    import subprocess
+    cmd = [sys.executable, os.path.abspath(__file__), "--in-process", "--emit-results", "--workload", ",".join(names),
+           "--steps", str(args.steps), "--warmup", str(args.warmup), "--trace-steps", str(args.trace_steps)]
+    if args.no_cpu:
+        cmd.append("--no-cpu")
+    out, note = "", None
+    try:
+        r = subprocess.run(cmd, stdout=subprocess.PIPE, text=True, timeout=limit_s)
+        out = r.stdout
+        if r.returncode != 0:
+            note = f"the measuring process ended with status {r.returncode}"
+    except subprocess.TimeoutExpired as e:
+        out = e.stdout if isinstance(e.stdout, str) else (e.stdout or b"").decode(errors="replace")
+        note = f"the measuring process was stopped after {limit_s} s"
+    got = {}
+    for line in out.splitlines():
+        if line.startswith(RESULT_TAG):
+            try:
+                r = json.loads(line[len(RESULT_TAG):])
+                got[r["workload"]] = r
+            except (ValueError, KeyError):
+                pass
+    return [got.get(n, dict(workload=n, error=note or "no result was reported")) for n in names]
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="all", help="one of %s, or all" % ", ".join(WORKLOADS))
+    ap.add_argument("--workload", default="all", help="one or more (comma-separated) of %s, or all" % ", ".join(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--trace-steps", type=int, default=10)
+    ap.add_argument("--in-process", action="store_true",
+                    help="measure every workload in this process. Default for 'all': the headline workload in one child "
+                         "process and the others in a second one, so that no workload can cost another its measurement; "
+                         "use this flag under a profiler, which must see the measuring process itself")
+    ap.add_argument("--emit-results", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--variants", default="",
                     help="semicolon-separated sets of per-call library switches to time after the default configuration, "
                          "e.g. 'NMTG_GELU_LUT;NMTG_GELU_LUT+NMTG_GEMM_ACT_TILE'. Each set is exported as NAME=1 for one "
@@ -641,54 +757,55 @@ def main():
         sys.stderr.write("bench.py measures one GPU: this build has no multi-GPU path (each op is independent per "
                          "token row / per (batch, head), so it would shard by data parallelism over tokens). Run with --gpus 1.\n")
         sys.exit(2)
-    if not torch.cuda.is_available():
-        sys.stderr.write("bench.py needs a GPU (MI355X); the ops have no CPU path.\n")
-        sys.exit(2)
-    torch.set_num_threads(os.cpu_count() or 1)
-    dev = torch.device("cuda:0")
-    names = list(WORKLOADS) if args.workload == "all" else [args.workload]
     table = dict(WORKLOADS, **EXTRA_WORKLOADS)
+    names = list(WORKLOADS) if args.workload == "all" else [n.strip() for n in args.workload.split(",") if n.strip()]
+    unknown = [n for n in names if n not in table]
+    if unknown or not names:
+        sys.stderr.write("bench.py: unknown workload %s; choose from %s\n" % (", ".join(unknown) or "''", ", ".join(table)))
+        sys.exit(2)
     if PRIMARY in names:                     # headline first
         names.remove(PRIMARY)
         names.insert(0, PRIMARY)
-    results = []
-    for n in names:
-        w = table[n]()
-        steps = args.steps if w.name not in ("xentropy", "generator_loss") else max(3, min(args.steps, 10))
-        try:
-            results.append(measure(w, dev, steps, args.warmup, not args.no_cpu, min(args.trace_steps, steps)))
-        except Exception as e:
-            if n == names[0]:
-                raise                    # no headline without the first workload
-            sys.stderr.write(f"[bench] workload {n} failed: {e}\n")
-            results.append(dict(workload=n, error=str(e)))
-        results[-1]["steps"] = steps
-        del w
-        torch.cuda.empty_cache()
-    # per-call switches of the library (staged kernel variants): the same workloads again under each requested set
+    split = args.workload == "all" and not args.in_process and not args.variants
     variants = []
-    for spec in [v.strip() for v in args.variants.split(";") if v.strip()]:
-        switches = [n.strip() for n in spec.split("+") if n.strip()]
-        saved = {n: os.environ.get(n) for n in switches}
-        os.environ.update({n: "1" for n in switches})
-        try:
-            for n in names:
-                w = table[n]()
-                steps = args.steps if w.name not in ("xentropy", "generator_loss") else max(3, min(args.steps, 10))
-                try:
-                    r = measure(w, dev, steps, args.warmup, False, min(args.trace_steps, steps))
-                    variants.append(dict(switches=switches, workload=n, value=r["value"], unit=r["unit"], ms_per_step=r["ms_per_step"],
-                                         kernels=r["kernels"]))
-                except Exception as e:
-                    variants.append(dict(switches=switches, workload=n, error=str(e)))
-                del w
-                torch.cuda.empty_cache()
-        finally:
-            for n, v in saved.items():
-                if v is None:
-                    os.environ.pop(n, None)
-                else:
-                    os.environ[n] = v
+    if split:
+        # This process never touches the GPU: it starts the two measuring processes and assembles their results.
+        results = _in_child(names[:1], args, 900) + _in_child(names[1:], args, 2400)
+        if "error" in results[0]:
+            sys.stderr.write(f"bench.py: the headline workload {names[0]} gave no result: {results[0]['error']}\n")
+            sys.exit(1)
+    else:
+        if not torch.cuda.is_available():
+            sys.stderr.write("bench.py needs a GPU (MI355X); the ops have no CPU path.\n")
+            sys.exit(2)
+        torch.set_num_threads(os.cpu_count() or 1)
+        dev = torch.device("cuda:0")
+        results = _run_workloads(names, args, dev, args.emit_results)
+        if args.emit_results:
+            return
+        # per-call switches of the library (staged kernel variants): the same workloads again under each requested set
+        for spec in [v.strip() for v in args.variants.split(";") if v.strip()]:
+            switches = [n.strip() for n in spec.split("+") if n.strip()]
+            saved = {n: os.environ.get(n) for n in switches}
+            os.environ.update({n: "1" for n in switches})
+            try:
+                for n in names:
+                    w = table[n]()
+                    steps = args.steps if w.name not in ("xentropy", "generator_loss") else max(3, min(args.steps, 10))
+                    try:
+                        r = measure(w, dev, steps, args.warmup, False, min(args.trace_steps, steps))
+                        variants.append(dict(switches=switches, workload=n, value=r["value"], unit=r["unit"],
+                                             ms_per_step=r["ms_per_step"], kernels=r["kernels"]))
+                    except Exception as e:
+                        variants.append(dict(switches=switches, workload=n, error=str(e)))
+                    del w
+                    torch.cuda.empty_cache()
+            finally:
+                for n, v in saved.items():
+                    if v is None:
+                        os.environ.pop(n, None)
+                    else:
+                        os.environ[n] = v
     head = results[0]
     line = {
         "metric": "MFMA TFLOP/s (fused MLP fwd+bwd)" if head["workload"] == "mlp" else head["metric"] + f" ({head['workload']})",

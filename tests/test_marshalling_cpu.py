@@ -16,8 +16,8 @@ import torch
 from nmtgminor_amd import _lib, _rng
 from nmtgminor_amd.native import (encdec_multihead_attn_bias_blaslt as ed, fast_layer_norm_cuda as ln,
                                   fused_dropout_add_cuda as da, fused_mlp_agelu, fused_mlp_gelu, fused_mlp_relu,
-                                  fused_mlp_silu, linear_gemm, mask_softmax_dropout_cuda as sm, mlp_gelu_blaslt,
-                                  self_multihead_attn_blaslt as sa, xentropy_cuda as xe)
+                                  fused_mlp_silu, linear_blaslt, linear_gemm, mask_softmax_dropout_cuda as sm, mlp_gelu_blaslt,
+                                  relative_position,                                  self_multihead_attn_blaslt as sa, xentropy_cuda as xe)
 
 
 def header_signatures():
@@ -180,3 +180,16 @@ def test_attention(recorder):
     ed.backward_compact(h, r(t, b, e), dr, sc, q_lin, kv_lin, dmask2, 0.1)
     ed.backward_recompute(h, r(t, b, e), x, x_kv, w_q, w_kv, b_q, b_kv, w_out, dmask2, padk, 0.1)
     assert {"nmtg_self_attn_fwd", "nmtg_self_attn_bwd", "nmtg_encdec_attn_fwd", "nmtg_encdec_attn_bwd"} <= set(recorder)
+
+
+def test_relative_position_column_sums_and_linear_layer(recorder):
+    r = lambda *s: torch.randn(*s).to(BF)
+    lin = r(5, 6, 3, 16)
+    relative_position.query_bias(lin[:, :, 0, :], r(2, 16), r(2, 16), 2)
+    relative_position.shift_add_(r(6, 5, 5), r(6, 5, 8))
+    relative_position.shift_backward(r(6, 5, 5), 8)
+    linear_gemm.colsum(r(40, 24))
+    linear_gemm.colsum(r(40, 32)[:, :24], out=torch.empty(24).to(BF))
+    linear_blaslt.forward(r(4, 3, 16), r(24, 16), r(24))
+    linear_blaslt.backward(r(4, 3, 16), r(24, 16), r(4, 3, 24), True)
+    assert {"nmtg_rel_query_bias", "nmtg_rel_shift_add", "nmtg_rel_shift_bwd", "nmtg_colsum", "nmtg_gemm"} <= set(recorder)
