@@ -308,6 +308,11 @@ int nmtg_colsum(const void* x, int64_t rows, int64_t cols, int64_t ld, void* out
  *
  * nmtg_rel_shift_bwd: the adjoint, grad_bd[b][i2][c - 1] = grad_scores[b][i][j] at the same
  *   correspondence (0 where j >= len_k or where p < len_q); grad_bd dense [batch, len_q, len_r].
+ *
+ * nmtg_add_rows: out[r][c] = a[r][c] + b[r][c] for r < rows, c < cols, each matrix with its own row
+ *   pitch; out may be a or b. The reference's elementwise sums of two gradient or score terms
+ *   (queries_grads.add_(queries_grads_bd), :678; the beta = 1 accumulation of the position scores
+ *   of learnable positions into matmul_ac, :264).
  * dtype: NMTG_F16, NMTG_BF16 or NMTG_F32.
  * ------------------------------------------------------------------------------------------ */
 int nmtg_rel_query_bias(const void* q, int64_t ld_q, const void* r_w_bias, const void* r_r_bias,
@@ -319,6 +324,9 @@ int nmtg_rel_shift_add(void* scores, const void* bd, int64_t batch, int64_t len_
 
 int nmtg_rel_shift_bwd(const void* grad_scores, void* grad_bd, int64_t batch, int64_t len_q,
                        int64_t len_k, int64_t len_r, int dtype, void* stream);
+
+int nmtg_add_rows(void* out, int64_t ld_out, const void* a, int64_t ld_a, const void* b, int64_t ld_b,
+                  int64_t rows, int64_t cols, int dtype, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Per-kernel timing for benchmarks (no counterpart in the reference, whose tests time whole ops

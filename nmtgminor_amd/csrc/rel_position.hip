@@ -114,6 +114,24 @@ __global__ __launch_bounds__(RP_THREADS) void rel_shift_bwd_kernel(const T* __re
   }
 }
 
+// out[r][c] = a[r][c] + b[r][c] over rows of `cols` elements with their own pitches (out may be a or b); one thread per
+// EPV consecutive columns of one row.
+template <typename T, int EPV>
+__global__ __launch_bounds__(RP_THREADS) void add_rows_kernel(T* out, int64_t ld_out, const T* a, int64_t ld_a,
+                                                              const T* b, int64_t ld_b, int64_t rows, int cols) {
+  const int per_row = cols / EPV;
+  const int64_t item = static_cast<int64_t>(blockIdx.x) * RP_THREADS + threadIdx.x;
+  if (item >= rows * per_row) return;
+  const int64_t r = item / per_row;
+  const int c = static_cast<int>(item - r * per_row) * EPV;
+  float av[EPV], bv[EPV];
+  load_pack<T, EPV>(a + r * ld_a + c, av);
+  load_pack<T, EPV>(b + r * ld_b + c, bv);
+#pragma unroll
+  for (int j = 0; j < EPV; ++j) av[j] += bv[j];
+  store_pack<T, EPV>(out + r * ld_out + c, av);
+}
+
 inline bool fits_grid(int64_t items, int64_t batch) {
   return (items + RP_THREADS - 1) / RP_THREADS <= 0x7fffffff && batch <= 65535;
 }
@@ -200,5 +218,30 @@ extern "C" int nmtg_rel_shift_bwd(const void* grad_scores, void* grad_bd, int64_
                               static_cast<const T*>(grad_scores), static_cast<T*>(grad_bd), static_cast<uint32_t>(len_q),
                               static_cast<uint32_t>(len_k), static_cast<uint32_t>(len_r)));
   NMTG_CHECK_LAUNCH("rel_shift_bwd");
+  return 0;
+}
+
+extern "C" int nmtg_add_rows(void* out, int64_t ld_out, const void* a, int64_t ld_a, const void* b, int64_t ld_b, int64_t rows,
+                             int64_t cols, int dtype, void* stream) {
+  NMTG_REQUIRE(rows >= 0 && cols >= 0 && cols <= INT32_MAX && rows * cols < (int64_t(1) << 40),
+               "add_rows: bad sizes (rows %lld, columns %lld)", (long long)rows, (long long)cols);
+  NMTG_REQUIRE(ld_out >= cols && ld_a >= cols && ld_b >= cols, "add_rows: a row pitch is below the number of columns %lld",
+               (long long)cols);
+  if (rows == 0 || cols == 0) return 0;
+  NMTG_REQUIRE(out && a && b, "add_rows: null pointer argument");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  TraceScope trace("add_rows", st);
+  NMTG_DISPATCH_DTYPE(
+      dtype, T, constexpr int WIDE = 16 / sizeof(T);
+      const bool wide = cols % WIDE == 0 && ld_out % WIDE == 0 && ld_a % WIDE == 0 && ld_b % WIDE == 0 && aligned16(out) &&
+                        aligned16(a) && aligned16(b);
+      const int64_t items = wide ? rows * (cols / WIDE) : rows * cols;
+      NMTG_REQUIRE((items + RP_THREADS - 1) / RP_THREADS <= 0x7fffffff, "add_rows: too many elements for one launch");
+      const unsigned grid = static_cast<unsigned>((items + RP_THREADS - 1) / RP_THREADS);
+      if (wide) hipLaunchKernelGGL((add_rows_kernel<T, WIDE>), dim3(grid), dim3(RP_THREADS), 0, st, static_cast<T*>(out), ld_out,
+                                   static_cast<const T*>(a), ld_a, static_cast<const T*>(b), ld_b, rows, static_cast<int>(cols));
+      else hipLaunchKernelGGL((add_rows_kernel<T, 1>), dim3(grid), dim3(RP_THREADS), 0, st, static_cast<T*>(out), ld_out,
+                              static_cast<const T*>(a), ld_a, static_cast<const T*>(b), ld_b, rows, static_cast<int>(cols)));
+  NMTG_CHECK_LAUNCH("add_rows");
   return 0;
 }

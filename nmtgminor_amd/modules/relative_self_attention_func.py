@@ -5,12 +5,15 @@ Mirrors RelativeShift, RelativeSelfAttnFunc and relative_self_attn_func of the r
 21 gradient slots. Every product is an MFMA GEMM (nmtg_gemm through native/linear_gemm.py and native/linear_blaslt.py),
 the additions of r_w_bias / r_r_bias, the relative shift with the sum of the two score terms and the shift's adjoint are
 the kernels of native/relative_position.py, softmax + dropout is the fused kernel of the other attention ops (mask fused,
-probabilities recomputed from the saved scores in the backward) and the bias gradients are column-sum kernels. What is
-left to PyTorch: views, allocation, and one elementwise add that joins the two query-gradient terms.
+probabilities recomputed from the saved scores in the backward), the bias gradients are column-sum kernels and the two
+query-gradient terms are joined by the row-add kernel. What is left to PyTorch: views and allocation.
 
-Covered: sinusoidal positions projected by pos_weights (learnable_pos=False), key-padding or time mask, training and
-inference, fp16 / bf16. Not covered, and raising instead of falling back: learnable position embeddings, incremental
-decoding. `recompute` is accepted and gives the same numbers; the intermediate tensors are kept either way. A 22nd
+Covered: sinusoidal positions projected by pos_weights (learnable_pos=False) and learnable position embeddings
+(learnable_pos=True: pos [len_q, len_k, head_dim], shared by heads and batch, no shift, no r_w_bias / r_r_bias, a gradient
+for pos), key-padding or time mask, training and inference, fp16 / bf16, and incremental decoding with projected positions
+(`incremental=True` with the reference's cache entries `k`, `v`, time-first [T, B, E]: the new keys and values are appended,
+the queries attend to everything cached; inference only). Not covered, and raising instead of falling back: incremental
+decoding with learnable positions. `recompute` is accepted and gives the same numbers; the intermediate tensors are kept either way. A 22nd
 optional argument replays an explicit dropout keep-mask."""
 import torch
 
@@ -53,33 +56,54 @@ class RelativeSelfAttnFunc(torch.autograd.Function):
     def forward(ctx, inputs, pos, use_time_mask, is_training, heads, input_weights, output_weights, pos_weights,
                 input_biases, output_biases, pos_biases, r_w_bias, r_r_bias, mask, dropout_prob, incremental,
                 incremental_cache, low_precision, learnable_pos, return_coverage, recompute, dropout_mask=None):
-        if learnable_pos:
-            raise NotImplementedError("relative_self_attn_func: learnable position embeddings have no HIP path")
-        if incremental:
-            raise NotImplementedError("relative_self_attn_func: incremental decoding has no HIP path")
+        if incremental and learnable_pos:
+            raise NotImplementedError("relative_self_attn_func: incremental decoding with learnable positions has no HIP path")
+        if incremental and (is_training or torch.is_grad_enabled() and inputs.requires_grad):
+            raise RuntimeError("relative_self_attn_func: incremental decoding is an inference path (no backward)")
         inputs = inputs.contiguous()
         len_q, bsz, embed = inputs.shape
         head_dim = embed // heads
         scale = head_dim ** -0.5
-        if pos.size(1) == 1:
-            pos = pos.repeat(1, bsz, 1)          # one position projection per batch column, as the reference lays it out
-        pos = pos.contiguous()
-        len_r = pos.size(0)
-        if len_r < len_q:
-            raise RuntimeError("relative_self_attn_func: %d relative positions for %d keys" % (len_r, len_q))
         mask_kw = _mask_kwargs(mask, use_time_mask)
 
         lin = linear_blaslt.forward(inputs, input_weights, input_biases)                  # [T, B, 3E]
-        pos_lin = linear_blaslt.forward(pos, pos_weights, pos_biases)                     # [R, B, E]
         lin4 = lin.view(len_q, bsz * heads, 3, head_dim)
         queries, keys, values = lin4[:, :, 0, :], lin4[:, :, 1, :], lin4[:, :, 2, :]
-        r_head_k = pos_lin.view(len_r, bsz * heads, head_dim)
-        rw_head_q, rr_head_q = relative_position.query_bias(queries, r_w_bias, r_r_bias, heads)
-
-        # AC = (q + r_w_bias) k^T, BD = shift((q + r_r_bias) r_k^T), both scaled by the GEMM
-        scores = linear_gemm.gemm(rw_head_q.transpose(0, 1), keys.transpose(0, 1), trans_b=True, alpha=scale)
-        matmul_bd = linear_gemm.gemm(rr_head_q.transpose(0, 1), r_head_k.transpose(0, 1), trans_b=True, alpha=scale)
-        relative_position.shift_add_(scores, matmul_bd)                                   # [B*H, T, T]
+        len_k = len_q
+        if incremental:
+            # the cache holds keys and values time-first as [T, B, E] (beam search re-indexes its batch dimension)
+            keys, values = keys.reshape(len_q, bsz, embed), values.reshape(len_q, bsz, embed)
+            if 'k' in incremental_cache and 'v' in incremental_cache:
+                keys = torch.cat([incremental_cache['k'], keys], dim=0)
+                values = torch.cat([incremental_cache['v'], values], dim=0)
+            incremental_cache['k'], incremental_cache['v'] = keys, values
+            len_k = keys.size(0)
+            keys, values = keys.view(len_k, bsz * heads, head_dim), values.view(len_k, bsz * heads, head_dim)
+        if learnable_pos:
+            # pos [len_q, len_k, head_dim]: scores[bh][i][j] = scale (q[i][bh] k[j][bh] + q[i][bh] pos[i][j]); the second
+            # product is batched over the query positions and written through the strides of the [B*H, T, T] layout
+            pos = pos.contiguous()
+            if pos.dim() != 3 or pos.shape != (len_q, len_q, head_dim):
+                raise RuntimeError("relative_self_attn_func: learnable positions must be [len_q, len_k, head_dim]")
+            pos_lin = rw_head_q = rr_head_q = None
+            scores = linear_gemm.gemm(queries.transpose(0, 1), keys.transpose(0, 1), trans_b=True, alpha=scale)
+            matmul_bd = torch.empty_like(scores)
+            linear_gemm.gemm(queries, pos, trans_b=True, alpha=scale, out=matmul_bd.transpose(0, 1))
+            relative_position.add_rows(scores, matmul_bd, out=scores)
+        else:
+            if pos.size(1) == 1:
+                pos = pos.repeat(1, bsz, 1)      # one position projection per batch column, as the reference lays it out
+            pos = pos.contiguous()
+            len_r = pos.size(0)
+            if len_r < len_k:
+                raise RuntimeError("relative_self_attn_func: %d relative positions for %d keys" % (len_r, len_k))
+            pos_lin = linear_blaslt.forward(pos, pos_weights, pos_biases)                 # [R, B, E]
+            r_head_k = pos_lin.view(len_r, bsz * heads, head_dim)
+            rw_head_q, rr_head_q = relative_position.query_bias(queries, r_w_bias, r_r_bias, heads)
+            # AC = (q + r_w_bias) k^T, BD = shift((q + r_r_bias) r_k^T), both scaled by the GEMM
+            scores = linear_gemm.gemm(rw_head_q.transpose(0, 1), keys.transpose(0, 1), trans_b=True, alpha=scale)
+            matmul_bd = linear_gemm.gemm(rr_head_q.transpose(0, 1), r_head_k.transpose(0, 1), trans_b=True, alpha=scale)
+            relative_position.shift_add_(scores, matmul_bd)                               # [B*H, T, T]
         del matmul_bd
 
         dmask, _, dropped = softmax_native.forward(is_training, heads, scores, dropout_prob, dropout_mask=dropout_mask,
@@ -88,9 +112,11 @@ class RelativeSelfAttnFunc(torch.autograd.Function):
         linear_gemm.gemm(dropped, values.transpose(0, 1), out=matmul2_results.transpose(0, 1))
         matmul2_results = matmul2_results.view(len_q, bsz, embed)
         outputs = linear_blaslt.forward(matmul2_results, output_weights, output_biases)
+        if incremental:
+            return (outputs, dropped) if return_coverage else outputs
 
         ctx.heads, ctx.p, ctx.scale = heads, dropout_prob if is_training else 0.0, scale
-        ctx.use_time_mask, ctx.return_coverage = use_time_mask, return_coverage
+        ctx.use_time_mask, ctx.return_coverage, ctx.learnable_pos = use_time_mask, return_coverage, learnable_pos
         ctx.save_for_backward(inputs, pos, input_weights, output_weights, pos_weights, lin, pos_lin, rw_head_q, rr_head_q,
                               scores, dropped, dmask, matmul2_results, mask)
         if return_coverage:
@@ -106,10 +132,8 @@ class RelativeSelfAttnFunc(torch.autograd.Function):
         output_grads = output_grads[0].contiguous()
         len_q, bsz, embed = inputs.shape
         head_dim = embed // heads
-        len_r = pos.size(0)
         lin4 = lin.view(len_q, bsz * heads, 3, head_dim)
-        keys, values = lin4[:, :, 1, :], lin4[:, :, 2, :]
-        r_head_k = pos_lin.view(len_r, bsz * heads, head_dim)
+        queries, keys, values = lin4[:, :, 0, :], lin4[:, :, 1, :], lin4[:, :, 2, :]
 
         output_lin_grads, output_weight_grads, output_bias_grads = \
             linear_blaslt.backward(matmul2_results, output_weights, output_grads, True)
@@ -124,27 +148,38 @@ class RelativeSelfAttnFunc(torch.autograd.Function):
                                                         **_mask_kwargs(mask, ctx.use_time_mask))
         del matmul2_dgrad1
 
-        # the score gradient flows to both terms: AC directly, BD through the adjoint of the shift
         queries_grads_ac = torch.empty(len_q, bsz * heads, head_dim, dtype=lin.dtype, device=lin.device)
-        linear_gemm.gemm(score_grads, keys.transpose(0, 1), alpha=scale, out=queries_grads_ac.transpose(0, 1))
-        linear_gemm.gemm(score_grads, rw_head_q.transpose(0, 1), trans_a=True, alpha=scale, out=keys_grads.transpose(0, 1))
-        r_w_bias_grads = linear_gemm.colsum(queries_grads_ac.view(len_q * bsz, embed)).view(heads, head_dim)
-
-        matmul_bd_grads = relative_position.shift_backward(score_grads, len_r)                     # [B*H, T, R]
-        del score_grads
         queries_grads_bd = torch.empty_like(queries_grads_ac)
-        linear_gemm.gemm(matmul_bd_grads, r_head_k.transpose(0, 1), alpha=scale, out=queries_grads_bd.transpose(0, 1))
-        r_head_k_grad = torch.empty(len_r, bsz * heads, head_dim, dtype=lin.dtype, device=lin.device)
-        linear_gemm.gemm(matmul_bd_grads, rr_head_q.transpose(0, 1), trans_a=True, alpha=scale,
-                         out=r_head_k_grad.transpose(0, 1))
-        r_r_bias_grads = linear_gemm.colsum(queries_grads_bd.view(len_q * bsz, embed)).view(heads, head_dim)
-        torch.add(queries_grads_ac, queries_grads_bd, out=queries_grads)
+        linear_gemm.gemm(score_grads, keys.transpose(0, 1), alpha=scale, out=queries_grads_ac.transpose(0, 1))
+        if ctx.learnable_pos:
+            # both products with the positions are batched over the query positions
+            linear_gemm.gemm(score_grads, queries.transpose(0, 1), trans_a=True, alpha=scale, out=keys_grads.transpose(0, 1))
+            by_query = score_grads.transpose(0, 1)                                                 # [T, B*H, T]
+            linear_gemm.gemm(by_query, pos, alpha=scale, out=queries_grads_bd)
+            pos_grads = linear_gemm.gemm(by_query, queries, trans_a=True, alpha=scale)             # [T, T, D]
+            r_w_bias_grads = r_r_bias_grads = pos_weight_grads = pos_bias_grads = None
+        else:
+            # the score gradient flows to both terms: AC directly, BD through the adjoint of the shift
+            len_r = pos.size(0)
+            r_head_k = pos_lin.view(len_r, bsz * heads, head_dim)
+            linear_gemm.gemm(score_grads, rw_head_q.transpose(0, 1), trans_a=True, alpha=scale, out=keys_grads.transpose(0, 1))
+            r_w_bias_grads = linear_gemm.colsum(queries_grads_ac.view(len_q * bsz, embed)).view(heads, head_dim)
+            matmul_bd_grads = relative_position.shift_backward(score_grads, len_r)                 # [B*H, T, R]
+            linear_gemm.gemm(matmul_bd_grads, r_head_k.transpose(0, 1), alpha=scale, out=queries_grads_bd.transpose(0, 1))
+            r_head_k_grad = torch.empty(len_r, bsz * heads, head_dim, dtype=lin.dtype, device=lin.device)
+            linear_gemm.gemm(matmul_bd_grads, rr_head_q.transpose(0, 1), trans_a=True, alpha=scale,
+                             out=r_head_k_grad.transpose(0, 1))
+            del matmul_bd_grads
+            r_r_bias_grads = linear_gemm.colsum(queries_grads_bd.view(len_q * bsz, embed)).view(heads, head_dim)
+            _, pos_weight_grads, pos_bias_grads = linear_blaslt.backward(pos, pos_weights,
+                                                                         r_head_k_grad.view(len_r, bsz, embed), False)
+            pos_grads = None
+        del score_grads
+        relative_position.add_rows(queries_grads_ac, queries_grads_bd, out=queries_grads)
 
-        _, pos_weight_grads, pos_bias_grads = linear_blaslt.backward(pos, pos_weights, r_head_k_grad.view(len_r, bsz, embed),
-                                                                     False)
         input_grads, input_weight_grads, input_bias_grads = \
             linear_blaslt.backward(inputs, input_weights, lin_grads.view(len_q, bsz, 3 * embed), True)
-        return (input_grads, None, None, None, None, input_weight_grads, output_weight_grads, pos_weight_grads,
+        return (input_grads, pos_grads, None, None, None, input_weight_grads, output_weight_grads, pos_weight_grads,
                 input_bias_grads, output_bias_grads, pos_bias_grads, r_w_bias_grads, r_r_bias_grads,
                 None, None, None, None, None, None, None, None, None)
 

@@ -53,3 +53,34 @@ def shift_backward(grad_scores, len_r):
     L.call("nmtg_rel_shift_bwd", L.ptr(grad_scores), L.ptr(out), L.i64(b), L.i64(tq), L.i64(tk), L.i64(len_r),
            L.i32(L.dtype_code(grad_scores)), L.stream_of(grad_scores))
     return out
+
+
+def _rows_view(t, what):
+    """(pointer tensor, rows, cols, pitch) of a tensor whose elements form rows of `cols` contiguous elements at one
+    uniform pitch (a dense tensor, or a slice of the last-but-one dimension such as the queries inside the in-projection
+    output)."""
+    _check(t.dim() >= 2 and t.stride(-1) == 1, what + ": innermost stride must be 1")
+    cols, ld = t.size(-1), t.stride(-2)
+    rows = t.numel() // max(cols, 1)
+    expect = ld
+    for dim in range(t.dim() - 2, -1, -1):
+        _check(t.size(dim) == 1 or t.stride(dim) == expect, what + ": rows must have one uniform pitch")
+        expect *= t.size(dim)
+    return rows, cols, ld
+
+
+def add_rows(a, b, out=None):
+    """out = a + b elementwise; the three tensors have equal shapes and each is a set of equally pitched rows (see
+    _rows_view). out defaults to a new dense tensor and may be a or b."""
+    L.require_cuda(a, b, out)
+    if out is None:
+        out = torch.empty(a.shape, dtype=a.dtype, device=a.device)
+    _check(a.shape == b.shape == out.shape and a.dtype == b.dtype == out.dtype, "add_rows: shapes or dtypes differ")
+    if a.numel() == 0:
+        return out
+    rows, cols, ld_a = _rows_view(a, "add_rows")
+    _, _, ld_b = _rows_view(b, "add_rows")
+    _, _, ld_o = _rows_view(out, "add_rows")
+    L.call("nmtg_add_rows", L.ptr(out), L.i64(ld_o), L.ptr(a), L.i64(ld_a), L.ptr(b), L.i64(ld_b), L.i64(rows), L.i64(cols),
+           L.i32(L.dtype_code(a)), L.stream_of(a))
+    return out

@@ -14,7 +14,8 @@ How it is pinned (tests/test_oracle_pins.py): the shift against the closed form 
 Python loops and against the Transformer-XL property it exists for (out[i][j] = x[i][R - 1 - (i - j)] for j <= i when
 R = T); its backward as the adjoint (<shift(x), y> = <x, shift_bwd(y)>) and against autograd of the forward; the
 attention forward against a per-element loop of the Transformer-XL definition under a causal mask; the attention
-backward against autograd of the forward in fp64.
+backward against autograd of the forward in fp64; the learnable-position branch (rel_learnable_attn_*) likewise against a
+per-element loop of its definition and fp64 autograd.
 """
 import torch
 
@@ -116,3 +117,60 @@ def rel_self_attn_bwd(dout, x, pos, w_in, w_out, w_pos, heads, fwd, p=0.0, dropo
     dpos_lin = dr_k.reshape(r * b, e)
     return dict(dx=(dlin @ w_in).view(t, b, e), dw_in=dlin.t() @ x2, db_in=dlin.sum(0), dw_out=dw_out, db_out=db_out,
                 dw_pos=dpos_lin.t() @ pos2, db_pos=dpos_lin.sum(0), dr_w_bias=dr_w_bias, dr_r_bias=dr_r_bias)
+
+
+def rel_learnable_attn_fwd(x, pos, w_in, w_out, b_in, b_out, heads, pad_mask=None, time_mask=None, p=0.0,
+                           dropout_mask=None, ctype=torch.float32, round_to=None, round_bd=False):
+    """The learnable-position branch (relative_self_attention_func.py:215-217, :254-263): pos [T, T, D] is an embedding of
+    the relative distance of every (query, key) pair, shared by heads and batch;
+    scores[bh][i][j] = (q[i][bh] . k[j][bh] + q[i][bh] . pos[i][j]) / sqrt(D); no shift, no r_w_bias / r_r_bias. The
+    reference accumulates the second product into the stored (rounded) first one and rounds the sum once; round_bd=True
+    models an implementation that stores the second product in `round_to` before the sum (one more rounding of one term)."""
+    t, b, e = x.shape
+    d = e // heads
+    scale = d ** -0.5
+    x, pos = x.to(ctype), pos.to(ctype)
+    lin = _r(_linear(x.reshape(t * b, e), w_in.to(ctype), None if b_in is None else b_in.to(ctype)), round_to)
+    lin = lin.view(t, b * heads, 3, d)
+    q, k, v = lin[:, :, 0, :], lin[:, :, 1, :], lin[:, :, 2, :]
+    ac = _r(torch.matmul(q.transpose(0, 1), k.transpose(0, 1).transpose(1, 2)) * scale, round_to)          # [BH, T, T]
+    bd = (torch.matmul(q, pos.transpose(1, 2)) * scale).transpose(0, 1)                                     # [T, BH, T] -> [BH, T, T]
+    if round_bd:
+        bd = _r(bd, round_to)
+    scores = masked_scores(_r(ac + bd, round_to), pad_mask, time_mask, heads)
+    sm, dr = softmax_dropout_fwd(scores, dropout_mask, p, ctype)
+    dr = _r(dr, round_to)
+    ctx = _r(torch.matmul(dr, v.transpose(0, 1)).transpose(0, 1), round_to).reshape(t, b, e)
+    out = _linear(ctx.reshape(t * b, e), w_out.to(ctype), None if b_out is None else b_out.to(ctype)).view(t, b, e)
+    return dict(input_lin_results=lin.reshape(t, b, 3 * e), attn_scores=scores, softmax_results=sm, dropout_results=dr,
+                matmul2_results=ctx, outputs=out)
+
+
+def rel_learnable_attn_bwd(dout, x, pos, w_in, w_out, heads, fwd, p=0.0, dropout_mask=None, ctype=torch.float32,
+                           round_to=None):
+    """Backward of the learnable-position branch (relative_self_attention_func.py:584-706). -> dict(dx, dpos [T, T, D],
+    dw_in, dw_out, db_in, db_out)."""
+    t, b, e = x.shape
+    d = e // heads
+    scale = d ** -0.5
+    x2, pos = x.to(ctype).reshape(t * b, e), pos.to(ctype)
+    w_in, w_out = w_in.to(ctype), w_out.to(ctype)
+    g = dout.to(ctype).reshape(t * b, e)
+    ctx = fwd["matmul2_results"].to(ctype).reshape(t * b, e)
+    dw_out, db_out = g.t() @ ctx, g.sum(0)
+    dctx = _r(g @ w_out, round_to).view(t, b * heads, d).transpose(0, 1)
+    lin = fwd["input_lin_results"].to(ctype).view(t, b * heads, 3, d)
+    q, k, v = lin[:, :, 0, :], lin[:, :, 1, :], lin[:, :, 2, :]
+    sm, dr = fwd["softmax_results"].to(ctype), fwd["dropout_results"].to(ctype)
+    d_dr = _r(torch.matmul(dctx, v.transpose(0, 1).transpose(1, 2)), round_to)
+    dv = _r(torch.matmul(dr.transpose(1, 2), dctx).transpose(0, 1), round_to)
+    ds = _r(softmax_dropout_bwd(d_dr, sm, dropout_mask, p, ctype), round_to)                               # [BH, T, T]
+    dq_ac = _r((torch.matmul(ds, k.transpose(0, 1)) * scale).transpose(0, 1), round_to)                    # [T, BH, D]
+    dk = _r((torch.matmul(ds.transpose(1, 2), q.transpose(0, 1)) * scale).transpose(0, 1), round_to)
+    by_query = ds.transpose(0, 1)                                                                           # [T, BH, T]
+    dq_bd = _r(torch.matmul(by_query, pos) * scale, round_to)                                               # [T, BH, D]
+    dpos = torch.matmul(by_query.transpose(1, 2), q) * scale                                                # [T, T, D]
+    dq = _r(dq_ac + dq_bd, round_to)
+    dlin = torch.stack([dq, dk, dv], dim=2).reshape(t * b, 3 * e)
+    return dict(dx=(dlin @ w_in).view(t, b, e), dpos=dpos, dw_in=dlin.t() @ x2, db_in=dlin.sum(0), dw_out=dw_out,
+                db_out=db_out)

@@ -475,6 +475,20 @@ def test_relative_attention(mi355x, dtype, t, b, e, h, len_r, pos_batch, causal,
 def test_relative_attention_module_and_inference(mi355x):
     trel.test_inference_returns_probabilities_and_single_output_form(CPU)
     trel.test_module_has_the_reference_parameters_and_runs(CPU)
+    trel.test_module_with_learnable_positions(CPU)
+    trel.test_step_by_step_decoding_reproduces_the_causal_rows(CPU)
+
+
+@pytest.mark.parametrize("dtype", HALVES)
+@pytest.mark.parametrize("t,b,e,h,causal,p", [(48, 2, 128, 2, False, 0.1), (33, 3, 192, 3, True, 0.0)])
+def test_relative_attention_with_learnable_positions(mi355x, dtype, t, b, e, h, causal, p):
+    trel.test_learnable_position_attention_matches_oracle(CPU, dtype, t, b, e, h, causal, p)
+
+
+@pytest.mark.parametrize("dtype", [BF16, F32])
+@pytest.mark.parametrize("shape,view", [((6, 8, 3, 16), "queries"), ((40, 24), "dense"), ((5, 7), "odd"), ((0, 8), "empty")])
+def test_row_add(mi355x, dtype, shape, view):
+    trel.test_row_add_on_dense_and_pitched_rows(CPU, dtype, shape, view)
 
 
 # ----------------------------------------------------------------------------- variants that are switched off by default

@@ -188,8 +188,11 @@ def test_relative_position_column_sums_and_linear_layer(recorder):
     relative_position.query_bias(lin[:, :, 0, :], r(2, 16), r(2, 16), 2)
     relative_position.shift_add_(r(6, 5, 5), r(6, 5, 8))
     relative_position.shift_backward(r(6, 5, 5), 8)
+    relative_position.add_rows(r(6, 5, 8), r(6, 5, 8))
+    relative_position.add_rows(r(6, 5, 8), r(6, 5, 3, 8)[:, :, 1, :], out=r(6, 5, 3, 8)[:, :, 0, :])
     linear_gemm.colsum(r(40, 24))
     linear_gemm.colsum(r(40, 32)[:, :24], out=torch.empty(24).to(BF))
     linear_blaslt.forward(r(4, 3, 16), r(24, 16), r(24))
     linear_blaslt.backward(r(4, 3, 16), r(24, 16), r(4, 3, 24), True)
-    assert {"nmtg_rel_query_bias", "nmtg_rel_shift_add", "nmtg_rel_shift_bwd", "nmtg_colsum", "nmtg_gemm"} <= set(recorder)
+    assert {"nmtg_rel_query_bias", "nmtg_rel_shift_add", "nmtg_rel_shift_bwd", "nmtg_add_rows", "nmtg_colsum",
+            "nmtg_gemm"} <= set(recorder)

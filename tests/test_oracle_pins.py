@@ -434,6 +434,40 @@ def test_relative_attention_backward_matches_autograd(causal, p, len_r, pos_batc
         assert leaves["pos"].grad.shape == d["pos"].shape
 
 
+def test_learnable_position_attention_matches_the_per_element_definition_and_autograd():
+    h, t, b, e = 2, 6, 2, 16
+    dh = e // h
+    d = inputs.self_attn_inputs(t, b, e, h, torch.float64, p=0.25, seed=11, zero_bias=False)
+    g = torch.Generator().manual_seed(12)
+    pos = torch.randn(t, t, dh, generator=g, dtype=D)
+    # forward, no dropout, no mask: out[i] = softmax_j((q_i . k_j + q_i . pos[i][j]) / sqrt(D)) v_j per (batch, head)
+    f0 = relative_attention.rel_learnable_attn_fwd(d["x"], pos, d["w_in"], d["w_out"], d["b_in"], d["b_out"], h, None, None, 0.0,
+                                                   None, D)
+    lin = (d["x"].reshape(t * b, e) @ d["w_in"].t() + d["b_in"]).view(t, b, h, 3, dh)
+    want = torch.zeros(t, b, e, dtype=D)
+    for n in range(b):
+        for hh in range(h):
+            q, k, v = lin[:, n, hh, 0], lin[:, n, hh, 1], lin[:, n, hh, 2]
+            for i in range(t):
+                s = torch.stack([(q[i] @ k[j] + q[i] @ pos[i, j]) * dh ** -0.5 for j in range(t)])
+                want[i, n, hh * dh:(hh + 1) * dh] = torch.softmax(s, 0) @ v
+    want = (want.reshape(t * b, e) @ d["w_out"].t() + d["b_out"]).view(t, b, e)
+    torch.testing.assert_close(f0["outputs"], want, rtol=1e-10, atol=1e-10)
+    # backward with key padding and dropout against autograd
+    names = ("x", "w_in", "w_out", "b_in", "b_out")
+    leaves = {k: d[k].clone().requires_grad_() for k in names}
+    pl = pos.clone().requires_grad_()
+    fa = relative_attention.rel_learnable_attn_fwd(leaves["x"], pl, leaves["w_in"], leaves["w_out"], leaves["b_in"],
+                                                   leaves["b_out"], h, d["pad_mask"], None, 0.25, d["dropout_mask"], D)
+    fa["outputs"].backward(d["dout"])
+    f = relative_attention.rel_learnable_attn_fwd(d["x"], pos, d["w_in"], d["w_out"], d["b_in"], d["b_out"], h, d["pad_mask"],
+                                                  None, 0.25, d["dropout_mask"], D)
+    gr = relative_attention.rel_learnable_attn_bwd(d["dout"], d["x"], pos, d["w_in"], d["w_out"], h, f, 0.25, d["dropout_mask"], D)
+    for k, gk in (("x", "dx"), ("w_in", "dw_in"), ("w_out", "dw_out"), ("b_in", "db_in"), ("b_out", "db_out")):
+        torch.testing.assert_close(gr[gk], leaves[k].grad, rtol=1e-9, atol=1e-10, msg=lambda m, k=k: f"{k}: {m}")
+    torch.testing.assert_close(gr["dpos"], pl.grad, rtol=1e-9, atol=1e-10)
+
+
 def _layer_params_from_torch(layer, heads, decoder):
     """nn.Transformer{En,De}coderLayer weights under the reference's key names and layouts."""
     sd = {k: v.detach() for k, v in layer.state_dict().items()}

@@ -163,7 +163,92 @@ def test_module_has_the_reference_parameters_and_runs(dev):
     assert_close(out, f["outputs"], torch.bfloat16, "module outputs")
     out.float().sum().backward()
     assert all(p.grad is not None for p in m.parameters())
-    with pytest.raises(NotImplementedError):
-        RelativeSelfMultiheadAttn(128, 4, learnable_pos=True, max_pos=8)
-    with pytest.raises(NotImplementedError):
-        m(x.to(dev), pos.to(dev), incremental=True, incremental_cache={})
+
+
+def test_step_by_step_decoding_reproduces_the_causal_rows(dev):
+    # Step i feeds one position and the positions of distances i..0; with the keys and values cached it must give row i of
+    # the full causal pass (the shift is the identity on a single query row).
+    dtype, t, b, e, h = torch.bfloat16, 10, 3, 128, 4
+    d = inputs.rel_self_attn_inputs(t, b, e, h, dtype, p=0.0, seed=21, causal=True)
+    a = {k: d[k].to(dev) for k in NAMES}
+    with torch.no_grad():
+        full = relative_self_attn_func(a["x"], a["pos"], True, False, h, a["w_in"], a["w_out"], a["w_pos"], a["b_in"], a["b_out"],
+                                       a["b_pos"], a["r_w_bias"], a["r_r_bias"], d["time_mask"].to(dev), 0.0, False, None, False,
+                                       False, False, False)
+        cache = {}
+        for i in range(t):
+            if i == 4:                                                     # beam search re-orders the hypotheses
+                order = torch.tensor([2, 0, 1], device=dev)
+                cache = {k: v.index_select(1, order) for k, v in cache.items()}
+                a["x"], full = a["x"].index_select(1, order), full.index_select(1, order)
+            step, cov = relative_self_attn_func(a["x"][i:i + 1], a["pos"][t - 1 - i:], False, False, h, a["w_in"], a["w_out"],
+                                                a["w_pos"], a["b_in"], a["b_out"], a["b_pos"], a["r_w_bias"], a["r_r_bias"], None,
+                                                0.0, True, cache, False, False, True, False)
+            assert step.shape == (1, b, e) and cov.shape == (b * h, 1, i + 1) and cache["k"].shape == (i + 1, b, e)
+            assert_close(step[0], full[i].float().cpu(), dtype, f"step {i}", atol=2e-3)
+    with pytest.raises(RuntimeError):
+        relative_self_attn_func(a["x"][:1], a["pos"], False, True, h, a["w_in"], a["w_out"], a["w_pos"], a["b_in"], a["b_out"],
+                                a["b_pos"], a["r_w_bias"], a["r_r_bias"], None, 0.0, True, {}, False, False, True, False)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape,view", [((6, 8, 3, 16), "queries"), ((40, 24), "dense"), ((5, 7), "odd"), ((0, 8), "empty")])
+def test_row_add_on_dense_and_pitched_rows(dev, dtype, shape, view):
+    g = torch.Generator().manual_seed(len(shape))
+    a, b = torch.randint(-8, 9, shape, generator=g).to(dtype), torch.randint(-8, 9, shape, generator=g).to(dtype)
+    ad, bd = a.to(dev), b.to(dev)
+    if view == "queries":                                       # the sum lands inside a [T, B*H, 3, D] gradient tensor
+        out = torch.full(shape, 99, dtype=dtype, device=dev)
+        got = relative_position.add_rows(ad[:, :, 0, :].contiguous(), bd[:, :, 1, :], out=out[:, :, 0, :])
+        assert torch.equal(out[:, :, 0, :].cpu(), a[:, :, 0, :] + b[:, :, 1, :]) and (out[:, :, 1:, :] == 99).all()
+        assert got.data_ptr() == out.data_ptr()
+        with pytest.raises(RuntimeError):
+            relative_position.add_rows(ad.transpose(0, 1)[:, :, 0, :], bd.transpose(0, 1)[:, :, 0, :])
+    else:
+        assert torch.equal(relative_position.add_rows(ad, bd).cpu(), a + b)
+        assert torch.equal(relative_position.add_rows(ad, bd, out=ad).cpu(), a + b)          # in place
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("t,b,e,h,causal,p", [(48, 2, 128, 2, False, 0.1), (33, 3, 192, 3, True, 0.0)])
+def test_learnable_position_attention_matches_oracle(dev, dtype, t, b, e, h, causal, p):
+    d = inputs.self_attn_inputs(t, b, e, h, dtype, p=p, seed=300 + t, zero_bias=False, causal=causal)
+    pos = (0.5 * torch.randn(t, t, e // h, generator=torch.Generator().manual_seed(t))).to(dtype)
+    names = ("x", "w_in", "w_out", "b_in", "b_out")
+    leaves = {k: d[k].to(dev).requires_grad_() for k in names}
+    pl = pos.to(dev).requires_grad_()
+    mask = d["time_mask"] if causal else d["pad_mask"]
+    dm = d["dropout_mask"].to(dev) if p > 0 else None
+    out, cov = relative_self_attn_func(leaves["x"], pl, causal, True, h, leaves["w_in"], leaves["w_out"], None, leaves["b_in"],
+                                       leaves["b_out"], None, None, None, mask.to(dev), p, False, None, False, True, True,
+                                       False, dm)
+    out.backward(d["dout"].to(dev))
+    # The HIP path stores the second score term in 16 bits before the sum; the reference accumulates it in fp32 into the
+    # stored first term. The oracle models the first (round_bd=True) for the comparison at the 16-bit tolerance; against
+    # the reference's own rounding points the outputs agree to 5e-3 absolute (a score whose final rounding flips moves its
+    # probability by 2^-8 relative, which shows in outputs that cancel to near zero).
+    args = (d["x"], pos, d["w_in"], d["w_out"], d["b_in"], d["b_out"], h, d["pad_mask"], d["time_mask"], p, d["dropout_mask"], D)
+    f = orel.rel_learnable_attn_fwd(*args, round_to=dtype, round_bd=True)
+    g = orel.rel_learnable_attn_bwd(d["dout"], d["x"], pos, d["w_in"], d["w_out"], h, f, p, d["dropout_mask"], D, round_to=dtype)
+    assert_close(out, orel.rel_learnable_attn_fwd(*args, round_to=dtype)["outputs"], dtype, "outputs, reference rounding", atol=5e-3)
+    assert_close(out, f["outputs"], dtype, "outputs", atol=2e-3)
+    assert_close(cov, f["dropout_results"], dtype, "coverage")
+    for k, gk in (("x", "dx"), ("w_in", "dw_in"), ("w_out", "dw_out"), ("b_in", "db_in"), ("b_out", "db_out")):
+        assert_close(leaves[k].grad, g[gk], dtype, "grad " + k, scale_atol=k != "x")
+    assert_close(pl.grad, g["dpos"], dtype, "grad pos", scale_atol=True)
+
+
+def test_module_with_learnable_positions(dev):
+    torch.manual_seed(6)
+    m = RelativeSelfMultiheadAttn(128, 4, dropout=0.0, learnable_pos=True, max_pos=16).to(dev).to(torch.bfloat16)
+    assert m.pos_proj_weight is None and tuple(m.pos_emb.weight.shape) == (33, 32)
+    t = 12
+    x = torch.randn(t, 2, 128, generator=torch.Generator().manual_seed(7)).to(torch.bfloat16)
+    dist = (torch.arange(t).view(t, 1) - torch.arange(t).view(1, t)).clamp(-16, 16) + 16           # [T, T] distance indices
+    out, cov = m(x.to(dev), dist.to(dev))
+    P = {k: v.detach().cpu() for k, v in m.named_parameters()}
+    f = orel.rel_learnable_attn_fwd(x, P["pos_emb.weight"][dist], P["in_proj_weight"], P["out_proj_weight"], P["in_proj_bias"],
+                                    P["out_proj_bias"], 4, None, None, 0.0, None, D, round_to=torch.bfloat16, round_bd=True)
+    assert_close(out, f["outputs"], torch.bfloat16, "module outputs", atol=2e-3)
+    out.float().sum().backward()
+    assert m.pos_emb.weight.grad is not None and m.in_proj_weight.grad is not None
