@@ -2,7 +2,8 @@
 
 Mirrors RelativeShift, RelativeSelfAttnFunc and relative_self_attn_func of the reference
 (onmt/modules/optimized/relative_self_attention_func.py:26-76, :79-726, :738-766): the same 21 positional arguments and
-21 gradient slots. Every product is an MFMA GEMM (nmtg_gemm through native/linear_gemm.py and native/linear_blaslt.py),
+21 gradient slots. The projected-position form runs in native/relative_self_attn_blaslt.py (the stand-in of the reference's
+extension of that name). Every product is an MFMA GEMM (nmtg_gemm through native/linear_gemm.py and native/linear_blaslt.py),
 the additions of r_w_bias / r_r_bias, the relative shift with the sum of the two score terms and the shift's adjoint are
 the kernels of native/relative_position.py, softmax + dropout is the fused kernel of the other attention ops (mask fused,
 probabilities recomputed from the saved scores in the backward), the bias gradients are column-sum kernels and the two
@@ -17,7 +18,8 @@ decoding with learnable positions. `recompute` is accepted and gives the same nu
 optional argument replays an explicit dropout keep-mask."""
 import torch
 
-from ..native import linear_blaslt, linear_gemm, mask_softmax_dropout_cuda as softmax_native, relative_position
+from ..native import (linear_blaslt, linear_gemm, mask_softmax_dropout_cuda as softmax_native, relative_position,
+                      relative_self_attn_blaslt as native)
 from ._autocast import cast_if_autocast_enabled, no_autocast
 
 
@@ -42,15 +44,6 @@ class RelativeShift(object):
         return relative_position.shift_backward(grad_x, grad_x.size(2))
 
 
-def _mask_kwargs(mask, use_time_mask):
-    if mask is None:
-        return {}
-    if use_time_mask:
-        assert mask.dim() == 2, "Timing mask is not 2D!"
-        return dict(time_mask=mask)
-    return dict(pad_mask=mask)
-
-
 class RelativeSelfAttnFunc(torch.autograd.Function):
     @staticmethod
     def forward(ctx, inputs, pos, use_time_mask, is_training, heads, input_weights, output_weights, pos_weights,
@@ -64,12 +57,28 @@ class RelativeSelfAttnFunc(torch.autograd.Function):
         len_q, bsz, embed = inputs.shape
         head_dim = embed // heads
         scale = head_dim ** -0.5
-        mask_kw = _mask_kwargs(mask, use_time_mask)
+        mask_kw = native._mask_kwargs(mask, use_time_mask)
+        ctx.heads, ctx.p = heads, dropout_prob if is_training else 0.0
+        ctx.use_time_mask, ctx.return_coverage, ctx.learnable_pos = use_time_mask, return_coverage, learnable_pos
+
+        if not learnable_pos:
+            if pos.size(1) == 1:
+                pos = pos.repeat(1, bsz, 1)      # one position projection per batch column, as the reference lays it out
+            pos = pos.contiguous()
+            if not incremental:
+                lin, pos_lin, scores, dropped, dmask, matmul2_results, outputs = native.forward(
+                    is_training, use_time_mask, heads, inputs, pos, input_weights, output_weights, pos_weights, input_biases,
+                    output_biases, pos_biases, r_w_bias, r_r_bias, mask, dropout_prob, dropout_mask=dropout_mask)
+                ctx.save_for_backward(inputs, pos, input_weights, output_weights, pos_weights, lin, pos_lin, r_w_bias, r_r_bias,
+                                      scores, dropped, dmask, matmul2_results, mask)
+                if return_coverage:
+                    ctx.mark_non_differentiable(dropped)
+                    return outputs, dropped
+                return outputs
 
         lin = linear_blaslt.forward(inputs, input_weights, input_biases)                  # [T, B, 3E]
         lin4 = lin.view(len_q, bsz * heads, 3, head_dim)
         queries, keys, values = lin4[:, :, 0, :], lin4[:, :, 1, :], lin4[:, :, 2, :]
-        len_k = len_q
         if incremental:
             # the cache holds keys and values time-first as [T, B, E] (beam search re-indexes its batch dimension)
             keys, values = keys.reshape(len_q, bsz, embed), values.reshape(len_q, bsz, embed)
@@ -79,109 +88,74 @@ class RelativeSelfAttnFunc(torch.autograd.Function):
             incremental_cache['k'], incremental_cache['v'] = keys, values
             len_k = keys.size(0)
             keys, values = keys.view(len_k, bsz * heads, head_dim), values.view(len_k, bsz * heads, head_dim)
-        if learnable_pos:
-            # pos [len_q, len_k, head_dim]: scores[bh][i][j] = scale (q[i][bh] k[j][bh] + q[i][bh] pos[i][j]); the second
-            # product is batched over the query positions and written through the strides of the [B*H, T, T] layout
+            pos_lin = linear_blaslt.forward(pos, pos_weights, pos_biases)                 # [R, B, E]
+            scores = native.relative_scores(queries, keys, pos_lin.view(pos.size(0), bsz * heads, head_dim), r_w_bias,
+                                            r_r_bias, heads, scale)
+        else:
+            # learnable positions, pos [len_q, len_k, head_dim]: scores[bh][i][j] = scale (q[i][bh] k[j][bh] + q[i][bh]
+            # pos[i][j]); the second product is batched over the query positions and written through the strides of the
+            # [B*H, T, T] layout
             pos = pos.contiguous()
             if pos.dim() != 3 or pos.shape != (len_q, len_q, head_dim):
                 raise RuntimeError("relative_self_attn_func: learnable positions must be [len_q, len_k, head_dim]")
-            pos_lin = rw_head_q = rr_head_q = None
             scores = linear_gemm.gemm(queries.transpose(0, 1), keys.transpose(0, 1), trans_b=True, alpha=scale)
             matmul_bd = torch.empty_like(scores)
             linear_gemm.gemm(queries, pos, trans_b=True, alpha=scale, out=matmul_bd.transpose(0, 1))
             relative_position.add_rows(scores, matmul_bd, out=scores)
-        else:
-            if pos.size(1) == 1:
-                pos = pos.repeat(1, bsz, 1)      # one position projection per batch column, as the reference lays it out
-            pos = pos.contiguous()
-            len_r = pos.size(0)
-            if len_r < len_k:
-                raise RuntimeError("relative_self_attn_func: %d relative positions for %d keys" % (len_r, len_k))
-            pos_lin = linear_blaslt.forward(pos, pos_weights, pos_biases)                 # [R, B, E]
-            r_head_k = pos_lin.view(len_r, bsz * heads, head_dim)
-            rw_head_q, rr_head_q = relative_position.query_bias(queries, r_w_bias, r_r_bias, heads)
-            # AC = (q + r_w_bias) k^T, BD = shift((q + r_r_bias) r_k^T), both scaled by the GEMM
-            scores = linear_gemm.gemm(rw_head_q.transpose(0, 1), keys.transpose(0, 1), trans_b=True, alpha=scale)
-            matmul_bd = linear_gemm.gemm(rr_head_q.transpose(0, 1), r_head_k.transpose(0, 1), trans_b=True, alpha=scale)
-            relative_position.shift_add_(scores, matmul_bd)                               # [B*H, T, T]
-        del matmul_bd
-
-        dmask, _, dropped = softmax_native.forward(is_training, heads, scores, dropout_prob, dropout_mask=dropout_mask,
-                                                   want_softmax=False, **mask_kw)
-        matmul2_results = torch.empty(len_q, bsz * heads, head_dim, dtype=inputs.dtype, device=inputs.device)
-        linear_gemm.gemm(dropped, values.transpose(0, 1), out=matmul2_results.transpose(0, 1))
-        matmul2_results = matmul2_results.view(len_q, bsz, embed)
+            del matmul_bd
+        dmask, dropped, context = native.attend(scores, values, is_training, heads, dropout_prob, mask_kw, dropout_mask)
+        matmul2_results = context.view(len_q, bsz, embed)
         outputs = linear_blaslt.forward(matmul2_results, output_weights, output_biases)
-        if incremental:
-            return (outputs, dropped) if return_coverage else outputs
-
-        ctx.heads, ctx.p, ctx.scale = heads, dropout_prob if is_training else 0.0, scale
-        ctx.use_time_mask, ctx.return_coverage, ctx.learnable_pos = use_time_mask, return_coverage, learnable_pos
-        ctx.save_for_backward(inputs, pos, input_weights, output_weights, pos_weights, lin, pos_lin, rw_head_q, rr_head_q,
-                              scores, dropped, dmask, matmul2_results, mask)
-        if return_coverage:
-            ctx.mark_non_differentiable(dropped)
-            return outputs, dropped
-        return outputs
+        if not incremental:
+            ctx.save_for_backward(inputs, pos, input_weights, output_weights, lin, scores, dropped, dmask, matmul2_results, mask)
+            if return_coverage:
+                ctx.mark_non_differentiable(dropped)
+        return (outputs, dropped) if return_coverage else outputs
 
     @staticmethod
     def backward(ctx, *output_grads):
-        (inputs, pos, input_weights, output_weights, pos_weights, lin, pos_lin, rw_head_q, rr_head_q, scores, dropped,
-         dmask, matmul2_results, mask) = ctx.saved_tensors
-        heads, p, scale = ctx.heads, ctx.p, ctx.scale
-        output_grads = output_grads[0].contiguous()
+        heads, p = ctx.heads, ctx.p
+        tail = (None,) * 9                                      # mask ... recompute, dropout_mask
+        if not ctx.learnable_pos:
+            (inputs, pos, input_weights, output_weights, pos_weights, lin, pos_lin, r_w_bias, r_r_bias, scores, dropped, dmask,
+             matmul2_results, mask) = ctx.saved_tensors
+            (input_grads, input_weight_grads, pos_weight_grads, output_weight_grads, input_bias_grads, pos_bias_grads,
+             output_bias_grads, r_w_bias_grads, r_r_bias_grads) = native.backward(
+                heads, output_grads[0], matmul2_results, dropped, scores, lin, pos_lin, r_w_bias, r_r_bias, inputs, pos,
+                input_weights, output_weights, pos_weights, dmask, p, **native._mask_kwargs(mask, ctx.use_time_mask))
+            return (input_grads, None, None, None, None, input_weight_grads, output_weight_grads, pos_weight_grads,
+                    input_bias_grads, output_bias_grads, pos_bias_grads, r_w_bias_grads, r_r_bias_grads) + tail
+
+        inputs, pos, input_weights, output_weights, lin, scores, dropped, dmask, matmul2_results, mask = ctx.saved_tensors
+        grads = output_grads[0].contiguous()
         len_q, bsz, embed = inputs.shape
         head_dim = embed // heads
+        scale = head_dim ** -0.5
         lin4 = lin.view(len_q, bsz * heads, 3, head_dim)
         queries, keys, values = lin4[:, :, 0, :], lin4[:, :, 1, :], lin4[:, :, 2, :]
-
-        output_lin_grads, output_weight_grads, output_bias_grads = \
-            linear_blaslt.backward(matmul2_results, output_weights, output_grads, True)
+        output_lin_grads, output_weight_grads, output_bias_grads = linear_blaslt.backward(matmul2_results, output_weights, grads, True)
         output_lin_grads = output_lin_grads.view(len_q, bsz * heads, head_dim).transpose(0, 1)      # [B*H, T, D]
-
         lin_grads = torch.empty_like(lin4)
         queries_grads, keys_grads, values_grads = lin_grads[:, :, 0, :], lin_grads[:, :, 1, :], lin_grads[:, :, 2, :]
         matmul2_dgrad1 = linear_gemm.gemm(output_lin_grads, values.transpose(0, 1), trans_b=True)  # [B*H, T, T]
         linear_gemm.gemm(dropped, output_lin_grads, trans_a=True, out=values_grads.transpose(0, 1))
-        # dropout and softmax backward in one kernel, probabilities recomputed from the saved scores (mask fused)
         score_grads = softmax_native.backward_recompute(heads, matmul2_dgrad1, None, scores, dmask, p,
-                                                        **_mask_kwargs(mask, ctx.use_time_mask))
+                                                        **native._mask_kwargs(mask, ctx.use_time_mask))
         del matmul2_dgrad1
-
         queries_grads_ac = torch.empty(len_q, bsz * heads, head_dim, dtype=lin.dtype, device=lin.device)
         queries_grads_bd = torch.empty_like(queries_grads_ac)
         linear_gemm.gemm(score_grads, keys.transpose(0, 1), alpha=scale, out=queries_grads_ac.transpose(0, 1))
-        if ctx.learnable_pos:
-            # both products with the positions are batched over the query positions
-            linear_gemm.gemm(score_grads, queries.transpose(0, 1), trans_a=True, alpha=scale, out=keys_grads.transpose(0, 1))
-            by_query = score_grads.transpose(0, 1)                                                 # [T, B*H, T]
-            linear_gemm.gemm(by_query, pos, alpha=scale, out=queries_grads_bd)
-            pos_grads = linear_gemm.gemm(by_query, queries, trans_a=True, alpha=scale)             # [T, T, D]
-            r_w_bias_grads = r_r_bias_grads = pos_weight_grads = pos_bias_grads = None
-        else:
-            # the score gradient flows to both terms: AC directly, BD through the adjoint of the shift
-            len_r = pos.size(0)
-            r_head_k = pos_lin.view(len_r, bsz * heads, head_dim)
-            linear_gemm.gemm(score_grads, rw_head_q.transpose(0, 1), trans_a=True, alpha=scale, out=keys_grads.transpose(0, 1))
-            r_w_bias_grads = linear_gemm.colsum(queries_grads_ac.view(len_q * bsz, embed)).view(heads, head_dim)
-            matmul_bd_grads = relative_position.shift_backward(score_grads, len_r)                 # [B*H, T, R]
-            linear_gemm.gemm(matmul_bd_grads, r_head_k.transpose(0, 1), alpha=scale, out=queries_grads_bd.transpose(0, 1))
-            r_head_k_grad = torch.empty(len_r, bsz * heads, head_dim, dtype=lin.dtype, device=lin.device)
-            linear_gemm.gemm(matmul_bd_grads, rr_head_q.transpose(0, 1), trans_a=True, alpha=scale,
-                             out=r_head_k_grad.transpose(0, 1))
-            del matmul_bd_grads
-            r_r_bias_grads = linear_gemm.colsum(queries_grads_bd.view(len_q * bsz, embed)).view(heads, head_dim)
-            _, pos_weight_grads, pos_bias_grads = linear_blaslt.backward(pos, pos_weights,
-                                                                         r_head_k_grad.view(len_r, bsz, embed), False)
-            pos_grads = None
+        linear_gemm.gemm(score_grads, queries.transpose(0, 1), trans_a=True, alpha=scale, out=keys_grads.transpose(0, 1))
+        # both products with the positions are batched over the query positions
+        by_query = score_grads.transpose(0, 1)                                                     # [T, B*H, T]
+        linear_gemm.gemm(by_query, pos, alpha=scale, out=queries_grads_bd)
+        pos_grads = linear_gemm.gemm(by_query, queries, trans_a=True, alpha=scale)                 # [T, T, D]
         del score_grads
         relative_position.add_rows(queries_grads_ac, queries_grads_bd, out=queries_grads)
-
         input_grads, input_weight_grads, input_bias_grads = \
             linear_blaslt.backward(inputs, input_weights, lin_grads.view(len_q, bsz, 3 * embed), True)
-        return (input_grads, pos_grads, None, None, None, input_weight_grads, output_weight_grads, pos_weight_grads,
-                input_bias_grads, output_bias_grads, pos_bias_grads, r_w_bias_grads, r_r_bias_grads,
-                None, None, None, None, None, None, None, None, None)
+        return (input_grads, pos_grads, None, None, None, input_weight_grads, output_weight_grads, None, input_bias_grads,
+                output_bias_grads, None, None, None) + tail
 
 
 def relative_self_attn_func(input, pos, use_mask, is_training, num_heads, in_proj_weight, out_proj_weight,

@@ -11,7 +11,7 @@ import torch
 
 from nmtgminor_amd.modules.relative_self_attention import RelativeSelfMultiheadAttn
 from nmtgminor_amd.modules.relative_self_attention_func import RelativeShift, relative_self_attn_func
-from nmtgminor_amd.native import linear_blaslt, linear_gemm, relative_position
+from nmtgminor_amd.native import linear_blaslt, linear_gemm, relative_position, relative_self_attn_blaslt
 from oracle import inputs, relative_attention as orel
 from util import assert_close
 
@@ -129,6 +129,32 @@ def test_relative_attention_matches_oracle(dev, dtype, t, b, e, h, len_r, pos_ba
     for name, key in GRADS:
         assert_close(leaves[name].grad, g[key], dtype, "grad " + name, scale_atol=name != "x")
     assert leaves["pos"].grad is None                                       # the reference returns no gradient for pos
+
+
+def test_extension_stand_in_keeps_the_reference_argument_order_and_lists(dev):
+    dtype, h, p = torch.bfloat16, 4, 0.1
+    d = inputs.rel_self_attn_inputs(32, 2, 128, h, dtype, p=p, seed=31, pos_batch=2)
+    a = {k: d[k].to(dev) for k in NAMES}
+    pad, dm, dout = d["pad_mask"].to(dev), d["dropout_mask"].to(dev), d["dout"].to(dev)
+    res = relative_self_attn_blaslt.forward(True, False, h, a["x"], a["pos"], a["w_in"], a["w_out"], a["w_pos"], a["b_in"],
+                                            a["b_out"], a["b_pos"], a["r_w_bias"], a["r_r_bias"], pad, p, dropout_mask=dm)
+    lin, pos_lin, scores, dropped, dmask, ctx, out = res
+    assert [tuple(t.shape) for t in res] == [(32, 2, 384), (32, 2, 128), (8, 32, 32), (8, 32, 32), (8, 32, 32), (32, 2, 128),
+                                             (32, 2, 128)]
+    grads = relative_self_attn_blaslt.backward(h, dout, ctx, dropped, scores, lin, pos_lin, a["r_w_bias"], a["r_r_bias"], a["x"],
+                                               a["pos"], a["w_in"], a["w_out"], a["w_pos"], dmask, p, pad_mask=pad)
+    f = orel.rel_self_attn_fwd(*(d[k] for k in NAMES), h, d["pad_mask"], None, p, d["dropout_mask"], D, round_to=dtype)
+    g = orel.rel_self_attn_bwd(d["dout"], d["x"], d["pos"], d["w_in"], d["w_out"], d["w_pos"], h, f, p, d["dropout_mask"], D,
+                               round_to=dtype)
+    assert_close(lin, f["input_lin_results"], dtype, "input_lin_results")
+    assert_close(pos_lin, f["pos_lin_results"], dtype, "pos_lin_results")
+    assert_close(ctx, f["matmul2_results"], dtype, "matmul2_results", atol=2e-3)
+    finite = torch.isfinite(f["attn_scores"])                  # the stored scores are unmasked; compare where the oracle's are
+    assert_close(scores.cpu().float()[finite], f["attn_scores"][finite], dtype, "attn_scores", atol=2e-2)   # one 16-bit ulp at |s| ~ 4
+    order = ("dx", "dw_in", "dw_pos", "dw_out", "db_in", "db_pos", "db_out", "dr_w_bias", "dr_r_bias")
+    assert len(grads) == 9
+    for got, key in zip(grads, order):
+        assert_close(got, g[key], dtype, key, scale_atol=key != "dx")
 
 
 def test_inference_returns_probabilities_and_single_output_form(dev):
