@@ -15,7 +15,7 @@ import bench  # noqa: E402
 
 
 def _args(**kw):
-    d = dict(steps=5, warmup=1, trace_steps=2, no_cpu=True)
+    d = dict(steps=5, warmup=1, trace_steps=2, no_cpu=True, cpu_time_allowance=240.0)
     d.update(kw)
     return types.SimpleNamespace(**d)
 
