@@ -480,6 +480,60 @@ class DropoutAddWL(Workload):
                     sample="full workload ([512 x 32 x 1024] bf16 fwd+bwd), median of 3")
 
 
+class FusedAdamWL(Workload):
+    name = "fused_adam"
+    bound = "hbm"
+    dtype = "f32"
+    description = ("AdamW update of a transformer-base parameter list in fp32: 6 + 6 layers of E=512 / inner 2048 weights and "
+                   "biases plus a 32000 x 512 embedding, 193 tensors, 60.5 M elements, one multi-tensor pass")
+    E, INNER, VOCAB, LAYERS = 512, 2048, 32000, 12
+
+    def shapes(self):
+        e, f = self.E, self.INNER
+        per_layer = [(3 * e, e), (3 * e,), (e, e), (e,), (f, e), (f,), (e, f), (e,), (e,), (e,), (e,), (e,)]
+        # decoder layers carry a cross-attention block as well
+        cross = [(e, e), (e,), (2 * e, e), (2 * e,), (e, e), (e,), (e,), (e,)]
+        out = [(self.VOCAB, e)]
+        for i in range(self.LAYERS):
+            out += per_layer + (cross if i >= self.LAYERS // 2 else [])
+        return out
+
+    def setup(self, dev):
+        from nmtgminor_amd.native import fused_optim
+        self.op = fused_optim.multi_tensor_adam
+        g = torch.Generator(device=dev).manual_seed(1007)
+        mk = lambda s, scale: scale * torch.randn(s, generator=g, device=dev)
+        shapes = self.shapes()
+        self.lists = [[mk(s, 1e-2) for s in shapes], [mk(s, 0.1) for s in shapes], [mk(s, 1e-3) for s in shapes],
+                      [mk(s, 1e-3).abs() for s in shapes]]
+        self.n = sum(t.numel() for t in self.lists[0])
+        self.step_no = 0
+
+    def step(self):
+        self.step_no += 1
+        self.op(65536, None, self.lists, 1e-4, 0.9, 0.98, 1e-8, self.step_no, 1, 1, 0.01)
+        return self.lists[1][0]
+
+    def work_per_step(self):
+        return 7 * 4 * self.n                                # g, p, m, v read; p, m, v written
+
+    def kernel_work(self):
+        return {"multi_tensor_adam": self.work_per_step()}
+
+    def cpu_baseline(self):
+        from oracle import fused_optim as o
+        k = 24                                               # the first tensors: the embedding and two layers
+        lists = [[t.detach().cpu() for t in lst[:k]] for lst in self.lists]
+        n = sum(t.numel() for t in lists[0])
+
+        def run():
+            for g, p, m, v in zip(*lists):
+                o.adam_step(g, p, m, v, 1e-4, 0.9, 0.98, 1e-8, 3, 1, True, 0.01)
+        t = _time_cpu(run, 3)
+        return dict(value=7 * 4 * n / t / 1e9, unit="GB/s", cores=torch.get_num_threads(), kind="port",
+                    sample=f"the first {k} of {len(self.lists[0])} tensors ({n} elements), fp32, median of 3")
+
+
 class GeneratorLossWL(Workload):
     name = "generator_loss"
     bound = "mfma"
@@ -552,7 +606,7 @@ class CopyWL(Workload):
 
 # the five benchmark configurations first, then the workloads added beside them
 WORKLOADS = {w.name: w for w in (LayerNormWL, MlpWL, SelfAttnWL, EncdecAttnWL, XentropyWL, SoftmaxDropoutWL, DropoutAddWL,
-                                    GeneratorLossWL, RelSelfAttnWL)}
+                                    GeneratorLossWL, RelSelfAttnWL, FusedAdamWL)}
 EXTRA_WORKLOADS = {CopyWL.name: CopyWL}
 PRIMARY = "mlp"
 

@@ -329,6 +329,40 @@ int nmtg_add_rows(void* out, int64_t ld_out, const void* a, int64_t ld_a, const 
                   int64_t rows, int64_t cols, int dtype, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Optimizer-side passes over a list of tensors (one launch per 48 tensors instead of one per tensor).
+ * Reference: fused_optim.multi_tensor_adam / multi_tensor_scale / multi_tensor_l2norm
+ *   (onmt/modules/extensions/fused_optim/frontend.cpp:45-53; multi_tensor_adam.cu:22-171,
+ *   multi_tensor_scale_kernel.cu:29-136, multi_tensor_l2norm_kernel.cu:27-232, :293-367), driven by
+ *   FusedAdam.step (onmt/modules/optimized/fused_adam.py:113-191).
+ * The lists are HOST arrays of n_tensors device pointers; sizes[t] is tensor t's element count (each
+ * tensor dense). fp32 arithmetic whatever the storage type.
+ *
+ * nmtg_multi_tensor_adam: per element, with g, p, m, v of grads / params / exp_avg / exp_avg_sq:
+ *   mode 0 (L2): g += weight_decay * p;  m = beta1 m + (1 - beta1) g;  v = beta2 v + (1 - beta2) g g;
+ *   update = (m / c1) / (sqrt(v / c2) + eps), mode 1 (decoupled decay): update += weight_decay * p;
+ *   p -= lr * update;  c1 = 1 - beta1^step, c2 = 1 - beta2^step, or 1 without bias_correction.
+ *   p, m, v are updated in place; the four lists share one dtype.
+ * nmtg_multi_tensor_scale: out = in * scale (dtypes may differ); *noop_flag (device int, may be NULL)
+ *   is set to 1 if any input element is inf or NaN, and left alone otherwise.
+ * nmtg_multi_tensor_l2norm: norm[0] = sqrt(sum over all tensors of x^2); per_tensor[t] (may be NULL)
+ *   = the norm of tensor t; both fp32 on the device; deterministic (fixed-order sums). workspace: fp32
+ *   scratch of nmtg_multi_tensor_l2norm_workspace_bytes(n_tensors, sizes) bytes.
+ * ------------------------------------------------------------------------------------------ */
+int nmtg_multi_tensor_adam(int n_tensors, const void* const* grads, void* const* params,
+                           void* const* exp_avg, void* const* exp_avg_sq, const int64_t* sizes, float lr,
+                           float beta1, float beta2, float eps, int step, int mode, int bias_correction,
+                           float weight_decay, int dtype, void* stream);
+
+int nmtg_multi_tensor_scale(int n_tensors, const void* const* in, void* const* out, const int64_t* sizes,
+                            float scale, int* noop_flag, int in_dtype, int out_dtype, void* stream);
+
+int64_t nmtg_multi_tensor_l2norm_workspace_bytes(int n_tensors, const int64_t* sizes);
+
+int nmtg_multi_tensor_l2norm(int n_tensors, const void* const* x, const int64_t* sizes, float* norm,
+                             float* per_tensor, void* workspace, int64_t workspace_bytes, int dtype,
+                             void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Per-kernel timing for benchmarks (no counterpart in the reference, whose tests time whole ops
  * with CUDA events, e.g. onmt/modules/test_layer_norm.py:14-31). Between nmtg_trace_begin() and
  * nmtg_trace_end() every kernel the library enqueues is bracketed by two HIP events on its

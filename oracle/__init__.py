@@ -22,5 +22,5 @@ tests/golden/make_fixtures.py from PyTorch's library routines and autograd (not 
 package), against which tests/test_golden_cpu.py checks every function here, including the
 fallback's 16-bit rounding points (round_to=).
 """
-from . import (attention, dropout_add, inputs, layer_norm, mlp, relative_attention, softmax_dropout,  # noqa: F401
+from . import (attention, dropout_add, fused_optim, inputs, layer_norm, mlp, relative_attention, softmax_dropout,  # noqa: F401
                transformer_layers, xentropy)

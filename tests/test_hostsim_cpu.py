@@ -42,6 +42,7 @@ import test_staged_gpu as tst  # noqa: E402
 import test_zz_golden_gpu as tgold  # noqa: E402
 import test_zzb_generator_loss_gpu as tgen  # noqa: E402
 import test_zzc_relative_attention_gpu as trel  # noqa: E402
+import test_zzd_fused_optim_gpu as topt  # noqa: E402
 
 pytestmark = pytest.mark.skipif(not hostsim_build.available(), reason="no host C++ compiler with __bf16 (ROCm clang++)")
 CPU = torch.device("cpu")
@@ -490,6 +491,28 @@ def test_relative_attention_with_learnable_positions(mi355x, dtype, t, b, e, h, 
 @pytest.mark.parametrize("shape,view", [((6, 8, 3, 16), "queries"), ((40, 24), "dense"), ((5, 7), "odd"), ((0, 8), "empty")])
 def test_row_add(mi355x, dtype, shape, view):
     trel.test_row_add_on_dense_and_pitched_rows(CPU, dtype, shape, view)
+
+
+# ----------------------------------------------------------------------------- multi-tensor optimizer passes
+@pytest.mark.parametrize("dtype", [F32, BF16, F16])
+@pytest.mark.parametrize("mode,bias_correction,wd", [(1, 1, 0.01), (0, 1, 0.01), (1, 0, 0.0)])
+def test_multi_tensor_adam(dtype, mode, bias_correction, wd):
+    topt.test_adam_update_of_a_list_of_tensors(CPU, dtype, mode, bias_correction, wd)
+
+
+def test_multi_tensor_scale_and_norm():
+    topt.test_adam_argument_checks(CPU)
+    for src, dst in ((F32, F32), (F16, F32), (F32, BF16), (BF16, BF16)):
+        topt.test_scale_with_overflow_flag(CPU, src, dst)
+    for dtype in (F32, BF16, F16):
+        topt.test_l2norm_of_a_list_of_tensors(CPU, dtype)
+    for max_norm in (0.5, 1e6, 0.0):
+        topt.test_clip_grad_norm_matches_torch(CPU, max_norm)
+
+
+@pytest.mark.parametrize("dtype,adam_w", [(F32, True), (F32, False), (BF16, True)])
+def test_fused_adam_optimizer(dtype, adam_w):
+    topt.test_fused_adam_follows_torch_adamw(CPU, dtype, adam_w)
 
 
 # ----------------------------------------------------------------------------- variants that are switched off by default

@@ -16,7 +16,7 @@ import torch
 from nmtgminor_amd import _lib, _rng
 from nmtgminor_amd.native import (encdec_multihead_attn_bias_blaslt as ed, fast_layer_norm_cuda as ln,
                                   fused_dropout_add_cuda as da, fused_mlp_agelu, fused_mlp_gelu, fused_mlp_relu,
-                                  fused_mlp_silu, linear_blaslt, linear_gemm, mask_softmax_dropout_cuda as sm, mlp_gelu_blaslt,
+                                  fused_mlp_silu, fused_optim, linear_blaslt, linear_gemm, mask_softmax_dropout_cuda as sm, mlp_gelu_blaslt,
                                   relative_position,                                  self_multihead_attn_blaslt as sa, xentropy_cuda as xe)
 
 
@@ -196,3 +196,12 @@ def test_relative_position_column_sums_and_linear_layer(recorder):
     linear_blaslt.backward(r(4, 3, 16), r(24, 16), r(4, 3, 24), True)
     assert {"nmtg_rel_query_bias", "nmtg_rel_shift_add", "nmtg_rel_shift_bwd", "nmtg_add_rows", "nmtg_colsum",
             "nmtg_gemm"} <= set(recorder)
+
+
+def test_multi_tensor_optimizer_passes(recorder):
+    t = lambda n=12: torch.zeros(n)
+    fused_optim.multi_tensor_adam(65536, None, [[t(), t(5)], [t(), t(5)], [t(), t(5)], [t(), t(5)]], 1e-3, 0.9, 0.99, 1e-8, 1, 1, 1, 0.0)
+    fused_optim.multi_tensor_scale(65536, torch.zeros(1, dtype=torch.int32), [[t().to(BF)], [t()]], 0.5)
+    fused_optim.multi_tensor_scale(65536, None, [[t()], [t()]], 0.5)
+    fused_optim.multi_tensor_l2norm(65536, None, [[t(), t(0), t(70000)]], True)
+    assert {"nmtg_multi_tensor_adam", "nmtg_multi_tensor_scale", "nmtg_multi_tensor_l2norm"} <= set(recorder)

@@ -10,7 +10,7 @@ import pytest
 import torch
 import torch.nn.functional as F
 
-from oracle import (attention, dropout_add, generator_loss, inputs, layer_norm, mlp, relative_attention, softmax_dropout,
+from oracle import (attention, dropout_add, fused_optim as ofo, generator_loss, inputs, layer_norm, mlp, relative_attention, softmax_dropout,
                     transformer_layers, xentropy)
 
 D = torch.float64
@@ -466,6 +466,43 @@ def test_learnable_position_attention_matches_the_per_element_definition_and_aut
     for k, gk in (("x", "dx"), ("w_in", "dw_in"), ("w_out", "dw_out"), ("b_in", "db_in"), ("b_out", "db_out")):
         torch.testing.assert_close(gr[gk], leaves[k].grad, rtol=1e-9, atol=1e-10, msg=lambda m, k=k: f"{k}: {m}")
     torch.testing.assert_close(gr["dpos"], pl.grad, rtol=1e-9, atol=1e-10)
+
+
+# ------------------------------------------------------------------ multi-tensor optimizer passes
+@pytest.mark.parametrize("adamw,wd,bias_correction", [(True, 0.01, True), (False, 0.01, True), (True, 0.0, True)])
+def test_adam_step_matches_torch_optimizers(adamw, wd, bias_correction):
+    g = torch.Generator().manual_seed(17)
+    p0 = torch.randn(37, 5, generator=g, dtype=D)
+    ref = p0.clone().requires_grad_()
+    opt = (torch.optim.AdamW if adamw else torch.optim.Adam)([ref], lr=3e-3, betas=(0.9, 0.98), eps=1e-8, weight_decay=wd)
+    p, m, v = p0.clone(), torch.zeros_like(p0), torch.zeros_like(p0)
+    for step in range(1, 5):
+        grad = torch.randn(37, 5, generator=g, dtype=D)
+        ref.grad = grad.clone()
+        opt.step()
+        p, m, v = ofo.adam_step(grad, p, m, v, 3e-3, 0.9, 0.98, 1e-8, step, 1 if adamw else 0, bias_correction, wd, D)
+        # torch applies eps after dividing sqrt(v) by sqrt(c2), the same quantity; AdamW decays p by (1 - lr wd) first,
+        # which equals subtracting lr wd p computed from the old p
+        torch.testing.assert_close(p, ref.detach(), rtol=1e-12, atol=1e-14)
+    # without bias correction the first step divides by 1: update = (1 - beta1) g / (sqrt((1 - beta2) g^2) + eps)
+    gr = torch.tensor([2.0, -3.0], dtype=D)
+    pn, _, _ = ofo.adam_step(gr, torch.zeros(2, dtype=D), torch.zeros(2, dtype=D), torch.zeros(2, dtype=D), 0.1, 0.9, 0.99, 0.0, 1,
+                             1, False, 0.0, D)
+    torch.testing.assert_close(pn, -0.1 * 0.1 * gr / (0.1 * gr.abs()), rtol=1e-12, atol=0)
+
+
+def test_scale_and_l2norm_match_library_routines():
+    g = torch.Generator().manual_seed(18)
+    xs = [torch.randn(n, generator=g, dtype=D) for n in (1, 77, 4096, 0, 300)]
+    total, each = ofo.l2norm(xs, D)
+    torch.testing.assert_close(total, torch.linalg.vector_norm(torch.cat(xs)), rtol=1e-12, atol=0)
+    torch.testing.assert_close(each, torch.stack([torch.linalg.vector_norm(x) for x in xs]), rtol=1e-12, atol=0)
+    y, bad = ofo.scale(xs[1], 0.25, D)
+    assert torch.equal(y, xs[1] * 0.25) and not bad
+    for poison in (float("inf"), float("-inf"), float("nan")):
+        x = xs[1].clone()
+        x[5] = poison
+        assert ofo.scale(x, 0.25, D)[1]
 
 
 def _layer_params_from_torch(layer, heads, decoder):
