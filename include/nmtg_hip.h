@@ -330,7 +330,8 @@ int nmtg_add_rows(void* out, int64_t ld_out, const void* a, int64_t ld_a, const 
 
 /* ------------------------------------------------------------------------------------------
  * Optimizer-side passes over a list of tensors (one launch per 48 tensors instead of one per tensor).
- * Reference: fused_optim.multi_tensor_adam / multi_tensor_scale / multi_tensor_l2norm
+ * Reference: fused_optim.multi_tensor_adam / multi_tensor_scale / multi_tensor_axpby / multi_tensor_l2norm /
+ *   multi_tensor_l2norm_scale
  *   (onmt/modules/extensions/fused_optim/frontend.cpp:45-53; multi_tensor_adam.cu:22-171,
  *   multi_tensor_scale_kernel.cu:29-136, multi_tensor_l2norm_kernel.cu:27-232, :293-367), driven by
  *   FusedAdam.step (onmt/modules/optimized/fused_adam.py:113-191).
@@ -344,9 +345,13 @@ int nmtg_add_rows(void* out, int64_t ld_out, const void* a, int64_t ld_a, const 
  *   p, m, v are updated in place; the four lists share one dtype.
  * nmtg_multi_tensor_scale: out = in * scale (dtypes may differ); *noop_flag (device int, may be NULL)
  *   is set to 1 if any input element is inf or NaN, and left alone otherwise.
+ * nmtg_multi_tensor_axpby: out = a x + b y; y and out share out_dtype; the flag is raised for inf / NaN
+ *   in x (arg_to_check 0), y (1) or either (-1) (multi_tensor_axpby_kernel.cu:27-126).
  * nmtg_multi_tensor_l2norm: norm[0] = sqrt(sum over all tensors of x^2); per_tensor[t] (may be NULL)
  *   = the norm of tensor t; both fp32 on the device; deterministic (fixed-order sums). workspace: fp32
  *   scratch of nmtg_multi_tensor_l2norm_workspace_bytes(n_tensors, sizes) bytes.
+ * nmtg_multi_tensor_l2norm_scale: the same norms of `in` (unscaled) while writing out = in * scale in
+ *   the same pass (multi_tensor_l2norm_scale_kernel.cu:28-125); same workspace.
  * ------------------------------------------------------------------------------------------ */
 int nmtg_multi_tensor_adam(int n_tensors, const void* const* grads, void* const* params,
                            void* const* exp_avg, void* const* exp_avg_sq, const int64_t* sizes, float lr,
@@ -356,11 +361,20 @@ int nmtg_multi_tensor_adam(int n_tensors, const void* const* grads, void* const*
 int nmtg_multi_tensor_scale(int n_tensors, const void* const* in, void* const* out, const int64_t* sizes,
                             float scale, int* noop_flag, int in_dtype, int out_dtype, void* stream);
 
+int nmtg_multi_tensor_axpby(int n_tensors, const void* const* x, const void* const* y, void* const* out,
+                            const int64_t* sizes, float a, float b, int arg_to_check, int* noop_flag,
+                            int x_dtype, int out_dtype, void* stream);
+
 int64_t nmtg_multi_tensor_l2norm_workspace_bytes(int n_tensors, const int64_t* sizes);
 
 int nmtg_multi_tensor_l2norm(int n_tensors, const void* const* x, const int64_t* sizes, float* norm,
                              float* per_tensor, void* workspace, int64_t workspace_bytes, int dtype,
                              void* stream);
+
+int nmtg_multi_tensor_l2norm_scale(int n_tensors, const void* const* in, void* const* out,
+                                   const int64_t* sizes, float scale, float* norm, float* per_tensor,
+                                   void* workspace, int64_t workspace_bytes, int in_dtype, int out_dtype,
+                                   void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Per-kernel timing for benchmarks (no counterpart in the reference, whose tests time whole ops

@@ -1,8 +1,10 @@
 // Optimizer-side elementwise passes over a LIST of tensors in one launch (per 48 tensors), for gfx950.
 //
-// Stand in for fused_optim.multi_tensor_adam / multi_tensor_scale / multi_tensor_l2norm of the reference
+// Stand in for fused_optim.multi_tensor_adam / multi_tensor_scale / multi_tensor_axpby / multi_tensor_l2norm /
+// multi_tensor_l2norm_scale of the reference
 // (onmt/modules/extensions/fused_optim/frontend.cpp:45-53; kernels multi_tensor_adam.cu:22-129,
-// multi_tensor_scale_kernel.cu:29-113, multi_tensor_l2norm_kernel.cu:27-232; launch machinery multi_tensor_apply.cuh).
+// multi_tensor_scale_kernel.cu:29-113, multi_tensor_axpby_kernel.cu:27-126, multi_tensor_l2norm_kernel.cu:27-232,
+// multi_tensor_l2norm_scale_kernel.cu:28-125; launch machinery multi_tensor_apply.cuh).
 // A model has hundreds of parameter tensors, most of them small: one launch per tensor would be launch-bound, so the
 // tensors' addresses and sizes travel in the kernel arguments (a table of up to MT_MAX tensors, 2 KB) and block b finds
 // its tensor and its 65536-element chunk from the table's prefix of block counts. All three passes are bandwidth bound:
@@ -163,8 +165,75 @@ __global__ __launch_bounds__(MT_THREADS) void mt_sumsq_kernel(const MtTable<1> t
   if (threadIdx.x == 0) partial[blockIdx.x] = s;
 }
 
+// out = a x + b y; a block that meets an inf or NaN in the checked operand(s) raises the flag. check: -1 both, 0 x, 1 y.
+template <typename TX, typename TO>
+__global__ __launch_bounds__(MT_THREADS) void mt_axpby_kernel(const MtTable<3> tab, float a, float b, int check,
+                                                              int* __restrict__ noop_flag) {
+  constexpr int EPV = 16 / (sizeof(TX) > sizeof(TO) ? sizeof(TX) : sizeof(TO));
+  int64_t first;
+  int n;
+  const int t = mt_locate(tab, first, n);
+  const TX* x = static_cast<const TX*>(tab.addr[0][t]) + first;
+  const TO* y = static_cast<const TO*>(tab.addr[1][t]) + first;
+  TO* out = static_cast<TO*>(tab.addr[2][t]) + first;
+  const bool vec = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+  const int nvec = vec ? n / EPV : 0;
+  const bool check_x = check != 1, check_y = check != 0;
+  bool ok = true;
+  for (int i = threadIdx.x; i < nvec; i += MT_THREADS) {
+    float xv[EPV], yv[EPV];
+    load_pack<TX, EPV>(x + i * EPV, xv);
+    load_pack<TO, EPV>(y + i * EPV, yv);
+#pragma unroll
+    for (int j = 0; j < EPV; ++j) {
+      ok = ok && (!check_x || is_finite_f(xv[j])) && (!check_y || is_finite_f(yv[j]));
+      xv[j] = a * xv[j] + b * yv[j];
+    }
+    store_pack<TO, EPV>(out + i * EPV, xv);
+  }
+  for (int i = nvec * EPV + threadIdx.x; i < n; i += MT_THREADS) {
+    const float xv = elem<TX>::to_float(x[i]), yv = elem<TO>::to_float(y[i]);
+    ok = ok && (!check_x || is_finite_f(xv)) && (!check_y || is_finite_f(yv));
+    out[i] = elem<TO>::from_float(a * xv + b * yv);
+  }
+  if (!ok && noop_flag) *noop_flag = 1;
+}
+
+// out = in * scale and partial[b] = sum of squares of block b's chunk of the UNSCALED input
+template <typename TI, typename TO>
+__global__ __launch_bounds__(MT_THREADS) void mt_sumsq_scale_kernel(const MtTable<2> tab, float scale, float* __restrict__ partial) {
+  constexpr int EPV = 16 / (sizeof(TI) > sizeof(TO) ? sizeof(TI) : sizeof(TO));
+  __shared__ float red[MT_WAVES];
+  int64_t first;
+  int n;
+  const int t = mt_locate(tab, first, n);
+  const TI* in = static_cast<const TI*>(tab.addr[0][t]) + first;
+  TO* out = static_cast<TO*>(tab.addr[1][t]) + first;
+  const bool vec = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+  const int nvec = vec ? n / EPV : 0;
+  float acc = 0.f;
+  for (int i = threadIdx.x; i < nvec; i += MT_THREADS) {
+    float v[EPV];
+    load_pack<TI, EPV>(in + i * EPV, v);
+#pragma unroll
+    for (int j = 0; j < EPV; ++j) {
+      acc += v[j] * v[j];
+      v[j] *= scale;
+    }
+    store_pack<TO, EPV>(out + i * EPV, v);
+  }
+  for (int i = nvec * EPV + threadIdx.x; i < n; i += MT_THREADS) {
+    const float v = elem<TI>::to_float(in[i]);
+    acc += v * v;
+    out[i] = elem<TO>::from_float(v * scale);
+  }
+  const float s = mt_block_sum(acc, red);
+  if (threadIdx.x == 0) partial[blockIdx.x] = s;
+}
+
 // tensor_sq[t] = sum of the partials of tensor t (block t of the launch); partial points at this launch's first block
-__global__ __launch_bounds__(MT_THREADS) void mt_tensor_sumsq_kernel(const MtTable<1> tab, const float* __restrict__ partial,
+template <int L>
+__global__ __launch_bounds__(MT_THREADS) void mt_tensor_sumsq_kernel(const MtTable<L> tab, const float* __restrict__ partial,
                                                                      float* __restrict__ tensor_sq) {
   __shared__ float red[MT_WAVES];
   const int t = blockIdx.x;
@@ -303,7 +372,7 @@ extern "C" int nmtg_multi_tensor_l2norm(int n_tensors, const void* const* x, con
       NMTG_CHECK_LAUNCH("multi_tensor_l2norm");
     }
     TraceScope trace("multi_tensor_tensor_sumsq", st);
-    hipLaunchKernelGGL(mt_tensor_sumsq_kernel, dim3(tab.count), dim3(MT_THREADS), 0, st, tab, partial + block_base, tensor_sq + t0);
+    hipLaunchKernelGGL((mt_tensor_sumsq_kernel<1>), dim3(tab.count), dim3(MT_THREADS), 0, st, tab, partial + block_base, tensor_sq + t0);
     NMTG_CHECK_LAUNCH("multi_tensor_l2norm");
     return 0;
   });
@@ -311,5 +380,58 @@ extern "C" int nmtg_multi_tensor_l2norm(int n_tensors, const void* const* x, con
   TraceScope trace("multi_tensor_norm_final", st);
   hipLaunchKernelGGL(mt_norm_final_kernel, dim3(1), dim3(MT_THREADS), 0, st, tensor_sq, n_tensors, norm, per_tensor);
   NMTG_CHECK_LAUNCH("multi_tensor_l2norm");
+  return 0;
+}
+
+extern "C" int nmtg_multi_tensor_axpby(int n_tensors, const void* const* x, const void* const* y, void* const* out,
+                                       const int64_t* sizes, float a, float b, int arg_to_check, int* noop_flag, int x_dtype,
+                                       int out_dtype, void* stream) {
+  const void* const* const lists[3] = {x, y, const_cast<const void* const*>(out)};
+  if (int rc = check_list("multi_tensor_axpby", n_tensors, sizes, {lists[0], lists[1], lists[2]})) return rc;
+  NMTG_REQUIRE(arg_to_check >= -1 && arg_to_check <= 1, "multi_tensor_axpby: arg_to_check must be -1 (both), 0 (x) or 1 (y)");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return mt_for_groups<3>(n_tensors, lists, sizes, [&](const MtTable<3>& tab, int blocks, int, int64_t) -> int {
+    if (blocks == 0) return 0;
+    TraceScope trace("multi_tensor_axpby", st);
+    NMTG_DISPATCH_DTYPE(x_dtype, TX,
+                        NMTG_DISPATCH_DTYPE(out_dtype, TO,
+                                            hipLaunchKernelGGL((mt_axpby_kernel<TX, TO>), dim3(blocks), dim3(MT_THREADS), 0, st,
+                                                               tab, a, b, arg_to_check, noop_flag)));
+    NMTG_CHECK_LAUNCH("multi_tensor_axpby");
+    return 0;
+  });
+}
+
+extern "C" int nmtg_multi_tensor_l2norm_scale(int n_tensors, const void* const* in, void* const* out, const int64_t* sizes,
+                                              float scale, float* norm, float* per_tensor, void* workspace, int64_t workspace_bytes,
+                                              int in_dtype, int out_dtype, void* stream) {
+  const void* const* const lists[2] = {in, const_cast<const void* const*>(out)};
+  if (int rc = check_list("multi_tensor_l2norm_scale", n_tensors, sizes, {lists[0], lists[1]})) return rc;
+  NMTG_REQUIRE(norm, "multi_tensor_l2norm_scale: null result pointer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int64_t need = nmtg_multi_tensor_l2norm_workspace_bytes(n_tensors, sizes);
+  NMTG_REQUIRE(n_tensors == 0 || (workspace && workspace_bytes >= need),
+               "multi_tensor_l2norm_scale: workspace of %lld bytes, need %lld", (long long)workspace_bytes, (long long)need);
+  float* tensor_sq = static_cast<float*>(workspace);
+  float* partial = tensor_sq + n_tensors;
+  int rc = mt_for_groups<2>(n_tensors, lists, sizes, [&](const MtTable<2>& tab, int blocks, int t0, int64_t block_base) -> int {
+    if (blocks > 0) {
+      TraceScope trace("multi_tensor_sumsq_scale", st);
+      NMTG_DISPATCH_DTYPE(in_dtype, TI,
+                          NMTG_DISPATCH_DTYPE(out_dtype, TO,
+                                              hipLaunchKernelGGL((mt_sumsq_scale_kernel<TI, TO>), dim3(blocks), dim3(MT_THREADS), 0,
+                                                                 st, tab, scale, partial + block_base)));
+      NMTG_CHECK_LAUNCH("multi_tensor_l2norm_scale");
+    }
+    TraceScope trace("multi_tensor_tensor_sumsq", st);
+    hipLaunchKernelGGL((mt_tensor_sumsq_kernel<2>), dim3(tab.count), dim3(MT_THREADS), 0, st, tab, partial + block_base,
+                       tensor_sq + t0);
+    NMTG_CHECK_LAUNCH("multi_tensor_l2norm_scale");
+    return 0;
+  });
+  if (rc) return rc;
+  TraceScope trace("multi_tensor_norm_final", st);
+  hipLaunchKernelGGL(mt_norm_final_kernel, dim3(1), dim3(MT_THREADS), 0, st, tensor_sq, n_tensors, norm, per_tensor);
+  NMTG_CHECK_LAUNCH("multi_tensor_l2norm_scale");
   return 0;
 }

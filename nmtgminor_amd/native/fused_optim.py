@@ -1,7 +1,7 @@
 """Stand-in for the reference's extension module `fused_optim` (onmt/modules/extensions/fused_optim/frontend.cpp:45-53):
-multi_tensor_adam, multi_tensor_scale, multi_tensor_l2norm with the reference's argument lists
-(chunk_size, noop_flag, tensor_lists, ...). `chunk_size` is accepted and not used: the kernels work in chunks of 65536
-elements. multi_tensor_axpby and multi_tensor_l2norm_scale have no HIP kernel and raise."""
+multi_tensor_adam, multi_tensor_scale, multi_tensor_axpby, multi_tensor_l2norm and multi_tensor_l2norm_scale with the
+reference's argument lists (chunk_size, noop_flag, tensor_lists, ...). `chunk_size` is accepted and not used: the kernels
+work in chunks of 65536 elements."""
 import ctypes
 
 import torch
@@ -79,9 +79,34 @@ def multi_tensor_l2norm(chunk_size, noop_flag, tensor_lists, per_tensor=False):
     return norm, each
 
 
-def multi_tensor_axpby(*args, **kwargs):
-    raise NotImplementedError("fused_optim.multi_tensor_axpby has no HIP kernel")
+def multi_tensor_axpby(chunk_size, noop_flag, tensor_lists, a, b, arg_to_check):
+    """tensor_lists = [x, y, out]: out = a x + b y (y and out of one dtype); noop_flag becomes 1 if the checked operand
+    (arg_to_check 0: x, 1: y, -1: both) holds an inf or NaN."""
+    n = _lists(tensor_lists, 3, "multi_tensor_axpby")
+    if n == 0:
+        return
+    x, y, out = tensor_lists
+    _check(y[0].dtype == out[0].dtype, "multi_tensor_axpby: y and out must share one dtype")
+    _check(noop_flag is None or (noop_flag.dtype == torch.int32 and noop_flag.numel() >= 1), "multi_tensor_axpby: noop_flag must be an int32 tensor")
+    L.require_cuda(noop_flag)
+    L.call("nmtg_multi_tensor_axpby", L.i32(n), _ptr_array(x), _ptr_array(y), _ptr_array(out), _size_array(x), L.f32(a), L.f32(b),
+           L.i32(arg_to_check), L.ptr(noop_flag), L.i32(L.dtype_code(x[0])), L.i32(L.dtype_code(out[0])), L.stream_of(x[0]))
 
 
-def multi_tensor_l2norm_scale(*args, **kwargs):
-    raise NotImplementedError("fused_optim.multi_tensor_l2norm_scale has no HIP kernel")
+def multi_tensor_l2norm_scale(chunk_size, noop_flag, tensor_lists, scale, per_tensor=False):
+    """tensor_lists = [inputs, outputs]: out = in * scale, and -> (norm of all inputs before scaling, fp32 [1]; per-tensor
+    norms, fp32 [n], or an empty tensor), in one pass over the inputs."""
+    n = _lists(tensor_lists, 2, "multi_tensor_l2norm_scale")
+    src, dst = tensor_lists
+    dev = src[0].device if n else (noop_flag.device if noop_flag is not None else torch.device("cuda"))
+    norm = torch.empty(1, dtype=torch.float32, device=dev)
+    each = torch.empty(n if per_tensor else 0, dtype=torch.float32, device=dev)
+    if n == 0:
+        return norm.zero_(), each
+    sizes = _size_array(src)
+    ws_bytes = int(L.load().nmtg_multi_tensor_l2norm_workspace_bytes(L.i32(n), sizes))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    L.call("nmtg_multi_tensor_l2norm_scale", L.i32(n), _ptr_array(src), _ptr_array(dst), sizes, L.f32(scale), L.ptr(norm),
+           L.ptr(each if per_tensor else None), L.ptr(ws), L.i64(ws_bytes), L.i32(L.dtype_code(src[0])), L.i32(L.dtype_code(dst[0])),
+           L.stream_of(src[0]))
+    return norm, each

@@ -1,8 +1,6 @@
 """Stand-in for the reference's extension module `linear_blaslt` (onmt/modules/extensions/mlp_blaslt/linear.cpp:21-56
 forward, :59-104 backward, :142-144 bindings; Python face onmt/modules/optimized/linear.py:25-73): a linear layer
 y = x W^T + b over the last dimension and its three gradients, on nmtg_gemm and nmtg_colsum."""
-import torch
-
 from . import linear_gemm
 
 

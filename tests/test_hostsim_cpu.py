@@ -508,6 +508,9 @@ def test_multi_tensor_scale_and_norm():
         topt.test_l2norm_of_a_list_of_tensors(CPU, dtype)
     for max_norm in (0.5, 1e6, 0.0):
         topt.test_clip_grad_norm_matches_torch(CPU, max_norm)
+    for a, b in ((F32, F32), (F16, F32), (BF16, BF16)):
+        topt.test_axpby_with_overflow_check(CPU, a, b)
+        topt.test_l2norm_with_scaling_in_one_pass(CPU, a, b)
 
 
 @pytest.mark.parametrize("dtype,adam_w", [(F32, True), (F32, False), (BF16, True)])

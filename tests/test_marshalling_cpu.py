@@ -204,4 +204,7 @@ def test_multi_tensor_optimizer_passes(recorder):
     fused_optim.multi_tensor_scale(65536, torch.zeros(1, dtype=torch.int32), [[t().to(BF)], [t()]], 0.5)
     fused_optim.multi_tensor_scale(65536, None, [[t()], [t()]], 0.5)
     fused_optim.multi_tensor_l2norm(65536, None, [[t(), t(0), t(70000)]], True)
-    assert {"nmtg_multi_tensor_adam", "nmtg_multi_tensor_scale", "nmtg_multi_tensor_l2norm"} <= set(recorder)
+    fused_optim.multi_tensor_axpby(65536, torch.zeros(1, dtype=torch.int32), [[t().to(BF)], [t()], [t()]], 1.0, 2.0, -1)
+    fused_optim.multi_tensor_l2norm_scale(65536, None, [[t()], [t().to(BF)]], 0.5, True)
+    assert {"nmtg_multi_tensor_adam", "nmtg_multi_tensor_scale", "nmtg_multi_tensor_l2norm", "nmtg_multi_tensor_axpby",
+            "nmtg_multi_tensor_l2norm_scale"} <= set(recorder)

@@ -1,7 +1,8 @@
 """The multi-tensor optimizer passes (Adam / AdamW update, scale with overflow flag, L2 norm) against the oracle
 (oracle/fused_optim.py) and FusedAdam against torch.optim.AdamW stepping a copy of the same parameters.
 
-What the reference computes here: fused_optim.multi_tensor_adam / multi_tensor_scale / multi_tensor_l2norm
+What the reference computes here: fused_optim.multi_tensor_adam / multi_tensor_scale / multi_tensor_axpby /
+multi_tensor_l2norm / multi_tensor_l2norm_scale
 (onmt/modules/extensions/fused_optim/frontend.cpp:45-53) under FusedAdam.step (onmt/modules/optimized/fused_adam.py:113-191).
 fp32 to 1e-5 relative; 16-bit parameters to the 16-bit tolerance (one rounding of p, m, v per step); the overflow flag and
 which elements change are exact.
@@ -60,8 +61,6 @@ def test_adam_argument_checks(dev):
     with pytest.raises(RuntimeError):
         fused_optim.multi_tensor_adam(0, None, [[t()], [t().half()], [t()], [t()]], 1e-3, 0.9, 0.99, 1e-8, 1, 1, 1, 0.0)
     fused_optim.multi_tensor_adam(0, None, [[], [], [], []], 1e-3, 0.9, 0.99, 1e-8, 1, 1, 1, 0.0)                    # nothing to do
-    with pytest.raises(NotImplementedError):
-        fused_optim.multi_tensor_axpby(0, None, [[t()], [t()], [t()]], 1.0, 1.0, -1)
 
 
 @pytest.mark.parametrize("src,dst", [(torch.float32, torch.float32), (torch.float16, torch.float32), (torch.float32, torch.bfloat16),
@@ -99,6 +98,41 @@ def test_l2norm_of_a_list_of_tensors(dev, dtype):
     assert torch.equal(again, total) and none.numel() == 0                         # deterministic: bit-identical on a second pass
     zero, _ = fused_optim.multi_tensor_l2norm(0, torch.zeros(1, dtype=torch.int32, device=dev), [[]], False)
     assert float(zero.item()) == 0.0
+
+
+@pytest.mark.parametrize("xdt,odt", [(torch.float32, torch.float32), (torch.float16, torch.float32), (torch.bfloat16, torch.bfloat16)])
+def test_axpby_with_overflow_check(dev, xdt, odt):
+    xs, ys = _tensors(SIZES[:12], xdt, 11), _tensors(SIZES[:12], odt, 12)
+    xd, yd = [t.to(dev) for t in xs], [t.to(dev) for t in ys]
+    out = [torch.empty(t.numel(), dtype=odt, device=dev) for t in xs]
+    flag = torch.zeros(1, dtype=torch.int32, device=dev)
+    multi_tensor_applier(fused_optim.multi_tensor_axpby, flag, [xd, yd, out], 0.5, -2.0, -1)
+    assert int(flag.item()) == 0
+    for o, x, y in zip(out, xs, ys):
+        assert_close(o, 0.5 * x.to(D) - 2.0 * y.to(D), odt, "a x + b y", atol=1e-6 if odt == torch.float32 else None)
+    bad_x = [t.clone() for t in xd]
+    bad_x[4][65535] = float("nan")
+    for check, want in ((-1, 1), (0, 1), (1, 0)):                       # the flag follows the operand that is checked
+        flag.zero_()
+        multi_tensor_applier(fused_optim.multi_tensor_axpby, flag, [bad_x, yd, out], 1.0, 1.0, check)
+        assert int(flag.item()) == want, check
+    with pytest.raises(RuntimeError):
+        fused_optim.multi_tensor_axpby(0, flag, [xd, yd, out], 1.0, 1.0, 2)
+
+
+@pytest.mark.parametrize("src,dst", [(torch.float32, torch.float32), (torch.float16, torch.float32), (torch.bfloat16, torch.bfloat16)])
+def test_l2norm_with_scaling_in_one_pass(dev, src, dst):
+    xs = _tensors(SIZES[:12], src, 13)
+    xd = [t.to(dev) for t in xs]
+    out = [torch.empty(t.numel(), dtype=dst, device=dev) for t in xs]
+    total, each = multi_tensor_applier(fused_optim.multi_tensor_l2norm_scale, None, [xd, out], 0.25, True)
+    want_total, want_each = ofo.l2norm(xs, D)                           # the norm of the inputs before scaling
+    assert_close(total[0], want_total, torch.float32, "norm", rtol=2e-6)
+    assert_close(each, want_each, torch.float32, "per-tensor norms", rtol=2e-6)
+    for o, x in zip(out, xs):
+        assert torch.equal(o.cpu(), (x.float() * 0.25).to(dst))
+    same, _ = multi_tensor_applier(fused_optim.multi_tensor_l2norm, None, [xd], False)
+    assert torch.equal(same, total)                                     # the same partial sums as the plain norm pass
 
 
 @pytest.mark.parametrize("dtype,adam_w", [(torch.float32, True), (torch.float32, False), (torch.bfloat16, True)])
