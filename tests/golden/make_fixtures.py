@@ -5,7 +5,7 @@
 
 The expected values come from PyTorch's own CPU library routines and autograd in fp64
 (F.layer_norm, F.softmax, F.cross_entropy(label_smoothing, ignore_index), F.linear, F.gelu, F.relu,
-F.silu, F.gelu(approximate="tanh")) on small seeded inputs — the routines the reference's
+F.silu, F.gelu(approximate="tanh"), torch.optim.Adam / AdamW, clip_grad_norm_) on small seeded inputs — the routines the reference's
 PyTorch fallback itself calls (onmt/modules/layer_norm.py:29-33, onmt/modules/mlp/mlp.py:14-42,
 onmt/modules/optimized/self_attention_func.py:141-287, encdec_attention_func_bias.py:141-351,
 relative_self_attention_func.py:128-345 with the relative shift written as an explicit gather,
@@ -259,7 +259,37 @@ def relative_attention():
          dr_w_bias=u.grad, dr_r_bias=v.grad)
 
 
+def fused_optim():
+    """Four AdamW steps and four Adam (L2) steps of torch.optim on three small fp32 tensors, the joint L2 norm of the last
+    gradients (torch.linalg.vector_norm) and those gradients clipped by torch.nn.utils.clip_grad_norm_."""
+    g = gen(109)
+    shapes = [(5, 7), (33,), (2, 3, 4)]
+    p0 = [torch.randn(s, generator=g, dtype=D) for s in shapes]
+    grads = [[torch.randn(s, generator=g, dtype=D) for s in shapes] for _ in range(4)]
+    kw = dict(lr=1e-2, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.05)
+    out = {}
+    for name, cls in (("adamw", torch.optim.AdamW), ("adam", torch.optim.Adam)):
+        ps = [t.clone().requires_grad_() for t in p0]
+        opt = cls(ps, **kw)
+        for step in grads:
+            for p, gr in zip(ps, step):
+                p.grad = gr.clone()
+            opt.step()
+        for i, p in enumerate(ps):
+            out[f"{name}_p{i}"] = p.detach()
+            out[f"{name}_m{i}"] = opt.state[p]["exp_avg"]
+            out[f"{name}_v{i}"] = opt.state[p]["exp_avg_sq"]
+    holders = [torch.zeros(s, dtype=D).requires_grad_() for s in shapes]
+    for h, gr in zip(holders, grads[-1]):
+        h.grad = gr.clone()
+    norm = torch.nn.utils.clip_grad_norm_(holders, 1.5)
+    save("fused_optim", lr=kw["lr"], beta1=kw["betas"][0], beta2=kw["betas"][1], eps=kw["eps"], weight_decay=kw["weight_decay"],
+         max_norm=1.5, norm=norm, **{f"p{i}": t for i, t in enumerate(p0)},
+         **{f"g{s}_{i}": t for s, step in enumerate(grads) for i, t in enumerate(step)},
+         **{f"clipped{i}": h.grad for i, h in enumerate(holders)}, **out)
+
+
 if __name__ == "__main__":
     torch.set_num_threads(1)
-    for f in (layer_norm, dropout_add, softmax_dropout, xentropy, mlp, self_attention, encdec_attention, relative_attention):
+    for f in (layer_norm, dropout_add, softmax_dropout, xentropy, mlp, self_attention, encdec_attention, relative_attention, fused_optim):
         f()

@@ -9,7 +9,7 @@ import os
 import numpy as np
 import torch
 
-from oracle import attention, dropout_add, layer_norm, mlp, relative_attention, softmax_dropout, xentropy
+from oracle import attention, dropout_add, fused_optim, layer_norm, mlp, relative_attention, softmax_dropout, xentropy
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 D = torch.float64
@@ -119,3 +119,22 @@ def test_relative_attention_fixture():
                                                f["dropout_mask"], D, round_to=BF)
     for k in ("dx", "dw_in", "dw_out", "dw_pos", "db_in", "db_out", "db_pos", "dr_w_bias", "dr_r_bias"):
         close(bwd[k], f[k], k, **F32)
+
+
+def test_fused_optim_fixture():
+    f = load("fused_optim")
+    hp = [float(f[k]) for k in ("lr", "beta1", "beta2", "eps")]
+    wd = float(f["weight_decay"])
+    for name, mode in (("adamw", 1), ("adam", 0)):
+        for i in range(3):
+            p, m, v = f[f"p{i}"], torch.zeros_like(f[f"p{i}"]), torch.zeros_like(f[f"p{i}"])
+            for step in range(4):
+                p, m, v = fused_optim.adam_step(f[f"g{step}_{i}"], p, m, v, *hp, step + 1, mode, True, wd, D)
+            close(p, f[f"{name}_p{i}"], f"{name} p{i}", rtol=1e-12, atol=1e-14)
+            close(m, f[f"{name}_m{i}"], f"{name} m{i}", rtol=1e-12, atol=1e-14)
+            close(v, f[f"{name}_v{i}"], f"{name} v{i}", rtol=1e-12, atol=1e-14)
+    total, _ = fused_optim.l2norm([f[f"g3_{i}"] for i in range(3)], D)
+    close(total, f["norm"], "norm", rtol=1e-12)
+    factor = min(1.0, float(f["max_norm"]) / (float(total) + 1e-6))
+    for i in range(3):
+        close(fused_optim.scale(f[f"g3_{i}"], factor, D)[0], f[f"clipped{i}"], f"clipped gradient {i}", rtol=1e-12)

@@ -570,7 +570,7 @@ def test_three_layer_mlp_backward_with_one_reduction_launch(mi355x):
 
 
 # ----------------------------------------------------------------------------- committed fixtures
-@pytest.mark.parametrize("name", [n for n in dir(tgold) if n.startswith("test_") and n != "test_mlp_fixture"])
+@pytest.mark.parametrize("name", [n for n in dir(tgold) if n.startswith("test_") and n not in ("test_mlp_fixture", "test_fused_optim_fixture")])
 def test_golden_fixtures(mi355x, name):
     getattr(tgold, name)(CPU)
 
@@ -578,6 +578,11 @@ def test_golden_fixtures(mi355x, name):
 @pytest.mark.parametrize("act", ["gelu", "relu", "silu", "agelu"])
 def test_golden_mlp_fixture(mi355x, act):
     tgold.test_mlp_fixture(CPU, act)
+
+
+@pytest.mark.parametrize("name,adam_w", [("adamw", True), ("adam", False)])
+def test_golden_fused_optim_fixture(name, adam_w):
+    tgold.test_fused_optim_fixture(CPU, name, adam_w)
 
 
 # ----------------------------------------------------------------------------- the same checks, bounds-checked

@@ -13,6 +13,8 @@ import pytest
 import torch
 
 from nmtgminor_amd.modules import mlp as mmlp
+from nmtgminor_amd.modules.fused_adam import FusedAdam
+from nmtgminor_amd.modules.fused_clip_norm import fused_clip_grad_norm
 from nmtgminor_amd.modules.encdec_attention_func_bias import encdec_attn_bias_func
 from nmtgminor_amd.modules.relative_self_attention_func import relative_self_attn_func
 from nmtgminor_amd.modules.self_attention_func import self_attn_func
@@ -147,3 +149,27 @@ def test_relative_attention_fixture(dev):
     for k, gk in (("x", "dx"), ("w_in", "dw_in"), ("w_out", "dw_out"), ("w_pos", "dw_pos"), ("b_in", "db_in"),
                   ("b_out", "db_out"), ("b_pos", "db_pos"), ("r_w_bias", "dr_w_bias"), ("r_r_bias", "dr_r_bias")):
         assert_close(t[k].grad, f[gk], BF, gk, scale_atol=True)
+
+
+@pytest.mark.parametrize("name,adam_w", [("adamw", True), ("adam", False)])
+def test_fused_optim_fixture(dev, name, adam_w):
+    f = load("fused_optim")
+    ps = [f[f"p{i}"].to(F32).to(dev).requires_grad_() for i in range(3)]
+    opt = FusedAdam(ps, lr=float(f["lr"]), betas=(float(f["beta1"]), float(f["beta2"])), eps=float(f["eps"]),
+                    weight_decay=float(f["weight_decay"]), adam_w_mode=adam_w)
+    for step in range(4):
+        for i, p in enumerate(ps):
+            p.grad = f[f"g{step}_{i}"].to(F32).to(dev)
+        if step == 3 and adam_w:                                  # the last gradients, clipped on copies
+            holders = [torch.zeros_like(p).requires_grad_() for p in ps]
+            for h, p in zip(holders, ps):
+                h.grad = p.grad.clone()
+            norm = fused_clip_grad_norm(holders, float(f["max_norm"]))
+            assert_close(norm, f["norm"], F32, "norm", rtol=2e-6)
+            for i, h in enumerate(holders):
+                assert_close(h.grad, f[f"clipped{i}"], F32, f"clipped gradient {i}")
+        opt.step()
+    for i, p in enumerate(ps):
+        assert_close(p, f[f"{name}_p{i}"], F32, f"{name} p{i}", rtol=2e-5)
+        assert_close(opt.state[p]["exp_avg"], f[f"{name}_m{i}"], F32, f"{name} m{i}", rtol=2e-5)
+        assert_close(opt.state[p]["exp_avg_sq"], f[f"{name}_v{i}"], F32, f"{name} v{i}", rtol=2e-5)
