@@ -570,7 +570,7 @@ def test_three_layer_mlp_backward_with_one_reduction_launch(mi355x):
 
 
 # ----------------------------------------------------------------------------- committed fixtures
-@pytest.mark.parametrize("name", [n for n in dir(tgold) if n.startswith("test_") and n not in ("test_mlp_fixture", "test_fused_optim_fixture")])
+@pytest.mark.parametrize("name", [n for n in dir(tgold) if n.startswith("test_") and n != "test_mlp_fixture"])
 def test_golden_fixtures(mi355x, name):
     getattr(tgold, name)(CPU)
 
@@ -582,7 +582,11 @@ def test_golden_mlp_fixture(mi355x, act):
 
 @pytest.mark.parametrize("name,adam_w", [("adamw", True), ("adam", False)])
 def test_golden_fused_optim_fixture(name, adam_w):
-    tgold.test_fused_optim_fixture(CPU, name, adam_w)
+    topt.test_fused_optim_golden_fixture(CPU, name, adam_w)
+
+
+def test_golden_relative_attention_fixture(mi355x):
+    trel.test_relative_attention_golden_fixture(CPU)
 
 
 # ----------------------------------------------------------------------------- the same checks, bounds-checked

@@ -6,31 +6,22 @@ bandwidth-bound ops run in fp32 (tolerance 1e-5 relative), the GEMM-based ops in
 relative, 1e-3 absolute; the fixtures carry the fallback's bf16 rounding points).
 Collected last on purpose: every other parity test has run when this file starts.
 """
-import os
-
-import numpy as np
 import pytest
 import torch
 
 from nmtgminor_amd.modules import mlp as mmlp
-from nmtgminor_amd.modules.fused_adam import FusedAdam
-from nmtgminor_amd.modules.fused_clip_norm import fused_clip_grad_norm
 from nmtgminor_amd.modules.encdec_attention_func_bias import encdec_attn_bias_func
-from nmtgminor_amd.modules.relative_self_attention_func import relative_self_attn_func
 from nmtgminor_amd.modules.self_attention_func import self_attn_func
 from nmtgminor_amd.native import (fast_layer_norm_cuda, fused_dropout_add_cuda, fused_mlp_gelu, mask_softmax_dropout_cuda,
                                   self_multihead_attn_blaslt as sa_native, xentropy_cuda)
-from util import assert_close
+from util import assert_close, load_golden
 
 pytestmark = pytest.mark.gpu
-GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 F32 = torch.float32
 BF = torch.bfloat16
 
 
-def load(name):
-    with np.load(os.path.join(GOLDEN, name + ".npz"), allow_pickle=False) as z:
-        return {k: torch.from_numpy(np.array(z[k])) for k in z.files}
+load = load_golden
 
 
 def test_layer_norm_fixture(dev):
@@ -133,43 +124,3 @@ def test_encdec_attention_fixture(dev):
                                      None)
     assert_close(out, f["outputs"], BF, "outputs")
     assert_close(cov, f["softmax_results"], BF, "softmax_results")
-
-
-def test_relative_attention_fixture(dev):
-    f = load("relative_attention")
-    p, h = float(f["p"]), int(f["heads"])
-    names = ("x", "pos", "w_in", "w_out", "w_pos", "b_in", "b_out", "b_pos", "r_w_bias", "r_r_bias")
-    t = {k: f[k].to(BF).to(dev).requires_grad_() for k in names}
-    out, cov = relative_self_attn_func(t["x"], t["pos"], False, True, h, t["w_in"], t["w_out"], t["w_pos"], t["b_in"],
-                                       t["b_out"], t["b_pos"], t["r_w_bias"], t["r_r_bias"], f["pad_mask"].bool().to(dev), p,
-                                       False, None, False, False, True, False, f["dropout_mask"].to(dev))
-    out.backward(f["dout"].to(BF).to(dev))
-    assert_close(out, f["outputs"], BF, "outputs", atol=2e-3)      # scores rounded three times (AC, BD, sum): see the op's test
-    assert_close(cov, f["dropout_results"], BF, "dropout_results")
-    for k, gk in (("x", "dx"), ("w_in", "dw_in"), ("w_out", "dw_out"), ("w_pos", "dw_pos"), ("b_in", "db_in"),
-                  ("b_out", "db_out"), ("b_pos", "db_pos"), ("r_w_bias", "dr_w_bias"), ("r_r_bias", "dr_r_bias")):
-        assert_close(t[k].grad, f[gk], BF, gk, scale_atol=True)
-
-
-@pytest.mark.parametrize("name,adam_w", [("adamw", True), ("adam", False)])
-def test_fused_optim_fixture(dev, name, adam_w):
-    f = load("fused_optim")
-    ps = [f[f"p{i}"].to(F32).to(dev).requires_grad_() for i in range(3)]
-    opt = FusedAdam(ps, lr=float(f["lr"]), betas=(float(f["beta1"]), float(f["beta2"])), eps=float(f["eps"]),
-                    weight_decay=float(f["weight_decay"]), adam_w_mode=adam_w)
-    for step in range(4):
-        for i, p in enumerate(ps):
-            p.grad = f[f"g{step}_{i}"].to(F32).to(dev)
-        if step == 3 and adam_w:                                  # the last gradients, clipped on copies
-            holders = [torch.zeros_like(p).requires_grad_() for p in ps]
-            for h, p in zip(holders, ps):
-                h.grad = p.grad.clone()
-            norm = fused_clip_grad_norm(holders, float(f["max_norm"]))
-            assert_close(norm, f["norm"], F32, "norm", rtol=2e-6)
-            for i, h in enumerate(holders):
-                assert_close(h.grad, f[f"clipped{i}"], F32, f"clipped gradient {i}")
-        opt.step()
-    for i, p in enumerate(ps):
-        assert_close(p, f[f"{name}_p{i}"], F32, f"{name} p{i}", rtol=2e-5)
-        assert_close(opt.state[p]["exp_avg"], f[f"{name}_m{i}"], F32, f"{name} m{i}", rtol=2e-5)
-        assert_close(opt.state[p]["exp_avg_sq"], f[f"{name}_v{i}"], F32, f"{name} v{i}", rtol=2e-5)

@@ -13,7 +13,7 @@ from nmtgminor_amd.modules.relative_self_attention import RelativeSelfMultiheadA
 from nmtgminor_amd.modules.relative_self_attention_func import RelativeShift, relative_self_attn_func
 from nmtgminor_amd.native import linear_blaslt, linear_gemm, relative_position, relative_self_attn_blaslt
 from oracle import inputs, relative_attention as orel
-from util import assert_close
+from util import assert_close, load_golden
 
 pytestmark = pytest.mark.gpu
 D = torch.float64
@@ -278,3 +278,21 @@ def test_module_with_learnable_positions(dev):
     assert_close(out, f["outputs"], torch.bfloat16, "module outputs", atol=2e-3)
     out.float().sum().backward()
     assert m.pos_emb.weight.grad is not None and m.in_proj_weight.grad is not None
+
+
+def test_relative_attention_golden_fixture(dev):
+    # tests/golden/relative_attention.npz: the shift as an explicit gather, fp64 autograd with the bf16 rounding points
+    BF = torch.bfloat16
+    f = load_golden("relative_attention")
+    p, h = float(f["p"]), int(f["heads"])
+    names = ("x", "pos", "w_in", "w_out", "w_pos", "b_in", "b_out", "b_pos", "r_w_bias", "r_r_bias")
+    t = {k: f[k].to(BF).to(dev).requires_grad_() for k in names}
+    out, cov = relative_self_attn_func(t["x"], t["pos"], False, True, h, t["w_in"], t["w_out"], t["w_pos"], t["b_in"],
+                                       t["b_out"], t["b_pos"], t["r_w_bias"], t["r_r_bias"], f["pad_mask"].bool().to(dev), p,
+                                       False, None, False, False, True, False, f["dropout_mask"].to(dev))
+    out.backward(f["dout"].to(BF).to(dev))
+    assert_close(out, f["outputs"], BF, "outputs", atol=2e-3)      # scores rounded three times (AC, BD, sum): see the op's test
+    assert_close(cov, f["dropout_results"], BF, "dropout_results")
+    for k, gk in (("x", "dx"), ("w_in", "dw_in"), ("w_out", "dw_out"), ("w_pos", "dw_pos"), ("b_in", "db_in"),
+                  ("b_out", "db_out"), ("b_pos", "db_pos"), ("r_w_bias", "dr_w_bias"), ("r_r_bias", "dr_r_bias")):
+        assert_close(t[k].grad, f[gk], BF, gk, scale_atol=True)

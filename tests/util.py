@@ -3,6 +3,9 @@
 Tolerances (stated by the benchmark definition): fp32 1e-5 relative; fp16 / bf16 2e-2 relative
 and 1e-3 absolute; integer / index / zero-on-padding results bit-exact.
 """
+import os
+
+import numpy as np
 import torch
 
 TOL = {
@@ -45,3 +48,10 @@ def rel_err(actual, expected):
     a = actual.detach().to("cpu", torch.float64)
     e = expected.detach().to("cpu", torch.float64)
     return float((a - e).norm() / e.norm().clamp_min(1e-30))
+
+
+def load_golden(name):
+    """A committed fixture tests/golden/<name>.npz as a dict of tensors (written by tests/golden/make_fixtures.py)."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", name + ".npz")
+    with np.load(path, allow_pickle=False) as z:
+        return {k: torch.from_numpy(np.array(z[k])) for k in z.files}
