@@ -7,9 +7,9 @@
 // multi_tensor_l2norm_scale_kernel.cu:28-125; launch machinery multi_tensor_apply.cuh).
 // A model has hundreds of parameter tensors, most of them small: one launch per tensor would be launch-bound, so the
 // tensors' addresses and sizes travel in the kernel arguments (a table of up to MT_MAX tensors, 2 KB) and block b finds
-// its tensor and its 65536-element chunk from the table's prefix of block counts. All three passes are bandwidth bound:
+// its tensor and its 32768-element chunk from the table's prefix of block counts. All three passes are bandwidth bound:
 // Adam reads g, p, m, v and writes p, m, v (28 B per fp32 element), scale reads and writes once, the norm reads once.
-// 16-byte accesses whenever a tensor's pointers are 16-byte aligned (chunks start on multiples of 65536 elements), with
+// 16-byte accesses whenever a tensor's pointers are 16-byte aligned (chunks start on multiples of 32768 elements), with
 // four loads in flight per lane in the Adam pass. fp32 arithmetic whatever the storage type. The norm is deterministic:
 // one partial per block, then fixed-order sums.
 #include "common.cuh"
@@ -21,7 +21,7 @@ namespace nmtg {
 namespace {
 
 constexpr int MT_MAX = 48;          // tensors per launch
-constexpr int MT_CHUNK = 65536;     // elements per block
+constexpr int MT_CHUNK = 32768;     // elements per block: a transformer-base parameter list then gives ~7 blocks per CU, all resident at once
 constexpr int MT_THREADS = 256;
 constexpr int MT_WAVES = MT_THREADS / kWave;
 

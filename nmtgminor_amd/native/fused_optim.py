@@ -1,7 +1,7 @@
 """Stand-in for the reference's extension module `fused_optim` (onmt/modules/extensions/fused_optim/frontend.cpp:45-53):
 multi_tensor_adam, multi_tensor_scale, multi_tensor_axpby, multi_tensor_l2norm and multi_tensor_l2norm_scale with the
 reference's argument lists (chunk_size, noop_flag, tensor_lists, ...). `chunk_size` is accepted and not used: the kernels
-work in chunks of 65536 elements."""
+work in chunks of 32768 elements."""
 import ctypes
 
 import torch
