@@ -19,3 +19,9 @@ def backward(input, weight, grad_output, compute_grad_input):
     d_bias = linear_gemm.colsum(g2)
     d_input = linear_gemm.gemm(g2, weight).view(input.shape) if compute_grad_input else None
     return d_input, d_weight, d_bias
+
+
+def backward_input_only(input, weight, grad_output):
+    """-> d_input (the weight is frozen: no weight or bias gradient; linear.cpp:108-140)."""
+    g2 = grad_output.reshape(-1, grad_output.size(-1))
+    return linear_gemm.gemm(g2, weight).view(input.shape)

@@ -463,6 +463,8 @@ def test_relative_position_elementwise_kernels_and_linear_layer(mi355x):
         for dtype in (BF16, F16, F32):
             trel.test_column_sums(CPU, dtype, rows, cols, pitch)
     trel.test_linear_layer_and_its_three_gradients(CPU, BF16)
+    trel.test_linear_module_and_frozen_weight(CPU, True)
+    trel.test_linear_module_and_frozen_weight(CPU, False)
 
 
 @pytest.mark.parametrize("dtype", HALVES)

@@ -9,6 +9,7 @@ it is compared exactly; the attention results to the 16-bit tolerance of the oth
 import pytest
 import torch
 
+from nmtgminor_amd.modules.linear import Linear, linear_function
 from nmtgminor_amd.modules.relative_self_attention import RelativeSelfMultiheadAttn
 from nmtgminor_amd.modules.relative_self_attention_func import RelativeShift, relative_self_attn_func
 from nmtgminor_amd.native import linear_blaslt, linear_gemm, relative_position, relative_self_attn_blaslt
@@ -86,6 +87,33 @@ def test_linear_layer_and_its_three_gradients(dev, dtype):
     assert_close(dw, gy.to(D).reshape(30, 96).t() @ x.to(D).reshape(30, 64), dtype, "linear grad weight", scale_atol=True)
     assert_close(db, gy.to(D).reshape(30, 96).sum(0), dtype, "linear grad bias", scale_atol=True)
     assert linear_blaslt.backward(x.to(dev), w.to(dev), gy.to(dev), False)[0] is None
+
+
+@pytest.mark.parametrize("bias", [True, False])
+def test_linear_module_and_frozen_weight(dev, bias):
+    torch.manual_seed(12)
+    m = Linear(64, 96, bias=bias).to(dev).to(torch.bfloat16)
+    ref = torch.nn.Linear(64, 96, bias=bias).double()
+    ref.weight.data.copy_(m.weight.detach().cpu())
+    if bias:
+        ref.bias.data.copy_(m.bias.detach().cpu())
+    g = torch.Generator().manual_seed(13)
+    x = torch.randn(7, 3, 64, generator=g).to(torch.bfloat16)
+    gy = torch.randn(7, 3, 96, generator=g).to(torch.bfloat16)
+    xd, xr = x.to(dev).requires_grad_(), x.double().requires_grad_()
+    m(xd).backward(gy.to(dev))
+    ref(xr).backward(gy.double())
+    assert_close(m(xd), ref(xr), torch.bfloat16, "linear module forward")
+    assert_close(xd.grad, xr.grad, torch.bfloat16, "grad input")
+    assert_close(m.weight.grad, ref.weight.grad, torch.bfloat16, "grad weight", scale_atol=True)
+    if bias:
+        assert_close(m.bias.grad, ref.bias.grad, torch.bfloat16, "grad bias", scale_atol=True)
+    m.zero_grad()
+    m.weight.requires_grad_(False)                              # frozen weight: only the input gradient is computed
+    x2 = x.to(dev).requires_grad_()
+    linear_function(x2, m.weight, m.bias).backward(gy.to(dev))
+    assert_close(x2.grad, xr.grad, torch.bfloat16, "grad input, frozen weight")
+    assert m.weight.grad is None
 
 
 NAMES = ("x", "pos", "w_in", "w_out", "w_pos", "b_in", "b_out", "b_pos", "r_w_bias", "r_r_bias")
