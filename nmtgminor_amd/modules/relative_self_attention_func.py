@@ -59,6 +59,16 @@ class RelativeSelfAttnFunc(torch.autograd.Function):
         scale = head_dim ** -0.5
         mask_kw = native._mask_kwargs(mask, use_time_mask)
         ctx.heads, ctx.p = heads, dropout_prob if is_training else 0.0
+        ctx.empty = inputs.numel() == 0 and not incremental
+        if ctx.empty:
+            # no positions or no sentences: empty results, and zero gradients for every parameter
+            ctx.shapes = [None if t is None else (t.shape, t.dtype, t.device) for t in
+                          (inputs, pos if learnable_pos else None, input_weights, output_weights, pos_weights, input_biases,
+                           output_biases, pos_biases, r_w_bias, r_r_bias)]
+            outputs = inputs.new_empty(len_q, bsz, embed)
+            coverage = inputs.new_empty(bsz * heads, len_q, len_q)
+            ctx.mark_non_differentiable(coverage)
+            return (outputs, coverage) if return_coverage else outputs
         ctx.use_time_mask, ctx.return_coverage, ctx.learnable_pos = use_time_mask, return_coverage, learnable_pos
 
         if not learnable_pos:
@@ -116,6 +126,9 @@ class RelativeSelfAttnFunc(torch.autograd.Function):
     def backward(ctx, *output_grads):
         heads, p = ctx.heads, ctx.p
         tail = (None,) * 9                                      # mask ... recompute, dropout_mask
+        if ctx.empty:
+            z = [None if s is None else torch.zeros(s[0], dtype=s[1], device=s[2]) for s in ctx.shapes]
+            return (z[0], z[1], None, None, None, z[2], z[3], z[4], z[5], z[6], z[7], z[8], z[9]) + tail
         if not ctx.learnable_pos:
             (inputs, pos, input_weights, output_weights, pos_weights, lin, pos_lin, r_w_bias, r_r_bias, scores, dropped, dmask,
              matmul2_results, mask) = ctx.saved_tensors

@@ -479,6 +479,8 @@ def test_relative_attention_module_and_inference(mi355x):
     trel.test_inference_returns_probabilities_and_single_output_form(CPU)
     trel.test_module_has_the_reference_parameters_and_runs(CPU)
     trel.test_module_with_learnable_positions(CPU)
+    trel.test_empty_batch_gives_empty_results_and_zero_parameter_gradients(CPU, 0, 2)
+    trel.test_empty_batch_gives_empty_results_and_zero_parameter_gradients(CPU, 5, 0)
     trel.test_extension_stand_in_keeps_the_reference_argument_order_and_lists(CPU)
     trel.test_step_by_step_decoding_reproduces_the_causal_rows(CPU)
 

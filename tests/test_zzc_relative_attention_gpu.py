@@ -185,6 +185,20 @@ def test_extension_stand_in_keeps_the_reference_argument_order_and_lists(dev):
         assert_close(got, g[key], dtype, key, scale_atol=key != "dx")
 
 
+@pytest.mark.parametrize("t,b", [(0, 2), (5, 0)])
+def test_empty_batch_gives_empty_results_and_zero_parameter_gradients(dev, t, b):
+    d = inputs.rel_self_attn_inputs(5, 2, 64, 2, torch.bfloat16, p=0.0, seed=3)
+    a = {k: d[k].to(dev).requires_grad_() for k in NAMES}
+    x = d["x"][:t, :b].to(dev).requires_grad_()
+    out, cov = relative_self_attn_func(x, a["pos"], False, True, 2, a["w_in"], a["w_out"], a["w_pos"], a["b_in"], a["b_out"], a["b_pos"],
+                                       a["r_w_bias"], a["r_r_bias"], None, 0.0, False, None, False, False, True, False)
+    assert out.shape == (t, b, 64) and cov.shape == (b * 2, t, t)
+    out.float().sum().backward()
+    assert x.grad.shape == x.shape
+    for k in NAMES[2:]:
+        assert a[k].grad is not None and not a[k].grad.any(), k
+
+
 def test_inference_returns_probabilities_and_single_output_form(dev):
     dtype, h = torch.bfloat16, 4
     d = inputs.rel_self_attn_inputs(32, 2, 128, h, dtype, p=0.3, seed=9)
