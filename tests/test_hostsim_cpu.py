@@ -517,6 +517,16 @@ def test_multi_tensor_scale_and_norm():
         topt.test_l2norm_with_scaling_in_one_pass(CPU, a, b)
 
 
+@pytest.mark.parametrize("seed", [3000, 3001, 3002, pytest.param(3003, marks=long_case), pytest.param(3004, marks=long_case)])
+def test_multi_tensor_random_lists(seed):
+    topt.test_randomly_drawn_tensor_lists(CPU, seed)
+
+
+@pytest.mark.parametrize("seed", range(2000, 2008))
+def test_relative_position_random_shapes(mi355x, seed):
+    trel.test_randomly_drawn_shapes(CPU, seed)
+
+
 @pytest.mark.parametrize("dtype,adam_w", [(F32, True), (F32, False), (BF16, True)])
 def test_fused_adam_optimizer(dtype, adam_w):
     topt.test_fused_adam_follows_torch_adamw(CPU, dtype, adam_w)

@@ -6,6 +6,8 @@ What the reference computes here: RelativeShift and RelativeSelfAttnFunc
 (onmt/modules/optimized/relative_self_attention_func.py:26-76, :79-726). The shift moves values without arithmetic, so
 it is compared exactly; the attention results to the 16-bit tolerance of the other attention tests.
 """
+import random
+
 import pytest
 import torch
 
@@ -338,3 +340,44 @@ def test_relative_attention_golden_fixture(dev):
     for k, gk in (("x", "dx"), ("w_in", "dw_in"), ("w_out", "dw_out"), ("w_pos", "dw_pos"), ("b_in", "db_in"),
                   ("b_out", "db_out"), ("b_pos", "db_pos"), ("r_w_bias", "dr_w_bias"), ("r_r_bias", "dr_r_bias")):
         assert_close(t[k].grad, f[gk], BF, gk, scale_atol=True)
+
+
+@pytest.mark.parametrize("seed", range(2000, 2016))
+def test_randomly_drawn_shapes(dev, seed):
+    # sizes nobody picked by hand: the drawn case is part of the failure message
+    rnd = random.Random(seed)
+    dtype = rnd.choice([torch.bfloat16, torch.float16, torch.float32])
+    g = torch.Generator().manual_seed(seed)
+    b, tq = rnd.choice([1, 2, 5]), rnd.choice([1, 2, 7, 16, 33, 64, 100])
+    tk = rnd.choice([t for t in (1, 3, 8, 16, 31, 64, 100) if t <= max(tq, 1) * 4])
+    r = tk + rnd.choice([0, 0, 1, 5, 8, 29])
+    case = f"seed {seed}: {dtype} batch {b} len_q {tq} len_k {tk} len_r {r}"
+    ac = torch.randint(-8, 9, (b, tq, tk), generator=g).to(dtype)
+    bd = torch.randint(-8, 9, (b, tq, r), generator=g).to(dtype)
+    got = relative_position.shift_add_(ac.clone().to(dev), bd.to(dev))
+    assert torch.equal(got.cpu().to(D), ac.to(D) + orel.relative_shift(bd.to(D))[:, :, :tk]), case
+    back = relative_position.shift_backward(ac.to(dev), r)
+    full = torch.cat([ac.to(D), torch.zeros(b, tq, r - tk, dtype=D)], dim=-1)
+    assert torch.equal(back.cpu().to(D), orel.relative_shift_bwd(full)), case
+    rows, cols, pad = rnd.choice([1, 3, 64, 129, 700]), rnd.choice([1, 8, 24, 100, 513]), rnd.choice([0, 0, 3, 8])
+    x = torch.randn(rows, cols + pad, generator=g).to(dtype)
+    assert_close(linear_gemm.colsum(x.to(dev)[:, :cols]), x[:, :cols].to(D).sum(0), dtype, case + f" colsum {rows}x{cols}+{pad}",
+                 scale_atol=True)
+    y = torch.randint(-8, 9, (rows, cols + pad), generator=g).to(dtype)
+    xi = torch.randint(-8, 9, (rows, cols + pad), generator=g).to(dtype)
+    assert torch.equal(relative_position.add_rows(xi.to(dev)[:, :cols], y.to(dev)[:, :cols]).cpu(), (xi + y)[:, :cols]), case
+    if dtype != torch.float32:
+        h, dh = rnd.choice([1, 2, 4]), rnd.choice([32, 64])
+        t, bsz, p, causal = rnd.choice([1, 2, 9, 33, 70]), rnd.choice([1, 2, 3]), rnd.choice([0.0, 0.1]), rnd.random() < 0.4
+        len_r = t + rnd.choice([0, 0, 3, 17])
+        case += f"; attention T {t} B {bsz} H {h} D {dh} R {len_r} p {p} causal {causal}"
+        d = inputs.rel_self_attn_inputs(t, bsz, h * dh, h, dtype, p=p, seed=seed, len_r=len_r, pos_batch=rnd.choice([1, bsz]),
+                                        causal=causal)
+        leaves, (out, cov) = _run(dev, d, h, True, causal, p)
+        out.backward(d["dout"].to(dev))
+        f = orel.rel_self_attn_fwd(*(d[k] for k in NAMES), h, d["pad_mask"], d["time_mask"], p, d["dropout_mask"], D, round_to=dtype)
+        gr = orel.rel_self_attn_bwd(d["dout"], d["x"], d["pos"], d["w_in"], d["w_out"], d["w_pos"], h, f, p, d["dropout_mask"], D,
+                                    round_to=dtype)
+        assert_close(out, f["outputs"], dtype, case + " outputs", atol=2e-3)
+        for name, key in GRADS:
+            assert_close(leaves[name].grad, gr[key], dtype, case + " grad " + name, scale_atol=True)

@@ -7,6 +7,8 @@ multi_tensor_l2norm / multi_tensor_l2norm_scale
 fp32 to 1e-5 relative; 16-bit parameters to the 16-bit tolerance (one rounding of p, m, v per step); the overflow flag and
 which elements change are exact.
 """
+import random
+
 import pytest
 import torch
 
@@ -214,3 +216,24 @@ def test_fused_optim_golden_fixture(dev, name, adam_w):
         assert_close(p, f[f"{name}_p{i}"], F32, f"{name} p{i}", rtol=2e-5)
         assert_close(opt.state[p]["exp_avg"], f[f"{name}_m{i}"], F32, f"{name} m{i}", rtol=2e-5)
         assert_close(opt.state[p]["exp_avg_sq"], f[f"{name}_v{i}"], F32, f"{name} v{i}", rtol=2e-5)
+
+
+@pytest.mark.parametrize("seed", range(3000, 3008))
+def test_randomly_drawn_tensor_lists(dev, seed):
+    rnd = random.Random(seed)
+    dtype = rnd.choice([torch.float32, torch.bfloat16, torch.float16])
+    sizes = [rnd.choice([0, 1, 3, 8, 100, 4097, 32767, 32768, 32769, 70001]) for _ in range(rnd.choice([1, 2, 47, 48, 49, 97]))]
+    case = f"seed {seed}: {dtype}, {len(sizes)} tensors, {sum(sizes)} elements"
+    g, p = _tensors(sizes, dtype, seed), _tensors(sizes, dtype, seed + 1)
+    m, v = _tensors(sizes, dtype, seed + 2, 0.1), _tensors(sizes, dtype, seed + 3, 0.01, positive=True)
+    gd, pd, md, vd = ([t.to(dev) for t in lst] for lst in (g, p, m, v))
+    mode, step = rnd.choice([0, 1]), rnd.choice([1, 2, 10])
+    fused_optim.multi_tensor_adam(0, None, [gd, pd, md, vd], 1e-2, 0.9, 0.99, 1e-8, step, mode, 1, 0.01)
+    for i in rnd.sample(range(len(sizes)), min(6, len(sizes))):
+        want = ofo.adam_step(g[i], p[i], m[i], v[i], 1e-2, 0.9, 0.99, 1e-8, step, mode, True, 0.01, D)
+        for got, exp, what in zip((pd[i], md[i], vd[i]), want, "pmv"):
+            assert_close(got, exp, dtype, f"{case}: {what} of tensor {i} ({sizes[i]})", atol=1e-6 if dtype == torch.float32 else None)
+    total, each = fused_optim.multi_tensor_l2norm(0, None, [gd], True)
+    want_total, want_each = ofo.l2norm(g, D)
+    assert_close(total[0], want_total, torch.float32, case + ": norm", rtol=2e-6)
+    assert_close(each, want_each, torch.float32, case + ": per-tensor norms", rtol=2e-6)
