@@ -7,22 +7,20 @@ zeros where labels == padding_idx; backward returns the logits gradient. The pad
 runs inside the kernels instead of the wrapper's two masked_fill_ passes."""
 import torch
 
-from ..native import xentropy_cuda
+from ..native import xentropy_cuda as native
 
 
 class SoftmaxCrossEntropyLoss(torch.autograd.Function):
     @staticmethod
     def forward(ctx, logits, labels, smoothing=0.0, padding_idx=-100, half_to_float=False):
-        losses, max_log_sum_exp = xentropy_cuda.forward(logits, labels, smoothing, half_to_float,
-                                                        padding_idx=padding_idx)
-        ctx.save_for_backward(logits, max_log_sum_exp, labels)
-        ctx.smoothing = smoothing
-        ctx.padding_idx = padding_idx
-        return losses
+        ctx.settings = (float(smoothing), int(padding_idx))
+        per_row, lse = native.forward(logits, labels, ctx.settings[0], half_to_float, padding_idx=ctx.settings[1])
+        ctx.save_for_backward(logits, lse, labels)
+        return per_row
 
     @staticmethod
-    def backward(ctx, grad_loss):
-        logits, max_log_sum_exp, labels = ctx.saved_tensors
-        grad_logits = xentropy_cuda.backward(grad_loss.contiguous(), logits, max_log_sum_exp, labels,
-                                             ctx.smoothing, padding_idx=ctx.padding_idx)
-        return grad_logits, None, None, None, None
+    def backward(ctx, upstream):
+        eps, pad = ctx.settings
+        logits, lse, labels = ctx.saved_tensors
+        # rows whose label is the padding index come back as exact zeros from the kernel
+        return native.backward(upstream.contiguous(), logits, lse, labels, eps, padding_idx=pad), None, None, None, None
