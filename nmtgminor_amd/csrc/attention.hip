@@ -56,10 +56,10 @@ int core_fwd(const Core& c, Strided q, Strided k, Strided v, const uint8_t* mask
   g.C = scores; g.ldc = c.tk; g.sC = static_cast<int64_t>(c.tq) * c.tk;
   g.M = c.tq; g.N = c.tk; g.K = c.d; g.batch = c.bh; g.alpha = c.scale;
   g.kmask = mask; g.kmask_kind = mask_kind; g.heads = c.heads;
-  // NMTG_ATTN_FUSED=1: scores, softmax and dropout in one kernel (rows of up to 512 keys). Compiled in but not
-  // yet through the GPU test-suite, hence opt-in; read per call so that a test can switch it.
+  // Scores, softmax and dropout in one kernel where the call qualifies (rows of up to 512 keys, 16-byte aligned
+  // operands); NMTG_ATTN_FUSED=0 always takes the two-kernel path.
   int fused = 0;
-  if (getenv("NMTG_ATTN_FUSED") != nullptr) {
+  if (!switched_off("NMTG_ATTN_FUSED")) {
     GemmArgs f = g;
     f.out2 = dropped;
     f.aux_out = softmax_out;
@@ -110,7 +110,7 @@ int core_bwd(const Core& c, Strided q, Strided k, Strided v, Strided dctx, const
     g.C = ds_buf; g.ldc = c.tk; g.sC = tt;
     g.M = c.tq; g.N = c.tk; g.K = c.d; g.batch = c.bh; g.alpha = 1.f;
     int fused = 0;
-    if (getenv("NMTG_ATTN_FUSED") != nullptr) {   // staged one-kernel form, see core_fwd
+    if (!switched_off("NMTG_ATTN_FUSED")) {   // one-kernel form, see core_fwd
       GemmArgs f = g;
       f.aux_in = scores;
       f.dmask = drop ? dmask : nullptr;

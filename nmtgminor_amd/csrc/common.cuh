@@ -8,6 +8,7 @@
 #include <string>
 #include <cstdio>
 #include <cstdarg>
+#include <cstdlib>
 
 #include "../../include/nmtg_hip.h"
 #include "trace.cuh"
@@ -37,6 +38,13 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 inline bool aligned8(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 7u) == 0; }
 
 int num_cus();  // compute units of the current device (cached per device)
+
+// Diagnostic switches: NAME=0 in the environment selects the plainer of two validated code paths (read on every
+// call, so that one process can run both and compare them).
+inline bool switched_off(const char* name) {
+  const char* e = getenv(name);
+  return e != nullptr && e[0] == '0';
+}
 
 constexpr int kWave = 64;
 

@@ -231,7 +231,21 @@ template <> struct raw_vec<8> { typedef uint4 type; };
 template <> struct raw_vec<4> { typedef uint2 type; };
 template <> struct raw_vec<1> { typedef uint16_t type; };
 
-// Loads elements [0, 8) at p (element e valid iff e < nvalid, nvalid a multiple of VEC or >= 8);
+// Zeroes the 16-bit elements e >= nvalid of an 8-element group (0 <= nvalid < 8).
+__device__ __forceinline__ uint4 keep_first(const uint4& v, int nvalid) {
+  uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int left = nvalid - 2 * i;   // valid elements of word i
+    w[i] = left >= 2 ? w[i] : left == 1 ? (w[i] & 0xffffu) : 0u;
+  }
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// Loads elements [0, 8) at p; element e is valid iff e < nvalid. A vector that holds at least one valid element is
+// read whole: p is VEC-aligned and the operand's pitch a multiple of VEC, so the access stays inside the row's own
+// pitch (and inside the aligned 2 VEC bytes that hold a valid element: same page, hence mapped, even at the end of
+// an allocation). With ZERO the invalid elements come back as zeros, without it they are unspecified.
 // `safe` is any mapped address of the same alignment class.
 template <int VEC, bool ZERO = true>
 __device__ __forceinline__ uint4 load8(const uint16_t* __restrict__ p, const uint16_t* __restrict__ safe, int nvalid) {
@@ -244,17 +258,29 @@ __device__ __forceinline__ uint4 load8(const uint16_t* __restrict__ p, const uin
     if (ZERO && !ok) val = R{};
     u.r[h] = val;
   }
+  if constexpr (ZERO && VEC > 1) {
+    if (nvalid > 0 && nvalid < 8 && nvalid % VEC != 0) u.v = keep_first(u.v, nvalid);
+  }
   return u.v;
 }
 
+// Stores the elements e < nvalid; a partly valid vector goes out element by element.
 template <int VEC>
 __device__ __forceinline__ void store8(uint16_t* __restrict__ p, const uint4& v, int nvalid) {
   typedef typename raw_vec<VEC>::type R;
-  union { uint4 v; R r[8 / VEC]; } u;
+  union { uint4 v; R r[8 / VEC]; uint16_t e[8]; } u;
   u.v = v;
 #pragma unroll
-  for (int h = 0; h < 8 / VEC; ++h)
-    if (h * VEC < nvalid) *reinterpret_cast<R*>(p + h * VEC) = u.r[h];
+  for (int h = 0; h < 8 / VEC; ++h) {
+    const int left = nvalid - h * VEC;
+    if (left >= VEC) {
+      *reinterpret_cast<R*>(p + h * VEC) = u.r[h];
+    } else if (VEC > 1 && left > 0) {
+#pragma unroll
+      for (int e = 0; e < VEC - 1; ++e)
+        if (e < left) p[h * VEC + e] = u.e[h * VEC + e];
+    }
+  }
 }
 
 template <int VEC, bool ZERO = true>
@@ -331,6 +357,7 @@ struct TileStage {
   static constexpr bool DEFER = VEC == 8;
   uint4 regs[NREG];
   uint32_t valid;
+  int kleft;   // valid k of the step being staged (>= 64: all of them)
 
   // base: operand pointer for this batch; rows_total / row0: extent and tile origin in the row
   // index; k0: first k of this step; kend: one past the last valid k.
@@ -338,6 +365,7 @@ struct TileStage {
                                        int kend, int tid) {
     const uint16_t* b16 = reinterpret_cast<const uint16_t*>(base);
     valid = 0;
+    kleft = kend - k0;
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int q = tid + i * NT;
@@ -370,6 +398,16 @@ struct TileStage {
 #pragma unroll
       for (int r = 0; r < NREG; ++r)
         if (!((valid >> r) & 1u)) regs[r] = make_uint4(0, 0, 0, 0);
+      if constexpr (KC) {
+        // last step of a reduction that is not a multiple of 8: the chunk that straddles the end keeps its valid k only
+        if (kleft < GEMM_BK && (kleft & 7) != 0) {
+#pragma unroll
+          for (int i = 0; i < PER; ++i) {
+            const int nv = kleft - ((tid + i * NT) & 7) * 8;
+            if (nv > 0 && nv < 8) regs[i] = keep_first(regs[i], nv);
+          }
+        }
+      }
     }
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
@@ -464,8 +502,10 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, acc16_t (&acc)[
     // bias values of this lane's columns, loaded together ahead of the conversion loop (one
     // uniform branch around all of them: loads inside per-iteration branches wait one by one)
     float bv[TN][4][4];
+    // the bias is not pitched: a tile that holds the ragged end of N (N not a multiple of 4) reads it element by element
+    const bool bias_vec = VEC >= 4 && !((g.N & 3) != 0 && n0 + BN > g.N);
     if (EPI != EPI_ACT_BWD && bias != nullptr) {
-      if constexpr (VEC >= 4) {
+      if (bias_vec) {
         uint2 braw[TN][4];
 #pragma unroll
         for (int j = 0; j < TN; ++j)

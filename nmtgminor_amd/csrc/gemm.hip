@@ -14,7 +14,7 @@ bool gemm_has(int layout, int tile, int epi) {
     return epi == EPI_ACT_BWD && (tile == TILE_L || tile == TILE_M);
   }
   if (layout == LAYOUT_TN) {
-    if (epi == EPI_PLAIN) return tile == TILE_M || tile == TILE_S;
+    if (epi == EPI_PLAIN) return true;
     return epi == EPI_SPLITK && (tile == TILE_L || tile == TILE_M);
   }
   return false;
@@ -79,20 +79,21 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
   if (!a.A || !a.B || !a.C) return fail(NMTG_ERR_INVALID, "gemm: null operand pointer");
   const bool a_kc = layout != LAYOUT_TN;
   const bool b_kc = layout == LAYOUT_NT;
-  // widest access every pointer, pitch and extent of this call allows (8, 4 or 1 elements)
+  // Widest access (8, 4 or 1 elements) that every pointer, pitch and batch stride of this call allows. Extents do not
+  // enter: a ragged M / N / K ends in a predicated last vector (loads stay inside the row's pitch, which is a multiple
+  // of the vector; the K tail is zeroed; the stores of a partial vector and the bias of a ragged last tile go element
+  // by element). Byte masks are addressed as row * N + n, so there N is the pitch and does count.
   int vec = 8;
-  auto narrow = [&](const void* p, int64_t ld, int64_t stride, int batch, int64_t extent) {
-    int v = vec_of(p, ld, stride, batch);
-    while (v > 1 && extent % v != 0) v = v == 8 ? 4 : 1;
-    vec = std::min(vec, v);
+  auto narrow = [&](const void* p, int64_t ld, int64_t stride, int batch) {
+    vec = std::min(vec, vec_of(p, ld, stride, batch));
   };
-  narrow(a.A, a.lda, a.sA, a.batch, a_kc ? a.K : a.M);
-  narrow(a.B, a.ldb, a.sB, a.batch, b_kc ? a.K : a.N);
-  narrow(a.C, a.ldc, a.sC, a.batch, a.N);
-  if (a.aux_out) narrow(a.aux_out, a.ldc, a.sC, a.batch, a.N);
-  if (a.bias) narrow(a.bias, 8, 0, 1, a.N);
-  if (a.aux_in) narrow(a.aux_in, a.ld_aux, 0, 1, a.N);
-  auto narrow_bytes = [&](const uint8_t* p) {   // byte masks addressed as row * N + n
+  narrow(a.A, a.lda, a.sA, a.batch);
+  narrow(a.B, a.ldb, a.sB, a.batch);
+  narrow(a.C, a.ldc, a.sC, a.batch);
+  if (a.aux_out) narrow(a.aux_out, a.ldc, a.sC, a.batch);
+  if (a.bias) narrow(a.bias, 8, 0, 1);
+  if (a.aux_in) narrow(a.aux_in, a.ld_aux, 0, 1);
+  auto narrow_bytes = [&](const uint8_t* p) {
     int v = 8;
     while (v > 1 && (reinterpret_cast<uintptr_t>(p) % v != 0 || a.N % v != 0)) v = v == 8 ? 4 : 1;
     vec = std::min(vec, v);
@@ -119,11 +120,6 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
   // NMTG_GEMM_TILE=0|1|2 (256x256 | 128x128 | 256x64) overrides the tile choice: a tuning aid.
   static const int forced_tile = [] { const char* e = getenv("NMTG_GEMM_TILE"); return e ? atoi(e) : -1; }();
   if (tile < 0 && forced_tile >= 0 && gemm_has(layout, forced_tile, epi) && (forced_tile != TILE_L || vec == 8)) tile = forced_tile;
-  // NMTG_GEMM_ACT_TILE=1 (read per call): the activation epilogues take the 128x128 tile, of which two blocks share a
-  // CU, so that one block's (VALU-bound) epilogue overlaps the other's main loop. Off until measured.
-  if (tile < 0 && (epi == EPI_ACT_FWD || epi == EPI_ACT_BWD) && gemm_has(layout, TILE_M, epi) &&
-      getenv("NMTG_GEMM_ACT_TILE") != nullptr)
-    tile = TILE_M;
   if (tile < 0) {
     const int cus = num_cus();
     const int64_t cnt_l = static_cast<int64_t>(ceil_div(a.M, 256)) * ceil_div(a.N, 256) * a.batch;
@@ -143,14 +139,13 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
   static const bool ring_off = getenv("NMTG_GEMM_NO_RING") != nullptr;
   const int64_t a_bytes = static_cast<int64_t>(a_kc ? a.M : a.K) * a.lda * 2;
   const int64_t b_bytes = static_cast<int64_t>(b_kc ? a.N : a.K) * a.ldb * 2;
-  // The 256x64 tile runs the ring loop only on request (NMTG_GEMM_RING_S=1): that instantiation has not been
-  // through the GPU test-suite yet.
-  const bool ring_s = getenv("NMTG_GEMM_RING_S") != nullptr;   // read per call so that a test can switch it
+  // NMTG_GEMM_RING_S=0 keeps the 256x64 tile (the per-head attention products) on the two-buffer loop.
+  const bool ring_s = !switched_off("NMTG_GEMM_RING_S");
   a.ring = (!ring_off && a.dma && vec == 8 && (tile != TILE_S || ring_s) && a_bytes < (int64_t{1} << 32) &&
             b_bytes < (int64_t{1} << 32)) ? 1 : 0;
-  // gelu through the LDS table: switched on per call by NMTG_GELU_LUT=1 (ring kernels only, they have the LDS room);
-  // off by default until it has been through the GPU test-suite and measured
-  a.act_lut = (a.ring && (epi == EPI_ACT_FWD || epi == EPI_ACT_BWD) && getenv("NMTG_GELU_LUT") != nullptr) ? 1 : 0;
+  // gelu and gelu' of the activation epilogues come from a table in LDS (ring kernels only, they have the LDS room);
+  // NMTG_GELU_LUT=0 evaluates the formula instead.
+  a.act_lut = (a.ring && (epi == EPI_ACT_FWD || epi == EPI_ACT_BWD) && !switched_off("NMTG_GELU_LUT")) ? 1 : 0;
   int bm, bn;
   tile_dims(tile, bm, bn);
   a.m_tiles = ceil_div(a.M, bm);

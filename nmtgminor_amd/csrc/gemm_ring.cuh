@@ -141,7 +141,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_ring_kernel(const
     } else {
       const int k = 4 * ii + (lane >> 4);
       const int c = (lane & 15) ^ (4 * ((lane >> 4) & 3));
-      const int row = min(row0 + 128 * j + 8 * c, rows_total - 8);
+      const int row = min(row0 + 128 * j + 8 * c, (rows_total - 1) & ~7);   // last (possibly partial) aligned group of 8 rows
       return static_cast<uint32_t>(static_cast<int64_t>(k) * ld_b + row * 2);
     }
   };

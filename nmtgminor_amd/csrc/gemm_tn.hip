@@ -4,7 +4,7 @@
 namespace nmtg {
 #define CASE(TILE, EPI) if (tile == TILE && epi == EPI) return gemm_launch_one<T, TILE, false, false, EPI>(a, st);
 template <typename T> static int run(int tile, int epi, const GemmArgs& a, hipStream_t st) {
-  CASE(TILE_M, EPI_PLAIN) CASE(TILE_S, EPI_PLAIN)
+  CASE(TILE_L, EPI_PLAIN) CASE(TILE_M, EPI_PLAIN) CASE(TILE_S, EPI_PLAIN)
   if (epi == EPI_SPLITK) {
     int rc = NMTG_ERR_UNSUPPORTED;
     if (tile == TILE_L) { rc = gemm_launch_one<T, TILE_L, false, false, EPI_SPLITK>(a, st); if (!rc && !a.defer_reduce) rc = splitk_reduce_launch<T, TILE_L>(a, st); return rc; }

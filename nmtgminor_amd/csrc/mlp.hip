@@ -32,7 +32,7 @@ struct BwdPlan {
   size_t splitk_bytes;   // largest weight-gradient split-K workspace
   int layers;
   // one column-sum and one split-K region per layer: with the reductions deferred to one launch at the end
-  // (NMTG_MLP_TAIL) every layer's partials stay alive until then
+  // every layer's partials stay alive until then
   size_t total() const { return 2 * dh_bytes + layers * (colsum_bytes + splitk_bytes); }
 };
 
@@ -150,9 +150,9 @@ extern "C" int nmtg_mlp_bwd(int num_layers, const void* x, const void* const* we
   NMTG_REQUIRE(batch == 0 || (x && grad_out), "mlp_bwd: null pointer argument");
   uint8_t* wsb = static_cast<uint8_t*>(workspace);
   void* dh[2] = {wsb, wsb + plan.dh_bytes};
-  // NMTG_MLP_TAIL=1 (read per call; off until validated on the GPU and measured): the split-K reductions and the final
-  // bias-gradient sums of all layers run as one launch at the end instead of two launches per layer
-  const bool tail_mode = getenv("NMTG_MLP_TAIL") != nullptr;
+  // The split-K reductions and the final bias-gradient sums of all layers run as one launch at the end;
+  // NMTG_MLP_TAIL=0 gives each its own launch (two per layer). Results are bit-identical.
+  const bool tail_mode = !switched_off("NMTG_MLP_TAIL");
   ReduceTail tail;
   auto colsum_region = [&](int layer) {
     return reinterpret_cast<float*>(wsb + 2 * plan.dh_bytes + (tail_mode ? layer : 0) * plan.colsum_bytes);

@@ -83,8 +83,9 @@ def forward(is_training, heads, inputs_q, inputs_kv, input_weights_q, input_weig
     A.check(input_weights_q.shape == (e, e) and input_weights_kv.shape == (2 * e, e) and output_weights.shape == (e, e),
             "weight shapes do not match the inputs")
     c = lambda z: z.contiguous() if z is not None else None
-    # switched on by NMTG_ATTN_PAD_KEYS=1 until it has been through the GPU test-suite and measured
-    if not is_training and tk % KEY_BLOCK != 0 and os.environ.get("NMTG_ATTN_PAD_KEYS") == "1":
+    # inference with a key length that is not a multiple of 64: keys / values padded with masked zero rows, so that every
+    # tensor of the middle section is 16-byte aligned (NMTG_ATTN_PAD_KEYS=0 keeps the exact-length buffers)
+    if not is_training and tk % KEY_BLOCK != 0 and os.environ.get("NMTG_ATTN_PAD_KEYS") != "0":
         return _fwd_padded_keys(heads, c(inputs_q), c(inputs_kv), c(input_weights_q), c(input_weights_kv), c(output_weights),
                                 c(input_biases_q), c(input_biases_kv), c(output_biases), pad_mask, tq, tk, b, e)
     return list(_fwd(is_training, heads, c(inputs_q), c(inputs_kv), c(input_weights_q), c(input_weights_kv),

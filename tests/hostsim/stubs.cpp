@@ -1,12 +1,44 @@
-// Pieces of the library that the CPU build does not take from the kernel sources (per-kernel event tracing is off),
-// and C hooks for the reduction kernels, which the real library only reaches from inside its GEMM-based operators.
+// Pieces of the library that the CPU build does not take from the kernel sources (per-kernel tracing counts launches
+// by name and reports zero time), and C hooks for the reduction kernels, which the real library only reaches from
+// inside its GEMM-based operators.
 #include "reduce.cuh"
+#include <algorithm>
+#include <cstring>
+#include <map>
+#include <string>
+
+namespace {
+bool g_trace = false;
+std::map<std::string, int> g_launches;
+}  // namespace
 
 namespace nmtg {
-bool trace_on() { return false; }
-void trace_open(const char*, hipStream_t, int*) {}
+bool trace_on() { return g_trace; }
+void trace_open(const char* name, hipStream_t, int* slot) {
+  ++g_launches[name];
+  *slot = -1;
+}
 void trace_close(hipStream_t, int) {}
 }  // namespace nmtg
+
+extern "C" int nmtg_trace_begin(void) {
+  g_launches.clear();
+  g_trace = true;
+  return 0;
+}
+
+// same text format as the library's: "name launches total_ms\n" per kernel name; returns the bytes needed
+extern "C" int64_t nmtg_trace_end(char* out, int64_t capacity) {
+  g_trace = false;
+  std::string text;
+  for (const auto& kv : g_launches) text += kv.first + " " + std::to_string(kv.second) + " 0.0\n";
+  if (out != nullptr && capacity > 0) {
+    const size_t n = std::min(text.size(), static_cast<size_t>(capacity - 1));
+    memcpy(out, text.data(), n);
+    out[n] = 0;
+  }
+  return static_cast<int64_t>(text.size()) + 1;
+}
 
 using namespace nmtg;
 

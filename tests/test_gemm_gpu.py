@@ -6,6 +6,7 @@ composite ops built on it (MLP, attention) are checked against the CPU oracle in
 import pytest
 import torch
 
+from nmtgminor_amd import _lib
 from nmtgminor_amd.native.linear_gemm import gemm
 from util import assert_close
 
@@ -87,3 +88,60 @@ def test_gemm_errors(dev):
         gemm(h, h, True, True)                            # A^T B^T not provided
     with pytest.raises(RuntimeError):
         gemm(h, torch.randn(4, 8, device=dev).half())     # inner dims differ
+
+
+def _pitched(rows, cols, dev, dtype, seed, pitch_to=64):
+    """[rows, cols] view of a buffer whose row pitch is cols rounded up to `pitch_to` elements; the pad columns hold
+    NaN so that a kernel that lets them into a sum is caught."""
+    pitch = (cols + pitch_to - 1) // pitch_to * pitch_to
+    buf = torch.full((rows, pitch), float("nan"), dtype=dtype, device=dev)
+    buf[:, :cols] = _mk((rows, cols), dev, dtype, seed)
+    return buf[:, :cols]
+
+
+def _traced(fn):
+    _lib.trace_begin()
+    out = fn()
+    return out, _lib.trace_end()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("v", [250054 % 4096 + 4096, 1030, 70, 6])     # v % 4 == 2: the vocabulary of the loss benchmark is 250 054
+def test_ragged_extents_keep_16_byte_accesses(dev, dtype, v):
+    """Extents that are not a multiple of the access width on 16-byte aligned, pitched operands (the chunk buffers of
+    the projection + cross-entropy module): the three products of that module must run the 16-byte kernels, and the
+    slot-ring loop wherever the reduction is a multiple of 64, with a predicated last vector / tile."""
+    assert v % 4 == 2
+    n, e = 320, 128
+    h = _mk((n, e), dev, dtype, 21)
+    w = _pitched(v, e, dev, dtype, 22)                       # [V, E], E % 64 == 0
+    bias = _mk((v,), dev, dtype, 23)
+    z = torch.full((n, (v + 63) // 64 * 64), float("nan"), dtype=dtype, device=dev)[:, :v]
+    # logits [N, V] = h W^T + b: ragged N
+    _, tr = _traced(lambda: gemm(h, w, trans_b=True, bias=bias, out=z))
+    assert_close(z, _ref(h, w, False, True, 1.0, bias).cpu(), dtype, f"nt ragged n={v}", scale_atol=True)
+    assert all(k.endswith("_ring") for k in tr), tr
+    dz = _pitched(n, v, dev, dtype, 24)
+    # dW [V, E] = dz^T h: ragged M, reduction over the 320 rows
+    dw, tr = _traced(lambda: gemm(dz, h, trans_a=True, split_k=False))
+    assert_close(dw, _ref(dz, h, True, False).cpu(), dtype, f"tn ragged m={v}", scale_atol=True)
+    assert all(k.endswith("_ring") for k in tr), tr
+    # dh [N, E] = dz W: ragged K (the two-buffer loop zeroes the tail of the last 16-byte vector)
+    dh, tr = _traced(lambda: gemm(dz, w))
+    assert_close(dh, _ref(dz, w, False, False).cpu(), dtype, f"nn ragged k={v}", scale_atol=True)
+    assert not any("_v1" in k or "_v4" in k for k in tr), tr
+    # the same with K as the contiguous index of both operands
+    a2, b2 = _pitched(96, v, dev, dtype, 25), _pitched(72, v, dev, dtype, 26)
+    c2, tr = _traced(lambda: gemm(a2, b2, trans_b=True))
+    assert_close(c2, _ref(a2, b2, False, True).cpu(), dtype, f"nt ragged k={v}", scale_atol=True)
+    assert not any("_v1" in k or "_v4" in k for k in tr), tr
+    # pad columns of the output buffer were not written
+    assert torch.isnan(z.as_strided((n, z.stride(0) - v), (z.stride(0), 1), v)).all()
+
+
+def test_transposed_product_without_workspace_runs_unsplit(dev):
+    # a transposed-A product may split K only when it is given a workspace; without one it runs unsplit
+    a, b = _mk((4096, 256), dev, torch.float16, 31), _mk((4096, 128), dev, torch.float16, 32)
+    c, tr = _traced(lambda: gemm(a, b, True, False, split_k=False))
+    assert not any("splitk" in k for k in tr), tr
+    assert_close(c, _ref(a, b, True, False).cpu(), torch.float16, "unsplit", scale_atol=True)

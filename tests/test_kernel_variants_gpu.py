@@ -1,17 +1,16 @@
-"""Kernel variants that are compiled into the library but switched off by default because they have
-not been through the GPU test-suite yet:
+"""Pairs of code paths that compute the same thing: the default one and the plainer one a diagnostic switch
+(NAME=0 in the environment, read by the library on every call) selects instead:
 
-  NMTG_GEMM_RING_S=1   the slot-ring main loop for the 256x64 tile (per-head products P V, dS K, Pd^T dC, dS^T Q)
-  NMTG_ATTN_FUSED=1    Q K^T -> mask -> softmax -> dropout in one kernel (rows of up to 512 keys)
-  NMTG_ATTN_PAD_KEYS=1 inference cross-attention with a key length that is not a multiple of 64: keys / values padded
-                       with masked zero rows so that every tensor of the middle section is 16-byte aligned
-  NMTG_GEMM_ACT_TILE=1 the activation epilogues of the MLP on the 128x128 tile (two blocks per CU) instead of 256x256
-  NMTG_MLP_TAIL=1      the MLP backward's split-K reductions and bias-gradient sums as one launch at its end
-  NMTG_GELU_LUT=1      gelu and its derivative in the MLP epilogues read from a 2049-entry table in LDS
+  NMTG_GEMM_RING_S=0   the 256x64 tile (per-head products P V, dS K, Pd^T dC, dS^T Q) on the two-buffer loop instead of
+                       the slot-ring loop
+  NMTG_ATTN_FUSED=0    Q K^T -> mask, then softmax -> dropout as two kernels instead of one (rows of up to 512 keys)
+  NMTG_ATTN_PAD_KEYS=0 inference cross-attention with a key length that is not a multiple of 64 on exact-length buffers
+                       instead of keys / values padded with masked zero rows (every tensor 16-byte aligned)
+  NMTG_MLP_TAIL=0      the MLP backward's split-K reductions and bias-gradient sums as launches of their own instead of
+                       one launch at its end
+  NMTG_GELU_LUT=0      gelu and its derivative in the MLP epilogues from the formula instead of the 2049-entry LDS table
 
-The library reads both switches on every call, so each test runs the default path and the staged
-path in one process and compares them (and the staged path with the CPU oracle). The tests only run
-when NMTG_TEST_STAGED=1 is set; once they have passed on the GPU the switches can become defaults.
+Each test runs both paths in one process and compares them with each other and the default one with the CPU oracle.
 """
 import os
 
@@ -23,21 +22,25 @@ from nmtgminor_amd.native.linear_gemm import gemm
 from oracle import attention as oat, inputs, mlp as omlp
 from util import assert_close
 
-pytestmark = [pytest.mark.gpu,
-              pytest.mark.skipif(os.environ.get("NMTG_TEST_STAGED") != "1",
-                                 reason="staged kernel variants: set NMTG_TEST_STAGED=1 to validate them")]
+pytestmark = pytest.mark.gpu
 D = torch.float64
 
 
-class switch:
+class off:
+    """NAME=0 inside the block, the previous setting afterwards."""
+
     def __init__(self, name):
         self.name = name
 
     def __enter__(self):
-        os.environ[self.name] = "1"
+        self.before = os.environ.get(self.name)
+        os.environ[self.name] = "0"
 
     def __exit__(self, *exc):
-        os.environ.pop(self.name, None)
+        if self.before is None:
+            os.environ.pop(self.name, None)
+        else:
+            os.environ[self.name] = self.before
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
@@ -47,11 +50,11 @@ def test_ring_256x64_matches_two_buffer_loop(dev, dtype, batch, m, n, k):
     a = torch.randn(batch, m, k, generator=g).to(dtype).to(dev)
     b_kn = torch.randn(batch, k, n, generator=g).to(dtype).to(dev)        # NN: P V, dS K
     a_km = torch.randn(batch, k, m, generator=g).to(dtype).to(dev)        # TN: Pd^T dC, dS^T Q
-    ref_nn = gemm(a, b_kn)
-    ref_tn = gemm(a_km, b_kn, trans_a=True, split_k=False)
-    with switch("NMTG_GEMM_RING_S"):
-        got_nn = gemm(a, b_kn)
-        got_tn = gemm(a_km, b_kn, trans_a=True, split_k=False)
+    with off("NMTG_GEMM_RING_S"):
+        ref_nn = gemm(a, b_kn)
+        ref_tn = gemm(a_km, b_kn, trans_a=True, split_k=False)
+    got_nn = gemm(a, b_kn)
+    got_tn = gemm(a_km, b_kn, trans_a=True, split_k=False)
     # same products in the same order: identical bits
     assert torch.equal(got_nn, ref_nn)
     assert torch.equal(got_tn, ref_tn)
@@ -64,8 +67,8 @@ def _self_fwd(dev, d, h, p, fused):
     dm = g("dropout_mask") if p > 0 else None
     mask = g("time_mask") if d["time_mask"] is not None else g("pad_mask")
     args = (d["time_mask"] is not None, True, h, g("x"), g("w_in"), g("w_out"), g("b_in"), g("b_out"), mask, p)
-    if fused:
-        with switch("NMTG_ATTN_FUSED"):
+    if not fused:
+        with off("NMTG_ATTN_FUSED"):
             return sa_native.forward(*args, dropout_mask=dm)
     return sa_native.forward(*args, dropout_mask=dm)
 
@@ -96,10 +99,10 @@ def test_fused_scores_softmax_rng_mask_is_the_same_stream(dev):
     g = lambda k: d[k].to(dev)
     args = (False, True, h, g("x"), g("w_in"), g("w_out"), g("b_in"), g("b_out"), g("pad_mask"), 0.3)
     torch.cuda.manual_seed(17)
-    r0 = sa_native.forward(*args)
+    with off("NMTG_ATTN_FUSED"):
+        r0 = sa_native.forward(*args)
     torch.cuda.manual_seed(17)
-    with switch("NMTG_ATTN_FUSED"):
-        r1 = sa_native.forward(*args)
+    r1 = sa_native.forward(*args)
     assert torch.equal(r0[3], r1[3])
     assert_close(r1[2].float(), r0[2].float().cpu(), dtype, "dropped (rng)")
 
@@ -112,9 +115,9 @@ def test_fused_softmax_backward_matches_two_kernel_path(dev, dtype, t, b, e, h, 
     lin, scores, dropped, dmask, ctx, out = _self_fwd(dev, d, h, p, fused=False)
     g = lambda k: d[k].to(dev)
     args = (causal, h, g("dout"), ctx, dropped, scores, lin, g("x"), g("w_in"), g("w_out"), dmask, p)
-    ref = sa_native.backward(*args)
-    with switch("NMTG_ATTN_FUSED"):
-        got = sa_native.backward(*args)
+    with off("NMTG_ATTN_FUSED"):
+        ref = sa_native.backward(*args)
+    got = sa_native.backward(*args)
     fwd = oat.self_attn_fwd(d["x"], d["w_in"], d["w_out"], d["b_in"], d["b_out"], h, d["pad_mask"], d["time_mask"], p,
                             d["dropout_mask"] if p > 0 else None, D, round_to=dtype)
     bwd = oat.self_attn_bwd(d["dout"], d["x"], d["w_in"], d["w_out"], h, fwd, p, d["dropout_mask"] if p > 0 else None, D,
@@ -135,11 +138,11 @@ def test_table_gelu_matches_the_formula(dev, dtype, tokens, dm, di, p):
     ins[0].requires_grad_()                                      # asks the backward for dx
     mask = d["mask"].to(dev) if p > 0 else None
     dy = d["dy"].to(dev)
-    ref = fused_mlp_gelu.forward(p, ins, mask)
-    gref = fused_mlp_gelu.backward(p, dy, ref, ins)
-    with switch("NMTG_GELU_LUT"):
-        got = fused_mlp_gelu.forward(p, ins, mask)
-        ggot = fused_mlp_gelu.backward(p, dy, ref, ins)          # same saved tensors: only the derivative differs
+    with off("NMTG_GELU_LUT"):
+        ref = fused_mlp_gelu.forward(p, ins, mask)
+        gref = fused_mlp_gelu.backward(p, dy, ref, ins)
+    got = fused_mlp_gelu.forward(p, ins, mask)
+    ggot = fused_mlp_gelu.backward(p, dy, ref, ins)              # same saved tensors: only the derivative differs
     assert torch.equal(got[2], ref[2])                           # pre-activations do not involve the activation
     pre = ref[2].float()
     assert pre.abs().max() > 6.5 and (pre.abs() < 0.05).any()
@@ -170,9 +173,9 @@ def test_padded_keys_give_the_same_cross_attention(dev, dtype, tq, tk, b, e, h, 
     g = lambda k: d[k].to(dev) if d[k] is not None else None
     pad = g("pad_mask") if masked else None
     args = (False, h, g("x_q"), g("x_kv"), g("w_q"), g("w_kv"), g("w_out"), g("b_q"), g("b_kv"), g("b_out"), pad, 0.0)
-    ref = ed_native.forward(*args)
-    with switch("NMTG_ATTN_PAD_KEYS"):
-        got = ed_native.forward(*args)
+    with off("NMTG_ATTN_PAD_KEYS"):
+        ref = ed_native.forward(*args)
+    got = ed_native.forward(*args)
     names = ("q_lin", "kv_lin", "scores", "dropped", "dropout_mask", "context", "outputs")
     assert got[2].shape == ref[2].shape == (b * h, tq, tk) and not got[2].is_contiguous()      # views of the padded rows
     ulp = 2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7
@@ -200,50 +203,19 @@ def test_padded_keys_give_the_same_cross_attention(dev, dtype, tq, tk, b, e, h, 
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("act", ["gelu", "relu"])
-def test_activation_epilogues_on_the_small_tile(dev, dtype, act):
-    # a shape whose activation GEMMs take the 256x256 tile by default: 16 x 12 tiles of 256 x 256 >= 3/4 of the 256 CUs
-    from nmtgminor_amd.native import fused_mlp_relu
-    tokens, dm, di, p = 4096, 128, 3072, 0.1
-    d = inputs.mlp_inputs(tokens, dm, di, dtype, p=p, seed=97, zero_bias=False)
-    ins = [d[k].to(dev) for k in ("x", "w1", "w2", "b1", "b2")]
-    ins[0].requires_grad_()
-    mask, dy = d["mask"].to(dev), d["dy"].to(dev)
-    if act == "gelu":
-        fwd = lambda: fused_mlp_gelu.forward(p, ins, mask)
-        bwd = lambda out: fused_mlp_gelu.backward(p, dy, out, ins)
-    else:
-        fwd = lambda: fused_mlp_relu.forward(p, True, ins, mask)
-        bwd = lambda out: fused_mlp_relu.backward(p, dy, out, ins)
-    ref = fwd()
-    gref = bwd(ref)
-    with switch("NMTG_GEMM_ACT_TILE"):
-        got = fwd()
-        ggot = bwd(ref)
-    # another blocking of the same products: every element is the same sum in the same order ...
-    for a_, r_ in zip(list(got) + list(ggot[:3]), list(ref) + list(gref[:3])):
-        if a_ is not None and a_.numel():
-            assert torch.equal(a_, r_)
-    # ... except the first layer's bias gradient, whose partial sums are taken per row tile (128 instead of 256 rows)
-    ulp = 2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7
-    for a_, r_ in zip(ggot[3:], gref[3:]):
-        assert_close(a_, r_.float().cpu(), dtype, "bias gradients", rtol=1.05 * ulp, atol=1e-4)
-
-
-@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("tokens,dm,di", [(4096, 128, 256), (1000, 192, 448), (8192, 512, 2048)])
 def test_mlp_backward_with_one_reduction_launch(dev, dtype, tokens, dm, di):
-    # NMTG_MLP_TAIL=1: split-K reductions and bias-gradient sums of all layers in one launch at the end
+    # split-K reductions and bias-gradient sums of all layers in one launch at the end, against launches of their own
     p = 0.1
     d = inputs.mlp_inputs(tokens, dm, di, dtype, p=p, seed=98, zero_bias=False)
     ins = [d[k].to(dev) for k in ("x", "w1", "w2", "b1", "b2")]
     ins[0].requires_grad_()
     mask, dy = d["mask"].to(dev), d["dy"].to(dev)
     out = fused_mlp_gelu.forward(p, ins, mask)
-    want = fused_mlp_gelu.backward(p, dy, out, ins)
-    with switch("NMTG_MLP_TAIL"):
-        got = fused_mlp_gelu.backward(p, dy, out, ins)
-        only_dx = fused_mlp_gelu.backward_input_only(p, dy, out, ins)
+    with off("NMTG_MLP_TAIL"):
+        want = fused_mlp_gelu.backward(p, dy, out, ins)
+    got = fused_mlp_gelu.backward(p, dy, out, ins)
+    only_dx = fused_mlp_gelu.backward_input_only(p, dy, out, ins)
     for a_, r_ in zip(got, want):
         assert torch.equal(a_, r_)                   # the same blocks do the same sums, only launched together
     assert torch.equal(only_dx[0], want[0])
@@ -259,9 +231,9 @@ def test_three_layer_mlp_backward_with_one_reduction_launch(dev):
     dy = torch.randn(tokens, sizes[-1], generator=g).to(dtype).to(dev)
     ins = [x] + ws + bs
     out = fused_mlp_gelu.forward(0.0, ins)
-    want = fused_mlp_gelu.backward(0.0, dy, out, ins)
-    with switch("NMTG_MLP_TAIL"):
-        got = fused_mlp_gelu.backward(0.0, dy, out, ins)
+    with off("NMTG_MLP_TAIL"):
+        want = fused_mlp_gelu.backward(0.0, dy, out, ins)
+    got = fused_mlp_gelu.backward(0.0, dy, out, ins)
     assert len(got) == 7
     for a_, r_ in zip(got, want):
         assert torch.equal(a_, r_)
