@@ -173,6 +173,18 @@ int nmtg_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float a
               int64_t ldc, int64_t stride_c, int64_t batch, const void* bias, void* workspace,
               int64_t workspace_bytes, int dtype, void* stream);
 
+/* nmtg_gemm without a workspace argument, for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc). No counterpart in the reference. The split-K
+ * partial sums go to an array of nmtg_gemm_static_max_workspace_bytes() (32 MiB) that the library keeps in device
+ * memory on every GPU it runs on until the process ends; a shape whose nmtg_gemm_workspace_bytes() exceeds that is
+ * rejected with NMTG_ERR_INVALID. The call itself allocates and frees nothing. All calls on one GPU share the array:
+ * calls that overlap in time on one GPU (different streams) race. Results are bit-identical to nmtg_gemm with a
+ * workspace. */
+int64_t nmtg_gemm_static_max_workspace_bytes(void);
+int nmtg_gemm_static(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alpha, const void* a,
+                     int64_t lda, int64_t stride_a, const void* b, int64_t ldb, int64_t stride_b, void* c,
+                     int64_t ldc, int64_t stride_c, int64_t batch, const void* bias, int dtype, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Fused MLP: y = W_n(... dropout(act(W_1 x + b_1)) ...) + b_n, nn.Linear weight layout [out, in].
  * Reference: fused_mlp_gelu.forward / backward / backward_input_only

@@ -3,6 +3,7 @@
 #include "gemm_inst.cuh"
 #include <algorithm>
 #include <cstdlib>
+#include <mutex>
 
 namespace nmtg {
 
@@ -240,4 +241,54 @@ extern "C" int nmtg_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t
   NMTG_REQUIRE(lda >= (trans_a ? m : k) && ldb >= (trans_b ? k : n) && ldc >= n, "gemm: leading dimension too small");
   return gemm_run(dtype, layout, EPI_PLAIN, g, workspace, static_cast<size_t>(std::max<int64_t>(0, workspace_bytes)),
                   static_cast<hipStream_t>(stream));
+}
+
+// ---------------------------------------------------------------------------------------------
+// nmtg_gemm for callers that cannot allocate: the split-K partials go to a fixed array in device
+// memory that belongs to the library (one copy per GPU, held until the process ends).
+// ---------------------------------------------------------------------------------------------
+namespace {
+constexpr size_t STATIC_SCRATCH_BYTES = size_t{32} << 20;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+// `scratch` names a host-side handle, not a device address: the address on the current device is asked for once per
+// device and kept.
+constexpr int SCRATCH_MAX_DEV = 64;
+void* scratch_ptr[SCRATCH_MAX_DEV] = {nullptr};
+std::mutex scratch_mutex;
+
+int scratch_on_current_device(void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= SCRATCH_MAX_DEV)
+    return nmtg::fail(NMTG_ERR_LAUNCH, "gemm_static: cannot identify the current device: %s", hipGetErrorString(e));
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr)
+      return nmtg::fail(NMTG_ERR_LAUNCH, "gemm_static: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+    scratch_ptr[dev] = p;
+  }
+  *out = scratch_ptr[dev];
+  return 0;
+}
+}  // namespace
+
+extern "C" int64_t nmtg_gemm_static_max_workspace_bytes(void) { return static_cast<int64_t>(STATIC_SCRATCH_BYTES); }
+
+extern "C" int nmtg_gemm_static(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alpha, const void* a, int64_t lda,
+                                int64_t stride_a, const void* b, int64_t ldb, int64_t stride_b, void* c, int64_t ldc,
+                                int64_t stride_c, int64_t batch, const void* bias, int dtype, void* stream) {
+  const int64_t need = nmtg_gemm_workspace_bytes(m, n, k, batch);
+  NMTG_REQUIRE(need <= static_cast<int64_t>(STATIC_SCRATCH_BYTES),
+               "gemm_static: this shape splits K over %lld bytes of partial sums, the built-in scratch holds %lld; use nmtg_gemm "
+               "with a workspace", (long long)need, (long long)STATIC_SCRATCH_BYTES);
+  void* ws = nullptr;
+  if (need > 0) {
+    if (int rc = scratch_on_current_device(&ws)) return rc;
+  }
+  // every split writes its whole partial tile before the reduction reads it: nothing has to be cleared between calls
+  return nmtg_gemm(trans_a, trans_b, m, n, k, alpha, a, lda, stride_a, b, ldb, stride_b, c, ldc, stride_c, batch, bias, ws, need,
+                   dtype, stream);
 }
