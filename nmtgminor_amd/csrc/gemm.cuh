@@ -85,7 +85,8 @@ struct GemmArgs {
 };
 
 #ifdef NMTG_GEMM_PROF
-#define NMTG_PROF_MARK(i) do { if (g.prof != nullptr && threadIdx.x == 0) g.prof[(static_cast<long long>(blockIdx.y) * gridDim.x + blockIdx.x) * 8 + (i)] = clock64(); } while (0)
+// slots 0..4: shader-clock stamps of the phases; slots 5 and 6: constant-rate (100 MHz) stamps of the block's start and end
+#define NMTG_PROF_MARK(i) do { if (g.prof != nullptr && threadIdx.x == 0) { long long* pr_ = g.prof + (static_cast<long long>(blockIdx.y) * gridDim.x + blockIdx.x) * 8; pr_[(i)] = clock64(); if ((i) == 0) pr_[5] = wall_clock64(); if ((i) == 4) pr_[6] = wall_clock64(); } } while (0)
 #else
 #define NMTG_PROF_MARK(i) do { } while (0)
 #endif
