@@ -736,6 +736,7 @@ def measure(w, dev, steps, warmup, do_cpu, trace_steps):
 
 
 RESULT_TAG = "NMTG_BENCH_RESULT "
+OTHER_TAG = "NMTG_BENCH_OTHER "     # full record of a workload other than the headline one (printed before the headline line)
 
 
 def _run_workloads(names, args, dev, emit):
@@ -813,8 +814,9 @@ def main():
     ap.add_argument("--emit-results", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--variants", default="",
                     help="semicolon-separated sets of per-call library switches to time after the default configuration, "
-                         "e.g. 'NMTG_GELU_LUT;NMTG_GELU_LUT+NMTG_GEMM_ACT_TILE'. Each set is exported as NAME=1 for one "
-                         "extra measurement of every selected workload (no CPU baseline); results go to 'variants'.")
+                         "e.g. 'NMTG_GELU_LUT=0;NMTG_GELU_LUT=0+NMTG_MLP_TAIL=0'. Each set is exported (NAME=VALUE, or NAME=1 "
+                         "when no value is given) for one extra measurement of every selected workload (no CPU baseline); "
+                         "results go to 'variants'.")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.stderr.write("bench.py measures one GPU: this build has no multi-GPU path (each op is independent per "
@@ -849,8 +851,9 @@ def main():
         # per-call switches of the library (staged kernel variants): the same workloads again under each requested set
         for spec in [v.strip() for v in args.variants.split(";") if v.strip()]:
             switches = [n.strip() for n in spec.split("+") if n.strip()]
-            saved = {n: os.environ.get(n) for n in switches}
-            os.environ.update({n: "1" for n in switches})
+            settings = dict((n.split("=", 1) + ["1"])[:2] for n in switches)
+            saved = {n: os.environ.get(n) for n in settings}
+            os.environ.update(settings)
             try:
                 for n in names:
                     w = table[n]()
@@ -870,6 +873,17 @@ def main():
                     else:
                         os.environ[n] = v
     head = results[0]
+    # The other workloads go out first, one line each, and the headline line carries only their summary: a reader of
+    # the tail of this output (the last few KB) then sees every workload's figures.
+    for r in results[1:]:
+        print(OTHER_TAG + json.dumps(r), flush=True)
+
+    def brief(r):
+        if "error" in r:
+            return dict(workload=r["workload"], error=r["error"])
+        roof = r.get("roofline") or {}
+        return dict(workload=r["workload"], value=r["value"], unit=r["unit"], ms_per_step=r["ms_per_step"],
+                    kernel=roof.get("kernel"), frac=roof.get("frac"), traffic=roof.get("traffic"))
     line = {
         "metric": "MFMA TFLOP/s (fused MLP fwd+bwd)" if head["workload"] == "mlp" else head["metric"] + f" ({head['workload']})",
         "value": head["value"], "unit": head["unit"], "n_gpus": 1, "steps": head["steps"], "warmup": args.warmup,
@@ -878,7 +892,7 @@ def main():
         "config": {"workload": head["description"], "timed": head["timed"],
                    "switches": {k: v for k, v in sorted(os.environ.items()) if k.startswith("NMTG_")}},
         "roofline": head["roofline"], "cpu_baseline": head["cpu_baseline"], "kernels": head["kernels"],
-        "others": results[1:],
+        "others": [brief(r) for r in results[1:]],
     }
     if variants:
         line["variants"] = variants

@@ -275,7 +275,14 @@ __device__ __forceinline__ void store8(uint16_t* __restrict__ p, const uint4& v,
   for (int h = 0; h < 8 / VEC; ++h) {
     const int left = nvalid - h * VEC;
     if (left >= VEC) {
-      *reinterpret_cast<R*>(p + h * VEC) = u.r[h];
+      // Non-temporal: the output is read next by another kernel (through another XCD's L2 at the earliest), so it
+      // should stream out to memory while the kernel runs instead of waiting in L2 for the write-back at its end.
+      if constexpr (VEC == 8) {
+        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+        __builtin_nontemporal_store(__builtin_bit_cast(u32x4, u.r[h]), reinterpret_cast<u32x4*>(p + h * VEC));
+      } else {
+        *reinterpret_cast<R*>(p + h * VEC) = u.r[h];
+      }
     } else if (VEC > 1 && left > 0) {
 #pragma unroll
       for (int e = 0; e < VEC - 1; ++e)

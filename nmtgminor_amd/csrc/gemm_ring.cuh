@@ -228,13 +228,16 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_ring_kernel(const
     if (pb >= RING) pb -= RING;
     const uint8_t* sa = lds_raw + pa * RING_SLOT_BYTES;
     const uint8_t* sb = lds_raw + pb * RING_SLOT_BYTES;
-#pragma unroll
-    for (int kk = 0; kk < GEMM_BK / 16; ++kk) {
-      uint4 fm[TM], fn[TN];
+    // Fragments are double-buffered in registers: the LDS reads of k-group kk + 1 are issued ahead of the MFMAs of
+    // k-group kk, so the matrix pipe does not wait for the LDS latency (with the 128x128 tile there is one wavefront
+    // per SIMD and nothing else to hide it).
+    uint4 fm[2][TM], fn[2][TN];
+    auto load_frags = [&](auto kk_tag, uint4 (&fm_)[TM], uint4 (&fn_)[TN]) {
+      constexpr int kk = decltype(kk_tag)::value;
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
         if constexpr (A_KC) {
-          fm[i] = *reinterpret_cast<const uint4*>(sa + fa[i][kk]);
+          fm_[i] = *reinterpret_cast<const uint4*>(sa + fa[i][kk]);
         } else {
           const uint8_t* p = sa + fa[i][0] + kk * 16 * 256;
           const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(p));
@@ -242,13 +245,13 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_ring_kernel(const
           union { short4_t s[2]; uint4 u; } cv;
           cv.s[0] = lo;
           cv.s[1] = hi;
-          fm[i] = cv.u;
+          fm_[i] = cv.u;
         }
       }
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
         if constexpr (B_KC) {
-          fn[j] = *reinterpret_cast<const uint4*>(sb + fb[j][kk]);
+          fn_[j] = *reinterpret_cast<const uint4*>(sb + fb[j][kk]);
         } else {
           const uint8_t* p = sb + fb[j][0] + kk * 16 * 256;
           const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(p));
@@ -256,14 +259,38 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_ring_kernel(const
           union { short4_t s[2]; uint4 u; } cv;
           cv.s[0] = lo;
           cv.s[1] = hi;
-          fn[j] = cv.u;
+          fn_[j] = cv.u;
         }
       }
+    };
+    load_frags(std::integral_constant<int, 0>{}, fm[0], fn[0]);
+    static_for<0, GEMM_BK / 16>([&](auto kk_tag) {
+      constexpr int kk = decltype(kk_tag)::value;
+      if constexpr (kk + 1 < GEMM_BK / 16) load_frags(std::integral_constant<int, kk + 1>{}, fm[(kk + 1) & 1], fn[(kk + 1) & 1]);
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j) mfma<T>::run(fn[j], fm[i], acc[i][j]);
-    }
+        for (int j = 0; j < TN; ++j) mfma<T>::run(fn[kk & 1][j], fm[kk & 1][i], acc[i][j]);
+    });
+    // Pin that order (the scheduler otherwise sinks the reads back down to save registers): the first k-group's reads,
+    // then for every k-group its MFMAs with the next group's reads dealt out one per MFMA from the start.
+    constexpr int READS = (A_KC ? TM : 2 * TM) + (B_KC ? TN : 2 * TN);   // LDS read instructions per k-group
+    constexpr int MFMAS = TM * TN;
+    __builtin_amdgcn_sched_group_barrier(0x100, READS, 0);
+    static_for<0, GEMM_BK / 16>([&](auto kk_tag) {
+      constexpr int kk = decltype(kk_tag)::value;
+      if constexpr (kk + 1 < GEMM_BK / 16) {
+        constexpr int PAIRS = READS < MFMAS ? READS : MFMAS;
+        static_for<0, PAIRS>([&](auto) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        });
+        if constexpr (READS > PAIRS) __builtin_amdgcn_sched_group_barrier(0x100, READS - PAIRS, 0);
+        if constexpr (MFMAS > PAIRS) __builtin_amdgcn_sched_group_barrier(0x008, MFMAS - PAIRS, 0);
+      } else {
+        __builtin_amdgcn_sched_group_barrier(0x008, MFMAS, 0);
+      }
+    });
     pos_r += SPS;
     if (pos_r >= RING) pos_r -= RING;
 

@@ -8,9 +8,10 @@ re-indexed along dimension 1):
     cross-attention    cache['c_k'], cache['c_v']  keys / values of the encoder states (computed at the first step)
 Inference only (no autograd graph, no dropout). The projections are GEMM calls of the library, the attention core is
 the compact cross-attention entry point (queries and a [Tk, B*H, 2, D] key/value block come in, the context goes
-out); the cache bookkeeping (slices, concatenation, the interleave of keys and values) is tensor movement on the
-device, exactly the reference's. A later step may carry one new position only: with more than one, the new
-positions would need a causal mask among themselves, which the cross-attention core does not take.
+out), which takes a key mask [B, Tk]: the mask of a one-position step (a time-mask row or a key-padding mask) is
+handed over in that form. The cache bookkeeping (slices, concatenation, the interleave of keys and values) is tensor
+movement on the device, exactly the reference's. A later step may carry one new position only: with more than one,
+the new positions would need a causal mask among themselves, which the cross-attention core does not take.
 """
 import torch
 
@@ -32,10 +33,33 @@ def _core(heads, q_lin, keys, values, pad_mask):
     return context, probs
 
 
+def _key_mask(mask, use_time_mask, b, tk, device):
+    """The mask of a one-position step as a key mask [B, Tk] (True = masked), or None. The reference fills the scores
+    [B*H, 1, Tk] with -inf where the mask is set (self_attention_func.py:203-215): a time mask is 2-D and broadcasts
+    over the batch (its one row, or the last row of a [T, Tk] mask, is the new position's), a key-padding mask is
+    [B, Tk]."""
+    if mask is None:
+        return None
+    mask = mask.to(device=device, dtype=torch.bool)
+    if use_time_mask:
+        if mask.dim() == 1:
+            mask = mask.unsqueeze(0)
+        if mask.dim() != 2 or mask.size(-1) != tk:
+            raise RuntimeError(f"incremental self-attention: time mask of shape {tuple(mask.shape)} does not cover {tk} keys")
+        return mask[-1:].expand(b, tk).contiguous()
+    if mask.dim() == 3:
+        mask = mask.squeeze(1)
+    if mask.shape != (b, tk):
+        raise RuntimeError(f"incremental self-attention: key-padding mask of shape {tuple(mask.shape)}, expected {(b, tk)}")
+    return mask.contiguous()
+
+
 @torch.no_grad()
-def self_attn_step(heads, inputs, input_weights, output_weights, input_biases, output_biases, mask, cache):
-    """inputs [T_new, B, E]: all positions at the first call (no 'k' in the cache; `mask` is then the usual time mask
-    [T, T]), one new position afterwards. -> (outputs [T_new, B, E], probabilities [B*H, T_new, T_total])."""
+def self_attn_step(heads, inputs, input_weights, output_weights, input_biases, output_biases, mask, cache,
+                   use_time_mask=True):
+    """inputs [T_new, B, E]: all positions at the first call (no 'k' in the cache), one new position afterwards.
+    mask: a time mask (use_time_mask: [T_new, T_total], True = masked) or a key-padding mask [B, T_total]; both are
+    applied as the reference applies them. -> (outputs [T_new, B, E], probabilities [B*H, T_new, T_total])."""
     t_new, b, e = inputs.shape
     d = e // heads
     lin = _project(inputs, input_weights, input_biases).view(t_new, b * heads, 3, d)
@@ -50,13 +74,14 @@ def self_attn_step(heads, inputs, input_weights, output_weights, input_biases, o
         values = torch.cat([cache["v"], values], dim=0)
     cache["k"], cache["v"] = keys, values
     if first and t_new > 1:
-        # a prefix of several positions: the full-sequence kernel with its time mask, fed with the same projection
+        # a prefix of several positions: the full-sequence kernel with its mask, fed with the same projection
         from ..native import self_multihead_attn_blaslt as sa_native
-        if mask is None:
-            mask = torch.triu(torch.ones(t_new, t_new, dtype=torch.bool, device=inputs.device), 1)
-        _, probs, _, context = sa_native.forward_compact(True, False, heads, lin.view(t_new, b, 3 * e), mask.to(torch.bool), 0.0)
+        if mask is not None:
+            mask = mask.to(torch.bool)
+        _, probs, _, context = sa_native.forward_compact(use_time_mask and mask is not None, False, heads,
+                                                         lin.view(t_new, b, 3 * e), mask, 0.0)
     else:
-        context, probs = _core(heads, queries, keys, values, None)
+        context, probs = _core(heads, queries, keys, values, _key_mask(mask, use_time_mask, b, keys.shape[0], inputs.device))
     return _project(context, output_weights, output_biases), probs
 
 

@@ -81,7 +81,7 @@ def self_attn_func(*args):
                 raise NotImplementedError("self_attn_func: rotary position encoding has no HIP kernel")
             if cache is None:
                 raise RuntimeError("self_attn_func: incremental decoding needs an incremental_cache dict")
-            return self_attn_step(heads, inputs, w_in, w_out, b_in, b_out, mask if use_time_mask else None, cache)
+            return self_attn_step(heads, inputs, w_in, w_out, b_in, b_out, mask, cache, bool(use_time_mask))
         return SelfAttnFunc.apply(*args)
 
 

@@ -95,6 +95,7 @@ static inline float rsqrtf(float v) { return 1.0f / std::sqrt(v); }
 static inline float __builtin_amdgcn_exp2f(float v) { return std::exp2(v); }
 static inline float __builtin_amdgcn_rcpf(float v) { return 1.0f / v; }
 static inline void __builtin_amdgcn_sched_barrier(int) {}
+static inline void __builtin_amdgcn_sched_group_barrier(int, int, int) {}
 static inline float __builtin_amdgcn_fmed3f(float a, float b, float c) { return std::fmax(std::fmin(a, b), std::fmin(std::fmax(a, b), c)); }
 static inline float __builtin_amdgcn_fractf(float v) { return v - std::floor(v); }
 

@@ -432,6 +432,7 @@ def test_cross_entropy_on_row_pitched_logits(mi355x, dtype, v, pitch, gpitch):
 @pytest.mark.parametrize("dtype", HALVES)
 def test_incremental_decoding(mi355x, dtype):
     tinc.test_self_attention_step_by_step(CPU, dtype, 3)
+    tinc.test_self_attention_steps_honour_a_key_padding_mask(CPU, dtype)
     tinc.test_cross_attention_with_cached_encoder_states(CPU, dtype)
 
 

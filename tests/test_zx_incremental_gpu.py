@@ -1,8 +1,10 @@
-"""Incremental decoding (one position per step, keys / values cached) against the full-sequence operators.
+"""Incremental decoding (one position per step, keys / values cached) against the CPU oracle's full-sequence rows.
 
-Decoding position by position with the cache must reproduce, row by row, what the same module computes for the whole
+Decoding position by position with the cache must reproduce, row by row, what the attention computes for the whole
 sequence under a causal mask: the property the reference's translator relies on
-(onmt/modules/optimized/self_attention_func.py:162-174, encdec_attention_func_bias.py:181-213). The cache entries
+(onmt/modules/optimized/self_attention_func.py:162-174, encdec_attention_func_bias.py:181-213). Every decoded row is
+compared with the oracle (fp64 on the rounded operands) at the 16-bit tolerance, and, as a secondary check, with the
+library's own full-sequence result. The cache entries
 ('k', 'v', 'c_k', 'c_v': time-first [T, B, E]) can be re-indexed along the batch dimension between steps, as beam
 search does.
 """
@@ -14,8 +16,10 @@ import torch
 from nmtgminor_amd.modules.encdec_attention import EncdecMultiheadAttn
 from nmtgminor_amd.modules.self_attention import SelfMultiheadAttn
 from nmtgminor_amd.modules.transformer_layers import DecoderLayer
-from oracle import inputs
+from oracle import attention as oat, inputs, transformer_layers as otl
 from util import assert_close
+
+D = torch.float64
 
 pytestmark = pytest.mark.gpu
 
@@ -29,8 +33,13 @@ def _randomise(module, seed):
 
 
 def close(a, b, dtype, what):
-    # the same products, accumulated by different kernels (a [1, T] row instead of a [T, T] tile)
+    # secondary check, library against library: the same products, accumulated by different kernels (a [1, T] row
+    # instead of a [T, T] tile), each rounded to 16 bits on its own
     assert_close(a, b.float().cpu(), dtype, what, rtol=2e-2, atol=4e-3 if dtype == torch.float16 else 3e-2)
+
+
+def _cpu(module, *names):
+    return [getattr(module, n).detach().cpu() for n in names]
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
@@ -54,11 +63,39 @@ def test_self_attention_step_by_step(dev, dtype, prefix):
             assert cache["k"].shape == (i + 1, b, e) and cache["v"].shape == (i + 1, b, e)
             assert cov.shape == (b * h, 1, i + 1)
             assert_close(cov.float().sum(-1), torch.ones(b * h, 1), dtype, "probabilities sum to one", atol=2e-2)
+    w_in, w_out, b_in, b_out = _cpu(attn, "in_proj_weight", "out_proj_weight", "in_proj_bias", "out_proj_bias")
+    want = oat.self_attn_fwd(x.cpu(), w_in, w_out, b_in, b_out, h, None, causal.cpu(), 0.0, None, D, round_to=dtype)
+    assert_close(torch.cat(rows), want["outputs"], dtype, "stepwise self-attention vs oracle")
+    assert_close(cov, want["dropout_results"][:, t - 1:t], dtype, "last step's probabilities vs oracle")
     close(torch.cat(rows), full, dtype, "stepwise self-attention")
     with pytest.raises(NotImplementedError):
         attn(x[:2], None, None, None, incremental=True, incremental_cache=cache)       # two positions onto a filled cache
     with pytest.raises(RuntimeError):
         attn(x[:1], None, None, None, incremental=True, incremental_cache=None)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_self_attention_steps_honour_a_key_padding_mask(dev, dtype):
+    # a batch whose prefixes start with padding: the padded keys must stay out of every step's softmax
+    # (reference: masked_fill_ of the scores for either mask kind, self_attention_func.py:203-215)
+    t, b, e, h = 9, 3, 128, 4
+    attn = _randomise(SelfMultiheadAttn(e, h, 0.1), 97).to(dev).to(dtype).eval()
+    x = torch.randn(t, b, e, generator=torch.Generator().manual_seed(98)).to(dtype).to(dev)
+    pads = torch.tensor([0, 2, 4])                                   # leading pad positions per batch entry
+    pad_mask = (torch.arange(t)[None, :] < pads[:, None])           # [B, T], True = pad
+    w_in, w_out, b_in, b_out = _cpu(attn, "in_proj_weight", "out_proj_weight", "in_proj_bias", "out_proj_bias")
+    cache = {}
+    with torch.no_grad():
+        for i in range(4, t):                                        # first call: a prefix of 5 positions, then one by one
+            lo = 0 if i == 4 else i
+            out, cov = attn(x[lo:i + 1], None, pad_mask[:, :i + 1].to(dev), None, incremental=True, incremental_cache=cache)
+            want = oat.self_attn_fwd(x[:i + 1].cpu(), w_in, w_out, b_in, b_out, h, pad_mask[:, :i + 1], None, 0.0, None, D,
+                                     round_to=dtype)
+            assert_close(out, want["outputs"][lo:], dtype, f"step {i}: outputs vs oracle")
+            assert_close(cov, want["dropout_results"][:, lo:], dtype, f"step {i}: probabilities vs oracle")
+            # exact zeros on the padded keys
+            for bi in range(b):
+                assert (cov[bi * h:(bi + 1) * h, :, :pads[bi]] == 0).all()
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
@@ -81,6 +118,10 @@ def test_cross_attention_with_cached_encoder_states(dev, dtype):
             rows.append(out)
             close(cov, full_cov[:, i:i + 1], dtype, "stepwise coverage")
         assert cache["c_k"].shape == (tk, b, e) and cache["c_v"].shape == (tk, b, e)
+    w_q, w_kv, w_out = _cpu(attn, "in_proj_weight_q", "in_proj_weight_kv", "out_proj_weight")
+    want = oat.encdec_attn_fwd(q.cpu(), ctxt.cpu(), w_q, w_kv, w_out, None, None, None, h, pad.cpu(), 0.0, None, D,
+                               round_to=dtype)
+    assert_close(torch.cat(rows), want["outputs"], dtype, "stepwise cross-attention vs oracle")
     close(torch.cat(rows), full, dtype, "stepwise cross-attention")
 
 
@@ -114,5 +155,16 @@ def test_decoder_layer_step_by_step_with_beam_reordering(dev):
             out, _, cache = layer(cur_x, cur_ctxt, causal[i:i + 1, :i + 1], cur_pad, incremental=True, incremental_cache=cache)
             rows.append(out)
         assert sorted(cache) == ["c_k", "c_v", "k", "v"]
+    # against the layer oracle (fp64, the weights the kernels saw): a whole layer rounds to 16 bits at every operator
+    # boundary and the oracle nowhere, hence the layer tolerance of tests/test_zy_layers_gpu.py
+    p64 = {k: v.detach().cpu().to(dtype).to(D) for k, v in layer.state_dict().items()}
+    want, _ = otl.decoder_layer(x.cpu().to(D), ctxt.cpu().to(D), p64, opt.n_heads, causal.cpu(), src_pad.cpu(), act="gelu",
+                                training=False)
+    x_mixed = torch.cat([x[:3][:, perm], x_after[3:]])
+    want_after, _ = otl.decoder_layer(x_mixed.cpu().to(D), ctxt[:, perm].cpu().to(D), p64, opt.n_heads, causal.cpu(),
+                                      src_pad[perm].cpu(), act="gelu", training=False)
+    tol = 2.5e-2 * max(1.0, float(want.abs().max()))
+    assert_close(torch.cat(rows[:3]), want[:3], dtype, "steps before the re-ordering vs oracle", rtol=3e-2, atol=tol)
+    assert_close(torch.cat(rows[3:]), want_after[3:], dtype, "steps after the re-ordering vs oracle", rtol=3e-2, atol=tol)
     close(torch.cat(rows[:3]), full[:3], dtype, "steps before the re-ordering")
     close(torch.cat(rows[3:]), full_after[3:], dtype, "steps after the re-ordering")
