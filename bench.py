@@ -645,9 +645,10 @@ def _cache_flushed(w, reps=20):
 
 
 def _measured_traffic():
-    """HBM bytes per step of each workload's dominant kernel group, measured offline with rocprofv3
-    --pmc FETCH_SIZE / WRITE_SIZE (counters cannot be read from inside this process); the file
-    holds the figures and the commands that produced them."""
+    """HBM bytes per step of each workload's kernel groups, measured offline with rocprofv3 --pmc FETCH_SIZE and
+    --pmc WRITE_SIZE (counters cannot be read from inside this process) and scaled by what the same counters read for
+    a 1 GiB copy; profiles/hbm_traffic_counters.txt holds the commands and the per-group table. roofline.traffic is
+    that figure per launch of the group (bytes per step / launches per step), like roofline.achieved's work."""
     path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
     try:
         with open(path) as f:
@@ -714,7 +715,7 @@ def measure(w, dev, steps, warmup, do_cpu, trace_steps):
         achieved = w.rate(work, us * 1e-6)
         launches = sum(k["launches_per_step"] for k in sel)
         roof = dict(bound=w.bound, achieved=round(achieved, 3), peak=w.peak, unit=w.unit, frac=round(achieved / w.peak, 4),
-                    traffic=traffic_table.get(prefix), kernel=(prefix + "*" if prefix.endswith("_") else prefix), launches_per_step=launches,
+                    traffic=(round(traffic_table[prefix] / launches) if traffic_table.get(prefix) and launches else None), kernel=(prefix + "*" if prefix.endswith("_") else prefix), launches_per_step=launches,
                     avg_launch_us=round(us / launches, 3), work_per_step=work)
     res = dict(workload=w.name, description=w.description, metric="achieved HBM GB/s" if w.bound == "hbm" else "MFMA TFLOP/s",
                value=round(w.rate(w.work_per_step(), per_step), 3), unit=w.unit, ms_per_step=round(per_step * 1e3, 5),
