@@ -179,22 +179,33 @@ __device__ __forceinline__ void store_pack(T* __restrict__ p, const float (&in)[
 // ---------------------------------------------------------------------------------------------
 // Wavefront (64 lanes) reductions: butterfly over lanes, every lane ends with the result.
 // ---------------------------------------------------------------------------------------------
+// Wavefront reductions on the DPP lane-exchange modifiers (no LDS traffic, no address arithmetic): four exchange steps
+// leave every lane of a 16-lane row with the row's total, then the four row totals are read as scalars. The pairing
+// is that of the xor butterfly (1, 2, 4, 8, 16, 32), so the result is the same in every lane, bit for bit.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float lane_f32(float v, int lane) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+template <typename Op>
+__device__ __forceinline__ float wave_reduce(float v, Op op) {
+  v = op(v, dpp_f32<0xB1>(v));    // quad_perm [1, 0, 3, 2]: lane ^ 1
+  v = op(v, dpp_f32<0x4E>(v));    // quad_perm [2, 3, 0, 1]: lane ^ 2
+  v = op(v, dpp_f32<0x141>(v));   // row_half_mirror: the other quad of each group of 8
+  v = op(v, dpp_f32<0x140>(v));   // row_mirror: the other half of each row of 16
+  return op(op(lane_f32(v, 0), lane_f32(v, 16)), op(lane_f32(v, 32), lane_f32(v, 48)));
+}
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
-  return v;
+  return wave_reduce(v, [](float a, float b) { return a + b; });
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, 64));
-  return v;
+  return wave_reduce(v, [](float a, float b) { return fmaxf(a, b); });
 }
 __device__ __forceinline__ void wave_sum2(float& a, float& b) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) {
-    a += __shfl_xor(a, m, 64);
-    b += __shfl_xor(b, m, 64);
-  }
+  a = wave_sum(a);
+  b = wave_sum(b);
 }
 
 
@@ -232,6 +243,10 @@ __device__ __forceinline__ float u01(uint32_t w) { return static_cast<float>(w >
 template <int N>
 __device__ __forceinline__ void philox_keep(const Philox& gen, uint64_t first, uint64_t offset, float keep_p,
                                             uint8_t (&keep)[N]) {
+#ifdef NMTG_NO_PHILOX   // tuning builds only
+  for (int i = 0; i < N; ++i) keep[i] = 1;
+  return;
+#endif
   if constexpr (N >= 4) {
 #pragma unroll
     for (int b = 0; b < N / 4; ++b) {

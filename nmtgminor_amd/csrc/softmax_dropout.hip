@@ -45,10 +45,19 @@ struct SoftmaxArgs {
   uint64_t seed, offset;
 };
 
+// 32-bit index arithmetic wherever the row count allows it (a 64-bit division is some 140 scalar instructions,
+// as much as the rest of a short row's work).
 __device__ __forceinline__ const uint8_t* kmask_row(const SoftmaxArgs& a, int64_t row) {
-  if (a.kmask_kind == SM_PAD) return a.kmask + (row / (static_cast<int64_t>(a.heads) * a.q_len)) * a.cols;
-  if (a.kmask_kind == SM_TIME) return a.kmask + (row % a.q_len) * static_cast<int64_t>(a.cols);
-  return nullptr;
+  if (a.kmask_kind == SM_NOMASK) return nullptr;
+  const int64_t group = a.kmask_kind == SM_PAD ? static_cast<int64_t>(a.heads) * a.q_len : a.q_len;
+  int64_t idx;
+  if (a.rows <= 0x7fffffff) {
+    const uint32_t r = static_cast<uint32_t>(row), g = static_cast<uint32_t>(group);
+    idx = a.kmask_kind == SM_PAD ? r / g : r % g;
+  } else {
+    idx = a.kmask_kind == SM_PAD ? row / group : row % group;
+  }
+  return a.kmask + idx * a.cols;
 }
 
 // Every kernel below issues all of a row's loads (scores, key mask, dropout mask, gradient) before it uses any of
@@ -110,101 +119,124 @@ __device__ __forceinline__ void row_softmax(const pack<T, EPV> (&rx)[VPL], const
     for (int j = 0; j < EPV; ++j) v[i][j] *= inv;
 }
 
-template <typename T, int EPV, int VPL>
+// A wavefront owns RPW consecutive rows: the loads of all of them are issued before the first is used, so that the
+// bytes in flight per wavefront (and with them the bandwidth of a kernel whose wavefronts otherwise wait out one
+// memory latency per row) grow RPW-fold; the rows are then normalised and stored one after the other.
+// RNG (the keep mask is drawn here from Philox and stored) is a compile-time switch: as a run-time branch the
+// generator's ~200 integer instructions per 8 elements were scheduled ahead of the branch and ran in every mode,
+// which made the kernel instruction-bound (about 290 vector instructions per 512-key row instead of about 90).
+template <typename T, int EPV, int VPL, int RPW, bool RNG>
 __global__ __launch_bounds__(SM_THREADS) void softmax_fwd_kernel(SoftmaxArgs a) {
   const int lane = threadIdx.x & (kWave - 1);
-  const int64_t row = static_cast<int64_t>(blockIdx.x) * SM_WAVES + threadIdx.x / kWave;
-  if (row >= a.rows) return;
-  const int64_t base = row * a.cols;
-  const uint8_t* km = kmask_row(a, row);
-  const bool mask_in = a.dropout_mode == SM_MASK_IN;
-  pack<T, EPV> rx[VPL];
-  pack<uint8_t, EPV> rk[VPL] = {}, rd[VPL] = {};
-  row_load<T, EPV, VPL>(static_cast<const T*>(a.in) + base, a.cols, lane, rx);
-  if (km != nullptr) row_load<uint8_t, EPV, VPL>(km, a.cols, lane, rk);
-  if (mask_in) row_load<uint8_t, EPV, VPL>(a.dmask + base, a.cols, lane, rd);
-  row_pin(rx); row_pin(rk); row_pin(rd);
-  float v[VPL][EPV];
-  row_softmax<T, EPV, VPL>(rx, rk, km != nullptr, a.cols, lane, v);
-  T* out = static_cast<T*>(a.out) + base;
-  T* out_sm = a.out_softmax ? static_cast<T*>(a.out_softmax) + base : nullptr;
-  const Philox gen(a.seed);
+  const int64_t row0 = (static_cast<int64_t>(blockIdx.x) * SM_WAVES + __builtin_amdgcn_readfirstlane(threadIdx.x / kWave)) * RPW;
+  if (row0 >= a.rows) return;
+  const bool mask_in = !RNG && a.dropout_mode == SM_MASK_IN;
+  const bool masked = a.kmask_kind != SM_NOMASK;
+  pack<T, EPV> rx[RPW][VPL];
+  pack<uint8_t, EPV> rk[RPW][VPL] = {}, rd[RPW][VPL] = {};
 #pragma unroll
-  for (int i = 0; i < VPL; ++i) {
-    const int col = row_col<EPV>(i, lane);
-    if (col < a.cols) {
-      if (out_sm) store_pack<T, EPV>(out_sm + col, v[i]);
-      if (a.dropout_mode != SM_NO_DROPOUT) {
-        uint8_t keep[EPV];
-        if (mask_in) {
+  for (int r = 0; r < RPW; ++r) {
+    const int64_t row = min(row0 + r, a.rows - 1);     // rows past the end: loaded again, not used
+    row_load<T, EPV, VPL>(static_cast<const T*>(a.in) + row * a.cols, a.cols, lane, rx[r]);
+    if (masked) row_load<uint8_t, EPV, VPL>(kmask_row(a, row), a.cols, lane, rk[r]);
+    if (mask_in) row_load<uint8_t, EPV, VPL>(a.dmask + row * a.cols, a.cols, lane, rd[r]);
+  }
 #pragma unroll
-          for (int j = 0; j < EPV; ++j) keep[j] = rd[i].v[j];
-        } else {
-          philox_keep<EPV>(gen, static_cast<uint64_t>(base + col), a.offset, a.keep_p, keep);
-          store_bytes<EPV>(a.dmask + base + col, keep);
+  for (int r = 0; r < RPW; ++r) { row_pin(rx[r]); row_pin(rk[r]); row_pin(rd[r]); }
+  [[maybe_unused]] const Philox gen(a.seed);
+#pragma unroll
+  for (int r = 0; r < RPW; ++r) {
+    if (row0 + r >= a.rows) break;
+    const int64_t base = (row0 + r) * a.cols;
+    float v[VPL][EPV];
+    row_softmax<T, EPV, VPL>(rx[r], rk[r], masked, a.cols, lane, v);
+    T* out = static_cast<T*>(a.out) + base;
+    T* out_sm = a.out_softmax ? static_cast<T*>(a.out_softmax) + base : nullptr;
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      const int col = row_col<EPV>(i, lane);
+      if (col < a.cols) {
+        if (out_sm) store_pack<T, EPV>(out_sm + col, v[i]);
+        if (a.dropout_mode != SM_NO_DROPOUT) {
+          uint8_t keep[EPV];
+          if constexpr (RNG) {
+            philox_keep<EPV>(gen, static_cast<uint64_t>(base + col), a.offset, a.keep_p, keep);
+            store_bytes<EPV>(a.dmask + base + col, keep);
+          } else {
+#pragma unroll
+            for (int j = 0; j < EPV; ++j) keep[j] = rd[r][i].v[j];
+          }
+#pragma unroll
+          for (int j = 0; j < EPV; ++j) v[i][j] = keep[j] ? v[i][j] * a.scale : 0.f;
         }
-#pragma unroll
-        for (int j = 0; j < EPV; ++j) v[i][j] = keep[j] ? v[i][j] * a.scale : 0.f;
+        store_pack<T, EPV>(out + col, v[i]);
       }
-      store_pack<T, EPV>(out + col, v[i]);
     }
   }
 }
 
 // dS = P * (g - sum_k P * g), g = keep * dP / (1 - p).
-template <typename T, int EPV, int VPL>
+template <typename T, int EPV, int VPL, int RPW>
 __global__ __launch_bounds__(SM_THREADS) void softmax_bwd_kernel(SoftmaxArgs a) {
   const int lane = threadIdx.x & (kWave - 1);
-  const int64_t row = static_cast<int64_t>(blockIdx.x) * SM_WAVES + threadIdx.x / kWave;
-  if (row >= a.rows) return;
-  const int64_t base = row * a.cols;
-  const uint8_t* km = a.from_scores ? kmask_row(a, row) : nullptr;
+  const int64_t row0 = (static_cast<int64_t>(blockIdx.x) * SM_WAVES + __builtin_amdgcn_readfirstlane(threadIdx.x / kWave)) * RPW;
+  if (row0 >= a.rows) return;
+  const bool masked = a.from_scores && a.kmask_kind != SM_NOMASK;
   const bool dropped = a.dropout_mode != SM_NO_DROPOUT;
-  pack<T, EPV> rs[VPL], rg[VPL];
-  pack<uint8_t, EPV> rk[VPL] = {}, rd[VPL] = {};
-  row_load<T, EPV, VPL>(static_cast<const T*>(a.saved) + base, a.cols, lane, rs);
-  row_load<T, EPV, VPL>(static_cast<const T*>(a.in) + base, a.cols, lane, rg);
-  if (km != nullptr) row_load<uint8_t, EPV, VPL>(km, a.cols, lane, rk);
-  if (dropped) row_load<uint8_t, EPV, VPL>(a.dmask + base, a.cols, lane, rd);
-  row_pin(rs); row_pin(rg); row_pin(rk); row_pin(rd);
-  float pr[VPL][EPV], g[VPL][EPV];
-  if (a.from_scores) {
-    row_softmax<T, EPV, VPL>(rs, rk, km != nullptr, a.cols, lane, pr);
-  } else {
+  pack<T, EPV> rs[RPW][VPL], rg[RPW][VPL];
+  pack<uint8_t, EPV> rk[RPW][VPL] = {}, rd[RPW][VPL] = {};
 #pragma unroll
-    for (int i = 0; i < VPL; ++i) {
-      if (row_col<EPV>(i, lane) < a.cols) unpack_raw<T, EPV>(rs[i], pr[i]);
-      else {
-#pragma unroll
-        for (int j = 0; j < EPV; ++j) pr[i][j] = 0.f;
-      }
-    }
+  for (int r = 0; r < RPW; ++r) {
+    const int64_t row = min(row0 + r, a.rows - 1);
+    row_load<T, EPV, VPL>(static_cast<const T*>(a.saved) + row * a.cols, a.cols, lane, rs[r]);
+    row_load<T, EPV, VPL>(static_cast<const T*>(a.in) + row * a.cols, a.cols, lane, rg[r]);
+    if (masked) row_load<uint8_t, EPV, VPL>(kmask_row(a, row), a.cols, lane, rk[r]);
+    if (dropped) row_load<uint8_t, EPV, VPL>(a.dmask + row * a.cols, a.cols, lane, rd[r]);
   }
-  float dot = 0.f;
 #pragma unroll
-  for (int i = 0; i < VPL; ++i) {
-    if (row_col<EPV>(i, lane) < a.cols) {
-      unpack_raw<T, EPV>(rg[i], g[i]);
-      if (dropped) {
+  for (int r = 0; r < RPW; ++r) { row_pin(rs[r]); row_pin(rg[r]); row_pin(rk[r]); row_pin(rd[r]); }
 #pragma unroll
-        for (int j = 0; j < EPV; ++j) g[i][j] = rd[i].v[j] ? g[i][j] * a.scale : 0.f;
-      }
-#pragma unroll
-      for (int j = 0; j < EPV; ++j) dot += pr[i][j] * g[i][j];
+  for (int r = 0; r < RPW; ++r) {
+    if (row0 + r >= a.rows) break;
+    float pr[VPL][EPV], g[VPL][EPV];
+    if (a.from_scores) {
+      row_softmax<T, EPV, VPL>(rs[r], rk[r], masked, a.cols, lane, pr);
     } else {
 #pragma unroll
-      for (int j = 0; j < EPV; ++j) g[i][j] = 0.f;
+      for (int i = 0; i < VPL; ++i) {
+        if (row_col<EPV>(i, lane) < a.cols) unpack_raw<T, EPV>(rs[r][i], pr[i]);
+        else {
+#pragma unroll
+          for (int j = 0; j < EPV; ++j) pr[i][j] = 0.f;
+        }
+      }
     }
-  }
-  dot = wave_sum(dot);
-  T* out = static_cast<T*>(a.out) + base;
+    float dot = 0.f;
 #pragma unroll
-  for (int i = 0; i < VPL; ++i) {
-    const int col = row_col<EPV>(i, lane);
-    if (col < a.cols) {
+    for (int i = 0; i < VPL; ++i) {
+      if (row_col<EPV>(i, lane) < a.cols) {
+        unpack_raw<T, EPV>(rg[r][i], g[i]);
+        if (dropped) {
 #pragma unroll
-      for (int j = 0; j < EPV; ++j) g[i][j] = pr[i][j] * (g[i][j] - dot);
-      store_pack<T, EPV>(out + col, g[i]);
+          for (int j = 0; j < EPV; ++j) g[i][j] = rd[r][i].v[j] ? g[i][j] * a.scale : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < EPV; ++j) dot += pr[i][j] * g[i][j];
+      } else {
+#pragma unroll
+        for (int j = 0; j < EPV; ++j) g[i][j] = 0.f;
+      }
+    }
+    dot = wave_sum(dot);
+    T* out = static_cast<T*>(a.out) + (row0 + r) * a.cols;
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      const int col = row_col<EPV>(i, lane);
+      if (col < a.cols) {
+#pragma unroll
+        for (int j = 0; j < EPV; ++j) g[i][j] = pr[i][j] * (g[i][j] - dot);
+        store_pack<T, EPV>(out + col, g[i]);
+      }
     }
   }
 }
@@ -235,14 +267,18 @@ int softmax_launch(const SoftmaxArgs& a, bool bwd, hipStream_t st) {
   const int vecs = (a.cols + epv - 1) / epv;
   int vpl = 1;
   while (vpl * kWave < vecs) vpl *= 2;
-  const unsigned grid = static_cast<unsigned>((a.rows + SM_WAVES - 1) / SM_WAVES);
+  // rows per wavefront: as many as keep the raw loads of a wavefront within about 32 registers per operand
   bool done = false;
+  const bool rng = !bwd && a.dropout_mode == SM_MASK_RNG;
   TraceScope trace(bwd ? "softmax_dropout_bwd" : "softmax_dropout_fwd", st);
-#define SM_CASE(E, V)                                                                                     \
-  if (!done && epv == E && vpl == V) {                                                                    \
-    if (bwd) hipLaunchKernelGGL((softmax_bwd_kernel<T, E, V>), dim3(grid), dim3(SM_THREADS), 0, st, a);   \
-    else hipLaunchKernelGGL((softmax_fwd_kernel<T, E, V>), dim3(grid), dim3(SM_THREADS), 0, st, a);       \
-    done = true;                                                                                          \
+#define SM_CASE(E, V)                                                                                             \
+  if (!done && epv == E && vpl == V) {                                                                            \
+    constexpr int R = V == 1 ? 4 : V == 2 ? 2 : 1;                                                                \
+    const unsigned grid = static_cast<unsigned>((a.rows + SM_WAVES * R - 1) / (SM_WAVES * R));                    \
+    if (bwd) hipLaunchKernelGGL((softmax_bwd_kernel<T, E, V, R>), dim3(grid), dim3(SM_THREADS), 0, st, a);        \
+    else if (rng) hipLaunchKernelGGL((softmax_fwd_kernel<T, E, V, R, true>), dim3(grid), dim3(SM_THREADS), 0, st, a);  \
+    else hipLaunchKernelGGL((softmax_fwd_kernel<T, E, V, R, false>), dim3(grid), dim3(SM_THREADS), 0, st, a);     \
+    done = true;                                                                                                  \
   }
   if constexpr (sizeof(T) == 2) { SM_CASE(8, 1) SM_CASE(8, 2) SM_CASE(8, 4) SM_CASE(8, 8) }
   SM_CASE(4, 1) SM_CASE(4, 2) SM_CASE(4, 4) SM_CASE(4, 8) SM_CASE(4, 16)

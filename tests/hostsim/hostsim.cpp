@@ -216,6 +216,24 @@ void land(const Transfer& t) {
 }
 }  // namespace
 
+namespace {
+void resolve_gather(void** payloads, int lanes) {
+  uint64_t in[WAVE];
+  for (int l = 0; l < lanes; ++l) in[l] = static_cast<Shuffle*>(payloads[l])->bits;
+  for (int l = 0; l < lanes; ++l) {
+    const int from = static_cast<Shuffle*>(payloads[l])->mask;
+    if (from < 0 || from >= lanes) die("lane exchange reads a lane that is not part of the wavefront");
+    static_cast<Shuffle*>(payloads[l])->bits = in[from];
+  }
+}
+}  // namespace
+
+uint64_t gather_bits(uint64_t bits, int source_lane) {
+  Shuffle s{bits, source_lane};
+  wave_collective(resolve_gather, &s);
+  return s.bits;
+}
+
 uint64_t shfl_xor_bits(uint64_t bits, int mask) {
   Shuffle s{bits, mask};
   wave_collective(resolve_shuffle, &s);

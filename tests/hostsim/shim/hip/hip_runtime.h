@@ -50,6 +50,7 @@ void wave_collective(Resolver resolver, void* payload);
 [[noreturn]] void fail(const char* what);
 unsigned lane_id();
 uint64_t shfl_xor_bits(uint64_t bits, int mask);
+uint64_t gather_bits(uint64_t bits, int source_lane);   // every lane names the lane whose value it reads
 void sync_block();
 // direct global -> LDS transfers (asynchronous; see hostsim.cpp for the two timing models)
 void dma_issue(const void* src, uint32_t lds_offset, int bytes);
@@ -87,6 +88,18 @@ static inline T __shfl_xor(T v, int mask, int width = 64) {
   return out;
 }
 static inline void __syncthreads() { hostsim::sync_block(); }
+
+// DPP lane exchange (all rows and banks enabled): the controls the kernels use
+static inline int __builtin_amdgcn_update_dpp(int, int src, int ctrl, int, int, bool) {
+  const int lane = static_cast<int>(hostsim::lane_id());
+  int from;
+  if (ctrl < 0x100) from = (lane & ~3) | ((ctrl >> (2 * (lane & 3))) & 3);   // quad_perm
+  else if (ctrl == 0x141) from = (lane & ~7) | (7 - (lane & 7));              // row_half_mirror
+  else if (ctrl == 0x140) from = (lane & ~15) | (15 - (lane & 15));           // row_mirror
+  else hostsim::fail("DPP control not modelled");
+  return static_cast<int>(hostsim::gather_bits(static_cast<uint32_t>(src), from));
+}
+static inline int __builtin_amdgcn_readlane(int v, int lane) { return static_cast<int>(hostsim::gather_bits(static_cast<uint32_t>(v), lane)); }
 
 static inline uint32_t __umulhi(uint32_t a, uint32_t b) { return static_cast<uint32_t>((static_cast<uint64_t>(a) * b) >> 32); }
 static inline float __uint_as_float(uint32_t u) { float f; std::memcpy(&f, &u, 4); return f; }
