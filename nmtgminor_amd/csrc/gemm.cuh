@@ -45,7 +45,10 @@ enum GemmEpi {
   // Backward counterpart on the same whole-row tile: acc = dP (gradient of the dropped probabilities, rounded to
   // T as the two-kernel path stores it); P is recomputed from the saved scores (aux_in, laid out like C) and
   // C = P * (g - sum_k P g), g = keep * dP / (1 - p).
-  EPI_DSOFTMAX = 6
+  EPI_DSOFTMAX = 6,
+  // EPI_SCORES_SOFTMAX with the dropout keep mask drawn from Philox in the kernel (and stored). Its own instantiation:
+  // as a run-time branch the generator's integer work is scheduled ahead of the branch and runs in every mode.
+  EPI_SCORES_SOFTMAX_RNG = 7
 };
 
 struct GemmArgs {
@@ -593,17 +596,18 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, acc16_t (&acc)[
     if (EPI == EPI_SCORES && g.kmask_kind == 1)
       padm = load8_bytes<VEC>(g.kmask + static_cast<int64_t>(bz / g.heads) * g.N + n, g.kmask, ncols);
 
-    if constexpr (EPI == EPI_SCORES_SOFTMAX) {
+    if constexpr (EPI == EPI_SCORES_SOFTMAX || EPI == EPI_SCORES_SOFTMAX_RNG) {
+      constexpr bool RNG = EPI == EPI_SCORES_SOFTMAX_RNG;
       // One wavefront per row: lane cc holds the row's elements 8 cc .. 8 cc + 7.
       static_assert(CPR == 64 && VEC == 8, "the row tile is 512 columns wide and moves 16-byte chunks");
       uint16_t* OUT2 = reinterpret_cast<uint16_t*>(g.out2) + static_cast<int64_t>(bz) * g.sC;
       const bool time_mask = g.kmask_kind == 2;
       const bool drop = g.dmask != nullptr;
-      const bool replay = drop && !g.rng;
+      const bool replay = drop && !RNG;
       uint2 padm2 = make_uint2(0, 0);
       if (g.kmask_kind == 1) padm2 = load8_bytes<VEC>(g.kmask + static_cast<int64_t>(bz / g.heads) * g.N + n, g.kmask, ncols);
       constexpr float LOG2E = 1.4426950408889634f;
-      const Philox gen(g.seed);
+      [[maybe_unused]] const Philox gen(g.seed);
       for (int p0 = 0; p0 < PASSES; p0 += GRP) {
         uint2 traw[GRP], draw[GRP];
         if (time_mask) {
@@ -661,7 +665,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmArgs& g, acc16_t (&acc)[
           if (AUX != nullptr) store8<VEC>(AUX + off, pack8<T>(v), nv);
           if (drop) {
             uint2 keep = draw[u];
-            if (g.rng) {
+            if constexpr (RNG) {
               uint8_t kb[8];
               const uint64_t first = (static_cast<uint64_t>(bz) * g.M + m) * g.N + n;
               philox_keep<8>(gen, first, g.offset, g.keep_p, kb);

@@ -196,7 +196,7 @@ int row_tile_try(int dtype, int epi, GemmArgs a, const void* extra_like_c, hipSt
 }  // namespace
 
 int gemm_scores_softmax_try(int dtype, GemmArgs a, hipStream_t st) {
-  return row_tile_try(dtype, EPI_SCORES_SOFTMAX, a, a.out2, st);
+  return row_tile_try(dtype, (a.dmask != nullptr && a.rng) ? EPI_SCORES_SOFTMAX_RNG : EPI_SCORES_SOFTMAX, a, a.out2, st);
 }
 
 int gemm_dsoftmax_try(int dtype, GemmArgs a, hipStream_t st) {

@@ -35,7 +35,7 @@ int gemm_launch_vec(const GemmArgs& a, hipStream_t st) {
   static const std::string name = std::string("gemm_") + (A_KC ? (B_KC ? "nt" : "nn") : "tn") + "_" +
                                   (TILE == TILE_L ? "256x256" : TILE == TILE_M ? "128x128" : TILE == TILE_R ? "128x512" : "256x64") + "_" +
                                   (EPI == EPI_PLAIN ? "plain" : EPI == EPI_ACT_FWD ? "actfwd" : EPI == EPI_ACT_BWD ? "actbwd"
-                                   : EPI == EPI_SCORES ? "scores" : EPI == EPI_SCORES_SOFTMAX ? "scores_softmax" : EPI == EPI_DSOFTMAX ? "dsoftmax"
+                                   : EPI == EPI_SCORES ? "scores" : (EPI == EPI_SCORES_SOFTMAX || EPI == EPI_SCORES_SOFTMAX_RNG) ? "scores_softmax" : EPI == EPI_DSOFTMAX ? "dsoftmax"
                                    : "splitk") +
                                   (VEC == 8 ? "" : VEC == 4 ? "_v4" : "_v1") +
                                   (DMA ? "_dma" : "");

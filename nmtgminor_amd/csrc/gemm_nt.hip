@@ -9,6 +9,7 @@ template <typename T> static int run(int tile, int epi, const GemmArgs& a, hipSt
   CASE(TILE_L, EPI_SCORES) CASE(TILE_M, EPI_SCORES)
   // whole-row tile with the fused softmax epilogue: 16-byte accesses only, two-buffer loop (K is one or two steps)
   if (tile == TILE_R && epi == EPI_SCORES_SOFTMAX) return gemm_launch_vec<T, TILE_R, true, true, EPI_SCORES_SOFTMAX, 8>(a, st);
+  if (tile == TILE_R && epi == EPI_SCORES_SOFTMAX_RNG) return gemm_launch_vec<T, TILE_R, true, true, EPI_SCORES_SOFTMAX_RNG, 8>(a, st);
   if (tile == TILE_R && epi == EPI_DSOFTMAX) return gemm_launch_vec<T, TILE_R, true, true, EPI_DSOFTMAX, 8>(a, st);
   return fail(NMTG_ERR_UNSUPPORTED, "gemm NT: no kernel for tile %d epilogue %d", tile, epi);
 }
