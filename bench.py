@@ -123,6 +123,42 @@ class LayerNormWL(Workload):
                     sample="full workload (4096 x 512 fp32 fwd+bwd), median of 5")
 
 
+class LayerNormLargeWL(LayerNormWL):
+    """The streaming rate of the LayerNorm kernels on tensors beyond the 256 MB last-level cache: 64 times the rows
+    of the largest shape the reference's own timing script uses (512 * 32 rows of 1024, onmt/modules/test_layer_norm.py:243-255),
+    in bf16 with bf16 weights."""
+    name = "layer_norm_large"
+    dtype = "bf16"
+    description = "LayerNorm fwd+bwd bf16 [65536 x 1024], eps 1e-5 (134 MB per tensor: beyond the last-level cache)"
+
+    def setup(self, dev):
+        from oracle import inputs
+        from nmtgminor_amd.native import fast_layer_norm_cuda as ln
+        self.ln = ln
+        self.cpu = inputs.layer_norm_inputs(65536, 1024, torch.bfloat16, seed=1011)
+        d = self.cpu
+        self.x, self.g, self.b, self.dy = (d[k].to(dev) for k in ("x", "gamma", "beta", "dy"))
+        self.rows, self.h = self.x.shape
+
+    def _bytes(self):
+        t = self.rows * self.h * 2
+        fwd = 2 * t + 2 * self.h * 2 + 2 * self.rows * 4
+        bwd = 3 * t + 2 * self.rows * 4 + 3 * self.h * 2
+        return fwd, bwd
+
+    def cpu_baseline(self):
+        from oracle import layer_norm as o
+        d = self.cpu
+        rows = 8192                                   # a bounded sample: one eighth of the rows
+
+        def run():
+            z, mu, rs = o.ln_fwd(d["x"][:rows], d["gamma"], d["beta"], d["eps"])
+            o.ln_bwd(d["dy"][:rows], d["x"][:rows], mu, rs, d["gamma"])
+        t = _time_cpu(run, 3)
+        return dict(value=self.work_per_step() * rows / self.rows / t / 1e9, unit="GB/s", cores=torch.get_num_threads(), kind="port",
+                    sample="the first 8192 of 65536 rows, fwd+bwd in fp32 on the bf16 values, median of 3")
+
+
 class MlpWL(Workload):
     name = "mlp"
     bound = "mfma"
@@ -606,7 +642,7 @@ class CopyWL(Workload):
 
 # the five benchmark configurations first, then the workloads added beside them
 WORKLOADS = {w.name: w for w in (LayerNormWL, MlpWL, SelfAttnWL, EncdecAttnWL, XentropyWL, SoftmaxDropoutWL, DropoutAddWL,
-                                    GeneratorLossWL, RelSelfAttnWL, FusedAdamWL)}
+                                    GeneratorLossWL, RelSelfAttnWL, FusedAdamWL, LayerNormLargeWL)}
 EXTRA_WORKLOADS = {CopyWL.name: CopyWL}
 PRIMARY = "mlp"
 
@@ -663,7 +699,15 @@ def measure(w, dev, steps, warmup, do_cpu, trace_steps):
     for _ in range(max(1, warmup)):
         w.step()
     _sync()
-    # one step captured into a HIP graph, replayed K times
+    # Steps are captured into a HIP graph and replayed: `unroll` steps per graph, so that the fixed cost of one graph
+    # launch (some 20 us here, more than a whole LayerNorm step) is spread over several steps; K steps are timed in all.
+    t0 = time.perf_counter()
+    w.step()
+    _sync()
+    est = time.perf_counter() - t0
+    unroll = 1
+    if est < 1e-3:
+        unroll = next((u for u in (10, 5, 4, 2) if steps % u == 0), 1)
     graph = None
     try:
         s = torch.cuda.Stream()
@@ -673,7 +717,8 @@ def measure(w, dev, steps, warmup, do_cpu, trace_steps):
             _sync()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, stream=s):
-                w.step()
+                for _ in range(unroll):
+                    w.step()
         _sync()
         graph.replay()
         _sync()
@@ -682,10 +727,11 @@ def measure(w, dev, steps, warmup, do_cpu, trace_steps):
         graph = None
     _sync()
     t0 = time.perf_counter()
-    for _ in range(steps):
-        if graph is not None:
+    if graph is not None:
+        for _ in range(steps // unroll):
             graph.replay()
-        else:
+    else:
+        for _ in range(steps):
             w.step()
     _sync()
     wall = time.perf_counter() - t0
@@ -720,7 +766,7 @@ def measure(w, dev, steps, warmup, do_cpu, trace_steps):
     res = dict(workload=w.name, description=w.description, metric="achieved HBM GB/s" if w.bound == "hbm" else "MFMA TFLOP/s",
                value=round(w.rate(w.work_per_step(), per_step), 3), unit=w.unit, ms_per_step=round(per_step * 1e3, 5),
                frac_of_peak=round(w.rate(w.work_per_step(), per_step) / w.peak, 4), dtype=w.dtype, data=w.data,
-               timed="hip graph replay" if graph is not None else "eager launches", roofline=roof,
+               timed=(f"hip graph replay, {unroll} steps per graph" if graph is not None else "eager launches"), roofline=roof,
                kernels=[dict(name=k["name"], launches_per_step=k["launches_per_step"], avg_us=round(k["avg_us"], 3))
                         for k in kernels])
     if w.name == "layer_norm":
