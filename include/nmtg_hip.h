@@ -146,6 +146,14 @@ int nmtg_xentropy_fwd(const void* logits, const int64_t* labels, float* losses, 
                       int64_t rows, int64_t vocab, int64_t ld_logits, float smoothing,
                       int64_t padding_idx, int dtype, void* stream);
 
+/* nmtg_xentropy_fwd that also writes argmax [rows] (int64): the index of each row's largest logit with
+ * torch.argmax's rule (NaN counts as the largest value; the lowest index among equals). Replaces the
+ * argmax over the logits in the reference's evaluation branch (NMTLossFunc.forward,
+ * onmt/modules/loss.py:293-311), which re-reads the whole logits tensor. */
+int nmtg_xentropy_fwd_argmax(const void* logits, const int64_t* labels, float* losses, float* lse,
+                             int64_t* argmax, int64_t rows, int64_t vocab, int64_t ld_logits,
+                             float smoothing, int64_t padding_idx, int dtype, void* stream);
+
 int nmtg_xentropy_bwd(const float* grad_loss, const void* logits, const float* lse,
                       const int64_t* labels, void* grad_logits, int64_t rows, int64_t vocab,
                       int64_t ld_logits, int64_t ld_grad, int64_t class_offset,

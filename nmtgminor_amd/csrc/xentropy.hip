@@ -29,7 +29,9 @@ constexpr int XE_WAVES = XE_THREADS / kWave;
 constexpr int XE_INFLIGHT = 4;
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
-constexpr float NEG_BIG = -3.0e38f;
+// start value of the running maximum: below every finite logit, and small enough in magnitude that NEG_BIG * LOG2E is
+// still finite (a lane that has only seen -inf logits must not turn them into NaN)
+constexpr float NEG_BIG = -1.0e30f;
 
 struct Online {
   float m, s;  // running max and sum of exp(x - m)
@@ -65,12 +67,33 @@ __device__ __forceinline__ void online_add(Online& st, float& sx, const float (&
   sx += sum;
 }
 
-template <typename T>
+// Running argmax with torch.argmax's rule: the largest value, NaN counting as larger than everything, and the lowest
+// index among equals (bf16 logits tie all the time, so the rule decides most rows).
+struct Best {
+  float v;
+  int64_t i;
+};
+__device__ __forceinline__ bool better(float v, int64_t i, const Best& b) {
+  const bool vn = v != v, bn = b.v != b.v;
+  if (vn || bn) return vn && (!bn || i < b.i);
+  return v > b.v || (v == b.v && i < b.i);
+}
+__device__ __forceinline__ void best_add(Best& b, float v, int64_t i) {
+  if (better(v, i, b)) { b.v = v; b.i = i; }
+}
+
+// ARGMAX: also writes the index of each row's largest logit (the evaluation branch of the loss counts correct
+// predictions from it, onmt/modules/loss.py:293-311); its own instantiation, the training forward pays nothing for it.
+template <typename T, bool ARGMAX>
 __global__ __launch_bounds__(XE_THREADS) void xentropy_fwd_kernel(
     const T* __restrict__ logits, const int64_t* __restrict__ labels, float* __restrict__ losses,
-    float* __restrict__ lse_out, int64_t vocab, int64_t ld, float smoothing, int64_t padding_idx) {
+    float* __restrict__ lse_out, int64_t* __restrict__ argmax_out, int64_t vocab, int64_t ld, float smoothing,
+    int64_t padding_idx) {
   constexpr int EPV = 16 / sizeof(T);
   __shared__ float sm_m[XE_WAVES], sm_s[XE_WAVES], sm_x[XE_WAVES];
+  __shared__ float sm_bv[ARGMAX ? XE_WAVES : 1];
+  __shared__ int64_t sm_bi[ARGMAX ? XE_WAVES : 1];
+  Best best{-INFINITY, INT64_MAX};
   const int64_t row = blockIdx.x;
   const T* x = logits + row * ld;
   const int tid = threadIdx.x;
@@ -86,6 +109,7 @@ __global__ __launch_bounds__(XE_THREADS) void xentropy_fwd_kernel(
   if (tid < head) {
     float v[1] = {elem<T>::to_float(x[tid])};
     online_add<1>(st, sx, v);
+    if constexpr (ARGMAX) best_add(best, v[0], tid);
   }
   const T* body = x + head;
   int64_t i = tid;
@@ -102,16 +126,25 @@ __global__ __launch_bounds__(XE_THREADS) void xentropy_fwd_kernel(
       float a[EPV];
       unpack_raw<T, EPV>(raw[u], a);
       online_add<EPV>(st, sx, a);
+      if constexpr (ARGMAX) {
+#pragma unroll
+        for (int j = 0; j < EPV; ++j) best_add(best, a[j], head + (i + u * XE_THREADS) * EPV + j);
+      }
     }
   }
   for (; i < nvec; i += XE_THREADS) {
     float a[EPV];
     load_pack<T, EPV>(body + i * EPV, a);
     online_add<EPV>(st, sx, a);
+    if constexpr (ARGMAX) {
+#pragma unroll
+      for (int j = 0; j < EPV; ++j) best_add(best, a[j], head + i * EPV + j);
+    }
   }
   if (tail0 + tid < vocab) {
     float v[1] = {elem<T>::to_float(x[tail0 + tid])};
     online_add<1>(st, sx, v);
+    if constexpr (ARGMAX) best_add(best, v[0], tail0 + tid);
   }
 
   // wavefront merge, then across the block's wavefronts
@@ -120,11 +153,24 @@ __global__ __launch_bounds__(XE_THREADS) void xentropy_fwd_kernel(
     Online o{__shfl_xor(st.m, m, 64), __shfl_xor(st.s, m, 64)};
     st = merge(st, o);
     sx += __shfl_xor(sx, m, 64);
+    if constexpr (ARGMAX) {
+      const float ov = __shfl_xor(best.v, m, 64);
+      const int64_t oi = __shfl_xor(best.i, m, 64);
+      best_add(best, ov, oi);
+    }
   }
   const int wave = tid / kWave, lane = tid & (kWave - 1);
-  if (lane == 0) { sm_m[wave] = st.m; sm_s[wave] = st.s; sm_x[wave] = sx; }
+  if (lane == 0) {
+    sm_m[wave] = st.m; sm_s[wave] = st.s; sm_x[wave] = sx;
+    if constexpr (ARGMAX) { sm_bv[wave] = best.v; sm_bi[wave] = best.i; }
+  }
   __syncthreads();
   if (tid == 0) {
+    if constexpr (ARGMAX) {
+      Best b{sm_bv[0], sm_bi[0]};
+      for (int w = 1; w < XE_WAVES; ++w) best_add(b, sm_bv[w], sm_bi[w]);
+      argmax_out[row] = b.i;
+    }
     Online tot{sm_m[0], sm_s[0]};
     float tx = sm_x[0];
 #pragma unroll
@@ -134,7 +180,9 @@ __global__ __launch_bounds__(XE_THREADS) void xentropy_fwd_kernel(
     float loss = 0.f;
     if (y != padding_idx) {
       const float xy = (y >= 0 && y < vocab) ? elem<T>::to_float(x[y]) : 0.f;
-      loss = smoothing * (lse - tx / static_cast<float>(vocab)) + (1.f - smoothing) * (lse - xy);
+      loss = (1.f - smoothing) * (lse - xy);
+      // without smoothing the mean logit does not enter (it is -inf when a class is masked out, and 0 * inf is NaN)
+      if (smoothing != 0.f) loss += smoothing * (lse - tx / static_cast<float>(vocab));
     }
     losses[row] = loss;
     lse_out[row] = lse;
@@ -223,23 +271,43 @@ __global__ __launch_bounds__(XE_THREADS) void xentropy_bwd_kernel(
 
 using namespace nmtg;
 
+namespace {
+int xentropy_fwd_run(const char* who, const void* logits, const int64_t* labels, float* losses, float* lse, int64_t* argmax,
+                     bool want_argmax, int64_t rows, int64_t vocab, int64_t ld_logits, float smoothing, int64_t padding_idx,
+                     int dtype, void* stream) {
+  NMTG_REQUIRE(rows >= 0 && rows <= INT32_MAX, "%s: bad row count %lld", who, (long long)rows);
+  NMTG_REQUIRE(vocab > 0, "%s: number of classes must be positive", who);
+  NMTG_REQUIRE(ld_logits >= vocab, "%s: row pitch %lld is below the number of classes %lld", who,
+               (long long)ld_logits, (long long)vocab);
+  if (rows == 0) return 0;
+  NMTG_REQUIRE(logits && labels && losses && lse && (!want_argmax || argmax), "%s: null pointer argument", who);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  TraceScope trace(want_argmax ? "xentropy_fwd_argmax" : "xentropy_fwd", st);
+  NMTG_DISPATCH_DTYPE(
+      dtype, T,
+      if (want_argmax) hipLaunchKernelGGL((xentropy_fwd_kernel<T, true>), dim3(static_cast<unsigned>(rows)), dim3(XE_THREADS), 0, st,
+                                          static_cast<const T*>(logits), labels, losses, lse, argmax, vocab, ld_logits, smoothing,
+                                          padding_idx);
+      else hipLaunchKernelGGL((xentropy_fwd_kernel<T, false>), dim3(static_cast<unsigned>(rows)), dim3(XE_THREADS), 0, st,
+                              static_cast<const T*>(logits), labels, losses, lse, static_cast<int64_t*>(nullptr), vocab, ld_logits,
+                              smoothing, padding_idx));
+  NMTG_CHECK_LAUNCH(who);
+  return 0;
+}
+}  // namespace
+
 extern "C" int nmtg_xentropy_fwd(const void* logits, const int64_t* labels, float* losses, float* lse, int64_t rows,
                                  int64_t vocab, int64_t ld_logits, float smoothing, int64_t padding_idx, int dtype,
                                  void* stream) {
-  NMTG_REQUIRE(rows >= 0 && rows <= INT32_MAX, "xentropy_fwd: bad row count %lld", (long long)rows);
-  NMTG_REQUIRE(vocab > 0, "xentropy_fwd: number of classes must be positive");
-  NMTG_REQUIRE(ld_logits >= vocab, "xentropy_fwd: row pitch %lld is below the number of classes %lld",
-               (long long)ld_logits, (long long)vocab);
-  if (rows == 0) return 0;
-  NMTG_REQUIRE(logits && labels && losses && lse, "xentropy_fwd: null pointer argument");
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  TraceScope trace("xentropy_fwd", st);
-  NMTG_DISPATCH_DTYPE(dtype, T,
-                      hipLaunchKernelGGL((xentropy_fwd_kernel<T>), dim3(static_cast<unsigned>(rows)), dim3(XE_THREADS), 0,
-                                         st, static_cast<const T*>(logits), labels, losses, lse, vocab, ld_logits,
-                                         smoothing, padding_idx));
-  NMTG_CHECK_LAUNCH("xentropy_fwd");
-  return 0;
+  return xentropy_fwd_run("xentropy_fwd", logits, labels, losses, lse, nullptr, false, rows, vocab, ld_logits, smoothing,
+                          padding_idx, dtype, stream);
+}
+
+extern "C" int nmtg_xentropy_fwd_argmax(const void* logits, const int64_t* labels, float* losses, float* lse, int64_t* argmax,
+                                        int64_t rows, int64_t vocab, int64_t ld_logits, float smoothing, int64_t padding_idx,
+                                        int dtype, void* stream) {
+  return xentropy_fwd_run("xentropy_fwd_argmax", logits, labels, losses, lse, argmax, true, rows, vocab, ld_logits, smoothing,
+                          padding_idx, dtype, stream);
 }
 
 extern "C" int nmtg_xentropy_bwd(const float* grad_loss, const void* logits, const float* lse, const int64_t* labels,

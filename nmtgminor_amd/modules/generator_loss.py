@@ -154,8 +154,9 @@ def linear_cross_entropy_eval(hidden, weight, bias, labels, padding_idx=-100, ch
             buf = _chunk_buffer(min(n, chunk_rows), v, hidden)
             for r0, r1 in _chunks(n, chunk_rows):
                 z = _logits(hidden, weight, bias, r0, r1, buf)
-                losses[r0:r1] = xentropy_cuda.forward(z, labels[r0:r1], 0.0, True, padding_idx=padding_idx)[0]
-                preds[r0:r1] = torch.argmax(z, dim=1)
+                part, _, best = xentropy_cuda.forward(z, labels[r0:r1], 0.0, True, padding_idx=padding_idx, want_argmax=True)
+                losses[r0:r1] = part
+                preds[r0:r1] = best          # from the loss kernel's own pass over the row: the chunk is not read again
     return losses, preds
 
 

@@ -28,8 +28,9 @@ def _rows(t):
     return t.contiguous()
 
 
-def forward(logits, labels, smoothing, half_to_float=False, *, padding_idx=None):
-    """-> [losses fp32 [N], max_log_sum_exp [N] (fp32 if half_to_float or fp32 logits)]."""
+def forward(logits, labels, smoothing, half_to_float=False, *, padding_idx=None, want_argmax=False):
+    """-> [losses fp32 [N], max_log_sum_exp [N] (fp32 if half_to_float or fp32 logits)]; with want_argmax a third
+    entry, int64 [N]: the index of each row's largest logit by torch.argmax's rule, from the same pass over the row."""
     L.require_cuda(logits, labels)
     if half_to_float:
         _check(logits.dtype in (torch.float16, torch.bfloat16), "conversion is supported for Half type only")
@@ -43,12 +44,18 @@ def forward(logits, labels, smoothing, half_to_float=False, *, padding_idx=None)
     n, v = logits.shape
     losses = torch.empty(n, dtype=torch.float32, device=logits.device)
     lse = torch.empty(n, dtype=torch.float32, device=logits.device)
-    L.call("nmtg_xentropy_fwd", L.ptr(logits), L.ptr(labels), L.ptr(losses), L.ptr(lse), L.i64(n), L.i64(v),
-           L.i64(logits.stride(0)), L.f32(smoothing), L.i64(_NO_PAD if padding_idx is None else padding_idx), L.i32(L.dtype_code(logits)),
-           L.stream_of(logits))
+    pad = L.i64(_NO_PAD if padding_idx is None else padding_idx)
+    best = None
+    if want_argmax:
+        best = torch.empty(n, dtype=torch.int64, device=logits.device)
+        L.call("nmtg_xentropy_fwd_argmax", L.ptr(logits), L.ptr(labels), L.ptr(losses), L.ptr(lse), L.ptr(best), L.i64(n), L.i64(v),
+               L.i64(logits.stride(0)), L.f32(smoothing), pad, L.i32(L.dtype_code(logits)), L.stream_of(logits))
+    else:
+        L.call("nmtg_xentropy_fwd", L.ptr(logits), L.ptr(labels), L.ptr(losses), L.ptr(lse), L.i64(n), L.i64(v),
+               L.i64(logits.stride(0)), L.f32(smoothing), pad, L.i32(L.dtype_code(logits)), L.stream_of(logits))
     if not half_to_float and logits.dtype != torch.float32:
         lse = lse.to(logits.dtype)
-    return [losses, lse]
+    return [losses, lse, best] if want_argmax else [losses, lse]
 
 
 def backward(grad_loss, logits, max_log_sum_exp, labels, smoothing, *, padding_idx=None, out=None, class_offset=0,

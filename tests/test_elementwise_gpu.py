@@ -237,6 +237,50 @@ def test_xentropy_autograd_function(dev):
     assert_close(x.grad, oxe.xentropy_bwd(torch.ones(48), d["logits"], lseo, d["labels"], 0.1, 1, D), torch.bfloat16, "fn grad")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n,v", [(33, 4099), (7, 1), (5, 250054 // 4 + 3), (64, 32320)])
+def test_xentropy_argmax_follows_torch_argmax_bit_for_bit(dev, dtype, n, v):
+    # coarse values: every row holds its maximum several times, so the lowest-index rule decides (onmt/modules/loss.py:293-311
+    # takes torch.argmax of the logits); rows 1 and 2 hold NaN, which torch.argmax treats as the largest value
+    g = torch.Generator().manual_seed(41)
+    logits = torch.randint(-4, 5, (n, v), generator=g).to(dtype)
+    if n > 2 and v > 40:
+        logits[1, 37] = float("nan")
+        logits[2, 5] = float("nan")
+        logits[2, 31] = float("nan")
+        logits[0, :16] = float("-inf")
+    labels = torch.randint(0, v, (n,), generator=g)
+    x = logits.to(dev)
+    losses, lse, best = xentropy_cuda.forward(x, labels.to(dev), 0.0, dtype != torch.float32, padding_idx=-1, want_argmax=True)
+    assert best.dtype == torch.int64
+    assert torch.equal(best.cpu(), torch.argmax(logits.float(), dim=1))
+    assert torch.equal(best, torch.argmax(x, dim=1))
+    plain, lse2 = xentropy_cuda.forward(x, labels.to(dev), 0.0, dtype != torch.float32, padding_idx=-1)
+    assert torch.equal(plain.isnan(), losses.isnan()) and torch.equal(plain[~plain.isnan()], losses[~losses.isnan()])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_xentropy_leading_block_of_minus_infinity(dev, dtype):
+    # a masked vocabulary block: lanes that have only seen -inf must not produce NaN (the reference takes the row maximum
+    # first, xentropy_kernel.cu:382-474, so such a row has a finite loss there)
+    n, v = 9, 5000
+    d = inputs.xentropy_inputs(n, v, dtype, 0.0, padding_idx=1, pad_fraction=0.0, seed=43)
+    logits = d["logits"].clone()
+    logits[:, :2048] = float("-inf")
+    logits[3, 2048:] = float("-inf")
+    logits[3, 77] = 1.5                                       # one finite class inside the block
+    labels = torch.randint(2048, v, (n,), generator=torch.Generator().manual_seed(44))
+    labels[3] = 77
+    losses, lse = xentropy_cuda.forward(logits.to(dev), labels.to(dev), 0.0, dtype != torch.float32, padding_idx=1)
+    want, want_lse = oxe.xentropy_fwd(logits, labels, 0.0, 1, torch.float64)
+    assert torch.isfinite(losses).all()
+    assert_close(losses, want, torch.float32, "losses with a -inf block", rtol=2e-5, atol=2e-5)
+    assert_close(lse.float(), want_lse, torch.float32, "lse with a -inf block", rtol=2e-5, atol=2e-5)
+    grad = xentropy_cuda.backward(torch.ones(n, device=dev), logits.to(dev), lse, labels.to(dev), 0.0, padding_idx=1)
+    assert (grad[:, :2048].cpu()[torch.arange(n) != 3] == 0).all()
+    assert_close(grad, oxe.xentropy_bwd(torch.ones(n), logits, want_lse, labels, 0.0, 1, torch.float64), dtype, "gradient with a -inf block")
+
+
 def test_xentropy_errors(dev):
     x = torch.randn(4, 10, device=dev)
     with pytest.raises(RuntimeError):
