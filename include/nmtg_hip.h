@@ -296,6 +296,38 @@ int nmtg_encdec_attn_bwd(const void* grad_out, const void* ctx, const void* drop
                          void* grad_kv_lin, void* workspace, int64_t workspace_bytes, int64_t tq,
                          int64_t tk, int64_t b, int64_t e, int heads, int dtype, void* stream);
 
+/* The backward of the bias-free extension, which saves the softmax results instead of the scores:
+ * encdec_multihead_attn_cuda.backward(heads, output_grads, matmul2_results, dropout_results,
+ * softmax_results, input_lin_q_results, input_lin_kv_results, inputs_q, inputs_kv, weights..., dropout_mask, p)
+ * (call site onmt/modules/optimized/encdec_attention_func.py:322-345). As nmtg_encdec_attn_bwd with
+ * `softmax_results` [B*H, Tq, Tk] (pre-dropout probabilities) in place of `scores`; nothing is
+ * recomputed, there are no biases. Same workspace. */
+int nmtg_encdec_attn_bwd_from_probs(const void* grad_out, const void* ctx, const void* dropped,
+                                    const void* softmax_results, const void* q_lin,
+                                    const void* kv_lin, const void* x_q, const void* x_kv,
+                                    const void* w_q, const void* w_kv, const void* w_out,
+                                    const uint8_t* dropout_mask, float p, void* grad_x_q,
+                                    void* grad_x_kv, void* grad_w_q, void* grad_w_kv,
+                                    void* grad_w_out, void* grad_q_lin, void* grad_kv_lin,
+                                    void* workspace, int64_t workspace_bytes, int64_t tq,
+                                    int64_t tk, int64_t b, int64_t e, int heads, int dtype,
+                                    void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Rotary position encoding of queries / keys, in place, and its transpose (backward).
+ * Reference: apply_rotary_pos_emb / rotate_half / rotate_backward and their call sites
+ *   (onmt/modules/optimized/self_attention_func.py:25-48, :178-184, :467-469;
+ *   onmt/modules/optimized/encdec_attention_func.py:21-34), which run as PyTorch ops there.
+ * x[pos * stride_t + head * stride_n + part * stride_part + j], j < d (d even), pos < t, head < n,
+ * part < nparts (strides in elements): y = x cos + rotate_half(x) sin with cos, sin [t, d] in the
+ * dtype of x; inverse != 0 applies the transpose, dx = g cos + rotate_backward(sin g). The query
+ * and key slots of the head-interleaved projection [T, B*H, 3, D] are two parts of one call
+ * (stride_t = B*H*3*D, stride_n = 3*D, stride_part = D).
+ * ------------------------------------------------------------------------------------------ */
+int nmtg_rotary(void* x, const void* cos_table, const void* sin_table, int64_t t, int64_t n,
+                int64_t d, int64_t nparts, int64_t stride_t, int64_t stride_n, int64_t stride_part,
+                int inverse, int dtype, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Column sums of a row-major matrix: out[c] = sum_r x[r * ld + c], fp32 accumulation in a fixed
  * order (partial sums per block of rows, then one sum over the partials), result in the dtype

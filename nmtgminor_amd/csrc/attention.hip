@@ -90,9 +90,11 @@ int core_fwd(const Core& c, Strided q, Strided k, Strided v, const uint8_t* mask
 
 // From dctx: dv = Pd^T dctx;  dP = dctx v^T;  dS = softmax'(...);  dq = scale dS k;  dk = scale dS^T q.
 // ds_buf [bh, tq, tk] is scratch.
+// saved_probs: `scores` holds the softmax results instead of the masked scores (the bias-free reference extension saves
+// those, encdec_multihead_attn_cuda: onmt/modules/optimized/encdec_attention_func.py:81-105); nothing is recomputed then.
 int core_bwd(const Core& c, Strided q, Strided k, Strided v, Strided dctx, const void* scores, const void* dropped,
              const uint8_t* dmask, float p, void* ds_buf, void* dq, int64_t ld_dq, int64_t s_dq, void* dk, int64_t ld_dk,
-             int64_t s_dk, void* dv, int64_t ld_dv, int64_t s_dv) {
+             int64_t s_dk, void* dv, int64_t ld_dv, int64_t s_dv, bool saved_probs = false) {
   const int64_t tt = static_cast<int64_t>(c.tq) * c.tk;
   {  // dv [tk, d] = Pd^T [tk, tq] dctx [tq, d]
     GemmArgs g{};
@@ -110,7 +112,7 @@ int core_bwd(const Core& c, Strided q, Strided k, Strided v, Strided dctx, const
     g.C = ds_buf; g.ldc = c.tk; g.sC = tt;
     g.M = c.tq; g.N = c.tk; g.K = c.d; g.batch = c.bh; g.alpha = 1.f;
     int fused = 0;
-    if (!switched_off("NMTG_ATTN_FUSED")) {   // one-kernel form, see core_fwd
+    if (!saved_probs && !switched_off("NMTG_ATTN_FUSED")) {   // one-kernel form, see core_fwd
       GemmArgs f = g;
       f.aux_in = scores;
       f.dmask = drop ? dmask : nullptr;
@@ -120,7 +122,7 @@ int core_bwd(const Core& c, Strided q, Strided k, Strided v, Strided dctx, const
     }
     if (!fused) {
       if (int rc = gemm_run(c.dtype, LAYOUT_NT, EPI_PLAIN, g, nullptr, 0, c.st)) return rc;
-      if (int rc = nmtg_softmax_dropout_bwd(ds_buf, scores, 1, nullptr, 0, drop ? dmask : nullptr, drop ? 1 : 0,
+      if (int rc = nmtg_softmax_dropout_bwd(ds_buf, scores, saved_probs ? 0 : 1, nullptr, 0, drop ? dmask : nullptr, drop ? 1 : 0,
                                             drop ? p : 0.f, ds_buf, static_cast<int64_t>(c.bh) * c.tq, c.tk, c.tq, c.heads,
                                             c.dtype, c.st))
         return rc;
@@ -326,13 +328,14 @@ extern "C" int64_t nmtg_encdec_attn_bwd_workspace_bytes(int64_t tq, int64_t tk, 
   return static_cast<int64_t>(plan_ws(tq, tk, b, e, heads, false).total());
 }
 
-extern "C" int nmtg_encdec_attn_bwd(const void* grad_out, const void* ctx, const void* dropped, const void* scores,
-                                    const void* q_lin, const void* kv_lin, const void* x_q, const void* x_kv,
-                                    const void* w_q, const void* w_kv, const void* w_out, const uint8_t* dropout_mask,
-                                    float p, void* grad_x_q, void* grad_x_kv, void* grad_w_q, void* grad_w_kv,
-                                    void* grad_w_out, void* grad_b_q, void* grad_b_kv, void* grad_b_out, void* grad_q_lin,
-                                    void* grad_kv_lin, void* workspace, int64_t workspace_bytes, int64_t tq, int64_t tk,
-                                    int64_t b, int64_t e, int heads, int dtype, void* stream) {
+namespace {
+int encdec_attn_bwd_run(bool saved_probs, const void* grad_out, const void* ctx, const void* dropped, const void* scores,
+                        const void* q_lin, const void* kv_lin, const void* x_q, const void* x_kv,
+                        const void* w_q, const void* w_kv, const void* w_out, const uint8_t* dropout_mask,
+                        float p, void* grad_x_q, void* grad_x_kv, void* grad_w_q, void* grad_w_kv,
+                        void* grad_w_out, void* grad_b_q, void* grad_b_kv, void* grad_b_out, void* grad_q_lin,
+                        void* grad_kv_lin, void* workspace, int64_t workspace_bytes, int64_t tq, int64_t tk,
+                        int64_t b, int64_t e, int heads, int dtype, void* stream) {
   if (int rc = check_attn("encdec_attn_bwd", tq, tk, b, e, heads, dtype)) return rc;
   NMTG_REQUIRE(grad_out && dropped && scores && q_lin && kv_lin, "encdec_attn_bwd: null tensor");
   const bool compact = w_out == nullptr;
@@ -363,11 +366,37 @@ extern "C" int nmtg_encdec_attn_bwd(const void* grad_out, const void* ctx, const
   Strided q{q_lin, b * e, d}, k{kv_lin, b * 2 * e, 2 * d}, v{offset16(kv_lin, d), b * 2 * e, 2 * d};
   Strided dc{dctx_src, b * e, d};
   if (int rc = core_bwd(c, q, k, v, dc, scores, dropped, dropout_mask, p, ds, dq, b * e, d, dkv, b * 2 * e, 2 * d,
-                        offset16(dkv, d), b * 2 * e, 2 * d))
+                        offset16(dkv, d), b * 2 * e, 2 * d, saved_probs))
     return rc;
   if (compact) return 0;
   if (int rc = linear_bwd(dtype, dq, x_q, w_q, grad_x_q, grad_w_q, grad_b_q, tq * b, e, e, splitk_ws, ws.splitk, colsum_ws, st))
     return rc;
   return linear_bwd(dtype, dkv, x_kv, w_kv, grad_x_kv, grad_w_kv, grad_b_kv, tk * b, e, 2 * e, splitk_ws, ws.splitk, colsum_ws,
                     st);
+}
+}  // namespace
+
+extern "C" int nmtg_encdec_attn_bwd(const void* grad_out, const void* ctx, const void* dropped, const void* scores,
+                                    const void* q_lin, const void* kv_lin, const void* x_q, const void* x_kv,
+                                    const void* w_q, const void* w_kv, const void* w_out, const uint8_t* dropout_mask,
+                                    float p, void* grad_x_q, void* grad_x_kv, void* grad_w_q, void* grad_w_kv,
+                                    void* grad_w_out, void* grad_b_q, void* grad_b_kv, void* grad_b_out, void* grad_q_lin,
+                                    void* grad_kv_lin, void* workspace, int64_t workspace_bytes, int64_t tq, int64_t tk,
+                                    int64_t b, int64_t e, int heads, int dtype, void* stream) {
+  return encdec_attn_bwd_run(false, grad_out, ctx, dropped, scores, q_lin, kv_lin, x_q, x_kv, w_q, w_kv, w_out, dropout_mask, p,
+                             grad_x_q, grad_x_kv, grad_w_q, grad_w_kv, grad_w_out, grad_b_q, grad_b_kv, grad_b_out, grad_q_lin,
+                             grad_kv_lin, workspace, workspace_bytes, tq, tk, b, e, heads, dtype, stream);
+}
+
+extern "C" int nmtg_encdec_attn_bwd_from_probs(const void* grad_out, const void* ctx, const void* dropped,
+                                               const void* softmax_results, const void* q_lin, const void* kv_lin,
+                                               const void* x_q, const void* x_kv, const void* w_q, const void* w_kv,
+                                               const void* w_out, const uint8_t* dropout_mask, float p, void* grad_x_q,
+                                               void* grad_x_kv, void* grad_w_q, void* grad_w_kv, void* grad_w_out,
+                                               void* grad_q_lin, void* grad_kv_lin, void* workspace, int64_t workspace_bytes,
+                                               int64_t tq, int64_t tk, int64_t b, int64_t e, int heads, int dtype,
+                                               void* stream) {
+  return encdec_attn_bwd_run(true, grad_out, ctx, dropped, softmax_results, q_lin, kv_lin, x_q, x_kv, w_q, w_kv, w_out,
+                             dropout_mask, p, grad_x_q, grad_x_kv, grad_w_q, grad_w_kv, grad_w_out, nullptr, nullptr, nullptr,
+                             grad_q_lin, grad_kv_lin, workspace, workspace_bytes, tq, tk, b, e, heads, dtype, stream);
 }

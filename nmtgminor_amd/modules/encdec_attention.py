@@ -7,7 +7,7 @@ import torch
 from torch import nn
 from torch.nn import Parameter
 
-from .encdec_attention_func_bias import encdec_attn_bias_func
+from .encdec_attention_func import encdec_attn_func
 
 
 class EncdecMultiheadAttn(nn.Module):
@@ -26,7 +26,7 @@ class EncdecMultiheadAttn(nn.Module):
         self.register_parameter("in_proj_bias_q", None)
         self.register_parameter("in_proj_bias_kv", None)
         self.out_proj_bias = None
-        self.attn_func = encdec_attn_bias_func
+        self.attn_func = encdec_attn_func
         self.reset_parameters()
 
     def reset_parameters(self, init="normal"):
@@ -46,8 +46,9 @@ class EncdecMultiheadAttn(nn.Module):
         mask = attn_mask
         if mask is not None and mask.dim() == 3:
             mask = mask.squeeze(1)
+        # the bias-free function, as in the reference (encdec_attention.py:145-151): double precision off, coverage on;
+        # the coverage is the probabilities before dropout
         outputs, coverage = self.attn_func(False, self.training, self.num_heads, query, key, self.in_proj_weight_q,
-                                           self.in_proj_weight_kv, self.out_proj_weight, self.in_proj_bias_q,
-                                           self.in_proj_bias_kv, self.out_proj_bias, mask, self.dropout, incremental,
-                                           incremental_cache, rotary_pos_enc, pos_emb_q, pos_emb_k, True, True)
+                                           self.in_proj_weight_kv, self.out_proj_weight, mask, self.dropout, incremental,
+                                           incremental_cache, rotary_pos_enc, pos_emb_q, pos_emb_k, False, True)
         return outputs, coverage

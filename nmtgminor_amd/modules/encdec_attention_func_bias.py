@@ -3,7 +3,8 @@
 Mirrors EncdecAttnBiasFunc / encdec_attn_bias_func and the compact variant of the reference
 (onmt/modules/optimized/encdec_attention_func_bias.py:41-668, :687-1011): the same 20 positional
 arguments and 20 gradient slots; biases may be None (the reference then leaves its fused path,
-:69-73; here the fused path takes them). Rotary encoding raises; incremental decoding (inference with a cache
+:69-73; here the fused path takes them). Rotary encodings take the composed path of nmtgminor_amd/modules/rotary.py;
+incremental decoding (inference with a cache
 dict) runs in nmtgminor_amd/modules/incremental.py. A 21st
 optional argument replays an explicit dropout keep-mask."""
 import torch
@@ -71,6 +72,15 @@ def encdec_attn_bias_func(*args):
                 raise RuntimeError("encdec_attn_bias_func: incremental decoding needs an incremental_cache dict")
             outputs, probs = encdec_attn_step(heads, inputs_q, inputs_kv, w_q, w_kv, w_out, b_q, b_kv, b_out, mask, cache)
             return (outputs, probs) if args[19] else (outputs,)
+        if len(args) > 15 and args[15]:               # rotary position encodings
+            from .rotary import EncdecAttnRotaryFunc
+            (_, is_training, heads, inputs_q, inputs_kv, w_q, w_kv, w_out, b_q, b_kv, b_out, mask, p, _, _, _, pos_q,
+             pos_k) = args[:18]
+            if pos_q is None or pos_k is None:
+                raise RuntimeError("encdec_attn_bias_func: rotary_pos_enc needs pos_emb_q and pos_emb_k, each (cos, sin)")
+            r = EncdecAttnRotaryFunc.apply(is_training, heads, inputs_q, inputs_kv, w_q, w_kv, w_out, b_q, b_kv, b_out, mask, p,
+                                           pos_q[0], pos_q[1], pos_k[0], pos_k[1], args[20] if len(args) > 20 else None)
+            return r if args[19] else (r[0],)
         return EncdecAttnBiasFunc.apply(*args)
 
 

@@ -3,8 +3,8 @@
 Mirrors SelfAttnFunc / self_attn_func and SelfAttnCompactFunc / self_attn_compact_func of the
 reference (onmt/modules/optimized/self_attention_func.py:50-520, :523-837): the same 17
 positional arguments and 17 gradient slots. Every call takes the fused path (fp16 or bf16, biases
-optional, T <= 4096); what the HIP path does not cover (rotary position encoding) raises instead of
-falling back. Incremental decoding (inference, `incremental=True` with a cache dict) runs in
+optional, T <= 4096). Rotary position encodings take the composed path of nmtgminor_amd/modules/rotary.py (projection
+GEMM, rotation kernel, compact core); rotary together with incremental decoding raises. Incremental decoding (inference, `incremental=True` with a cache dict) runs in
 nmtgminor_amd/modules/incremental.py. As in the reference's fused branch the result is always
 the pair (outputs, dropout_results). An 18th optional argument replays an explicit dropout
 keep-mask."""
@@ -82,6 +82,14 @@ def self_attn_func(*args):
             if cache is None:
                 raise RuntimeError("self_attn_func: incremental decoding needs an incremental_cache dict")
             return self_attn_step(heads, inputs, w_in, w_out, b_in, b_out, mask, cache, bool(use_time_mask))
+        if len(args) > 11 and args[10]:               # rotary position encodings: projection, rotation, compact core
+            from .rotary import SelfAttnRotaryFunc
+            (use_time_mask, is_training, heads, inputs, w_in, w_out, b_in, b_out, mask, p, _, pos_emb) = args[:12]
+            if pos_emb is None:
+                raise RuntimeError("self_attn_func: rotary_pos_enc needs pos_emb = (cos, sin)")
+            cos, sin = pos_emb
+            return SelfAttnRotaryFunc.apply(use_time_mask, is_training, heads, inputs, w_in, w_out, b_in, b_out, mask, p, cos,
+                                            sin, args[17] if len(args) > 17 else None)
         return SelfAttnFunc.apply(*args)
 
 

@@ -25,7 +25,7 @@ def _shapes(q3, kv3, heads, kv_last):
 
 
 def _fwd(is_training, heads, x_q, x_kv, w_q, w_kv, w_out, b_q, b_kv, b_out, q_lin, kv_lin, pad_mask, p, dropout_mask,
-         tq, tk, b, e, dev, dt):
+         tq, tk, b, e, dev, dt, softmax_out=None):
     km, kind = A.mask_arg(pad_mask, False, b, tq, tk)
     bh = b * heads
     if q_lin is None:
@@ -40,7 +40,7 @@ def _fwd(is_training, heads, x_q, x_kv, w_q, w_kv, w_out, b_q, b_kv, b_out, q_li
     if tq == 0 or b == 0:       # an empty batch / no query position: the (empty) buffers are the result
         return q_lin, kv_lin, scores, dropped, dmask, ctx, out
     L.call("nmtg_encdec_attn_fwd", L.ptr(x_q), L.ptr(x_kv), L.ptr(w_q), L.ptr(w_kv), L.ptr(w_out), L.ptr(b_q), L.ptr(b_kv),
-           L.ptr(b_out), L.ptr(km), L.ptr(q_lin), L.ptr(kv_lin), L.ptr(scores), L.ptr(None), L.ptr(dropped),
+           L.ptr(b_out), L.ptr(km), L.ptr(q_lin), L.ptr(kv_lin), L.ptr(scores), L.ptr(softmax_out), L.ptr(dropped),
            L.ptr(dmask if mode else None), L.i32(mode), L.f32(p), A.u64(seed), A.u64(offset), L.ptr(ctx), L.ptr(out),
            L.i64(tq), L.i64(tk), L.i64(b), L.i64(e), L.i32(heads), L.i32(L.dtype_code(ctx)), L.stream_of(ctx))
     return q_lin, kv_lin, scores, dropped, dmask, ctx, out
@@ -106,7 +106,9 @@ def forward_compact(is_training, heads, input_lin_q_results, input_lin_kv_result
 
 
 def _bwd(heads, output_grads, matmul2_results, dropout_results, attn_scores, q_lin, kv_lin, inputs_q, inputs_kv, w_q, w_kv,
-         w_out, dropout_mask, p, want_weights=True, want_biases=True):
+         w_out, dropout_mask, p, want_weights=True, want_biases=True, from_probs=False):
+    """from_probs: `attn_scores` holds the softmax results (what the bias-free extension saves); no bias gradients."""
+    want_biases = want_biases and not from_probs
     L.require_cuda(output_grads, dropout_results, attn_scores, q_lin, kv_lin, inputs_q, inputs_kv, w_q, w_kv, w_out)
     A.check_half(output_grads, dropout_results, attn_scores, q_lin, kv_lin, inputs_q, inputs_kv, w_q, w_kv, w_out)
     tq, tk, b, e = _shapes(q_lin, kv_lin, heads, 2)
@@ -141,6 +143,13 @@ def _bwd(heads, output_grads, matmul2_results, dropout_results, attn_scores, q_l
     (matmul2_results, dropout_results, attn_scores, q_lin, kv_lin, inputs_q, inputs_kv, w_q, w_kv, w_out) = map(
         c, (matmul2_results, dropout_results, attn_scores, q_lin, kv_lin, inputs_q, inputs_kv, w_q, w_kv, w_out))
     dropout_mask = c(dropout_mask) if use_mask else None
+    if from_probs:
+        L.call("nmtg_encdec_attn_bwd_from_probs", L.ptr(g), L.ptr(matmul2_results), L.ptr(dropout_results), L.ptr(attn_scores),
+               L.ptr(q_lin), L.ptr(kv_lin), L.ptr(inputs_q), L.ptr(inputs_kv), L.ptr(w_q), L.ptr(w_kv),
+               L.ptr(w_out), L.ptr(dropout_mask), L.f32(p), L.ptr(n["dxq"]), L.ptr(n["dxkv"]),
+               L.ptr(n["dwq"]), L.ptr(n["dwkv"]), L.ptr(n["dwo"]), L.ptr(n["dq"]), L.ptr(n["dkv"]), L.ptr(ws), L.i64(ws.numel()),
+               L.i64(tq), L.i64(tk), L.i64(b), L.i64(e), L.i32(heads), L.i32(L.dtype_code(g)), L.stream_of(g))
+        return n
     L.call("nmtg_encdec_attn_bwd", L.ptr(g), L.ptr(matmul2_results), L.ptr(dropout_results), L.ptr(attn_scores),
            L.ptr(q_lin), L.ptr(kv_lin), L.ptr(inputs_q), L.ptr(inputs_kv), L.ptr(w_q), L.ptr(w_kv),
            L.ptr(w_out), L.ptr(dropout_mask), L.f32(p), L.ptr(n["dxq"]), L.ptr(n["dxkv"]),

@@ -104,7 +104,7 @@ def test_self_attention_rng_dropout_eval_and_no_bias(dev):
     assert dmask.shape == (b * h, t, t) and abs(dmask.float().mean().item() - 0.7) < 0.02
     fwd2 = oat.self_attn_fwd(d["x"], d["w_in"], d["w_out"], None, None, h, d["pad_mask"], None, 0.3, dmask.cpu(), D, round_to=dtype)
     assert_close(r[5], fwd2["outputs"], dtype, "rng dropout outputs")
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(RuntimeError):            # rotary encodings without their (cos, sin) tables
         self_attn_func(False, False, h, g("x"), g("w_in"), g("w_out"), None, None, None, 0.0, True, None, False, None, True, True, False)
     with pytest.raises(RuntimeError):
         sa_native.forward(False, False, h, g("x").float(), g("w_in").float(), g("w_out").float(), None, None, None, 0.0)
@@ -155,6 +155,108 @@ def test_encdec_attention_without_biases_and_compact(dev):
     assert torch.equal(ctx2, ctx) and torch.equal(cov2, dropped)
     dq, dkv = ed_native.backward_compact(4, d["dout"].to(dev), dropped, scores, q_lin, kv_lin, dmask, 0.1)
     assert dq.shape == q_lin.shape and dkv.shape == kv_lin.shape and torch.isfinite(dq.float()).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("tq,tk,b,e,h,p,recompute", [(48, 300, 2, 256, 4, 0.1, False), (33, 512, 3, 128, 2, 0.25, True),
+                                                     (16, 70, 2, 128, 2, 0.0, False)])
+def test_bias_free_encdec_function_returns_the_pre_dropout_probabilities(dev, dtype, tq, tk, b, e, h, p, recompute):
+    # EncdecAttnFunc (onmt/modules/optimized/encdec_attention_func.py:36-568): 17 arguments, no biases; its fused branch
+    # hands back softmax_results as coverage (:123-124) and its backward starts from them (:322-345)
+    from nmtgminor_amd.modules.encdec_attention_func import encdec_attn_func
+    from nmtgminor_amd.native import encdec_multihead_attn_cuda as free_native
+    d = inputs.encdec_attn_inputs(tq, tk, b, e, h, dtype, p=p, seed=75, zero_bias=False)
+    fwd = oat.encdec_attn_fwd(d["x_q"], d["x_kv"], d["w_q"], d["w_kv"], d["w_out"], None, None, None, h, d["pad_mask"], p,
+                              d["dropout_mask"], D, round_to=dtype)
+    # this backward starts from the probabilities as stored (rounded to 16 bits), not from the scores
+    saved = dict(fwd, softmax_results=fwd["softmax_results"].to(dtype).to(D))
+    bwd = oat.encdec_attn_bwd(d["dout"], d["x_q"], d["x_kv"], d["w_q"], d["w_kv"], d["w_out"], h, saved, p, d["dropout_mask"], D,
+                              round_to=dtype)
+    names = ("x_q", "x_kv", "w_q", "w_kv", "w_out")
+    leaf = {k: d[k].to(dev).requires_grad_() for k in names}
+    dm = d["dropout_mask"].to(dev) if p > 0 else None
+    mask3 = d["pad_mask"].to(dev).unsqueeze(1)                     # the broadcast form the reference's callers pass
+    out, cov = encdec_attn_func(recompute, True, h, leaf["x_q"], leaf["x_kv"], leaf["w_q"], leaf["w_kv"], leaf["w_out"], mask3, p,
+                                False, None, False, None, None, False, True, dm)
+    out.backward(d["dout"].to(dev))
+    assert_close(out, fwd["outputs"], dtype, "outputs")
+    assert_close(cov, fwd["softmax_results"], dtype, "coverage = probabilities before dropout")
+    if p > 0:
+        assert not torch.equal(cov.cpu() == 0, fwd["dropout_results"].to(dtype) == 0)      # no dropped units in it
+    assert_close(cov.float().sum(-1), torch.ones(b * h, tq), dtype, "rows sum to one", atol=2e-2)
+    for key, n in (("dx_q", "x_q"), ("dx_kv", "x_kv"), ("dw_q", "w_q"), ("dw_kv", "w_kv"), ("dw_out", "w_out")):
+        assert_close(leaf[n].grad, bwd[key], dtype, key, scale_atol=True)
+    # the extension's own lists
+    r = free_native.forward(True, h, d["x_q"].to(dev), d["x_kv"].to(dev), d["w_q"].to(dev), d["w_kv"].to(dev), d["w_out"].to(dev),
+                            d["pad_mask"].to(dev), p, dropout_mask=dm)
+    assert len(r) == 7 and r[2].shape == (b * h, tq, tk) and torch.equal(r[2], cov)
+    g = free_native.backward(h, d["dout"].to(dev), r[5], r[3], r[2], r[0], r[1], d["x_q"].to(dev), d["x_kv"].to(dev),
+                             d["w_q"].to(dev), d["w_kv"].to(dev), d["w_out"].to(dev), r[4], p)
+    assert len(g) == 5
+    assert_close(g[3], bwd["dw_kv"], dtype, "dw_kv from the extension's backward", scale_atol=True)
+    out1 = encdec_attn_func(False, False, h, d["x_q"].to(dev), d["x_kv"].to(dev), d["w_q"].to(dev), d["w_kv"].to(dev),
+                            d["w_out"].to(dev), None, p, False, None, False, None, None, False, False)
+    assert isinstance(out1, tuple) and len(out1) == 1
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("t,b,e,h,causal", [(40, 2, 128, 2, False), (64, 3, 256, 4, True)])
+def test_self_attention_with_rotary_position_encodings(dev, dtype, t, b, e, h, causal):
+    # self_attn_func with rotary_pos_enc = True and pos_emb = (cos, sin) [T, 1, D] (self_attention_func.py:178-184, :467-469)
+    from oracle import rotary as orot
+    d = inputs.self_attn_inputs(t, b, e, h, dtype, p=0.0, seed=76, causal=causal, zero_bias=False)
+    cos, sin = orot.tables(torch.arange(t), e // h)
+    cos, sin = cos.to(dtype), sin.to(dtype)
+    names = ("x", "w_in", "w_out", "b_in", "b_out")
+    leaf = {k: d[k].to(dev).requires_grad_() for k in names}
+    mask = d["time_mask"] if causal else d["pad_mask"]
+    out, cov = self_attn_func(causal, True, h, leaf["x"], leaf["w_in"], leaf["w_out"], leaf["b_in"], leaf["b_out"], mask.to(dev), 0.0,
+                              True, (cos.to(dev), sin.to(dev)), False, None, True, True, False)
+    out.backward(d["dout"].to(dev))
+    ref = {k: d[k].to(D).requires_grad_() for k in names}
+    want, wcov = orot.self_attn_rotary(ref["x"], ref["w_in"], ref["w_out"], ref["b_in"], ref["b_out"], h,
+                                       None if causal else d["pad_mask"], d["time_mask"] if causal else None, cos.to(D), sin.to(D),
+                                       round_to=dtype)
+    want.backward(d["dout"].to(D))
+    assert_close(out, want.detach(), dtype, "outputs")
+    assert_close(cov, wcov.detach(), dtype, "coverage")
+    for k in names:
+        assert_close(leaf[k].grad, ref[k].grad, dtype, "d " + k, scale_atol=True)
+    # the rotation kernel alone, forward then transposed, on the strided head slots
+    from nmtgminor_amd.native import rotary_position as rot
+    lin = torch.randn(t, b, 3 * e, generator=torch.Generator().manual_seed(77)).to(dtype)
+    got = rot.rotate_qk_(lin.clone().to(dev), cos.to(dev), sin.to(dev), b * h, e // h)
+    v4 = lin.to(D).view(t, b * h, 3, e // h)
+    assert_close(got.view(t, b * h, 3, -1)[:, :, 0], orot.apply_rotary(v4[:, :, 0], cos.to(D), sin.to(D)), dtype, "rotated q")
+    assert_close(got.view(t, b * h, 3, -1)[:, :, 1], orot.apply_rotary(v4[:, :, 1], cos.to(D), sin.to(D)), dtype, "rotated k")
+    assert torch.equal(got.view(t, b * h, 3, -1)[:, :, 2].cpu(), lin.view(t, b * h, 3, -1)[:, :, 2])      # values untouched
+    back = rot.rotate_qk_(lin.clone().to(dev), cos.to(dev), sin.to(dev), b * h, e // h, inverse=True)
+    assert_close(back.view(t, b * h, 3, -1)[:, :, 1], orot.apply_rotary_transposed(v4[:, :, 1], cos.to(D), sin.to(D)), dtype,
+                 "transposed rotation")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_encdec_attention_with_rotary_position_encodings(dev, dtype):
+    from nmtgminor_amd.modules.encdec_attention_func import encdec_attn_func
+    from oracle import rotary as orot
+    tq, tk, b, e, h = 24, 70, 2, 128, 2
+    d = inputs.encdec_attn_inputs(tq, tk, b, e, h, dtype, p=0.0, seed=78, zero_bias=False)
+    cq, sq = (z.to(dtype) for z in orot.tables(torch.arange(tq), e // h))
+    ck, sk = (z.to(dtype) for z in orot.tables(torch.arange(tk), e // h))
+    names = ("x_q", "x_kv", "w_q", "w_kv", "w_out")
+    leaf = {k: d[k].to(dev).requires_grad_() for k in names}
+    out, cov = encdec_attn_func(False, True, h, leaf["x_q"], leaf["x_kv"], leaf["w_q"], leaf["w_kv"], leaf["w_out"],
+                                d["pad_mask"].to(dev), 0.0, False, None, True, (cq.to(dev), sq.to(dev)), (ck.to(dev), sk.to(dev)),
+                                False, True)
+    out.backward(d["dout"].to(dev))
+    ref = {k: d[k].to(D).requires_grad_() for k in names}
+    want, wcov = orot.encdec_attn_rotary(ref["x_q"], ref["x_kv"], ref["w_q"], ref["w_kv"], ref["w_out"], h, d["pad_mask"],
+                                         cq.to(D), sq.to(D), ck.to(D), sk.to(D), round_to=dtype)
+    want.backward(d["dout"].to(D))
+    assert_close(out, want.detach(), dtype, "outputs")
+    assert_close(cov, wcov.detach(), dtype, "coverage")
+    for k in names:
+        assert_close(leaf[k].grad, ref[k].grad, dtype, "d " + k, scale_atol=True)
 
 
 def test_modules_state_dict_names_and_forward(dev):

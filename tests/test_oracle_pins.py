@@ -597,3 +597,68 @@ def test_zipf_targets_and_masks_are_seeded():
     counts = torch.bincount(a["labels"], minlength=1000)
     counts[1] = 0
     assert int(counts.argmax()) == 0
+
+
+# ----------------------------------------------------------------------------- rotary position encoding
+def test_rotary_rotation_is_orthogonal_relative_and_its_backward_is_the_transpose():
+    from oracle import rotary as orot
+    g = torch.Generator().manual_seed(401)
+    t, n, d = 9, 3, 16
+    cos, sin = orot.tables(torch.arange(t), d)
+    x = torch.randn(t, n, d, generator=g, dtype=D)
+    y = orot.apply_rotary(x, cos, sin)
+    h = d // 2
+    # a plane rotation of every pair (j, j + D/2): the pair's norm is kept, and by hand for one element
+    assert torch.allclose(x[..., :h] ** 2 + x[..., h:] ** 2, y[..., :h] ** 2 + y[..., h:] ** 2, atol=1e-12)
+    i, j = 4, 3
+    want = x[i, 1, j] * cos[i, 0, j] - x[i, 1, j + h] * sin[i, 0, j]
+    assert abs(y[i, 1, j] - want) < 1e-12
+    want = x[i, 1, j + h] * cos[i, 0, j + h] + x[i, 1, j] * sin[i, 0, j + h]
+    assert abs(y[i, 1, j + h] - want) < 1e-12
+    # the property rotary encodings exist for: <rot(q, m), rot(k, n)> depends on m - n only
+    q, k = torch.randn(d, generator=g, dtype=D), torch.randn(d, generator=g, dtype=D)
+    rq = orot.apply_rotary(q.expand(t, 1, d), cos, sin)[:, 0]
+    rk = orot.apply_rotary(k.expand(t, 1, d), cos, sin)[:, 0]
+    s = rq @ rk.t()
+    for delta in (0, 1, 3):
+        diag = torch.diagonal(s, -delta)
+        assert torch.allclose(diag, diag[0].expand_as(diag), atol=1e-10)
+    assert not torch.allclose(torch.diagonal(s, 0)[0], torch.diagonal(s, -1)[0])
+    # the gradient rule of the reference is the transpose of the forward map: <A x, g> == <x, A^T g>, and autograd agrees
+    gr = torch.randn(t, n, d, generator=g, dtype=D)
+    assert abs((y * gr).sum() - (x * orot.apply_rotary_transposed(gr, cos, sin)).sum()) < 1e-10
+    xr = x.clone().requires_grad_()
+    orot.apply_rotary(xr, cos, sin).backward(gr)
+    assert torch.allclose(xr.grad, orot.apply_rotary_transposed(gr, cos, sin), atol=1e-12)
+
+
+def test_rotary_attention_reduces_to_plain_attention_at_angle_zero_and_to_a_per_head_loop():
+    from oracle import rotary as orot
+    d_in = inputs.self_attn_inputs(12, 2, 32, 2, torch.float32, p=0.0, seed=402, zero_bias=False)
+    x, w_in, w_out, b_in, b_out = (d_in[k].to(D) for k in ("x", "w_in", "w_out", "b_in", "b_out"))
+    one, zero = torch.ones(12, 1, 16, dtype=D), torch.zeros(12, 1, 16, dtype=D)
+    # angle zero: the plain attention oracle (itself pinned against nn.MultiheadAttention above)
+    out, cov = orot.self_attn_rotary(x, w_in, w_out, b_in, b_out, 2, d_in["pad_mask"], None, one, zero)
+    plain = attention.self_attn_fwd(x, w_in, w_out, b_in, b_out, 2, d_in["pad_mask"], None, 0.0, None, D)
+    assert torch.allclose(out, plain["outputs"], atol=1e-12) and torch.allclose(cov, plain["dropout_results"], atol=1e-12)
+    # one (batch, head) by hand: rotate its queries and keys, softmax(q k^T / sqrt(D)) v, against the batched form
+    cos, sin = orot.tables(torch.arange(12), 16)
+    out2, cov2 = orot.self_attn_rotary(x, w_in, w_out, b_in, b_out, 2, None, None, cos, sin)
+    lin = (x.reshape(24, 32) @ w_in.t() + b_in).view(12, 2, 2, 3, 16)        # [T, B, H, {q,k,v}, D]
+    b_i, h_i = 1, 0
+    q = orot.apply_rotary(lin[:, b_i, h_i, 0][:, None], cos, sin)[:, 0]
+    k = orot.apply_rotary(lin[:, b_i, h_i, 1][:, None], cos, sin)[:, 0]
+    probs = torch.softmax(q @ k.t() / 4.0, -1)
+    assert torch.allclose(cov2[b_i * 2 + h_i], probs, atol=1e-12)
+    ctx = (out2 - b_out).reshape(24, 32) @ torch.linalg.inv(w_out.t())         # undo the output projection
+    assert torch.allclose(ctx.view(12, 2, 2, 16)[:, b_i, h_i], probs @ lin[:, b_i, h_i, 2], atol=1e-9)
+    # the cross-attention form rotates queries and keys with their own tables
+    de = inputs.encdec_attn_inputs(5, 9, 2, 32, 2, torch.float32, p=0.0, seed=403, zero_bias=False)
+    cq, sq = orot.tables(torch.arange(5), 16)
+    ck, sk = orot.tables(torch.arange(9), 16)
+    oe, ce = orot.encdec_attn_rotary(de["x_q"], de["x_kv"], de["w_q"], de["w_kv"], de["w_out"], 2, None, cq, sq, ck, sk)
+    ql = (de["x_q"].to(D).reshape(10, 32) @ de["w_q"].to(D).t()).view(5, 2, 2, 16)
+    kl = (de["x_kv"].to(D).reshape(18, 32) @ de["w_kv"].to(D).t()).view(9, 2, 2, 2, 16)
+    q = orot.apply_rotary(ql[:, 0, 1][:, None], cq, sq)[:, 0]
+    k = orot.apply_rotary(kl[:, 0, 1, 0][:, None], ck, sk)[:, 0]
+    assert torch.allclose(ce[1], torch.softmax(q @ k.t() / 4.0, -1), atol=1e-12)
