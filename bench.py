@@ -305,6 +305,62 @@ class SelfAttnWL(Workload):
                     kind="port", sample=f"{nb} of {self.B} batch columns (independent), fp32 on the bf16-rounded values, median of 3")
 
 
+class FlashAttnWL(Workload):
+    name = "flash_attn"
+    bound = "mfma"
+    dtype = "bf16"
+    description = ("attention core over packed sequences fwd+bwd bf16 (no [heads, T, T] tensor): 32 sequences of lengths "
+                   "U[256,512] packed as [tokens, 3, 16 heads, 64], softmax dropout 0.1 drawn on the device")
+    B, H, D, P = 32, 16, 64, 0.1
+
+    def setup(self, dev):
+        from nmtgminor_amd.native import flash_attn_cuda as m
+        self.m = m
+        g = torch.Generator().manual_seed(5)
+        self.lens = torch.randint(256, 513, (self.B,), generator=g).tolist()
+        cu = torch.zeros(self.B + 1, dtype=torch.int32)
+        cu[1:] = torch.cumsum(torch.tensor(self.lens), 0)
+        total = int(cu[-1])
+        self.cpu = dict(qkv=torch.randn(total, 3, self.H, self.D, generator=g).to(torch.bfloat16),
+                        dout=torch.randn(total, self.H, self.D, generator=g).to(torch.bfloat16), cu=cu)
+        self.qkv, self.dout, self.cu = self.cpu["qkv"].to(dev), self.cpu["dout"].to(dev), cu.to(dev)
+        self.out = torch.empty_like(self.dout)
+        self.dqkv = torch.empty_like(self.qkv)
+        self.max_len = max(self.lens)
+        self.scale = self.D ** -0.5
+
+    def step(self):
+        q, k, v = self.qkv[:, 0], self.qkv[:, 1], self.qkv[:, 2]
+        lse, = self.m.fwd(q, k, v, self.out, self.cu, self.cu, self.max_len, self.max_len, self.P, self.scale, False, False,
+                          False)
+        return self.m.bwd(self.dout, q, k, v, self.out, lse, self.dqkv[:, 0], self.dqkv[:, 1], self.dqkv[:, 2], self.cu, self.cu,
+                          self.max_len, self.max_len, self.P, self.scale, False, False)
+
+    def _flops_fwd(self):
+        return sum(2 * 2.0 * self.H * n * n * self.D for n in self.lens)        # Q K^T and P V per sequence and head
+
+    def work_per_step(self):
+        return 3 * self._flops_fwd()                                            # backward: dP, dV, dQ, dK
+
+    def kernel_work(self):
+        return {"flash_attn_fwd": self._flops_fwd(), "flash_attn_bwd": 2 * self._flops_fwd()}
+
+    def cpu_baseline(self):
+        from oracle import flash_attention as o
+        nb = 2
+        cu = self.cpu["cu"][:nb + 1]
+        n = int(cu[-1])
+        qkv, dout = self.cpu["qkv"][:n].float(), self.cpu["dout"][:n].float()
+        keep = (torch.rand(nb, self.H, self.max_len, self.max_len, generator=torch.Generator().manual_seed(6)) >= self.P).to(torch.uint8)
+
+        def run():
+            o.flash_attn_bwd(dout, qkv[:, 0], qkv[:, 1], qkv[:, 2], cu, cu, self.max_len, None, False, self.P, keep, torch.float32)
+        t = _time_cpu(run, 3)
+        work = 3 * sum(2 * 2.0 * self.H * x * x * self.D for x in self.lens[:nb])
+        return dict(value=work / t / 1e12, unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
+                    sample=f"{nb} of {self.B} sequences (independent), fp32 on the bf16-rounded values, forward + autograd backward, median of 3")
+
+
 class RelSelfAttnWL(Workload):
     name = "rel_self_attn"
     bound = "mfma"
@@ -642,7 +698,7 @@ class CopyWL(Workload):
 
 # the five benchmark configurations first, then the workloads added beside them
 WORKLOADS = {w.name: w for w in (LayerNormWL, MlpWL, SelfAttnWL, EncdecAttnWL, XentropyWL, SoftmaxDropoutWL, DropoutAddWL,
-                                    GeneratorLossWL, RelSelfAttnWL, FusedAdamWL, LayerNormLargeWL)}
+                                    GeneratorLossWL, RelSelfAttnWL, FusedAdamWL, LayerNormLargeWL, FlashAttnWL)}
 EXTRA_WORKLOADS = {CopyWL.name: CopyWL}
 PRIMARY = "mlp"
 

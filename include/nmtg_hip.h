@@ -329,6 +329,53 @@ int nmtg_rotary(void* x, const void* cos_table, const void* sin_table, int64_t t
                 int inverse, int dtype, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Attention over packed variable-length sequences without a [heads, len_q, len_k] tensor.
+ * Reference: flash_attn_cuda.fwd / .bwd as bound at onmt/modules/optimized/flash_mha.py:43-75
+ *   (callers FlashAttnQKVPackedFunc / FlashAttnKVPackedFunc :104-183,
+ *   onmt/models/speech_recognizer/whisper_encoder.py:329-356).
+ * q [total_q, heads, head_dim], k / v [total_k, heads, head_dim], out like q: 16-bit views with a
+ * contiguous head_dim (64 or 128), token and head strides in elements (multiples of 8), 16-byte
+ * aligned (the slots of a packed [total, 3, heads, head_dim] projection qualify). Sequence b owns
+ * tokens cu_seqlens[b] .. cu_seqlens[b+1]-1 (device int32 [batch + 1]); lengths must not exceed
+ * max_seqlen_q / max_seqlen_k (longer ones are cut there). Per sequence and head:
+ *   P = softmax_rows(softmax_scale * Q K^T)   (1e-6 <= |softmax_scale| <= 1e6; causal: keys j > i
+ *   masked, aligned at the first token of both), out = (keep * P * dropout_scale) V, softmax_lse [batch, heads, max_seqlen_q]
+ *   = log sum exp of the scaled scores (fp32; entries past a sequence's length are not written;
+ *   -inf for a sequence without keys, whose out rows are 0).
+ * dropout_mode 0: none. 1: replay dropout_mask (uint8 keep flags [batch, heads, max_seqlen_q,
+ * max_seqlen_k]), scale 1 / (1 - p). 2: draw from Philox (seed, offset): element (i, j) is kept when
+ * byte 4 (i % 4) + (j % 4) of block ((b heads + h) ceil(max_q / 4) + i / 4) ceil(max_k / 4) + j / 4
+ * is below t = round(256 (1 - p)), scale 256 / t; dropout_mask_out, when not null, receives the
+ * keep flags in the layout of dropout_mask. The backward regenerates the same mask from the same
+ * (seed, offset).
+ * nmtg_flash_attn_bwd: dq, dk, dv in views like q, k, v (every row of every sequence written),
+ * softmax_d [batch, heads, max_seqlen_q] = rowsum(dout * out) (fp32, written). Deterministic: no
+ * atomics.
+ * ------------------------------------------------------------------------------------------ */
+int nmtg_flash_attn_fwd(const void* q, const void* k, const void* v, void* out,
+                        const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, float* softmax_lse,
+                        int64_t batch, int64_t heads, int64_t head_dim, int64_t max_seqlen_q,
+                        int64_t max_seqlen_k, int64_t q_stride_t, int64_t q_stride_h,
+                        int64_t k_stride_t, int64_t k_stride_h, int64_t v_stride_t, int64_t v_stride_h,
+                        int64_t out_stride_t, int64_t out_stride_h, float softmax_scale, int causal,
+                        int dropout_mode, float dropout_p, const uint8_t* dropout_mask,
+                        uint8_t* dropout_mask_out, uint64_t seed, uint64_t offset, int dtype,
+                        void* stream);
+
+int nmtg_flash_attn_bwd(const void* dout, const void* q, const void* k, const void* v,
+                        const void* out, const float* softmax_lse, void* dq, void* dk, void* dv,
+                        float* softmax_d, const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k,
+                        int64_t batch, int64_t heads, int64_t head_dim, int64_t max_seqlen_q,
+                        int64_t max_seqlen_k, int64_t dout_stride_t, int64_t dout_stride_h,
+                        int64_t q_stride_t, int64_t q_stride_h, int64_t k_stride_t, int64_t k_stride_h,
+                        int64_t v_stride_t, int64_t v_stride_h, int64_t out_stride_t,
+                        int64_t out_stride_h, int64_t dq_stride_t, int64_t dq_stride_h,
+                        int64_t dk_stride_t, int64_t dk_stride_h, int64_t dv_stride_t,
+                        int64_t dv_stride_h, float softmax_scale, int causal, int dropout_mode,
+                        float dropout_p, const uint8_t* dropout_mask, uint64_t seed, uint64_t offset,
+                        int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Column sums of a row-major matrix: out[c] = sum_r x[r * ld + c], fp32 accumulation in a fixed
  * order (partial sums per block of rows, then one sum over the partials), result in the dtype
  * of x. The bias gradients of the reference's linear layers: torch.sum(grads, 0)

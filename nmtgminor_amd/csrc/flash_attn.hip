@@ -1,0 +1,843 @@
+// Attention over packed variable-length sequences without the [heads, len_q, len_k] score tensor: what the reference
+// gets from the third-party module flash_attn_cuda (onmt/modules/optimized/flash_mha.py:32-75: fwd / bwd over
+// [total_tokens, heads, head_dim] tensors with cumulative sequence lengths).
+//
+// Forward, one block per (sequence, head, 128 queries), four wavefronts of 32 queries each:
+//   the wavefront's query rows stay in registers as MFMA operands; keys and values arrive in tiles of 64 keys through
+//   LDS (loaded into registers one tile ahead, two LDS buffers, one barrier per tile);
+//   S^T = K Q^T on v_mfma_f32_32x32x16 puts one query per lane pair (l, l ^ 32) and 32 of the tile's 64 keys in each
+//   lane's accumulators, so the running maximum and sum of the online softmax are per-lane scalars;
+//   the probabilities are rounded to the 16-bit type, moved from accumulator to operand layout with two
+//   v_permlane32_swap per 16 keys, and multiplied with V^T, read from LDS with the transposing read.
+// Backward, two kernels with the same tiling, both recomputing S from Q, K and the saved log-sum-exp:
+//   dQ kernel  (block = 128 queries, loop over key tiles): D = rowsum(dO * O), dP^T = V dO^T, dS = P (dP - D),
+//              dQ^T += K^T dS^T;
+//   dK/dV kernel (block = 128 keys, loop over query tiles of 64): the mirror image with one key per lane pair:
+//              dV^T += dO^T P, dK^T += Q^T dS.
+//   No atomics and no accumulation across blocks: results do not depend on scheduling.
+// Dropout keeps element (query i, key j) of (sequence b, head h) when byte 4 (i % 4) + (j % 4) of the Philox block with
+// index ((b H + h) ceil(max_q / 4) + i / 4) ceil(max_k / 4) + j / 4 is below round(256 (1 - p)); kept probabilities are
+// scaled by 256 / that threshold, so the expectation is exact although p is quantised to 1/256. A 4 x 4 patch per
+// block serves both tilings (a lane holds four consecutive keys of one query in one, four consecutive queries of one
+// key in the other); the four lanes that share a patch split the generator calls between them (one call per 16 elements).
+#include "gemm.cuh"
+
+namespace nmtg {
+namespace {
+
+constexpr int FA_ROWS = 128;   // queries (forward, dQ) or keys (dK/dV) per block: 32 per wavefront
+constexpr int FA_TILE = 64;    // rows of the streamed operand per LDS tile
+constexpr int FA_THREADS = 256;
+constexpr float FA_NEG = -1e30f;
+constexpr float FA_LAZY = 8.f;   // log2 of the growth of a row maximum that moves the softmax's reference point
+constexpr float FA_LOG2E = 1.4426950408889634f;
+
+struct FaArgs {
+  const void *q, *k, *v, *o, *d_o;
+  void *out, *dq, *dk, *dv;
+  float* lse;      // [B, H, max_q]
+  float* delta;    // [B, H, max_q]
+  const int32_t *cu_q, *cu_k;
+  int64_t q_st, q_sh, k_st, k_sh, v_st, v_sh, o_st, o_sh, do_st, do_sh, dq_st, dq_sh, dk_st, dk_sh, dv_st, dv_sh;
+  int heads, max_q, max_k;
+  float scale, scale_log2;
+  int causal;
+  const uint8_t* mask;   // explicit keep-mask [B, H, max_q, max_k] (DROP == 1)
+  uint8_t* mask_out;     // where the drawn mask is written, or null (DROP == 2)
+  uint32_t thr;          // keep when byte < thr (DROP == 2)
+  float drop_scale;
+  uint64_t seed, offset;
+};
+
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+
+// lanes 32..63 of `a` change places with lanes 0..31 of `b`
+__device__ __forceinline__ void swap_halves(uint32_t& a, uint32_t& b) {
+  const u32x2_t r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+  a = r[0];
+  b = r[1];
+}
+// f(own value, value of lane ^ 32)
+__device__ __forceinline__ float pair_max(float v) {
+  uint32_t a = __float_as_uint(v), b = a;
+  swap_halves(a, b);
+  return fmaxf(__uint_as_float(a), __uint_as_float(b));
+}
+__device__ __forceinline__ float pair_sum(float v) {
+  uint32_t a = __float_as_uint(v), b = a;
+  swap_halves(a, b);
+  return __uint_as_float(a) + __uint_as_float(b);
+}
+
+// two floats rounded (to nearest even) into one register of two 16-bit elements, one conversion instruction
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+template <typename T> struct pair_of;
+template <> struct pair_of<f16_t> { typedef _Float16 type __attribute__((ext_vector_type(2))); };
+template <> struct pair_of<bf16_t> { typedef __bf16 type __attribute__((ext_vector_type(2))); };
+template <typename T>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, typename pair_of<T>::type));
+}
+
+// Accumulator registers r0 .. r0+7 of a 32 x 32 tile (lane (col, half) holds rows 8 (r / 4) + 4 half + r % 4) as the
+// B operand of the next product: lane (col, half) holds rows 16 (r0 / 8) + 8 half .. + 7.
+template <typename T>
+__device__ __forceinline__ uint4 acc_to_operand(const float* p) {
+  uint32_t g0a = pack2<T>(p[0], p[1]), g0b = pack2<T>(p[2], p[3]), g1a = pack2<T>(p[4], p[5]), g1b = pack2<T>(p[6], p[7]);
+  swap_halves(g0a, g1a);
+  swap_halves(g0b, g1b);
+  return make_uint4(g0a, g0b, g1a, g1b);
+}
+
+// ---- LDS images of a [64 rows][D] tile, rows of D 16-bit elements = D / 8 chunks of 16 bytes ----
+// "row image": chunk c of row r at position c ^ (r & 7); read as the A operand (lane = row, 8 consecutive columns).
+// "transposed image": chunk c of row r at position c ^ 2 (r & 3); read with ds_read_b64_tr_b16 as the A operand of the
+// transposed tile (lane = column, 8 consecutive rows).
+template <int D>
+__device__ __forceinline__ uint32_t row_image_at(int r, int c) { return static_cast<uint32_t>(r * (2 * D) + ((c ^ (r & 7)) * 16)); }
+template <int D>
+__device__ __forceinline__ uint32_t tr_image_at(int r, int c) { return static_cast<uint32_t>(r * (2 * D) + ((c ^ (2 * (r & 3))) * 16)); }
+
+template <int D>
+struct Staged {
+  static constexpr int CH = D / 8;
+  static constexpr int N = FA_TILE * CH / FA_THREADS;
+  uint4 v[N];
+  // rows row0 .. row0+63 of a sequence of `len` rows that starts at `base` (head offset applied); rows past the end are zeros
+  template <typename T>
+  __device__ __forceinline__ void load(const T* base, int64_t stride, int row0, int len) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int id = static_cast<int>(threadIdx.x) + FA_THREADS * i;
+      const int r = id / CH, c = id % CH;
+      v[i] = make_uint4(0, 0, 0, 0);
+      if (row0 + r < len) v[i] = *reinterpret_cast<const uint4*>(base + static_cast<int64_t>(row0 + r) * stride + 8 * c);
+    }
+  }
+  __device__ __forceinline__ void store_rows(uint8_t* img) const {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int id = static_cast<int>(threadIdx.x) + FA_THREADS * i;
+      *reinterpret_cast<uint4*>(img + row_image_at<D>(id / CH, id % CH)) = v[i];
+    }
+  }
+  __device__ __forceinline__ void store_transposed(uint8_t* img) const {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int id = static_cast<int>(threadIdx.x) + FA_THREADS * i;
+      *reinterpret_cast<uint4*>(img + tr_image_at<D>(id / CH, id % CH)) = v[i];
+    }
+  }
+};
+
+// A operand from the row image: rows 32 i + (lane & 31), columns 16 s + 8 (lane >> 5) .. + 7
+template <int D>
+__device__ __forceinline__ uint4 read_rows(const uint8_t* img, int i, int s, int lane) {
+  return *reinterpret_cast<const uint4*>(img + row_image_at<D>(32 * i + (lane & 31), 2 * s + (lane >> 5)));
+}
+// A operand of the transposed tile: columns 32 i + (lane & 31), rows 16 kk + 8 (lane >> 5) .. + 7. Within 16 lanes the
+// transposing read takes 4 rows x 16 columns and hands each lane the 4 rows of its own column.
+template <int D>
+__device__ __forceinline__ uint4 read_transposed(const uint8_t* img, int i, int kk, int lane) {
+  const int r = 16 * kk + 8 * (lane >> 5) + ((lane >> 2) & 3);
+  const int c = 4 * i + 2 * ((lane >> 4) & 1) + ((lane >> 1) & 1);
+  const uint8_t* p = img + tr_image_at<D>(r, c) + (lane & 1) * 8;      // r + 4 has the same r & 3: same swizzle
+  const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p));
+  const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(p + 4 * 2 * D));
+  union { s16x4_t s[2]; uint4 u; } cv;
+  cv.s[0] = lo;
+  cv.s[1] = hi;
+  return cv.u;
+}
+
+// The wavefront's 32 resident rows as the B operand: lane (row, half) holds columns 16 s + 8 half .. + 7
+template <typename T, int D>
+__device__ __forceinline__ void load_resident(uint4 (&f)[D / 16], const T* base, int64_t stride, int row, int len, int lane) {
+  const T* p = base + static_cast<int64_t>(row) * stride + 8 * (lane >> 5);
+#pragma unroll
+  for (int s = 0; s < D / 16; ++s) f[s] = row < len ? *reinterpret_cast<const uint4*>(p + 16 * s) : make_uint4(0, 0, 0, 0);
+}
+
+template <int CTRL>
+__device__ __forceinline__ uint32_t quad_dpp(uint32_t v) {
+  return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), CTRL, 0xf, 0xf, true));
+}
+
+// The random bytes of this lane's 32 elements of a 64-row tile of the streamed kind: bytes[n][g] holds, in byte e, the byte
+// of element (registers 4 g + e of accumulator n). `fixed` is the lane's own index (query in the query-major kernels, key
+// in the key-major one); consecutive lanes hold consecutive indices, so the four lanes of a quad share each 4 x 4 patch:
+// every lane runs the generator for two of the quad's eight patches (g = its position in the quad, n = 0, 1) and the
+// words travel inside the quad: transposed when a lane needs its own row of every patch (query-major: word i % 4),
+// broadcast when it needs its own column (key-major: byte j % 4 of every word). An integer multiply runs at a quarter of
+// the VALU rate, which makes the ten rounds the expensive part of the softmax: hence one call per 16 elements.
+template <bool QUERY_MAJOR>
+__device__ __forceinline__ void tile_random_bytes(const FaArgs& a, const Philox& gen, int bh, int fixed, int tile, int half,
+                                                  int lane, uint32_t (&bytes)[2][4]) {
+  const int c = lane & 3;
+  const uint64_t q4 = static_cast<uint64_t>((a.max_q + 3) / 4), k4 = static_cast<uint64_t>((a.max_k + 3) / 4);
+#pragma unroll
+  for (int n = 0; n < 2; ++n) {
+    const uint64_t streamed = static_cast<uint64_t>(16 * tile + 8 * n + 2 * c + half);     // group of four of the streamed kind
+    const uint64_t own = static_cast<uint64_t>(fixed / 4);
+    const uint64_t block = QUERY_MAJOR ? (static_cast<uint64_t>(bh) * q4 + own) * k4 + streamed
+                                       : (static_cast<uint64_t>(bh) * q4 + streamed) * k4 + own;
+    const uint4 r = gen(block, a.offset);
+    uint32_t w[4] = {r.x, r.y, r.z, r.w};
+    if constexpr (QUERY_MAJOR) {
+      // 4 x 4 transpose across the quad: afterwards w[g] is word (lane & 3) of the patch that lane g of the quad drew
+      const bool odd = (c & 1) != 0, up = (c & 2) != 0;
+      uint32_t s0 = odd ? w[0] : w[1], s1 = odd ? w[2] : w[3];
+      s0 = quad_dpp<0xB1>(s0);
+      s1 = quad_dpp<0xB1>(s1);
+      if (odd) { w[0] = s0; w[2] = s1; } else { w[1] = s0; w[3] = s1; }
+      s0 = up ? w[0] : w[2];
+      s1 = up ? w[1] : w[3];
+      s0 = quad_dpp<0x4E>(s0);
+      s1 = quad_dpp<0x4E>(s1);
+      if (up) { w[0] = s0; w[1] = s1; } else { w[2] = s0; w[3] = s1; }
+#pragma unroll
+      for (int g = 0; g < 4; ++g) bytes[n][g] = w[g];
+    } else {
+      const int sh = 8 * (fixed & 3);
+      uint32_t all[4][4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        all[0][e] = quad_dpp<0x00>(w[e]);
+        all[1][e] = quad_dpp<0x55>(w[e]);
+        all[2][e] = quad_dpp<0xAA>(w[e]);
+        all[3][e] = quad_dpp<0xFF>(w[e]);
+      }
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+        bytes[n][g] = ((all[g][0] >> sh) & 0xffu) | (((all[g][1] >> sh) & 0xffu) << 8) | (((all[g][2] >> sh) & 0xffu) << 16) |
+                      (((all[g][3] >> sh) & 0xffu) << 24);
+    }
+  }
+}
+
+// Keep-flags of the four elements of accumulator group g (registers 4 g .. 4 g + 3): `fixed` is the lane's own index and
+// `first` the first of the four consecutive indices of the other kind; `bytes` is that group's word of tile_random_bytes.
+template <int DROP, bool QUERY_MAJOR>
+__device__ __forceinline__ void keep_flags(const FaArgs& a, uint32_t bytes, int bh, int fixed, int first, int lq, int lk,
+                                           bool (&keep)[4]) {
+  if constexpr (DROP == 0) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) keep[e] = true;
+  } else if constexpr (DROP == 1) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int qi = QUERY_MAJOR ? fixed : first + e, kj = QUERY_MAJOR ? first + e : fixed;
+      keep[e] = qi < lq && kj < lk && a.mask[(static_cast<int64_t>(bh) * a.max_q + qi) * a.max_k + kj] != 0;
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) keep[e] = ((bytes >> (8 * e)) & 0xffu) < a.thr;
+  }
+}
+
+// Writes the wavefront's 32 rows x D accumulators (acc[i][r]: column 32 i + 8 (r / 4) + 4 half + r % 4 of row lane & 31)
+// through its own LDS patch as whole 16-byte chunks, rows past `len` skipped.
+template <typename T, int D>
+__device__ __forceinline__ void store_rows_out(const acc16_t (&acc)[D / 32], float mul, uint8_t* patch, T* base, int64_t stride,
+                                               int row0, int len, int lane) {
+  const int half = lane >> 5, row = lane & 31;
+#pragma unroll
+  for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int col = 32 * i + 8 * g + 4 * half;
+      uint2 w;
+      w.x = pack2<T>(acc[i][4 * g + 0] * mul, acc[i][4 * g + 1] * mul);
+      w.y = pack2<T>(acc[i][4 * g + 2] * mul, acc[i][4 * g + 3] * mul);
+      *reinterpret_cast<uint2*>(patch + row_image_at<D>(row, col / 8) + (col % 8) * 2) = w;
+    }
+  __syncthreads();
+  constexpr int CH = D / 8;
+#pragma unroll
+  for (int i = 0; i < 32 * CH / 64; ++i) {
+    const int id = lane + 64 * i;
+    const int r = id / CH, c = id % CH;
+    if (row0 + r < len)
+      *reinterpret_cast<uint4*>(base + static_cast<int64_t>(row0 + r) * stride + 8 * c) =
+          *reinterpret_cast<const uint4*>(patch + row_image_at<D>(r, c));
+  }
+}
+
+// -------------------------------------------------------------------------------------------------------------------
+// forward
+// -------------------------------------------------------------------------------------------------------------------
+template <typename T, int D, int DROP>
+__global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_fwd_kernel(FaArgs a) {
+  extern __shared__ __align__(16) uint8_t lds_raw[];
+  constexpr int IMG = FA_TILE * D * 2;
+  const int b = blockIdx.z, h = blockIdx.y, q0 = static_cast<int>(blockIdx.x) * FA_ROWS;
+  const int qs = a.cu_q[b], lq = min(a.cu_q[b + 1] - qs, a.max_q), ks = a.cu_k[b], lk = min(a.cu_k[b + 1] - ks, a.max_k);
+  if (q0 >= lq) return;
+  const int lane = static_cast<int>(threadIdx.x) & 63, wave = static_cast<int>(threadIdx.x) >> 6, half = lane >> 5;
+  const int bh = b * a.heads + h;
+  const int qrow = q0 + 32 * wave + (lane & 31);
+  const T* qb = static_cast<const T*>(a.q) + static_cast<int64_t>(qs) * a.q_st + static_cast<int64_t>(h) * a.q_sh;
+  const T* kb = static_cast<const T*>(a.k) + static_cast<int64_t>(ks) * a.k_st + static_cast<int64_t>(h) * a.k_sh;
+  const T* vb = static_cast<const T*>(a.v) + static_cast<int64_t>(ks) * a.v_st + static_cast<int64_t>(h) * a.v_sh;
+  uint4 qf[D / 16];
+  load_resident<T, D>(qf, qb, a.q_st, qrow, lq, lane);
+
+  const int nkeys = a.causal ? min(lk, q0 + FA_ROWS) : lk;
+  const int ntiles = (nkeys + FA_TILE - 1) / FA_TILE;
+  const Philox gen(a.seed);
+
+  acc16_t o[D / 32];
+#pragma unroll
+  for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
+  float m = FA_NEG, l = 0.f;
+  const float dead_raw = FA_NEG / a.scale_log2;   // the raw score that the scale turns into -1e30
+
+  Staged<D> sk, sv;
+  if (ntiles > 0) {
+    sk.load(kb, a.k_st, 0, lk);
+    sv.load(vb, a.v_st, 0, lk);
+    sk.store_rows(lds_raw);
+    sv.store_transposed(lds_raw + IMG);
+  }
+  __syncthreads();
+  for (int t = 0; t < ntiles; ++t) {
+    const uint8_t* kimg = lds_raw + (t & 1) * 2 * IMG;
+    const uint8_t* vimg = kimg + IMG;
+    if (t + 1 < ntiles) {
+      sk.load(kb, a.k_st, (t + 1) * FA_TILE, lk);
+      sv.load(vb, a.v_st, (t + 1) * FA_TILE, lk);
+    }
+    acc16_t s[2];
+#pragma unroll
+    for (int n = 0; n < 2; ++n)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[n][r] = 0.f;
+#pragma unroll
+    for (int ss = 0; ss < D / 16; ++ss)
+#pragma unroll
+      for (int n = 0; n < 2; ++n) mfma<T>::run(read_rows<D>(kimg, n, ss, lane), qf[ss], s[n]);
+    // Masking only where the tile crosses the end of the keys or the causal diagonal (the same for the whole wavefront).
+    // A masked raw score is the value that the scale turns into -1e30 or beyond: its probability is exp2 of that, 0.
+    const bool edge = (t + 1) * FA_TILE > lk || (a.causal && t * FA_TILE + FA_TILE - 1 > q0 + 32 * wave);
+    if (edge) {
+#pragma unroll
+      for (int n = 0; n < 2; ++n)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = t * FA_TILE + 32 * n + 8 * (r / 4) + 4 * half + r % 4;
+          if (key >= lk || (a.causal && key > qrow)) s[n][r] = dead_raw;
+        }
+    }
+    // tile maximum of the scaled scores from the extreme raw score (one multiplication instead of 32)
+    float ext = s[0][0];
+    if (a.scale_log2 >= 0.f) {
+#pragma unroll
+      for (int n = 0; n < 2; ++n)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) ext = fmaxf(ext, s[n][r]);
+    } else {
+#pragma unroll
+      for (int n = 0; n < 2; ++n)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) ext = fminf(ext, s[n][r]);
+    }
+    const float mx = pair_max(ext * a.scale_log2);
+    // The reference point m follows the running maximum lazily: it moves (and the accumulators are rescaled) only when a
+    // row's maximum has grown by more than 2^8, so probabilities relative to m stay below 256, inside every type here,
+    // and most tiles skip the rescaling. out = O / l does not depend on m. Every row sees a live key in its first tile
+    // (key 0), so m leaves its initial value there.
+    const bool grow = mx > m + FA_LAZY;
+    if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+      const float m_new = grow ? mx : m;
+      const float alpha = fast_exp2(m - m_new);
+      m = m_new;
+      l *= alpha;
+#pragma unroll
+      for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[i][r] *= alpha;
+    }
+    float lsum = 0.f;
+#pragma unroll
+    for (int n = 0; n < 2; ++n)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float pr = fast_exp2(__builtin_fmaf(s[n][r], a.scale_log2, -m));
+        s[n][r] = pr;
+        lsum += pr;
+      }
+    l += lsum;
+    if constexpr (DROP != 0) {
+      uint32_t rnd[2][4] = {};
+      if constexpr (DROP == 2) tile_random_bytes<true>(a, gen, bh, qrow, t, half, lane, rnd);
+#pragma unroll
+      for (int n = 0; n < 2; ++n)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          bool keep[4];
+          keep_flags<DROP, true>(a, rnd[n][g], bh, qrow, t * FA_TILE + 32 * n + 8 * g + 4 * half, lq, lk, keep);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) s[n][4 * g + e] = keep[e] ? s[n][4 * g + e] : 0.f;      // the scale waits for the end
+        }
+      if constexpr (DROP == 2) {
+        if (a.mask_out != nullptr && qrow < lq) {
+          uint8_t* row = a.mask_out + (static_cast<int64_t>(bh) * a.max_q + qrow) * a.max_k;
+#pragma unroll
+          for (int n = 0; n < 2; ++n)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int key = t * FA_TILE + 32 * n + 8 * (r / 4) + 4 * half + r % 4;
+              if (key < lk) row[key] = ((rnd[n][r / 4] >> (8 * (r % 4))) & 0xffu) < a.thr;
+            }
+        }
+      }
+    }
+#pragma unroll
+    for (int kk = 0; kk < FA_TILE / 16; ++kk) {
+      float pv[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) pv[e] = s[kk / 2][8 * (kk % 2) + e];
+      const uint4 pf = acc_to_operand<T>(pv);
+#pragma unroll
+      for (int i = 0; i < D / 32; ++i) mfma<T>::run(read_transposed<D>(vimg, i, kk, lane), pf, o[i]);
+    }
+    if (t + 1 < ntiles) {
+      uint8_t* nk = lds_raw + ((t + 1) & 1) * 2 * IMG;
+      sk.store_rows(nk);
+      sv.store_transposed(nk + IMG);
+    }
+    __syncthreads();
+  }
+  l = pair_sum(l);
+  const float inv = l > 0.f ? a.drop_scale / l : 0.f;
+  if (half == 0 && qrow < lq)
+    a.lse[static_cast<int64_t>(bh) * a.max_q + qrow] = l > 0.f ? (m + log2f(l)) * (1.0f / FA_LOG2E) : -INFINITY;
+  T* ob = static_cast<T*>(a.out) + static_cast<int64_t>(qs) * a.o_st + static_cast<int64_t>(h) * a.o_sh;
+  store_rows_out<T, D>(o, inv, lds_raw + wave * (32 * D * 2), ob, a.o_st, q0 + 32 * wave, lq, lane);
+}
+
+// -------------------------------------------------------------------------------------------------------------------
+// backward, dQ and D = rowsum(dO * O)
+// -------------------------------------------------------------------------------------------------------------------
+template <typename T, int D, int DROP>
+__global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dq_kernel(FaArgs a) {
+  extern __shared__ __align__(16) uint8_t lds_raw[];
+  constexpr int IMG = FA_TILE * D * 2;
+  const int b = blockIdx.z, h = blockIdx.y, q0 = static_cast<int>(blockIdx.x) * FA_ROWS;
+  const int qs = a.cu_q[b], lq = min(a.cu_q[b + 1] - qs, a.max_q), ks = a.cu_k[b], lk = min(a.cu_k[b + 1] - ks, a.max_k);
+  if (q0 >= lq) return;
+  const int lane = static_cast<int>(threadIdx.x) & 63, wave = static_cast<int>(threadIdx.x) >> 6, half = lane >> 5;
+  const int bh = b * a.heads + h;
+  const int qrow = q0 + 32 * wave + (lane & 31);
+  const T* qb = static_cast<const T*>(a.q) + static_cast<int64_t>(qs) * a.q_st + static_cast<int64_t>(h) * a.q_sh;
+  const T* kb = static_cast<const T*>(a.k) + static_cast<int64_t>(ks) * a.k_st + static_cast<int64_t>(h) * a.k_sh;
+  const T* vb = static_cast<const T*>(a.v) + static_cast<int64_t>(ks) * a.v_st + static_cast<int64_t>(h) * a.v_sh;
+  const T* ob = static_cast<const T*>(a.o) + static_cast<int64_t>(qs) * a.o_st + static_cast<int64_t>(h) * a.o_sh;
+  const T* gb = static_cast<const T*>(a.d_o) + static_cast<int64_t>(qs) * a.do_st + static_cast<int64_t>(h) * a.do_sh;
+  uint4 qf[D / 16], gf[D / 16];
+  load_resident<T, D>(qf, qb, a.q_st, qrow, lq, lane);
+  load_resident<T, D>(gf, gb, a.do_st, qrow, lq, lane);
+  float delta = 0.f;
+  {
+    uint4 of[D / 16];
+    load_resident<T, D>(of, ob, a.o_st, qrow, lq, lane);
+#pragma unroll
+    for (int s = 0; s < D / 16; ++s) {
+      const T* x = reinterpret_cast<const T*>(&of[s]);
+      const T* y = reinterpret_cast<const T*>(&gf[s]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) delta += elem<T>::to_float(x[e]) * elem<T>::to_float(y[e]);
+    }
+    delta = pair_sum(delta);
+  }
+  const int64_t stat = static_cast<int64_t>(bh) * a.max_q + qrow;
+  float lse2 = -FA_NEG;   // rows past the sequence: probability 0
+  if (qrow < lq) {
+    const float v = a.lse[stat];
+    lse2 = v == -INFINITY ? -FA_NEG : v * FA_LOG2E;
+    if (half == 0) a.delta[stat] = delta;
+  }
+
+  const int nkeys = a.causal ? min(lk, q0 + FA_ROWS) : lk;
+  const int ntiles = (nkeys + FA_TILE - 1) / FA_TILE;
+  const Philox gen(a.seed);
+  const float dead_raw = FA_NEG / a.scale_log2;   // the raw score that the scale turns into -1e30
+  acc16_t dq[D / 32];
+#pragma unroll
+  for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dq[i][r] = 0.f;
+
+  // per buffer: K row image, K transposed image, V row image
+  Staged<D> sk, sv;
+  if (ntiles > 0) {
+    sk.load(kb, a.k_st, 0, lk);
+    sv.load(vb, a.v_st, 0, lk);
+    sk.store_rows(lds_raw);
+    sk.store_transposed(lds_raw + IMG);
+    sv.store_rows(lds_raw + 2 * IMG);
+  }
+  __syncthreads();
+  for (int t = 0; t < ntiles; ++t) {
+    const uint8_t* kimg = lds_raw + (t & 1) * 3 * IMG;
+    const uint8_t* ktimg = kimg + IMG;
+    const uint8_t* vimg = kimg + 2 * IMG;
+    if (t + 1 < ntiles) {
+      sk.load(kb, a.k_st, (t + 1) * FA_TILE, lk);
+      sv.load(vb, a.v_st, (t + 1) * FA_TILE, lk);
+    }
+    acc16_t s[2], dp[2];
+#pragma unroll
+    for (int n = 0; n < 2; ++n)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { s[n][r] = 0.f; dp[n][r] = 0.f; }
+#pragma unroll
+    for (int ss = 0; ss < D / 16; ++ss)
+#pragma unroll
+      for (int n = 0; n < 2; ++n) {
+        mfma<T>::run(read_rows<D>(kimg, n, ss, lane), qf[ss], s[n]);
+        mfma<T>::run(read_rows<D>(vimg, n, ss, lane), gf[ss], dp[n]);
+      }
+    // masking as in the forward: only where the tile crosses the end of the keys or the causal diagonal
+    if ((t + 1) * FA_TILE > lk || (a.causal && t * FA_TILE + FA_TILE - 1 > q0 + 32 * wave)) {
+#pragma unroll
+      for (int n = 0; n < 2; ++n)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = t * FA_TILE + 32 * n + 8 * (r / 4) + 4 * half + r % 4;
+          if (key >= lk || (a.causal && key > qrow)) s[n][r] = dead_raw;
+        }
+    }
+    uint32_t rnd[2][4] = {};
+    if constexpr (DROP == 2) tile_random_bytes<true>(a, gen, bh, qrow, t, half, lane, rnd);
+#pragma unroll
+    for (int n = 0; n < 2; ++n)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int key0 = t * FA_TILE + 32 * n + 8 * g + 4 * half;
+        bool keep[4];
+        keep_flags<DROP, true>(a, rnd[n][g], bh, qrow, key0, lq, lk, keep);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int r = 4 * g + e;
+          const float pr = fast_exp2(__builtin_fmaf(s[n][r], a.scale_log2, -lse2));
+          const float kscale = DROP != 0 ? (keep[e] ? a.drop_scale : 0.f) : 1.f;
+          s[n][r] = pr * __builtin_fmaf(dp[n][r], kscale, -delta);     // dS
+        }
+      }
+#pragma unroll
+    for (int kk = 0; kk < FA_TILE / 16; ++kk) {
+      float dsv[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dsv[e] = s[kk / 2][8 * (kk % 2) + e];
+      const uint4 df = acc_to_operand<T>(dsv);
+#pragma unroll
+      for (int i = 0; i < D / 32; ++i) mfma<T>::run(read_transposed<D>(ktimg, i, kk, lane), df, dq[i]);
+    }
+    if (t + 1 < ntiles) {
+      uint8_t* nk = lds_raw + ((t + 1) & 1) * 3 * IMG;
+      sk.store_rows(nk);
+      sk.store_transposed(nk + IMG);
+      sv.store_rows(nk + 2 * IMG);
+    }
+    __syncthreads();
+  }
+  T* dqb = static_cast<T*>(a.dq) + static_cast<int64_t>(qs) * a.dq_st + static_cast<int64_t>(h) * a.dq_sh;
+  store_rows_out<T, D>(dq, a.scale, lds_raw + wave * (32 * D * 2), dqb, a.dq_st, q0 + 32 * wave, lq, lane);
+}
+
+// -------------------------------------------------------------------------------------------------------------------
+// backward, dK and dV: one key per lane pair, query tiles of 64 streamed through LDS
+// -------------------------------------------------------------------------------------------------------------------
+template <typename T, int D, int DROP>
+__global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dkv_kernel(FaArgs a) {
+  extern __shared__ __align__(16) uint8_t lds_raw[];
+  constexpr int IMG = FA_TILE * D * 2;
+  constexpr int BUF = 4 * IMG + 2 * FA_TILE * 4;   // Q rows, Q transposed, dO rows, dO transposed, lse2[64], delta[64]
+  const int b = blockIdx.z, h = blockIdx.y, k0 = static_cast<int>(blockIdx.x) * FA_ROWS;
+  const int qs = a.cu_q[b], lq = min(a.cu_q[b + 1] - qs, a.max_q), ks = a.cu_k[b], lk = min(a.cu_k[b + 1] - ks, a.max_k);
+  if (k0 >= lk) return;
+  const int lane = static_cast<int>(threadIdx.x) & 63, wave = static_cast<int>(threadIdx.x) >> 6, half = lane >> 5;
+  const int bh = b * a.heads + h;
+  const int krow = k0 + 32 * wave + (lane & 31);
+  const T* qb = static_cast<const T*>(a.q) + static_cast<int64_t>(qs) * a.q_st + static_cast<int64_t>(h) * a.q_sh;
+  const T* kb = static_cast<const T*>(a.k) + static_cast<int64_t>(ks) * a.k_st + static_cast<int64_t>(h) * a.k_sh;
+  const T* vb = static_cast<const T*>(a.v) + static_cast<int64_t>(ks) * a.v_st + static_cast<int64_t>(h) * a.v_sh;
+  const T* gb = static_cast<const T*>(a.d_o) + static_cast<int64_t>(qs) * a.do_st + static_cast<int64_t>(h) * a.do_sh;
+  uint4 kf[D / 16], vf[D / 16];
+  load_resident<T, D>(kf, kb, a.k_st, krow, lk, lane);
+  load_resident<T, D>(vf, vb, a.v_st, krow, lk, lane);
+
+  // causal: queries before the block's first key see none of its keys
+  const int t0 = a.causal ? k0 / FA_TILE : 0;
+  const int ntiles = (lq + FA_TILE - 1) / FA_TILE;
+  const Philox gen(a.seed);
+  const float dead_raw = FA_NEG / a.scale_log2;   // the raw score that the scale turns into -1e30
+  acc16_t dk[D / 32], dv[D / 32];
+#pragma unroll
+  for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { dk[i][r] = 0.f; dv[i][r] = 0.f; }
+
+  Staged<D> sq, sg;
+  float st_val = 0.f;   // threads 0..63: lse2 of the tile's query, 64..127: its D
+  auto load_stats = [&](int t) {
+    const int tid = static_cast<int>(threadIdx.x);
+    if (tid < 2 * FA_TILE) {
+      const int qi = t * FA_TILE + (tid & (FA_TILE - 1));
+      if (tid < FA_TILE) {
+        st_val = -FA_NEG;
+        if (qi < lq) {
+          const float v = a.lse[static_cast<int64_t>(bh) * a.max_q + qi];
+          st_val = v == -INFINITY ? -FA_NEG : v * FA_LOG2E;
+        }
+      } else {
+        st_val = qi < lq ? a.delta[static_cast<int64_t>(bh) * a.max_q + qi] : 0.f;
+      }
+    }
+  };
+  auto store_tile = [&](uint8_t* buf) {
+    sq.store_rows(buf);
+    sq.store_transposed(buf + IMG);
+    sg.store_rows(buf + 2 * IMG);
+    sg.store_transposed(buf + 3 * IMG);
+    if (threadIdx.x < 2 * FA_TILE) reinterpret_cast<float*>(buf + 4 * IMG)[threadIdx.x] = st_val;
+  };
+  if (t0 < ntiles) {
+    sq.load(qb, a.q_st, t0 * FA_TILE, lq);
+    sg.load(gb, a.do_st, t0 * FA_TILE, lq);
+    load_stats(t0);
+    store_tile(lds_raw + (t0 & 1) * BUF);
+  }
+  __syncthreads();
+  for (int t = t0; t < ntiles; ++t) {
+    const uint8_t* qimg = lds_raw + (t & 1) * BUF;
+    const uint8_t* qtimg = qimg + IMG;
+    const uint8_t* gimg = qimg + 2 * IMG;
+    const uint8_t* gtimg = qimg + 3 * IMG;
+    const float* stats = reinterpret_cast<const float*>(qimg + 4 * IMG);
+    if (t + 1 < ntiles) {
+      sq.load(qb, a.q_st, (t + 1) * FA_TILE, lq);
+      sg.load(gb, a.do_st, (t + 1) * FA_TILE, lq);
+      load_stats(t + 1);
+    }
+    acc16_t s[2], dp[2];
+#pragma unroll
+    for (int n = 0; n < 2; ++n)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { s[n][r] = 0.f; dp[n][r] = 0.f; }
+#pragma unroll
+    for (int ss = 0; ss < D / 16; ++ss)
+#pragma unroll
+      for (int n = 0; n < 2; ++n) {
+        mfma<T>::run(read_rows<D>(qimg, n, ss, lane), kf[ss], s[n]);
+        mfma<T>::run(read_rows<D>(gimg, n, ss, lane), vf[ss], dp[n]);
+      }
+    // s[n][r]: query 32 n + 8 (r / 4) + 4 half + r % 4 of the tile, key krow. P (dropped, scaled) stays in dp's place
+    // for dV, dS goes to s for dK.
+    if (k0 + 32 * wave + 31 >= lk || (a.causal && t * FA_TILE < k0 + 32 * wave + 31)) {
+#pragma unroll
+      for (int n = 0; n < 2; ++n)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int qi = t * FA_TILE + 32 * n + 8 * (r / 4) + 4 * half + r % 4;
+          if (krow >= lk || (a.causal && krow > qi)) s[n][r] = dead_raw;
+        }
+    }
+    uint32_t rnd[2][4] = {};
+    if constexpr (DROP == 2) tile_random_bytes<false>(a, gen, bh, krow, t, half, lane, rnd);
+#pragma unroll
+    for (int n = 0; n < 2; ++n)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int ql = 32 * n + 8 * g + 4 * half;          // first of four consecutive queries, within the tile
+        const float4 l4 = *reinterpret_cast<const float4*>(stats + ql);
+        const float4 d4 = *reinterpret_cast<const float4*>(stats + FA_TILE + ql);
+        const float lse2[4] = {l4.x, l4.y, l4.z, l4.w}, dl[4] = {d4.x, d4.y, d4.z, d4.w};
+        bool keep[4];
+        keep_flags<DROP, false>(a, rnd[n][g], bh, krow, t * FA_TILE + ql, lq, lk, keep);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int r = 4 * g + e;
+          const float pr = fast_exp2(__builtin_fmaf(s[n][r], a.scale_log2, -lse2[e]));
+          const float kscale = DROP != 0 ? (keep[e] ? a.drop_scale : 0.f) : 1.f;
+          s[n][r] = pr * __builtin_fmaf(dp[n][r], kscale, -dl[e]);   // dS
+          dp[n][r] = DROP != 0 ? (keep[e] ? pr : 0.f) : pr;          // kept probabilities; their scale waits for the end
+        }
+      }
+#pragma unroll
+    for (int kk = 0; kk < FA_TILE / 16; ++kk) {
+      float pv[8], dsv[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { pv[e] = dp[kk / 2][8 * (kk % 2) + e]; dsv[e] = s[kk / 2][8 * (kk % 2) + e]; }
+      const uint4 pf = acc_to_operand<T>(pv), df = acc_to_operand<T>(dsv);
+#pragma unroll
+      for (int i = 0; i < D / 32; ++i) {
+        mfma<T>::run(read_transposed<D>(gtimg, i, kk, lane), pf, dv[i]);
+        mfma<T>::run(read_transposed<D>(qtimg, i, kk, lane), df, dk[i]);
+      }
+    }
+    if (t + 1 < ntiles) store_tile(lds_raw + ((t + 1) & 1) * BUF);
+    __syncthreads();
+  }
+  T* dkb = static_cast<T*>(a.dk) + static_cast<int64_t>(ks) * a.dk_st + static_cast<int64_t>(h) * a.dk_sh;
+  T* dvb = static_cast<T*>(a.dv) + static_cast<int64_t>(ks) * a.dv_st + static_cast<int64_t>(h) * a.dv_sh;
+  uint8_t* patch = lds_raw + wave * (32 * D * 2);
+  store_rows_out<T, D>(dk, a.scale, patch, dkb, a.dk_st, k0 + 32 * wave, lk, lane);
+  __syncthreads();
+  store_rows_out<T, D>(dv, a.drop_scale, patch, dvb, a.dv_st, k0 + 32 * wave, lk, lane);
+}
+
+template <int D> constexpr int fwd_lds() { return 2 * 2 * FA_TILE * D * 2; }
+template <int D> constexpr int dq_lds() { return 2 * 3 * FA_TILE * D * 2; }
+template <int D> constexpr int dkv_lds() { return 2 * (4 * FA_TILE * D * 2 + 2 * FA_TILE * 4); }
+
+template <typename K>
+int launch(K kern, const char* what, dim3 grid, int lds, hipStream_t st, const FaArgs& a) {
+  if (lds > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) return fail(NMTG_ERR_LAUNCH, "%s: cannot reserve %d bytes of LDS: %s", what, lds, hipGetErrorString(e));
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(FA_THREADS), lds, st, a);
+  return 0;
+}
+
+template <typename T, int D>
+int fwd_launch(const FaArgs& a, int drop, dim3 grid, hipStream_t st) {
+  TraceScope trace("flash_attn_fwd", st);
+  if (drop == 0) return launch(flash_fwd_kernel<T, D, 0>, "flash_attn_fwd", grid, fwd_lds<D>(), st, a);
+  if (drop == 1) return launch(flash_fwd_kernel<T, D, 1>, "flash_attn_fwd", grid, fwd_lds<D>(), st, a);
+  return launch(flash_fwd_kernel<T, D, 2>, "flash_attn_fwd", grid, fwd_lds<D>(), st, a);
+}
+template <typename T, int D>
+int bwd_launch(const FaArgs& a, int drop, dim3 grid_q, dim3 grid_k, hipStream_t st) {
+  int rc = 0;
+  if (grid_q.x > 0) {
+    TraceScope trace("flash_attn_bwd_dq", st);
+    rc = drop == 0   ? launch(flash_bwd_dq_kernel<T, D, 0>, "flash_attn_bwd", grid_q, dq_lds<D>(), st, a)
+         : drop == 1 ? launch(flash_bwd_dq_kernel<T, D, 1>, "flash_attn_bwd", grid_q, dq_lds<D>(), st, a)
+                     : launch(flash_bwd_dq_kernel<T, D, 2>, "flash_attn_bwd", grid_q, dq_lds<D>(), st, a);
+  }
+  if (rc || grid_k.x == 0) return rc;
+  TraceScope trace("flash_attn_bwd_dkv", st);
+  return drop == 0   ? launch(flash_bwd_dkv_kernel<T, D, 0>, "flash_attn_bwd", grid_k, dkv_lds<D>(), st, a)
+         : drop == 1 ? launch(flash_bwd_dkv_kernel<T, D, 1>, "flash_attn_bwd", grid_k, dkv_lds<D>(), st, a)
+                     : launch(flash_bwd_dkv_kernel<T, D, 2>, "flash_attn_bwd", grid_k, dkv_lds<D>(), st, a);
+}
+
+bool view_ok(const void* p, int64_t st, int64_t sh, int64_t heads, int64_t d) {
+  return aligned16(p) && st % 8 == 0 && sh % 8 == 0 && sh >= d && st >= (heads - 1) * sh + d;
+}
+
+int check_common(const char* what, int64_t batch, int64_t heads, int64_t d, int64_t max_q, int64_t max_k, int drop_mode, float p,
+                 float scale, int dtype) {
+  NMTG_REQUIRE(fabsf(scale) >= 1e-6f && fabsf(scale) <= 1e6f, "%s: softmax_scale %g (magnitudes from 1e-6 to 1e6 are handled)", what,
+               (double)scale);
+  NMTG_REQUIRE(batch >= 0 && heads >= 1 && max_q >= 0 && max_k >= 0, "%s: bad shape batch=%lld heads=%lld max_q=%lld max_k=%lld",
+               what, (long long)batch, (long long)heads, (long long)max_q, (long long)max_k);
+  NMTG_REQUIRE(d == 64 || d == 128, "%s: head dimension %lld (64 and 128 are built)", what, (long long)d);
+  NMTG_REQUIRE(dtype == NMTG_F16 || dtype == NMTG_BF16, "%s: fp16 or bf16 tensors required (matrix-core kernel)", what);
+  NMTG_REQUIRE(drop_mode >= 0 && drop_mode <= 2, "%s: dropout mode %d", what, drop_mode);
+  NMTG_REQUIRE(drop_mode == 0 || (p >= 0.f && p < 1.f), "%s: dropout probability %g outside [0, 1)", what, (double)p);
+  NMTG_REQUIRE(heads <= 65535 && batch <= 65535, "%s: more than 65535 heads or sequences in one launch", what);
+  NMTG_REQUIRE(batch * heads * (max_q + 3) / 4 * ((max_k + 3) / 4) < (1ll << 62) && max_q <= (1 << 24) && max_k <= (1 << 24),
+               "%s: sequence lengths too large", what);
+  return 0;
+}
+
+void set_dropout(FaArgs& a, int drop_mode, float p, uint64_t seed, uint64_t offset) {
+  a.thr = 256;
+  a.drop_scale = 1.f;
+  if (drop_mode == 1) a.drop_scale = 1.f / (1.f - p);
+  if (drop_mode == 2) {
+    long thr = lroundf(256.f * (1.f - p));
+    a.thr = static_cast<uint32_t>(thr < 1 ? 1 : thr > 256 ? 256 : thr);
+    a.drop_scale = 256.f / static_cast<float>(a.thr);
+  }
+  a.seed = seed;
+  a.offset = offset;
+}
+
+}  // namespace
+}  // namespace nmtg
+
+using namespace nmtg;
+
+extern "C" int nmtg_flash_attn_fwd(const void* q, const void* k, const void* v, void* out, const int32_t* cu_seqlens_q,
+                                   const int32_t* cu_seqlens_k, float* softmax_lse, int64_t batch, int64_t heads,
+                                   int64_t head_dim, int64_t max_seqlen_q, int64_t max_seqlen_k, int64_t q_stride_t,
+                                   int64_t q_stride_h, int64_t k_stride_t, int64_t k_stride_h, int64_t v_stride_t,
+                                   int64_t v_stride_h, int64_t out_stride_t, int64_t out_stride_h, float softmax_scale,
+                                   int causal, int dropout_mode, float dropout_p, const uint8_t* dropout_mask,
+                                   uint8_t* dropout_mask_out, uint64_t seed, uint64_t offset, int dtype, void* stream) {
+  if (int rc = check_common("flash_attn_fwd", batch, heads, head_dim, max_seqlen_q, max_seqlen_k, dropout_mode, dropout_p, softmax_scale, dtype)) return rc;
+  if (batch == 0 || max_seqlen_q == 0) return 0;
+  NMTG_REQUIRE(q && k && v && out && cu_seqlens_q && cu_seqlens_k && softmax_lse, "flash_attn_fwd: null pointer argument");
+  NMTG_REQUIRE(dropout_mode != 1 || dropout_mask, "flash_attn_fwd: dropout mode 1 replays a keep-mask and none was given");
+  NMTG_REQUIRE(view_ok(q, q_stride_t, q_stride_h, heads, head_dim) && view_ok(k, k_stride_t, k_stride_h, heads, head_dim) &&
+                   view_ok(v, v_stride_t, v_stride_h, heads, head_dim) && view_ok(out, out_stride_t, out_stride_h, heads, head_dim),
+               "flash_attn_fwd: q, k, v and out must be 16-byte aligned [tokens, heads, head_dim] views with a contiguous "
+               "head_dim and strides that are multiples of 8 elements");
+  FaArgs a = {};
+  a.q = q; a.k = k; a.v = v; a.out = out; a.lse = softmax_lse; a.cu_q = cu_seqlens_q; a.cu_k = cu_seqlens_k;
+  a.q_st = q_stride_t; a.q_sh = q_stride_h; a.k_st = k_stride_t; a.k_sh = k_stride_h; a.v_st = v_stride_t; a.v_sh = v_stride_h;
+  a.o_st = out_stride_t; a.o_sh = out_stride_h;
+  a.heads = static_cast<int>(heads); a.max_q = static_cast<int>(max_seqlen_q); a.max_k = static_cast<int>(max_seqlen_k);
+  a.scale = softmax_scale; a.scale_log2 = softmax_scale * FA_LOG2E; a.causal = causal != 0;
+  a.mask = dropout_mask; a.mask_out = dropout_mask_out;
+  set_dropout(a, dropout_mode, dropout_p, seed, offset);
+  const dim3 grid(static_cast<unsigned>((max_seqlen_q + FA_ROWS - 1) / FA_ROWS), static_cast<unsigned>(heads), static_cast<unsigned>(batch));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  int rc;
+  if (dtype == NMTG_F16) rc = head_dim == 64 ? fwd_launch<f16_t, 64>(a, dropout_mode, grid, st) : fwd_launch<f16_t, 128>(a, dropout_mode, grid, st);
+  else rc = head_dim == 64 ? fwd_launch<bf16_t, 64>(a, dropout_mode, grid, st) : fwd_launch<bf16_t, 128>(a, dropout_mode, grid, st);
+  if (rc) return rc;
+  NMTG_CHECK_LAUNCH("flash_attn_fwd");
+  return 0;
+}
+
+extern "C" int nmtg_flash_attn_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out,
+                                   const float* softmax_lse, void* dq, void* dk, void* dv, float* softmax_d,
+                                   const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int64_t batch, int64_t heads,
+                                   int64_t head_dim, int64_t max_seqlen_q, int64_t max_seqlen_k, int64_t dout_stride_t,
+                                   int64_t dout_stride_h, int64_t q_stride_t, int64_t q_stride_h, int64_t k_stride_t,
+                                   int64_t k_stride_h, int64_t v_stride_t, int64_t v_stride_h, int64_t out_stride_t,
+                                   int64_t out_stride_h, int64_t dq_stride_t, int64_t dq_stride_h, int64_t dk_stride_t,
+                                   int64_t dk_stride_h, int64_t dv_stride_t, int64_t dv_stride_h, float softmax_scale,
+                                   int causal, int dropout_mode, float dropout_p, const uint8_t* dropout_mask,
+                                   uint64_t seed, uint64_t offset, int dtype, void* stream) {
+  if (int rc = check_common("flash_attn_bwd", batch, heads, head_dim, max_seqlen_q, max_seqlen_k, dropout_mode, dropout_p, softmax_scale, dtype)) return rc;
+  if (batch == 0) return 0;
+  NMTG_REQUIRE(dout && q && k && v && out && softmax_lse && dq && dk && dv && softmax_d && cu_seqlens_q && cu_seqlens_k,
+               "flash_attn_bwd: null pointer argument");
+  NMTG_REQUIRE(dropout_mode != 1 || dropout_mask, "flash_attn_bwd: dropout mode 1 replays a keep-mask and none was given");
+  NMTG_REQUIRE(view_ok(q, q_stride_t, q_stride_h, heads, head_dim) && view_ok(k, k_stride_t, k_stride_h, heads, head_dim) &&
+                   view_ok(v, v_stride_t, v_stride_h, heads, head_dim) && view_ok(out, out_stride_t, out_stride_h, heads, head_dim) &&
+                   view_ok(dout, dout_stride_t, dout_stride_h, heads, head_dim) && view_ok(dq, dq_stride_t, dq_stride_h, heads, head_dim) &&
+                   view_ok(dk, dk_stride_t, dk_stride_h, heads, head_dim) && view_ok(dv, dv_stride_t, dv_stride_h, heads, head_dim),
+               "flash_attn_bwd: every tensor must be a 16-byte aligned [tokens, heads, head_dim] view with a contiguous "
+               "head_dim and strides that are multiples of 8 elements");
+  FaArgs a = {};
+  a.q = q; a.k = k; a.v = v; a.o = out; a.d_o = dout; a.dq = dq; a.dk = dk; a.dv = dv;
+  a.lse = const_cast<float*>(softmax_lse); a.delta = softmax_d; a.cu_q = cu_seqlens_q; a.cu_k = cu_seqlens_k;
+  a.q_st = q_stride_t; a.q_sh = q_stride_h; a.k_st = k_stride_t; a.k_sh = k_stride_h; a.v_st = v_stride_t; a.v_sh = v_stride_h;
+  a.o_st = out_stride_t; a.o_sh = out_stride_h; a.do_st = dout_stride_t; a.do_sh = dout_stride_h;
+  a.dq_st = dq_stride_t; a.dq_sh = dq_stride_h; a.dk_st = dk_stride_t; a.dk_sh = dk_stride_h; a.dv_st = dv_stride_t; a.dv_sh = dv_stride_h;
+  a.heads = static_cast<int>(heads); a.max_q = static_cast<int>(max_seqlen_q); a.max_k = static_cast<int>(max_seqlen_k);
+  a.scale = softmax_scale; a.scale_log2 = softmax_scale * FA_LOG2E; a.causal = causal != 0;
+  a.mask = dropout_mask; a.mask_out = nullptr;
+  set_dropout(a, dropout_mode, dropout_p, seed, offset);
+  const dim3 grid_q(static_cast<unsigned>((max_seqlen_q + FA_ROWS - 1) / FA_ROWS), static_cast<unsigned>(heads), static_cast<unsigned>(batch));
+  const dim3 grid_k(static_cast<unsigned>((max_seqlen_k + FA_ROWS - 1) / FA_ROWS), static_cast<unsigned>(heads), static_cast<unsigned>(batch));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  int rc;
+  if (dtype == NMTG_F16) rc = head_dim == 64 ? bwd_launch<f16_t, 64>(a, dropout_mode, grid_q, grid_k, st) : bwd_launch<f16_t, 128>(a, dropout_mode, grid_q, grid_k, st);
+  else rc = head_dim == 64 ? bwd_launch<bf16_t, 64>(a, dropout_mode, grid_q, grid_k, st) : bwd_launch<bf16_t, 128>(a, dropout_mode, grid_q, grid_k, st);
+  if (rc) return rc;
+  NMTG_CHECK_LAUNCH("flash_attn_bwd");
+  return 0;
+}

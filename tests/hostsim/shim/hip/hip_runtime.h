@@ -101,6 +101,22 @@ static inline int __builtin_amdgcn_update_dpp(int, int src, int ctrl, int, int, 
 }
 static inline int __builtin_amdgcn_readlane(int v, int lane) { return static_cast<int>(hostsim::gather_bits(static_cast<uint32_t>(v), lane)); }
 
+// v_permlane32_swap_b32: lanes 32..63 of the first operand change places with lanes 0..31 of the second; returns both
+typedef unsigned int hostsim_u32x2 __attribute__((ext_vector_type(2)));
+static inline hostsim_u32x2 __builtin_amdgcn_permlane32_swap(unsigned int vdst, unsigned int vsrc, bool, bool) {
+  const int lane = static_cast<int>(hostsim::lane_id());
+  const unsigned int other_dst = static_cast<unsigned int>(hostsim::gather_bits(vdst, lane ^ 32));
+  const unsigned int other_src = static_cast<unsigned int>(hostsim::gather_bits(vsrc, lane ^ 32));
+  return lane < 32 ? hostsim_u32x2{vdst, other_dst} : hostsim_u32x2{other_src, vsrc};
+}
+
+// v_cmp into a wavefront-wide mask: bit l is lane l's predicate
+static inline uint64_t __builtin_amdgcn_ballot_w64(bool pred) {
+  uint64_t mask = 0;
+  for (int l = 0; l < 64; ++l) mask |= (hostsim::gather_bits(pred ? 1 : 0, l) & 1u) << l;
+  return mask;
+}
+
 static inline uint32_t __umulhi(uint32_t a, uint32_t b) { return static_cast<uint32_t>((static_cast<uint64_t>(a) * b) >> 32); }
 static inline float __uint_as_float(uint32_t u) { float f; std::memcpy(&f, &u, 4); return f; }
 static inline uint32_t __float_as_uint(float f) { uint32_t u; std::memcpy(&u, &f, 4); return u; }

@@ -43,6 +43,7 @@ import test_zz_golden_gpu as tgold  # noqa: E402
 import test_zzb_generator_loss_gpu as tgen  # noqa: E402
 import test_zzc_relative_attention_gpu as trel  # noqa: E402
 import test_zzd_fused_optim_gpu as topt  # noqa: E402
+import test_zze_flash_attention_gpu as tfl  # noqa: E402
 
 pytestmark = pytest.mark.skipif(not hostsim_build.available(), reason="no host C++ compiler with __bf16 (ROCm clang++)")
 CPU = torch.device("cpu")
@@ -596,6 +597,28 @@ def test_mlp_backward_with_one_reduction_launch(mi355x, dtype, tokens, dm, di):
 @long_case
 def test_three_layer_mlp_backward_with_one_reduction_launch(mi355x):
     tst.test_three_layer_mlp_backward_with_one_reduction_launch(CPU)
+
+
+# ----------------------------------------------------------------------------- attention over packed sequences
+@pytest.mark.parametrize("dtype", HALVES)
+@pytest.mark.parametrize("d,causal", [(64, False), (64, True), pytest.param(128, True, marks=long_case)])
+def test_packed_attention_ragged(dtype, d, causal):
+    tfl.test_ragged_self_attention_matches_the_oracle(CPU, dtype, d, causal)
+
+
+def test_packed_attention_unequal_lengths_and_empty_sequences():
+    tfl.test_different_query_and_key_lengths_and_an_empty_sequence(CPU, BF16)
+
+
+@pytest.mark.parametrize("dtype,d,causal", [(BF16, 64, True), pytest.param(F16, 128, False, marks=long_case)])
+def test_packed_attention_dropout_replay(dtype, d, causal):
+    tfl.test_dropout_with_a_replayed_mask(CPU, dtype, d, causal)
+
+
+def test_packed_attention_dropout_philox_and_autograd_functions():
+    tfl.test_dropout_drawn_on_the_device_is_the_documented_philox_stream_in_both_passes(CPU, F16, 64)
+    tfl.test_packed_qkv_function_takes_strided_slots_and_fills_one_gradient_tensor(CPU, BF16)
+    tfl.test_packed_kv_function_with_dropout_repeats_its_mask_in_the_backward(CPU)
 
 
 # ----------------------------------------------------------------------------- committed fixtures

@@ -662,3 +662,68 @@ def test_rotary_attention_reduces_to_plain_attention_at_angle_zero_and_to_a_per_
     q = orot.apply_rotary(ql[:, 0, 1][:, None], cq, sq)[:, 0]
     k = orot.apply_rotary(kl[:, 0, 1, 0][:, None], ck, sk)[:, 0]
     assert torch.allclose(ce[1], torch.softmax(q @ k.t() / 4.0, -1), atol=1e-12)
+
+
+# ----------------------------------------------------------------------------- attention over packed sequences
+def _packed_case(seed, lq, lk, heads=2, d=8):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(sum(lq), heads, d, generator=g, dtype=D)
+    k = torch.randn(sum(lk), heads, d, generator=g, dtype=D)
+    v = torch.randn(sum(lk), heads, d, generator=g, dtype=D)
+    do = torch.randn(sum(lq), heads, d, generator=g, dtype=D)
+    cu = lambda n: torch.tensor([0] + list(torch.cumsum(torch.tensor(n), 0)), dtype=torch.int32)
+    return q, k, v, do, cu(lq), cu(lk)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_packed_attention_is_library_attention_on_every_sequence_by_itself(causal):
+    from oracle import flash_attention as ofa
+    lq = lk = [5, 1, 9]                                     # causal in the library aligns the first tokens too
+    q, k, v, do, cu_q, cu_k = _packed_case(501, lq, lk)
+    scale = 0.37
+    out, lse = ofa.flash_attn_fwd(q, k, v, cu_q, cu_k, max(lq), scale, causal)
+    dq, dk, dv, delta = ofa.flash_attn_bwd(do, q, k, v, cu_q, cu_k, max(lq), scale, causal)
+    for b in range(3):
+        sq, sk = slice(int(cu_q[b]), int(cu_q[b + 1])), slice(int(cu_k[b]), int(cu_k[b + 1]))
+        qb, kb, vb = (t.transpose(0, 1).clone().requires_grad_() for t in (q[sq], k[sk], v[sk]))       # [H, L, D]
+        lib = F.scaled_dot_product_attention(qb, kb, vb, is_causal=causal, scale=scale)
+        lib.backward(do[sq].transpose(0, 1))
+        assert torch.allclose(out[sq].transpose(0, 1), lib.detach(), atol=1e-12)
+        assert torch.allclose(dq[sq].transpose(0, 1), qb.grad, atol=1e-12)
+        assert torch.allclose(dk[sk].transpose(0, 1), kb.grad, atol=1e-12)
+        assert torch.allclose(dv[sk].transpose(0, 1), vb.grad, atol=1e-12)
+        s = torch.einsum("hid,hjd->hij", qb.detach(), kb.detach()) * scale
+        if causal:
+            s = s.masked_fill(torch.ones(lq[b], lk[b], dtype=torch.bool).triu(1), -math.inf)
+        assert torch.allclose(lse[b, :, :lq[b]], torch.logsumexp(s, -1), atol=1e-12)
+        assert bool((lse[b, :, lq[b]:] == 0).all())
+        # D = rowsum(dO * O) = rowsum(P * dP): the identity the backward kernels rest on
+        dp = torch.einsum("hid,hjd->hij", do[sq].transpose(0, 1), vb.detach())
+        assert torch.allclose(delta[b, :, :lq[b]], (torch.softmax(s, -1) * dp).sum(-1), atol=1e-12)
+
+
+def test_packed_attention_with_unequal_lengths_dropout_and_an_empty_sequence_by_loops():
+    from oracle import flash_attention as ofa
+    lq, lk = [3, 2, 4], [5, 0, 2]
+    q, k, v, do, cu_q, cu_k = _packed_case(502, lq, lk, heads=1, d=4)
+    p = 0.25
+    keep = (torch.rand(3, 1, max(lq), max(lk), generator=torch.Generator().manual_seed(7)) < 0.75).to(torch.uint8)
+    out, lse = ofa.flash_attn_fwd(q, k, v, cu_q, cu_k, max(lq), None, True, p, keep)
+    for b in range(3):
+        for i in range(lq[b]):
+            row = torch.zeros(4, dtype=D)
+            visible = [j for j in range(lk[b]) if j <= i]                        # causal: aligned at the first tokens
+            z = sum(math.exp(float(q[cu_q[b] + i, 0] @ k[cu_k[b] + j, 0]) * 0.5) for j in visible)     # scale 1 / sqrt(4)
+            for j in visible:
+                pr = math.exp(float(q[cu_q[b] + i, 0] @ k[cu_k[b] + j, 0]) * 0.5) / z
+                row += pr * float(keep[b, 0, i, j]) / (1 - p) * v[cu_k[b] + j, 0]      # dropout after the normalisation
+            assert torch.allclose(out[cu_q[b] + i, 0], row, atol=1e-12), (b, i)
+            assert (math.isinf(float(lse[b, 0, i])) and lse[b, 0, i] < 0) if not visible else abs(float(lse[b, 0, i]) - math.log(z)) < 1e-12
+    # the gradient of that loop, by finite differences on one element of each input
+    dq, dk, dv, _ = ofa.flash_attn_bwd(do, q, k, v, cu_q, cu_k, max(lq), None, True, p, keep)
+    f = lambda q_, k_, v_: float((ofa.flash_attn_fwd(q_, k_, v_, cu_q, cu_k, max(lq), None, True, p, keep)[0] * do).sum())
+    for t, gr, idx in ((q, dq, (1, 0, 2)), (k, dk, (0, 0, 1)), (v, dv, (6, 0, 3)), (q, dq, (4, 0, 0))):
+        e = torch.zeros_like(t)
+        e[idx] = 1e-6
+        args = lambda s: [x + s * e if x is t else x for x in (q, k, v)]
+        assert abs((f(*args(1)) - f(*args(-1))) / 2e-6 - float(gr[idx])) < 1e-7, idx
