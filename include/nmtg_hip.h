@@ -217,6 +217,11 @@ int nmtg_mlp_fwd(int num_layers, const void* x, const void* const* weights,
 
 int64_t nmtg_mlp_bwd_workspace_bytes(int num_layers, const int64_t* out_features, int64_t batch,
                                      int64_t in_features);
+/* The same for a given element type: fp32 (the precision of the reference's own MLP tests,
+ * onmt/modules/mlp/test_mlp_gelu.py:229-307) needs twice the room for the hidden gradients; the
+ * function above sizes for the 16-bit types. */
+int64_t nmtg_mlp_bwd_dtype_workspace_bytes(int num_layers, const int64_t* out_features,
+                                           int64_t batch, int64_t in_features, int dtype);
 
 /* grad_x may be NULL (the reference skips it when x does not require grad); grad_weights /
  * grad_biases may be NULL or hold NULL entries (backward_input_only). mask NULL or p == 0: no

@@ -1004,6 +1004,8 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
              int* m_tiles_out = nullptr, GemmArgs* planned_out = nullptr);
 // planned_out (optional) receives the arguments as launched (splits, tiles, vec, ws, tile_used): with a.defer_reduce
 // set and planned_out->splits > 1 the caller owes the reduction of the partials (tail_add_splitk).
+// dtype NMTG_F32 goes to the fp32 matrix-core kernel (gemm_f32.hip): plain and the two activation epilogues, no split-K.
+int gemm_f32_run(int layout, int epi, GemmArgs a, hipStream_t st, int* m_tiles_out, GemmArgs* planned_out);
 
 // Fused Q K^T -> mask -> softmax -> dropout (EPI_SCORES_SOFTMAX) for rows of at most 512 keys. `a` is filled as
 // for EPI_SCORES plus out2 (dropped probabilities), aux_out (softmax, optional), dmask / rng / keep_p / dscale /

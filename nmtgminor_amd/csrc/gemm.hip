@@ -78,6 +78,7 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
   if (a.M <= 0 || a.N <= 0 || a.batch <= 0) return 0;
   if (a.K < 0) return fail(NMTG_ERR_INVALID, "gemm: negative K");
   if (!a.A || !a.B || !a.C) return fail(NMTG_ERR_INVALID, "gemm: null operand pointer");
+  if (dtype == NMTG_F32) return gemm_f32_run(layout, epi, a, st, m_tiles_out, planned_out);
   const bool a_kc = layout != LAYOUT_TN;
   const bool b_kc = layout == LAYOUT_NT;
   // Widest access (8, 4 or 1 elements) that every pointer, pitch and batch stride of this call allows. Extents do not

@@ -36,7 +36,7 @@ struct BwdPlan {
   size_t total() const { return 2 * dh_bytes + layers * (colsum_bytes + splitk_bytes); }
 };
 
-BwdPlan plan_bwd(int num_layers, const int64_t* out_features, int64_t batch, int64_t in_features) {
+BwdPlan plan_bwd(int num_layers, const int64_t* out_features, int64_t batch, int64_t in_features, size_t esz) {
   BwdPlan p{0, 0, 0, num_layers};
   int64_t max_hidden = 0, max_out = 0;
   for (int i = 0; i < num_layers; ++i) {
@@ -47,7 +47,7 @@ BwdPlan plan_bwd(int num_layers, const int64_t* out_features, int64_t batch, int
                                                                           static_cast<int>(in_i),
                                                                           static_cast<int>(batch), 1));
   }
-  p.dh_bytes = align_up(static_cast<size_t>(batch) * max_hidden * 2);
+  p.dh_bytes = align_up(static_cast<size_t>(batch) * max_hidden * esz);
   const size_t parts = static_cast<size_t>(std::max<int64_t>(colsum_parts(static_cast<int>(batch)), (batch + 127) / 128));
   p.colsum_bytes = align_up(parts * max_out * sizeof(float));
   p.splitk_bytes = align_up(p.splitk_bytes);
@@ -62,7 +62,7 @@ int check_shapes(const char* who, int num_layers, const int64_t* out_features, i
   NMTG_REQUIRE(batch >= 0 && batch <= INT32_MAX && in_features > 0 && in_features <= INT32_MAX, "%s: bad input shape", who);
   for (int i = 0; i < num_layers; ++i)
     NMTG_REQUIRE(out_features[i] > 0 && out_features[i] <= INT32_MAX, "%s: bad out_features[%d]", who, i);
-  NMTG_REQUIRE(dtype == NMTG_F16 || dtype == NMTG_BF16, "%s: dtype %d not supported (fp16 and bf16 run on MFMA)", who, dtype);
+  NMTG_REQUIRE(dtype == NMTG_F16 || dtype == NMTG_BF16 || dtype == NMTG_F32, "%s: dtype %d not supported (fp32, fp16 and bf16 are)", who, dtype);
   NMTG_REQUIRE(act >= NMTG_ACT_NONE && act <= NMTG_ACT_AGELU, "%s: unknown activation %d", who, act);
   return 0;
 }
@@ -87,6 +87,7 @@ extern "C" int nmtg_mlp_fwd(int num_layers, const void* x, const void* const* we
   hipStream_t st = static_cast<hipStream_t>(stream);
   const void* in = x;
   int64_t in_f = in_features;
+  const int64_t esz = dtype == NMTG_F32 ? 4 : 2;
   int64_t elt_off = 0;  // element offset into the concatenated hidden buffers
   for (int i = 0; i < num_layers; ++i) {
     NMTG_REQUIRE(weights[i] != nullptr, "mlp_fwd: weights[%d] is null", i);
@@ -103,8 +104,8 @@ extern "C" int nmtg_mlp_fwd(int num_layers, const void* x, const void* const* we
       g.C = out;
       rc = gemm_run(dtype, LAYOUT_NT, EPI_PLAIN, g, nullptr, 0, st);
     } else {
-      g.C = static_cast<uint8_t*>(post_acts) + elt_off * 2;
-      g.aux_out = pre_acts ? static_cast<uint8_t*>(pre_acts) + elt_off * 2 : nullptr;
+      g.C = static_cast<uint8_t*>(post_acts) + elt_off * esz;
+      g.aux_out = pre_acts ? static_cast<uint8_t*>(pre_acts) + elt_off * esz : nullptr;
       g.act = act;
       if (mask_mode != 0) {
         g.dmask = mask + elt_off;
@@ -127,7 +128,13 @@ extern "C" int nmtg_mlp_fwd(int num_layers, const void* x, const void* const* we
 extern "C" int64_t nmtg_mlp_bwd_workspace_bytes(int num_layers, const int64_t* out_features, int64_t batch,
                                                 int64_t in_features) {
   if (num_layers < 1 || num_layers > MAX_LAYERS || !out_features || batch <= 0 || in_features <= 0) return 0;
-  return static_cast<int64_t>(plan_bwd(num_layers, out_features, batch, in_features).total());
+  return static_cast<int64_t>(plan_bwd(num_layers, out_features, batch, in_features, 2).total());
+}
+
+extern "C" int64_t nmtg_mlp_bwd_dtype_workspace_bytes(int num_layers, const int64_t* out_features, int64_t batch,
+                                                      int64_t in_features, int dtype) {
+  if (num_layers < 1 || num_layers > MAX_LAYERS || !out_features || batch <= 0 || in_features <= 0) return 0;
+  return static_cast<int64_t>(plan_bwd(num_layers, out_features, batch, in_features, dtype == NMTG_F32 ? 4 : 2).total());
 }
 
 extern "C" int nmtg_mlp_bwd(int num_layers, const void* x, const void* const* weights, const int64_t* out_features,
@@ -142,7 +149,8 @@ extern "C" int nmtg_mlp_bwd(int num_layers, const void* x, const void* const* we
   NMTG_REQUIRE(num_layers == 1 || pre_acts != nullptr || act == NMTG_ACT_RELU || act == NMTG_ACT_NONE,
                "mlp_bwd: pre-activation buffer required for this activation");
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const BwdPlan plan = plan_bwd(num_layers, out_features, std::max<int64_t>(batch, 1), in_features);
+  const int64_t esz = dtype == NMTG_F32 ? 4 : 2;
+  const BwdPlan plan = plan_bwd(num_layers, out_features, std::max<int64_t>(batch, 1), in_features, static_cast<size_t>(esz));
   NMTG_REQUIRE(workspace != nullptr && static_cast<size_t>(std::max<int64_t>(workspace_bytes, 0)) >= plan.total() &&
                    (reinterpret_cast<uintptr_t>(workspace) & 255u) == 0,
                "mlp_bwd: workspace of %zu bytes (256-byte aligned) required, got %lld", plan.total(),
@@ -171,7 +179,7 @@ extern "C" int nmtg_mlp_bwd(int num_layers, const void* x, const void* const* we
   for (int i = num_layers - 1; i >= 0; --i) {
     const int64_t out_i = out_features[i];
     const int64_t in_i = i == 0 ? in_features : out_features[i - 1];
-    const void* input_i = i == 0 ? x : static_cast<const uint8_t*>(post_acts) + offs[i - 1] * 2;
+    const void* input_i = i == 0 ? x : static_cast<const uint8_t*>(post_acts) + offs[i - 1] * esz;
     int rc;
     // bias gradient (its partial rows: written by the data-gradient GEMM of the layer above, or by a kernel of its own)
     float* colsum_ws = colsum_region(i);
@@ -217,8 +225,8 @@ extern "C" int nmtg_mlp_bwd(int num_layers, const void* x, const void* const* we
       g.batch = 1; g.alpha = 1.f;
       g.act = act;
       const bool have_pre = pre_acts != nullptr;
-      g.aux_in = have_pre ? static_cast<const uint8_t*>(pre_acts) + offs[i - 1] * 2
-                          : static_cast<const uint8_t*>(post_acts) + offs[i - 1] * 2;
+      g.aux_in = have_pre ? static_cast<const uint8_t*>(pre_acts) + offs[i - 1] * esz
+                          : static_cast<const uint8_t*>(post_acts) + offs[i - 1] * esz;
       g.ld_aux = in_i;
       g.dscale = 1.f;
       if (have_pre) {

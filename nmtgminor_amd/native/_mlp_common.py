@@ -33,8 +33,8 @@ def _ptr_array(tensors):
 
 def _validate(x, weights, biases):
     L.require_cuda(x, *weights, *biases)
-    _check(x.dtype in (torch.float16, torch.bfloat16),
-           "mlp: fp16 and bf16 are supported (the MFMA path has no fp32 / fp64 kernels)")
+    _check(x.dtype in (torch.float16, torch.bfloat16, torch.float32),
+           "mlp: fp32, fp16 and bf16 are supported (there is no fp64 kernel)")
     in_f = x.shape[-1]
     for w, b in zip(weights, biases):
         _check(w.dtype == x.dtype and w.dim() == 2 and w.shape[1] == in_f, "mlp: weight shape / dtype mismatch")
@@ -105,7 +105,7 @@ def backward(act, p, grad_o, post, pre, mask, inputs, input_only=False, need_dx=
         dx_empty = dx.view(x.shape) if dx is not None else None
         return [dx_empty] if input_only else [dx_empty] + dws + dbs
     of = (ctypes.c_int64 * n)(*outs)
-    ws_bytes = int(L.load().nmtg_mlp_bwd_workspace_bytes(L.i32(n), of, L.i64(batch), L.i64(in_f)))
+    ws_bytes = int(L.load().nmtg_mlp_bwd_dtype_workspace_bytes(L.i32(n), of, L.i64(batch), L.i64(in_f), L.i32(L.dtype_code(x))))
     ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
     use_mask = mask is not None and mask.numel() > 0 and p > 0.0
     have_pre = pre is not None and pre.numel() > 0

@@ -19,8 +19,8 @@ def gemm(a, b, trans_a=False, trans_b=False, alpha=1.0, bias=None, out=None, spl
         raise RuntimeError("gemm: operands must be [batch, rows, cols] with equal batch")
     if a3.stride(2) != 1 or b3.stride(2) != 1:
         raise RuntimeError("gemm: innermost stride must be 1")
-    if a3.dtype != b3.dtype or a3.dtype not in (torch.float16, torch.bfloat16):
-        raise RuntimeError("gemm: fp16 or bf16 operands of one dtype required")
+    if a3.dtype != b3.dtype or a3.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+        raise RuntimeError("gemm: fp32, fp16 or bf16 operands of one dtype required")
     batch = a3.shape[0]
     m, k = (a3.shape[2], a3.shape[1]) if trans_a else (a3.shape[1], a3.shape[2])
     kb, n = (b3.shape[2], b3.shape[1]) if trans_b else (b3.shape[1], b3.shape[2])
@@ -36,7 +36,7 @@ def gemm(a, b, trans_a=False, trans_b=False, alpha=1.0, bias=None, out=None, spl
         return out if a.dim() == 3 else o3[0]
     ws = None
     ws_bytes = 0
-    if split_k and trans_a and not trans_b:
+    if split_k and trans_a and not trans_b and a3.dtype != torch.float32:      # the fp32 kernel never splits K
         ws_bytes = int(L.load().nmtg_gemm_workspace_bytes(L.i64(m), L.i64(n), L.i64(k), L.i64(batch)))
         if ws_bytes:
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a3.device)

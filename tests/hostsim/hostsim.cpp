@@ -303,6 +303,24 @@ static void resolve_mfma(void** payloads, int lanes) {
     }
   }
 }
+// v_mfma_f32_32x32x2_f32: lane l holds A[l & 31][l >> 5] and B[l >> 5][l & 31]
+void resolve_mfma_f32(void** payloads, int lanes) {
+  if (lanes != 64) fail("MFMA in a partial wavefront");
+  float A[32][2], B[2][32];
+  for (int l = 0; l < 64; ++l) {
+    const MfmaF32* m = static_cast<const MfmaF32*>(payloads[l]);
+    A[l & 31][l >> 5] = m->a;
+    B[l >> 5][l & 31] = m->b;
+  }
+  for (int l = 0; l < 64; ++l) {
+    float* c = static_cast<MfmaF32*>(payloads[l])->c;
+    const int j = l & 31;
+    for (int r = 0; r < 16; ++r) {
+      const int i = 8 * (r / 4) + 4 * (l >> 5) + r % 4;
+      c[r] = std::fmaf(A[i][1], B[1][j], std::fmaf(A[i][0], B[0][j], c[r]));
+    }
+  }
+}
 void resolve_mfma_f16(void** payloads, int lanes) { resolve_mfma<false>(payloads, lanes); }
 void resolve_mfma_bf16(void** payloads, int lanes) { resolve_mfma<true>(payloads, lanes); }
 

@@ -196,6 +196,19 @@ static inline hostsim_float16 mfma(V a, V b, hostsim_float16 c) {
   return d;
 }
 }  // namespace hostsim
+namespace hostsim {
+struct MfmaF32 { float a, b; float* c; };
+void resolve_mfma_f32(void** payloads, int lanes);
+}  // namespace hostsim
+static inline hostsim_float16 __builtin_amdgcn_mfma_f32_32x32x2f32(float a, float b, hostsim_float16 c, int, int, int) {
+  float cv[16];
+  std::memcpy(cv, &c, 64);
+  hostsim::MfmaF32 m{a, b, cv};
+  hostsim::wave_collective(hostsim::resolve_mfma_f32, &m);
+  hostsim_float16 d;
+  std::memcpy(&d, cv, 64);
+  return d;
+}
 typedef _Float16 hostsim_half8 __attribute__((ext_vector_type(8)));
 typedef __bf16 hostsim_bf16x8 __attribute__((ext_vector_type(8)));
 static inline hostsim_float16 __builtin_amdgcn_mfma_f32_32x32x16_f16(hostsim_half8 a, hostsim_half8 b, hostsim_float16 c, int, int, int) {

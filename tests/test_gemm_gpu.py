@@ -69,6 +69,35 @@ def test_gemm_bias_and_batched_strided_views(dev):
     assert_close(gemm(x, w, False, True, bias=bias), _ref(x, w, False, True, 1.0, bias).cpu(), dtype, "bias", scale_atol=True)
 
 
+@pytest.mark.parametrize("m,n,k", [(256, 256, 64), (300, 200, 72), (1, 8, 8), (257, 129, 1000), (130, 70, 33), (1024, 64, 512)])
+@pytest.mark.parametrize("layout", ["nt", "nn", "tn"])
+def test_gemm_fp32_layouts_against_fp64(dev, m, n, k, layout):
+    """The fp32 matrix-core kernel: fp32 products and sums, so the yardstick is the fp64 product of the same operands
+    (rtol 1e-5 with an absolute part of 1e-6 times the largest result: the rounding of a sum over k terms)."""
+    ta, tb = layout[0] == "t", layout[1] == "t"
+    a = _mk((k, m) if ta else (m, k), dev, torch.float32, 21)
+    b = _mk((n, k) if tb else (k, n), dev, torch.float32, 22)
+    bias = _mk((n,), dev, torch.float32, 23)
+    c = gemm(a, b, ta, tb, alpha=0.5, bias=bias)
+    ad, bd = a.double().cpu(), b.double().cpu()
+    want = 0.5 * ((ad.t() if ta else ad) @ (bd.t() if tb else bd)) + bias.double().cpu()
+    assert_close(c, want, torch.float32, f"fp32 {layout} {m}x{n}x{k}", rtol=1e-5, atol=1e-6, scale_atol=True)
+
+
+def test_gemm_fp32_batched_strided_views(dev):
+    t, bh, d = 40, 3, 24
+    qkv = _mk((t, bh, 3, d), dev, torch.float32, 24)
+    q, k, v = (qkv[:, :, i, :].transpose(0, 1) for i in range(3))      # [bh, t, d] views, row stride bh*3*d
+    s = gemm(q, k, False, True, alpha=0.25)
+    assert_close(s, 0.25 * (q.double() @ k.double().transpose(1, 2)).cpu(), torch.float32, "scores", rtol=1e-5, atol=1e-6, scale_atol=True)
+    out = torch.empty(t, bh, d, dtype=torch.float32, device=dev)
+    gemm(s, v, False, False, out=out.transpose(0, 1))
+    assert_close(out.transpose(0, 1), (s.double() @ v.double()).cpu(), torch.float32, "context", rtol=1e-5, atol=1e-6, scale_atol=True)
+    dv = gemm(s, out.transpose(0, 1), True, False)
+    assert_close(dv, (s.double().transpose(1, 2) @ out.transpose(0, 1).double()).cpu(), torch.float32, "tn", rtol=1e-5, atol=1e-6,
+                 scale_atol=True)
+
+
 def test_gemm_split_k_is_deterministic(dev):
     a, b = _mk((8192, 512), dev, torch.float16, 11), _mk((8192, 256), dev, torch.float16, 12)
     c1 = gemm(a, b, True, False)
@@ -82,7 +111,7 @@ def test_gemm_split_k_is_deterministic(dev):
 def test_gemm_errors(dev):
     a = torch.randn(8, 8, device=dev)
     with pytest.raises(RuntimeError):
-        gemm(a, a)                                        # fp32 is not an MFMA input type here
+        gemm(a.double(), a.double())                      # there is no fp64 kernel
     h = a.half()
     with pytest.raises(RuntimeError):
         gemm(h, h, True, True)                            # A^T B^T not provided

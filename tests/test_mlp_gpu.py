@@ -135,12 +135,53 @@ def test_mlp_three_layers_and_rng_mask(dev):
         assert_close(grads[4 + i], dbs[i], torch.float16, f"3-layer db{i}", scale_atol=True)
 
 
+# fp32: the precision the reference's own MLP tests run in (test_mlp_gelu.py:262-300: sizes [1024, 4096, 1024], a
+# token count drawn as a multiple of 8, dropout 0 / 0.2 / 0.5 / 0.7, output atol = rtol = 1e-3, gradients rtol 1e-5 on
+# a loss scaled to make them tiny). Here against the fp64 oracle at rtol 1e-4, atol 1e-5 (times the largest expected
+# magnitude for the sums over tokens): fp32 products summed over up to 4096 terms, and a gelu whose normal CDF is
+# accurate to 1.5e-7.
+F32 = dict(rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("act,tokens,dm,di,p", [("gelu", 520, 1024, 4096, 0.0), ("gelu", 520, 1024, 4096, 0.2),
+                                                ("gelu", 136, 1024, 4096, 0.7), ("relu", 72, 96, 200, 0.5),
+                                                ("silu", 257, 130, 66, 0.2), ("agelu", 64, 33, 129, 0.0)])
+def test_mlp_fp32(dev, act, tokens, dm, di, p):
+    dtype = torch.float32
+    d = inputs.mlp_inputs(tokens, dm, di, dtype, p=p, seed=67, zero_bias=False)
+    fn = getattr(mmlp, f"mlp_{act}_function")
+    leaves = [d[k].to(dev).requires_grad_() for k in ("x", "w1", "w2", "b1", "b2")]
+    y = fn(p, False, *leaves, mask=d["mask"].to(dev) if p > 0 else None)
+    y.backward(d["dy"].to(dev))
+    gpost = None
+    if act == "relu":
+        _, gpost, _ = fused_mlp_relu.forward(p, False, [t.detach() for t in leaves], d["mask"].to(dev) if p > 0 else None)
+    wy, _, _, wdx, wdws, wdbs = _oracle(d, act, p, [d["mask"]] if p > 0 else None, gate_from=gpost)
+    assert_close(y, wy, dtype, "y", **F32)
+    assert_close(leaves[0].grad, wdx, dtype, "dx", scale_atol=True, **F32)
+    for i in range(2):
+        assert_close(leaves[1 + i].grad, wdws[i], dtype, f"dW{i + 1}", scale_atol=True, **F32)
+        assert_close(leaves[3 + i].grad, wdbs[i], dtype, f"db{i + 1}", scale_atol=True, **F32)
+
+
+def test_mlp_fp32_draws_the_same_dropout_stream_as_the_16_bit_kernels(dev):
+    d = inputs.mlp_inputs(96, 64, 128, torch.float32, p=0.3, seed=68, zero_bias=False)
+    ins = [d[k].to(dev) for k in ("x", "w1", "w2", "b1", "b2")]
+    torch.cuda.manual_seed(77)
+    _, post, _, mask32 = fused_mlp_gelu.forward(0.3, ins)
+    torch.cuda.manual_seed(77)
+    _, _, _, mask16 = fused_mlp_gelu.forward(0.3, [t.half() for t in ins])
+    assert torch.equal(mask32, mask16)
+    assert 0.6 < float(mask32.float().mean()) < 0.8
+    assert bool((post.view(96, 128)[mask32.view(96, 128) == 0] == 0).all())
+
+
 def test_mlp_errors(dev):
     x = torch.randn(8, 16, device=dev)
     w1, w2 = torch.randn(32, 16, device=dev), torch.randn(16, 32, device=dev)
     b1, b2 = torch.zeros(32, device=dev), torch.zeros(16, device=dev)
     with pytest.raises(RuntimeError):
-        fused_mlp_gelu.forward(0.0, [x, w1, w2, b1, b2])                   # fp32 has no MFMA kernel here
+        fused_mlp_gelu.forward(0.0, [t.double() for t in (x, w1, w2, b1, b2)])   # there is no fp64 kernel
     h = [t.half() for t in (x, w1, w2, b1, b2)]
     with pytest.raises(RuntimeError):
         fused_mlp_gelu.forward(0.0, [h[0], h[2], h[1], h[3], h[4]])        # weight shapes do not chain
