@@ -381,6 +381,27 @@ int nmtg_flash_attn_bwd(const void* dout, const void* q, const void* k, const vo
                         int dtype, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Gated feed-forward activation with dropout.
+ * Reference: the gated branch of PositionWiseFeedForward.forward, PyTorch ops there
+ *   (onmt/modules/optimized/feed_forward.py:188-200), and variational_dropout
+ *   (onmt/modules/dropout.py:32-48).
+ * x [rows, 2 * inner] (row pitch ld_x elements): a = x[:, :inner], b = x[:, inner:];
+ *   act = an nmtg_act code: y = act(a) * b;   act = 5: y = a * sigmoid(b)  (F.glu);
+ * then y <- y * keep / (1 - p). dropout_mode 0 none, 1 read `mask`, 2 draw it from Philox
+ * (element index row * inner + j, as the other dropout kernels) and store it. mask is uint8
+ * [mask_rows, inner]; row m uses mask row m % mask_rows: mask_rows == rows is ordinary dropout,
+ * mask_rows == batch over a [time, batch, inner] tensor the reference's variational dropout.
+ * y [rows, inner] dense. nmtg_glu_bwd: grad_x [rows, 2 * inner] (pitch ld_grad_x) from grad_y.
+ * ------------------------------------------------------------------------------------------ */
+int nmtg_glu_fwd(const void* x, int64_t ld_x, void* y, uint8_t* mask, int64_t mask_rows,
+                 int64_t rows, int64_t inner, int act, int dropout_mode, float p, uint64_t seed,
+                 uint64_t offset, int dtype, void* stream);
+
+int nmtg_glu_bwd(const void* grad_y, const void* x, int64_t ld_x, const uint8_t* mask,
+                 int64_t mask_rows, void* grad_x, int64_t ld_grad_x, int64_t rows, int64_t inner,
+                 int act, int dropout_mode, float p, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Column sums of a row-major matrix: out[c] = sum_r x[r * ld + c], fp32 accumulation in a fixed
  * order (partial sums per block of rows, then one sum over the partials), result in the dtype
  * of x. The bias gradients of the reference's linear layers: torch.sum(grads, 0)

@@ -44,6 +44,7 @@ import test_zzb_generator_loss_gpu as tgen  # noqa: E402
 import test_zzc_relative_attention_gpu as trel  # noqa: E402
 import test_zzd_fused_optim_gpu as topt  # noqa: E402
 import test_zze_flash_attention_gpu as tfl  # noqa: E402
+import test_zzf_feed_forward_gpu as tff  # noqa: E402
 
 pytestmark = pytest.mark.skipif(not hostsim_build.available(), reason="no host C++ compiler with __bf16 (ROCm clang++)")
 CPU = torch.device("cpu")
@@ -619,6 +620,35 @@ def test_packed_attention_dropout_philox_and_autograd_functions():
     tfl.test_dropout_drawn_on_the_device_is_the_documented_philox_stream_in_both_passes(CPU, F16, 64)
     tfl.test_packed_qkv_function_takes_strided_slots_and_fills_one_gradient_tensor(CPU, BF16)
     tfl.test_packed_kv_function_with_dropout_repeats_its_mask_in_the_backward(CPU)
+
+
+# ----------------------------------------------------------------------------- gated / variational feed-forward, fp32 products
+@pytest.mark.parametrize("dtype", [BF16, F32])
+@pytest.mark.parametrize("act,rows,inner,p", [("gelu", 37, 72, 0.25), ("sigmoid", 5, 7, 0.5), ("relu", 64, 256, 0.0)])
+def test_gated_activation_kernel(dtype, act, rows, inner, p):
+    tff.test_gated_activation_kernel(CPU, dtype, act, rows, inner, p)
+
+
+def test_gated_activation_kernel_pitched_shared_mask_and_philox():
+    tff.test_gated_activation_kernel_on_a_pitched_input_with_a_mask_row_per_batch_column(CPU)
+    tff.test_gated_activation_kernel_draws_the_documented_philox_stream(CPU, 9, 10)
+
+
+@pytest.mark.parametrize("act,glu,residual", [("gelu", False, True), ("silu", True, False)])
+def test_feed_forward_layer_variants(mi355x, act, glu, residual):
+    tff.test_variational_dropout_uses_one_mask_row_per_batch_column(CPU, act, glu, residual)
+    tff.test_gated_layer_in_evaluation_mode(CPU, BF16, act if glu else "sigmoid")
+
+
+@pytest.mark.parametrize("act,tokens,dm,di,p", [("relu", 72, 96, 200, 0.5), ("agelu", 64, 33, 129, 0.0)])
+def test_mlp_fp32(mi355x, act, tokens, dm, di, p):
+    tm.test_mlp_fp32(CPU, act, tokens, dm, di, p)
+
+
+@pytest.mark.parametrize("layout", ["nt", "nn", "tn"])
+def test_gemm_fp32(mi355x, layout):
+    tg.test_gemm_fp32_layouts_against_fp64(CPU, 130, 70, 33, layout)
+    tg.test_gemm_fp32_batched_strided_views(CPU)
 
 
 # ----------------------------------------------------------------------------- committed fixtures

@@ -727,3 +727,46 @@ def test_packed_attention_with_unequal_lengths_dropout_and_an_empty_sequence_by_
         e[idx] = 1e-6
         args = lambda s: [x + s * e if x is t else x for x in (q, k, v)]
         assert abs((f(*args(1)) - f(*args(-1))) / 2e-6 - float(gr[idx])) < 1e-7, idx
+
+
+# ----------------------------------------------------------------------------- gated / variational feed-forward
+@pytest.mark.parametrize("act", ["relu", "gelu", "silu", "agelu", "sigmoid"])
+def test_gated_feed_forward_is_the_chain_of_library_ops(act):
+    from oracle import feed_forward as off
+    g = torch.Generator().manual_seed(601)
+    t, b, dm, di = 5, 3, 8, 6
+    x = torch.randn(t, b, dm, generator=g, dtype=D)
+    w_in, b_in = torch.randn(2 * di, dm, generator=g, dtype=D), torch.randn(2 * di, generator=g, dtype=D)
+    w_out, b_out = torch.randn(dm, di, generator=g, dtype=D), torch.randn(dm, generator=g, dtype=D)
+    got = off.feed_forward(x, w_in, b_in, w_out, b_out, act, glu=True)
+    lin = F.linear(x, w_in, b_in)
+    if act == "sigmoid":
+        hidden = F.glu(lin)                                   # the reference's act for 'sigmoid' (feed_forward.py:57-58)
+    else:
+        a, gate = lin.chunk(2, dim=-1)
+        fn = {"relu": F.relu, "gelu": F.gelu, "silu": F.silu, "agelu": lambda v: F.gelu(v, approximate="tanh")}[act]
+        hidden = fn(a) * gate
+    assert torch.allclose(got, F.linear(hidden, w_out, b_out), atol=1e-12)
+
+
+def test_variational_dropout_shares_one_mask_row_over_time_and_the_residual_form_adds_the_input():
+    from oracle import feed_forward as off
+    g = torch.Generator().manual_seed(602)
+    t, b, dm, di, p = 4, 3, 6, 10, 0.25
+    x = torch.randn(t, b, dm, generator=g, dtype=D)
+    w_in, b_in = torch.randn(di, dm, generator=g, dtype=D), torch.randn(di, generator=g, dtype=D)
+    w_out, b_out = torch.randn(dm, di, generator=g, dtype=D), torch.randn(dm, generator=g, dtype=D)
+    keep = (torch.rand(1, b, di, generator=g) < 0.75).to(D)
+    res_keep = (torch.rand(1, b, dm, generator=g) < 0.75).to(D)
+    got = off.feed_forward(x, w_in, b_in, w_out, b_out, "relu", False, p, keep, True, p, res_keep)
+    for ti in range(t):                                       # time step by time step, the same mask row each time
+        h = F.relu(F.linear(x[ti], w_in, b_in)) * keep[0] / (1 - p)
+        o = F.linear(h, w_out, b_out) * res_keep[0] / (1 - p) + x[ti]
+        assert torch.allclose(got[ti], o, atol=1e-12)
+    # and what variational_dropout is for: E[mask / (1 - p)] = 1, so the expectation over masks is the undropped layer
+    plain = off.feed_forward(x, w_in, b_in, w_out, b_out, "relu")
+    acc = torch.zeros_like(plain)
+    n = 4000
+    for _ in range(n):
+        acc += off.feed_forward(x, w_in, b_in, w_out, b_out, "relu", False, p, (torch.rand(1, b, di, generator=g) < 0.75).to(D))
+    assert float((acc / n - plain).abs().max()) < 0.25

@@ -201,5 +201,8 @@ def test_layers_with_dropout_and_unsupported_options(dev):
             EncoderLayer(options(**{field: False}))
     with pytest.raises(NotImplementedError):
         DecoderLayer(options(fast_xattention=False))
-    with pytest.raises(NotImplementedError):
-        EncoderLayer(options(ffn_glu=True))
+    gated = EncoderLayer(options(ffn_glu=True)).to(dev).bfloat16().train()          # the gated feed-forward block is built and runs
+    assert gated.feedforward.in_proj_weight.shape[0] == 2 * gated.feedforward.inner_size
+    xg = x.detach().clone().requires_grad_()
+    gated(xg, pad).float().sum().backward()
+    assert torch.isfinite(xg.grad.float()).all()
