@@ -467,6 +467,75 @@ class EncdecAttnWL(Workload):
 
 
 
+class DecodeStepWL(Workload):
+    name = "decode_step"
+    bound = "hbm"
+    dtype = "bf16"
+    description = ("one incremental decoding step of the decoder's attention, bf16: cross-attention of 1 new position over "
+                   "1500 cached encoder keys / values (B=32 hypotheses, E=1024, 16 heads, key-padding lengths U[750,1500]) + "
+                   "self-attention of the new position over 127 cached positions (cache grown by concatenation, as the reference does)")
+    TK, TPREV, B, E, H = 1500, 127, 32, 1024, 16
+
+    def setup(self, dev):
+        from oracle import inputs
+        from nmtgminor_amd.modules import incremental as inc
+        self.inc = inc
+        d = inputs.encdec_attn_inputs(1, self.TK, self.B, self.E, self.H, seed=1010)
+        s = inputs.self_attn_inputs(self.TPREV + 1, self.B, self.E, self.H, p=0.0, seed=1011)
+        self.cpu, self.cpu_self = d, s
+        self.a = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in d.items()}
+        self.s = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in s.items()}
+        self.cross_cache, self_cache = {}, {}
+        a, sa = self.a, self.s
+        inc.encdec_attn_step(self.H, a["x_q"], a["x_kv"], a["w_q"], a["w_kv"], a["w_out"], a["b_q"], a["b_kv"], a["b_out"],
+                             a["pad_mask"], self.cross_cache)                       # fills c_k / c_v: not part of a step
+        inc.self_attn_step(self.H, sa["x"][:self.TPREV], sa["w_in"], sa["w_out"], sa["b_in"], sa["b_out"], None, self_cache, False)
+        self.prev_k, self.prev_v = self_cache["k"], self_cache["v"]
+
+    def step(self):
+        a, sa = self.a, self.s
+        cache = {"k": self.prev_k, "v": self.prev_v}                                  # every step appends to the same 127 positions
+        r1 = self.inc.self_attn_step(self.H, sa["x"][self.TPREV:], sa["w_in"], sa["w_out"], sa["b_in"], sa["b_out"], None, cache,
+                                     False)
+        r2 = self.inc.encdec_attn_step(self.H, a["x_q"], None, a["w_q"], None, a["w_out"], a["b_q"], None, a["b_out"],
+                                       a["pad_mask"], self.cross_cache)
+        return r1[0], r2[0]
+
+    def _bytes(self):
+        tk, tp, b, e, h = self.TK, self.TPREV, self.B, self.E, self.H
+        cross = 2 * tk * b * e * 2 + 2 * e * e * 2 + b * h * tk * 2 + 4 * b * e * 2         # K, V cache; W_q, W_out; probabilities; rows
+        self_ = 2 * (tp + tp + 1) * b * e * 2 + 4 * e * e * 2 + b * h * (tp + 1) * 2 + 5 * b * e * 2   # cache read + rewritten
+        return cross + self_
+
+    def work_per_step(self):
+        return self._bytes()
+
+    def kernel_work(self):
+        tk, tp, b, e, h = self.TK, self.TPREV, self.B, self.E, self.H
+        # the two launches of the cache-streaming kernel: keys and values read once, probabilities written, a row in and out
+        return {"attn_decode": 2 * (tk + tp + 1) * b * e * 2 + b * h * (tk + tp + 1) * 2 + 4 * b * e * 2}
+
+    def cpu_baseline(self):
+        from oracle import attention as o
+        d, s = self.cpu, self.cpu_self
+        f = lambda z: z.float() if z is not None and z.is_floating_point() else z
+        kv = (f(d["x_kv"]).view(-1, self.E) @ f(d["w_kv"]).t()).view(self.TK, self.B, 2 * self.E)   # the cached projection
+
+        def run():
+            # the step's arithmetic: the new position's row of both attentions, keys / values already projected
+            o.self_attn_fwd(f(s["x"]), f(s["w_in"]), f(s["w_out"]), f(s["b_in"]), f(s["b_out"]), self.H, None, None)
+            q = f(d["x_q"]).view(-1, self.E) @ f(d["w_q"]).t()
+            dd = self.E // self.H
+            k4 = kv.view(self.TK, self.B * self.H, 2, dd)
+            sc = torch.einsum("bd,tbd->bt", q.view(self.B * self.H, dd), k4[:, :, 0]) * dd ** -0.5
+            pr = torch.softmax(sc.masked_fill(d["pad_mask"].repeat_interleave(self.H, 0), float("-inf")), -1)
+            ctx = torch.einsum("bt,tbd->bd", pr, k4[:, :, 1]).reshape(self.B, self.E)
+            return ctx @ f(d["w_out"]).t()
+        t = _time_cpu(run, 3)
+        return dict(value=self._bytes() / t / 1e9, unit="GB/s", cores=torch.get_num_threads(), kind="port",
+                    sample="full step in fp32 on the bf16-rounded values (self-attention recomputed over its 128 positions), median of 3")
+
+
 class SoftmaxDropoutWL(Workload):
     name = "softmax_dropout"
     bound = "hbm"
@@ -698,7 +767,7 @@ class CopyWL(Workload):
 
 # the five benchmark configurations first, then the workloads added beside them
 WORKLOADS = {w.name: w for w in (LayerNormWL, MlpWL, SelfAttnWL, EncdecAttnWL, XentropyWL, SoftmaxDropoutWL, DropoutAddWL,
-                                    GeneratorLossWL, RelSelfAttnWL, FusedAdamWL, LayerNormLargeWL, FlashAttnWL)}
+                                    GeneratorLossWL, RelSelfAttnWL, FusedAdamWL, LayerNormLargeWL, FlashAttnWL, DecodeStepWL)}
 EXTRA_WORKLOADS = {CopyWL.name: CopyWL}
 PRIMARY = "mlp"
 

@@ -381,6 +381,25 @@ int nmtg_flash_attn_bwd(const void* dout, const void* q, const void* k, const vo
                         int dtype, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Attention of ONE new query position over cached keys / values (incremental decoding).
+ * Reference: the incremental branches of SelfAttnFunc (onmt/modules/optimized/
+ *   self_attention_func.py:162-174, one query row against the concatenated cache) and of
+ *   EncdecAttnBiasFunc (encdec_attention_func_bias.py:181-213, cached encoder keys / values),
+ *   run there as one-row batched GEMMs and a softmax.
+ * q [batch, heads * head_dim] (row stride q_stride_b); keys, values: element (t, b, h, d) at
+ * t * stride_t + b * stride_b + h * head_dim + d (the reference's time-first cache [Tk, B, E] has
+ * stride_t = B * E, stride_b = E); key_mask [batch, tk] (1 = masked key) or NULL.
+ * probs [batch * heads, tk] = softmax(round(scale * q . k)) in the tensors' 16-bit type (rows without
+ * a live key: zeros), context [batch, heads * head_dim] (row stride ctx_stride_b) = probs x values.
+ * head_dim 32, 64 or 128; tk <= 16384; fp16 / bf16; strides multiples of 8 elements.
+ * ------------------------------------------------------------------------------------------ */
+int nmtg_attn_decode(const void* q, int64_t q_stride_b, const void* keys, int64_t k_stride_t,
+                     int64_t k_stride_b, const void* values, int64_t v_stride_t, int64_t v_stride_b,
+                     const uint8_t* key_mask, void* probs, void* context, int64_t ctx_stride_b,
+                     int64_t batch, int64_t heads, int64_t head_dim, int64_t tk, float scale,
+                     int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Gated feed-forward activation with dropout.
  * Reference: the gated branch of PositionWiseFeedForward.forward, PyTorch ops there
  *   (onmt/modules/optimized/feed_forward.py:188-200), and variational_dropout

@@ -209,6 +209,19 @@ __device__ __forceinline__ void wave_sum2(float& a, float& b) {
 }
 
 
+// acc + a.lo * b.lo + a.hi * b.hi on one register of two 16-bit elements each (v_dot2c_f32_f16 / v_dot2c_f32_bf16): the
+// inner step of the bandwidth-bound products (few-row projections, one-row attention), where converting every element
+// to fp32 first would cost more instructions than the multiplications.
+template <typename T> __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc);
+template <> __device__ __forceinline__ float dot2<f16_t>(uint32_t a, uint32_t b, float acc) {
+  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, a), __builtin_bit_cast(h2, b), acc, false);
+}
+template <> __device__ __forceinline__ float dot2<bf16_t>(uint32_t a, uint32_t b, float acc) {
+  typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(b2, a), __builtin_bit_cast(b2, b), acc, false);
+}
+
 // ---------------------------------------------------------------------------------------------
 // Philox4x32-10 counter-based generator (Salmon et al., SC'11). One call turns a 128-bit
 // counter and a 64-bit key into four 32-bit words. Dropout draws u = (word >> 8) * 2^-24 in

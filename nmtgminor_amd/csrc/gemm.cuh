@@ -1006,6 +1006,10 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
 // set and planned_out->splits > 1 the caller owes the reduction of the partials (tail_add_splitk).
 // dtype NMTG_F32 goes to the fp32 matrix-core kernel (gemm_f32.hip): plain and the two activation epilogues, no split-K.
 int gemm_f32_run(int layout, int epi, GemmArgs a, hipStream_t st, int* m_tiles_out, GemmArgs* planned_out);
+// Products with at most 32 rows against a row-major weight (the projections of a decoding step): one output column per
+// wavefront (gemm_skinny.hip).
+bool gemm_skinny_ok(int dtype, int layout, int epi, const GemmArgs& a);
+int gemm_skinny_run(int dtype, const GemmArgs& a, hipStream_t st);
 
 // Fused Q K^T -> mask -> softmax -> dropout (EPI_SCORES_SOFTMAX) for rows of at most 512 keys. `a` is filled as
 // for EPI_SCORES plus out2 (dropped probabilities), aux_out (softmax, optional), dmask / rng / keep_p / dscale /

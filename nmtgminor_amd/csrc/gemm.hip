@@ -79,6 +79,13 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
   if (a.K < 0) return fail(NMTG_ERR_INVALID, "gemm: negative K");
   if (!a.A || !a.B || !a.C) return fail(NMTG_ERR_INVALID, "gemm: null operand pointer");
   if (dtype == NMTG_F32) return gemm_f32_run(layout, epi, a, st, m_tiles_out, planned_out);
+  if (gemm_skinny_ok(dtype, layout, epi, a)) {
+    a.splits = 1;
+    a.defer_reduce = 0;
+    a.tile_used = -1;
+    if (planned_out) *planned_out = a;
+    return gemm_skinny_run(dtype, a, st);
+  }
   const bool a_kc = layout != LAYOUT_TN;
   const bool b_kc = layout == LAYOUT_NT;
   // Widest access (8, 4 or 1 elements) that every pointer, pitch and batch stride of this call allows. Extents do not

@@ -13,8 +13,11 @@ handed over in that form. The cache bookkeeping (slices, concatenation, the inte
 movement on the device, exactly the reference's. A later step may carry one new position only: with more than one,
 the new positions would need a causal mask among themselves, which the cross-attention core does not take.
 """
+import os
+
 import torch
 
+from .. import _lib as L
 from ..native import encdec_multihead_attn_bias_blaslt as ed_native
 from ..native.linear_gemm import gemm
 
@@ -24,8 +27,37 @@ def _project(x, weight, bias):
     return gemm(x.reshape(t * b, e), weight, False, True, bias=bias).view(t, b, weight.shape[0])
 
 
+def _decode_core(heads, q_lin, keys, values, pad_mask):
+    """One query position: the cache-streaming kernel (nmtg_attn_decode) reads keys and values where they lie."""
+    tk, b, e = keys.shape
+    d = e // heads
+    q_lin = q_lin.contiguous()
+    km = None
+    if pad_mask is not None:
+        km = pad_mask.to(torch.uint8).contiguous()
+        if km.shape != (b, tk):
+            raise RuntimeError(f"incremental attention: key mask of shape {tuple(km.shape)}, expected {(b, tk)}")
+    probs = torch.empty(b * heads, 1, tk, dtype=q_lin.dtype, device=q_lin.device)
+    context = torch.empty(1, b, e, dtype=q_lin.dtype, device=q_lin.device)
+    L.call("nmtg_attn_decode", L.ptr(q_lin), L.i64(e), L.ptr(keys), L.i64(keys.stride(0)), L.i64(keys.stride(1)), L.ptr(values),
+           L.i64(values.stride(0)), L.i64(values.stride(1)), L.ptr(km), L.ptr(probs), L.ptr(context), L.i64(e), L.i64(b),
+           L.i64(heads), L.i64(d), L.i64(tk), L.f32(d ** -0.5), L.i32(L.dtype_code(q_lin)), L.stream_of(q_lin))
+    return context, probs
+
+
+def _decode_ok(q_lin, keys, values, heads):
+    """NMTG_ATTN_DECODE=0 keeps one-position steps on the GEMM path (the plainer of the two validated paths)."""
+    e = keys.shape[2]
+    return (q_lin.shape[0] == 1 and os.environ.get("NMTG_ATTN_DECODE", "1") != "0" and e // heads in (32, 64, 128)
+            and 0 < keys.shape[0] <= 16384 and q_lin.dtype in (torch.float16, torch.bfloat16)
+            and keys.stride(2) == 1 and values.stride(2) == 1 and all(s % 8 == 0 for s in keys.stride()[:2] + values.stride()[:2])
+            and keys.data_ptr() % 16 == 0 and values.data_ptr() % 16 == 0)
+
+
 def _core(heads, q_lin, keys, values, pad_mask):
     """q_lin [Tq, B, E]; keys, values [Tk, B, E] -> (context [Tq, B, E], probabilities [B*H, Tq, Tk])."""
+    if _decode_ok(q_lin, keys, values, heads):
+        return _decode_core(heads, q_lin, keys, values, pad_mask)
     tk, b, e = keys.shape
     d = e // heads
     kv = torch.stack([keys.view(tk, b * heads, d), values.view(tk, b * heads, d)], dim=-2).view(tk, b, 2 * e)

@@ -11,10 +11,10 @@ query-gradient terms are joined by the row-add kernel. What is left to PyTorch: 
 
 Covered: sinusoidal positions projected by pos_weights (learnable_pos=False) and learnable position embeddings
 (learnable_pos=True: pos [len_q, len_k, head_dim], shared by heads and batch, no shift, no r_w_bias / r_r_bias, a gradient
-for pos), key-padding or time mask, training and inference, fp16 / bf16, and incremental decoding with projected positions
-(`incremental=True` with the reference's cache entries `k`, `v`, time-first [T, B, E]: the new keys and values are appended,
-the queries attend to everything cached; inference only). Not covered, and raising instead of falling back: incremental
-decoding with learnable positions. `recompute` is accepted and gives the same numbers; the intermediate tensors are kept either way. A 22nd
+for pos), key-padding or time mask, training and inference, fp16 / bf16, and incremental decoding with either kind of
+positions (`incremental=True` with the reference's cache entries `k`, `v`, time-first [T, B, E]: the new keys and values
+are appended, the queries attend to everything cached; learnable positions then come as [new queries, cached + new keys,
+head_dim]; inference only). `recompute` is accepted and gives the same numbers; the intermediate tensors are kept either way. A 22nd
 optional argument replays an explicit dropout keep-mask."""
 import torch
 
@@ -49,8 +49,6 @@ class RelativeSelfAttnFunc(torch.autograd.Function):
     def forward(ctx, inputs, pos, use_time_mask, is_training, heads, input_weights, output_weights, pos_weights,
                 input_biases, output_biases, pos_biases, r_w_bias, r_r_bias, mask, dropout_prob, incremental,
                 incremental_cache, low_precision, learnable_pos, return_coverage, recompute, dropout_mask=None):
-        if incremental and learnable_pos:
-            raise NotImplementedError("relative_self_attn_func: incremental decoding with learnable positions has no HIP path")
         if incremental and (is_training or torch.is_grad_enabled() and inputs.requires_grad):
             raise RuntimeError("relative_self_attn_func: incremental decoding is an inference path (no backward)")
         inputs = inputs.contiguous()
@@ -98,15 +96,19 @@ class RelativeSelfAttnFunc(torch.autograd.Function):
             incremental_cache['k'], incremental_cache['v'] = keys, values
             len_k = keys.size(0)
             keys, values = keys.view(len_k, bsz * heads, head_dim), values.view(len_k, bsz * heads, head_dim)
+        else:
+            len_k = len_q
+        if not learnable_pos:
             pos_lin = linear_blaslt.forward(pos, pos_weights, pos_biases)                 # [R, B, E]
             scores = native.relative_scores(queries, keys, pos_lin.view(pos.size(0), bsz * heads, head_dim), r_w_bias,
                                             r_r_bias, heads, scale)
         else:
             # learnable positions, pos [len_q, len_k, head_dim]: scores[bh][i][j] = scale (q[i][bh] k[j][bh] + q[i][bh]
             # pos[i][j]); the second product is batched over the query positions and written through the strides of the
-            # [B*H, T, T] layout
+            # [B*H, T, T] layout. Incremental decoding: len_k counts the cached keys too, pos has a row per new query
+            # (relative_self_attention_func.py:187-204, :254-263).
             pos = pos.contiguous()
-            if pos.dim() != 3 or pos.shape != (len_q, len_q, head_dim):
+            if pos.dim() != 3 or pos.shape != (len_q, len_k, head_dim):
                 raise RuntimeError("relative_self_attn_func: learnable positions must be [len_q, len_k, head_dim]")
             scores = linear_gemm.gemm(queries.transpose(0, 1), keys.transpose(0, 1), trans_b=True, alpha=scale)
             matmul_bd = torch.empty_like(scores)

@@ -110,6 +110,16 @@ static inline hostsim_u32x2 __builtin_amdgcn_permlane32_swap(unsigned int vdst, 
   return lane < 32 ? hostsim_u32x2{vdst, other_dst} : hostsim_u32x2{other_src, vsrc};
 }
 
+// v_dot2c_f32_f16 / v_dot2c_f32_bf16: acc + a[0] b[0] + a[1] b[1] in fp32
+typedef _Float16 hostsim_half2 __attribute__((ext_vector_type(2)));
+typedef __bf16 hostsim_bf16x2 __attribute__((ext_vector_type(2)));
+static inline float __builtin_amdgcn_fdot2(hostsim_half2 a, hostsim_half2 b, float acc, bool) {
+  return acc + static_cast<float>(a[0]) * static_cast<float>(b[0]) + static_cast<float>(a[1]) * static_cast<float>(b[1]);
+}
+static inline float __builtin_amdgcn_fdot2_f32_bf16(hostsim_bf16x2 a, hostsim_bf16x2 b, float acc, bool) {
+  return acc + static_cast<float>(a[0]) * static_cast<float>(b[0]) + static_cast<float>(a[1]) * static_cast<float>(b[1]);
+}
+
 // v_cmp into a wavefront-wide mask: bit l is lane l's predicate
 static inline uint64_t __builtin_amdgcn_ballot_w64(bool pred) {
   uint64_t mask = 0;

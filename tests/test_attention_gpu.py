@@ -297,4 +297,4 @@ def test_feed_forward_module(dev):
     yo, _, _ = omlp.mlp_fwd(x.cpu().view(80, 128), w, bb, "relu", 0.0, None, D, round_to=torch.float16)
     assert_close(yr.view(80, 128), yo.to(torch.float16).to(D) + x.cpu().view(80, 128).to(D), torch.float16, "residual")
     with pytest.raises(NotImplementedError):
-        PositionWiseFeedForward(128, 512, glu=True)
+        PositionWiseFeedForward(128, 512, activation="tanh")

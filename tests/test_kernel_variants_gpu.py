@@ -9,6 +9,10 @@
   NMTG_MLP_TAIL=0      the MLP backward's split-K reductions and bias-gradient sums as launches of their own instead of
                        one launch at its end
   NMTG_GELU_LUT=0      gelu and its derivative in the MLP epilogues from the formula instead of the 2049-entry LDS table
+  NMTG_GEMM_SKINNY=0   a product with at most 32 rows against a row-major weight on the tiled kernels instead of the
+                       kernel that gives every wavefront one output column
+  NMTG_ATTN_DECODE=0   a one-position decoding step as one-row batched GEMMs and a softmax instead of the kernel that
+                       streams the cached keys and values once
 
 Each test runs both paths in one process and compares them with each other and the default one with the CPU oracle.
 """
@@ -237,3 +241,55 @@ def test_three_layer_mlp_backward_with_one_reduction_launch(dev):
     assert len(got) == 7
     for a_, r_ in zip(got, want):
         assert torch.equal(a_, r_)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("tk,b,e,h,masked", [(1500, 3, 256, 4, True), (127, 2, 128, 4, False), (70, 2, 256, 2, True),
+                                             (300, 2, 256, 8, True), (1, 1, 128, 2, False)])
+def test_decode_step_kernel_matches_the_gemm_path_and_the_oracle(dev, dtype, tk, b, e, h, masked):
+    from nmtgminor_amd.modules import incremental as inc
+    g = torch.Generator().manual_seed(tk + e)
+    q = torch.randn(1, b, e, generator=g).to(dtype)
+    keys = torch.randn(tk, b, e, generator=g).to(dtype)
+    values = torch.randn(tk, b, e, generator=g).to(dtype)
+    pad = None
+    if masked:
+        lengths = torch.randint(max(1, tk // 2), tk + 1, (b,), generator=g)
+        lengths[0] = 0 if tk > 1 else 1                                   # a sentence without any live key: zeros
+        pad = torch.arange(tk).view(1, tk) >= lengths.view(b, 1)
+    args = (h, q.to(dev), keys.to(dev), values.to(dev), None if pad is None else pad.to(dev))
+    ctx, probs = inc._core(*args)
+    with off("NMTG_ATTN_DECODE"):
+        ctx_g, probs_g = inc._core(*args)
+    d = e // h
+    qh, kh, vh = (t.to(D).view(-1, b * h, d).transpose(0, 1) for t in (q, keys, values))          # [B*H, T, D]
+    sc = (qh @ kh.transpose(1, 2) * d ** -0.5).to(dtype).to(D)                                    # stored in 16 bits
+    if pad is not None:
+        sc = sc.masked_fill(pad.repeat_interleave(h, 0).view(b * h, 1, tk), float("-inf"))
+    want_p = torch.nan_to_num(torch.softmax(sc, -1), nan=0.0).to(dtype).to(D)
+    want_c = (want_p @ vh).transpose(0, 1).reshape(1, b, e)
+    assert probs.shape == (b * h, 1, tk) and ctx.shape == (1, b, e)
+    assert_close(probs, want_p, dtype, "probabilities")
+    assert_close(ctx, want_c, dtype, "context", atol=2e-3)
+    assert_close(probs, probs_g.cpu(), dtype, "probabilities, both paths")
+    assert_close(ctx, ctx_g.cpu(), dtype, "context, both paths", atol=2e-3)
+    if masked and tk > 1:
+        assert float(probs[:h].abs().max()) == 0.0 and float(ctx[:, 0].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m,n,k", [(32, 1024, 1024), (1, 256, 64), (7, 100, 2056), (32, 64, 8), (20, 1000, 3000), (32, 4096, 1024)])
+def test_few_row_products_match_the_tiled_kernels(dev, dtype, m, n, k):
+    g = torch.Generator().manual_seed(m + n + k)
+    x = torch.randn(m, k, generator=g).to(dtype).to(dev)
+    w = (torch.randn(n, k, generator=g) * k ** -0.5).to(dtype).to(dev)
+    bias = torch.randn(n, generator=g).to(dtype).to(dev)
+    got = gemm(x, w, False, True, alpha=0.5, bias=bias)
+    with off("NMTG_GEMM_SKINNY"):
+        tiled = gemm(x, w, False, True, alpha=0.5, bias=bias)
+    want = 0.5 * (x.double() @ w.double().t()).cpu() + bias.double().cpu()
+    assert_close(got, want, dtype, "one column per wavefront")
+    assert_close(tiled, want, dtype, "tiled")
+    pitched = torch.full((m, k + 24), float("nan"), dtype=dtype, device=dev)      # rows with a pitch, NaN in the padding
+    pitched[:, :k] = x
+    assert torch.equal(gemm(pitched[:, :k], w, False, True, alpha=0.5, bias=bias), got)

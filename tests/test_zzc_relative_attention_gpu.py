@@ -324,6 +324,38 @@ def test_module_with_learnable_positions(dev):
     assert m.pos_emb.weight.grad is not None and m.in_proj_weight.grad is not None
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("prefix", [1, 5])
+def test_learnable_positions_step_by_step(dev, dtype, prefix):
+    """Incremental decoding with learnable positions (relative_self_attention_func.py:187-204, :254-263): a prefix in one
+    call, then one position per call onto the cache, each with the [new queries, all keys] rows of the distance table.
+    Every decoded row is the row of the oracle's causal full-sequence result."""
+    torch.manual_seed(8)
+    t, b, e, h, max_pos = 11, 3, 128, 4, 16
+    m = RelativeSelfMultiheadAttn(e, h, dropout=0.0, learnable_pos=True, max_pos=max_pos).to(dev).to(dtype).eval()
+    x = torch.randn(t, b, e, generator=torch.Generator().manual_seed(9)).to(dtype)
+    dist = (torch.arange(t).view(t, 1) - torch.arange(t).view(1, t)).clamp(-max_pos, max_pos) + max_pos
+    causal = torch.ones(t, t, dtype=torch.bool).triu(1)
+    P = {k: v.detach().cpu() for k, v in m.named_parameters()}
+    want = orel.rel_learnable_attn_fwd(x, P["pos_emb.weight"][dist], P["in_proj_weight"], P["out_proj_weight"], P["in_proj_bias"],
+                                       P["out_proj_bias"], h, None, causal, 0.0, None, D, round_to=dtype, round_bd=True)
+    cache, rows, covs = {}, [], []
+    with torch.no_grad():
+        lo = 0
+        for hi in [prefix] + list(range(prefix + 1, t + 1)):
+            out, cov = m(x[lo:hi].to(dev), dist[lo:hi, :hi].to(dev), None, causal[lo:hi, :hi].to(dev), incremental=True,
+                         incremental_cache=cache)
+            assert out.shape == (hi - lo, b, e) and cov.shape == (b * h, hi - lo, hi) and cache["k"].shape == (hi, b, e)
+            rows.append(out)
+            covs.append(cov)
+            lo = hi
+    assert_close(torch.cat(rows, 0), want["outputs"], dtype, "decoded rows", atol=2e-3)
+    for i, cov in enumerate(covs[1:], start=prefix):
+        assert_close(cov[:, 0, :], want["dropout_results"][:, i, :i + 1], dtype, f"coverage of step {i}")
+    with pytest.raises(RuntimeError):
+        m(x[:1].to(dev), dist[:1, :3].to(dev), None, None, incremental=True, incremental_cache={})     # table wider than the keys
+
+
 def test_relative_attention_golden_fixture(dev):
     # tests/golden/relative_attention.npz: the shift as an explicit gather, fp64 autograd with the bf16 rounding points
     BF = torch.bfloat16
