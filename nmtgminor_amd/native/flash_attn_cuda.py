@@ -14,6 +14,7 @@ Differences from the CUDA module, all on the dropout side:
    (or `generator`) and remembers it in `last_rng`, bwd takes it from the keyword `rng` (the autograd functions of
    nmtgminor_amd/modules/flash_mha.py carry it from forward to backward) or, without it, replays `last_rng`; restoring
    the generator state before bwd, as the reference does, is harmless and not needed;
+ * keyword `rng=(seed, offset)` on fwd fixes the Philox state instead of drawing one from the generator;
  * return_softmax hands back the keep-mask (uint8 [B, H, max_seqlen_q, max_seqlen_k]) instead of the sign-encoded
    probability matrix, which exists nowhere in this kernel; keyword `dropout_mask` replays such a mask (tests);
  * num_splits is accepted and ignored: the kernels never accumulate across blocks, so results do not depend on it."""
@@ -60,7 +61,7 @@ def _draw(device, count, generator):
 
 
 def fwd(q, k, v, out, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale, zero_tensors,
-        causal, return_softmax, num_splits=0, generator=None, *, dropout_mask=None):
+        causal, return_softmax, num_splits=0, generator=None, *, dropout_mask=None, rng=None):
     global last_rng
     batch, heads, d = _common(q, k, v, cu_seqlens_q, cu_seqlens_k)
     if out is None:
@@ -79,7 +80,9 @@ def fwd(q, k, v, out, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dr
         else:
             mode = 2
             blocks = batch * heads * ((max_seqlen_q + 3) // 4) * ((max_seqlen_k + 3) // 4)
-            seed, offset = _draw(q.device, 4 * blocks, generator)
+            # rng=(seed, offset): a Philox state fixed by the caller (a step that is captured into a graph cannot ask
+            # the generator for one)
+            seed, offset = rng if rng is not None else _draw(q.device, 4 * blocks, generator)
             if return_softmax:
                 mask_out = torch.zeros(batch, heads, max_seqlen_q, max_seqlen_k, dtype=torch.uint8, device=q.device)
     last_rng = (mode, seed, offset, dropout_mask)

@@ -106,6 +106,9 @@ def on_the_cpu(hostsim_lib, monkeypatch):
     # elementwise kernels: few compute units, so that grid-stride loops make several trips and last groups are partial
     monkeypatch.setenv("HOSTSIM_CUS", "2")
     monkeypatch.delenv("HOSTSIM_DMA", raising=False)
+    # products with few rows stay on the tiled kernels here: the one-column-per-wavefront kernel costs the simulator a
+    # block of 256 fibers per four output columns; it has its own test below
+    monkeypatch.setenv("NMTG_GEMM_SKINNY", "0")
 
 
 @pytest.fixture
@@ -620,6 +623,23 @@ def test_packed_attention_dropout_philox_and_autograd_functions():
     tfl.test_dropout_drawn_on_the_device_is_the_documented_philox_stream_in_both_passes(CPU, F16, 64)
     tfl.test_packed_qkv_function_takes_strided_slots_and_fills_one_gradient_tensor(CPU, BF16)
     tfl.test_packed_kv_function_with_dropout_repeats_its_mask_in_the_backward(CPU)
+
+
+# ----------------------------------------------------------------------------- decoding step
+@pytest.mark.parametrize("m,n,k", [(32, 64, 8), (7, 100, 2056), (1, 256, 64)])
+def test_few_row_products(monkeypatch, mi355x, m, n, k):
+    monkeypatch.delenv("NMTG_GEMM_SKINNY")
+    tst.test_few_row_products_match_the_tiled_kernels(CPU, BF16, m, n, k)
+
+
+@pytest.mark.parametrize("dtype", HALVES)
+@pytest.mark.parametrize("tk,b,e,h,masked", [(70, 2, 256, 2, True), (300, 2, 256, 8, True), (127, 2, 128, 4, False)])
+def test_decode_step_kernel(mi355x, dtype, tk, b, e, h, masked):
+    tst.test_decode_step_kernel_matches_the_gemm_path_and_the_oracle(CPU, dtype, tk, b, e, h, masked)
+
+
+def test_incremental_decoding_with_learnable_positions(mi355x):
+    trel.test_learnable_positions_step_by_step(CPU, BF16, 5)
 
 
 # ----------------------------------------------------------------------------- gated / variational feed-forward, fp32 products
