@@ -2,6 +2,7 @@
 // by name and reports zero time), and C hooks for the reduction kernels, which the real library only reaches from
 // inside its GEMM-based operators.
 #include "reduce.cuh"
+#include "gemm.cuh"
 #include <algorithm>
 #include <cstring>
 #include <map>
@@ -66,4 +67,15 @@ extern "C" int hostsim_splitk_reduce(int dtype, int tile, const float* ws, void*
   }
   NMTG_DISPATCH_DTYPE(dtype, T, return (splitk<T, 256, 256, 2, 4>(ws, C, ldc, M, N, m_tiles, n_tiles, batch, sC, splits, alpha, c_vec)));
   return -1;
+}
+
+// gemm_run asked for the split-K epilogue directly (only internal callers can) without the fp32 workspace its partial
+// tiles go to: the call must be refused before any launch. -> gemm_run's status
+extern "C" int hostsim_gemm_splitk_without_workspace(int dtype, const void* a, const void* b, void* c, int m, int n, int k) {
+  GemmArgs g{};
+  g.A = a; g.B = b; g.C = c;
+  g.lda = m; g.ldb = n; g.ldc = n;
+  g.M = m; g.N = n; g.K = k;
+  g.batch = 1; g.alpha = 1.f;
+  return gemm_run(dtype, LAYOUT_TN, EPI_SPLITK, g, nullptr, 0, nullptr);
 }

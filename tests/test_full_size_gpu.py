@@ -53,6 +53,29 @@ def test_self_attention_workload(dev):
     assert_close(grads[3], dlin.view(-1, 3 * E).float().sum(0).cpu(), BF, "db_in", scale_atol=True)
 
 
+def test_self_attention_workload_weight_gradients_against_the_oracle(dev):
+    """Weight and bias gradients sum over every token, so no single batch column pins them. A fixed sub-batch of four
+    columns of the workload (full length, width and head count; its own HIP call) is small enough for the fp64 oracle:
+    every gradient of that call is compared with it."""
+    T, B, E, H = 512, 32, 1024, 16
+    d = inputs.self_attn_inputs(T, B, E, H)
+    cols = torch.tensor([0, 1, B - 2, B - 1])
+    x, dout, pad = d["x"][:, cols].contiguous(), d["dout"][:, cols].contiguous(), d["pad_mask"][cols].contiguous()
+    dm = d["dropout_mask"].view(B, H, T, T)[cols].reshape(len(cols) * H, T, T).contiguous()
+    g = lambda t: t.to(dev)
+    lin, scores, dropped, dmask, ctx, out = sa.forward(False, True, H, g(x), g(d["w_in"]), g(d["w_out"]), g(d["b_in"]),
+                                                        g(d["b_out"]), g(pad), 0.1, dropout_mask=g(dm))
+    grads = sa.backward(False, H, g(dout), ctx, dropped, scores, lin, g(x), g(d["w_in"]), g(d["w_out"]), dmask, 0.1)
+    f = oat.self_attn_fwd(x, d["w_in"], d["w_out"], d["b_in"], d["b_out"], H, pad, None, 0.1, dm, D, round_to=BF)
+    bw = oat.self_attn_bwd(dout, x, d["w_in"], d["w_out"], H, f, 0.1, dm, D, round_to=BF)
+    assert_close(out, f["outputs"], BF, "outputs")
+    assert_close(grads[0], bw["dx"], BF, "dx", scale_atol=True)
+    assert_close(grads[1], bw["dw_in"], BF, "dW_in", scale_atol=True)
+    assert_close(grads[2], bw["dw_out"], BF, "dW_out", scale_atol=True)
+    assert_close(grads[3], bw["db_in"], BF, "db_in", scale_atol=True)
+    assert_close(grads[4], bw["db_out"], BF, "db_out", scale_atol=True)
+
+
 def test_decoder_attention_workload(dev):
     TQ, TK, B, E, H = 128, 1500, 16, 1024, 16
     d = inputs.encdec_attn_inputs(TQ, TK, B, E, H)               # seed 1004, bf16, eval

@@ -625,6 +625,20 @@ def test_packed_attention_dropout_philox_and_autograd_functions():
     tfl.test_packed_kv_function_with_dropout_repeats_its_mask_in_the_backward(CPU)
 
 
+def test_split_k_epilogue_without_a_workspace_is_refused_before_any_launch(hostsim_lib):
+    a = torch.randn(512, 128).to(BF16)
+    b = torch.randn(512, 128).to(BF16)
+    c = torch.zeros(128, 128, dtype=BF16)
+    harness_lib = hostsim_lib
+    harness_lib.nmtg_trace_begin()
+    rc = harness_lib.hostsim_gemm_splitk_without_workspace(2, ctypes.c_void_p(a.data_ptr()), ctypes.c_void_p(b.data_ptr()),
+                                                           ctypes.c_void_p(c.data_ptr()), 128, 128, 512)
+    buf = ctypes.create_string_buffer(4096)
+    harness_lib.nmtg_trace_end(buf, 4096)
+    assert rc == -1 and b"workspace" in harness_lib.nmtg_last_error()          # NMTG_ERR_INVALID
+    assert buf.value == b"" and float(c.abs().max()) == 0.0                    # nothing was launched, nothing written
+
+
 # ----------------------------------------------------------------------------- decoding step
 @pytest.mark.parametrize("m,n,k", [(32, 64, 8), (7, 100, 2056), (1, 256, 64)])
 def test_few_row_products(monkeypatch, mi355x, m, n, k):
