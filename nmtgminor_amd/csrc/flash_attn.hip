@@ -269,7 +269,7 @@ __device__ __forceinline__ void store_rows_out(const acc16_t (&acc)[D / 32], flo
 // forward
 // -------------------------------------------------------------------------------------------------------------------
 template <typename T, int D, int DROP>
-__global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_fwd_kernel(FaArgs a) {
+__global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(FaArgs a) {
   extern __shared__ __align__(16) uint8_t lds_raw[];
   constexpr int IMG = FA_TILE * D * 2;
   const int b = blockIdx.z, h = blockIdx.y, q0 = static_cast<int>(blockIdx.x) * FA_ROWS;

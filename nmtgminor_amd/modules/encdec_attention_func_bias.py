@@ -19,10 +19,8 @@ class EncdecAttnBiasFunc(torch.autograd.Function):
                 output_weights, input_bias_q, input_bias_kv, output_bias, mask, dropout_prob, incremental,
                 incremental_cache, rotary_pos_enc, pos_emb_q, pos_emb_k, low_precision, return_coverage,
                 dropout_mask=None):
-        if rotary_pos_enc:
-            raise NotImplementedError("encdec_attn_bias_func: rotary position encoding has no HIP kernel")
-        if incremental:
-            raise NotImplementedError("encdec_attn_bias_func: incremental decoding has no HIP kernel")
+        if rotary_pos_enc or incremental:           # encdec_attn_bias_func routes both before it gets here
+            raise RuntimeError("EncdecAttnBiasFunc: call encdec_attn_bias_func for rotary encodings / incremental decoding")
         ctx.heads, ctx.p, ctx.recompute, ctx.return_coverage = heads, dropout_prob, recompute, return_coverage
         ctx.has_bias = (input_bias_q is not None, input_bias_kv is not None, output_bias is not None)
         q_lin, kv_lin, scores, dropped, dmask, ctx_t, outputs = native.forward(
