@@ -127,14 +127,21 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
     }
   }
   // NMTG_GEMM_TILE=0|1|2 (256x256 | 128x128 | 256x64) overrides the tile choice: a tuning aid.
-  static const int forced_tile = [] { const char* e = getenv("NMTG_GEMM_TILE"); return e ? atoi(e) : -1; }();
+  const int forced_tile = [] { const char* e = getenv("NMTG_GEMM_TILE"); return e ? atoi(e) : -1; }();
   if (tile < 0 && forced_tile >= 0 && gemm_has(layout, forced_tile, epi) && (forced_tile != TILE_L || vec == 8)) tile = forced_tile;
   if (tile < 0) {
     const int cus = num_cus();
     const int64_t cnt_l = static_cast<int64_t>(ceil_div(a.M, 256)) * ceil_div(a.N, 256) * a.batch;
     const bool l_ok = vec == 8 && gemm_has(layout, TILE_L, epi);
+    // share of a tile grid's area that is output: a 256-row tile on 128 rows (the scores of 128 decoder positions)
+    // multiplies and stages twice what it stores. The 256x256 loop sustains about 1.6 times the MFMA rate of the
+    // 128x128 one, so it keeps the call unless it wastes more than that.
+    auto fill = [&](int bm, int bn) {
+      return static_cast<double>(a.M) * a.N / (static_cast<double>(ceil_div(a.M, bm)) * bm * ceil_div(a.N, bn) * bn);
+    };
+    const bool l_fills = fill(256, 256) * 1.6 >= fill(128, 128) || !gemm_has(layout, TILE_M, epi);
     if (a.N <= 64 && gemm_has(layout, TILE_S, epi)) tile = TILE_S;
-    else if (cnt_l * 4 >= cus * 3 && l_ok) tile = TILE_L;
+    else if (cnt_l * 4 >= cus * 3 && l_ok && l_fills) tile = TILE_L;
     else if (gemm_has(layout, TILE_M, epi)) tile = TILE_M;
     else if (l_ok) tile = TILE_L;
     else tile = TILE_S;
