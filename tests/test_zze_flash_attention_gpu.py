@@ -3,11 +3,12 @@ the autograd functions of nmtgminor_amd/modules/flash_mha.py) against the per-se
 (oracle/flash_attention.py, pinned against torch's scaled_dot_product_attention in tests/test_oracle_pins.py).
 
 What the reference computes here: flash_attn_cuda.fwd / .bwd as called from onmt/modules/optimized/flash_mha.py:43-183.
-Tolerance: 2e-2 relative as in the other attention tests. The absolute part is 4e-3 for bf16 and 1e-3 for fp16 outputs: the
+Tolerance: 2e-2 relative as in the other attention tests. The absolute part is 8e-3 for bf16 and 2e-3 for fp16 outputs: the
 probabilities are rounded to the 16-bit type before they multiply V, relative to the running maximum in the kernel and
-to the final normalisation in the oracle, so an output row carries up to one rounding unit (2^-9 / 2^-12) of max |v| of
-difference between two equally accurate results; for the gradients it is scaled by the largest expected magnitude
-(they sum over up to a few hundred keys or queries). With dropout the kept probabilities grow by 1 / (1 - p) past 1, where
+to the final normalisation in the oracle, so an output row carries up to one rounding unit of a probability near 1
+(2^-8 / 2^-11) times max |v| (about 3 here) of difference between two equally accurate results; for the gradients it is
+scaled by the largest expected magnitude (they sum over up to a few hundred keys or queries) and by 1 / (1 - p): dS = P (dP - D)
+cancels where one key dominates, down to the rounding of the stored output inside D. With dropout the kept probabilities grow by 1 / (1 - p) past 1, where
 the rounding unit doubles: the absolute part is 2 / (1 - p) times larger there. The log-sum-exp, an fp32 result of 16-bit
 inputs, to 2e-3 absolute; rowsum(dO * O) to fp32 accuracy against the same sum over the output the kernel itself stored.
 """
@@ -20,7 +21,7 @@ from nmtgminor_amd.native import flash_attn_cuda
 from oracle import flash_attention as ofa
 from util import assert_close
 
-ATOL = {torch.bfloat16: 4e-3, torch.float16: 1e-3}
+ATOL = {torch.bfloat16: 8e-3, torch.float16: 2e-3}
 
 pytestmark = pytest.mark.gpu
 D = torch.float64
@@ -67,6 +68,7 @@ def _check_fwd_bwd(dev, q, k, v, do, lq, lk, causal, p=0.0, mask=None, scale=Non
     _, _, _, sd = flash_attn_cuda.bwd(dod, qd, kd, vd, out, lse, dq, dk, dv, cu_q.to(dev), cu_k.to(dev), mq, mk, p, scale,
                                       False, causal, 0, None, rng=rng)
     wdq, wdk, wdv, wsd = ofa.flash_attn_bwd(do, q, k, v, cu_q, cu_k, mq, scale, causal, p_eff, mask, D, round_to=dtype)
+    grad_atol = grad_atol / (1.0 - p)
     assert_close(dq, wdq, dtype, "dq", scale_atol=True, atol=grad_atol)
     assert_close(dk, wdk, dtype, "dk", scale_atol=True, atol=grad_atol)
     assert_close(dv, wdv, dtype, "dv", scale_atol=True, atol=grad_atol)
@@ -170,6 +172,33 @@ def test_packed_kv_function_with_dropout_repeats_its_mask_in_the_backward(dev):
     assert_close(qd.grad, wdq, dtype, "dq", scale_atol=True, atol=4e-3)
     assert_close(kvd.grad[:, 0], wdk, dtype, "dk", scale_atol=True, atol=4e-3)
     assert_close(kvd.grad[:, 1], wdv, dtype, "dv", scale_atol=True, atol=4e-3)
+
+
+@pytest.mark.parametrize("seed", range(3000, 3010))
+def test_randomly_drawn_shapes(dev, seed):
+    """Lengths around the tile sizes (64 keys, 128 queries), head counts, both head dimensions, causal or not, dropout
+    replayed, drawn or off, query and key lengths equal or independent, scale drawn too."""
+    import random
+    rnd = random.Random(seed)
+    batch, heads, d = rnd.randint(1, 5), rnd.randint(1, 4), rnd.choice([64, 128])
+    pick = lambda: rnd.choice([0, 1, 2, 63, 64, 65, 127, 128, 129, rnd.randint(1, 200), rnd.randint(1, 200)])
+    lq = [pick() for _ in range(batch)]
+    lk = lq if rnd.random() < 0.5 else [pick() for _ in range(batch)]
+    if max(lq) == 0:
+        lq = [7] + lq[1:]
+        lk = lq if lk is lq else lk
+    if max(lk) == 0:
+        lk = [9] + lk[1:]
+    dtype = rnd.choice([torch.bfloat16, torch.float16])
+    causal = rnd.random() < 0.5
+    mode = rnd.choice(["none", "replay", "philox"])
+    p = 0.0 if mode == "none" else rnd.choice([0.1, 0.3, 0.5])
+    q, k, v, do = _inputs(lq, lk, heads, d, dtype, seed)
+    mask = None
+    if mode == "replay":
+        mask = (torch.rand(batch, heads, max(lq), max(lk), generator=torch.Generator().manual_seed(seed)) >= p).to(torch.uint8)
+    _check_fwd_bwd(dev, q, k, v, do, lq, lk, causal, p=p, mask=mask, scale=rnd.choice([None, 0.05, 0.3]), philox=mode == "philox",
+                   grad_atol=1e-2)
 
 
 def test_unsupported_inputs_are_refused(dev):
