@@ -472,6 +472,32 @@ int nmtg_rel_shift_bwd(const void* grad_scores, void* grad_bd, int64_t batch, in
 int nmtg_add_rows(void* out, int64_t ld_out, const void* a, int64_t ld_a, const void* b, int64_t ld_b,
                   int64_t rows, int64_t cols, int dtype, void* stream);
 
+/* The relative shift folded into the softmax kernels, so that the score tensor is not passed over once more on either
+ * side (reference: the same lines as above plus the softmax + dropout between them,
+ * relative_self_attention_func.py:246-300 and :560-630; softmax_apex.h as for nmtg_softmax_dropout_*).
+ *
+ * nmtg_rel_softmax_dropout_fwd: scores [batch, len_q, len_k] holds the content term on entry; on return it holds
+ *   content + shift(bd)[:, :, :len_k] (bd dense [batch, len_q, len_r]; the sum rounded to the dtype as
+ *   nmtg_rel_shift_add rounds it), which the backward recomputes the probabilities from, and dropped_out
+ *   [batch, len_q, len_k] holds dropout(softmax(masked sum)). key_mask / mask_kind / heads / dropout_mask /
+ *   dropout_mode / p / seed / offset as for nmtg_softmax_dropout_fwd with rows = batch * len_q, cols = len_k,
+ *   q_len = len_q.
+ * nmtg_rel_softmax_dropout_bwd: grad_scores [batch, len_q, len_k] = softmax-dropout backward from the saved summed
+ *   scores (as nmtg_softmax_dropout_bwd with saved_is_scores = 1), and grad_bd [batch, len_q, len_r] = the shift's
+ *   adjoint of grad_scores (as nmtg_rel_shift_bwd), every element written.
+ * Both need len_k a multiple of 16 bytes of elements, 16-byte aligned tensors, len_r >= len_k, at most 4096 keys
+ * (2048 in fp32), len_q * (len_r + 1) < 2^31 and batch * len_q < 2^31; other shapes go through the separate calls.
+ * dtype: NMTG_F16, NMTG_BF16 or NMTG_F32. */
+int nmtg_rel_softmax_dropout_fwd(void* scores, const void* bd, int64_t len_r, const uint8_t* key_mask,
+                                 int mask_kind, void* dropped_out, uint8_t* dropout_mask, int dropout_mode,
+                                 float p, uint64_t seed, uint64_t offset, int64_t batch, int64_t len_q,
+                                 int64_t len_k, int64_t heads, int dtype, void* stream);
+
+int nmtg_rel_softmax_dropout_bwd(const void* grad_dropped, const void* scores, const uint8_t* key_mask,
+                                 int mask_kind, const uint8_t* dropout_mask, int dropout_mode, float p,
+                                 void* grad_scores, void* grad_bd, int64_t len_r, int64_t batch,
+                                 int64_t len_q, int64_t len_k, int64_t heads, int dtype, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Optimizer-side passes over a list of tensors (one launch per 48 tensors instead of one per tensor).
  * Reference: fused_optim.multi_tensor_adam / multi_tensor_scale / multi_tensor_axpby / multi_tensor_l2norm /

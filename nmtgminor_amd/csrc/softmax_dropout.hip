@@ -43,7 +43,43 @@ struct SoftmaxArgs {
   int from_scores;         // bwd: saved holds scores (1) or probabilities (0)
   float keep_p, scale;
   uint64_t seed, offset;
+  // relative-position form (REL kernels): rows = batch * q_len, every row also takes (forward) or feeds (backward) the
+  // shifted position term
+  const void* bd;          // fwd: position scores [batch, q_len, len_r]
+  void* scores_out;        // fwd: the summed scores, [batch, q_len, cols] (may be `in`)
+  void* grad_bd;           // bwd: gradient of the position scores [batch, q_len, len_r]
+  int len_r;
 };
+
+// The relative shift as seen from row i of a [q_len, cols] score matrix (relative_self_attention_func.py:26-50 of the
+// reference: a zero column in front of bd [q_len, len_r], the padded buffer read as [len_r + 1, q_len], first row
+// dropped). Element j of the row is padded element p = i * len_r + q_len + j, which lies in padded row i2 = p / (len_r + 1)
+// at column c = p % (len_r + 1): zero if c == 0, bd[i2][c - 1] otherwise. A row is shorter than a padded row, so it
+// crosses at most one padded-row boundary: with i2 and c0 taken for j = 0, element j has c = c0 + j counted from the
+// start of padded row i2, c == len_r + 1 is the zero column of the next padded row and anything beyond it lies one
+// element earlier in bd than c - 1 says.
+struct RelRow {
+  uint32_t i;              // the row's query position
+  uint32_t c0;             // column of the row's first element inside its padded row
+  int64_t first;           // element offset of bd[b][i2][0]
+};
+__device__ __forceinline__ RelRow rel_row(int64_t row, uint32_t q_len, uint32_t len_r) {   // row < 2^31 (checked at entry)
+  const uint32_t b = static_cast<uint32_t>(row) / q_len, i = static_cast<uint32_t>(row) - b * q_len;
+  const uint32_t p0 = i * len_r + q_len, i2 = p0 / (len_r + 1);
+  return RelRow{i, p0 - i2 * (len_r + 1), (static_cast<int64_t>(b) * q_len + i2) * len_r};
+}
+// Orders a wavefront's LDS writes before its later LDS reads of other lanes' data (and the reverse): the hardware runs
+// one wavefront's LDS instructions in order, the fences keep the compiler from moving them.
+__device__ __forceinline__ void wave_lds_fence() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+// offset from RelRow::first of the bd element behind column c, or -1 for the zero column
+__device__ __forceinline__ int rel_source(uint32_t c, uint32_t len_r) {
+  if (c == 0 || c == len_r + 1) return -1;
+  return static_cast<int>(c) - 1 - (c > len_r + 1 ? 1 : 0);
+}
 
 // 32-bit index arithmetic wherever the row count allows it (a 64-bit division is some 140 scalar instructions,
 // as much as the rest of a short row's work).
@@ -125,7 +161,11 @@ __device__ __forceinline__ void row_softmax(const pack<T, EPV> (&rx)[VPL], const
 // RNG (the keep mask is drawn here from Philox and stored) is a compile-time switch: as a run-time branch the
 // generator's ~200 integer instructions per 8 elements were scheduled ahead of the branch and ran in every mode,
 // which made the kernel instruction-bound (about 290 vector instructions per 512-key row instead of about 90).
-template <typename T, int EPV, int VPL, int RPW, bool RNG>
+// REL: the scores are the sum of the content term (a.in) and the shifted position term (a.bd); the sum, rounded to T as
+// a separate addition would round it, is stored to a.scores_out for the backward and is what the softmax sees. The
+// shifted operand is not aligned with the row, so it is read element by element (consecutive lanes, consecutive
+// addresses) and turned into the row's register layout through LDS.
+template <typename T, int EPV, int VPL, int RPW, bool RNG, bool REL = false>
 __global__ __launch_bounds__(SM_THREADS) void softmax_fwd_kernel(SoftmaxArgs a) {
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t row0 = (static_cast<int64_t>(blockIdx.x) * SM_WAVES + __builtin_amdgcn_readfirstlane(threadIdx.x / kWave)) * RPW;
@@ -133,6 +173,8 @@ __global__ __launch_bounds__(SM_THREADS) void softmax_fwd_kernel(SoftmaxArgs a) 
   const bool mask_in = !RNG && a.dropout_mode == SM_MASK_IN;
   const bool masked = a.kmask_kind != SM_NOMASK;
   pack<T, EPV> rx[RPW][VPL];
+  [[maybe_unused]] pack<T, VPL * EPV> rb[REL ? RPW : 1];
+  [[maybe_unused]] __shared__ __align__(16) T stage_all[REL ? SM_WAVES * RPW * EPV * VPL * kWave : 1];
   pack<uint8_t, EPV> rk[RPW][VPL] = {}, rd[RPW][VPL] = {};
 #pragma unroll
   for (int r = 0; r < RPW; ++r) {
@@ -140,14 +182,48 @@ __global__ __launch_bounds__(SM_THREADS) void softmax_fwd_kernel(SoftmaxArgs a) 
     row_load<T, EPV, VPL>(static_cast<const T*>(a.in) + row * a.cols, a.cols, lane, rx[r]);
     if (masked) row_load<uint8_t, EPV, VPL>(kmask_row(a, row), a.cols, lane, rk[r]);
     if (mask_in) row_load<uint8_t, EPV, VPL>(a.dmask + row * a.cols, a.cols, lane, rd[r]);
+    if constexpr (REL) {
+      // lane l takes elements l, 64 + l, ... of the shifted row: consecutive lanes read consecutive addresses
+      const RelRow rr = rel_row(row, a.q_len, a.len_r);
+      const T* src = static_cast<const T*>(a.bd) + rr.first;
+#pragma unroll
+      for (int k = 0; k < VPL * EPV; ++k) {
+        const int e = k * kWave + lane;
+        const int at = e < a.cols ? rel_source(rr.c0 + e, a.len_r) : -1;
+        rb[r].v[k] = at >= 0 ? src[at] : elem<T>::from_float(0.f);
+      }
+    }
   }
 #pragma unroll
   for (int r = 0; r < RPW; ++r) { row_pin(rx[r]); row_pin(rk[r]); row_pin(rd[r]); }
+  if constexpr (REL) {
+    // through the wavefront's strips of LDS into the layout of the other operands (lane l: elements EPV l ...)
+    T* strip = stage_all + (threadIdx.x / kWave) * (RPW * EPV * VPL * kWave);
+#pragma unroll
+    for (int r = 0; r < RPW; ++r)
+#pragma unroll
+      for (int k = 0; k < VPL * EPV; ++k) strip[r * (EPV * VPL * kWave) + k * kWave + lane] = rb[r].v[k];
+    wave_lds_fence();
+  }
   [[maybe_unused]] const Philox gen(a.seed);
 #pragma unroll
   for (int r = 0; r < RPW; ++r) {
     if (row0 + r >= a.rows) break;
     const int64_t base = (row0 + r) * a.cols;
+    if constexpr (REL) {
+#pragma unroll
+      for (int i = 0; i < VPL; ++i) {
+        const int col = row_col<EPV>(i, lane);
+        if (col < a.cols) {
+          float x[EPV], sh[EPV];
+          unpack_raw<T, EPV>(rx[r][i], x);
+          load_pack<T, EPV>(stage_all + ((threadIdx.x / kWave) * RPW + r) * (EPV * VPL * kWave) + col, sh);
+#pragma unroll
+          for (int u = 0; u < EPV; ++u) rx[r][i].v[u] = elem<T>::from_float(x[u] + sh[u]);
+          *reinterpret_cast<pack<T, EPV>*>(static_cast<T*>(a.scores_out) + base + col) = rx[r][i];
+        }
+      }
+    }
     float v[VPL][EPV];
     row_softmax<T, EPV, VPL>(rx[r], rk[r], masked, a.cols, lane, v);
     T* out = static_cast<T*>(a.out) + base;
@@ -176,8 +252,14 @@ __global__ __launch_bounds__(SM_THREADS) void softmax_fwd_kernel(SoftmaxArgs a) 
 }
 
 // dS = P * (g - sum_k P * g), g = keep * dP / (1 - p).
-template <typename T, int EPV, int VPL, int RPW>
+// REL: the score gradient also leaves through the adjoint of the relative shift (relative_self_attention_func.py:52-76
+// of the reference), as grad_bd [batch, q_len, len_r]. Row i of the scores owns the padded elements from its own first
+// one up to the next row's first one (row 0 also those in front of it): its len_k gradients, then zeros. The
+// destinations are not aligned with the row either, so the row goes through the wavefront's strip of LDS and is
+// stored element by element, consecutive lanes to consecutive addresses.
+template <typename T, int EPV, int VPL, int RPW, bool REL = false>
 __global__ __launch_bounds__(SM_THREADS) void softmax_bwd_kernel(SoftmaxArgs a) {
+  [[maybe_unused]] __shared__ __align__(16) T stage_all[REL ? SM_WAVES * EPV * VPL * kWave : 1];
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t row0 = (static_cast<int64_t>(blockIdx.x) * SM_WAVES + __builtin_amdgcn_readfirstlane(threadIdx.x / kWave)) * RPW;
   if (row0 >= a.rows) return;
@@ -236,7 +318,27 @@ __global__ __launch_bounds__(SM_THREADS) void softmax_bwd_kernel(SoftmaxArgs a) 
 #pragma unroll
         for (int j = 0; j < EPV; ++j) g[i][j] = pr[i][j] * (g[i][j] - dot);
         store_pack<T, EPV>(out + col, g[i]);
+        if constexpr (REL) store_pack<T, EPV>(stage_all + (threadIdx.x / kWave) * (EPV * VPL * kWave) + col, g[i]);
       }
+    }
+    if constexpr (REL) {
+      const T* stage = stage_all + (threadIdx.x / kWave) * (EPV * VPL * kWave);
+      const uint32_t len_r = a.len_r, q_len = a.q_len;
+      const RelRow rr = rel_row(row0 + r, q_len, len_r);
+      T* dst = static_cast<T*>(a.grad_bd) + rr.first;
+      wave_lds_fence();                                  // the strip is written and read by different lanes
+      for (uint32_t j = lane; j < len_r; j += kWave) {   // the row's gradients, then zeros up to the next row's start
+        const int at = rel_source(rr.c0 + j, len_r);
+        if (at >= 0) dst[at] = j < static_cast<uint32_t>(a.cols) ? stage[j] : elem<T>::from_float(0.f);
+      }
+      if (rr.i == 0) {                                   // the padded elements in front of row 0
+        T* head = static_cast<T*>(a.grad_bd) + (row0 + r) * static_cast<int64_t>(len_r);
+        for (uint32_t p = lane; p < q_len; p += kWave) {
+          const uint32_t i2 = p / (len_r + 1);
+          if (p != i2 * (len_r + 1)) head[p - i2 - 1] = elem<T>::from_float(0.f);
+        }
+      }
+      wave_lds_fence();                                  // before the next row overwrites the strip
     }
   }
 }
@@ -289,6 +391,43 @@ int softmax_launch(const SoftmaxArgs& a, bool bwd, hipStream_t st) {
     return fail(NMTG_ERR_UNSUPPORTED,
                 "softmax: row length %d is beyond what one wavefront holds at vector width %d "
                 "(limit 4096 keys for aligned 16-bit rows, 2048 otherwise)", a.cols, epv);
+  return 0;
+}
+
+// The relative-position kernels exist at full vector width only (rows of a multiple of 16 bytes).
+template <typename T>
+int softmax_rel_launch(const SoftmaxArgs& a, bool bwd, hipStream_t st) {
+  constexpr int E = 16 / sizeof(T);
+  const int vecs = a.cols / E;
+  int vpl = 1;
+  while (vpl * kWave < vecs) vpl *= 2;
+  const bool rng = !bwd && a.dropout_mode == SM_MASK_RNG;
+  TraceScope trace(bwd ? "rel_softmax_dropout_bwd" : "rel_softmax_dropout_fwd", st);
+  bool done = false;
+#define REL_CASE(V)                                                                                                     \
+  if (!done && vpl == V) {                                                                                              \
+    constexpr int R = V == 1 ? 4 : V == 2 ? 2 : 1;                                                                      \
+    const unsigned grid = static_cast<unsigned>((a.rows + SM_WAVES * R - 1) / (SM_WAVES * R));                          \
+    if (bwd) hipLaunchKernelGGL((softmax_bwd_kernel<T, E, V, R, true>), dim3(grid), dim3(SM_THREADS), 0, st, a);        \
+    else if (rng) hipLaunchKernelGGL((softmax_fwd_kernel<T, E, V, R, true, true>), dim3(grid), dim3(SM_THREADS), 0, st, a);  \
+    else hipLaunchKernelGGL((softmax_fwd_kernel<T, E, V, R, false, true>), dim3(grid), dim3(SM_THREADS), 0, st, a);     \
+    done = true;                                                                                                        \
+  }
+  REL_CASE(1) REL_CASE(2) REL_CASE(4) REL_CASE(8)
+#undef REL_CASE
+  if (!done) return fail(NMTG_ERR_UNSUPPORTED, "rel_softmax_dropout: %d keys are beyond what one wavefront holds (%d)", a.cols, 8 * kWave * E);
+  return 0;
+}
+
+int check_rel(const char* who, const void* const* ptrs, int n_ptrs, int64_t batch, int64_t len_q, int64_t len_k, int64_t len_r, int dtype) {
+  NMTG_REQUIRE(batch >= 0 && len_q >= 0 && len_k > 0 && len_r >= len_k, "%s: bad shape batch=%lld len_q=%lld len_k=%lld len_r=%lld (len_r >= len_k)",
+               who, (long long)batch, (long long)len_q, (long long)len_k, (long long)len_r);
+  NMTG_REQUIRE(len_q * (len_r + 1) < (int64_t{1} << 31) && batch * len_q < (int64_t{1} << 31),
+               "%s: sizes beyond the kernel's 32-bit indices (len_q * (len_r + 1) and batch * len_q below 2^31)", who);
+  const int wide = dtype == NMTG_F32 ? 4 : 8;
+  NMTG_REQUIRE(len_k % wide == 0, "%s: len_k = %lld is not a multiple of %d elements (use the separate shift and softmax calls)", who,
+               (long long)len_k, wide);
+  for (int k = 0; k < n_ptrs; ++k) NMTG_REQUIRE(aligned16(ptrs[k]), "%s: 16-byte aligned tensors required", who);
   return 0;
 }
 
@@ -355,5 +494,53 @@ extern "C" int nmtg_softmax_dropout_bwd(const void* grad_dropped, const void* sa
   NMTG_DISPATCH_DTYPE(dtype, T, rc = softmax_launch<T>(a, true, static_cast<hipStream_t>(stream)));
   if (rc) return rc;
   NMTG_CHECK_LAUNCH("softmax_dropout_bwd");
+  return 0;
+}
+
+
+extern "C" int nmtg_rel_softmax_dropout_fwd(void* scores, const void* bd, int64_t len_r, const uint8_t* key_mask, int mask_kind,
+                                            void* dropped_out, uint8_t* dropout_mask, int dropout_mode, float p, uint64_t seed,
+                                            uint64_t offset, int64_t batch, int64_t len_q, int64_t len_k, int64_t heads, int dtype,
+                                            void* stream) {
+  const void* ptrs[] = {scores, bd, dropped_out};
+  if (int rc = check_rel("rel_softmax_dropout_fwd", ptrs, 3, batch, len_q, len_k, len_r, dtype)) return rc;
+  NMTG_REQUIRE(heads >= 0 && heads <= INT32_MAX, "rel_softmax_dropout_fwd: bad heads");
+  SoftmaxArgs a{};
+  a.in = scores; a.scores_out = scores; a.bd = bd; a.len_r = static_cast<int>(len_r);
+  a.out = dropped_out; a.dmask = dropout_mask; a.kmask = key_mask;
+  a.rows = batch * len_q; a.cols = static_cast<int>(len_k); a.q_len = static_cast<int>(len_q); a.heads = static_cast<int>(heads);
+  a.kmask_kind = mask_kind; a.dropout_mode = dropout_mode;
+  a.keep_p = 1.f - p; a.scale = 1.f / (1.f - p); a.seed = seed; a.offset = offset;
+  if (a.rows == 0) return 0;
+  if (int rc = check_common("rel_softmax_dropout_fwd", a, p)) return rc;
+  NMTG_REQUIRE(scores && bd && dropped_out, "rel_softmax_dropout_fwd: null pointer argument");
+  int rc = 0;
+  NMTG_DISPATCH_DTYPE(dtype, T, rc = softmax_rel_launch<T>(a, false, static_cast<hipStream_t>(stream)));
+  if (rc) return rc;
+  NMTG_CHECK_LAUNCH("rel_softmax_dropout_fwd");
+  return 0;
+}
+
+extern "C" int nmtg_rel_softmax_dropout_bwd(const void* grad_dropped, const void* scores, const uint8_t* key_mask, int mask_kind,
+                                            const uint8_t* dropout_mask, int dropout_mode, float p, void* grad_scores,
+                                            void* grad_bd, int64_t len_r, int64_t batch, int64_t len_q, int64_t len_k,
+                                            int64_t heads, int dtype, void* stream) {
+  const void* ptrs[] = {grad_dropped, scores, grad_scores, grad_bd};
+  if (int rc = check_rel("rel_softmax_dropout_bwd", ptrs, 4, batch, len_q, len_k, len_r, dtype)) return rc;
+  NMTG_REQUIRE(heads >= 0 && heads <= INT32_MAX, "rel_softmax_dropout_bwd: bad heads");
+  NMTG_REQUIRE(dropout_mode != SM_MASK_RNG, "rel_softmax_dropout_bwd: the backward replays a stored mask (mode 0 or 1)");
+  SoftmaxArgs a{};
+  a.in = grad_dropped; a.saved = scores; a.out = grad_scores; a.grad_bd = grad_bd; a.len_r = static_cast<int>(len_r);
+  a.dmask = const_cast<uint8_t*>(dropout_mask); a.kmask = key_mask;
+  a.rows = batch * len_q; a.cols = static_cast<int>(len_k); a.q_len = static_cast<int>(len_q); a.heads = static_cast<int>(heads);
+  a.kmask_kind = mask_kind; a.dropout_mode = dropout_mode; a.from_scores = 1;
+  a.keep_p = 1.f - p; a.scale = 1.f / (1.f - p);
+  if (a.rows == 0) return 0;
+  if (int rc = check_common("rel_softmax_dropout_bwd", a, p)) return rc;
+  NMTG_REQUIRE(grad_dropped && scores && grad_scores && grad_bd, "rel_softmax_dropout_bwd: null pointer argument");
+  int rc = 0;
+  NMTG_DISPATCH_DTYPE(dtype, T, rc = softmax_rel_launch<T>(a, true, static_cast<hipStream_t>(stream)));
+  if (rc) return rc;
+  NMTG_CHECK_LAUNCH("rel_softmax_dropout_bwd");
   return 0;
 }

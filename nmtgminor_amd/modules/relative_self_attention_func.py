@@ -4,9 +4,10 @@ Mirrors RelativeShift, RelativeSelfAttnFunc and relative_self_attn_func of the r
 (onmt/modules/optimized/relative_self_attention_func.py:26-76, :79-726, :738-766): the same 21 positional arguments and
 21 gradient slots. The projected-position form runs in native/relative_self_attn_blaslt.py (the stand-in of the reference's
 extension of that name). Every product is an MFMA GEMM (nmtg_gemm through native/linear_gemm.py and native/linear_blaslt.py),
-the additions of r_w_bias / r_r_bias, the relative shift with the sum of the two score terms and the shift's adjoint are
-the kernels of native/relative_position.py, softmax + dropout is the fused kernel of the other attention ops (mask fused,
-probabilities recomputed from the saved scores in the backward), the bias gradients are column-sum kernels and the two
+the additions of r_w_bias / r_r_bias are a kernel of native/relative_position.py, the relative shift with the sum of the two
+score terms runs inside the softmax + dropout kernel and the shift's adjoint inside that kernel's backward (mask fused,
+probabilities recomputed from the saved scores in the backward; separate shift kernels for key lengths the wide kernels do
+not take), the bias gradients are column-sum kernels and the two
 query-gradient terms are joined by the row-add kernel. What is left to PyTorch: views and allocation.
 
 Covered: sinusoidal positions projected by pos_weights (learnable_pos=False) and learnable position embeddings

@@ -1,9 +1,14 @@
 """Thin Python face of the elementwise kernels of self-attention with relative position encodings: the additions of
 r_w_bias / r_r_bias to the queries, RelativeShift.forward fused with the sum of the two score terms, and
-RelativeShift.backward (onmt/modules/optimized/relative_self_attention_func.py:26-76, :210-217, :246-253, :621-630)."""
+RelativeShift.backward (onmt/modules/optimized/relative_self_attention_func.py:26-76, :210-217, :246-253, :621-630); and
+of the two kernels that run the shift inside the softmax + dropout pass and its adjoint inside that pass's backward."""
+import ctypes
+import os
+
 import torch
 
 from .. import _lib as L
+from .._rng import philox_seed_offset
 
 
 def _check(cond, msg):
@@ -53,6 +58,70 @@ def shift_backward(grad_scores, len_r):
     L.call("nmtg_rel_shift_bwd", L.ptr(grad_scores), L.ptr(out), L.i64(b), L.i64(tq), L.i64(tk), L.i64(len_r),
            L.i32(L.dtype_code(grad_scores)), L.stream_of(grad_scores))
     return out
+
+
+def fused_ok(scores_shape, dtype, len_r):
+    """Whether the softmax kernels can take the shift along (rel_softmax_dropout_*): rows of a multiple of 16 bytes, at
+    most 4096 keys (2048 in fp32), 32-bit indices inside the kernel; NMTG_REL_FUSED=0 switches the route off."""
+    if os.environ.get("NMTG_REL_FUSED", "1") == "0":
+        return False
+    b, tq, tk = scores_shape
+    wide = 4 if dtype == torch.float32 else 8
+    return (b > 0 and tq > 0 and tk > 0 and tk % wide == 0 and tk <= 512 * wide and len_r >= tk
+            and tq * (len_r + 1) < 2 ** 31 and b * tq < 2 ** 31)
+
+
+def shift_add_softmax_dropout(scores, bd, is_training, heads, dropout_prob, mask, mask_kind, dropout_mask=None):
+    """scores [batch, len_q, len_k] (content term; replaced by the sum with the shifted position term bd
+    [batch, len_q, len_r]) -> (dropout_mask, dropped probabilities). One pass instead of shift_add_ followed by the
+    softmax; mask / mask_kind as the softmax kernels take them (uint8, 1 = pad mask [batch/heads, len_k], 2 = time mask)."""
+    L.require_cuda(scores, bd, mask, dropout_mask)
+    _check(scores.dim() == 3 and bd.dim() == 3 and scores.is_contiguous() and bd.is_contiguous()
+           and scores.shape[:2] == bd.shape[:2] and scores.dtype == bd.dtype,
+           "shift_add_softmax_dropout: contiguous [batch, len_q, len_k] and [batch, len_q, len_r] tensors of one dtype required")
+    b, tq, tk = scores.shape
+    dropped = torch.empty_like(scores)
+    if is_training and dropout_prob > 0.0:
+        if dropout_mask is not None:
+            _check(dropout_mask.dtype == torch.uint8 and dropout_mask.numel() == scores.numel(), "shift_add_softmax_dropout: bad dropout mask")
+            dropout_mask, mode, seed, offset = dropout_mask.contiguous(), 1, 0, 0
+        else:
+            dropout_mask, mode = torch.empty(scores.shape, dtype=torch.uint8, device=scores.device), 2
+            seed, offset = philox_seed_offset(scores.device, scores.numel())
+    else:
+        mode, seed, offset = 0, 0, 0
+        dropout_mask = torch.empty(0, dtype=torch.uint8, device=scores.device)
+    L.call("nmtg_rel_softmax_dropout_fwd", L.ptr(scores), L.ptr(bd), L.i64(bd.shape[2]), L.ptr(mask), L.i32(mask_kind),
+           L.ptr(dropped), L.ptr(dropout_mask if mode else None), L.i32(mode), L.f32(dropout_prob), ctypes.c_uint64(seed),
+           ctypes.c_uint64(offset), L.i64(b), L.i64(tq), L.i64(tk), L.i64(heads), L.i32(L.dtype_code(scores)),
+           L.stream_of(scores))
+    return dropout_mask, dropped
+
+
+def softmax_dropout_shift_backward(grad_dropped, scores, len_r, heads, dropout_mask, dropout_prob, mask, mask_kind, *,
+                                   grad_bd=None):
+    """-> (grad wrt the summed scores [batch, len_q, len_k], its shift adjoint [batch, len_q, len_r]) from the gradient of
+    the dropped probabilities and the saved summed scores, in one pass. `grad_bd`: a buffer to write the adjoint to."""
+    L.require_cuda(grad_dropped, scores, dropout_mask, mask)
+    grad_dropped = grad_dropped.contiguous()
+    _check(scores.is_contiguous() and scores.shape == grad_dropped.shape and scores.dtype == grad_dropped.dtype,
+           "softmax_dropout_shift_backward: saved scores must match the gradient")
+    b, tq, tk = scores.shape
+    use_mask = dropout_mask is not None and dropout_mask.numel() > 0 and dropout_prob > 0.0
+    if use_mask:
+        _check(dropout_mask.dtype == torch.uint8 and dropout_mask.numel() == scores.numel(), "softmax_dropout_shift_backward: bad dropout mask")
+        dropout_mask = dropout_mask.contiguous()
+    grad_scores = torch.empty_like(scores)
+    if grad_bd is None:
+        grad_bd = torch.empty(b, tq, len_r, dtype=scores.dtype, device=scores.device)
+    _check(grad_bd.shape == (b, tq, len_r) and grad_bd.dtype == scores.dtype and grad_bd.is_contiguous(),
+           "softmax_dropout_shift_backward: grad_bd must be a contiguous [batch, len_q, len_r] tensor of the scores' dtype")
+    L.require_cuda(grad_bd)
+    L.call("nmtg_rel_softmax_dropout_bwd", L.ptr(grad_dropped), L.ptr(scores), L.ptr(mask), L.i32(mask_kind),
+           L.ptr(dropout_mask if use_mask else None), L.i32(1 if use_mask else 0), L.f32(dropout_prob), L.ptr(grad_scores),
+           L.ptr(grad_bd), L.i64(len_r), L.i64(b), L.i64(tq), L.i64(tk), L.i64(heads), L.i32(L.dtype_code(scores)),
+           L.stream_of(scores))
+    return grad_scores, grad_bd
 
 
 def _rows_view(t, what):

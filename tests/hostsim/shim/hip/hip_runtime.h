@@ -120,6 +120,12 @@ static inline float __builtin_amdgcn_fdot2_f32_bf16(hostsim_bf16x2 a, hostsim_bf
   return acc + static_cast<float>(a[0]) * static_cast<float>(b[0]) + static_cast<float>(a[1]) * static_cast<float>(b[1]);
 }
 
+// Wavefront barrier: every lane arrives before any continues (the lanes run as fibers, so this is what makes one
+// lane's earlier LDS writes visible to the others); the fences around it only constrain the device compiler.
+static inline void hostsim_no_resolver(void**, int) {}
+static inline void __builtin_amdgcn_wave_barrier() { hostsim::wave_collective(hostsim_no_resolver, nullptr); }
+#define __builtin_amdgcn_fence(order, scope) ((void)0)
+
 // v_cmp into a wavefront-wide mask: bit l is lane l's predicate
 static inline uint64_t __builtin_amdgcn_ballot_w64(bool pred) {
   uint64_t mask = 0;

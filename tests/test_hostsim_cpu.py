@@ -472,6 +472,14 @@ def test_relative_shift_kernels(mi355x, dtype, b, tq, tk, r):
     trel.test_shift_add_and_its_adjoint_move_values_exactly(CPU, dtype, b, tq, tk, r)
 
 
+@pytest.mark.parametrize("dtype", [BF16, F32])
+@pytest.mark.parametrize("bh,heads,tq,tk,r,mask,p", [(4, 2, 24, 24, 40, "pad", 0.25), (2, 1, 40, 16, 16, "time", 0.25),
+                                                     (2, 2, 5, 1032, 1032, None, 0.1), (3, 1, 1, 8, 8, None, 0.0)])
+def test_relative_shift_folded_into_the_softmax(mi355x, dtype, bh, heads, tq, tk, r, mask, p):
+    trel.test_shift_folded_into_the_softmax_matches_the_separate_kernels(CPU, dtype, bh, heads, tq, tk, r, mask, p)
+    trel.test_fused_shift_is_refused_for_rows_the_wide_kernels_cannot_take(CPU)
+
+
 def test_relative_position_elementwise_kernels_and_linear_layer(mi355x):
     trel.test_shift_refuses_fewer_positions_than_keys(CPU)
     for t, b, h, d in ((5, 2, 4, 64), (3, 1, 3, 20), (4, 2, 2, 7)):

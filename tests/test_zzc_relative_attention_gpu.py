@@ -40,6 +40,67 @@ def test_shift_add_and_its_adjoint_move_values_exactly(dev, dtype, b, tq, tk, r)
         assert torch.equal(RelativeShift.backward(gs.to(dev), True, False).cpu().to(D), orel.relative_shift_bwd(gs.to(D)))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("bh,heads,tq,tk,r,mask,p", [
+    (4, 2, 16, 16, 16, None, 0.0), (4, 2, 24, 24, 40, "pad", 0.25), (2, 1, 40, 16, 16, "time", 0.25), (6, 3, 5, 72, 80, "pad", 0.5),
+    (2, 2, 9, 1032, 1032, None, 0.1), (2, 1, 3, 2048, 2049, "time", 0.1), (1, 1, 130, 64, 64, None, 0.3), (3, 1, 1, 8, 8, None, 0.0)])
+def test_shift_folded_into_the_softmax_matches_the_separate_kernels(dev, dtype, bh, heads, tq, tk, r, mask, p):
+    """One kernel for shift + sum + softmax + dropout, and one for their adjoints, against the chain of separate kernels:
+    the same roundings in the same places. The summed scores that are kept for the backward and the movement of the
+    score gradient into the position term's gradient are compared bit for bit (that buffer starts out as NaN, so an
+    element left unwritten shows); probabilities and score gradients to four units in the last place of the dtype,
+    because the separate softmax spreads a short row over the lanes differently and so adds the row up in another
+    order. The keep mask that the fused kernel draws is replayed in the separate chain (the generator's stream depends
+    on how a row is spread over the lanes)."""
+    from nmtgminor_amd.native import mask_softmax_dropout_cuda as softmax_native
+    assert relative_position.fused_ok((bh, tq, tk), dtype, r)
+    g = torch.Generator().manual_seed(bh * 1000 + tq * 10 + r)
+    ac, bd = torch.randn(bh, tq, tk, generator=g).to(dtype).to(dev), torch.randn(bh, tq, r, generator=g).to(dtype).to(dev)
+    grad = torch.randn(bh, tq, tk, generator=g).to(dtype).to(dev)
+    mask_kw, km, kind = {}, None, 0
+    if mask == "pad":
+        pad = torch.rand(bh // heads, tk, generator=g) < 0.3
+        pad[:, 0] = False
+        pad[-1, :] = tq > 5                                                 # one sentence without any live key
+        mask_kw, km, kind = dict(pad_mask=pad.to(dev)), pad.to(torch.uint8).to(dev), 1
+    elif mask == "time":
+        tm = torch.triu(torch.ones(tq, tk), diagonal=1).bool()
+        mask_kw, km, kind = dict(time_mask=tm.to(dev)), tm.to(torch.uint8).to(dev), 2
+    training = p > 0
+    s2 = ac.clone()
+    dm2, dr2 = relative_position.shift_add_softmax_dropout(s2, bd, training, heads, p, km, kind)        # mask drawn in the kernel
+    s1 = relative_position.shift_add_(ac.clone(), bd)
+    dm1, _, dr1 = softmax_native.forward(training, heads, s1, p, want_softmax=False, dropout_mask=dm2 if training else None,
+                                         **mask_kw)                                                     # the same mask replayed
+    ulp2 = 4 * torch.finfo(dtype).eps
+    assert torch.equal(s1, s2)
+    torch.testing.assert_close(dr2.float(), dr1.float(), rtol=ulp2, atol=1e-4 * ulp2)
+    if training:
+        assert dm2.shape == (bh, tq, tk) and abs(dm2.float().mean().item() - (1 - p)) < 4 * (p * (1 - p) / dm2.numel()) ** 0.5 + 1e-3
+        dm3, dr3 = relative_position.shift_add_softmax_dropout(ac.clone(), bd, training, heads, p, km, kind, dm2)   # replayed mask
+        assert torch.equal(dr3.view(torch.uint8), dr2.view(torch.uint8)) and dm3 is not None
+    gs1 = softmax_native.backward_recompute(heads, grad, None, s1, dm1, p, **mask_kw)
+    gb1 = relative_position.shift_backward(gs1, r)
+    gb2 = torch.full((bh, tq, r), float("nan"), dtype=dtype, device=dev)
+    gs2, _ = relative_position.softmax_dropout_shift_backward(grad, s2, r, heads, dm2, p, km, kind, grad_bd=gb2)
+    torch.testing.assert_close(gs2.float(), gs1.float(), rtol=ulp2, atol=ulp2)       # p (g - sum p g): a difference of O(1) terms
+    assert not torch.isnan(gb2).any()
+    assert torch.equal(gb2, relative_position.shift_backward(gs2, r))
+    torch.testing.assert_close(gb2.float(), gb1.float(), rtol=ulp2, atol=ulp2)
+
+
+def test_fused_shift_is_refused_for_rows_the_wide_kernels_cannot_take(dev):
+    assert not relative_position.fused_ok((2, 8, 12, ), torch.bfloat16, 16)       # not a multiple of 16 bytes
+    assert not relative_position.fused_ok((2, 8, 4104), torch.bfloat16, 4104)     # beyond one wavefront's row
+    assert not relative_position.fused_ok((2, 8, 16), torch.bfloat16, 8)          # fewer positions than keys
+    with pytest.raises(RuntimeError, match="multiple"):
+        relative_position.shift_add_softmax_dropout(torch.zeros(1, 4, 12, dtype=torch.bfloat16, device=dev),
+                                                    torch.zeros(1, 4, 16, dtype=torch.bfloat16, device=dev), False, 1, 0.0, None, 0)
+    with pytest.raises(RuntimeError, match="len_r"):
+        relative_position.softmax_dropout_shift_backward(torch.zeros(1, 4, 16, dtype=torch.bfloat16, device=dev),
+                                                         torch.zeros(1, 4, 16, dtype=torch.bfloat16, device=dev), 8, 1, None, 0.0, None, 0)
+
+
 def test_shift_refuses_fewer_positions_than_keys(dev):
     with pytest.raises(RuntimeError):
         relative_position.shift_add_(torch.zeros(1, 4, 8, dtype=torch.bfloat16, device=dev),
