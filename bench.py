@@ -334,7 +334,7 @@ class FlashAttnWL(Workload):
         lse, = self.m.fwd(q, k, v, self.out, self.cu, self.cu, self.max_len, self.max_len, self.P, self.scale, False, False,
                           False, rng=(20250101, 0))        # a fixed Philox state: the step is captured into a graph
         return self.m.bwd(self.dout, q, k, v, self.out, lse, self.dqkv[:, 0], self.dqkv[:, 1], self.dqkv[:, 2], self.cu, self.cu,
-                          self.max_len, self.max_len, self.P, self.scale, False, False, rng=(2, 20250101, 0, None))
+                          self.max_len, self.max_len, self.P, self.scale, False, False, rng=self.m.last_rng)   # with the forward's keep bits
 
     def _flops_fwd(self):
         return sum(2 * 2.0 * self.H * n * n * self.D for n in self.lens)        # Q K^T and P V per sequence and head

@@ -353,10 +353,20 @@ int nmtg_rotary(void* x, const void* cos_table, const void* sin_table, int64_t t
  * is below t = round(256 (1 - p)), scale 256 / t; dropout_mask_out, when not null, receives the
  * keep flags in the layout of dropout_mask. The backward regenerates the same mask from the same
  * (seed, offset).
+ * dropout_bits (modes 1 and 2; may be NULL in mode 0): device workspace of
+ * nmtg_flash_attn_dropout_bits_bytes(batch, heads, max_seqlen_q, max_seqlen_k) bytes, 16-byte
+ * aligned. A small kernel ahead of the attention kernels fills it with the keep decisions, one bit
+ * per element, and the attention kernels read only that (the generator's integer arithmetic would
+ * otherwise cost them more than the softmax). A caller that keeps the workspace of the forward
+ * call hands it to the backward with dropout_bits_ready = 1, which then neither runs the generator
+ * nor reads dropout_mask; with 0 the backward fills it again from (seed, offset) or the mask.
  * nmtg_flash_attn_bwd: dq, dk, dv in views like q, k, v (every row of every sequence written),
  * softmax_d [batch, heads, max_seqlen_q] = rowsum(dout * out) (fp32, written). Deterministic: no
  * atomics.
  * ------------------------------------------------------------------------------------------ */
+int64_t nmtg_flash_attn_dropout_bits_bytes(int64_t batch, int64_t heads, int64_t max_seqlen_q,
+                                           int64_t max_seqlen_k);
+
 int nmtg_flash_attn_fwd(const void* q, const void* k, const void* v, void* out,
                         const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, float* softmax_lse,
                         int64_t batch, int64_t heads, int64_t head_dim, int64_t max_seqlen_q,
@@ -364,8 +374,8 @@ int nmtg_flash_attn_fwd(const void* q, const void* k, const void* v, void* out,
                         int64_t k_stride_t, int64_t k_stride_h, int64_t v_stride_t, int64_t v_stride_h,
                         int64_t out_stride_t, int64_t out_stride_h, float softmax_scale, int causal,
                         int dropout_mode, float dropout_p, const uint8_t* dropout_mask,
-                        uint8_t* dropout_mask_out, uint64_t seed, uint64_t offset, int dtype,
-                        void* stream);
+                        uint8_t* dropout_mask_out, void* dropout_bits, uint64_t seed, uint64_t offset,
+                        int dtype, void* stream);
 
 int nmtg_flash_attn_bwd(const void* dout, const void* q, const void* k, const void* v,
                         const void* out, const float* softmax_lse, void* dq, void* dk, void* dv,
@@ -377,8 +387,8 @@ int nmtg_flash_attn_bwd(const void* dout, const void* q, const void* k, const vo
                         int64_t out_stride_h, int64_t dq_stride_t, int64_t dq_stride_h,
                         int64_t dk_stride_t, int64_t dk_stride_h, int64_t dv_stride_t,
                         int64_t dv_stride_h, float softmax_scale, int causal, int dropout_mode,
-                        float dropout_p, const uint8_t* dropout_mask, uint64_t seed, uint64_t offset,
-                        int dtype, void* stream);
+                        float dropout_p, const uint8_t* dropout_mask, void* dropout_bits,
+                        int dropout_bits_ready, uint64_t seed, uint64_t offset, int dtype, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Attention of ONE new query position over cached keys / values (incremental decoding).

@@ -17,9 +17,13 @@
 //   No atomics and no accumulation across blocks: results do not depend on scheduling.
 // Dropout keeps element (query i, key j) of (sequence b, head h) when byte 4 (i % 4) + (j % 4) of the Philox block with
 // index ((b H + h) ceil(max_q / 4) + i / 4) ceil(max_k / 4) + j / 4 is below round(256 (1 - p)); kept probabilities are
-// scaled by 256 / that threshold, so the expectation is exact although p is quantised to 1/256. A 4 x 4 patch per
-// block serves both tilings (a lane holds four consecutive keys of one query in one, four consecutive queries of one
-// key in the other); the four lanes that share a patch split the generator calls between them (one call per 16 elements).
+// scaled by 256 / that threshold, so the expectation is exact although p is quantised to 1/256. The three kernels do
+// not run the generator (its ten rounds of quarter-rate integer multiplies cost more than the softmax): a small kernel
+// ahead of them turns the decisions into one bit per element, one 32-bit word per (group of 32 queries, key). In the
+// query-major kernels (forward, dQ) a lane pair is a query and an accumulator register a key, so the pair of words
+// of the two keys that a register holds in the two halves of the wavefront IS the lane mask of a select: it is loaded
+// into scalar registers and costs no vector instruction besides the select. The key-major kernel (dK / dV) loads its
+// key's word per group of queries and tests bits. An explicit byte mask is turned into the same words.
 #include "gemm.cuh"
 
 namespace nmtg {
@@ -42,12 +46,19 @@ struct FaArgs {
   int heads, max_q, max_k;
   float scale, scale_log2;
   int causal;
-  const uint8_t* mask;   // explicit keep-mask [B, H, max_q, max_k] (DROP == 1)
-  uint8_t* mask_out;     // where the drawn mask is written, or null (DROP == 2)
-  uint32_t thr;          // keep when byte < thr (DROP == 2)
+  const uint8_t* mask;   // explicit keep-mask [B, H, max_q, max_k] (bit kernel, mode 1)
+  uint8_t* mask_out;     // where the drawn mask is written as bytes, or null (bit kernel, mode 2)
+  uint32_t thr;          // keep when byte < thr (bit kernel, mode 2)
   float drop_scale;
   uint64_t seed, offset;
+  // keep bits [B H, q32 groups of 32 queries, kp keys]: bit (i % 32) of word bit_slot(j) of row (b H + h, i / 32)
+  uint32_t* bits;
+  int q32, kp;           // 4 ceil(max_q / 128) and 64 ceil(max_k / 64)
 };
+
+// Inside each group of eight keys the words are stored in the order 0, 4, 1, 5, 2, 6, 3, 7: the two keys that one
+// accumulator register holds in the two halves of a wavefront (j and j + 4) lie side by side as one 64-bit lane mask.
+__device__ __forceinline__ int bit_slot(int key) { return (key & ~7) | ((key & 3) << 1) | ((key >> 2) & 1); }
 
 typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
@@ -160,81 +171,69 @@ __device__ __forceinline__ void load_resident(uint4 (&f)[D / 16], const T* base,
   for (int s = 0; s < D / 16; ++s) f[s] = row < len ? *reinterpret_cast<const uint4*>(p + 16 * s) : make_uint4(0, 0, 0, 0);
 }
 
-template <int CTRL>
-__device__ __forceinline__ uint32_t quad_dpp(uint32_t v) {
-  return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), CTRL, 0xf, 0xf, true));
-}
-
-// The random bytes of this lane's 32 elements of a 64-row tile of the streamed kind: bytes[n][g] holds, in byte e, the byte
-// of element (registers 4 g + e of accumulator n). `fixed` is the lane's own index (query in the query-major kernels, key
-// in the key-major one); consecutive lanes hold consecutive indices, so the four lanes of a quad share each 4 x 4 patch:
-// every lane runs the generator for two of the quad's eight patches (g = its position in the quad, n = 0, 1) and the
-// words travel inside the quad: transposed when a lane needs its own row of every patch (query-major: word i % 4),
-// broadcast when it needs its own column (key-major: byte j % 4 of every word). An integer multiply runs at a quarter of
-// the VALU rate, which makes the ten rounds the expensive part of the softmax: hence one call per 16 elements.
-template <bool QUERY_MAJOR>
-__device__ __forceinline__ void tile_random_bytes(const FaArgs& a, const Philox& gen, int bh, int fixed, int tile, int half,
-                                                  int lane, uint32_t (&bytes)[2][4]) {
-  const int c = lane & 3;
+// Keep bits from the generator: one thread per (head of a sequence, group of 32 queries, group of four keys) runs the
+// eight generator calls of its 32 x 4 elements (one call per 4 x 4 patch) and writes the four keys' words.
+__global__ __launch_bounds__(256) void flash_bits_rng_kernel(FaArgs a, int64_t total) {
+  const int64_t id = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (id >= total) return;
+  const int k4n = a.kp / 4;
+  const int j4 = static_cast<int>(id % k4n);
+  const int64_t row = id / k4n;                      // (b H + h) q32 + group
+  const int grp = static_cast<int>(row % a.q32);
+  const int bh = static_cast<int>(row / a.q32), b = bh / a.heads;
+  const int lq = min(a.cu_q[b + 1] - a.cu_q[b], a.max_q), lk = min(a.cu_k[b + 1] - a.cu_k[b], a.max_k);
+  if (32 * grp >= lq || 4 * j4 >= lk) return;        // never read: every element there is masked or not stored
+  const Philox gen(a.seed);
   const uint64_t q4 = static_cast<uint64_t>((a.max_q + 3) / 4), k4 = static_cast<uint64_t>((a.max_k + 3) / 4);
+  uint32_t word[4] = {0, 0, 0, 0};
 #pragma unroll
-  for (int n = 0; n < 2; ++n) {
-    const uint64_t streamed = static_cast<uint64_t>(16 * tile + 8 * n + 2 * c + half);     // group of four of the streamed kind
-    const uint64_t own = static_cast<uint64_t>(fixed / 4);
-    const uint64_t block = QUERY_MAJOR ? (static_cast<uint64_t>(bh) * q4 + own) * k4 + streamed
-                                       : (static_cast<uint64_t>(bh) * q4 + streamed) * k4 + own;
-    const uint4 r = gen(block, a.offset);
-    uint32_t w[4] = {r.x, r.y, r.z, r.w};
-    if constexpr (QUERY_MAJOR) {
-      // 4 x 4 transpose across the quad: afterwards w[g] is word (lane & 3) of the patch that lane g of the quad drew
-      const bool odd = (c & 1) != 0, up = (c & 2) != 0;
-      uint32_t s0 = odd ? w[0] : w[1], s1 = odd ? w[2] : w[3];
-      s0 = quad_dpp<0xB1>(s0);
-      s1 = quad_dpp<0xB1>(s1);
-      if (odd) { w[0] = s0; w[2] = s1; } else { w[1] = s0; w[3] = s1; }
-      s0 = up ? w[0] : w[2];
-      s1 = up ? w[1] : w[3];
-      s0 = quad_dpp<0x4E>(s0);
-      s1 = quad_dpp<0x4E>(s1);
-      if (up) { w[0] = s0; w[1] = s1; } else { w[2] = s0; w[3] = s1; }
+  for (int u = 0; u < 8; ++u) {
+    const uint4 r = gen((static_cast<uint64_t>(bh) * q4 + static_cast<uint64_t>(8 * grp + u)) * k4 + static_cast<uint64_t>(j4), a.offset);
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
 #pragma unroll
-      for (int g = 0; g < 4; ++g) bytes[n][g] = w[g];
-    } else {
-      const int sh = 8 * (fixed & 3);
-      uint32_t all[4][4];
+    for (int qi = 0; qi < 4; ++qi)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        all[0][e] = quad_dpp<0x00>(w[e]);
-        all[1][e] = quad_dpp<0x55>(w[e]);
-        all[2][e] = quad_dpp<0xAA>(w[e]);
-        all[3][e] = quad_dpp<0xFF>(w[e]);
-      }
+      for (int kj = 0; kj < 4; ++kj)
+        word[kj] |= (((w[qi] >> (8 * kj)) & 0xffu) < a.thr ? 1u : 0u) << (4 * u + qi);
+  }
+  uint32_t* out = a.bits + row * a.kp;
 #pragma unroll
-      for (int g = 0; g < 4; ++g)
-        bytes[n][g] = ((all[g][0] >> sh) & 0xffu) | (((all[g][1] >> sh) & 0xffu) << 8) | (((all[g][2] >> sh) & 0xffu) << 16) |
-                      (((all[g][3] >> sh) & 0xffu) << 24);
+  for (int kj = 0; kj < 4; ++kj) out[bit_slot(4 * j4 + kj)] = word[kj];
+  if (a.mask_out != nullptr) {
+#pragma unroll
+    for (int kj = 0; kj < 4; ++kj) {
+      const int key = 4 * j4 + kj;
+      if (key < lk)
+        for (int i = 0; i < 32; ++i) {
+          const int qi = 32 * grp + i;
+          if (qi < lq) a.mask_out[(static_cast<int64_t>(bh) * a.max_q + qi) * a.max_k + key] = (word[kj] >> i) & 1u;
+        }
     }
   }
 }
 
-// Keep-flags of the four elements of accumulator group g (registers 4 g .. 4 g + 3): `fixed` is the lane's own index and
-// `first` the first of the four consecutive indices of the other kind; `bytes` is that group's word of tile_random_bytes.
-template <int DROP, bool QUERY_MAJOR>
-__device__ __forceinline__ void keep_flags(const FaArgs& a, uint32_t bytes, int bh, int fixed, int first, int lq, int lk,
-                                           bool (&keep)[4]) {
-  if constexpr (DROP == 0) {
-#pragma unroll
-    for (int e = 0; e < 4; ++e) keep[e] = true;
-  } else if constexpr (DROP == 1) {
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int qi = QUERY_MAJOR ? fixed : first + e, kj = QUERY_MAJOR ? first + e : fixed;
-      keep[e] = qi < lq && kj < lk && a.mask[(static_cast<int64_t>(bh) * a.max_q + qi) * a.max_k + kj] != 0;
-    }
-  } else {
-#pragma unroll
-    for (int e = 0; e < 4; ++e) keep[e] = ((bytes >> (8 * e)) & 0xffu) < a.thr;
+// Keep bits from an explicit byte mask [B, H, max_q, max_k]: one thread per (head of a sequence, group of 32 queries, key).
+__global__ __launch_bounds__(256) void flash_bits_mask_kernel(FaArgs a, int64_t total) {
+  const int64_t id = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (id >= total) return;
+  const int key = static_cast<int>(id % a.kp);
+  const int64_t row = id / a.kp;
+  const int grp = static_cast<int>(row % a.q32);
+  const int bh = static_cast<int>(row / a.q32), b = bh / a.heads;
+  const int lq = min(a.cu_q[b + 1] - a.cu_q[b], a.max_q), lk = min(a.cu_k[b + 1] - a.cu_k[b], a.max_k);
+  if (32 * grp >= lq || key >= lk) return;
+  uint32_t word = 0;
+  for (int i = 0; i < 32; ++i) {
+    const int qi = 32 * grp + i;
+    if (qi < lq && a.mask[(static_cast<int64_t>(bh) * a.max_q + qi) * a.max_k + key] != 0) word |= 1u << i;
   }
+  a.bits[row * a.kp + bit_slot(key)] = word;
+}
+
+// The 32 lane masks of one 64-key tile for the wavefront's group of 32 queries: mask e belongs to accumulator register
+// e % 16 of accumulator e / 16 (keys 32 (e / 16) + 8 ((e % 16) / 4) + e % 4 in lanes 0..31 and that + 4 in lanes 32..63).
+__device__ __forceinline__ const uint64_t* tile_lane_masks(const FaArgs& a, int bh, int group, int tile) {
+  return reinterpret_cast<const uint64_t*>(a.bits + (static_cast<int64_t>(bh) * a.q32 + group) * a.kp + FA_TILE * tile);
 }
 
 // Writes the wavefront's 32 rows x D accumulators (acc[i][r]: column 32 i + 8 (r / 4) + 4 half + r % 4 of row lane & 31)
@@ -286,7 +285,7 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
 
   const int nkeys = a.causal ? min(lk, q0 + FA_ROWS) : lk;
   const int ntiles = (nkeys + FA_TILE - 1) / FA_TILE;
-  const Philox gen(a.seed);
+  const int group = static_cast<int>(blockIdx.x) * (FA_ROWS / 32) + __builtin_amdgcn_readfirstlane(wave);   // of 32 queries
 
   acc16_t o[D / 32];
 #pragma unroll
@@ -372,29 +371,12 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
       }
     l += lsum;
     if constexpr (DROP != 0) {
-      uint32_t rnd[2][4] = {};
-      if constexpr (DROP == 2) tile_random_bytes<true>(a, gen, bh, qrow, t, half, lane, rnd);
+      const uint64_t* lane_mask = tile_lane_masks(a, bh, group, t);
 #pragma unroll
       for (int n = 0; n < 2; ++n)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          bool keep[4];
-          keep_flags<DROP, true>(a, rnd[n][g], bh, qrow, t * FA_TILE + 32 * n + 8 * g + 4 * half, lq, lk, keep);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) s[n][4 * g + e] = keep[e] ? s[n][4 * g + e] : 0.f;      // the scale waits for the end
-        }
-      if constexpr (DROP == 2) {
-        if (a.mask_out != nullptr && qrow < lq) {
-          uint8_t* row = a.mask_out + (static_cast<int64_t>(bh) * a.max_q + qrow) * a.max_k;
-#pragma unroll
-          for (int n = 0; n < 2; ++n)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const int key = t * FA_TILE + 32 * n + 8 * (r / 4) + 4 * half + r % 4;
-              if (key < lk) row[key] = ((rnd[n][r / 4] >> (8 * (r % 4))) & 0xffu) < a.thr;
-            }
-        }
-      }
+        for (int r = 0; r < 16; ++r)
+          s[n][r] = __builtin_amdgcn_inverse_ballot_w64(lane_mask[16 * n + r]) ? s[n][r] : 0.f;   // the scale waits for the end
     }
 #pragma unroll
     for (int kk = 0; kk < FA_TILE / 16; ++kk) {
@@ -464,7 +446,7 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dq_kern
 
   const int nkeys = a.causal ? min(lk, q0 + FA_ROWS) : lk;
   const int ntiles = (nkeys + FA_TILE - 1) / FA_TILE;
-  const Philox gen(a.seed);
+  const int group = static_cast<int>(blockIdx.x) * (FA_ROWS / 32) + __builtin_amdgcn_readfirstlane(wave);   // of 32 queries
   const float dead_raw = FA_NEG / a.scale_log2;   // the raw score that the scale turns into -1e30
   acc16_t dq[D / 32];
 #pragma unroll
@@ -512,22 +494,15 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dq_kern
           if (key >= lk || (a.causal && key > qrow)) s[n][r] = dead_raw;
         }
     }
-    uint32_t rnd[2][4] = {};
-    if constexpr (DROP == 2) tile_random_bytes<true>(a, gen, bh, qrow, t, half, lane, rnd);
+    [[maybe_unused]] const uint64_t* lane_mask = DROP != 0 ? tile_lane_masks(a, bh, group, t) : nullptr;
 #pragma unroll
     for (int n = 0; n < 2; ++n)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int key0 = t * FA_TILE + 32 * n + 8 * g + 4 * half;
-        bool keep[4];
-        keep_flags<DROP, true>(a, rnd[n][g], bh, qrow, key0, lq, lk, keep);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int r = 4 * g + e;
-          const float pr = fast_exp2(__builtin_fmaf(s[n][r], a.scale_log2, -lse2));
-          const float kscale = DROP != 0 ? (keep[e] ? a.drop_scale : 0.f) : 1.f;
-          s[n][r] = pr * __builtin_fmaf(dp[n][r], kscale, -delta);     // dS
-        }
+      for (int r = 0; r < 16; ++r) {
+        const float pr = fast_exp2(__builtin_fmaf(s[n][r], a.scale_log2, -lse2));
+        float kscale = 1.f;
+        if constexpr (DROP != 0) kscale = __builtin_amdgcn_inverse_ballot_w64(lane_mask[16 * n + r]) ? a.drop_scale : 0.f;
+        s[n][r] = pr * __builtin_fmaf(dp[n][r], kscale, -delta);     // dS
       }
 #pragma unroll
     for (int kk = 0; kk < FA_TILE / 16; ++kk) {
@@ -575,7 +550,6 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dkv_ker
   // causal: queries before the block's first key see none of its keys
   const int t0 = a.causal ? k0 / FA_TILE : 0;
   const int ntiles = (lq + FA_TILE - 1) / FA_TILE;
-  const Philox gen(a.seed);
   const float dead_raw = FA_NEG / a.scale_log2;   // the raw score that the scale turns into -1e30
   acc16_t dk[D / 32], dv[D / 32];
 #pragma unroll
@@ -648,8 +622,15 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dkv_ker
           if (krow >= lk || (a.causal && krow > qi)) s[n][r] = dead_raw;
         }
     }
-    uint32_t rnd[2][4] = {};
-    if constexpr (DROP == 2) tile_random_bytes<false>(a, gen, bh, krow, t, half, lane, rnd);
+    // keep bits of this lane's key for the tile's two groups of 32 queries, shifted so that bit 8 g + c is register 4 g + c
+    uint32_t kbits[2] = {0, 0};
+    if constexpr (DROP != 0) {
+      if (krow < lk) {
+        const uint32_t* w = a.bits + (static_cast<int64_t>(bh) * a.q32 + 2 * t) * a.kp + bit_slot(krow);
+        kbits[0] = w[0] >> (4 * half);
+        kbits[1] = w[a.kp] >> (4 * half);
+      }
+    }
 #pragma unroll
     for (int n = 0; n < 2; ++n)
 #pragma unroll
@@ -658,15 +639,14 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dkv_ker
         const float4 l4 = *reinterpret_cast<const float4*>(stats + ql);
         const float4 d4 = *reinterpret_cast<const float4*>(stats + FA_TILE + ql);
         const float lse2[4] = {l4.x, l4.y, l4.z, l4.w}, dl[4] = {d4.x, d4.y, d4.z, d4.w};
-        bool keep[4];
-        keep_flags<DROP, false>(a, rnd[n][g], bh, krow, t * FA_TILE + ql, lq, lk, keep);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int r = 4 * g + e;
           const float pr = fast_exp2(__builtin_fmaf(s[n][r], a.scale_log2, -lse2[e]));
-          const float kscale = DROP != 0 ? (keep[e] ? a.drop_scale : 0.f) : 1.f;
+          const bool keep = DROP == 0 || ((kbits[n] >> (8 * g + e)) & 1u) != 0;
+          const float kscale = DROP != 0 ? (keep ? a.drop_scale : 0.f) : 1.f;
           s[n][r] = pr * __builtin_fmaf(dp[n][r], kscale, -dl[e]);   // dS
-          dp[n][r] = DROP != 0 ? (keep[e] ? pr : 0.f) : pr;          // kept probabilities; their scale waits for the end
+          dp[n][r] = keep ? pr : 0.f;                                // kept probabilities; their scale waits for the end
         }
       }
 #pragma unroll
@@ -710,23 +690,41 @@ template <typename T, int D>
 int fwd_launch(const FaArgs& a, int drop, dim3 grid, hipStream_t st) {
   TraceScope trace("flash_attn_fwd", st);
   if (drop == 0) return launch(flash_fwd_kernel<T, D, 0>, "flash_attn_fwd", grid, fwd_lds<D>(), st, a);
-  if (drop == 1) return launch(flash_fwd_kernel<T, D, 1>, "flash_attn_fwd", grid, fwd_lds<D>(), st, a);
-  return launch(flash_fwd_kernel<T, D, 2>, "flash_attn_fwd", grid, fwd_lds<D>(), st, a);
+  return launch(flash_fwd_kernel<T, D, 1>, "flash_attn_fwd", grid, fwd_lds<D>(), st, a);
 }
 template <typename T, int D>
 int bwd_launch(const FaArgs& a, int drop, dim3 grid_q, dim3 grid_k, hipStream_t st) {
   int rc = 0;
   if (grid_q.x > 0) {
     TraceScope trace("flash_attn_bwd_dq", st);
-    rc = drop == 0   ? launch(flash_bwd_dq_kernel<T, D, 0>, "flash_attn_bwd", grid_q, dq_lds<D>(), st, a)
-         : drop == 1 ? launch(flash_bwd_dq_kernel<T, D, 1>, "flash_attn_bwd", grid_q, dq_lds<D>(), st, a)
-                     : launch(flash_bwd_dq_kernel<T, D, 2>, "flash_attn_bwd", grid_q, dq_lds<D>(), st, a);
+    rc = drop == 0 ? launch(flash_bwd_dq_kernel<T, D, 0>, "flash_attn_bwd", grid_q, dq_lds<D>(), st, a)
+                   : launch(flash_bwd_dq_kernel<T, D, 1>, "flash_attn_bwd", grid_q, dq_lds<D>(), st, a);
   }
   if (rc || grid_k.x == 0) return rc;
   TraceScope trace("flash_attn_bwd_dkv", st);
-  return drop == 0   ? launch(flash_bwd_dkv_kernel<T, D, 0>, "flash_attn_bwd", grid_k, dkv_lds<D>(), st, a)
-         : drop == 1 ? launch(flash_bwd_dkv_kernel<T, D, 1>, "flash_attn_bwd", grid_k, dkv_lds<D>(), st, a)
-                     : launch(flash_bwd_dkv_kernel<T, D, 2>, "flash_attn_bwd", grid_k, dkv_lds<D>(), st, a);
+  return drop == 0 ? launch(flash_bwd_dkv_kernel<T, D, 0>, "flash_attn_bwd", grid_k, dkv_lds<D>(), st, a)
+                   : launch(flash_bwd_dkv_kernel<T, D, 1>, "flash_attn_bwd", grid_k, dkv_lds<D>(), st, a);
+}
+
+int64_t bits_q32(int64_t max_q) { return 4 * ((max_q + FA_ROWS - 1) / FA_ROWS); }
+int64_t bits_kp(int64_t max_k) { return FA_TILE * ((max_k + FA_TILE - 1) / FA_TILE); }
+
+// The keep bits of a call with dropout: drawn from the generator (mode 2) or taken from the byte mask (mode 1).
+int bits_launch(const char* what, FaArgs& a, int drop_mode, int64_t batch, void* bits, bool ready, hipStream_t st) {
+  if (drop_mode == 0) return 0;
+  NMTG_REQUIRE(bits != nullptr && aligned16(bits), "%s: dropout needs the 16-byte aligned keep-bit workspace (nmtg_flash_attn_dropout_bits_bytes)", what);
+  a.bits = static_cast<uint32_t*>(bits);
+  a.q32 = static_cast<int>(bits_q32(a.max_q));
+  a.kp = static_cast<int>(bits_kp(a.max_k));
+  if (ready || a.max_q == 0 || a.max_k == 0) return 0;
+  const int64_t rows = batch * a.heads * a.q32;
+  const int64_t total = rows * (drop_mode == 2 ? a.kp / 4 : a.kp);
+  NMTG_REQUIRE((total + 255) / 256 <= 0x7fffffff, "%s: keep-bit workspace beyond one launch", what);
+  TraceScope trace("flash_attn_keep_bits", st);
+  const dim3 grid(static_cast<unsigned>((total + 255) / 256));
+  if (drop_mode == 2) hipLaunchKernelGGL(flash_bits_rng_kernel, grid, dim3(256), 0, st, a, total);
+  else hipLaunchKernelGGL(flash_bits_mask_kernel, grid, dim3(256), 0, st, a, total);
+  return 0;
 }
 
 bool view_ok(const void* p, int64_t st, int64_t sh, int64_t heads, int64_t d) {
@@ -767,13 +765,19 @@ void set_dropout(FaArgs& a, int drop_mode, float p, uint64_t seed, uint64_t offs
 
 using namespace nmtg;
 
+extern "C" int64_t nmtg_flash_attn_dropout_bits_bytes(int64_t batch, int64_t heads, int64_t max_seqlen_q, int64_t max_seqlen_k) {
+  if (batch <= 0 || heads <= 0 || max_seqlen_q <= 0 || max_seqlen_k <= 0) return 0;
+  return batch * heads * bits_q32(max_seqlen_q) * bits_kp(max_seqlen_k) * 4;
+}
+
 extern "C" int nmtg_flash_attn_fwd(const void* q, const void* k, const void* v, void* out, const int32_t* cu_seqlens_q,
                                    const int32_t* cu_seqlens_k, float* softmax_lse, int64_t batch, int64_t heads,
                                    int64_t head_dim, int64_t max_seqlen_q, int64_t max_seqlen_k, int64_t q_stride_t,
                                    int64_t q_stride_h, int64_t k_stride_t, int64_t k_stride_h, int64_t v_stride_t,
                                    int64_t v_stride_h, int64_t out_stride_t, int64_t out_stride_h, float softmax_scale,
                                    int causal, int dropout_mode, float dropout_p, const uint8_t* dropout_mask,
-                                   uint8_t* dropout_mask_out, uint64_t seed, uint64_t offset, int dtype, void* stream) {
+                                   uint8_t* dropout_mask_out, void* dropout_bits, uint64_t seed, uint64_t offset, int dtype,
+                                   void* stream) {
   if (int rc = check_common("flash_attn_fwd", batch, heads, head_dim, max_seqlen_q, max_seqlen_k, dropout_mode, dropout_p, softmax_scale, dtype)) return rc;
   if (batch == 0 || max_seqlen_q == 0) return 0;
   NMTG_REQUIRE(q && k && v && out && cu_seqlens_q && cu_seqlens_k && softmax_lse, "flash_attn_fwd: null pointer argument");
@@ -792,7 +796,8 @@ extern "C" int nmtg_flash_attn_fwd(const void* q, const void* k, const void* v, 
   set_dropout(a, dropout_mode, dropout_p, seed, offset);
   const dim3 grid(static_cast<unsigned>((max_seqlen_q + FA_ROWS - 1) / FA_ROWS), static_cast<unsigned>(heads), static_cast<unsigned>(batch));
   hipStream_t st = static_cast<hipStream_t>(stream);
-  int rc;
+  int rc = bits_launch("flash_attn_fwd", a, dropout_mode, batch, dropout_bits, false, st);
+  if (rc) return rc;
   if (dtype == NMTG_F16) rc = head_dim == 64 ? fwd_launch<f16_t, 64>(a, dropout_mode, grid, st) : fwd_launch<f16_t, 128>(a, dropout_mode, grid, st);
   else rc = head_dim == 64 ? fwd_launch<bf16_t, 64>(a, dropout_mode, grid, st) : fwd_launch<bf16_t, 128>(a, dropout_mode, grid, st);
   if (rc) return rc;
@@ -809,12 +814,14 @@ extern "C" int nmtg_flash_attn_bwd(const void* dout, const void* q, const void* 
                                    int64_t out_stride_h, int64_t dq_stride_t, int64_t dq_stride_h, int64_t dk_stride_t,
                                    int64_t dk_stride_h, int64_t dv_stride_t, int64_t dv_stride_h, float softmax_scale,
                                    int causal, int dropout_mode, float dropout_p, const uint8_t* dropout_mask,
-                                   uint64_t seed, uint64_t offset, int dtype, void* stream) {
+                                   void* dropout_bits, int dropout_bits_ready, uint64_t seed, uint64_t offset, int dtype,
+                                   void* stream) {
   if (int rc = check_common("flash_attn_bwd", batch, heads, head_dim, max_seqlen_q, max_seqlen_k, dropout_mode, dropout_p, softmax_scale, dtype)) return rc;
   if (batch == 0) return 0;
   NMTG_REQUIRE(dout && q && k && v && out && softmax_lse && dq && dk && dv && softmax_d && cu_seqlens_q && cu_seqlens_k,
                "flash_attn_bwd: null pointer argument");
-  NMTG_REQUIRE(dropout_mode != 1 || dropout_mask, "flash_attn_bwd: dropout mode 1 replays a keep-mask and none was given");
+  NMTG_REQUIRE(dropout_mode != 1 || dropout_mask || dropout_bits_ready,
+               "flash_attn_bwd: dropout mode 1 replays a keep-mask and none was given");
   NMTG_REQUIRE(view_ok(q, q_stride_t, q_stride_h, heads, head_dim) && view_ok(k, k_stride_t, k_stride_h, heads, head_dim) &&
                    view_ok(v, v_stride_t, v_stride_h, heads, head_dim) && view_ok(out, out_stride_t, out_stride_h, heads, head_dim) &&
                    view_ok(dout, dout_stride_t, dout_stride_h, heads, head_dim) && view_ok(dq, dq_stride_t, dq_stride_h, heads, head_dim) &&
@@ -834,7 +841,8 @@ extern "C" int nmtg_flash_attn_bwd(const void* dout, const void* q, const void* 
   const dim3 grid_q(static_cast<unsigned>((max_seqlen_q + FA_ROWS - 1) / FA_ROWS), static_cast<unsigned>(heads), static_cast<unsigned>(batch));
   const dim3 grid_k(static_cast<unsigned>((max_seqlen_k + FA_ROWS - 1) / FA_ROWS), static_cast<unsigned>(heads), static_cast<unsigned>(batch));
   hipStream_t st = static_cast<hipStream_t>(stream);
-  int rc;
+  int rc = bits_launch("flash_attn_bwd", a, dropout_mode, batch, dropout_bits, dropout_bits_ready != 0, st);
+  if (rc) return rc;
   if (dtype == NMTG_F16) rc = head_dim == 64 ? bwd_launch<f16_t, 64>(a, dropout_mode, grid_q, grid_k, st) : bwd_launch<f16_t, 128>(a, dropout_mode, grid_q, grid_k, st);
   else rc = head_dim == 64 ? bwd_launch<bf16_t, 64>(a, dropout_mode, grid_q, grid_k, st) : bwd_launch<bf16_t, 128>(a, dropout_mode, grid_q, grid_k, st);
   if (rc) return rc;

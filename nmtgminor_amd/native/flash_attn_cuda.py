@@ -15,6 +15,9 @@ Differences from the CUDA module, all on the dropout side:
    nmtgminor_amd/modules/flash_mha.py carry it from forward to backward) or, without it, replays `last_rng`; restoring
    the generator state before bwd, as the reference does, is harmless and not needed;
  * keyword `rng=(seed, offset)` on fwd fixes the Philox state instead of drawing one from the generator;
+ * the kernels read the keep decisions as one bit per element from a workspace that a small kernel fills ahead of them;
+   fwd allocates it and hands it on inside `last_rng` (a fifth entry), and a bwd that receives it runs no generator;
+   a four-entry state makes bwd fill a workspace of its own from (seed, offset) or the mask;
  * return_softmax hands back the keep-mask (uint8 [B, H, max_seqlen_q, max_seqlen_k]) instead of the sign-encoded
    probability matrix, which exists nowhere in this kernel; keyword `dropout_mask` replays such a mask (tests);
  * num_splits is accepted and ignored: the kernels never accumulate across blocks, so results do not depend on it."""
@@ -60,6 +63,11 @@ def _draw(device, count, generator):
     return seed, offset
 
 
+def _bits(batch, heads, max_q, max_k, device):
+    n = L.load().nmtg_flash_attn_dropout_bits_bytes(L.i64(batch), L.i64(heads), L.i64(max_q), L.i64(max_k))
+    return torch.empty(max(int(n), 16) // 4, dtype=torch.int32, device=device)
+
+
 def fwd(q, k, v, out, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale, zero_tensors,
         causal, return_softmax, num_splits=0, generator=None, *, dropout_mask=None, rng=None):
     global last_rng
@@ -70,8 +78,9 @@ def fwd(q, k, v, out, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dr
     if zero_tensors:
         out.zero_()
     lse = torch.zeros(batch, heads, max_seqlen_q, dtype=torch.float32, device=q.device)
-    mode, seed, offset, mask_out = 0, 0, 0, None
+    mode, seed, offset, mask_out, bits = 0, 0, 0, None, None
     if dropout_p > 0.0:
+        bits = _bits(batch, heads, max_seqlen_q, max_seqlen_k, q.device)
         if dropout_mask is not None:
             _check(dropout_mask.dtype == torch.uint8 and tuple(dropout_mask.shape) == (batch, heads, max_seqlen_q, max_seqlen_k)
                    and dropout_mask.is_contiguous(), "flash_attn: dropout_mask must be contiguous uint8 [B, H, max_q, max_k]")
@@ -85,12 +94,12 @@ def fwd(q, k, v, out, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dr
             seed, offset = rng if rng is not None else _draw(q.device, 4 * blocks, generator)
             if return_softmax:
                 mask_out = torch.zeros(batch, heads, max_seqlen_q, max_seqlen_k, dtype=torch.uint8, device=q.device)
-    last_rng = (mode, seed, offset, dropout_mask)
+    last_rng = (mode, seed, offset, dropout_mask, bits)
     L.call("nmtg_flash_attn_fwd", L.ptr(q), L.ptr(k), L.ptr(v), L.ptr(out), L.ptr(cu_seqlens_q), L.ptr(cu_seqlens_k),
            L.ptr(lse), L.i64(batch), L.i64(heads), L.i64(d), L.i64(max_seqlen_q), L.i64(max_seqlen_k),
            *_view(q, "q"), *_view(k, "k", heads, d), *_view(v, "v", heads, d), *_view(out, "out", heads, d),
            L.f32(softmax_scale), L.i32(int(bool(causal))), L.i32(mode), L.f32(dropout_p), L.ptr(dropout_mask if mode == 1 else None),
-           L.ptr(mask_out), ctypes.c_uint64(seed), ctypes.c_uint64(offset), L.i32(L.dtype_code(q)), L.stream_of(q))
+           L.ptr(mask_out), L.ptr(bits), ctypes.c_uint64(seed), ctypes.c_uint64(offset), L.i32(L.dtype_code(q)), L.stream_of(q))
     if return_softmax:
         return [lse, dropout_mask if mode == 1 else mask_out]
     return [lse]
@@ -107,17 +116,22 @@ def bwd(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k,
            softmax_lse.is_contiguous(), "flash_attn: softmax_lse must be contiguous fp32 [B, H, max_seqlen_q]")
     if zero_tensors:
         dq.zero_(), dk.zero_(), dv.zero_()
-    mode, seed, offset, mask = 0, 0, 0, None
+    mode, seed, offset, mask, bits, ready = 0, 0, 0, None, None, 0
     if dropout_p > 0.0:
         state = rng if rng is not None else last_rng
         _check(state is not None and state[0] != 0, "flash_attn: backward with dropout needs the forward's generator state")
-        mode, seed, offset, mask = state
+        mode, seed, offset, mask = state[:4]
+        bits = state[4] if len(state) > 4 else None
+        ready = int(bits is not None)
+        if bits is None:
+            bits = _bits(batch, heads, max_seqlen_q, max_seqlen_k, q.device)
+        L.require_cuda(bits)
     softmax_d = torch.zeros(batch, heads, max_seqlen_q, dtype=torch.float32, device=q.device)
     L.call("nmtg_flash_attn_bwd", L.ptr(dout), L.ptr(q), L.ptr(k), L.ptr(v), L.ptr(out), L.ptr(softmax_lse), L.ptr(dq),
            L.ptr(dk), L.ptr(dv), L.ptr(softmax_d), L.ptr(cu_seqlens_q), L.ptr(cu_seqlens_k), L.i64(batch), L.i64(heads),
            L.i64(d), L.i64(max_seqlen_q), L.i64(max_seqlen_k), *_view(dout, "dout", heads, d), *_view(q, "q"),
            *_view(k, "k", heads, d), *_view(v, "v", heads, d), *_view(out, "out", heads, d), *_view(dq, "dq", heads, d),
            *_view(dk, "dk", heads, d), *_view(dv, "dv", heads, d), L.f32(softmax_scale), L.i32(int(bool(causal))),
-           L.i32(mode), L.f32(dropout_p), L.ptr(mask if mode == 1 else None), ctypes.c_uint64(seed), ctypes.c_uint64(offset),
-           L.i32(L.dtype_code(q)), L.stream_of(q))
+           L.i32(mode), L.f32(dropout_p), L.ptr(mask if mode == 1 else None), L.ptr(bits), L.i32(ready), ctypes.c_uint64(seed),
+           ctypes.c_uint64(offset), L.i32(L.dtype_code(q)), L.stream_of(q))
     return dq, dk, dv, softmax_d

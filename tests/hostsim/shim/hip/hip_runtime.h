@@ -126,6 +126,9 @@ static inline void hostsim_no_resolver(void**, int) {}
 static inline void __builtin_amdgcn_wave_barrier() { hostsim::wave_collective(hostsim_no_resolver, nullptr); }
 #define __builtin_amdgcn_fence(order, scope) ((void)0)
 
+// a wavefront-uniform 64-bit mask as a per-lane predicate (the operand form of v_cndmask)
+static inline bool __builtin_amdgcn_inverse_ballot_w64(uint64_t mask) { return ((mask >> hostsim::lane_id()) & 1u) != 0; }
+
 // v_cmp into a wavefront-wide mask: bit l is lane l's predicate
 static inline uint64_t __builtin_amdgcn_ballot_w64(bool pred) {
   uint64_t mask = 0;
