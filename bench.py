@@ -86,7 +86,7 @@ class LayerNormWL(Workload):
     description = "LayerNorm fwd+bwd fp32 [4096 x 512], eps 1e-5"
 
     def setup(self, dev):
-        from oracle import inputs
+        from nmtgminor_amd import synthetic as inputs
         from nmtgminor_amd.native import fast_layer_norm_cuda as ln
         self.ln = ln
         self.cpu = inputs.layer_norm_inputs()
@@ -132,7 +132,7 @@ class LayerNormLargeWL(LayerNormWL):
     description = "LayerNorm fwd+bwd bf16 [65536 x 1024], eps 1e-5 (134 MB per tensor: beyond the last-level cache)"
 
     def setup(self, dev):
-        from oracle import inputs
+        from nmtgminor_amd import synthetic as inputs
         from nmtgminor_amd.native import fast_layer_norm_cuda as ln
         self.ln = ln
         self.cpu = inputs.layer_norm_inputs(65536, 1024, torch.bfloat16, seed=1011)
@@ -166,7 +166,7 @@ class MlpWL(Workload):
     description = "fused MLP fwd+bwd fp16: x [8192 x 512], 512->2048->512, gelu, dropout 0.1 (explicit mask)"
 
     def setup(self, dev):
-        from oracle import inputs
+        from nmtgminor_amd import synthetic as inputs
         from nmtgminor_amd.native import fused_mlp_gelu as m
         self.m = m
         self.cpu = inputs.mlp_inputs()
@@ -210,7 +210,7 @@ class XentropyWL(Workload):
     rows, vocab = 16384, 250054
 
     def setup(self, dev):
-        from oracle import inputs
+        from nmtgminor_amd import synthetic as inputs
         from nmtgminor_amd.native import xentropy_cuda as xe
         self.xe = xe
         d = inputs.xentropy_inputs(self.rows, self.vocab, with_logits=False)
@@ -263,7 +263,7 @@ class SelfAttnWL(Workload):
     T, B, E, H = 512, 32, 1024, 16
 
     def setup(self, dev):
-        from oracle import inputs
+        from nmtgminor_amd import synthetic as inputs
         from nmtgminor_amd.native import self_multihead_attn_blaslt as m
         self.m = m
         d = inputs.self_attn_inputs(self.T, self.B, self.E, self.H)
@@ -371,7 +371,7 @@ class RelSelfAttnWL(Workload):
     NAMES = ("x", "pos", "w_in", "w_out", "w_pos", "b_in", "b_out", "b_pos", "r_w_bias", "r_r_bias")
 
     def setup(self, dev):
-        from oracle import inputs
+        from nmtgminor_amd import synthetic as inputs
         from nmtgminor_amd.modules.relative_self_attention_func import relative_self_attn_func
         self.fn = relative_self_attn_func
         d = inputs.rel_self_attn_inputs(self.T, self.B, self.E, self.H, torch.bfloat16, p=0.1, seed=1006)
@@ -426,7 +426,7 @@ class EncdecAttnWL(Workload):
     TQ, TK, B, E, H = 128, 1500, 16, 1024, 16
 
     def setup(self, dev):
-        from oracle import inputs
+        from nmtgminor_amd import synthetic as inputs
         from nmtgminor_amd.native import encdec_multihead_attn_bias_blaslt as m, self_multihead_attn_blaslt as sm
         self.m, self.sm = m, sm
         d = inputs.encdec_attn_inputs(self.TQ, self.TK, self.B, self.E, self.H)
@@ -477,7 +477,7 @@ class DecodeStepWL(Workload):
     TK, TPREV, B, E, H = 1500, 127, 32, 1024, 16
 
     def setup(self, dev):
-        from oracle import inputs
+        from nmtgminor_amd import synthetic as inputs
         from nmtgminor_amd.modules import incremental as inc
         self.inc = inc
         d = inputs.encdec_attn_inputs(1, self.TK, self.B, self.E, self.H, seed=1010)
@@ -545,7 +545,7 @@ class SoftmaxDropoutWL(Workload):
     HEADS, BATCH, T = 16, 32, 512
 
     def setup(self, dev):
-        from oracle import inputs
+        from nmtgminor_amd import synthetic as inputs
         from nmtgminor_amd.native import mask_softmax_dropout_cuda as sm
         self.sm = sm
         g = torch.Generator().manual_seed(1003)
@@ -599,7 +599,7 @@ class DropoutAddWL(Workload):
     SHAPE = (512, 32, 1024)
 
     def setup(self, dev):
-        from oracle import inputs
+        from nmtgminor_amd import synthetic as inputs
         from nmtgminor_amd.native import fused_dropout_add_cuda as da
         self.da = da
         g = torch.Generator().manual_seed(1006)
@@ -704,7 +704,7 @@ class GeneratorLossWL(Workload):
     ROWS, MODEL, VOCAB, CHUNK = 16384, 1024, 250054, 4096
 
     def setup(self, dev):
-        from oracle import inputs
+        from nmtgminor_amd import synthetic as inputs
         from nmtgminor_amd.modules.generator_loss import LinearSoftmaxCrossEntropy
         self.fn = LinearSoftmaxCrossEntropy
         n, e, v = self.ROWS, self.MODEL, self.VOCAB
