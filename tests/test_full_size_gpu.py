@@ -4,13 +4,16 @@ Where the CPU oracle cannot run the whole workload in seconds, parity is checked
 that are independent (attention: batch columns; cross-entropy: rows) and the rest through
 size-independent properties: probability rows sum to one, exact zeros on masked keys / padded
 rows, gradient rows sum to zero, determinism. (The MLP and LayerNorm workloads run whole against
-the oracle in test_mlp_gpu.py / test_layer_norm_gpu.py.)
+the oracle in test_mlp_gpu.py / test_layer_norm_gpu.py.) The packed-attention and relative-position
+workloads are also held against a second, independent computation of the whole batch: fp32 matrix
+products on the device, and the chain of separate kernels.
 """
 import pytest
 import torch
 
-from nmtgminor_amd.native import encdec_multihead_attn_bias_blaslt as ed, self_multihead_attn_blaslt as sa, xentropy_cuda
-from oracle import attention as oat, inputs, xentropy as oxe
+from nmtgminor_amd.native import (encdec_multihead_attn_bias_blaslt as ed, flash_attn_cuda, relative_self_attn_blaslt as rel,
+                                  self_multihead_attn_blaslt as sa, xentropy_cuda)
+from oracle import attention as oat, flash_attention as ofa, inputs, relative_attention as orel, xentropy as oxe
 from util import assert_close
 
 pytestmark = pytest.mark.gpu
@@ -135,3 +138,108 @@ def test_xentropy_workload(dev):
     assert row_sums[~pad].abs().max() < 5e-2                                       # softmax - target distribution sums to 0
     tgt = grad[torch.arange(N, device=dev)[~pad], labels[~pad]].float()
     assert (tgt < 0).all() and (tgt > -1.0).all()                                  # target logit gradient in (-(1-eps), 0)
+
+
+def test_packed_attention_workload(dev):
+    """The benchmark's packed workload (32 sequences of U[256, 512] tokens, 16 heads of 64, dropout 0.1 drawn on the
+    device): two sequences against the oracle, and every sequence against the same arithmetic written with fp32
+    matrix products on the device (scores, softmax, the drawn mask with its scale, autograd for the gradients), to the
+    tolerances of test_zze_flash_attention_gpu.py (probabilities rounded to bf16 relative to different reference points)."""
+    B, H, Dh, p = 32, 16, 64, 0.1
+    g = torch.Generator().manual_seed(5)
+    lens = torch.randint(256, 513, (B,), generator=g).tolist()
+    cu = torch.zeros(B + 1, dtype=torch.int32)
+    cu[1:] = torch.cumsum(torch.tensor(lens), 0)
+    total, mx = int(cu[-1]), max(lens)
+    qkv = torch.randn(total, 3, H, Dh, generator=g).to(BF)
+    dout = torch.randn(total, H, Dh, generator=g).to(BF)
+    qkv_d, dout_d, cu_d = qkv.to(dev), dout.to(dev), cu.to(dev)
+    q, k, v = qkv_d[:, 0], qkv_d[:, 1], qkv_d[:, 2]
+    scale = Dh ** -0.5
+    torch.cuda.manual_seed(77)
+    out = torch.full_like(dout_d, float("nan"))
+    lse, mask = flash_attn_cuda.fwd(q, k, v, out, cu_d, cu_d, mx, mx, p, scale, False, False, True)
+    state = flash_attn_cuda.last_rng
+    dqkv = torch.full_like(qkv_d, float("nan"))
+    flash_attn_cuda.bwd(dout_d, q, k, v, out, lse, dqkv[:, 0], dqkv[:, 1], dqkv[:, 2], cu_d, cu_d, mx, mx, p, scale, False, False,
+                        rng=state)
+    assert not torch.isnan(out).any() and not torch.isnan(dqkv).any()
+    keep_scale = 256.0 / round(256 * (1 - p))
+    p_eff = 1.0 - 1.0 / keep_scale
+    kept = sum(float(mask[b, :, :n, :n].float().sum()) for b, n in enumerate(lens)) / sum(H * n * n for n in lens)
+    assert abs(kept - 1 / keep_scale) < 1e-3
+    atol, gatol = 8e-3 * 2 / (1 - p), 4e-3 / (1 - p)
+    # (a) the oracle on the first and the last sequence
+    for b in (0, B - 1):
+        sl = slice(int(cu[b]), int(cu[b + 1]))
+        n = lens[b]
+        one = torch.tensor([0, n], dtype=torch.int32)
+        m1 = mask[b:b + 1, :, :n, :n].cpu()
+        want, _ = ofa.flash_attn_fwd(qkv[sl, 0], qkv[sl, 1], qkv[sl, 2], one, one, n, scale, False, p_eff, m1, D, round_to=BF)
+        wdq, wdk, wdv, _ = ofa.flash_attn_bwd(dout[sl], qkv[sl, 0], qkv[sl, 1], qkv[sl, 2], one, one, n, scale, False, p_eff, m1, D,
+                                              round_to=BF)
+        assert_close(out[sl], want, BF, f"out[{b}]", atol=atol)
+        for i, (name, w) in enumerate((("dq", wdq), ("dk", wdk), ("dv", wdv))):
+            assert_close(dqkv[sl, i], w, BF, f"{name}[{b}]", scale_atol=True, atol=gatol)
+    # (b) every sequence against fp32 matrix products on the device
+    for b, n in enumerate(lens):
+        sl = slice(int(cu[b]), int(cu[b + 1]))
+        x = qkv_d[sl].float().requires_grad_()
+        qs, ks, vs = (x[:, i].transpose(0, 1) for i in range(3))                   # [H, n, Dh]
+        prob = torch.softmax(qs @ ks.transpose(1, 2) * scale, dim=-1) * mask[b, :, :n, :n].float() * keep_scale
+        ref = (prob @ vs).transpose(0, 1)
+        ref.backward(dout_d[sl].float())
+        assert_close(out[sl], ref.detach().cpu(), BF, f"out of sequence {b}", atol=atol)
+        assert_close(lse[b, :, :n], torch.logsumexp(qs.detach() @ ks.detach().transpose(1, 2) * scale, -1).cpu(), torch.float32,
+                     f"lse of sequence {b}", rtol=1e-3, atol=2e-3)
+        for i, name in enumerate(("dq", "dk", "dv")):
+            assert_close(dqkv[sl, i], x.grad[:, i].cpu(), BF, f"{name} of sequence {b}", scale_atol=True, atol=gatol)
+    # (c) deterministic, and the backward that refills its own keep bits from the generator state agrees bit for bit
+    again = torch.full_like(qkv_d, float("nan"))
+    flash_attn_cuda.bwd(dout_d, q, k, v, out, lse, again[:, 0], again[:, 1], again[:, 2], cu_d, cu_d, mx, mx, p, scale, False, False,
+                        rng=state[:4])
+    assert torch.equal(again, dqkv)
+
+
+def test_relative_attention_workload(dev, monkeypatch):
+    """The benchmark's relative-position workload (T = 512, B = 32, E = 1024, 16 heads, 512 positions): the kernels that run
+    the shift inside the softmax against the chain of separate kernels on the whole batch (same rounding points, rows
+    added up in another order: four 16-bit units on the probabilities, the usual tolerances behind the products), and
+    two batch columns against the oracle."""
+    T, B, E, H, p = 512, 32, 1024, 16, 0.1
+    names = ("x", "pos", "w_in", "w_out", "w_pos", "b_in", "b_out", "b_pos", "r_w_bias", "r_r_bias")
+    d = inputs.rel_self_attn_inputs(T, B, E, H, BF, p=p, seed=1006)
+    a = {k: d[k].to(dev) for k in names}
+    a["pos"] = a["pos"].repeat(1, B, 1).contiguous()          # one position projection per batch column, as the extension lays it out
+    pad, dm, dout = d["pad_mask"].to(dev), d["dropout_mask"].to(dev), d["dout"].to(dev)
+
+    def run():
+        res = rel.forward(True, False, H, a["x"], a["pos"], a["w_in"], a["w_out"], a["w_pos"], a["b_in"], a["b_out"], a["b_pos"],
+                          a["r_w_bias"], a["r_r_bias"], pad, p, dropout_mask=dm)
+        lin, pos_lin, scores, dropped, dmask, ctx, out = res
+        grads = rel.backward(H, dout, ctx, dropped, scores, lin, pos_lin, a["r_w_bias"], a["r_r_bias"], a["x"], a["pos"], a["w_in"],
+                             a["w_out"], a["w_pos"], dmask, p, pad_mask=pad)
+        return scores, dropped, out, grads
+
+    scores, dropped, out, grads = run()
+    monkeypatch.setenv("NMTG_REL_FUSED", "0")
+    scores0, dropped0, out0, grads0 = run()
+    monkeypatch.delenv("NMTG_REL_FUSED")
+    assert torch.equal(scores, scores0)                                   # the summed scores: same additions, same rounding
+    ulp4 = 4 * torch.finfo(BF).eps
+    torch.testing.assert_close(dropped.float(), dropped0.float(), rtol=ulp4, atol=1e-4 * ulp4)
+    assert_close(out, out0.cpu(), BF, "outputs, fused against separate")
+    for i, (x, y) in enumerate(zip(grads, grads0)):
+        assert_close(x, y.cpu(), BF, f"gradient {i}, fused against separate", scale_atol=True)
+    cov = dropped.view(B, H, T, T)
+    assert (cov.permute(0, 3, 1, 2)[pad] == 0).all() and (cov[dm.view(B, H, T, T) == 0] == 0).all()
+    # two batch columns against the oracle (every result but the weight gradients is independent per column)
+    for col in (0, B - 1):
+        sub = {k: (d[k][:, col:col + 1] if k == "x" else d[k]) for k in names}      # the positions are shared by the columns
+        dm1 = d["dropout_mask"].view(B, H, T, T)[col].reshape(H, T, T)
+        f = orel.rel_self_attn_fwd(*(sub[k] for k in names), H, d["pad_mask"][col:col + 1], None, p, dm1, D, round_to=BF)
+        g = orel.rel_self_attn_bwd(d["dout"][:, col:col + 1], sub["x"], sub["pos"], d["w_in"], d["w_out"], d["w_pos"], H, f, p, dm1, D,
+                                   round_to=BF)
+        assert_close(out[:, col:col + 1], f["outputs"], BF, f"outputs[{col}]", atol=2e-3)
+        assert_close(cov[col], f["dropout_results"], BF, f"dropout_results[{col}]")
+        assert_close(grads[0][:, col:col + 1], g["dx"], BF, f"dx[{col}]", scale_atol=True)
