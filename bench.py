@@ -437,9 +437,10 @@ class EncdecAttnWL(Workload):
 
     def step(self):
         s, a = self.s, self.a
-        r1 = self.sm.forward(True, False, self.H, s["x"], s["w_in"], s["w_out"], s["b_in"], s["b_out"], s["time_mask"], 0.0)
-        r2 = self.m.forward(False, self.H, a["x_q"], a["x_kv"], a["w_q"], a["w_kv"], a["w_out"], a["b_q"], a["b_kv"],
-                            a["b_out"], a["pad_mask"], 0.0)
+        with torch.no_grad():            # inference, as the reference's translator runs its decoder
+            r1 = self.sm.forward(True, False, self.H, s["x"], s["w_in"], s["w_out"], s["b_in"], s["b_out"], s["time_mask"], 0.0)
+            r2 = self.m.forward(False, self.H, a["x_q"], a["x_kv"], a["w_q"], a["w_kv"], a["w_out"], a["b_q"], a["b_kv"],
+                                a["b_out"], a["pad_mask"], 0.0)
         return r1[-1], r2[-1]
 
     def work_per_step(self):

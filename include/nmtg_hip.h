@@ -247,6 +247,10 @@ int nmtg_mlp_bwd(int num_layers, const void* x, const void* const* weights,
  * mask (1 = masked): mask_kind 0 none, 1 key padding [B, T], 2 time mask [T, T].
  * scores [B*H, T, T]: scaled, masked (-inf) pre-softmax scores; softmax_out (may be NULL) the
  * probabilities before dropout; dropped the probabilities after dropout (what multiplies v).
+ * scores may be NULL for an inference call (dropout_mode 0, softmax_out NULL) with head dimension
+ * 64 or 128 and a key count that is a multiple of 4: probabilities and context then come from one
+ * kernel and no score tensor is written (the backward needs it, so a call that will be
+ * back-propagated passes it). Same for nmtg_encdec_attn_fwd (its Tk then has no upper limit).
  * dropout_mode 0 none, 1 replay dropout_mask [B*H, T, T], 2 draw it (Philox) and store it.
  * ctx [T, B, E]; out [T, B, E] (NULL together with w_out in the compact form).
  * dtype NMTG_F16 or NMTG_BF16 (the reference is fp16 only); T <= 4096.

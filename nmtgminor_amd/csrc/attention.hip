@@ -56,6 +56,22 @@ int core_fwd(const Core& c, Strided q, Strided k, Strided v, const uint8_t* mask
   g.C = scores; g.ldc = c.tk; g.sC = static_cast<int64_t>(c.tq) * c.tk;
   g.M = c.tq; g.N = c.tk; g.K = c.d; g.batch = c.bh; g.alpha = c.scale;
   g.kmask = mask; g.kmask_kind = mask_kind; g.heads = c.heads;
+  // Without a score buffer (inference: nothing will be back-propagated) the probabilities and the context come from one
+  // kernel that never writes the scores.
+  if (scores == nullptr) {
+    AttnProbsCall a{};
+    a.q = q.p; a.k = k.p; a.v = v.p; a.ctx = ctx; a.probs = dropped;
+    a.q_st = q.ld; a.q_sh = q.stride; a.q_sb = q.stride * c.heads;
+    a.k_st = k.ld; a.k_sh = k.stride; a.k_sb = k.stride * c.heads;
+    a.v_st = v.ld; a.v_sh = v.stride; a.v_sb = v.stride * c.heads;
+    a.c_st = ld_ctx; a.c_sh = stride_ctx; a.c_sb = stride_ctx * c.heads;
+    a.mask = mask_kind != 0 ? mask : nullptr; a.mask_kind = mask_kind;
+    a.batch = c.bh / c.heads; a.heads = c.heads; a.d = c.d; a.tq = c.tq; a.tk = c.tk; a.scale = c.scale; a.dtype = c.dtype;
+    if (dropout_mode != 0 || softmax_out != nullptr || !attn_probs_ok(a))
+      return fail(NMTG_ERR_INVALID, "attention forward: the score buffer may only be left out for an inference call (no dropout) "
+                                    "with 16-bit tensors, head dimension 64 or 128 and a key count that is a multiple of 4");
+    return attn_probs_run(a, c.st);
+  }
   // Scores, softmax and dropout in one kernel where the call qualifies (rows of up to 512 keys, 16-byte aligned
   // operands); NMTG_ATTN_FUSED=0 always takes the two-kernel path.
   int fused = 0;
@@ -227,7 +243,7 @@ extern "C" int nmtg_self_attn_fwd(const void* x, const void* w_in, const void* w
                                   uint64_t offset, void* ctx, void* out, int64_t t, int64_t b, int64_t e, int heads,
                                   int dtype, void* stream) {
   if (int rc = check_attn("self_attn_fwd", t, t, b, e, heads, dtype)) return rc;
-  NMTG_REQUIRE(lin && scores && dropped && ctx, "self_attn_fwd: null buffer");
+  NMTG_REQUIRE(lin && dropped && ctx, "self_attn_fwd: null buffer");
   NMTG_REQUIRE(mask_kind >= 0 && mask_kind <= 2 && (mask_kind == 0 || mask != nullptr), "self_attn_fwd: bad mask arguments");
   NMTG_REQUIRE((x == nullptr) == (w_in == nullptr), "self_attn_fwd: x and w_in go together (both NULL = compact form)");
   NMTG_REQUIRE((out == nullptr) == (w_out == nullptr), "self_attn_fwd: out and w_out go together (both NULL = compact form)");
@@ -301,7 +317,7 @@ extern "C" int nmtg_encdec_attn_fwd(const void* x_q, const void* x_kv, const voi
                                     void* ctx, void* out, int64_t tq, int64_t tk, int64_t b, int64_t e, int heads,
                                     int dtype, void* stream) {
   if (int rc = check_attn("encdec_attn_fwd", tq, tk, b, e, heads, dtype)) return rc;
-  NMTG_REQUIRE(q_lin && kv_lin && scores && dropped && ctx, "encdec_attn_fwd: null buffer");
+  NMTG_REQUIRE(q_lin && kv_lin && dropped && ctx, "encdec_attn_fwd: null buffer");
   NMTG_REQUIRE((x_q == nullptr) == (w_q == nullptr) && (x_kv == nullptr) == (w_kv == nullptr),
                "encdec_attn_fwd: an input and its weight go together (both NULL = projection done by the caller)");
   NMTG_REQUIRE((out == nullptr) == (w_out == nullptr), "encdec_attn_fwd: out and w_out go together");

@@ -212,6 +212,14 @@ __device__ __forceinline__ void wave_sum2(float& a, float& b) {
 // acc + a.lo * b.lo + a.hi * b.hi on one register of two 16-bit elements each (v_dot2c_f32_f16 / v_dot2c_f32_bf16): the
 // inner step of the bandwidth-bound products (few-row projections, one-row attention), where converting every element
 // to fp32 first would cost more instructions than the multiplications.
+// Orders a wavefront's LDS writes before its later LDS reads of other lanes' data (and the reverse): the hardware runs
+// one wavefront's LDS instructions in order, the fences keep the compiler from moving them.
+__device__ __forceinline__ void wave_lds_fence() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 template <typename T> __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc);
 template <> __device__ __forceinline__ float dot2<f16_t>(uint32_t a, uint32_t b, float acc) {
   typedef _Float16 h2 __attribute__((ext_vector_type(2)));

@@ -121,7 +121,7 @@ struct Staged {
   __device__ __forceinline__ void load(const T* base, int64_t stride, int row0, int len) {
 #pragma unroll
     for (int i = 0; i < N; ++i) {
-      const int id = static_cast<int>(threadIdx.x) + FA_THREADS * i;
+      const int id = (static_cast<int>(threadIdx.x) & (FA_THREADS - 1)) + FA_THREADS * i;   // a block may hold several groups of FA_THREADS
       const int r = id / CH, c = id % CH;
       v[i] = make_uint4(0, 0, 0, 0);
       if (row0 + r < len) v[i] = *reinterpret_cast<const uint4*>(base + static_cast<int64_t>(row0 + r) * stride + 8 * c);
@@ -130,14 +130,14 @@ struct Staged {
   __device__ __forceinline__ void store_rows(uint8_t* img) const {
 #pragma unroll
     for (int i = 0; i < N; ++i) {
-      const int id = static_cast<int>(threadIdx.x) + FA_THREADS * i;
+      const int id = (static_cast<int>(threadIdx.x) & (FA_THREADS - 1)) + FA_THREADS * i;   // a block may hold several groups of FA_THREADS
       *reinterpret_cast<uint4*>(img + row_image_at<D>(id / CH, id % CH)) = v[i];
     }
   }
   __device__ __forceinline__ void store_transposed(uint8_t* img) const {
 #pragma unroll
     for (int i = 0; i < N; ++i) {
-      const int id = static_cast<int>(threadIdx.x) + FA_THREADS * i;
+      const int id = (static_cast<int>(threadIdx.x) & (FA_THREADS - 1)) + FA_THREADS * i;   // a block may hold several groups of FA_THREADS
       *reinterpret_cast<uint4*>(img + tr_image_at<D>(id / CH, id % CH)) = v[i];
     }
   }
@@ -672,6 +672,257 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dkv_ker
   store_rows_out<T, D>(dv, a.drop_scale, patch, dvb, a.dv_st, k0 + 32 * wave, lk, lane);
 }
 
+// -------------------------------------------------------------------------------------------------------------------
+// inference: probabilities and context in one kernel, two passes over the keys
+// -------------------------------------------------------------------------------------------------------------------
+// The reference's inference calls return the probabilities (its coverage), so they have to be written once; the scores
+// do not, and with them goes a write, a read and two launches of the [heads, tq, tk] tensor. The tiling is the
+// forward's above. Pass 1 streams the key tiles and keeps the running maximum and sum of each row; pass 2 streams keys
+// and values, recomputes the scores, writes the normalised probabilities (through a strip of LDS per wavefront, so that a
+// row's 64 keys leave as 128 contiguous bytes) and multiplies them with the values. The scores are rounded to the
+// tensors' 16-bit type before the softmax, as a stored score tensor would round them.
+constexpr int PA_PITCH = FA_TILE * 2 + 8;    // bytes per row of a wavefront's probability strip
+// The score of a masked key, and the running maximum before any key: a power of two, so that its product with log2(e)
+// is exact and exp2(fma(dead, log2e, -(dead * log2e))) is exactly 1 for a row that has seen no live key yet (any other
+// constant leaves the fma a rounding residue of 1e22, whose exp2 overflows).
+constexpr float PA_DEAD = -0x1p100f;
+
+// the two 16-bit elements of a register as floats
+template <typename T> __device__ __forceinline__ float unpack_lo(uint32_t w);
+template <typename T> __device__ __forceinline__ float unpack_hi(uint32_t w);
+template <> __device__ __forceinline__ float unpack_lo<bf16_t>(uint32_t w) { return __uint_as_float(w << 16); }
+template <> __device__ __forceinline__ float unpack_hi<bf16_t>(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+template <> __device__ __forceinline__ float unpack_lo<f16_t>(uint32_t w) {
+  return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(w & 0xffffu)));
+}
+template <> __device__ __forceinline__ float unpack_hi<f16_t>(uint32_t w) {
+  return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(w >> 16)));
+}
+
+// mask bytes (1 = masked) of the four keys key0 .. key0 + 3 for this lane's query, keys past the end count as masked.
+// The load is unconditional (from a clamped address) and the eight words of a tile are requested together, ahead of
+// the products: as loads inside branches they were waited for one by one.
+template <int MASK>
+__device__ __forceinline__ uint32_t mask_word(const AttnProbsCall& a, int b, int qrow, int key0) {
+  if constexpr (MASK == 0) return key0 < a.tk ? 0u : 0x01010101u;
+  const int kc = min(key0, a.tk - 4);                 // tk is a positive multiple of 4
+  const int64_t row = MASK == 1 ? b : min(qrow, a.tq - 1);
+  const uint32_t w = *reinterpret_cast<const uint32_t*>(a.mask + row * a.tk + kc);
+  return key0 < a.tk ? w : 0x01010101u;
+}
+template <int MASK>
+__device__ __forceinline__ void tile_mask_words(const AttnProbsCall& a, int b, int qrow, int t, int half, uint32_t (&mw)[2][4]) {
+#pragma unroll
+  for (int n = 0; n < 2; ++n)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) mw[n][g] = mask_word<MASK>(a, b, qrow, t * FA_TILE + 32 * n + 8 * g + 4 * half);
+}
+
+// G groups of four wavefronts share the block's 128 queries and take the key tiles in turn (tile t goes to group
+// t % G); each group has its own tile buffers, the row statistics after pass 1 and the context accumulators after pass 2
+// are combined through LDS. G = 2 is for calls with so few blocks (a decoder's 128 positions: one block per head and
+// sentence) that four wavefronts per compute unit would leave the vector units waiting on every dependency.
+template <typename T, int D, int MASK, int G>
+__global__ __launch_bounds__(FA_THREADS * G, (D == 64 && G == 1) ? 2 : 1) void attn_probs_kernel(AttnProbsCall a) {
+  extern __shared__ __align__(16) uint8_t lds_raw[];
+  constexpr int IMG = FA_TILE * D * 2, NWAVE = 4 * G;
+  const int b = blockIdx.z, h = blockIdx.y, q0 = static_cast<int>(blockIdx.x) * FA_ROWS;
+  const int lane = static_cast<int>(threadIdx.x) & 63, half = lane >> 5;
+  const int wave_all = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);
+  const int group = wave_all / 4, wave = wave_all % 4;
+  const int qrow = q0 + 32 * wave + (lane & 31);
+  const T* qb = static_cast<const T*>(a.q) + b * a.q_sb + h * a.q_sh;
+  const T* kb = static_cast<const T*>(a.k) + b * a.k_sb + h * a.k_sh;
+  const T* vb = static_cast<const T*>(a.v) + b * a.v_sb + h * a.v_sh;
+  uint4 qf[D / 16];
+  load_resident<T, D>(qf, qb, a.q_st, qrow, a.tq, lane);
+  const int ntiles = (a.tk + FA_TILE - 1) / FA_TILE;
+  const int rounds = (ntiles + G - 1) / G;           // every group runs the same number of rounds (block barriers inside)
+  uint8_t* tiles = lds_raw + group * (4 * IMG);
+  uint8_t* strip = lds_raw + G * (4 * IMG) + wave_all * (32 * PA_PITCH);
+  float* stats = reinterpret_cast<float*>(lds_raw + G * (4 * IMG) + NWAVE * (32 * PA_PITCH));   // [G][128][2]
+
+  // the tile's 32 scores of this lane, rounded and masked
+  auto tile_scores = [&](const uint8_t* kimg, int t, acc16_t (&s)[2]) {
+    uint32_t mw[2][4];
+    tile_mask_words<MASK>(a, b, qrow, t, half, mw);
+#pragma unroll
+    for (int n = 0; n < 2; ++n)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[n][r] = 0.f;
+#pragma unroll
+    for (int ss = 0; ss < D / 16; ++ss)
+#pragma unroll
+      for (int n = 0; n < 2; ++n) mfma<T>::run(read_rows<D>(kimg, n, ss, lane), qf[ss], s[n]);
+    // scaled, rounded to the 16-bit type two at a time (one packed conversion, two unpacking shifts), masked; natural units
+#pragma unroll
+    for (int n = 0; n < 2; ++n)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+#pragma unroll
+        for (int e = 0; e < 4; e += 2) {
+          const uint32_t pr = pack2<T>(s[n][4 * g + e] * a.scale, s[n][4 * g + e + 1] * a.scale);
+          const float lo = unpack_lo<T>(pr), hi = unpack_hi<T>(pr);
+          s[n][4 * g + e] = ((mw[n][g] >> (8 * e)) & 0xffu) != 0 ? PA_DEAD : lo;
+          s[n][4 * g + e + 1] = ((mw[n][g] >> (8 * e + 8)) & 0xffu) != 0 ? PA_DEAD : hi;
+        }
+      }
+  };
+
+  // ---- pass 1: row maximum and sum over this group's tiles ----
+  float m = PA_DEAD, l = 0.f;
+  Staged<D> sk, sv;
+  if (group < ntiles) {
+    sk.load(kb, a.k_st, group * FA_TILE, a.tk);
+    sk.store_rows(tiles);
+  }
+  __syncthreads();
+  for (int it = 0; it < rounds; ++it) {
+    const int t = it * G + group;
+    const uint8_t* kimg = tiles + (it & 1) * 2 * IMG;
+    if (t + G < ntiles) sk.load(kb, a.k_st, (t + G) * FA_TILE, a.tk);
+    if (t < ntiles) {
+      acc16_t s[2];
+      tile_scores(kimg, t, s);
+      float mx = s[0][0];
+#pragma unroll
+      for (int n = 0; n < 2; ++n)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[n][r]);
+      const float m_new = fmaxf(m, pair_max(mx));
+      const float m2 = m_new * FA_LOG2E;
+      float sum = 0.f;
+#pragma unroll
+      for (int n = 0; n < 2; ++n)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sum += fast_exp2(__builtin_fmaf(s[n][r], FA_LOG2E, -m2));
+      l = l * fast_exp2((m - m_new) * FA_LOG2E) + sum;
+      m = m_new;
+    }
+    if (t + G < ntiles) sk.store_rows(tiles + ((it + 1) & 1) * 2 * IMG);
+    __syncthreads();
+  }
+  l = pair_sum(l);
+  if constexpr (G > 1) {
+    if (half == 0) {
+      stats[((group * 4 + wave) * 32 + lane) * 2] = m;
+      stats[((group * 4 + wave) * 32 + lane) * 2 + 1] = l;
+    }
+    __syncthreads();
+    float mm = PA_DEAD, ll = 0.f;
+#pragma unroll
+    for (int gg = 0; gg < G; ++gg) mm = fmaxf(mm, stats[((gg * 4 + wave) * 32 + (lane & 31)) * 2]);
+#pragma unroll
+    for (int gg = 0; gg < G; ++gg) {
+      const float* st2 = stats + ((gg * 4 + wave) * 32 + (lane & 31)) * 2;
+      ll += st2[1] * fast_exp2((st2[0] - mm) * FA_LOG2E);
+    }
+    m = mm;
+    l = ll;
+  }
+  // a row without a live key keeps the initial maximum: its probabilities are zeros (the reference turns the NaN into 0)
+  const float inv = (m > 0.5f * PA_DEAD && l > 0.f) ? 1.f / l : 0.f;
+
+  // ---- pass 2: probabilities out, context accumulated ----
+  const float m2 = m * FA_LOG2E;
+  acc16_t o[D / 32];
+#pragma unroll
+  for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
+  if (group < ntiles) {
+    sk.load(kb, a.k_st, group * FA_TILE, a.tk);
+    sv.load(vb, a.v_st, group * FA_TILE, a.tk);
+    sk.store_rows(tiles);
+    sv.store_transposed(tiles + IMG);
+  }
+  __syncthreads();
+  T* prow = static_cast<T*>(a.probs) + (static_cast<int64_t>(b) * a.heads + h) * a.tq * a.tk;
+  for (int it = 0; it < rounds; ++it) {
+    const int t = it * G + group;
+    const uint8_t* kimg = tiles + (it & 1) * 2 * IMG;
+    const uint8_t* vimg = kimg + IMG;
+    if (t + G < ntiles) {
+      sk.load(kb, a.k_st, (t + G) * FA_TILE, a.tk);
+      sv.load(vb, a.v_st, (t + G) * FA_TILE, a.tk);
+    }
+    if (t < ntiles) {
+      acc16_t s[2];
+      tile_scores(kimg, t, s);
+#pragma unroll
+      for (int n = 0; n < 2; ++n)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[n][r] = fast_exp2(__builtin_fmaf(s[n][r], FA_LOG2E, -m2)) * inv;
+      // this lane's 4-key groups into the wavefront's strip: row = its query, 8 bytes per group
+#pragma unroll
+      for (int n = 0; n < 2; ++n)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          uint2 w;
+          w.x = pack2<T>(s[n][4 * g + 0], s[n][4 * g + 1]);
+          w.y = pack2<T>(s[n][4 * g + 2], s[n][4 * g + 3]);
+          *reinterpret_cast<uint2*>(strip + (lane & 31) * PA_PITCH + (32 * n + 8 * g + 4 * half) * 2) = w;
+        }
+#pragma unroll
+      for (int kk = 0; kk < FA_TILE / 16; ++kk) {
+        float pv[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) pv[e] = s[kk / 2][8 * (kk % 2) + e];
+        const uint4 pf = acc_to_operand<T>(pv);
+#pragma unroll
+        for (int i = 0; i < D / 32; ++i) mfma<T>::run(read_transposed<D>(vimg, i, kk, lane), pf, o[i]);
+      }
+      wave_lds_fence();
+      // 16 lanes take one row's 64 keys (8 bytes each), four rows per step
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int r = 4 * j + (lane >> 4), key = t * FA_TILE + 4 * (lane & 15);
+        const int row = q0 + 32 * wave + r;
+        if (row < a.tq && key < a.tk)
+          *reinterpret_cast<uint2*>(prow + static_cast<int64_t>(row) * a.tk + key) =
+              *reinterpret_cast<const uint2*>(strip + r * PA_PITCH + 8 * (lane & 15));
+      }
+      wave_lds_fence();
+    }
+    if (t + G < ntiles) {
+      uint8_t* nk = tiles + ((it + 1) & 1) * 2 * IMG;
+      sk.store_rows(nk);
+      sv.store_transposed(nk + IMG);
+    }
+    __syncthreads();
+  }
+  if constexpr (G > 1) {
+    // the other groups' partial contexts through LDS (over the tile buffers, which nobody reads any more)
+    float4* part = reinterpret_cast<float4*>(lds_raw);
+    if (group != 0) {
+#pragma unroll
+      for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+          part[((((group - 1) * 4 + wave) * (D / 32) + i) * 4 + g) * 64 + lane] =
+              make_float4(o[i][4 * g], o[i][4 * g + 1], o[i][4 * g + 2], o[i][4 * g + 3]);
+    }
+    __syncthreads();
+    if (group == 0) {
+#pragma unroll
+      for (int gg = 0; gg < G - 1; ++gg)
+#pragma unroll
+        for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const float4 x = part[(((gg * 4 + wave) * (D / 32) + i) * 4 + g) * 64 + lane];
+            o[i][4 * g] += x.x; o[i][4 * g + 1] += x.y; o[i][4 * g + 2] += x.z; o[i][4 * g + 3] += x.w;
+          }
+    }
+    __syncthreads();
+  }
+  T* cb = static_cast<T*>(a.ctx) + b * a.c_sb + h * a.c_sh;
+  // every wavefront takes part in the store's barrier; only group 0 holds rows to store
+  store_rows_out<T, D>(o, 1.f, lds_raw + wave_all * (32 * D * 2), cb, a.c_st, q0 + 32 * wave, group == 0 ? a.tq : 0, lane);
+}
+
+template <int D, int G> constexpr int probs_lds() { return G * (4 * FA_TILE * D * 2 + 4 * 32 * PA_PITCH + 128 * 2 * 4); }
+
 template <int D> constexpr int fwd_lds() { return 2 * 2 * FA_TILE * D * 2; }
 template <int D> constexpr int dq_lds() { return 2 * 3 * FA_TILE * D * 2; }
 template <int D> constexpr int dkv_lds() { return 2 * (4 * FA_TILE * D * 2 + 2 * FA_TILE * 4); }
@@ -760,7 +1011,59 @@ void set_dropout(FaArgs& a, int drop_mode, float p, uint64_t seed, uint64_t offs
   a.offset = offset;
 }
 
+template <typename T, int D, int G>
+int probs_launch(const AttnProbsCall& c, dim3 grid, hipStream_t st) {
+  auto go = [&](auto kern) {
+    constexpr int lds = probs_lds<D, G>();
+    if (lds > 64 * 1024) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+      if (e != hipSuccess) return fail(NMTG_ERR_LAUNCH, "attn_probs: cannot reserve %d bytes of LDS: %s", lds, hipGetErrorString(e));
+    }
+    hipLaunchKernelGGL(kern, grid, dim3(FA_THREADS * G), lds, st, c);
+    return 0;
+  };
+  if (c.mask == nullptr || c.mask_kind == 0) return go(attn_probs_kernel<T, D, 0, G>);
+  if (c.mask_kind == 1) return go(attn_probs_kernel<T, D, 1, G>);
+  return go(attn_probs_kernel<T, D, 2, G>);
+}
+
 }  // namespace
+
+bool attn_probs_ok(const AttnProbsCall& c) {
+  if (switched_off("NMTG_ATTN_PROBS")) return false;
+  auto view = [&](const void* p, int64_t st, int64_t sb, int64_t sh) {
+    return aligned16(p) && st % 8 == 0 && sb % 8 == 0 && sh % 8 == 0 && st >= 0 && sb >= 0 && sh >= 0;
+  };
+  return (c.dtype == NMTG_F16 || c.dtype == NMTG_BF16) && (c.d == 64 || c.d == 128) && c.tk >= 1 && c.tk % 4 == 0 && c.tq >= 1 &&
+         c.batch >= 1 && c.batch <= 65535 && c.heads >= 1 && c.heads <= 65535 && view(c.q, c.q_st, c.q_sb, c.q_sh) &&
+         view(c.k, c.k_st, c.k_sb, c.k_sh) && view(c.v, c.v_st, c.v_sb, c.v_sh) && view(c.ctx, c.c_st, c.c_sb, c.c_sh) &&
+         reinterpret_cast<uintptr_t>(c.probs) % 8 == 0 &&
+         (c.mask == nullptr || c.mask_kind == 0 || reinterpret_cast<uintptr_t>(c.mask) % 4 == 0) && fabsf(c.scale) <= 1e6f;
+}
+
+int attn_probs_run(const AttnProbsCall& c, hipStream_t st) {
+  // Two groups of wavefronts per block when the blocks alone would not give every SIMD two wavefronts and there are
+  // key tiles to share out. NMTG_ATTN_PROBS_SPLIT=0 / =1 forces one form or the other.
+  const dim3 grid(static_cast<unsigned>((c.tq + FA_ROWS - 1) / FA_ROWS), static_cast<unsigned>(c.heads), static_cast<unsigned>(c.batch));
+  const int64_t blocks = static_cast<int64_t>(grid.x) * grid.y * grid.z;
+  const char* forced = getenv("NMTG_ATTN_PROBS_SPLIT");
+  // (head dimension 64 only: at 128 the tile buffers of two groups do not fit the LDS)
+  const bool split = c.d == 64 && (forced != nullptr && (forced[0] == '0' || forced[0] == '1') ? forced[0] == '1'
+                                                                                               : blocks < 2 * 256 && c.tk > 2 * FA_TILE);
+  TraceScope trace(split ? "attn_probs_2groups" : "attn_probs", st);
+  int rc;
+  if (split) {
+    rc = c.dtype == NMTG_F16 ? probs_launch<f16_t, 64, 2>(c, grid, st) : probs_launch<bf16_t, 64, 2>(c, grid, st);
+  } else {
+    if (c.dtype == NMTG_F16) rc = c.d == 64 ? probs_launch<f16_t, 64, 1>(c, grid, st) : probs_launch<f16_t, 128, 1>(c, grid, st);
+    else rc = c.d == 64 ? probs_launch<bf16_t, 64, 1>(c, grid, st) : probs_launch<bf16_t, 128, 1>(c, grid, st);
+  }
+  if (rc) return rc;
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(NMTG_ERR_LAUNCH, "attn_probs: launch failed: %s", hipGetErrorString(e));
+  return 0;
+}
+
 }  // namespace nmtg
 
 using namespace nmtg;

@@ -1011,6 +1011,22 @@ int gemm_f32_run(int layout, int epi, GemmArgs a, hipStream_t st, int* m_tiles_o
 bool gemm_skinny_ok(int dtype, int layout, int epi, const GemmArgs& a);
 int gemm_skinny_run(int dtype, const GemmArgs& a, hipStream_t st);
 
+// Attention probabilities and context of an inference call in one kernel (flash_attn.hip): probs [batch * heads, tq, tk]
+// = softmax over the keys of round(scale q k^T) with masked keys at -inf (rows without a live key: zeros), ctx = probs v.
+// The score tensor is never written. q, k, v, ctx: element (token t, sentence b, head h, :) at t * st + b * sb + h * sh.
+struct AttnProbsCall {
+  const void *q, *k, *v;
+  void *ctx, *probs;
+  int64_t q_st, q_sb, q_sh, k_st, k_sb, k_sh, v_st, v_sb, v_sh, c_st, c_sb, c_sh;
+  const uint8_t* mask;      // mask_kind 1: [batch, tk] key padding; 2: [tq, tk] time mask; 1 = masked
+  int mask_kind;
+  int batch, heads, d, tq, tk;
+  float scale;
+  int dtype;
+};
+bool attn_probs_ok(const AttnProbsCall& c);    // NMTG_ATTN_PROBS=0 switches the kernel off
+int attn_probs_run(const AttnProbsCall& c, hipStream_t st);
+
 // Fused Q K^T -> mask -> softmax -> dropout (EPI_SCORES_SOFTMAX) for rows of at most 512 keys. `a` is filled as
 // for EPI_SCORES plus out2 (dropped probabilities), aux_out (softmax, optional), dmask / rng / keep_p / dscale /
 // seed / offset. Returns 1 if the kernel was launched, 0 if the call does not qualify (the caller then runs the

@@ -68,13 +68,6 @@ __device__ __forceinline__ RelRow rel_row(int64_t row, uint32_t q_len, uint32_t 
   const uint32_t p0 = i * len_r + q_len, i2 = p0 / (len_r + 1);
   return RelRow{i, p0 - i2 * (len_r + 1), (static_cast<int64_t>(b) * q_len + i2) * len_r};
 }
-// Orders a wavefront's LDS writes before its later LDS reads of other lanes' data (and the reverse): the hardware runs
-// one wavefront's LDS instructions in order, the fences keep the compiler from moving them.
-__device__ __forceinline__ void wave_lds_fence() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
 // offset from RelRow::first of the bd element behind column c, or -1 for the zero column
 __device__ __forceinline__ int rel_source(uint32_t c, uint32_t len_r) {
   if (c == 0 || c == len_r + 1) return -1;

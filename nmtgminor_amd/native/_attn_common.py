@@ -1,5 +1,6 @@
 """Shared plumbing of the attention stand-in modules."""
 import ctypes
+import os
 
 import torch
 
@@ -46,6 +47,16 @@ def dropout_args(is_training, p, shape, device, dropout_mask):
         seed, offset = philox_seed_offset(device, n)
         return m, 2, seed, offset
     return torch.empty(0, dtype=torch.uint8, device=device), 0, 0, 0
+
+
+def scores_needed(is_training, dtype, head_dim, tk):
+    """Whether a forward call has to keep the pre-softmax scores. They exist for the backward; a call that is neither in
+    training mode nor recorded by autograd (inference under torch.no_grad()) leaves them out where the one-kernel
+    inference path takes the shape (16-bit tensors, head dimension 64 or 128, a key count that is a multiple of 4), and
+    the stand-in then returns an empty tensor in their place. NMTG_ATTN_PROBS=0 keeps them always."""
+    if is_training or torch.is_grad_enabled() or os.environ.get("NMTG_ATTN_PROBS", "1") == "0":
+        return True
+    return not (dtype in (torch.float16, torch.bfloat16) and head_dim in (64, 128) and tk >= 1 and tk % 4 == 0)
 
 
 def u64(v):

@@ -20,7 +20,8 @@ def _dims(inputs, heads, last):
 
 def forward(use_time_mask, is_training, heads, inputs, input_weights, output_weights, input_biases, output_biases,
             pad_mask, dropout_prob, *, dropout_mask=None):
-    """-> [input_lin_results, attn_scores, dropout_results, dropout_mask, matmul2_results, outputs]"""
+    """-> [input_lin_results, attn_scores, dropout_results, dropout_mask, matmul2_results, outputs]; attn_scores is empty
+    for an inference call under torch.no_grad() (see _attn_common.scores_needed)."""
     L.require_cuda(inputs, input_weights, output_weights, input_biases, output_biases, pad_mask, dropout_mask)
     A.check(input_weights.dim() == 2 and output_weights.dim() == 2, "expected 2D tensor")
     A.check_half(inputs, input_weights, output_weights, input_biases, output_biases)
@@ -34,7 +35,8 @@ def forward(use_time_mask, is_training, heads, inputs, input_weights, output_wei
     km, kind = A.mask_arg(pad_mask, use_time_mask, b, t, t)
     bh = b * heads
     lin = torch.empty(t, b, 3 * e, dtype=dt, device=dev)
-    scores = torch.empty(bh, t, t, dtype=dt, device=dev)
+    keep_scores = A.scores_needed(is_training, dt, e // heads, t)
+    scores = torch.empty((bh, t, t) if keep_scores else (0,), dtype=dt, device=dev)
     dropped = torch.empty(bh, t, t, dtype=dt, device=dev)
     ctx = torch.empty(t, b, e, dtype=dt, device=dev)
     out = torch.empty(t, b, e, dtype=dt, device=dev)
@@ -42,7 +44,7 @@ def forward(use_time_mask, is_training, heads, inputs, input_weights, output_wei
     if t == 0 or b == 0:        # an empty batch: the (empty) buffers are the result
         return [lin, scores, dropped, dmask, ctx, out]
     L.call("nmtg_self_attn_fwd", L.ptr(x), L.ptr(w_in), L.ptr(w_out), L.ptr(b_in), L.ptr(b_out), L.ptr(km), L.i32(kind),
-           L.ptr(lin), L.ptr(scores), L.ptr(None), L.ptr(dropped), L.ptr(dmask if mode else None), L.i32(mode),
+           L.ptr(lin), L.ptr(scores if keep_scores else None), L.ptr(None), L.ptr(dropped), L.ptr(dmask if mode else None), L.i32(mode),
            L.f32(dropout_prob), A.u64(seed), A.u64(offset), L.ptr(ctx), L.ptr(out), L.i64(t), L.i64(b), L.i64(e),
            L.i32(heads), L.i32(L.dtype_code(x)), L.stream_of(x))
     return [lin, scores, dropped, dmask, ctx, out]

@@ -298,3 +298,79 @@ def test_feed_forward_module(dev):
     assert_close(yr.view(80, 128), yo.to(torch.float16).to(D) + x.cpu().view(80, 128).to(D), torch.float16, "residual")
     with pytest.raises(NotImplementedError):
         PositionWiseFeedForward(128, 512, activation="tanh")
+
+
+# ----------------------------------------------------------------------------- inference without a score tensor
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("split", ["0", "1"])
+@pytest.mark.parametrize("t,b,e,h,causal", [(100, 3, 256, 4, False), (72, 2, 256, 2, True), (200, 2, 128, 2, False), (36, 2, 256, 4, True)])
+def test_self_attention_inference_without_the_score_tensor(dev, monkeypatch, dtype, t, b, e, h, causal, split):
+    """Under torch.no_grad() an inference call returns no scores and runs the one-kernel path (probabilities and context
+    from two passes over the keys). Held against the oracle and against the score-keeping path of the same library
+    (the same rounding points: scores rounded to the 16-bit type, probabilities rounded before they multiply v). `split`
+    forces one of the kernel's two forms: blocks of 128 queries, or blocks of 32 queries whose wavefronts share the keys."""
+    monkeypatch.setenv("NMTG_ATTN_PROBS_SPLIT", split)
+    d = inputs.self_attn_inputs(t, b, e, h, dtype, p=0.0, seed=300 + t, causal=causal)
+    if not causal:
+        d["pad_mask"][-1, :] = True                                        # a sentence without any live key: zeros, not NaN
+    fwd = oat.self_attn_fwd(d["x"], d["w_in"], d["w_out"], d["b_in"], d["b_out"], h, d["pad_mask"], d["time_mask"], 0.0, None, D,
+                            round_to=dtype)
+    g = lambda k: d[k].to(dev)
+    mask = g("time_mask") if causal else g("pad_mask")
+    args = (causal, False, h, g("x"), g("w_in"), g("w_out"), g("b_in"), g("b_out"), mask, 0.1)
+    with torch.no_grad():
+        lin, scores, dropped, dmask, ctx, out = sa_native.forward(*args)
+    assert scores.numel() == 0 and dmask.numel() == 0 and dropped.shape == (b * h, t, t)
+    lin2, scores2, dropped2, _, ctx2, out2 = sa_native.forward(*args)     # recorded by autograd: keeps the scores
+    assert scores2.shape == (b * h, t, t)
+    assert_close(out, fwd["outputs"], dtype, "outputs")
+    assert_close(dropped, fwd["dropout_results"], dtype, "probabilities")
+    assert_close(dropped, dropped2.cpu(), dtype, "probabilities, against the score-keeping path")
+    assert_close(ctx, ctx2.cpu(), dtype, "context, against the score-keeping path")
+    assert not torch.isnan(dropped.float()).any()
+    cov = dropped.float().cpu().view(b, h, t, t)
+    if causal:
+        assert (cov[:, :, torch.triu(torch.ones(t, t), 1).bool()] == 0).all()
+    else:
+        assert (cov.permute(0, 3, 1, 2)[d["pad_mask"]] == 0).all() and (cov[-1] == 0).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("tq,tk,b,e,h,masked", [(32, 1500, 2, 256, 4, True), (17, 100, 3, 128, 2, True), (130, 64, 2, 512, 4, False),
+                                                (5, 260, 1, 128, 1, True)])
+@pytest.mark.parametrize("split", ["0", "1"])
+def test_encdec_attention_inference_without_the_score_tensor(dev, monkeypatch, dtype, tq, tk, b, e, h, masked, split):
+    monkeypatch.setenv("NMTG_ATTN_PROBS_SPLIT", split)
+    d = inputs.encdec_attn_inputs(tq, tk, b, e, h, dtype, p=0.0, seed=400 + tq)
+    pad = d["pad_mask"] if masked else None
+    fwd = oat.encdec_attn_fwd(d["x_q"], d["x_kv"], d["w_q"], d["w_kv"], d["w_out"], d["b_q"], d["b_kv"], d["b_out"], h, pad, 0.0,
+                              None, D, round_to=dtype)
+    g = lambda k: d[k].to(dev)
+    args = (False, h, g("x_q"), g("x_kv"), g("w_q"), g("w_kv"), g("w_out"), g("b_q"), g("b_kv"), g("b_out"),
+            None if pad is None else pad.to(dev), 0.0)
+    with torch.no_grad():
+        q_lin, kv_lin, scores, dropped, dmask, ctx, out = ed_native.forward(*args)
+    assert scores.numel() == 0 and dropped.shape == (b * h, tq, tk) and kv_lin.shape == (tk, b, 2 * e)
+    r2 = ed_native.forward(*args)
+    assert r2[2].shape == (b * h, tq, tk)
+    assert_close(out, fwd["outputs"], dtype, "outputs")
+    assert_close(dropped, fwd["dropout_results"], dtype, "probabilities")
+    assert_close(dropped, r2[3].cpu(), dtype, "probabilities, against the score-keeping path")
+    assert_close(ctx, r2[5].cpu(), dtype, "context, against the score-keeping path")
+    if masked:
+        assert (dropped.float().cpu().view(b, h, tq, tk).permute(0, 3, 1, 2)[d["pad_mask"]] == 0).all()
+    assert (dropped.float().sum(-1) - 1).abs().max() < 2e-2
+
+
+def test_inference_keeps_the_score_tensor_where_the_one_kernel_path_does_not_apply(dev, monkeypatch):
+    d = inputs.self_attn_inputs(30, 2, 64, 2, torch.bfloat16, p=0.0, seed=9)        # head dimension 32, 30 keys
+    g = lambda k: d[k].to(dev)
+    with torch.no_grad():
+        r = sa_native.forward(False, False, 2, g("x"), g("w_in"), g("w_out"), g("b_in"), g("b_out"), g("pad_mask"), 0.0)
+    assert r[1].shape == (4, 30, 30)
+    d = inputs.self_attn_inputs(64, 2, 128, 2, torch.bfloat16, p=0.0, seed=9)
+    g = lambda k: d[k].to(dev)
+    monkeypatch.setenv("NMTG_ATTN_PROBS", "0")
+    with torch.no_grad():
+        r = sa_native.forward(False, False, 2, g("x"), g("w_in"), g("w_out"), g("b_in"), g("b_out"), g("pad_mask"), 0.0)
+    assert r[1].shape == (4, 64, 64)

@@ -373,6 +373,15 @@ def test_encdec_attention(mi355x, dtype, tq, tk, b, e, h, p):
 
 
 @long_case
+@pytest.mark.parametrize("split", ["0", "1"])
+def test_attention_inference_without_the_score_tensor(mi355x, monkeypatch, split):
+    tat.test_self_attention_inference_without_the_score_tensor(CPU, monkeypatch, BF16, 100, 3, 256, 4, False, split)
+    tat.test_self_attention_inference_without_the_score_tensor(CPU, monkeypatch, F16, 72, 2, 256, 2, True, split)
+    tat.test_encdec_attention_inference_without_the_score_tensor(CPU, monkeypatch, BF16, 17, 100, 3, 128, 2, True, split)
+    tat.test_encdec_attention_inference_without_the_score_tensor(CPU, monkeypatch, F16, 5, 260, 1, 128, 1, True, split)
+    tat.test_inference_keeps_the_score_tensor_where_the_one_kernel_path_does_not_apply(CPU, monkeypatch)
+
+
 def test_encdec_attention_without_biases_compact_and_modules(mi355x):
     tat.test_encdec_attention_without_biases_and_compact(CPU)
     tat.test_modules_state_dict_names_and_forward(CPU)
