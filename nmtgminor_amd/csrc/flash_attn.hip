@@ -737,10 +737,30 @@ __global__ __launch_bounds__(FA_THREADS * G, (D == 64 && G == 1) ? 2 : 1) void a
   uint4 qf[D / 16];
   load_resident<T, D>(qf, qb, a.q_st, qrow, a.tq, lane);
   const int ntiles = (a.tk + FA_TILE - 1) / FA_TILE;
-  const int rounds = (ntiles + G - 1) / G;           // every group runs the same number of rounds (block barriers inside)
   uint8_t* tiles = lds_raw + group * (4 * IMG);
   uint8_t* strip = lds_raw + G * (4 * IMG) + wave_all * (32 * PA_PITCH);
   float* stats = reinterpret_cast<float*>(lds_raw + G * (4 * IMG) + NWAVE * (32 * PA_PITCH));   // [G][128][2]
+  // With a key-padding mask the sentence's keys end somewhere before tk (padding sits at the end of a batch's shorter
+  // sentences): the tiles behind the last live key are not computed, their probabilities are written as the zeros they are.
+  int live_tiles = ntiles;
+  if constexpr (MASK == 1) {
+    int last = -1;
+    const uint8_t* mrow = a.mask + static_cast<int64_t>(b) * a.tk;
+    for (int j = 4 * static_cast<int>(threadIdx.x); j < a.tk; j += 4 * FA_THREADS * G) {
+      const uint32_t w = *reinterpret_cast<const uint32_t*>(mrow + j);
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (((w >> (8 * e)) & 0xffu) == 0) last = j + e;
+    }
+    const float wl = wave_max(static_cast<float>(last));     // key indices are far below 2^24: exact in fp32
+    if (lane == 0) stats[wave_all] = wl;
+    __syncthreads();
+    float bl = stats[0];
+#pragma unroll
+    for (int w = 1; w < NWAVE; ++w) bl = fmaxf(bl, stats[w]);
+    live_tiles = (static_cast<int>(bl) + 1 + FA_TILE - 1) / FA_TILE;
+    __syncthreads();                                        // stats is written again after pass 1
+  }
 
   // the tile's 32 scores of this lane, rounded and masked
   auto tile_scores = [&](const uint8_t* kimg, int t, acc16_t (&s)[2]) {
@@ -772,16 +792,17 @@ __global__ __launch_bounds__(FA_THREADS * G, (D == 64 && G == 1) ? 2 : 1) void a
   // ---- pass 1: row maximum and sum over this group's tiles ----
   float m = PA_DEAD, l = 0.f;
   Staged<D> sk, sv;
-  if (group < ntiles) {
+  const int live_rounds = (live_tiles + G - 1) / G;
+  if (group < live_tiles) {
     sk.load(kb, a.k_st, group * FA_TILE, a.tk);
     sk.store_rows(tiles);
   }
   __syncthreads();
-  for (int it = 0; it < rounds; ++it) {
+  for (int it = 0; it < live_rounds; ++it) {
     const int t = it * G + group;
     const uint8_t* kimg = tiles + (it & 1) * 2 * IMG;
-    if (t + G < ntiles) sk.load(kb, a.k_st, (t + G) * FA_TILE, a.tk);
-    if (t < ntiles) {
+    if (t + G < live_tiles) sk.load(kb, a.k_st, (t + G) * FA_TILE, a.tk);
+    if (t < live_tiles) {
       acc16_t s[2];
       tile_scores(kimg, t, s);
       float mx = s[0][0];
@@ -799,7 +820,7 @@ __global__ __launch_bounds__(FA_THREADS * G, (D == 64 && G == 1) ? 2 : 1) void a
       l = l * fast_exp2((m - m_new) * FA_LOG2E) + sum;
       m = m_new;
     }
-    if (t + G < ntiles) sk.store_rows(tiles + ((it + 1) & 1) * 2 * IMG);
+    if (t + G < live_tiles) sk.store_rows(tiles + ((it + 1) & 1) * 2 * IMG);
     __syncthreads();
   }
   l = pair_sum(l);
@@ -830,7 +851,7 @@ __global__ __launch_bounds__(FA_THREADS * G, (D == 64 && G == 1) ? 2 : 1) void a
   for (int i = 0; i < D / 32; ++i)
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
-  if (group < ntiles) {
+  if (group < live_tiles) {
     sk.load(kb, a.k_st, group * FA_TILE, a.tk);
     sv.load(vb, a.v_st, group * FA_TILE, a.tk);
     sk.store_rows(tiles);
@@ -838,15 +859,23 @@ __global__ __launch_bounds__(FA_THREADS * G, (D == 64 && G == 1) ? 2 : 1) void a
   }
   __syncthreads();
   T* prow = static_cast<T*>(a.probs) + (static_cast<int64_t>(b) * a.heads + h) * a.tq * a.tk;
-  for (int it = 0; it < rounds; ++it) {
+  // the tiles behind the last live key: zeros, no arithmetic (every wavefront of the block takes its share of them)
+  for (int t = live_tiles + group; t < ntiles; t += G) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int row = q0 + 32 * wave + 4 * j + (lane >> 4), key = t * FA_TILE + 4 * (lane & 15);
+      if (row < a.tq && key < a.tk) *reinterpret_cast<uint2*>(prow + static_cast<int64_t>(row) * a.tk + key) = make_uint2(0, 0);
+    }
+  }
+  for (int it = 0; it < live_rounds; ++it) {
     const int t = it * G + group;
     const uint8_t* kimg = tiles + (it & 1) * 2 * IMG;
     const uint8_t* vimg = kimg + IMG;
-    if (t + G < ntiles) {
+    if (t + G < live_tiles) {
       sk.load(kb, a.k_st, (t + G) * FA_TILE, a.tk);
       sv.load(vb, a.v_st, (t + G) * FA_TILE, a.tk);
     }
-    if (t < ntiles) {
+    if (t < live_tiles) {
       acc16_t s[2];
       tile_scores(kimg, t, s);
 #pragma unroll
@@ -884,7 +913,7 @@ __global__ __launch_bounds__(FA_THREADS * G, (D == 64 && G == 1) ? 2 : 1) void a
       }
       wave_lds_fence();
     }
-    if (t + G < ntiles) {
+    if (t + G < live_tiles) {
       uint8_t* nk = tiles + ((it + 1) & 1) * 2 * IMG;
       sk.store_rows(nk);
       sv.store_transposed(nk + IMG);
