@@ -250,7 +250,9 @@ int nmtg_mlp_bwd(int num_layers, const void* x, const void* const* weights,
  * scores may be NULL for an inference call (dropout_mode 0, softmax_out NULL) with head dimension
  * 64 or 128 and a key count that is a multiple of 4: probabilities and context then come from one
  * kernel and no score tensor is written (the backward needs it, so a call that will be
- * back-propagated passes it). Same for nmtg_encdec_attn_fwd (its Tk then has no upper limit).
+ * back-propagated passes it); `dropped` may then be NULL too, for a caller that does not return
+ * the probabilities (no [B*H, T, T] tensor at all). Same for nmtg_encdec_attn_fwd (its Tk then
+ * has no upper limit).
  * dropout_mode 0 none, 1 replay dropout_mask [B*H, T, T], 2 draw it (Philox) and store it.
  * ctx [T, B, E]; out [T, B, E] (NULL together with w_out in the compact form).
  * dtype NMTG_F16 or NMTG_BF16 (the reference is fp16 only); T <= 4096.

@@ -243,7 +243,7 @@ extern "C" int nmtg_self_attn_fwd(const void* x, const void* w_in, const void* w
                                   uint64_t offset, void* ctx, void* out, int64_t t, int64_t b, int64_t e, int heads,
                                   int dtype, void* stream) {
   if (int rc = check_attn("self_attn_fwd", t, t, b, e, heads, dtype)) return rc;
-  NMTG_REQUIRE(lin && dropped && ctx, "self_attn_fwd: null buffer");
+  NMTG_REQUIRE(lin && ctx && (dropped || !scores), "self_attn_fwd: null buffer");
   NMTG_REQUIRE(mask_kind >= 0 && mask_kind <= 2 && (mask_kind == 0 || mask != nullptr), "self_attn_fwd: bad mask arguments");
   NMTG_REQUIRE((x == nullptr) == (w_in == nullptr), "self_attn_fwd: x and w_in go together (both NULL = compact form)");
   NMTG_REQUIRE((out == nullptr) == (w_out == nullptr), "self_attn_fwd: out and w_out go together (both NULL = compact form)");
@@ -317,7 +317,7 @@ extern "C" int nmtg_encdec_attn_fwd(const void* x_q, const void* x_kv, const voi
                                     void* ctx, void* out, int64_t tq, int64_t tk, int64_t b, int64_t e, int heads,
                                     int dtype, void* stream) {
   if (int rc = check_attn("encdec_attn_fwd", tq, tk, b, e, heads, dtype)) return rc;
-  NMTG_REQUIRE(q_lin && kv_lin && dropped && ctx, "encdec_attn_fwd: null buffer");
+  NMTG_REQUIRE(q_lin && kv_lin && ctx && (dropped || !scores), "encdec_attn_fwd: null buffer");
   NMTG_REQUIRE((x_q == nullptr) == (w_q == nullptr) && (x_kv == nullptr) == (w_kv == nullptr),
                "encdec_attn_fwd: an input and its weight go together (both NULL = projection done by the caller)");
   NMTG_REQUIRE((out == nullptr) == (w_out == nullptr), "encdec_attn_fwd: out and w_out go together");

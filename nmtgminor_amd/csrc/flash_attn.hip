@@ -860,7 +860,7 @@ __global__ __launch_bounds__(FA_THREADS * G, (D == 64 && G == 1) ? 2 : 1) void a
   __syncthreads();
   T* prow = static_cast<T*>(a.probs) + (static_cast<int64_t>(b) * a.heads + h) * a.tq * a.tk;
   // the tiles behind the last live key: zeros, no arithmetic (every wavefront of the block takes its share of them)
-  for (int t = live_tiles + group; t < ntiles; t += G) {
+  for (int t = live_tiles + group; a.probs != nullptr && t < ntiles; t += G) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int row = q0 + 32 * wave + 4 * j + (lane >> 4), key = t * FA_TILE + 4 * (lane & 15);
@@ -882,16 +882,19 @@ __global__ __launch_bounds__(FA_THREADS * G, (D == 64 && G == 1) ? 2 : 1) void a
       for (int n = 0; n < 2; ++n)
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[n][r] = fast_exp2(__builtin_fmaf(s[n][r], FA_LOG2E, -m2)) * inv;
-      // this lane's 4-key groups into the wavefront's strip: row = its query, 8 bytes per group
+      // this lane's 4-key groups into the wavefront's strip: row = its query, 8 bytes per group (a caller that does not
+      // want the probabilities passes no buffer for them)
+      if (a.probs != nullptr) {
 #pragma unroll
-      for (int n = 0; n < 2; ++n)
+        for (int n = 0; n < 2; ++n)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          uint2 w;
-          w.x = pack2<T>(s[n][4 * g + 0], s[n][4 * g + 1]);
-          w.y = pack2<T>(s[n][4 * g + 2], s[n][4 * g + 3]);
-          *reinterpret_cast<uint2*>(strip + (lane & 31) * PA_PITCH + (32 * n + 8 * g + 4 * half) * 2) = w;
-        }
+          for (int g = 0; g < 4; ++g) {
+            uint2 w;
+            w.x = pack2<T>(s[n][4 * g + 0], s[n][4 * g + 1]);
+            w.y = pack2<T>(s[n][4 * g + 2], s[n][4 * g + 3]);
+            *reinterpret_cast<uint2*>(strip + (lane & 31) * PA_PITCH + (32 * n + 8 * g + 4 * half) * 2) = w;
+          }
+      }
 #pragma unroll
       for (int kk = 0; kk < FA_TILE / 16; ++kk) {
         float pv[8];
@@ -901,17 +904,19 @@ __global__ __launch_bounds__(FA_THREADS * G, (D == 64 && G == 1) ? 2 : 1) void a
 #pragma unroll
         for (int i = 0; i < D / 32; ++i) mfma<T>::run(read_transposed<D>(vimg, i, kk, lane), pf, o[i]);
       }
-      wave_lds_fence();
-      // 16 lanes take one row's 64 keys (8 bytes each), four rows per step
+      if (a.probs != nullptr) {
+        wave_lds_fence();
+        // 16 lanes take one row's 64 keys (8 bytes each), four rows per step
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int r = 4 * j + (lane >> 4), key = t * FA_TILE + 4 * (lane & 15);
-        const int row = q0 + 32 * wave + r;
-        if (row < a.tq && key < a.tk)
-          *reinterpret_cast<uint2*>(prow + static_cast<int64_t>(row) * a.tk + key) =
-              *reinterpret_cast<const uint2*>(strip + r * PA_PITCH + 8 * (lane & 15));
+        for (int j = 0; j < 8; ++j) {
+          const int r = 4 * j + (lane >> 4), key = t * FA_TILE + 4 * (lane & 15);
+          const int row = q0 + 32 * wave + r;
+          if (row < a.tq && key < a.tk)
+            *reinterpret_cast<uint2*>(prow + static_cast<int64_t>(row) * a.tk + key) =
+                *reinterpret_cast<const uint2*>(strip + r * PA_PITCH + 8 * (lane & 15));
+        }
+        wave_lds_fence();
       }
-      wave_lds_fence();
     }
     if (t + G < live_tiles) {
       uint8_t* nk = tiles + ((it + 1) & 1) * 2 * IMG;

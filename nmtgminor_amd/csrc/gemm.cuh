@@ -1012,7 +1012,8 @@ bool gemm_skinny_ok(int dtype, int layout, int epi, const GemmArgs& a);
 int gemm_skinny_run(int dtype, const GemmArgs& a, hipStream_t st);
 
 // Attention probabilities and context of an inference call in one kernel (flash_attn.hip): probs [batch * heads, tq, tk]
-// = softmax over the keys of round(scale q k^T) with masked keys at -inf (rows without a live key: zeros), ctx = probs v.
+// = softmax over the keys of round(scale q k^T) with masked keys at -inf (rows without a live key: zeros), ctx = probs v;
+// probs may be null (context only).
 // The score tensor is never written. q, k, v, ctx: element (token t, sentence b, head h, :) at t * st + b * sb + h * sh.
 struct AttnProbsCall {
   const void *q, *k, *v;

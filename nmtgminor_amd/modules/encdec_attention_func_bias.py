@@ -25,7 +25,7 @@ class EncdecAttnBiasFunc(torch.autograd.Function):
         ctx.has_bias = (input_bias_q is not None, input_bias_kv is not None, output_bias is not None)
         q_lin, kv_lin, scores, dropped, dmask, ctx_t, outputs = native.forward(
             is_training, heads, inputs_q, inputs_kv, input_weights_q, input_weights_kv, output_weights, input_bias_q,
-            input_bias_kv, output_bias, mask, dropout_prob, dropout_mask=dropout_mask)
+            input_bias_kv, output_bias, mask, dropout_prob, dropout_mask=dropout_mask, want_probs=bool(return_coverage))
         if recompute:
             ctx.save_for_backward(inputs_q, inputs_kv, input_weights_q, input_weights_kv, output_weights, input_bias_q,
                                   input_bias_kv, mask, dmask)

@@ -25,7 +25,7 @@ def _shapes(q3, kv3, heads, kv_last):
 
 
 def _fwd(is_training, heads, x_q, x_kv, w_q, w_kv, w_out, b_q, b_kv, b_out, q_lin, kv_lin, pad_mask, p, dropout_mask,
-         tq, tk, b, e, dev, dt, softmax_out=None):
+         tq, tk, b, e, dev, dt, softmax_out=None, want_probs=True):
     km, kind = A.mask_arg(pad_mask, False, b, tq, tk)
     bh = b * heads
     if q_lin is None:
@@ -34,14 +34,16 @@ def _fwd(is_training, heads, x_q, x_kv, w_q, w_kv, w_out, b_q, b_kv, b_out, q_li
         kv_lin = torch.empty(tk, b, 2 * e, dtype=dt, device=dev)
     keep_scores = softmax_out is not None or A.scores_needed(is_training, dt, e // heads, tk)
     scores = torch.empty((bh, tq, tk) if keep_scores else (0,), dtype=dt, device=dev)
-    dropped = torch.empty(bh, tq, tk, dtype=dt, device=dev)
+    keep_probs = want_probs or keep_scores
+    dropped = torch.empty((bh, tq, tk) if keep_probs else (0,), dtype=dt, device=dev)
     ctx = torch.empty(tq, b, e, dtype=dt, device=dev)
     out = torch.empty(tq, b, e, dtype=dt, device=dev) if w_out is not None else None
     dmask, mode, seed, offset = A.dropout_args(is_training, p, (bh, tq, tk), dev, dropout_mask)
     if tq == 0 or b == 0:       # an empty batch / no query position: the (empty) buffers are the result
         return q_lin, kv_lin, scores, dropped, dmask, ctx, out
     L.call("nmtg_encdec_attn_fwd", L.ptr(x_q), L.ptr(x_kv), L.ptr(w_q), L.ptr(w_kv), L.ptr(w_out), L.ptr(b_q), L.ptr(b_kv),
-           L.ptr(b_out), L.ptr(km), L.ptr(q_lin), L.ptr(kv_lin), L.ptr(scores if keep_scores else None), L.ptr(softmax_out), L.ptr(dropped),
+           L.ptr(b_out), L.ptr(km), L.ptr(q_lin), L.ptr(kv_lin), L.ptr(scores if keep_scores else None), L.ptr(softmax_out),
+           L.ptr(dropped if keep_probs else None),
            L.ptr(dmask if mode else None), L.i32(mode), L.f32(p), A.u64(seed), A.u64(offset), L.ptr(ctx), L.ptr(out),
            L.i64(tq), L.i64(tk), L.i64(b), L.i64(e), L.i32(heads), L.i32(L.dtype_code(ctx)), L.stream_of(ctx))
     return q_lin, kv_lin, scores, dropped, dmask, ctx, out
@@ -73,10 +75,10 @@ def _fwd_padded_keys(heads, x_q, x_kv, w_q, w_kv, w_out, b_q, b_kv, b_out, pad_m
 
 
 def forward(is_training, heads, inputs_q, inputs_kv, input_weights_q, input_weights_kv, output_weights, input_biases_q,
-            input_biases_kv, output_biases, pad_mask, dropout_prob, *, dropout_mask=None):
+            input_biases_kv, output_biases, pad_mask, dropout_prob, *, dropout_mask=None, want_probs=True):
     """-> [input_lin_q_results, input_lin_kv_results, attn_scores, dropout_results, dropout_mask,
     matmul2_results, outputs]; attn_scores is empty for an inference call under torch.no_grad() (see
-    _attn_common.scores_needed)."""
+    _attn_common.scores_needed), and so is dropout_results when such a call says want_probs=False."""
     tensors = (inputs_q, inputs_kv, input_weights_q, input_weights_kv, output_weights, input_biases_q, input_biases_kv,
                output_biases)
     L.require_cuda(*tensors, pad_mask, dropout_mask)
@@ -93,7 +95,7 @@ def forward(is_training, heads, inputs_q, inputs_kv, input_weights_q, input_weig
                                 c(input_biases_q), c(input_biases_kv), c(output_biases), pad_mask, tq, tk, b, e)
     return list(_fwd(is_training, heads, c(inputs_q), c(inputs_kv), c(input_weights_q), c(input_weights_kv),
                      c(output_weights), c(input_biases_q), c(input_biases_kv), c(output_biases), None, None, pad_mask,
-                     dropout_prob, dropout_mask, tq, tk, b, e, inputs_q.device, inputs_q.dtype))
+                     dropout_prob, dropout_mask, tq, tk, b, e, inputs_q.device, inputs_q.dtype, want_probs=want_probs))
 
 
 def forward_compact(is_training, heads, input_lin_q_results, input_lin_kv_results, pad_mask, dropout_prob, *,

@@ -19,9 +19,10 @@ def _dims(inputs, heads, last):
 
 
 def forward(use_time_mask, is_training, heads, inputs, input_weights, output_weights, input_biases, output_biases,
-            pad_mask, dropout_prob, *, dropout_mask=None):
+            pad_mask, dropout_prob, *, dropout_mask=None, want_probs=True):
     """-> [input_lin_results, attn_scores, dropout_results, dropout_mask, matmul2_results, outputs]; attn_scores is empty
-    for an inference call under torch.no_grad() (see _attn_common.scores_needed)."""
+    for an inference call under torch.no_grad() (see _attn_common.scores_needed); such a call with want_probs=False
+    (the caller does not return the coverage) leaves dropout_results empty too: no [B*H, T, T] tensor exists then."""
     L.require_cuda(inputs, input_weights, output_weights, input_biases, output_biases, pad_mask, dropout_mask)
     A.check(input_weights.dim() == 2 and output_weights.dim() == 2, "expected 2D tensor")
     A.check_half(inputs, input_weights, output_weights, input_biases, output_biases)
@@ -37,14 +38,15 @@ def forward(use_time_mask, is_training, heads, inputs, input_weights, output_wei
     lin = torch.empty(t, b, 3 * e, dtype=dt, device=dev)
     keep_scores = A.scores_needed(is_training, dt, e // heads, t)
     scores = torch.empty((bh, t, t) if keep_scores else (0,), dtype=dt, device=dev)
-    dropped = torch.empty(bh, t, t, dtype=dt, device=dev)
+    keep_probs = want_probs or keep_scores
+    dropped = torch.empty((bh, t, t) if keep_probs else (0,), dtype=dt, device=dev)
     ctx = torch.empty(t, b, e, dtype=dt, device=dev)
     out = torch.empty(t, b, e, dtype=dt, device=dev)
     dmask, mode, seed, offset = A.dropout_args(is_training, dropout_prob, (bh, t, t), dev, dropout_mask)
     if t == 0 or b == 0:        # an empty batch: the (empty) buffers are the result
         return [lin, scores, dropped, dmask, ctx, out]
     L.call("nmtg_self_attn_fwd", L.ptr(x), L.ptr(w_in), L.ptr(w_out), L.ptr(b_in), L.ptr(b_out), L.ptr(km), L.i32(kind),
-           L.ptr(lin), L.ptr(scores if keep_scores else None), L.ptr(None), L.ptr(dropped), L.ptr(dmask if mode else None), L.i32(mode),
+           L.ptr(lin), L.ptr(scores if keep_scores else None), L.ptr(None), L.ptr(dropped if keep_probs else None), L.ptr(dmask if mode else None), L.i32(mode),
            L.f32(dropout_prob), A.u64(seed), A.u64(offset), L.ptr(ctx), L.ptr(out), L.i64(t), L.i64(b), L.i64(e),
            L.i32(heads), L.i32(L.dtype_code(x)), L.stream_of(x))
     return [lin, scores, dropped, dmask, ctx, out]

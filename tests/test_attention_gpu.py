@@ -374,3 +374,34 @@ def test_inference_keeps_the_score_tensor_where_the_one_kernel_path_does_not_app
     with torch.no_grad():
         r = sa_native.forward(False, False, 2, g("x"), g("w_in"), g("w_out"), g("b_in"), g("b_out"), g("pad_mask"), 0.0)
     assert r[1].shape == (4, 64, 64)
+
+
+@pytest.mark.parametrize("split", ["0", "1"])
+def test_inference_without_coverage_writes_no_probability_tensor(dev, monkeypatch, split):
+    """A caller that does not return the coverage (return_coverage=False) gets the same outputs from an inference call
+    under torch.no_grad(), and neither the scores nor the probabilities exist as tensors."""
+    monkeypatch.setenv("NMTG_ATTN_PROBS_SPLIT", split)
+    dtype, h = torch.bfloat16, 4
+    d = inputs.self_attn_inputs(136, 2, 256, h, dtype, p=0.0, seed=77)
+    g = lambda k: d[k].to(dev)
+    args = (False, False, h, g("x"), g("w_in"), g("w_out"), g("b_in"), g("b_out"), g("pad_mask"), 0.0)
+    with torch.no_grad():
+        full = sa_native.forward(*args)
+        lean = sa_native.forward(*args, want_probs=False)
+        out_func, cov_func = self_attn_func(False, False, h, g("x"), g("w_in"), g("w_out"), g("b_in"), g("b_out"), g("pad_mask"), 0.0,
+                                            False, None, False, None, False, False, False)
+    assert lean[1].numel() == 0 and lean[2].numel() == 0 and full[2].shape == (2 * h, 136, 136)
+    assert torch.equal(lean[4], full[4]) and torch.equal(lean[5], full[5]) and torch.equal(out_func, full[5]) and cov_func.numel() == 0
+    e = inputs.encdec_attn_inputs(40, 300, 2, 256, h, dtype, p=0.0, seed=78)
+    ge = lambda k: e[k].to(dev)
+    eargs = (False, h, ge("x_q"), ge("x_kv"), ge("w_q"), ge("w_kv"), ge("w_out"), ge("b_q"), ge("b_kv"), ge("b_out"), ge("pad_mask"), 0.0)
+    with torch.no_grad():
+        full = ed_native.forward(*eargs)
+        lean = ed_native.forward(*eargs, want_probs=False)
+        res = encdec_attn_bias_func(False, False, h, ge("x_q"), ge("x_kv"), ge("w_q"), ge("w_kv"), ge("w_out"), ge("b_q"), ge("b_kv"),
+                                    ge("b_out"), ge("pad_mask"), 0.0, False, None, False, None, None, False, False)
+    assert lean[2].numel() == 0 and lean[3].numel() == 0 and torch.equal(lean[6], full[6])
+    assert torch.equal(res[0] if isinstance(res, tuple) else res, full[6])
+    # recorded by autograd (or in training mode) the tensors are kept whatever the caller asks for
+    kept = sa_native.forward(*args, want_probs=False)
+    assert kept[1].shape == (2 * h, 136, 136) and kept[2].shape == (2 * h, 136, 136)
