@@ -379,8 +379,8 @@ def test_attention_inference_without_the_score_tensor(mi355x, monkeypatch, split
     tat.test_self_attention_inference_without_the_score_tensor(CPU, monkeypatch, F16, 72, 2, 256, 2, True, split)
     tat.test_encdec_attention_inference_without_the_score_tensor(CPU, monkeypatch, BF16, 17, 100, 3, 128, 2, True, split)
     tat.test_encdec_attention_inference_without_the_score_tensor(CPU, monkeypatch, F16, 5, 260, 1, 128, 1, True, split)
-    tat.test_inference_keeps_the_score_tensor_where_the_one_kernel_path_does_not_apply(CPU, monkeypatch)
     tat.test_inference_without_coverage_writes_no_probability_tensor(CPU, monkeypatch, split)
+    tat.test_inference_keeps_the_score_tensor_where_the_one_kernel_path_does_not_apply(CPU, monkeypatch)   # sets a switch: last
 
 
 def test_encdec_attention_without_biases_compact_and_modules(mi355x):
