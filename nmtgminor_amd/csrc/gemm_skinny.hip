@@ -3,84 +3,63 @@
 // calls like any other linear layer (onmt/modules/extensions/mlp_blaslt/linear.cpp:142-144).
 //
 // With so few rows the product is a read of W: 2 MB of weight against 64 KB of activations, and a 128 x 128 output
-// tile leaves all but eight compute units idle while each of those walks the whole reduction. Here every wavefront
-// owns one output column: its 64 lanes read the column's weight row with 16-byte loads, 16 elements per lane and
-// 1024-element chunk of k, and multiply them with the same k-elements of all 32 activation rows, which the block
-// stages in LDS once per chunk (64 KB); 32 wavefront reductions then leave row m's sum in lane m. A block of four
-// wavefronts covers four columns, so a [1024 x 1024] weight spreads over 256 blocks.
+// tile leaves all but eight compute units idle while each of those walks the whole reduction. What counts is the
+// latency of one block, so the reduction is spread over the wavefronts of a block instead: a block owns 32 output
+// columns and all (at most 32) rows, its eight wavefronts each take an eighth of k, load their slices of X and W
+// straight into matrix-core operand layout (a lane's 16 bytes of its row: no LDS staging, every load of a 128-k chunk in
+// flight at once), run v_mfma_f32_32x32x16 over them, and leave their 32 x 32 partial sums in LDS, where the block adds
+// the eight of them up in a fixed order. A [1024 x 1024] weight is 32 blocks of one load latency each.
 #include "gemm.cuh"
 
 namespace nmtg {
 namespace {
 
-constexpr int SK_ROWS = 32, SK_CHUNK = 1024, SK_THREADS = 256;
+constexpr int SK_ROWS = 32, SK_COLS = 32, SK_WAVES = 8, SK_THREADS = 64 * SK_WAVES, SK_CHUNK = 128;
 
 template <typename T>
 __global__ __launch_bounds__(SK_THREADS) void gemm_skinny_kernel(const GemmArgs g) {
-  extern __shared__ __align__(16) uint8_t lds_raw[];
-  T* xs = reinterpret_cast<T*>(lds_raw);                 // [32][SK_CHUNK]
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int n = static_cast<int>(blockIdx.x) * (SK_THREADS / 64) + wave;
+  __shared__ float part[SK_WAVES][16][64];               // partial tiles in accumulator layout
+  const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n0 = static_cast<int>(blockIdx.x) * SK_COLS;
   const T* X = static_cast<const T*>(g.A);
   const T* W = static_cast<const T*>(g.B);
-  float acc[SK_ROWS];
+  // this wavefront's share of k: whole 16-k steps, dealt out in chunks of 128 so that the loads in flight stay bounded
+  const int steps = (g.K + 15) / 16, per = (steps + SK_WAVES - 1) / SK_WAVES;
+  const int k_begin = wave * per * 16, k_end = min(g.K, (wave + 1) * per * 16);
+  const int m = lane & 31, n = n0 + (lane & 31);
+  const T* xrow = X + static_cast<int64_t>(m) * g.lda + 8 * half;
+  const T* wrow = W + static_cast<int64_t>(n) * g.ldb + 8 * half;
+  acc16_t acc;
 #pragma unroll
-  for (int m = 0; m < SK_ROWS; ++m) acc[m] = 0.f;
-
-  for (int k0 = 0; k0 < g.K; k0 += SK_CHUNK) {
-    const int kc = min(SK_CHUNK, g.K - k0);              // a multiple of 8
-    // the column's weights of this chunk: lane l holds k0 + 16 l .. + 15 (two 16-byte loads), zeros past the end
-    pack<T, 8> wraw[2];
+  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+  for (int k0 = k_begin; k0 < k_end; k0 += SK_CHUNK) {
+    uint4 xf[SK_CHUNK / 16], wf[SK_CHUNK / 16];
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int k = 16 * lane + 8 * u;
-      wraw[u] = pack<T, 8>{};
-      if (n < g.N && k < kc) wraw[u] = load_raw<T, 8>(W + static_cast<int64_t>(n) * g.ldb + k0 + k);
+    for (int s = 0; s < SK_CHUNK / 16; ++s) {
+      const int k = k0 + 16 * s + 8 * half;               // K is a multiple of 8: a lane's 8 elements are all in or all out
+      const bool in = k < k_end;
+      xf[s] = in && m < g.M ? *reinterpret_cast<const uint4*>(xrow + k0 + 16 * s) : make_uint4(0, 0, 0, 0);
+      wf[s] = in && n < g.N ? *reinterpret_cast<const uint4*>(wrow + k0 + 16 * s) : make_uint4(0, 0, 0, 0);
     }
-    // the chunk of X: all loads in flight before the first LDS store (16 per lane)
-    constexpr int PER = SK_ROWS * (SK_CHUNK / 8) / SK_THREADS;
-    pack<T, 8> xraw[PER];
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      // every block needs the same rows: each starts at another one, so that at any moment the blocks ask the L2 for
-      // different lines instead of all for the same
-      const int id = (tid + SK_THREADS * (i + static_cast<int>(blockIdx.x))) % (SK_ROWS * (SK_CHUNK / 8));
-      const int m = id / (SK_CHUNK / 8), k = 8 * (id % (SK_CHUNK / 8));
-      xraw[i] = pack<T, 8>{};
-      if (m < g.M && k < kc) xraw[i] = load_raw<T, 8>(X + static_cast<int64_t>(m) * g.lda + k0 + k);
-    }
-    if (k0 > 0) __syncthreads();                         // the previous chunk has been consumed
-#pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int id = (tid + SK_THREADS * (i + static_cast<int>(blockIdx.x))) % (SK_ROWS * (SK_CHUNK / 8));
-      *reinterpret_cast<pack<T, 8>*>(xs + (id / (SK_CHUNK / 8)) * SK_CHUNK + 8 * (id % (SK_CHUNK / 8))) = xraw[i];
-    }
-    __syncthreads();
-    uint32_t wv[8];
-    __builtin_memcpy(wv, &wraw[0], 16);
-    __builtin_memcpy(wv + 4, &wraw[1], 16);
-#pragma unroll
-    for (int m = 0; m < SK_ROWS; ++m) {
-      const uint4 x0 = *reinterpret_cast<const uint4*>(xs + m * SK_CHUNK + 16 * lane);
-      const uint4 x1 = *reinterpret_cast<const uint4*>(xs + m * SK_CHUNK + 16 * lane + 8);
-      const uint32_t xv[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
-      float s = acc[m];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) s = dot2<T>(xv[e], wv[e], s);
-      acc[m] = s;
-    }
+    for (int s = 0; s < SK_CHUNK / 16; ++s) mfma<T>::run(xf[s], wf[s], acc);   // acc[r], lane (j, half): row 8 (r / 4) + 4 half + r % 4, column j
   }
-  // row m's sum over the wavefront ends in lane m
-  float mine = 0.f;
 #pragma unroll
-  for (int m = 0; m < SK_ROWS; ++m) {
-    const float s = wave_sum(acc[m]);
-    if (lane == m) mine = s;
-  }
-  if (lane < g.M && n < g.N) {
-    float v = mine * g.alpha;
-    if (g.bias != nullptr) v += elem<T>::to_float(static_cast<const T*>(g.bias)[n]);
-    static_cast<T*>(g.C)[static_cast<int64_t>(lane) * g.ldc + n] = elem<T>::from_float(v);
+  for (int r = 0; r < 16; ++r) part[wave][r][lane] = acc[r];
+  __syncthreads();
+  // 1024 outputs, two per thread; the eight partial sums are added in wavefront order
+  for (int o = tid; o < 16 * 64; o += SK_THREADS) {
+    const int r = o >> 6, l = o & 63;
+    float v = 0.f;
+#pragma unroll
+    for (int w = 0; w < SK_WAVES; ++w) v += part[w][r][l];
+    const int row = 8 * (r / 4) + 4 * (l >> 5) + r % 4, col = n0 + (l & 31);
+    if (row < g.M && col < g.N) {
+      v *= g.alpha;
+      if (g.bias != nullptr) v += elem<T>::to_float(static_cast<const T*>(g.bias)[col]);
+      static_cast<T*>(g.C)[static_cast<int64_t>(row) * g.ldc + col] = elem<T>::from_float(v);
+    }
   }
 }
 
@@ -96,11 +75,10 @@ bool gemm_skinny_ok(int dtype, int layout, int epi, const GemmArgs& a) {
 }
 
 int gemm_skinny_run(int dtype, const GemmArgs& a, hipStream_t st) {
-  const unsigned grid = static_cast<unsigned>((a.N + SK_THREADS / 64 - 1) / (SK_THREADS / 64));
-  const int lds = SK_ROWS * SK_CHUNK * 2;
+  const unsigned grid = static_cast<unsigned>((a.N + SK_COLS - 1) / SK_COLS);
   TraceScope trace("gemm_nt_skinny", st);
-  if (dtype == NMTG_F16) hipLaunchKernelGGL((gemm_skinny_kernel<f16_t>), dim3(grid), dim3(SK_THREADS), lds, st, a);
-  else hipLaunchKernelGGL((gemm_skinny_kernel<bf16_t>), dim3(grid), dim3(SK_THREADS), lds, st, a);
+  if (dtype == NMTG_F16) hipLaunchKernelGGL((gemm_skinny_kernel<f16_t>), dim3(grid), dim3(SK_THREADS), 0, st, a);
+  else hipLaunchKernelGGL((gemm_skinny_kernel<bf16_t>), dim3(grid), dim3(SK_THREADS), 0, st, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(NMTG_ERR_LAUNCH, "gemm: launch failed: %s", hipGetErrorString(e));
   return 0;

@@ -106,8 +106,8 @@ def on_the_cpu(hostsim_lib, monkeypatch):
     # elementwise kernels: few compute units, so that grid-stride loops make several trips and last groups are partial
     monkeypatch.setenv("HOSTSIM_CUS", "2")
     monkeypatch.delenv("HOSTSIM_DMA", raising=False)
-    # products with few rows stay on the tiled kernels here: the one-column-per-wavefront kernel costs the simulator a
-    # block of 256 fibers per four output columns; it has its own test below
+    # products with few rows stay on the tiled kernels here (the few-row kernel has its own test below), so that the
+    # layers' small test shapes keep exercising the tiled kernels' edge handling
     monkeypatch.setenv("NMTG_GEMM_SKINNY", "0")
 
 

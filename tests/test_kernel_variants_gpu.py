@@ -288,7 +288,7 @@ def test_few_row_products_match_the_tiled_kernels(dev, dtype, m, n, k):
     with off("NMTG_GEMM_SKINNY"):
         tiled = gemm(x, w, False, True, alpha=0.5, bias=bias)
     want = 0.5 * (x.double() @ w.double().t()).cpu() + bias.double().cpu()
-    assert_close(got, want, dtype, "one column per wavefront")
+    assert_close(got, want, dtype, "few-row kernel")
     assert_close(tiled, want, dtype, "tiled")
     pitched = torch.full((m, k + 24), float("nan"), dtype=dtype, device=dev)      # rows with a pitch, NaN in the padding
     pitched[:, :k] = x
