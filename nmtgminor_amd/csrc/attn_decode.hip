@@ -47,7 +47,7 @@ __global__ __launch_bounds__(DEC_THREADS) void attn_decode_kernel(DecArgs a) {
   extern __shared__ __align__(16) float lds[];
   float* sc = lds;                       // [tk]
   float* red = lds + a.tk;               // [4] + [4][8 * LPR]
-  constexpr int D = 8 * LPR, RPS = DEC_THREADS / LPR, U = 4;
+  constexpr int D = 8 * LPR, RPS = DEC_THREADS / LPR, U = 8;   // U loads of 16 bytes in flight per lane
   const int bh = blockIdx.x, b = bh / a.heads, h = bh % a.heads;
   const int tid = threadIdx.x, slot = tid / LPR, c = tid % LPR;
   const int64_t head_off = static_cast<int64_t>(h) * D + 8 * c;
