@@ -1,5 +1,5 @@
 // Library-wide plumbing of libnmtg_hip.so: version, per-thread error text, device facts.
-#include "common.cuh"
+#include "common.hip.h"
 #include <mutex>
 
 namespace nmtg {

@@ -16,7 +16,7 @@
 // the key-padding / time mask is applied in the epilogue of the Q K^T product (no separate
 // masked_fill pass over the [B*H, Tq, Tk] tensor); bias gradients are column-sum kernels with a
 // fixed reduction order; weight gradients split the token dimension over the chip.
-#include "gemm.cuh"
+#include "gemm.hip.h"
 #include <cstdlib>
 #include <algorithm>
 

@@ -9,7 +9,7 @@
 // whole row in LDS, normalises them, writes the probabilities (the reference returns them as coverage) and accumulates
 // the context from the values in a second pass. Rounding points as on the GEMM path: scores and probabilities are
 // rounded to the 16-bit type where that path stores them.
-#include "common.cuh"
+#include "common.hip.h"
 
 namespace nmtg {
 namespace {

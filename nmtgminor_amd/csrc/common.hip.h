@@ -11,7 +11,7 @@
 #include <cstdlib>
 
 #include "../../include/nmtg_hip.h"
-#include "trace.cuh"
+#include "trace.hip.h"
 
 namespace nmtg {
 

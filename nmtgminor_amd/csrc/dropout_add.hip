@@ -9,7 +9,7 @@
 // Bandwidth bound: forward reads x and residual, writes x and 1 B/element of mask; backward
 // reads g and the mask, writes dx. Each lane moves 16 bytes per access; the grid covers the
 // tensor once (no grid-stride tail) so every CU streams contiguous 4 KiB wavefront chunks.
-#include "common.cuh"
+#include "common.hip.h"
 
 namespace nmtg {
 namespace {

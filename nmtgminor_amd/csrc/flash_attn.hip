@@ -24,7 +24,7 @@
 // of the two keys that a register holds in the two halves of the wavefront IS the lane mask of a select: it is loaded
 // into scalar registers and costs no vector instruction besides the select. The key-major kernel (dK / dV) loads its
 // key's word per group of queries and tests bits. An explicit byte mask is turned into the same words.
-#include "gemm.cuh"
+#include "gemm.hip.h"
 
 namespace nmtg {
 namespace {

@@ -1,6 +1,6 @@
 // Host side of the MFMA GEMM core: tile / split selection, alignment analysis, the column-sum
 // (bias gradient) helpers and the stand-alone C entry point nmtg_gemm.
-#include "gemm_inst.cuh"
+#include "gemm_inst.hip.h"
 #include <algorithm>
 #include <cstdlib>
 #include <mutex>

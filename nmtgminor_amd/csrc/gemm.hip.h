@@ -26,8 +26,8 @@
 //   * blockIdx.x is remapped so that each of the 8 XCDs (which receive consecutive block ids
 //     round-robin) works on a contiguous run of tiles and re-uses A / B through its own L2.
 #pragma once
-#include "common.cuh"
-#include "reduce.cuh"
+#include "common.hip.h"
+#include "reduce.hip.h"
 #include <type_traits>
 
 namespace nmtg {
@@ -63,7 +63,7 @@ struct GemmArgs {
   float alpha;
   int vec;                  // widest access (elements: 8, 4 or 1) every operand and extent allows
   int dma;                  // every 64-k step of every split is full: direct-to-LDS loads allowed
-  int ring;                 // the call meets the requirements of the slot-ring kernel (gemm_ring.cuh)
+  int ring;                 // the call meets the requirements of the slot-ring kernel (gemm_ring.hip.h)
   const void* bias;
   void* aux_out;
   void* out2;               // EPI_SCORES_SOFTMAX: dropped probabilities, laid out like C

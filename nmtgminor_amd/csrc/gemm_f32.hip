@@ -13,7 +13,7 @@
 // fp32 is the reference's checking precision, not its training precision: this kernel is written to be exact (fp32
 // products and sums in the matrix core, no re-association across blocks: no split-K) and simple, not to reach the fp32
 // MFMA roof.
-#include "gemm.cuh"
+#include "gemm.hip.h"
 
 namespace nmtg {
 namespace {

@@ -5,13 +5,13 @@
 //   S: 256x64  tile, 4x1 wavefronts (each 64x64),  256 threads  — N <= 64 (per-head attention products)
 //   R: 128x512 tile, 4x2 wavefronts (each 32x256), 512 threads  — whole score rows (fused softmax epilogue only)
 #pragma once
-#include "gemm.cuh"
-#include "gemm_ring.cuh"
+#include "gemm.hip.h"
+#include "gemm_ring.hip.h"
 #include <string>
 
 namespace nmtg {
 
-// GemmTile and tile_cfg<TILE> (block tile and wavefront grid of each tile) live in reduce.cuh: the reduction kernels need them too.
+// GemmTile and tile_cfg<TILE> (block tile and wavefront grid of each tile) live in reduce.hip.h: the reduction kernels need them too.
 
 inline void tile_dims(int tile, int& bm, int& bn) {
   if (tile == TILE_L) { bm = 256; bn = 256; }
@@ -45,7 +45,7 @@ int gemm_launch_vec(const GemmArgs& a, hipStream_t st) {
 }
 
 
-// Slot-ring kernel (gemm_ring.cuh): the 256x256 tile owns the whole LDS (10 slots), the 128x128
+// Slot-ring kernel (gemm_ring.hip.h): the 256x256 tile owns the whole LDS (10 slots), the 128x128
 // tile takes 5 slots so that two blocks share a CU and one block's epilogue overlaps the other's
 // main loop.
 template <int TILE> struct ring_slots { static constexpr int value = TILE == TILE_M ? 5 : 10; };

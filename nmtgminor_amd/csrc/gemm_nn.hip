@@ -1,6 +1,6 @@
 // GEMM instantiations for A [M][K] reduction-contiguous, B [K][N] (row index contiguous):
 // data gradients dX = dY W, P V, dQ = dS K.
-#include "gemm_inst.cuh"
+#include "gemm_inst.hip.h"
 namespace nmtg {
 #define CASE(TILE, EPI) if (tile == TILE && epi == EPI) return gemm_launch_one<T, TILE, true, false, EPI>(a, st);
 template <typename T> static int run(int tile, int epi, const GemmArgs& a, hipStream_t st) {

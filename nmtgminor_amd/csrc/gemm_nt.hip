@@ -1,6 +1,6 @@
 // GEMM instantiations for A [M][K], B [N][K] (both reduction-contiguous): forward linears,
 // Q K^T scores, dP = dC V^T.
-#include "gemm_inst.cuh"
+#include "gemm_inst.hip.h"
 namespace nmtg {
 #define CASE(TILE, EPI) if (tile == TILE && epi == EPI) return gemm_launch_one<T, TILE, true, true, EPI>(a, st);
 template <typename T> static int run(int tile, int epi, const GemmArgs& a, hipStream_t st) {

@@ -1,7 +1,7 @@
 // GEMM main loop fed by a ring of LDS slots that the gfx950 direct global -> LDS loads fill several
 // 64-k steps ahead of the MFMA work.
 //
-// Why a second main loop: with one 64-k step of prefetch (the two-buffer loop in gemm.cuh) a step
+// Why a second main loop: with one 64-k step of prefetch (the two-buffer loop in gemm.hip.h) a step
 // cannot be shorter than the latency of its own loads (~2000 clocks on a loaded chip), while the
 // MFMA work of a 128x128 step is 256 clocks and that of a 256x256 step 2048. Keeping several steps
 // in flight turns the loads from a latency into a throughput problem (measured: ~44 B/clk/CU from L2
@@ -31,7 +31,7 @@
 // elements, K a multiple of 64 per split, 16-byte aligned operands and leading dimensions, operand
 // extents below 4 GB (32-bit lane offsets).
 #pragma once
-#include "gemm.cuh"
+#include "gemm.hip.h"
 
 #include <type_traits>
 

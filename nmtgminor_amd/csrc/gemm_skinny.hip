@@ -9,7 +9,7 @@
 // straight into matrix-core operand layout (a lane's 16 bytes of its row: no LDS staging, every load of a 128-k chunk in
 // flight at once), run v_mfma_f32_32x32x16 over them, and leave their 32 x 32 partial sums in LDS, where the block adds
 // the eight of them up in a fixed order. A [1024 x 1024] weight is 32 blocks of one load latency each.
-#include "gemm.cuh"
+#include "gemm.hip.h"
 
 namespace nmtg {
 namespace {

@@ -1,6 +1,6 @@
 // GEMM instantiations for A [K][M], B [K][N] (both row-index contiguous): weight gradients
 // dW = dY^T X (split over the token dimension), dV = P^T dC, dK = dS^T Q.
-#include "gemm_inst.cuh"
+#include "gemm_inst.hip.h"
 namespace nmtg {
 #define CASE(TILE, EPI) if (tile == TILE && epi == EPI) return gemm_launch_one<T, TILE, false, false, EPI>(a, st);
 template <typename T> static int run(int tile, int epi, const GemmArgs& a, hipStream_t st) {

@@ -9,7 +9,7 @@
 //
 // Bandwidth bound: the forward reads 2 * inner and writes inner elements per row (+ 1 byte of mask per output when the
 // mask is drawn here), the backward reads 3 * inner and writes 2 * inner. Each lane moves 16 bytes per access.
-#include "gemm.cuh"
+#include "gemm.hip.h"
 
 namespace nmtg {
 namespace {

@@ -13,7 +13,7 @@
 //   forward : read x, write z, +8 B (mu, rsigma)          -> 2 H elements
 //   backward: read dz, x, write dx, +8 B                  -> 3 H elements (+ the [n_part, H]
 //             fp32 partials once written and once read)
-#include "common.cuh"
+#include "common.hip.h"
 #include <algorithm>
 
 namespace nmtg {

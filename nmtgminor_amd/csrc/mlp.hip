@@ -14,7 +14,7 @@
 //             layer's bias.
 // The reference runs a GEMM and then separate element-wise kernels over the [tokens, inner]
 // tensors; here those tensors cross HBM once per direction.
-#include "gemm.cuh"
+#include "gemm.hip.h"
 #include <algorithm>
 #include <cstdlib>
 #include <vector>

@@ -12,7 +12,7 @@
 // 16-byte accesses whenever a tensor's pointers are 16-byte aligned (chunks start on multiples of 32768 elements), with
 // four loads in flight per lane in the Adam pass. fp32 arithmetic whatever the storage type. The norm is deterministic:
 // one partial per block, then fixed-order sums.
-#include "common.cuh"
+#include "common.hip.h"
 
 #include <algorithm>
 #include <cmath>

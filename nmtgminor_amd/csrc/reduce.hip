@@ -1,5 +1,5 @@
 // Column sums out[n] = sum_m X[m][n] (bias gradients): partial sums per row block, then a fixed-order final sum.
-#include "reduce.cuh"
+#include "reduce.hip.h"
 #include <algorithm>
 
 namespace nmtg {

@@ -1,12 +1,12 @@
 // Small fixed-order reduction kernels that follow a GEMM: the sum over split-K partials and the column sums behind
 // every bias gradient. They are latency-bound (a few blocks, short dependent chains), so each keeps a batch of loads
-// in flight before the first add. Hosts: reduce.hip (column sums), gemm_inst.cuh (split-K).
+// in flight before the first add. Hosts: reduce.hip (column sums), gemm_inst.hip.h (split-K).
 #pragma once
-#include "common.cuh"
+#include "common.hip.h"
 
 namespace nmtg {
 
-// Sums the split-K partials (in the accumulator layout the GEMM kernels' split-K epilogue writes, gemm.cuh), scales, converts to T and
+// Sums the split-K partials (in the accumulator layout the GEMM kernels' split-K epilogue writes, gemm.hip.h), scales, converts to T and
 // writes row-major C; fixed summation order.
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N>
 __device__ __forceinline__ void splitk_reduce_slot(int64_t idx, const float* __restrict__ ws, T* __restrict__ C, int64_t ldc,

@@ -13,7 +13,7 @@
 // the shifted operand is read element by element (coalesced across the lanes of a wavefront) while the operand that
 // keeps its place moves in 16-byte accesses. All three kernels are bandwidth bound: one read of each operand, one
 // write of the result.
-#include "common.cuh"
+#include "common.hip.h"
 
 namespace nmtg {
 namespace {

@@ -12,7 +12,7 @@
 // The operand is addressed as x[t * stride_t + n * stride_n + part * stride_part + j]: the query and key slots of the
 // head-interleaved projection [T, B*H, 3, D] are two parts of one launch. One thread owns EPV pairs. Bandwidth bound:
 // one read and one write of the rotated slots.
-#include "common.cuh"
+#include "common.hip.h"
 
 namespace nmtg {
 namespace {

@@ -17,7 +17,7 @@
 // Bandwidth bound. Per element: forward reads the score (+1 B mask in replay mode), writes the
 // result (+1 B mask in RNG mode); backward reads grad, the saved scores or probabilities and the
 // mask byte, writes the score gradient.
-#include "common.cuh"
+#include "common.hip.h"
 
 namespace nmtg {
 namespace {

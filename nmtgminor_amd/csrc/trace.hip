@@ -1,6 +1,6 @@
 // Event-based kernel timing behind nmtg_trace_begin / nmtg_trace_end.
-#include "common.cuh"
-#include "trace.cuh"
+#include "common.hip.h"
+#include "trace.hip.h"
 #include <cstring>
 #include <algorithm>
 #include <atomic>

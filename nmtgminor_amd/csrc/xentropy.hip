@@ -17,7 +17,7 @@
 //
 // Bandwidth bound: forward reads N*V elements once; backward reads them once and writes N*V
 // (rows whose label is the padding index are written as zeros without reading the logits).
-#include "common.cuh"
+#include "common.hip.h"
 
 namespace nmtg {
 namespace {

@@ -32,7 +32,7 @@ LIB = os.path.join(BUILD, "libnmtg_hostsim_asan.so" if SANITIZE else "libnmtg_ho
 
 KERNEL_SOURCES = ["api.hip", "layer_norm.hip", "softmax_dropout.hip", "dropout_add.hip", "xentropy.hip", "reduce.hip",
                   "gemm.hip", "gemm_nt.hip", "gemm_nn.hip", "gemm_tn.hip", "mlp.hip", "attention.hip", "rel_position.hip", "multi_tensor.hip", "rotary.hip", "flash_attn.hip", "gemm_f32.hip", "glu.hip", "attn_decode.hip", "gemm_skinny.hip"]
-HEADERS = ["common.cuh", "trace.cuh", "reduce.cuh", "gemm.cuh", "gemm_ring.cuh", "gemm_inst.cuh"]
+HEADERS = ["common.hip.h", "trace.hip.h", "reduce.hip.h", "gemm.hip.h", "gemm_ring.hip.h", "gemm_inst.hip.h"]
 OWN_SOURCES = ["hostsim.cpp", "stubs.cpp"]
 
 
@@ -88,12 +88,12 @@ def build(verbose=False):
         src = os.path.join(CSRC, name)
         if not os.path.exists(src):
             continue
-        dst = os.path.join(BUILD, name if name.endswith(".cuh") else name.replace(".hip", ".cpp"))
+        dst = os.path.join(BUILD, name if name.endswith(".hip.h") else name[:-len(".hip")] + ".cpp")
         with open(src) as f:
             text = '#line 1 "%s"\n' % src + transform(f.read())
         with open(dst, "w") as f:
             f.write(text)
-        if not name.endswith(".cuh"):
+        if not name.endswith(".hip.h"):
             units.append(dst)
     units += [os.path.join(HERE, n) for n in OWN_SOURCES]
     flags = ["-x", "c++", "-std=c++17", OPT, "-gline-tables-only", "-fPIC", "-fno-strict-aliasing", "-Wno-unknown-pragmas",

@@ -1,8 +1,8 @@
 // Pieces of the library that the CPU build does not take from the kernel sources (per-kernel tracing counts launches
 // by name and reports zero time), and C hooks for the reduction kernels, which the real library only reaches from
 // inside its GEMM-based operators.
-#include "reduce.cuh"
-#include "gemm.cuh"
+#include "reduce.hip.h"
+#include "gemm.hip.h"
 #include <algorithm>
 #include <cstring>
 #include <map>
@@ -49,7 +49,7 @@ extern "C" int hostsim_colsum(int dtype, const void* X, int64_t ld, int M, int N
   return colsum_run(dtype, X, ld, M, N, part, out, nullptr);
 }
 
-// Split-K reduction for the 128x128 tile (2 x 2 wavefronts) and the 256x256 tile (2 x 4), launched as gemm_inst.cuh does.
+// Split-K reduction for the 128x128 tile (2 x 2 wavefronts) and the 256x256 tile (2 x 4), launched as gemm_inst.hip.h does.
 template <typename T, int BM, int BN, int WM, int WN>
 static int splitk(const float* ws, void* C, int64_t ldc, int M, int N, int m_tiles, int n_tiles, int batch, int64_t sC,
                   int splits, float alpha, int c_vec) {

@@ -1,4 +1,4 @@
-"""Index-math check of the slot layouts of the GEMM ring loop (nmtgminor_amd/csrc/gemm_ring.cuh).
+"""Index-math check of the slot layouts of the GEMM ring loop (nmtgminor_amd/csrc/gemm_ring.hip.h).
 
 A numpy model fills one 16 KB LDS slot exactly as the kernel's one-kilobyte global -> LDS transfers
 do (lane l of transfer ii writes its 16 bytes at ii * 1024 + 16 l; the swizzle is applied to the

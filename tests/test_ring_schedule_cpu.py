@@ -1,4 +1,4 @@
-"""Hazard check of the slot-ring schedule of the GEMM main loop (nmtgminor_amd/csrc/gemm_ring.cuh).
+"""Hazard check of the slot-ring schedule of the GEMM main loop (nmtgminor_amd/csrc/gemm_ring.hip.h).
 
 A small event model of one wavefront replays the kernel's issue / wait / barrier / read sequence
 with the kernel's own bookkeeping formulas (ring positions, number of transfers allowed to stay in
