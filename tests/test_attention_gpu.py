@@ -405,3 +405,48 @@ def test_inference_without_coverage_writes_no_probability_tensor(dev, monkeypatc
     # recorded by autograd (or in training mode) the tensors are kept whatever the caller asks for
     kept = sa_native.forward(*args, want_probs=False)
     assert kept[1].shape == (2 * h, 136, 136) and kept[2].shape == (2 * h, 136, 136)
+
+
+@pytest.mark.parametrize("seed", range(4000, 4012))
+def test_inference_kernel_on_randomly_drawn_shapes(dev, monkeypatch, seed):
+    """Query counts around the block and wavefront sizes, key counts from 4 up (multiples of 4: around the 64-key tile,
+    one tile, many), both head dimensions, both forms of the kernel, key-padding masks with fully masked sentences and
+    time masks: probabilities and context against the score-keeping path, which shares no kernel with it."""
+    import random
+    rnd = random.Random(seed)
+    dtype = rnd.choice([torch.bfloat16, torch.float16])
+    h, dh = rnd.choice([1, 2, 3]), rnd.choice([64, 128])
+    e, b = h * dh, rnd.choice([1, 2, 3])
+    monkeypatch.setenv("NMTG_ATTN_PROBS_SPLIT", rnd.choice(["0", "1"]))
+    g = torch.Generator().manual_seed(seed)
+    if rnd.random() < 0.5:                                                    # self-attention, key padding or time mask
+        t = 4 * rnd.choice([1, 2, 8, 15, 16, 17, 31, 33, 48, 65])
+        causal = rnd.random() < 0.5
+        d = inputs.self_attn_inputs(t, b, e, h, dtype, p=0.0, seed=seed, causal=causal)
+        if not causal and b > 1 and rnd.random() < 0.5:
+            d["pad_mask"][0, :] = True
+        gd = lambda k: d[k].to(dev)
+        args = (causal, False, h, gd("x"), gd("w_in"), gd("w_out"), gd("b_in"), gd("b_out"), gd("time_mask") if causal else gd("pad_mask"), 0.0)
+        with torch.no_grad():
+            lean = sa_native.forward(*args)
+        full = sa_native.forward(*args)
+        pairs = ((lean[2], full[2], "probabilities"), (lean[4], full[4], "context"), (lean[5], full[5], "outputs"))
+        assert lean[1].numel() == 0
+    else:                                                                     # encoder-decoder attention
+        tq = rnd.choice([1, 5, 31, 32, 33, 64, 100, 128, 129, 200])
+        tk = 4 * rnd.choice([1, 3, 15, 16, 17, 40, 100, 129, 375])
+        d = inputs.encdec_attn_inputs(tq, tk, b, e, h, dtype, p=0.0, seed=seed)
+        pad = d["pad_mask"] if rnd.random() < 0.7 else None
+        if pad is not None and b > 1 and rnd.random() < 0.5:
+            pad[-1, :] = True
+        gd = lambda k: d[k].to(dev)
+        args = (False, h, gd("x_q"), gd("x_kv"), gd("w_q"), gd("w_kv"), gd("w_out"), gd("b_q"), gd("b_kv"), gd("b_out"),
+                None if pad is None else pad.to(dev), 0.0)
+        with torch.no_grad():
+            lean = ed_native.forward(*args)
+        full = ed_native.forward(*args)
+        pairs = ((lean[3], full[3], "probabilities"), (lean[5], full[5], "context"), (lean[6], full[6], "outputs"))
+        assert lean[2].numel() == 0
+    for got, want, what in pairs:
+        assert not torch.isnan(got.float()).any(), what
+        assert_close(got, want.cpu(), dtype, f"{what} (seed {seed})", atol=2e-3)

@@ -383,6 +383,11 @@ def test_attention_inference_without_the_score_tensor(mi355x, monkeypatch, split
     tat.test_inference_keeps_the_score_tensor_where_the_one_kernel_path_does_not_apply(CPU, monkeypatch)   # sets a switch: last
 
 
+@pytest.mark.parametrize("seed", [4000, 4003, 4005, 4008] if SANITIZER_RUN else list(range(4000, 4012)))
+def test_attention_inference_random_shapes(mi355x, monkeypatch, seed):
+    tat.test_inference_kernel_on_randomly_drawn_shapes(CPU, monkeypatch, seed)
+
+
 def test_encdec_attention_without_biases_compact_and_modules(mi355x):
     tat.test_encdec_attention_without_biases_and_compact(CPU)
     tat.test_modules_state_dict_names_and_forward(CPU)
