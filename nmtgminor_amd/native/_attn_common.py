@@ -28,9 +28,14 @@ def mask_arg(mask, use_time_mask, batch, len_q, len_k):
         return None, 0
     if use_time_mask:
         check(mask.numel() == len_q * len_k, "time mask must be [len_q, len_k]")
-        return mask.reshape(len_q, len_k).to(torch.uint8).contiguous(), 2
+        return _word_aligned(mask.reshape(len_q, len_k).to(torch.uint8).contiguous()), 2
     check(mask.numel() == batch * len_k, "key padding mask must be [batch, len_k]")
-    return mask.reshape(batch, len_k).to(torch.uint8).contiguous(), 1
+    return _word_aligned(mask.reshape(batch, len_k).to(torch.uint8).contiguous()), 1
+
+
+def _word_aligned(mask):
+    """The kernels read mask bytes four (or eight) at a time: a uint8 view that starts at an odd address is copied."""
+    return mask if mask.data_ptr() % 8 == 0 else mask.clone()
 
 
 def dropout_args(is_training, p, shape, device, dropout_mask):

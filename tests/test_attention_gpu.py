@@ -450,3 +450,17 @@ def test_inference_kernel_on_randomly_drawn_shapes(dev, monkeypatch, seed):
     for got, want, what in pairs:
         assert not torch.isnan(got.float()).any(), what
         assert_close(got, want.cpu(), dtype, f"{what} (seed {seed})", atol=2e-3)
+
+
+def test_a_mask_view_at_an_odd_address_is_accepted(dev):
+    """A uint8 mask that is a view into a larger buffer (odd start address) reaches the kernels as an aligned copy."""
+    d = inputs.self_attn_inputs(64, 2, 128, 2, torch.bfloat16, p=0.0, seed=5)
+    g = lambda k: d[k].to(dev)
+    buf = torch.zeros(2 * 64 + 3, dtype=torch.uint8, device=dev)
+    buf[3:] = d["pad_mask"].to(torch.uint8).reshape(-1).to(dev)
+    odd = buf[3:].view(2, 64)
+    assert odd.data_ptr() % 4 != 0
+    with torch.no_grad():
+        a = sa_native.forward(False, False, 2, g("x"), g("w_in"), g("w_out"), g("b_in"), g("b_out"), odd, 0.0)
+        b = sa_native.forward(False, False, 2, g("x"), g("w_in"), g("w_out"), g("b_in"), g("b_out"), g("pad_mask"), 0.0)
+    assert torch.equal(a[5], b[5]) and torch.equal(a[2], b[2])
