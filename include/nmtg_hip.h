@@ -397,6 +397,54 @@ int nmtg_flash_attn_bwd(const void* dout, const void* q, const void* k, const vo
                         int dropout_bits_ready, uint64_t seed, uint64_t offset, int dtype, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * The same kernels over a padded batch: the training call of the attention core when nobody reads
+ * the probabilities.
+ * Reference: the core of SelfAttnFunc / EncdecAttnFunc between the two projections
+ *   (onmt/modules/optimized/self_attention_func.py:136-283 forward, :296-520 backward;
+ *   encdec_attention_func_bias.py:20-213), whose [heads, len_q, len_k] score, probability and
+ *   dropout tensors exist only for the backward and for return_coverage.
+ * q [len_q, batch, heads, head_dim], k / v [len_k, batch, heads, head_dim], out like q: 16-bit views
+ * with a contiguous head_dim (64 or 128) and position, batch and head strides in elements
+ * (multiples of 8), 16-byte aligned; the slots of the head-interleaved projections
+ * [len, batch, heads, 3 | 2, head_dim] qualify. Every sequence has len_q queries.
+ * key_padding_mask: NULL, or uint8 [batch, len_k], 1 = masked, any pattern. A query whose keys are
+ * all masked has out = 0 and softmax_lse = -inf (the reference's softmax yields NaN there).
+ * key_info: with a mask, device workspace of nmtg_flash_attn_key_info_bytes(batch, len_k) bytes,
+ * 4-byte aligned; a small kernel ahead of the others writes each sequence's last live key and
+ * which 64-key tiles hold masked keys in front of it (only those tiles read the mask again).
+ * causal, dropout_*, seed, offset, softmax_lse [batch, heads, len_q], softmax_d: as above, with
+ * max_seqlen_* = len_*.
+ * nmtg_flash_attn_batched_bwd: dout has the strides of out; dq, dk, dv have the strides of q, k, v
+ * and are written whole (zeros at masked keys). Deterministic: no atomics.
+ * ------------------------------------------------------------------------------------------ */
+int64_t nmtg_flash_attn_key_info_bytes(int64_t batch, int64_t len_k);
+
+int nmtg_flash_attn_batched_fwd(const void* q, const void* k, const void* v, void* out,
+                                const uint8_t* key_padding_mask, void* key_info, float* softmax_lse,
+                                int64_t batch, int64_t heads, int64_t head_dim, int64_t len_q,
+                                int64_t len_k, int64_t q_stride_t, int64_t q_stride_b,
+                                int64_t q_stride_h, int64_t k_stride_t, int64_t k_stride_b,
+                                int64_t k_stride_h, int64_t v_stride_t, int64_t v_stride_b,
+                                int64_t v_stride_h, int64_t out_stride_t, int64_t out_stride_b,
+                                int64_t out_stride_h, float softmax_scale, int causal,
+                                int dropout_mode, float dropout_p, const uint8_t* dropout_mask,
+                                uint8_t* dropout_mask_out, void* dropout_bits, uint64_t seed,
+                                uint64_t offset, int dtype, void* stream);
+
+int nmtg_flash_attn_batched_bwd(const void* dout, const void* q, const void* k, const void* v,
+                                const void* out, const float* softmax_lse, void* dq, void* dk,
+                                void* dv, float* softmax_d, const uint8_t* key_padding_mask,
+                                void* key_info, int64_t batch, int64_t heads, int64_t head_dim,
+                                int64_t len_q, int64_t len_k, int64_t q_stride_t, int64_t q_stride_b,
+                                int64_t q_stride_h, int64_t k_stride_t, int64_t k_stride_b,
+                                int64_t k_stride_h, int64_t v_stride_t, int64_t v_stride_b,
+                                int64_t v_stride_h, int64_t out_stride_t, int64_t out_stride_b,
+                                int64_t out_stride_h, float softmax_scale, int causal,
+                                int dropout_mode, float dropout_p, const uint8_t* dropout_mask,
+                                void* dropout_bits, int dropout_bits_ready, uint64_t seed,
+                                uint64_t offset, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Attention of ONE new query position over cached keys / values (incremental decoding).
  * Reference: the incremental branches of SelfAttnFunc (onmt/modules/optimized/
  *   self_attention_func.py:162-174, one query row against the concatenated cache) and of

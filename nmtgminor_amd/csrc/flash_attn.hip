@@ -41,8 +41,12 @@ struct FaArgs {
   void *out, *dq, *dk, *dv;
   float* lse;      // [B, H, max_q]
   float* delta;    // [B, H, max_q]
-  const int32_t *cu_q, *cu_k;
+  const int32_t *cu_q, *cu_k;   // both null: batch-strided call, see seq_span()
   int64_t q_st, q_sh, k_st, k_sh, v_st, v_sh, o_st, o_sh, do_st, do_sh, dq_st, dq_sh, dk_st, dk_sh, dv_st, dv_sh;
+  int64_t q_sb, k_sb, v_sb, o_sb, do_sb, dq_sb, dk_sb, dv_sb;   // per sequence, 0 in packed calls
+  const uint8_t* pad;    // batch-strided calls: key padding mask [B, max_k], 1 = masked, or null
+  const int32_t* kinfo;  // with pad: [B, kinfo_pitch], see flash_key_info_kernel
+  int kinfo_pitch;       // 1 + ceil(max_k / 64)
   int heads, max_q, max_k;
   float scale, scale_log2;
   int causal;
@@ -171,6 +175,52 @@ __device__ __forceinline__ void load_resident(uint4 (&f)[D / 16], const T* base,
   for (int s = 0; s < D / 16; ++s) f[s] = row < len ? *reinterpret_cast<const uint4*>(p + 16 * s) : make_uint4(0, 0, 0, 0);
 }
 
+// Where sequence b lies and how long it is. Packed calls read the cumulative lengths. Batch-strided calls (no cumulative
+// lengths) give every sequence max_q queries and max_k keys, b * *_sb elements into each tensor; a key padding mask cuts
+// the keys at the last live one, and masked keys below that are handled tile by tile (pad_tile()).
+struct SeqSpan { int qs, lq, ks, lk; };
+__device__ __forceinline__ SeqSpan seq_span(const FaArgs& a, int b) {
+  SeqSpan s;
+  if (a.cu_q != nullptr) {
+    s.qs = a.cu_q[b];
+    s.lq = min(a.cu_q[b + 1] - s.qs, a.max_q);
+    s.ks = a.cu_k[b];
+    s.lk = min(a.cu_k[b + 1] - s.ks, a.max_k);
+  } else {
+    s.qs = 0;
+    s.lq = a.max_q;
+    s.ks = 0;
+    s.lk = a.pad != nullptr ? a.kinfo[static_cast<int64_t>(b) * a.kinfo_pitch] : a.max_k;
+  }
+  return s;
+}
+// whether key tile t of sequence b holds a masked key in front of the sequence's last live key
+__device__ __forceinline__ bool pad_tile(const FaArgs& a, int b, int t) {
+  return a.pad != nullptr && a.kinfo[static_cast<int64_t>(b) * a.kinfo_pitch + 1 + t] != 0;
+}
+
+// Key padding mask [B, max_k] -> key_info [B, 1 + ceil(max_k / 64)]: word 0 = 1 + the index of the last live key (0 when
+// every key is masked), word 1 + t = whether tile t has a masked key below that. One block per sequence.
+__global__ __launch_bounds__(256) void flash_key_info_kernel(const uint8_t* pad, int max_k, int32_t* kinfo, int pitch) {
+  __shared__ int part[4];
+  const int b = blockIdx.x, tid = static_cast<int>(threadIdx.x);
+  const uint8_t* row = pad + static_cast<int64_t>(b) * max_k;
+  int last = 0;
+  for (int j = tid; j < max_k; j += 256)
+    if (row[j] == 0) last = j + 1;
+  for (int off = 32; off > 0; off >>= 1) last = max(last, __shfl_xor(last, off, 64));
+  if ((tid & 63) == 0) part[tid >> 6] = last;
+  __syncthreads();
+  const int lk = max(max(part[0], part[1]), max(part[2], part[3]));
+  int32_t* out = kinfo + static_cast<int64_t>(b) * pitch;
+  if (tid == 0) out[0] = lk;
+  for (int t = tid; t < pitch - 1; t += 256) {
+    int any = 0;
+    for (int j = FA_TILE * t; j < min(FA_TILE * t + FA_TILE, lk); ++j) any |= row[j];
+    out[1 + t] = any != 0;
+  }
+}
+
 // Keep bits from the generator: one thread per (head of a sequence, group of 32 queries, group of four keys) runs the
 // eight generator calls of its 32 x 4 elements (one call per 4 x 4 patch) and writes the four keys' words.
 __global__ __launch_bounds__(256) void flash_bits_rng_kernel(FaArgs a, int64_t total) {
@@ -181,7 +231,8 @@ __global__ __launch_bounds__(256) void flash_bits_rng_kernel(FaArgs a, int64_t t
   const int64_t row = id / k4n;                      // (b H + h) q32 + group
   const int grp = static_cast<int>(row % a.q32);
   const int bh = static_cast<int>(row / a.q32), b = bh / a.heads;
-  const int lq = min(a.cu_q[b + 1] - a.cu_q[b], a.max_q), lk = min(a.cu_k[b + 1] - a.cu_k[b], a.max_k);
+  const SeqSpan sp = seq_span(a, b);
+  const int lq = sp.lq, lk = sp.lk;
   if (32 * grp >= lq || 4 * j4 >= lk) return;        // never read: every element there is masked or not stored
   const Philox gen(a.seed);
   const uint64_t q4 = static_cast<uint64_t>((a.max_q + 3) / 4), k4 = static_cast<uint64_t>((a.max_k + 3) / 4);
@@ -220,7 +271,8 @@ __global__ __launch_bounds__(256) void flash_bits_mask_kernel(FaArgs a, int64_t 
   const int64_t row = id / a.kp;
   const int grp = static_cast<int>(row % a.q32);
   const int bh = static_cast<int>(row / a.q32), b = bh / a.heads;
-  const int lq = min(a.cu_q[b + 1] - a.cu_q[b], a.max_q), lk = min(a.cu_k[b + 1] - a.cu_k[b], a.max_k);
+  const SeqSpan sp = seq_span(a, b);
+  const int lq = sp.lq, lk = sp.lk;
   if (32 * grp >= lq || key >= lk) return;
   uint32_t word = 0;
   for (int i = 0; i < 32; ++i) {
@@ -272,14 +324,15 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
   extern __shared__ __align__(16) uint8_t lds_raw[];
   constexpr int IMG = FA_TILE * D * 2;
   const int b = blockIdx.z, h = blockIdx.y, q0 = static_cast<int>(blockIdx.x) * FA_ROWS;
-  const int qs = a.cu_q[b], lq = min(a.cu_q[b + 1] - qs, a.max_q), ks = a.cu_k[b], lk = min(a.cu_k[b + 1] - ks, a.max_k);
+  const SeqSpan sp = seq_span(a, b);
+  const int qs = sp.qs, lq = sp.lq, ks = sp.ks, lk = sp.lk;
   if (q0 >= lq) return;
   const int lane = static_cast<int>(threadIdx.x) & 63, wave = static_cast<int>(threadIdx.x) >> 6, half = lane >> 5;
   const int bh = b * a.heads + h;
   const int qrow = q0 + 32 * wave + (lane & 31);
-  const T* qb = static_cast<const T*>(a.q) + static_cast<int64_t>(qs) * a.q_st + static_cast<int64_t>(h) * a.q_sh;
-  const T* kb = static_cast<const T*>(a.k) + static_cast<int64_t>(ks) * a.k_st + static_cast<int64_t>(h) * a.k_sh;
-  const T* vb = static_cast<const T*>(a.v) + static_cast<int64_t>(ks) * a.v_st + static_cast<int64_t>(h) * a.v_sh;
+  const T* qb = static_cast<const T*>(a.q) + static_cast<int64_t>(qs) * a.q_st + static_cast<int64_t>(b) * a.q_sb + static_cast<int64_t>(h) * a.q_sh;
+  const T* kb = static_cast<const T*>(a.k) + static_cast<int64_t>(ks) * a.k_st + static_cast<int64_t>(b) * a.k_sb + static_cast<int64_t>(h) * a.k_sh;
+  const T* vb = static_cast<const T*>(a.v) + static_cast<int64_t>(ks) * a.v_st + static_cast<int64_t>(b) * a.v_sb + static_cast<int64_t>(h) * a.v_sh;
   uint4 qf[D / 16];
   load_resident<T, D>(qf, qb, a.q_st, qrow, lq, lane);
 
@@ -294,6 +347,7 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
     for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
   float m = FA_NEG, l = 0.f;
   const float dead_raw = FA_NEG / a.scale_log2;   // the raw score that the scale turns into -1e30
+  const uint8_t* padrow = a.pad != nullptr ? a.pad + static_cast<int64_t>(b) * a.max_k : nullptr;   // read below lk only
 
   Staged<D> sk, sv;
   if (ntiles > 0) {
@@ -321,14 +375,15 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
       for (int n = 0; n < 2; ++n) mfma<T>::run(read_rows<D>(kimg, n, ss, lane), qf[ss], s[n]);
     // Masking only where the tile crosses the end of the keys or the causal diagonal (the same for the whole wavefront).
     // A masked raw score is the value that the scale turns into -1e30 or beyond: its probability is exp2 of that, 0.
-    const bool edge = (t + 1) * FA_TILE > lk || (a.causal && t * FA_TILE + FA_TILE - 1 > q0 + 32 * wave);
+    const bool padt = pad_tile(a, b, t);
+    const bool edge = (t + 1) * FA_TILE > lk || (a.causal && t * FA_TILE + FA_TILE - 1 > q0 + 32 * wave) || padt;
     if (edge) {
 #pragma unroll
       for (int n = 0; n < 2; ++n)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int key = t * FA_TILE + 32 * n + 8 * (r / 4) + 4 * half + r % 4;
-          if (key >= lk || (a.causal && key > qrow)) s[n][r] = dead_raw;
+          if (key >= lk || (a.causal && key > qrow) || (padt && padrow[key] != 0)) s[n][r] = dead_raw;
         }
     }
     // tile maximum of the scaled scores from the extreme raw score (one multiplication instead of 32)
@@ -369,6 +424,19 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
         s[n][r] = pr;
         lsum += pr;
       }
+    if (padt) {
+      // A row that has met no live key yet still has the initial m, against which a dead score is not small: such
+      // probabilities are set to 0 by hand. (Without masked keys inside the sequence, key 0 is live for every row.)
+      lsum = 0.f;
+#pragma unroll
+      for (int n = 0; n < 2; ++n)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = t * FA_TILE + 32 * n + 8 * (r / 4) + 4 * half + r % 4;
+          if (key >= lk || (a.causal && key > qrow) || padrow[key] != 0) s[n][r] = 0.f;
+          lsum += s[n][r];
+        }
+    }
     l += lsum;
     if constexpr (DROP != 0) {
       const uint64_t* lane_mask = tile_lane_masks(a, bh, group, t);
@@ -398,7 +466,7 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
   const float inv = l > 0.f ? a.drop_scale / l : 0.f;
   if (half == 0 && qrow < lq)
     a.lse[static_cast<int64_t>(bh) * a.max_q + qrow] = l > 0.f ? (m + log2f(l)) * (1.0f / FA_LOG2E) : -INFINITY;
-  T* ob = static_cast<T*>(a.out) + static_cast<int64_t>(qs) * a.o_st + static_cast<int64_t>(h) * a.o_sh;
+  T* ob = static_cast<T*>(a.out) + static_cast<int64_t>(qs) * a.o_st + static_cast<int64_t>(b) * a.o_sb + static_cast<int64_t>(h) * a.o_sh;
   store_rows_out<T, D>(o, inv, lds_raw + wave * (32 * D * 2), ob, a.o_st, q0 + 32 * wave, lq, lane);
 }
 
@@ -410,16 +478,17 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dq_kern
   extern __shared__ __align__(16) uint8_t lds_raw[];
   constexpr int IMG = FA_TILE * D * 2;
   const int b = blockIdx.z, h = blockIdx.y, q0 = static_cast<int>(blockIdx.x) * FA_ROWS;
-  const int qs = a.cu_q[b], lq = min(a.cu_q[b + 1] - qs, a.max_q), ks = a.cu_k[b], lk = min(a.cu_k[b + 1] - ks, a.max_k);
+  const SeqSpan sp = seq_span(a, b);
+  const int qs = sp.qs, lq = sp.lq, ks = sp.ks, lk = sp.lk;
   if (q0 >= lq) return;
   const int lane = static_cast<int>(threadIdx.x) & 63, wave = static_cast<int>(threadIdx.x) >> 6, half = lane >> 5;
   const int bh = b * a.heads + h;
   const int qrow = q0 + 32 * wave + (lane & 31);
-  const T* qb = static_cast<const T*>(a.q) + static_cast<int64_t>(qs) * a.q_st + static_cast<int64_t>(h) * a.q_sh;
-  const T* kb = static_cast<const T*>(a.k) + static_cast<int64_t>(ks) * a.k_st + static_cast<int64_t>(h) * a.k_sh;
-  const T* vb = static_cast<const T*>(a.v) + static_cast<int64_t>(ks) * a.v_st + static_cast<int64_t>(h) * a.v_sh;
-  const T* ob = static_cast<const T*>(a.o) + static_cast<int64_t>(qs) * a.o_st + static_cast<int64_t>(h) * a.o_sh;
-  const T* gb = static_cast<const T*>(a.d_o) + static_cast<int64_t>(qs) * a.do_st + static_cast<int64_t>(h) * a.do_sh;
+  const T* qb = static_cast<const T*>(a.q) + static_cast<int64_t>(qs) * a.q_st + static_cast<int64_t>(b) * a.q_sb + static_cast<int64_t>(h) * a.q_sh;
+  const T* kb = static_cast<const T*>(a.k) + static_cast<int64_t>(ks) * a.k_st + static_cast<int64_t>(b) * a.k_sb + static_cast<int64_t>(h) * a.k_sh;
+  const T* vb = static_cast<const T*>(a.v) + static_cast<int64_t>(ks) * a.v_st + static_cast<int64_t>(b) * a.v_sb + static_cast<int64_t>(h) * a.v_sh;
+  const T* ob = static_cast<const T*>(a.o) + static_cast<int64_t>(qs) * a.o_st + static_cast<int64_t>(b) * a.o_sb + static_cast<int64_t>(h) * a.o_sh;
+  const T* gb = static_cast<const T*>(a.d_o) + static_cast<int64_t>(qs) * a.do_st + static_cast<int64_t>(b) * a.do_sb + static_cast<int64_t>(h) * a.do_sh;
   uint4 qf[D / 16], gf[D / 16];
   load_resident<T, D>(qf, qb, a.q_st, qrow, lq, lane);
   load_resident<T, D>(gf, gb, a.do_st, qrow, lq, lane);
@@ -448,6 +517,7 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dq_kern
   const int ntiles = (nkeys + FA_TILE - 1) / FA_TILE;
   const int group = static_cast<int>(blockIdx.x) * (FA_ROWS / 32) + __builtin_amdgcn_readfirstlane(wave);   // of 32 queries
   const float dead_raw = FA_NEG / a.scale_log2;   // the raw score that the scale turns into -1e30
+  const uint8_t* padrow = a.pad != nullptr ? a.pad + static_cast<int64_t>(b) * a.max_k : nullptr;   // read below lk only
   acc16_t dq[D / 32];
 #pragma unroll
   for (int i = 0; i < D / 32; ++i)
@@ -485,13 +555,14 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dq_kern
         mfma<T>::run(read_rows<D>(vimg, n, ss, lane), gf[ss], dp[n]);
       }
     // masking as in the forward: only where the tile crosses the end of the keys or the causal diagonal
-    if ((t + 1) * FA_TILE > lk || (a.causal && t * FA_TILE + FA_TILE - 1 > q0 + 32 * wave)) {
+    const bool padt = pad_tile(a, b, t);
+    if ((t + 1) * FA_TILE > lk || (a.causal && t * FA_TILE + FA_TILE - 1 > q0 + 32 * wave) || padt) {
 #pragma unroll
       for (int n = 0; n < 2; ++n)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int key = t * FA_TILE + 32 * n + 8 * (r / 4) + 4 * half + r % 4;
-          if (key >= lk || (a.causal && key > qrow)) s[n][r] = dead_raw;
+          if (key >= lk || (a.causal && key > qrow) || (padt && padrow[key] != 0)) s[n][r] = dead_raw;
         }
     }
     [[maybe_unused]] const uint64_t* lane_mask = DROP != 0 ? tile_lane_masks(a, bh, group, t) : nullptr;
@@ -521,7 +592,7 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dq_kern
     }
     __syncthreads();
   }
-  T* dqb = static_cast<T*>(a.dq) + static_cast<int64_t>(qs) * a.dq_st + static_cast<int64_t>(h) * a.dq_sh;
+  T* dqb = static_cast<T*>(a.dq) + static_cast<int64_t>(qs) * a.dq_st + static_cast<int64_t>(b) * a.dq_sb + static_cast<int64_t>(h) * a.dq_sh;
   store_rows_out<T, D>(dq, a.scale, lds_raw + wave * (32 * D * 2), dqb, a.dq_st, q0 + 32 * wave, lq, lane);
 }
 
@@ -534,15 +605,36 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dkv_ker
   constexpr int IMG = FA_TILE * D * 2;
   constexpr int BUF = 4 * IMG + 2 * FA_TILE * 4;   // Q rows, Q transposed, dO rows, dO transposed, lse2[64], delta[64]
   const int b = blockIdx.z, h = blockIdx.y, k0 = static_cast<int>(blockIdx.x) * FA_ROWS;
-  const int qs = a.cu_q[b], lq = min(a.cu_q[b + 1] - qs, a.max_q), ks = a.cu_k[b], lk = min(a.cu_k[b + 1] - ks, a.max_k);
-  if (k0 >= lk) return;
+  const SeqSpan sp = seq_span(a, b);
+  const int qs = sp.qs, lq = sp.lq, ks = sp.ks, lk = sp.lk;
+  // Packed calls write the rows of the sequence's keys; batch-strided calls write all max_k rows (zeros past the last
+  // live key: the gradient of the projection reads every row).
+  const int lk_out = a.cu_q != nullptr ? lk : a.max_k;
+  if (k0 >= lk) {
+    if (k0 < lk_out) {
+      T* dkz = static_cast<T*>(a.dk) + static_cast<int64_t>(b) * a.dk_sb + static_cast<int64_t>(h) * a.dk_sh;
+      T* dvz = static_cast<T*>(a.dv) + static_cast<int64_t>(b) * a.dv_sb + static_cast<int64_t>(h) * a.dv_sh;
+      constexpr int CH = D / 8;
+      for (int id = static_cast<int>(threadIdx.x); id < FA_ROWS * CH; id += FA_THREADS) {
+        const int row = k0 + id / CH, c = id % CH;
+        if (row < lk_out) {
+          *reinterpret_cast<uint4*>(dkz + static_cast<int64_t>(row) * a.dk_st + 8 * c) = make_uint4(0, 0, 0, 0);
+          *reinterpret_cast<uint4*>(dvz + static_cast<int64_t>(row) * a.dv_st + 8 * c) = make_uint4(0, 0, 0, 0);
+        }
+      }
+    }
+    return;
+  }
   const int lane = static_cast<int>(threadIdx.x) & 63, wave = static_cast<int>(threadIdx.x) >> 6, half = lane >> 5;
   const int bh = b * a.heads + h;
   const int krow = k0 + 32 * wave + (lane & 31);
-  const T* qb = static_cast<const T*>(a.q) + static_cast<int64_t>(qs) * a.q_st + static_cast<int64_t>(h) * a.q_sh;
-  const T* kb = static_cast<const T*>(a.k) + static_cast<int64_t>(ks) * a.k_st + static_cast<int64_t>(h) * a.k_sh;
-  const T* vb = static_cast<const T*>(a.v) + static_cast<int64_t>(ks) * a.v_st + static_cast<int64_t>(h) * a.v_sh;
-  const T* gb = static_cast<const T*>(a.d_o) + static_cast<int64_t>(qs) * a.do_st + static_cast<int64_t>(h) * a.do_sh;
+  // this lane's key is masked (past the end, or padded), and whether any key of the wavefront is
+  const bool kdead = krow >= lk || (a.pad != nullptr && a.pad[static_cast<int64_t>(b) * a.max_k + krow] != 0);
+  const bool wave_dead = __builtin_amdgcn_ballot_w64(kdead) != 0;
+  const T* qb = static_cast<const T*>(a.q) + static_cast<int64_t>(qs) * a.q_st + static_cast<int64_t>(b) * a.q_sb + static_cast<int64_t>(h) * a.q_sh;
+  const T* kb = static_cast<const T*>(a.k) + static_cast<int64_t>(ks) * a.k_st + static_cast<int64_t>(b) * a.k_sb + static_cast<int64_t>(h) * a.k_sh;
+  const T* vb = static_cast<const T*>(a.v) + static_cast<int64_t>(ks) * a.v_st + static_cast<int64_t>(b) * a.v_sb + static_cast<int64_t>(h) * a.v_sh;
+  const T* gb = static_cast<const T*>(a.d_o) + static_cast<int64_t>(qs) * a.do_st + static_cast<int64_t>(b) * a.do_sb + static_cast<int64_t>(h) * a.do_sh;
   uint4 kf[D / 16], vf[D / 16];
   load_resident<T, D>(kf, kb, a.k_st, krow, lk, lane);
   load_resident<T, D>(vf, vb, a.v_st, krow, lk, lane);
@@ -613,13 +705,13 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dkv_ker
       }
     // s[n][r]: query 32 n + 8 (r / 4) + 4 half + r % 4 of the tile, key krow. P (dropped, scaled) stays in dp's place
     // for dV, dS goes to s for dK.
-    if (k0 + 32 * wave + 31 >= lk || (a.causal && t * FA_TILE < k0 + 32 * wave + 31)) {
+    if (wave_dead || (a.causal && t * FA_TILE < k0 + 32 * wave + 31)) {
 #pragma unroll
       for (int n = 0; n < 2; ++n)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int qi = t * FA_TILE + 32 * n + 8 * (r / 4) + 4 * half + r % 4;
-          if (krow >= lk || (a.causal && krow > qi)) s[n][r] = dead_raw;
+          if (kdead || (a.causal && krow > qi)) s[n][r] = dead_raw;
         }
     }
     // keep bits of this lane's key for the tile's two groups of 32 queries, shifted so that bit 8 g + c is register 4 g + c
@@ -664,12 +756,12 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dkv_ker
     if (t + 1 < ntiles) store_tile(lds_raw + ((t + 1) & 1) * BUF);
     __syncthreads();
   }
-  T* dkb = static_cast<T*>(a.dk) + static_cast<int64_t>(ks) * a.dk_st + static_cast<int64_t>(h) * a.dk_sh;
-  T* dvb = static_cast<T*>(a.dv) + static_cast<int64_t>(ks) * a.dv_st + static_cast<int64_t>(h) * a.dv_sh;
+  T* dkb = static_cast<T*>(a.dk) + static_cast<int64_t>(ks) * a.dk_st + static_cast<int64_t>(b) * a.dk_sb + static_cast<int64_t>(h) * a.dk_sh;
+  T* dvb = static_cast<T*>(a.dv) + static_cast<int64_t>(ks) * a.dv_st + static_cast<int64_t>(b) * a.dv_sb + static_cast<int64_t>(h) * a.dv_sh;
   uint8_t* patch = lds_raw + wave * (32 * D * 2);
-  store_rows_out<T, D>(dk, a.scale, patch, dkb, a.dk_st, k0 + 32 * wave, lk, lane);
+  store_rows_out<T, D>(dk, a.scale, patch, dkb, a.dk_st, k0 + 32 * wave, lk_out, lane);
   __syncthreads();
-  store_rows_out<T, D>(dv, a.drop_scale, patch, dvb, a.dv_st, k0 + 32 * wave, lk, lane);
+  store_rows_out<T, D>(dv, a.drop_scale, patch, dvb, a.dv_st, k0 + 32 * wave, lk_out, lane);
 }
 
 // -------------------------------------------------------------------------------------------------------------------
@@ -1045,6 +1137,50 @@ void set_dropout(FaArgs& a, int drop_mode, float p, uint64_t seed, uint64_t offs
   a.offset = offset;
 }
 
+// the launches of a forward call whose arguments are in place: keep bits, then the attention kernel
+int fwd_run(const char* what, FaArgs& a, int64_t batch, int64_t d, int drop_mode, void* bits, int dtype, hipStream_t st) {
+  const dim3 grid(static_cast<unsigned>((a.max_q + FA_ROWS - 1) / FA_ROWS), static_cast<unsigned>(a.heads), static_cast<unsigned>(batch));
+  int rc = bits_launch(what, a, drop_mode, batch, bits, false, st);
+  if (rc) return rc;
+  if (dtype == NMTG_F16) rc = d == 64 ? fwd_launch<f16_t, 64>(a, drop_mode, grid, st) : fwd_launch<f16_t, 128>(a, drop_mode, grid, st);
+  else rc = d == 64 ? fwd_launch<bf16_t, 64>(a, drop_mode, grid, st) : fwd_launch<bf16_t, 128>(a, drop_mode, grid, st);
+  if (rc) return rc;
+  NMTG_CHECK_LAUNCH(what);
+  return 0;
+}
+
+int bwd_run(const char* what, FaArgs& a, int64_t batch, int64_t d, int drop_mode, void* bits, bool bits_ready, int dtype, hipStream_t st) {
+  const dim3 grid_q(static_cast<unsigned>((a.max_q + FA_ROWS - 1) / FA_ROWS), static_cast<unsigned>(a.heads), static_cast<unsigned>(batch));
+  const dim3 grid_k(static_cast<unsigned>((a.max_k + FA_ROWS - 1) / FA_ROWS), static_cast<unsigned>(a.heads), static_cast<unsigned>(batch));
+  int rc = bits_launch(what, a, drop_mode, batch, bits, bits_ready, st);
+  if (rc) return rc;
+  if (dtype == NMTG_F16) rc = d == 64 ? bwd_launch<f16_t, 64>(a, drop_mode, grid_q, grid_k, st) : bwd_launch<f16_t, 128>(a, drop_mode, grid_q, grid_k, st);
+  else rc = d == 64 ? bwd_launch<bf16_t, 64>(a, drop_mode, grid_q, grid_k, st) : bwd_launch<bf16_t, 128>(a, drop_mode, grid_q, grid_k, st);
+  if (rc) return rc;
+  NMTG_CHECK_LAUNCH(what);
+  return 0;
+}
+
+// a [len, batch, heads, head_dim] view: as view_ok, and a batch stride that keeps the alignment
+bool batched_view_ok(const void* p, int64_t st, int64_t sb, int64_t sh, int64_t heads, int64_t d) {
+  return aligned16(p) && st % 8 == 0 && sb % 8 == 0 && sh % 8 == 0 && sh >= d && sb >= 0 && st >= 0;
+}
+
+// the key padding mask of a batch-strided call: fills key_info ahead of every kernel that reads it
+int key_info_launch(const char* what, FaArgs& a, int64_t batch, const uint8_t* pad, void* key_info, hipStream_t st) {
+  if (pad == nullptr) return 0;
+  NMTG_REQUIRE(key_info != nullptr && reinterpret_cast<uintptr_t>(key_info) % 4 == 0,
+               "%s: a key padding mask needs the key_info workspace (nmtg_flash_attn_key_info_bytes)", what);
+  a.pad = pad;
+  a.kinfo = static_cast<const int32_t*>(key_info);
+  a.kinfo_pitch = 1 + (a.max_k + FA_TILE - 1) / FA_TILE;
+  if (a.max_k == 0) return 0;
+  TraceScope trace("flash_attn_key_info", st);
+  hipLaunchKernelGGL(flash_key_info_kernel, dim3(static_cast<unsigned>(batch)), dim3(256), 0, st, pad, a.max_k,
+                     static_cast<int32_t*>(key_info), a.kinfo_pitch);
+  return 0;
+}
+
 template <typename T, int D, int G>
 int probs_launch(const AttnProbsCall& c, dim3 grid, hipStream_t st) {
   auto go = [&](auto kern) {
@@ -1131,15 +1267,7 @@ extern "C" int nmtg_flash_attn_fwd(const void* q, const void* k, const void* v, 
   a.scale = softmax_scale; a.scale_log2 = softmax_scale * FA_LOG2E; a.causal = causal != 0;
   a.mask = dropout_mask; a.mask_out = dropout_mask_out;
   set_dropout(a, dropout_mode, dropout_p, seed, offset);
-  const dim3 grid(static_cast<unsigned>((max_seqlen_q + FA_ROWS - 1) / FA_ROWS), static_cast<unsigned>(heads), static_cast<unsigned>(batch));
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  int rc = bits_launch("flash_attn_fwd", a, dropout_mode, batch, dropout_bits, false, st);
-  if (rc) return rc;
-  if (dtype == NMTG_F16) rc = head_dim == 64 ? fwd_launch<f16_t, 64>(a, dropout_mode, grid, st) : fwd_launch<f16_t, 128>(a, dropout_mode, grid, st);
-  else rc = head_dim == 64 ? fwd_launch<bf16_t, 64>(a, dropout_mode, grid, st) : fwd_launch<bf16_t, 128>(a, dropout_mode, grid, st);
-  if (rc) return rc;
-  NMTG_CHECK_LAUNCH("flash_attn_fwd");
-  return 0;
+  return fwd_run("flash_attn_fwd", a, batch, head_dim, dropout_mode, dropout_bits, dtype, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int nmtg_flash_attn_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out,
@@ -1175,14 +1303,80 @@ extern "C" int nmtg_flash_attn_bwd(const void* dout, const void* q, const void* 
   a.scale = softmax_scale; a.scale_log2 = softmax_scale * FA_LOG2E; a.causal = causal != 0;
   a.mask = dropout_mask; a.mask_out = nullptr;
   set_dropout(a, dropout_mode, dropout_p, seed, offset);
-  const dim3 grid_q(static_cast<unsigned>((max_seqlen_q + FA_ROWS - 1) / FA_ROWS), static_cast<unsigned>(heads), static_cast<unsigned>(batch));
-  const dim3 grid_k(static_cast<unsigned>((max_seqlen_k + FA_ROWS - 1) / FA_ROWS), static_cast<unsigned>(heads), static_cast<unsigned>(batch));
+  return bwd_run("flash_attn_bwd", a, batch, head_dim, dropout_mode, dropout_bits, dropout_bits_ready != 0, dtype,
+                 static_cast<hipStream_t>(stream));
+}
+
+extern "C" int64_t nmtg_flash_attn_key_info_bytes(int64_t batch, int64_t len_k) {
+  if (batch <= 0 || len_k < 0) return 0;
+  return batch * (1 + (len_k + FA_TILE - 1) / FA_TILE) * 4;
+}
+
+extern "C" int nmtg_flash_attn_batched_fwd(const void* q, const void* k, const void* v, void* out, const uint8_t* key_padding_mask,
+                                           void* key_info, float* softmax_lse, int64_t batch, int64_t heads, int64_t head_dim,
+                                           int64_t len_q, int64_t len_k, int64_t q_stride_t, int64_t q_stride_b, int64_t q_stride_h,
+                                           int64_t k_stride_t, int64_t k_stride_b, int64_t k_stride_h, int64_t v_stride_t,
+                                           int64_t v_stride_b, int64_t v_stride_h, int64_t out_stride_t, int64_t out_stride_b,
+                                           int64_t out_stride_h, float softmax_scale, int causal, int dropout_mode, float dropout_p,
+                                           const uint8_t* dropout_mask, uint8_t* dropout_mask_out, void* dropout_bits,
+                                           uint64_t seed, uint64_t offset, int dtype, void* stream) {
+  const char* what = "flash_attn_batched_fwd";
+  if (int rc = check_common(what, batch, heads, head_dim, len_q, len_k, dropout_mode, dropout_p, softmax_scale, dtype)) return rc;
+  if (batch == 0 || len_q == 0) return 0;
+  NMTG_REQUIRE(q && k && v && out && softmax_lse, "%s: null pointer argument", what);
+  NMTG_REQUIRE(dropout_mode != 1 || dropout_mask, "%s: dropout mode 1 replays a keep-mask and none was given", what);
+  NMTG_REQUIRE(batched_view_ok(q, q_stride_t, q_stride_b, q_stride_h, heads, head_dim) &&
+                   batched_view_ok(k, k_stride_t, k_stride_b, k_stride_h, heads, head_dim) &&
+                   batched_view_ok(v, v_stride_t, v_stride_b, v_stride_h, heads, head_dim) &&
+                   batched_view_ok(out, out_stride_t, out_stride_b, out_stride_h, heads, head_dim),
+               "%s: q, k, v and out must be 16-byte aligned [len, batch, heads, head_dim] views with a contiguous head_dim and "
+               "strides that are multiples of 8 elements", what);
+  FaArgs a = {};
+  a.q = q; a.k = k; a.v = v; a.out = out; a.lse = softmax_lse;
+  a.q_st = q_stride_t; a.q_sb = q_stride_b; a.q_sh = q_stride_h; a.k_st = k_stride_t; a.k_sb = k_stride_b; a.k_sh = k_stride_h;
+  a.v_st = v_stride_t; a.v_sb = v_stride_b; a.v_sh = v_stride_h; a.o_st = out_stride_t; a.o_sb = out_stride_b; a.o_sh = out_stride_h;
+  a.heads = static_cast<int>(heads); a.max_q = static_cast<int>(len_q); a.max_k = static_cast<int>(len_k);
+  a.scale = softmax_scale; a.scale_log2 = softmax_scale * FA_LOG2E; a.causal = causal != 0;
+  a.mask = dropout_mask; a.mask_out = dropout_mask_out;
+  set_dropout(a, dropout_mode, dropout_p, seed, offset);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  int rc = bits_launch("flash_attn_bwd", a, dropout_mode, batch, dropout_bits, dropout_bits_ready != 0, st);
-  if (rc) return rc;
-  if (dtype == NMTG_F16) rc = head_dim == 64 ? bwd_launch<f16_t, 64>(a, dropout_mode, grid_q, grid_k, st) : bwd_launch<f16_t, 128>(a, dropout_mode, grid_q, grid_k, st);
-  else rc = head_dim == 64 ? bwd_launch<bf16_t, 64>(a, dropout_mode, grid_q, grid_k, st) : bwd_launch<bf16_t, 128>(a, dropout_mode, grid_q, grid_k, st);
-  if (rc) return rc;
-  NMTG_CHECK_LAUNCH("flash_attn_bwd");
-  return 0;
+  if (int rc = key_info_launch(what, a, batch, key_padding_mask, key_info, st)) return rc;
+  return fwd_run(what, a, batch, head_dim, dropout_mode, dropout_bits, dtype, st);
+}
+
+extern "C" int nmtg_flash_attn_batched_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out,
+                                           const float* softmax_lse, void* dq, void* dk, void* dv, float* softmax_d,
+                                           const uint8_t* key_padding_mask, void* key_info, int64_t batch, int64_t heads,
+                                           int64_t head_dim, int64_t len_q, int64_t len_k, int64_t q_stride_t, int64_t q_stride_b,
+                                           int64_t q_stride_h, int64_t k_stride_t, int64_t k_stride_b, int64_t k_stride_h,
+                                           int64_t v_stride_t, int64_t v_stride_b, int64_t v_stride_h, int64_t out_stride_t,
+                                           int64_t out_stride_b, int64_t out_stride_h, float softmax_scale, int causal,
+                                           int dropout_mode, float dropout_p, const uint8_t* dropout_mask, void* dropout_bits,
+                                           int dropout_bits_ready, uint64_t seed, uint64_t offset, int dtype, void* stream) {
+  const char* what = "flash_attn_batched_bwd";
+  if (int rc = check_common(what, batch, heads, head_dim, len_q, len_k, dropout_mode, dropout_p, softmax_scale, dtype)) return rc;
+  if (batch == 0) return 0;
+  NMTG_REQUIRE(dout && q && k && v && out && softmax_lse && dq && dk && dv && softmax_d, "%s: null pointer argument", what);
+  NMTG_REQUIRE(dropout_mode != 1 || dropout_mask || dropout_bits_ready, "%s: dropout mode 1 replays a keep-mask and none was given", what);
+  NMTG_REQUIRE(batched_view_ok(q, q_stride_t, q_stride_b, q_stride_h, heads, head_dim) &&
+                   batched_view_ok(k, k_stride_t, k_stride_b, k_stride_h, heads, head_dim) &&
+                   batched_view_ok(v, v_stride_t, v_stride_b, v_stride_h, heads, head_dim) &&
+                   batched_view_ok(out, out_stride_t, out_stride_b, out_stride_h, heads, head_dim) && aligned16(dout) &&
+                   aligned16(dq) && aligned16(dk) && aligned16(dv),
+               "%s: every tensor must be a 16-byte aligned [len, batch, heads, head_dim] view with a contiguous head_dim and "
+               "strides that are multiples of 8 elements", what);
+  FaArgs a = {};
+  a.q = q; a.k = k; a.v = v; a.o = out; a.d_o = dout; a.dq = dq; a.dk = dk; a.dv = dv;
+  a.lse = const_cast<float*>(softmax_lse); a.delta = softmax_d;
+  a.q_st = a.dq_st = q_stride_t; a.q_sb = a.dq_sb = q_stride_b; a.q_sh = a.dq_sh = q_stride_h;
+  a.k_st = a.dk_st = k_stride_t; a.k_sb = a.dk_sb = k_stride_b; a.k_sh = a.dk_sh = k_stride_h;
+  a.v_st = a.dv_st = v_stride_t; a.v_sb = a.dv_sb = v_stride_b; a.v_sh = a.dv_sh = v_stride_h;
+  a.o_st = a.do_st = out_stride_t; a.o_sb = a.do_sb = out_stride_b; a.o_sh = a.do_sh = out_stride_h;
+  a.heads = static_cast<int>(heads); a.max_q = static_cast<int>(len_q); a.max_k = static_cast<int>(len_k);
+  a.scale = softmax_scale; a.scale_log2 = softmax_scale * FA_LOG2E; a.causal = causal != 0;
+  a.mask = dropout_mask; a.mask_out = nullptr;
+  set_dropout(a, dropout_mode, dropout_p, seed, offset);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (int rc = key_info_launch(what, a, batch, key_padding_mask, key_info, st)) return rc;
+  return bwd_run(what, a, batch, head_dim, dropout_mode, dropout_bits, dropout_bits_ready != 0, dtype, st);
 }

@@ -6,7 +6,8 @@ arguments and 20 gradient slots; biases may be None (the reference then leaves i
 :69-73; here the fused path takes them). Rotary encodings take the composed path of nmtgminor_amd/modules/rotary.py;
 incremental decoding (inference with a cache
 dict) runs in nmtgminor_amd/modules/incremental.py. A 21st
-optional argument replays an explicit dropout keep-mask."""
+optional argument replays an explicit dropout keep-mask. A training call with return_coverage false runs the tiled
+attention core of nmtgminor_amd/modules/flash_core.py."""
 import torch
 
 from ..native import encdec_multihead_attn_bias_blaslt as native
@@ -79,6 +80,12 @@ def encdec_attn_bias_func(*args):
             r = EncdecAttnRotaryFunc.apply(is_training, heads, inputs_q, inputs_kv, w_q, w_kv, w_out, b_q, b_kv, b_out, mask, p,
                                            pos_q[0], pos_q[1], pos_k[0], pos_k[1], args[20] if len(args) > 20 else None)
             return r if args[19] else (r[0],)
+        if len(args) >= 20:                           # training call whose coverage nobody reads: no [B*H, Tq, Tk] tensor
+            from . import flash_core
+            (recompute, is_training, heads, inputs_q, inputs_kv, w_q, w_kv, w_out, b_q, b_kv, b_out, mask, p) = args[:13]
+            if flash_core.eligible(is_training, args[19], False, recompute, inputs_q, heads) and inputs_kv.dtype == inputs_q.dtype:
+                return (flash_core.EncdecAttnFlashFunc.apply(heads, inputs_q, inputs_kv, w_q, w_kv, w_out, b_q, b_kv, b_out, mask,
+                                                             p, args[20] if len(args) > 20 else None),)
         return EncdecAttnBiasFunc.apply(*args)
 
 

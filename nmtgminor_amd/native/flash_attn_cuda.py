@@ -135,3 +135,94 @@ def bwd(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k,
            L.i32(mode), L.f32(dropout_p), L.ptr(mask if mode == 1 else None), L.ptr(bits), L.i32(ready), ctypes.c_uint64(seed),
            ctypes.c_uint64(offset), L.i32(L.dtype_code(q)), L.stream_of(q))
     return dq, dk, dv, softmax_d
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# The same kernels over a padded batch (no counterpart in the CUDA module): what the training calls of self_attn_func /
+# encdec_attn_func use when the caller does not return the coverage, so that no [B*H, len_q, len_k] tensor is written.
+# ---------------------------------------------------------------------------------------------------------------------
+def _view4(t, name, heads, d):
+    _check(t.dim() == 4 and t.shape[2] == heads and t.shape[3] == d, f"flash_attn: {name} must be [len, batch, {heads}, {d}]")
+    _check(t.stride(3) == 1, f"flash_attn: the head dimension of {name} must be contiguous")
+    return [L.i64(t.stride(0)), L.i64(t.stride(1)), L.i64(t.stride(2))]
+
+
+def _key_info(batch, len_k, device):
+    n = L.load().nmtg_flash_attn_key_info_bytes(L.i64(batch), L.i64(len_k))
+    return torch.empty(max(int(n), 4) // 4, dtype=torch.int32, device=device)
+
+
+def _pad_mask(mask, batch, len_k):
+    if mask is None:
+        return None
+    _check(mask.dtype == torch.uint8 and tuple(mask.shape) == (batch, len_k) and mask.is_contiguous(),
+           "flash_attn: key_padding_mask must be contiguous uint8 [batch, len_k]")
+    L.require_cuda(mask)
+    return mask
+
+
+def fwd_batched(q, k, v, key_padding_mask, dropout_p, softmax_scale, causal, *, dropout_mask=None, rng=None, want_mask=False):
+    """q [len_q, B, H, D], k / v [len_k, B, H, D] (views with a contiguous D), key_padding_mask uint8 [B, len_k] or None
+    -> (out [len_q, B, H, D] contiguous, softmax_lse [B, H, len_q], state); `state` goes to bwd_batched as it is (dropout
+    mode, Philox pair, explicit mask, keep bits, drawn mask when want_mask)."""
+    L.require_cuda(q, k, v)
+    _check(q.dtype in (torch.float16, torch.bfloat16) and k.dtype == q.dtype and v.dtype == q.dtype,
+           "flash_attn: q, k and v must share a 16-bit dtype")
+    _check(q.dim() == 4 and k.shape == v.shape, "flash_attn: q [len_q, B, H, D], k and v [len_k, B, H, D]")
+    len_q, batch, heads, d = q.shape
+    len_k = k.shape[0]
+    _check(tuple(k.shape[1:]) == (batch, heads, d), "flash_attn: k and v must have q's batch, heads and head_dim")
+    pad = _pad_mask(key_padding_mask, batch, len_k)
+    kinfo = _key_info(batch, len_k, q.device) if pad is not None else None
+    out = torch.empty(len_q, batch, heads, d, dtype=q.dtype, device=q.device)
+    lse = torch.empty(batch, heads, len_q, dtype=torch.float32, device=q.device)
+    mode, seed, offset, mask_out, bits = 0, 0, 0, None, None
+    if dropout_p > 0.0:
+        bits = _bits(batch, heads, len_q, len_k, q.device)
+        if dropout_mask is not None:
+            _check(dropout_mask.dtype == torch.uint8 and dropout_mask.numel() == batch * heads * len_q * len_k and
+                   dropout_mask.is_contiguous(), "flash_attn: dropout_mask must be contiguous uint8 [B, H, len_q, len_k]")
+            L.require_cuda(dropout_mask)
+            mode = 1
+        else:
+            mode = 2
+            blocks = batch * heads * ((len_q + 3) // 4) * ((len_k + 3) // 4)
+            seed, offset = rng if rng is not None else philox_seed_offset(q.device, 4 * blocks)
+            if want_mask:
+                mask_out = torch.zeros(batch, heads, len_q, len_k, dtype=torch.uint8, device=q.device)
+    L.call("nmtg_flash_attn_batched_fwd", L.ptr(q), L.ptr(k), L.ptr(v), L.ptr(out), L.ptr(pad), L.ptr(kinfo), L.ptr(lse),
+           L.i64(batch), L.i64(heads), L.i64(d), L.i64(len_q), L.i64(len_k), *_view4(q, "q", heads, d), *_view4(k, "k", heads, d),
+           *_view4(v, "v", heads, d), *_view4(out, "out", heads, d), L.f32(softmax_scale), L.i32(int(bool(causal))), L.i32(mode),
+           L.f32(dropout_p), L.ptr(dropout_mask if mode == 1 else None), L.ptr(mask_out), L.ptr(bits), ctypes.c_uint64(seed),
+           ctypes.c_uint64(offset), L.i32(L.dtype_code(q)), L.stream_of(q))
+    return out, lse, (mode, seed, offset, dropout_mask if mode == 1 else None, bits, mask_out)
+
+
+def bwd_batched(dout, q, k, v, out, softmax_lse, dq, dk, dv, key_padding_mask, dropout_p, softmax_scale, causal, state):
+    """Writes dq, dk, dv (views with the strides of q, k, v: the slots of one projection-gradient buffer) -> softmax_d."""
+    L.require_cuda(dout, q, k, v, out, softmax_lse, dq, dk, dv)
+    len_q, batch, heads, d = q.shape
+    len_k = k.shape[0]
+    _check(all(t.dtype == q.dtype for t in (dout, k, v, out, dq, dk, dv)), "flash_attn: every tensor must have q's dtype")
+    _check(dout.shape == q.shape and out.shape == q.shape and dq.shape == q.shape and dk.shape == k.shape and dv.shape == v.shape,
+           "flash_attn: dout, out and dq must look like q, dk like k, dv like v")
+    _check(dout.stride() == out.stride() and dq.stride() == q.stride() and dk.stride() == k.stride() and dv.stride() == v.stride(),
+           "flash_attn: dout must have the strides of out, and dq, dk, dv those of q, k, v")
+    _check(softmax_lse.dtype == torch.float32 and tuple(softmax_lse.shape) == (batch, heads, len_q) and softmax_lse.is_contiguous(),
+           "flash_attn: softmax_lse must be contiguous fp32 [B, H, len_q]")
+    pad = _pad_mask(key_padding_mask, batch, len_k)
+    kinfo = _key_info(batch, len_k, q.device) if pad is not None else None
+    mode, seed, offset, mask, bits = state[:5]
+    if dropout_p <= 0.0:
+        mode, bits = 0, None
+    ready = int(bits is not None)
+    if mode != 0 and bits is None:
+        bits = _bits(batch, heads, len_q, len_k, q.device)
+    softmax_d = torch.empty(batch, heads, len_q, dtype=torch.float32, device=q.device)
+    L.call("nmtg_flash_attn_batched_bwd", L.ptr(dout), L.ptr(q), L.ptr(k), L.ptr(v), L.ptr(out), L.ptr(softmax_lse), L.ptr(dq),
+           L.ptr(dk), L.ptr(dv), L.ptr(softmax_d), L.ptr(pad), L.ptr(kinfo), L.i64(batch), L.i64(heads), L.i64(d), L.i64(len_q),
+           L.i64(len_k), *_view4(q, "q", heads, d), *_view4(k, "k", heads, d), *_view4(v, "v", heads, d),
+           *_view4(out, "out", heads, d), L.f32(softmax_scale), L.i32(int(bool(causal))), L.i32(mode), L.f32(dropout_p),
+           L.ptr(mask if mode == 1 else None), L.ptr(bits), L.i32(ready), ctypes.c_uint64(seed), ctypes.c_uint64(offset),
+           L.i32(L.dtype_code(q)), L.stream_of(q))
+    return softmax_d

@@ -1,0 +1,175 @@
+"""Training calls of self_attn_func / encdec_attn_bias_func with return_coverage=False: the attention core runs as the
+tiled kernels over the padded batch (nmtg_flash_attn_batched_fwd / _bwd) and no [B*H, len_q, len_k] tensor is written.
+
+What the reference computes: onmt/modules/optimized/self_attention_func.py:50-520 and encdec_attention_func_bias.py:41-668
+with return_coverage false; checked against the same oracle as the calls that return the coverage (oracle/attention.py),
+to the same relative tolerance (util.assert_close: 2e-2, gradients' absolute part scaled by their magnitude). The absolute
+part is 4e-3 for bf16 instead of 1e-3: the oracle rounds the scores to the 16-bit type, as the extension's stored score
+tensor does, while the tiled core keeps them in fp32. A bf16 score of magnitude 4 moves by up to 2^-7 in that rounding and
+its probability by 0.8 %, which the signed sums of the context and of the output projection (values of order 0.1 to 1)
+turn into a few 1e-3 of absolute difference between two equally accurate results; fp16 rounds eight times finer.
+The batch-strided entry points are also held bit for bit against the packed ones on the sequences that both can express.
+"""
+import pytest
+import torch
+
+from nmtgminor_amd.modules.encdec_attention_func_bias import encdec_attn_bias_func
+from nmtgminor_amd.modules.self_attention_func import self_attn_func
+from nmtgminor_amd.native import flash_attn_cuda as fa
+from oracle import attention as oat, inputs
+from util import assert_close
+
+pytestmark = pytest.mark.gpu
+D = torch.float64
+ATOL = {torch.bfloat16: 4e-3, torch.float16: None}
+
+
+def _self_case(dev, t, b, e, h, dtype, p, pad_mask=None, seed=171, biases=True):
+    d = inputs.self_attn_inputs(t, b, e, h, dtype, p=p, seed=seed, zero_bias=False)
+    if pad_mask is not None:
+        d["pad_mask"] = pad_mask
+    if not biases:
+        d["b_in"] = d["b_out"] = None
+    fwd = oat.self_attn_fwd(d["x"], d["w_in"], d["w_out"], d["b_in"], d["b_out"], h, d["pad_mask"], None, p, d["dropout_mask"], D,
+                            round_to=dtype)
+    bwd = oat.self_attn_bwd(d["dout"], d["x"], d["w_in"], d["w_out"], h, fwd, p, d["dropout_mask"], D, round_to=dtype)
+    names = ("x", "w_in", "w_out", "b_in", "b_out")
+    leaves = [d[k].to(dev).requires_grad_() if d[k] is not None else None for k in names]
+    dm = d["dropout_mask"].to(dev) if p > 0 else None
+    out, cov = self_attn_func(False, True, h, leaves[0], leaves[1], leaves[2], leaves[3], leaves[4], d["pad_mask"].to(dev), p,
+                              False, None, False, None, True, False, False, dm)
+    assert cov.numel() == 0                               # the tiled core: no probability tensor exists
+    out.backward(d["dout"].to(dev))
+    assert_close(out, fwd["outputs"], dtype, "outputs", atol=ATOL[dtype])
+    for leaf, key in zip(leaves, ("dx", "dw_in", "dw_out", "db_in", "db_out")):
+        if leaf is not None:
+            assert_close(leaf.grad, bwd[key], dtype, key, atol=ATOL[dtype], scale_atol=True)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("t,b,e,h,p", [(64, 4, 256, 4, 0.0), (128, 3, 512, 8, 0.1), (200, 2, 256, 4, 0.25), (33, 2, 128, 2, 0.1),
+                                       (96, 2, 256, 2, 0.1)])
+def test_self_attention_training_without_coverage(dev, dtype, t, b, e, h, p):
+    _self_case(dev, t, b, e, h, dtype, p, biases=(t != 200))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_self_attention_with_masked_keys_anywhere(dev, dtype):
+    """The reference's mask is a byte per key, not a length: leading, scattered and trailing masked keys, a sequence whose
+    first two tiles of 64 keys are masked entirely, and one without masked keys."""
+    t, b = 200, 5
+    g = torch.Generator().manual_seed(9)
+    m = torch.zeros(b, t, dtype=torch.bool)
+    m[0, :3] = True
+    m[0, 150:] = True
+    m[1] = torch.rand(t, generator=g) < 0.3
+    m[1, 199] = False
+    m[2, :130] = True
+    m[3, 77] = True
+    _self_case(dev, t, b, 256, 4, dtype, 0.1, pad_mask=m)
+
+
+def _encdec_case(dev, tq, tk, b, e, h, dtype, p, seed=174, biases=True):
+    d = inputs.encdec_attn_inputs(tq, tk, b, e, h, dtype, p=p, seed=seed, zero_bias=False)
+    if not biases:
+        d["b_q"] = d["b_kv"] = d["b_out"] = None
+    fwd = oat.encdec_attn_fwd(d["x_q"], d["x_kv"], d["w_q"], d["w_kv"], d["w_out"], d["b_q"], d["b_kv"], d["b_out"], h,
+                              d["pad_mask"], p, d["dropout_mask"], D, round_to=dtype)
+    bwd = oat.encdec_attn_bwd(d["dout"], d["x_q"], d["x_kv"], d["w_q"], d["w_kv"], d["w_out"], h, fwd, p, d["dropout_mask"], D,
+                              round_to=dtype)
+    names = ("x_q", "x_kv", "w_q", "w_kv", "w_out", "b_q", "b_kv", "b_out")
+    leaf = {k: (d[k].to(dev).requires_grad_() if d[k] is not None else None) for k in names}
+    dm = d["dropout_mask"].to(dev) if p > 0 else None
+    res = encdec_attn_bias_func(False, True, h, leaf["x_q"], leaf["x_kv"], leaf["w_q"], leaf["w_kv"], leaf["w_out"], leaf["b_q"],
+                                leaf["b_kv"], leaf["b_out"], d["pad_mask"].to(dev), p, False, None, False, None, None, True, False,
+                                dm)
+    assert len(res) == 1
+    res[0].backward(d["dout"].to(dev))
+    assert_close(res[0], fwd["outputs"], dtype, "outputs", atol=ATOL[dtype])
+    for key, n in (("dx_q", "x_q"), ("dx_kv", "x_kv"), ("dw_q", "w_q"), ("dw_kv", "w_kv"), ("dw_out", "w_out"), ("db_q", "b_q"),
+                   ("db_kv", "b_kv"), ("db_out", "b_out")):
+        if leaf[n] is not None:
+            assert_close(leaf[n].grad, bwd[key], dtype, key, atol=ATOL[dtype], scale_atol=True)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("tq,tk,b,e,h,p", [(64, 512, 4, 256, 4, 0.0), (32, 1500, 2, 256, 4, 0.1), (17, 100, 3, 128, 2, 0.2),
+                                           (40, 130, 2, 256, 2, 0.1)])
+def test_encdec_attention_training_without_coverage(dev, dtype, tq, tk, b, e, h, p):
+    _encdec_case(dev, tq, tk, b, e, h, dtype, p, biases=(tq != 17))
+
+
+def test_the_switch_keeps_the_extension_path(dev, monkeypatch):
+    d = inputs.self_attn_inputs(32, 2, 128, 2, torch.bfloat16, p=0.0, seed=5)
+    g = lambda k: d[k].to(dev)
+    call = lambda: self_attn_func(False, True, 2, g("x"), g("w_in"), g("w_out"), g("b_in"), g("b_out"), g("pad_mask"), 0.0, False,
+                                  None, False, None, True, False, False)
+    out_tiled, cov = call()
+    assert cov.numel() == 0
+    monkeypatch.setenv("NMTG_ATTN_FLASH_TRAIN", "0")
+    out_ext, cov = call()
+    assert cov.shape == (4, 32, 32)
+    # two bf16 results, each within the tolerance of the exact one: twice the absolute part between them
+    assert_close(out_tiled, out_ext.float().cpu(), torch.bfloat16, "outputs of the two paths", atol=4e-3)
+
+
+def test_a_sequence_with_every_key_masked(dev):
+    """out = 0, lse = -inf and zero gradients for that sequence; the others are untouched by it."""
+    t, b, h, d = 70, 3, 2, 64
+    g = torch.Generator().manual_seed(3)
+    qkv = torch.randn(t, b, h, 3, d, generator=g).to(torch.bfloat16).to(dev)
+    do = torch.randn(t, b, h, d, generator=g).to(torch.bfloat16).to(dev)
+    pad = torch.zeros(b, t, dtype=torch.uint8)
+    pad[1] = 1
+    pad[2, 60:] = 1
+    pad = pad.to(dev)
+    q, k, v = qkv[:, :, :, 0], qkv[:, :, :, 1], qkv[:, :, :, 2]
+    out, lse, state = fa.fwd_batched(q, k, v, pad, 0.0, d ** -0.5, False)
+    assert (out[:, 1] == 0).all() and torch.isinf(lse[1]).all() and (lse[1] < 0).all()
+    assert torch.isfinite(out).all() and torch.isfinite(lse[0]).all() and torch.isfinite(lse[2]).all()
+    dqkv = torch.full_like(qkv, float("nan"))
+    fa.bwd_batched(do, q, k, v, out, lse, dqkv[:, :, :, 0], dqkv[:, :, :, 1], dqkv[:, :, :, 2], pad, 0.0, d ** -0.5, False, state)
+    assert torch.isfinite(dqkv).all()
+    assert (dqkv[:, 1] == 0).all() and (dqkv[60:, 2, :, 1:] == 0).all()
+
+
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("causal,p", [(False, 0.0), (True, 0.0), (False, 0.2), (True, 0.2)])
+def test_batch_strided_call_equals_packed_call_bit_for_bit(dev, d, causal, p):
+    """Sequences that end in masked keys are what both forms can express. The padded queries of the batch-strided call get
+    a zero output gradient, so that they add exact zeros to dK and dV; everything else must agree in every bit, the
+    Philox keep decisions included (they are indexed by sequence, head, query and key in both)."""
+    t, h, dtype = 150, 3, torch.float16
+    lens = [150, 97, 64, 1]
+    b = len(lens)
+    g = torch.Generator().manual_seed(17 + d)
+    qkv = torch.randn(t, b, h, 3, d, generator=g).to(dtype).to(dev)
+    do = torch.randn(t, b, h, d, generator=g).to(dtype).to(dev)
+    pad = torch.zeros(b, t, dtype=torch.uint8)
+    for i, n in enumerate(lens):
+        pad[i, n:] = 1
+        do[n:, i] = 0
+    pad = pad.to(dev)
+    scale, rng = d ** -0.5, (1234, 8)
+    q, k, v = qkv[:, :, :, 0], qkv[:, :, :, 1], qkv[:, :, :, 2]
+    out, lse, state = fa.fwd_batched(q, k, v, pad, p, scale, causal, rng=rng)
+    dqkv = torch.full_like(qkv, float("nan"))
+    fa.bwd_batched(do, q, k, v, out, lse, dqkv[:, :, :, 0], dqkv[:, :, :, 1], dqkv[:, :, :, 2], pad, p, scale, causal, state)
+
+    cu = torch.zeros(b + 1, dtype=torch.int32)
+    cu[1:] = torch.cumsum(torch.tensor(lens), 0)
+    cu = cu.to(dev)
+    pack = lambda x: torch.cat([x[:n, i] for i, n in enumerate(lens)], 0).contiguous()       # [tokens, ...]
+    pq, pk, pv, pdo = pack(q), pack(k), pack(v), pack(do)
+    pout = torch.empty_like(pq)
+    plse = fa.fwd(pq, pk, pv, pout, cu, cu, t, t, p, scale, False, causal, False, 0, None, rng=rng)[0]
+    pdq, pdk, pdv = torch.empty_like(pq), torch.empty_like(pk), torch.empty_like(pv)
+    fa.bwd(pdo, pq, pk, pv, pout, plse, pdq, pdk, pdv, cu, cu, t, t, p, scale, False, causal, 0, None, rng=fa.last_rng)
+    assert torch.equal(pack(out), pout)
+    for i, n in enumerate(lens):
+        assert torch.equal(lse[i, :, :n], plse[i, :, :n])
+    assert torch.equal(pack(dqkv[:, :, :, 0]), pdq)
+    assert torch.equal(pack(dqkv[:, :, :, 1]), pdk)
+    assert torch.equal(pack(dqkv[:, :, :, 2]), pdv)
+    for i, n in enumerate(lens):                                                              # masked keys: zero gradients
+        assert (dqkv[n:, i, :, 1:] == 0).all()
