@@ -305,6 +305,37 @@ class SelfAttnWL(Workload):
                     kind="port", sample=f"{nb} of {self.B} batch columns (independent), fp32 on the bf16-rounded values, median of 3")
 
 
+class _PlainCtx:
+    """What an autograd function's forward / backward need of their ctx, for a step that calls the two directly."""
+
+    def save_for_backward(self, *tensors):
+        self.saved_tensors = tensors
+
+
+class SelfAttnNoCoverageWL(SelfAttnWL):
+    name = "self_attn_no_coverage"
+    description = ("the self_attn workload as self_attn_func runs it in training with return_coverage=False: projections as "
+                   "GEMMs, attention core as tiled kernels over the padded batch, no [B*H, T, T] tensor (same inputs, mask, "
+                   "explicit dropout mask and FLOP count as self_attn)")
+
+    def setup(self, dev):
+        super().setup(dev)
+        from nmtgminor_amd.modules.flash_core import SelfAttnFlashFunc
+        self.fn = SelfAttnFlashFunc
+        self.w_in.requires_grad_()
+
+    def step(self):
+        with torch.no_grad():
+            c = _PlainCtx()
+            self.fn.forward(c, self.H, self.x, self.w_in, self.w_out, self.b_in, self.b_out, self.pad, 0.1, self.dm)
+            return self.fn.backward(c, self.dout)
+
+    def kernel_work(self):
+        t, b, e, h = self.T, self.B, self.E, self.H
+        core = 2 * (2.0 * b * h * t * t * (e // h))
+        return {"gemm_": 3 * (self._flops_fwd() - core), "flash_attn_bwd": 2 * core}
+
+
 class FlashAttnWL(Workload):
     name = "flash_attn"
     bound = "mfma"
@@ -768,7 +799,8 @@ class CopyWL(Workload):
 
 # the five benchmark configurations first, then the workloads added beside them
 WORKLOADS = {w.name: w for w in (LayerNormWL, MlpWL, SelfAttnWL, EncdecAttnWL, XentropyWL, SoftmaxDropoutWL, DropoutAddWL,
-                                    GeneratorLossWL, RelSelfAttnWL, FusedAdamWL, LayerNormLargeWL, FlashAttnWL, DecodeStepWL)}
+                                    GeneratorLossWL, RelSelfAttnWL, FusedAdamWL, LayerNormLargeWL, FlashAttnWL, DecodeStepWL,
+                                    SelfAttnNoCoverageWL)}
 EXTRA_WORKLOADS = {CopyWL.name: CopyWL}
 PRIMARY = "mlp"
 

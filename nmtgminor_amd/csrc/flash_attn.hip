@@ -214,10 +214,12 @@ __global__ __launch_bounds__(256) void flash_key_info_kernel(const uint8_t* pad,
   const int lk = max(max(part[0], part[1]), max(part[2], part[3]));
   int32_t* out = kinfo + static_cast<int64_t>(b) * pitch;
   if (tid == 0) out[0] = lk;
-  for (int t = tid; t < pitch - 1; t += 256) {
-    int any = 0;
-    for (int j = FA_TILE * t; j < min(FA_TILE * t + FA_TILE, lk); ++j) any |= row[j];
-    out[1 + t] = any != 0;
+  // one wavefront per tile: a key per lane
+  for (int t = tid >> 6; t < pitch - 1; t += 4) {
+    const int key = FA_TILE * t + (tid & 63);
+    const bool masked = key < lk && row[key] != 0;
+    const bool any = __builtin_amdgcn_ballot_w64(masked) != 0;
+    if ((tid & 63) == 0) out[1 + t] = any ? 1 : 0;
   }
 }
 
@@ -280,6 +282,31 @@ __global__ __launch_bounds__(256) void flash_bits_mask_kernel(FaArgs a, int64_t 
     if (qi < lq && a.mask[(static_cast<int64_t>(bh) * a.max_q + qi) * a.max_k + key] != 0) word |= 1u << i;
   }
   a.bits[row * a.kp + bit_slot(key)] = word;
+}
+
+// The same for four keys per thread, read as one word per query (max_k a multiple of 4, mask 4-byte aligned).
+__global__ __launch_bounds__(256) void flash_bits_mask4_kernel(FaArgs a, int64_t total) {
+  const int64_t id = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (id >= total) return;
+  const int k4n = a.kp / 4;
+  const int key0 = 4 * static_cast<int>(id % k4n);
+  const int64_t row = id / k4n;
+  const int grp = static_cast<int>(row % a.q32);
+  const int bh = static_cast<int>(row / a.q32), b = bh / a.heads;
+  const SeqSpan sp = seq_span(a, b);
+  if (32 * grp >= sp.lq || key0 >= sp.lk) return;     // key0 < lk <= max_k and max_k is a multiple of 4: key0 + 3 < max_k
+  const uint8_t* src = a.mask + (static_cast<int64_t>(bh) * a.max_q + 32 * grp) * a.max_k + key0;
+  const int nq = min(32, sp.lq - 32 * grp);
+  uint32_t word[4] = {0, 0, 0, 0};
+#pragma unroll 8
+  for (int i = 0; i < nq; ++i) {
+    const uint32_t m = *reinterpret_cast<const uint32_t*>(src + static_cast<int64_t>(i) * a.max_k);
+#pragma unroll
+    for (int kj = 0; kj < 4; ++kj) word[kj] |= (((m >> (8 * kj)) & 0xffu) != 0 ? 1u : 0u) << i;
+  }
+  uint32_t* out = a.bits + row * a.kp;
+#pragma unroll
+  for (int kj = 0; kj < 4; ++kj) out[bit_slot(key0 + kj)] = word[kj];
 }
 
 // The 32 lane masks of one 64-key tile for the wavefront's group of 32 queries: mask e belongs to accumulator register
@@ -1095,11 +1122,13 @@ int bits_launch(const char* what, FaArgs& a, int drop_mode, int64_t batch, void*
   a.kp = static_cast<int>(bits_kp(a.max_k));
   if (ready || a.max_q == 0 || a.max_k == 0) return 0;
   const int64_t rows = batch * a.heads * a.q32;
-  const int64_t total = rows * (drop_mode == 2 ? a.kp / 4 : a.kp);
+  const bool words = drop_mode == 1 && a.max_k % 4 == 0 && reinterpret_cast<uintptr_t>(a.mask) % 4 == 0;   // four keys per thread
+  const int64_t total = rows * (drop_mode == 2 || words ? a.kp / 4 : a.kp);
   NMTG_REQUIRE((total + 255) / 256 <= 0x7fffffff, "%s: keep-bit workspace beyond one launch", what);
   TraceScope trace("flash_attn_keep_bits", st);
   const dim3 grid(static_cast<unsigned>((total + 255) / 256));
   if (drop_mode == 2) hipLaunchKernelGGL(flash_bits_rng_kernel, grid, dim3(256), 0, st, a, total);
+  else if (words) hipLaunchKernelGGL(flash_bits_mask4_kernel, grid, dim3(256), 0, st, a, total);
   else hipLaunchKernelGGL(flash_bits_mask_kernel, grid, dim3(256), 0, st, a, total);
   return 0;
 }
