@@ -79,6 +79,43 @@ def test_self_attention_workload_weight_gradients_against_the_oracle(dev):
     assert_close(grads[4], bw["db_out"], BF, "db_out", scale_atol=True)
 
 
+def test_self_attention_workload_without_coverage(dev):
+    """The same workload through self_attn_func(return_coverage=False): the tiled core over the padded batch. Output and
+    input gradient of two batch columns against the oracle (every op up to dx is independent per column; bf16 absolute
+    part 4e-3, see tests/test_zzg_attention_no_coverage_gpu.py), weight gradients against those of the extension path on
+    the same inputs (two 16-bit results of the same sums), and a second run must repeat the first bit for bit."""
+    from nmtgminor_amd.modules.self_attention_func import self_attn_func
+    T, B, E, H = 512, 32, 1024, 16
+    d = inputs.self_attn_inputs(T, B, E, H)
+    names = ("x", "w_in", "w_out", "b_in", "b_out")
+
+    def run():
+        leaves = [d[k].to(dev).requires_grad_() for k in names]
+        out, cov = self_attn_func(False, True, H, *leaves, d["pad_mask"].to(dev), 0.1, False, None, False, None, True, False, False,
+                                  d["dropout_mask"].to(dev))
+        assert cov.numel() == 0
+        out.backward(d["dout"].to(dev))
+        return [out.detach()] + [z.grad for z in leaves]
+
+    got = run()
+    for col in (0, B - 1):
+        x1 = d["x"][:, col:col + 1]
+        dm1 = d["dropout_mask"].view(B, H, T, T)[col].reshape(H, T, T)
+        f = oat.self_attn_fwd(x1, d["w_in"], d["w_out"], d["b_in"], d["b_out"], H, d["pad_mask"][col:col + 1], None, 0.1, dm1,
+                              D, round_to=BF)
+        bw = oat.self_attn_bwd(d["dout"][:, col:col + 1], x1, d["w_in"], d["w_out"], H, f, 0.1, dm1, D, round_to=BF)
+        assert_close(got[0][:, col:col + 1], f["outputs"], BF, f"outputs[{col}]", atol=4e-3)
+        assert_close(got[1][:, col:col + 1], bw["dx"], BF, f"dx[{col}]", atol=4e-3, scale_atol=True)
+    g = lambda k: d[k].to(dev)
+    lin, scores, dropped, dmask, ctx, out = sa.forward(False, True, H, g("x"), g("w_in"), g("w_out"), g("b_in"), g("b_out"),
+                                                        g("pad_mask"), 0.1, dropout_mask=g("dropout_mask"))
+    ext = sa.backward(False, H, g("dout"), ctx, dropped, scores, lin, g("x"), g("w_in"), g("w_out"), dmask, 0.1)
+    for i, what in ((1, "dW_in"), (2, "dW_out"), (3, "db_in"), (4, "db_out")):
+        assert_close(got[1 + i], ext[i].float().cpu(), BF, what, atol=8e-3, scale_atol=True)
+    again = run()
+    assert all(torch.equal(a, b) for a, b in zip(got, again))
+
+
 def test_decoder_attention_workload(dev):
     TQ, TK, B, E, H = 128, 1500, 16, 1024, 16
     d = inputs.encdec_attn_inputs(TQ, TK, B, E, H)               # seed 1004, bf16, eval

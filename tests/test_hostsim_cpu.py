@@ -45,6 +45,7 @@ import test_zzc_relative_attention_gpu as trel  # noqa: E402
 import test_zzd_fused_optim_gpu as topt  # noqa: E402
 import test_zze_flash_attention_gpu as tfl  # noqa: E402
 import test_zzf_feed_forward_gpu as tff  # noqa: E402
+import test_zzg_attention_no_coverage_gpu as tnc  # noqa: E402
 
 pytestmark = pytest.mark.skipif(not hostsim_build.available(), reason="no host C++ compiler with __bf16 (ROCm clang++)")
 CPU = torch.device("cpu")
@@ -646,6 +647,22 @@ def test_packed_attention_dropout_philox_and_autograd_functions():
     tfl.test_dropout_drawn_on_the_device_is_the_documented_philox_stream_in_both_passes(CPU, F16, 64)
     tfl.test_packed_qkv_function_takes_strided_slots_and_fills_one_gradient_tensor(CPU, BF16)
     tfl.test_packed_kv_function_with_dropout_repeats_its_mask_in_the_backward(CPU)
+
+
+# ----------------------------------------------------------------------------- the same kernels over a padded batch
+def test_training_attention_without_coverage(mi355x, monkeypatch):
+    tnc.test_self_attention_training_without_coverage(CPU, BF16, 128, 3, 512, 8, 0.1)
+    tnc.test_self_attention_training_without_coverage(CPU, F16, 33, 2, 128, 2, 0.1)
+    tnc.test_self_attention_with_masked_keys_anywhere(CPU, BF16)
+    tnc.test_encdec_attention_training_without_coverage(CPU, F16, 17, 100, 3, 128, 2, 0.2)
+    tnc.test_encdec_attention_training_without_coverage(CPU, BF16, 40, 130, 2, 256, 2, 0.1)
+    tnc.test_a_sequence_with_every_key_masked(CPU)
+    tnc.test_the_switch_keeps_the_extension_path(CPU, monkeypatch)   # sets a switch: last
+
+
+@pytest.mark.parametrize("d,causal,p", [(64, True, 0.2), pytest.param(128, False, 0.2, marks=long_case), (64, False, 0.0)])
+def test_batch_strided_attention_equals_packed_attention_bit_for_bit(d, causal, p):
+    tnc.test_batch_strided_call_equals_packed_call_bit_for_bit(CPU, d, causal, p)
 
 
 def test_split_k_epilogue_without_a_workspace_is_refused_before_any_launch(hostsim_lib):
