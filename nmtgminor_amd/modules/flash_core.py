@@ -34,7 +34,8 @@ def _pad(mask, batch, len_k):
         return None
     if mask.numel() != batch * len_k:
         raise RuntimeError("key padding mask must be [batch, len_k]")
-    return mask.reshape(batch, len_k).to(torch.uint8).contiguous()
+    mask = mask.reshape(batch, len_k).contiguous()
+    return mask.view(torch.uint8) if mask.dtype == torch.bool else mask.to(torch.uint8)     # a bool mask is its bytes
 
 
 class SelfAttnFlashFunc(torch.autograd.Function):
