@@ -196,7 +196,7 @@ __device__ __forceinline__ SeqSpan seq_span(const FaArgs& a, int b) {
 }
 // whether key tile t of sequence b holds a masked key in front of the sequence's last live key
 __device__ __forceinline__ bool pad_tile(const FaArgs& a, int b, int t) {
-  return a.pad != nullptr && a.kinfo[static_cast<int64_t>(b) * a.kinfo_pitch + 1 + t] != 0;
+  return a.kinfo[static_cast<int64_t>(b) * a.kinfo_pitch + 1 + t] != 0;
 }
 
 // Key padding mask [B, max_k] -> key_info [B, 1 + ceil(max_k / 64)]: word 0 = 1 + the index of the last live key (0 when
@@ -346,7 +346,8 @@ __device__ __forceinline__ void store_rows_out(const acc16_t (&acc)[D / 32], flo
 // -------------------------------------------------------------------------------------------------------------------
 // forward
 // -------------------------------------------------------------------------------------------------------------------
-template <typename T, int D, int DROP>
+// PAD: the call has a key padding mask (batch-strided calls only); without it no mask code is compiled in.
+template <typename T, int D, int DROP, int PAD>
 __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(FaArgs a) {
   extern __shared__ __align__(16) uint8_t lds_raw[];
   constexpr int IMG = FA_TILE * D * 2;
@@ -374,7 +375,7 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
     for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
   float m = FA_NEG, l = 0.f;
   const float dead_raw = FA_NEG / a.scale_log2;   // the raw score that the scale turns into -1e30
-  const uint8_t* padrow = a.pad != nullptr ? a.pad + static_cast<int64_t>(b) * a.max_k : nullptr;   // read below lk only
+  [[maybe_unused]] const uint8_t* padrow = PAD != 0 ? a.pad + static_cast<int64_t>(b) * a.max_k : nullptr;   // read below lk only
 
   Staged<D> sk, sv;
   if (ntiles > 0) {
@@ -402,7 +403,7 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
       for (int n = 0; n < 2; ++n) mfma<T>::run(read_rows<D>(kimg, n, ss, lane), qf[ss], s[n]);
     // Masking only where the tile crosses the end of the keys or the causal diagonal (the same for the whole wavefront).
     // A masked raw score is the value that the scale turns into -1e30 or beyond: its probability is exp2 of that, 0.
-    const bool padt = pad_tile(a, b, t);
+    const bool padt = PAD != 0 && pad_tile(a, b, t);
     const bool edge = (t + 1) * FA_TILE > lk || (a.causal && t * FA_TILE + FA_TILE - 1 > q0 + 32 * wave) || padt;
     if (edge) {
 #pragma unroll
@@ -451,7 +452,7 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
         s[n][r] = pr;
         lsum += pr;
       }
-    if (padt) {
+    if (PAD != 0 && padt) {
       // A row that has met no live key yet still has the initial m, against which a dead score is not small: such
       // probabilities are set to 0 by hand. (Without masked keys inside the sequence, key 0 is live for every row.)
       lsum = 0.f;
@@ -500,7 +501,7 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
 // -------------------------------------------------------------------------------------------------------------------
 // backward, dQ and D = rowsum(dO * O)
 // -------------------------------------------------------------------------------------------------------------------
-template <typename T, int D, int DROP>
+template <typename T, int D, int DROP, int PAD>
 __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dq_kernel(FaArgs a) {
   extern __shared__ __align__(16) uint8_t lds_raw[];
   constexpr int IMG = FA_TILE * D * 2;
@@ -544,7 +545,7 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dq_kern
   const int ntiles = (nkeys + FA_TILE - 1) / FA_TILE;
   const int group = static_cast<int>(blockIdx.x) * (FA_ROWS / 32) + __builtin_amdgcn_readfirstlane(wave);   // of 32 queries
   const float dead_raw = FA_NEG / a.scale_log2;   // the raw score that the scale turns into -1e30
-  const uint8_t* padrow = a.pad != nullptr ? a.pad + static_cast<int64_t>(b) * a.max_k : nullptr;   // read below lk only
+  [[maybe_unused]] const uint8_t* padrow = PAD != 0 ? a.pad + static_cast<int64_t>(b) * a.max_k : nullptr;   // read below lk only
   acc16_t dq[D / 32];
 #pragma unroll
   for (int i = 0; i < D / 32; ++i)
@@ -582,7 +583,7 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dq_kern
         mfma<T>::run(read_rows<D>(vimg, n, ss, lane), gf[ss], dp[n]);
       }
     // masking as in the forward: only where the tile crosses the end of the keys or the causal diagonal
-    const bool padt = pad_tile(a, b, t);
+    const bool padt = PAD != 0 && pad_tile(a, b, t);
     if ((t + 1) * FA_TILE > lk || (a.causal && t * FA_TILE + FA_TILE - 1 > q0 + 32 * wave) || padt) {
 #pragma unroll
       for (int n = 0; n < 2; ++n)
@@ -1093,16 +1094,23 @@ int launch(K kern, const char* what, dim3 grid, int lds, hipStream_t st, const F
 template <typename T, int D>
 int fwd_launch(const FaArgs& a, int drop, dim3 grid, hipStream_t st) {
   TraceScope trace("flash_attn_fwd", st);
-  if (drop == 0) return launch(flash_fwd_kernel<T, D, 0>, "flash_attn_fwd", grid, fwd_lds<D>(), st, a);
-  return launch(flash_fwd_kernel<T, D, 1>, "flash_attn_fwd", grid, fwd_lds<D>(), st, a);
+  if (a.pad != nullptr)
+    return drop == 0 ? launch(flash_fwd_kernel<T, D, 0, 1>, "flash_attn_fwd", grid, fwd_lds<D>(), st, a)
+                     : launch(flash_fwd_kernel<T, D, 1, 1>, "flash_attn_fwd", grid, fwd_lds<D>(), st, a);
+  return drop == 0 ? launch(flash_fwd_kernel<T, D, 0, 0>, "flash_attn_fwd", grid, fwd_lds<D>(), st, a)
+                   : launch(flash_fwd_kernel<T, D, 1, 0>, "flash_attn_fwd", grid, fwd_lds<D>(), st, a);
 }
 template <typename T, int D>
 int bwd_launch(const FaArgs& a, int drop, dim3 grid_q, dim3 grid_k, hipStream_t st) {
   int rc = 0;
   if (grid_q.x > 0) {
     TraceScope trace("flash_attn_bwd_dq", st);
-    rc = drop == 0 ? launch(flash_bwd_dq_kernel<T, D, 0>, "flash_attn_bwd", grid_q, dq_lds<D>(), st, a)
-                   : launch(flash_bwd_dq_kernel<T, D, 1>, "flash_attn_bwd", grid_q, dq_lds<D>(), st, a);
+    if (a.pad != nullptr)
+      rc = drop == 0 ? launch(flash_bwd_dq_kernel<T, D, 0, 1>, "flash_attn_bwd", grid_q, dq_lds<D>(), st, a)
+                     : launch(flash_bwd_dq_kernel<T, D, 1, 1>, "flash_attn_bwd", grid_q, dq_lds<D>(), st, a);
+    else
+      rc = drop == 0 ? launch(flash_bwd_dq_kernel<T, D, 0, 0>, "flash_attn_bwd", grid_q, dq_lds<D>(), st, a)
+                     : launch(flash_bwd_dq_kernel<T, D, 1, 0>, "flash_attn_bwd", grid_q, dq_lds<D>(), st, a);
   }
   if (rc || grid_k.x == 0) return rc;
   TraceScope trace("flash_attn_bwd_dkv", st);
