@@ -8,7 +8,8 @@ and 17 gradient slots. As in the reference's fused branch (:81-126) the coverage
 probabilities BEFORE dropout (its Python fallback returns the dropped ones, :288-293). The mask is a key-padding mask
 [B, Tk] (or the broadcast form [B, 1, Tk]). Incremental decoding runs in nmtgminor_amd/modules/incremental.py; rotary
 encodings are applied by nmtgminor_amd/modules/rotary.py around the compact core. An 18th optional argument replays an
-explicit dropout keep-mask."""
+explicit dropout keep-mask. A training call with return_coverage false runs the tiled attention core of
+nmtgminor_amd/modules/flash_core.py."""
 import torch
 
 from ..native import encdec_multihead_attn_cuda as native
@@ -80,4 +81,10 @@ def encdec_attn_func(*args):
             r = EncdecAttnRotaryFunc.apply(is_training, heads, inputs_q, inputs_kv, w_q, w_kv, w_out, None, None, None, mask, p,
                                            pos_q[0], pos_q[1], pos_k[0], pos_k[1], args[17] if len(args) > 17 else None)
             return r if args[16] else (r[0],)
+        if len(args) >= 17 and not args[15]:          # training call whose coverage nobody reads: no [B*H, Tq, Tk] tensor
+            from . import flash_core
+            (recompute, is_training, heads, inputs_q, inputs_kv, w_q, w_kv, w_out, mask, p) = args[:10]
+            if flash_core.eligible(is_training, args[16], False, recompute, inputs_q, heads) and inputs_kv.dtype == inputs_q.dtype:
+                return (flash_core.EncdecAttnFlashFunc.apply(heads, inputs_q, inputs_kv, w_q, w_kv, w_out, None, None, None, mask, p,
+                                                             args[17] if len(args) > 17 else None),)
         return EncdecAttnFunc.apply(*args)

@@ -13,6 +13,7 @@ The batch-strided entry points are also held bit for bit against the packed ones
 import pytest
 import torch
 
+from nmtgminor_amd.modules.encdec_attention_func import encdec_attn_func
 from nmtgminor_amd.modules.encdec_attention_func_bias import encdec_attn_bias_func
 from nmtgminor_amd.modules.self_attention_func import self_attn_func
 from nmtgminor_amd.native import flash_attn_cuda as fa
@@ -97,6 +98,27 @@ def _encdec_case(dev, tq, tk, b, e, h, dtype, p, seed=174, biases=True):
                                            (40, 130, 2, 256, 2, 0.1)])
 def test_encdec_attention_training_without_coverage(dev, dtype, tq, tk, b, e, h, p):
     _encdec_case(dev, tq, tk, b, e, h, dtype, p, biases=(tq != 17))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_bias_free_encdec_function_without_coverage(dev, dtype):
+    """encdec_attn_func, the function the reference's EncdecMultiheadAttn binds, with the broadcast mask form [B, 1, Tk]."""
+    tq, tk, b, e, h, p = 24, 200, 3, 256, 4, 0.1
+    d = inputs.encdec_attn_inputs(tq, tk, b, e, h, dtype, p=p, seed=175)
+    fwd = oat.encdec_attn_fwd(d["x_q"], d["x_kv"], d["w_q"], d["w_kv"], d["w_out"], None, None, None, h, d["pad_mask"], p,
+                              d["dropout_mask"], D, round_to=dtype)
+    bwd = oat.encdec_attn_bwd(d["dout"], d["x_q"], d["x_kv"], d["w_q"], d["w_kv"], d["w_out"], h, fwd, p, d["dropout_mask"], D,
+                              round_to=dtype)
+    names = ("x_q", "x_kv", "w_q", "w_kv", "w_out")
+    leaf = {k: d[k].to(dev).requires_grad_() for k in names}
+    res = encdec_attn_func(False, True, h, leaf["x_q"], leaf["x_kv"], leaf["w_q"], leaf["w_kv"], leaf["w_out"],
+                           d["pad_mask"].to(dev).unsqueeze(1), p, False, None, False, None, None, False, False,
+                           d["dropout_mask"].to(dev))
+    assert len(res) == 1
+    res[0].backward(d["dout"].to(dev))
+    assert_close(res[0], fwd["outputs"], dtype, "outputs", atol=ATOL[dtype])
+    for key, n in (("dx_q", "x_q"), ("dx_kv", "x_kv"), ("dw_q", "w_q"), ("dw_kv", "w_kv"), ("dw_out", "w_out")):
+        assert_close(leaf[n].grad, bwd[key], dtype, key, atol=ATOL[dtype], scale_atol=True)
 
 
 def test_the_switch_keeps_the_extension_path(dev, monkeypatch):
