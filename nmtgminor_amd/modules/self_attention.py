@@ -36,8 +36,10 @@ class SelfMultiheadAttn(nn.Module):
         nn.init.constant_(self.out_proj_bias, 0.)
 
     def forward(self, inputs, pos=None, key_padding_mask=None, attn_mask=None, incremental=False,
-                incremental_cache=None, **kwargs):
-        """inputs [T, B, E]; key_padding_mask [B, T] (1 = pad) or attn_mask [T, T] (1 = masked)."""
+                incremental_cache=None, return_coverage=True, **kwargs):
+        """inputs [T, B, E]; key_padding_mask [B, T] (1 = pad) or attn_mask [T, T] (1 = masked). return_coverage (not in
+        the reference's module, which always asks for it): a caller that drops the coverage passes False, and a training
+        call with a key padding mask then writes no [B*H, T, T] tensor (the second result is an empty tensor)."""
         mask = None
         if key_padding_mask is not None:
             assert attn_mask is None, "ERROR attn_mask and key_padding_mask should not be both defined!"
@@ -52,5 +54,5 @@ class SelfMultiheadAttn(nn.Module):
         outputs, coverage = self.attn_func(attn_mask is not None, self.training, self.num_heads, inputs,
                                            self.in_proj_weight, self.out_proj_weight, self.in_proj_bias,
                                            self.out_proj_bias, mask, self.dropout, self.rotary_pos_enc, pos, incremental,
-                                           incremental_cache, True, True, False)
+                                           incremental_cache, True, bool(return_coverage), False)
         return outputs, coverage

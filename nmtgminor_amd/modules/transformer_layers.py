@@ -116,7 +116,7 @@ class EncoderLayer(_Layer):
         if self._alive():
             input = self._macaron_step(input)
             query = self.preprocess_attn(input)
-            out, _ = self.multihead(query, None, attn_mask, None)
+            out, _ = self.multihead(query, None, attn_mask, None, return_coverage=False)    # the coverage is dropped here
             input = self.postprocess_attn(self._survivor_scale(out), input)
             input = self._ffn_step(input)
         return _clamp_non_finite_(input)

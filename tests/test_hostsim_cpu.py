@@ -408,6 +408,10 @@ def test_encoder_layer(mi355x, dtype, macaron, training):
     tla.test_encoder_layer_matches_the_oracle(CPU, dtype, macaron, training)
 
 
+def test_encoder_layer_on_the_tiled_attention_core(mi355x, monkeypatch):
+    tla.test_encoder_layer_with_head_dimension_64_drops_the_coverage_and_runs_the_tiled_core(CPU, BF16, monkeypatch)
+
+
 @pytest.mark.parametrize("dtype", HALVES)
 @pytest.mark.parametrize("ignore_source", [False, pytest.param(True, marks=long_case)])
 def test_decoder_layer(mi355x, dtype, ignore_source):
@@ -657,6 +661,7 @@ def test_training_attention_without_coverage(mi355x, monkeypatch):
     tnc.test_encdec_attention_training_without_coverage(CPU, F16, 17, 100, 3, 128, 2, 0.2)
     tnc.test_encdec_attention_training_without_coverage(CPU, BF16, 40, 130, 2, 256, 2, 0.1)
     tnc.test_a_sequence_with_every_key_masked(CPU)
+    tnc.test_bias_free_encdec_function_without_coverage(CPU, F16)
     tnc.test_the_switch_keeps_the_extension_path(CPU, monkeypatch)   # sets a switch: last
 
 

@@ -92,8 +92,8 @@ def test_pre_post_processing_sequences(dev, dtype):
         PrePostProcessing(e, 0.1, multilingual=True, n_languages=3)
 
 
-def _encoder_case(dev, dtype, macaron, training, death_rate=0.0, seed=84):
-    opt = options(macaron=macaron)
+def _encoder_case(dev, dtype, macaron, training, death_rate=0.0, seed=84, **more):
+    opt = options(macaron=macaron, **more)
     t, b = 40, 3
     g = torch.Generator().manual_seed(seed)
     layer = randomise(EncoderLayer(opt, death_rate=death_rate), seed + 1)
@@ -130,6 +130,18 @@ def test_encoder_layer_matches_the_oracle(dev, dtype, macaron, training):
                   "mcr_feedforward.in_proj_weight", "mcr_feedforward.out_proj_weight", "mcr_feedforward.in_proj_bias",
                   "mcr_feedforward.out_proj_bias"}
     assert set(layer.state_dict()) == names
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_encoder_layer_with_head_dimension_64_drops_the_coverage_and_runs_the_tiled_core(dev, dtype, monkeypatch):
+    """The layer drops the coverage, so in training its self-attention writes no [B*H, T, T] tensor where the tiled core
+    takes the shape (head dimension 64 or 128; the other layer tests run heads of 32). Same oracle, same tolerance."""
+    from nmtgminor_amd.native import flash_attn_cuda
+    calls = []
+    real = flash_attn_cuda.fwd_batched
+    monkeypatch.setattr(flash_attn_cuda, "fwd_batched", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    _encoder_case(dev, dtype, False, True, model_size=256, inner_size=512, seed=86)
+    assert calls == [1]
 
 
 def test_encoder_layer_stochastic_depth(dev):
