@@ -327,7 +327,7 @@ class SelfAttnNoCoverageWL(SelfAttnWL):
     def step(self):
         with torch.no_grad():
             c = _PlainCtx()
-            self.fn.forward(c, self.H, self.x, self.w_in, self.w_out, self.b_in, self.b_out, self.pad, 0.1, self.dm)
+            self.fn.forward(c, False, self.H, self.x, self.w_in, self.w_out, self.b_in, self.b_out, self.pad, 0.1, self.dm)
             return self.fn.backward(c, self.dout)
 
     def kernel_work(self):

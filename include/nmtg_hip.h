@@ -412,6 +412,13 @@ int nmtg_flash_attn_bwd(const void* dout, const void* q, const void* k, const vo
  * key_info: with a mask, device workspace of nmtg_flash_attn_key_info_bytes(batch, len_k) bytes,
  * 4-byte aligned; a small kernel ahead of the others writes each sequence's last live key and
  * which 64-key tiles hold masked keys in front of it (only those tiles read the mask again).
+ * time_mask: NULL, or uint8 [len_q, len_k], 1 = masked, shared by every sequence and head (the
+ * reference's use_time_mask form; any pattern, a causal one included); not together with
+ * key_padding_mask. time_info: with it, device workspace of
+ * nmtg_flash_attn_time_info_bytes(len_q, len_k) bytes, 4-byte aligned: a small kernel classifies
+ * the mask by patches of 32 x 64 (no masked element / some / all) for both kernel orientations, the
+ * attention kernels stop at the last key tile (start at the first query tile) with a live element
+ * and read mask bytes only in patches that hold masked ones.
  * causal, dropout_*, seed, offset, softmax_lse [batch, heads, len_q], softmax_d: as above, with
  * max_seqlen_* = len_*.
  * nmtg_flash_attn_batched_bwd: dout has the strides of out; dq, dk, dv have the strides of q, k, v
@@ -419,8 +426,11 @@ int nmtg_flash_attn_bwd(const void* dout, const void* q, const void* k, const vo
  * ------------------------------------------------------------------------------------------ */
 int64_t nmtg_flash_attn_key_info_bytes(int64_t batch, int64_t len_k);
 
+int64_t nmtg_flash_attn_time_info_bytes(int64_t len_q, int64_t len_k);
+
 int nmtg_flash_attn_batched_fwd(const void* q, const void* k, const void* v, void* out,
-                                const uint8_t* key_padding_mask, void* key_info, float* softmax_lse,
+                                const uint8_t* key_padding_mask, void* key_info,
+                                const uint8_t* time_mask, void* time_info, float* softmax_lse,
                                 int64_t batch, int64_t heads, int64_t head_dim, int64_t len_q,
                                 int64_t len_k, int64_t q_stride_t, int64_t q_stride_b,
                                 int64_t q_stride_h, int64_t k_stride_t, int64_t k_stride_b,
@@ -434,7 +444,8 @@ int nmtg_flash_attn_batched_fwd(const void* q, const void* k, const void* v, voi
 int nmtg_flash_attn_batched_bwd(const void* dout, const void* q, const void* k, const void* v,
                                 const void* out, const float* softmax_lse, void* dq, void* dk,
                                 void* dv, float* softmax_d, const uint8_t* key_padding_mask,
-                                void* key_info, int64_t batch, int64_t heads, int64_t head_dim,
+                                void* key_info, const uint8_t* time_mask, void* time_info,
+                                int64_t batch, int64_t heads, int64_t head_dim,
                                 int64_t len_q, int64_t len_k, int64_t q_stride_t, int64_t q_stride_b,
                                 int64_t q_stride_h, int64_t k_stride_t, int64_t k_stride_b,
                                 int64_t k_stride_h, int64_t v_stride_t, int64_t v_stride_b,

@@ -47,6 +47,9 @@ struct FaArgs {
   const uint8_t* pad;    // batch-strided calls: key padding mask [B, max_k], 1 = masked, or null
   const int32_t* kinfo;  // with pad: [B, kinfo_pitch], see flash_key_info_kernel
   int kinfo_pitch;       // 1 + ceil(max_k / 64)
+  const uint8_t* tmask;  // batch-strided calls: time mask [max_q, max_k] shared by every sequence and head, 1 = masked, or null
+  const int32_t *qinfo, *kqinfo;   // with tmask: summaries by 32 queries x 64 keys and by 32 keys x 64 queries (flash_time_info_kernel)
+  int qinfo_pitch, kqinfo_pitch;   // 1 + ceil(max_k / 64) and 2 + ceil(max_q / 64)
   int heads, max_q, max_k;
   float scale, scale_log2;
   int causal;
@@ -194,9 +197,70 @@ __device__ __forceinline__ SeqSpan seq_span(const FaArgs& a, int b) {
   }
   return s;
 }
-// whether key tile t of sequence b holds a masked key in front of the sequence's last live key
-__device__ __forceinline__ bool pad_tile(const FaArgs& a, int b, int t) {
-  return a.kinfo[static_cast<int64_t>(b) * a.kinfo_pitch + 1 + t] != 0;
+// Whether key tile t holds masked keys that the sequence length does not already cut off, for the wavefront's group of
+// 32 queries. MODE 1: key padding mask (the same for every query of sequence b). MODE 2: time mask (the same for every
+// sequence). A tile of a time mask whose keys are all masked counts too (class 2; the blocks skip such tiles where they
+// lie behind the last live one, see tile_bound()).
+template <int MODE>
+__device__ __forceinline__ bool masked_tile(const FaArgs& a, int b, int group, int t) {
+  if constexpr (MODE == 1) return a.kinfo[static_cast<int64_t>(b) * a.kinfo_pitch + 1 + t] != 0;
+  else return a.qinfo[static_cast<int64_t>(group) * a.qinfo_pitch + 1 + t] != 0;
+}
+// the mask byte of (query qr, key): both inside the tensors
+template <int MODE>
+__device__ __forceinline__ bool masked_key(const FaArgs& a, const uint8_t* padrow, int qr, int key) {
+  if constexpr (MODE == 1) return padrow[key] != 0;
+  else return a.tmask[static_cast<int64_t>(qr) * a.max_k + key] != 0;
+}
+// time mask: the number of key tiles that a block of 128 queries has to visit (behind it every key is masked for all of them)
+__device__ __forceinline__ int tile_bound(const FaArgs& a, int block) {
+  const int groups = (a.max_q + 31) / 32;
+  int n = 0;
+  for (int i = 0; i < FA_ROWS / 32; ++i) n = max(n, a.qinfo[static_cast<int64_t>(min(4 * block + i, groups - 1)) * a.qinfo_pitch]);
+  return n;
+}
+
+// Time mask [max_q, max_k] -> the two summaries. Blocks 0 .. ceil(max_q / 32) - 1 write qinfo: per group of 32 queries,
+// word 0 = 1 + the last key tile with a live key (0: none), word 1 + t = class of tile t (0 no masked key, 1 some, 2 all).
+// The other blocks write kqinfo: per group of 32 keys, word 0 = the first tile of 64 queries with a live element (the tile
+// count if none), word 1 = 1 + the last one, word 2 + t = class of query tile t. Elements outside the mask do not count.
+__global__ __launch_bounds__(256) void flash_time_info_kernel(const uint8_t* tmask, int max_q, int max_k, int32_t* qinfo,
+                                                              int qpitch, int32_t* kqinfo, int kpitch) {
+  __shared__ int first[4], last[4];
+  const int tid = static_cast<int>(threadIdx.x), wave = tid >> 6, lane = tid & 63;
+  const int qgroups = (max_q + 31) / 32;
+  const bool by_query = static_cast<int>(blockIdx.x) < qgroups;
+  const int g = by_query ? static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x) - qgroups;
+  const int ntiles = by_query ? qpitch - 1 : kpitch - 2;
+  int32_t* out = by_query ? qinfo + static_cast<int64_t>(g) * qpitch + 1 : kqinfo + static_cast<int64_t>(g) * kpitch + 2;
+  int lo = ntiles, hi = 0;
+  for (int t = wave; t < ntiles; t += 4) {
+    // by_query: this lane's key against the group's 32 queries; otherwise this lane's query against the group's 32 keys
+    const int mine = FA_TILE * t + lane;
+    const bool valid = mine < (by_query ? max_k : max_q);
+    bool any = false, all = true;
+    if (valid)
+      for (int r = 0; r < 32; ++r) {
+        const int other = 32 * g + r;
+        if (other >= (by_query ? max_q : max_k)) break;
+        const int q = by_query ? other : mine, k = by_query ? mine : other;
+        const bool m = tmask[static_cast<int64_t>(q) * max_k + k] != 0;
+        any |= m;
+        all &= m;
+      }
+    const bool none_live = __builtin_amdgcn_ballot_w64(valid && !all) == 0;
+    const bool some_masked = __builtin_amdgcn_ballot_w64(valid && any) != 0;
+    const int cls = none_live ? 2 : some_masked ? 1 : 0;
+    if (lane == 0) out[t] = cls;
+    if (cls != 2) { lo = min(lo, t); hi = max(hi, t + 1); }
+  }
+  if (lane == 0) { first[wave] = lo; last[wave] = hi; }
+  __syncthreads();
+  if (tid == 0) {
+    const int f = min(min(first[0], first[1]), min(first[2], first[3])), l = max(max(last[0], last[1]), max(last[2], last[3]));
+    if (by_query) out[-1] = l;
+    else { out[-2] = f; out[-1] = l; }
+  }
 }
 
 // Key padding mask [B, max_k] -> key_info [B, 1 + ceil(max_k / 64)]: word 0 = 1 + the index of the last live key (0 when
@@ -365,7 +429,8 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
   load_resident<T, D>(qf, qb, a.q_st, qrow, lq, lane);
 
   const int nkeys = a.causal ? min(lk, q0 + FA_ROWS) : lk;
-  const int ntiles = (nkeys + FA_TILE - 1) / FA_TILE;
+  int ntiles = (nkeys + FA_TILE - 1) / FA_TILE;
+  if constexpr (PAD == 2) ntiles = min(ntiles, tile_bound(a, static_cast<int>(blockIdx.x)));
   const int group = static_cast<int>(blockIdx.x) * (FA_ROWS / 32) + __builtin_amdgcn_readfirstlane(wave);   // of 32 queries
 
   acc16_t o[D / 32];
@@ -375,7 +440,8 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
     for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
   float m = FA_NEG, l = 0.f;
   const float dead_raw = FA_NEG / a.scale_log2;   // the raw score that the scale turns into -1e30
-  [[maybe_unused]] const uint8_t* padrow = PAD != 0 ? a.pad + static_cast<int64_t>(b) * a.max_k : nullptr;   // read below lk only
+  [[maybe_unused]] const uint8_t* padrow = PAD == 1 ? a.pad + static_cast<int64_t>(b) * a.max_k : nullptr;   // read below lk only
+  [[maybe_unused]] const int qr = min(qrow, lq - 1);   // the row whose time-mask bytes this lane reads
 
   Staged<D> sk, sv;
   if (ntiles > 0) {
@@ -403,7 +469,22 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
       for (int n = 0; n < 2; ++n) mfma<T>::run(read_rows<D>(kimg, n, ss, lane), qf[ss], s[n]);
     // Masking only where the tile crosses the end of the keys or the causal diagonal (the same for the whole wavefront).
     // A masked raw score is the value that the scale turns into -1e30 or beyond: its probability is exp2 of that, 0.
-    const bool padt = PAD != 0 && pad_tile(a, b, t);
+    // bit 16 n + r of mdead: the mask hides key (n, r) of the tile from this lane's query. The 32 bytes are requested
+    // together, ahead of the masking.
+    bool padt = false;
+    [[maybe_unused]] uint32_t mdead = 0;
+    if constexpr (PAD != 0) {
+      padt = masked_tile<PAD>(a, b, min(group, (a.max_q + 31) / 32 - 1), t);
+      if (padt) {
+#pragma unroll
+        for (int n = 0; n < 2; ++n)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int key = t * FA_TILE + 32 * n + 8 * (r / 4) + 4 * half + r % 4;
+            mdead |= (masked_key<PAD>(a, padrow, qr, min(key, lk - 1)) ? 1u : 0u) << (16 * n + r);
+          }
+      }
+    }
     const bool edge = (t + 1) * FA_TILE > lk || (a.causal && t * FA_TILE + FA_TILE - 1 > q0 + 32 * wave) || padt;
     if (edge) {
 #pragma unroll
@@ -411,7 +492,9 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int key = t * FA_TILE + 32 * n + 8 * (r / 4) + 4 * half + r % 4;
-          if (key >= lk || (a.causal && key > qrow) || (padt && padrow[key] != 0)) s[n][r] = dead_raw;
+          bool dead = key >= lk || (a.causal && key > qrow);
+          if constexpr (PAD != 0) dead = dead || ((mdead >> (16 * n + r)) & 1u) != 0;
+          if (dead) s[n][r] = dead_raw;
         }
     }
     // tile maximum of the scaled scores from the extreme raw score (one multiplication instead of 32)
@@ -452,7 +535,7 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
         s[n][r] = pr;
         lsum += pr;
       }
-    if (PAD != 0 && padt) {
+    if constexpr (PAD != 0) if (padt) {
       // A row that has met no live key yet still has the initial m, against which a dead score is not small: such
       // probabilities are set to 0 by hand. (Without masked keys inside the sequence, key 0 is live for every row.)
       lsum = 0.f;
@@ -461,7 +544,7 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int key = t * FA_TILE + 32 * n + 8 * (r / 4) + 4 * half + r % 4;
-          if (key >= lk || (a.causal && key > qrow) || padrow[key] != 0) s[n][r] = 0.f;
+          if (key >= lk || (a.causal && key > qrow) || ((mdead >> (16 * n + r)) & 1u) != 0) s[n][r] = 0.f;
           lsum += s[n][r];
         }
     }
@@ -542,10 +625,12 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dq_kern
   }
 
   const int nkeys = a.causal ? min(lk, q0 + FA_ROWS) : lk;
-  const int ntiles = (nkeys + FA_TILE - 1) / FA_TILE;
+  int ntiles = (nkeys + FA_TILE - 1) / FA_TILE;
+  if constexpr (PAD == 2) ntiles = min(ntiles, tile_bound(a, static_cast<int>(blockIdx.x)));
   const int group = static_cast<int>(blockIdx.x) * (FA_ROWS / 32) + __builtin_amdgcn_readfirstlane(wave);   // of 32 queries
   const float dead_raw = FA_NEG / a.scale_log2;   // the raw score that the scale turns into -1e30
-  [[maybe_unused]] const uint8_t* padrow = PAD != 0 ? a.pad + static_cast<int64_t>(b) * a.max_k : nullptr;   // read below lk only
+  [[maybe_unused]] const uint8_t* padrow = PAD == 1 ? a.pad + static_cast<int64_t>(b) * a.max_k : nullptr;   // read below lk only
+  [[maybe_unused]] const int qr = min(qrow, lq - 1);   // the row whose time-mask bytes this lane reads
   acc16_t dq[D / 32];
 #pragma unroll
   for (int i = 0; i < D / 32; ++i)
@@ -583,14 +668,31 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dq_kern
         mfma<T>::run(read_rows<D>(vimg, n, ss, lane), gf[ss], dp[n]);
       }
     // masking as in the forward: only where the tile crosses the end of the keys or the causal diagonal
-    const bool padt = PAD != 0 && pad_tile(a, b, t);
+    // bit 16 n + r of mdead: the mask hides key (n, r) of the tile from this lane's query. The 32 bytes are requested
+    // together, ahead of the masking.
+    bool padt = false;
+    [[maybe_unused]] uint32_t mdead = 0;
+    if constexpr (PAD != 0) {
+      padt = masked_tile<PAD>(a, b, min(group, (a.max_q + 31) / 32 - 1), t);
+      if (padt) {
+#pragma unroll
+        for (int n = 0; n < 2; ++n)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int key = t * FA_TILE + 32 * n + 8 * (r / 4) + 4 * half + r % 4;
+            mdead |= (masked_key<PAD>(a, padrow, qr, min(key, lk - 1)) ? 1u : 0u) << (16 * n + r);
+          }
+      }
+    }
     if ((t + 1) * FA_TILE > lk || (a.causal && t * FA_TILE + FA_TILE - 1 > q0 + 32 * wave) || padt) {
 #pragma unroll
       for (int n = 0; n < 2; ++n)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int key = t * FA_TILE + 32 * n + 8 * (r / 4) + 4 * half + r % 4;
-          if (key >= lk || (a.causal && key > qrow) || (padt && padrow[key] != 0)) s[n][r] = dead_raw;
+          bool dead = key >= lk || (a.causal && key > qrow);
+          if constexpr (PAD != 0) dead = dead || ((mdead >> (16 * n + r)) & 1u) != 0;
+          if (dead) s[n][r] = dead_raw;
         }
     }
     [[maybe_unused]] const uint64_t* lane_mask = DROP != 0 ? tile_lane_masks(a, bh, group, t) : nullptr;
@@ -627,7 +729,8 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dq_kern
 // -------------------------------------------------------------------------------------------------------------------
 // backward, dK and dV: one key per lane pair, query tiles of 64 streamed through LDS
 // -------------------------------------------------------------------------------------------------------------------
-template <typename T, int D, int DROP>
+// TM: the call has a time mask; without it none of that code is compiled in.
+template <typename T, int D, int DROP, int TM>
 __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dkv_kernel(FaArgs a) {
   extern __shared__ __align__(16) uint8_t lds_raw[];
   constexpr int IMG = FA_TILE * D * 2;
@@ -668,8 +771,22 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dkv_ker
   load_resident<T, D>(vf, vb, a.v_st, krow, lk, lane);
 
   // causal: queries before the block's first key see none of its keys
-  const int t0 = a.causal ? k0 / FA_TILE : 0;
-  const int ntiles = (lq + FA_TILE - 1) / FA_TILE;
+  int t0 = a.causal ? k0 / FA_TILE : 0;
+  int ntiles = (lq + FA_TILE - 1) / FA_TILE;
+  // time mask: the block's four groups of 32 keys know the first and the last query tile with a live element
+  const int kgroups = (a.max_k + 31) / 32;
+  const int kgroup = min(static_cast<int>(blockIdx.x) * (FA_ROWS / 32) + __builtin_amdgcn_readfirstlane(wave), kgroups - 1);
+  if constexpr (TM != 0) {
+    int lo = ntiles, hi = 0;
+    for (int i = 0; i < FA_ROWS / 32; ++i) {
+      const int32_t* row = a.kqinfo + static_cast<int64_t>(min(static_cast<int>(blockIdx.x) * (FA_ROWS / 32) + i, kgroups - 1)) * a.kqinfo_pitch;
+      lo = min(lo, row[0]);
+      hi = max(hi, row[1]);
+    }
+    t0 = max(t0, lo);
+    ntiles = min(ntiles, hi);
+  }
+  const int krow_c = min(krow, a.max_k - 1);   // the column whose time-mask bytes this lane reads
   const float dead_raw = FA_NEG / a.scale_log2;   // the raw score that the scale turns into -1e30
   acc16_t dk[D / 32], dv[D / 32];
 #pragma unroll
@@ -733,13 +850,30 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dkv_ker
       }
     // s[n][r]: query 32 n + 8 (r / 4) + 4 half + r % 4 of the tile, key krow. P (dropped, scaled) stays in dp's place
     // for dV, dS goes to s for dK.
-    if (wave_dead || (a.causal && t * FA_TILE < k0 + 32 * wave + 31)) {
+    // time mask: bit 16 n + r of tdead = the mask hides query (n, r) of the tile from this lane's key; the 32 bytes are
+    // requested together, ahead of the masking. (Here and in the other two kernels a form with each byte load inside
+    // the masking condition of its element passed on the CPU and gave wrong gradients on the GPU in some of the
+    // head-dimension-64 variants; with the loads gathered first every variant agrees bit for bit with the causal flag.)
+    bool tmt = false;
+    if constexpr (TM != 0) tmt = a.kqinfo[static_cast<int64_t>(kgroup) * a.kqinfo_pitch + 2 + t] != 0;
+    uint32_t tdead = 0;
+    if (TM != 0 && tmt) {
+      const uint8_t* col = a.tmask + krow_c;
 #pragma unroll
       for (int n = 0; n < 2; ++n)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int qi = t * FA_TILE + 32 * n + 8 * (r / 4) + 4 * half + r % 4;
-          if (kdead || (a.causal && krow > qi)) s[n][r] = dead_raw;
+          tdead |= (col[static_cast<int64_t>(min(qi, lq - 1)) * a.max_k] != 0 ? 1u : 0u) << (16 * n + r);
+        }
+    }
+    if (wave_dead || (a.causal && t * FA_TILE < k0 + 32 * wave + 31) || tmt) {
+#pragma unroll
+      for (int n = 0; n < 2; ++n)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int qi = t * FA_TILE + 32 * n + 8 * (r / 4) + 4 * half + r % 4;
+          if (kdead || (a.causal && krow > qi) || ((tdead >> (16 * n + r)) & 1u) != 0) s[n][r] = dead_raw;
         }
     }
     // keep bits of this lane's key for the tile's two groups of 32 queries, shifted so that bit 8 g + c is register 4 g + c
@@ -1094,6 +1228,9 @@ int launch(K kern, const char* what, dim3 grid, int lds, hipStream_t st, const F
 template <typename T, int D>
 int fwd_launch(const FaArgs& a, int drop, dim3 grid, hipStream_t st) {
   TraceScope trace("flash_attn_fwd", st);
+  if (a.tmask != nullptr)
+    return drop == 0 ? launch(flash_fwd_kernel<T, D, 0, 2>, "flash_attn_fwd", grid, fwd_lds<D>(), st, a)
+                     : launch(flash_fwd_kernel<T, D, 1, 2>, "flash_attn_fwd", grid, fwd_lds<D>(), st, a);
   if (a.pad != nullptr)
     return drop == 0 ? launch(flash_fwd_kernel<T, D, 0, 1>, "flash_attn_fwd", grid, fwd_lds<D>(), st, a)
                      : launch(flash_fwd_kernel<T, D, 1, 1>, "flash_attn_fwd", grid, fwd_lds<D>(), st, a);
@@ -1105,7 +1242,10 @@ int bwd_launch(const FaArgs& a, int drop, dim3 grid_q, dim3 grid_k, hipStream_t 
   int rc = 0;
   if (grid_q.x > 0) {
     TraceScope trace("flash_attn_bwd_dq", st);
-    if (a.pad != nullptr)
+    if (a.tmask != nullptr)
+      rc = drop == 0 ? launch(flash_bwd_dq_kernel<T, D, 0, 2>, "flash_attn_bwd", grid_q, dq_lds<D>(), st, a)
+                     : launch(flash_bwd_dq_kernel<T, D, 1, 2>, "flash_attn_bwd", grid_q, dq_lds<D>(), st, a);
+    else if (a.pad != nullptr)
       rc = drop == 0 ? launch(flash_bwd_dq_kernel<T, D, 0, 1>, "flash_attn_bwd", grid_q, dq_lds<D>(), st, a)
                      : launch(flash_bwd_dq_kernel<T, D, 1, 1>, "flash_attn_bwd", grid_q, dq_lds<D>(), st, a);
     else
@@ -1114,8 +1254,11 @@ int bwd_launch(const FaArgs& a, int drop, dim3 grid_q, dim3 grid_k, hipStream_t 
   }
   if (rc || grid_k.x == 0) return rc;
   TraceScope trace("flash_attn_bwd_dkv", st);
-  return drop == 0 ? launch(flash_bwd_dkv_kernel<T, D, 0>, "flash_attn_bwd", grid_k, dkv_lds<D>(), st, a)
-                   : launch(flash_bwd_dkv_kernel<T, D, 1>, "flash_attn_bwd", grid_k, dkv_lds<D>(), st, a);
+  if (a.tmask != nullptr)
+    return drop == 0 ? launch(flash_bwd_dkv_kernel<T, D, 0, 1>, "flash_attn_bwd", grid_k, dkv_lds<D>(), st, a)
+                     : launch(flash_bwd_dkv_kernel<T, D, 1, 1>, "flash_attn_bwd", grid_k, dkv_lds<D>(), st, a);
+  return drop == 0 ? launch(flash_bwd_dkv_kernel<T, D, 0, 0>, "flash_attn_bwd", grid_k, dkv_lds<D>(), st, a)
+                   : launch(flash_bwd_dkv_kernel<T, D, 1, 0>, "flash_attn_bwd", grid_k, dkv_lds<D>(), st, a);
 }
 
 int64_t bits_q32(int64_t max_q) { return 4 * ((max_q + FA_ROWS - 1) / FA_ROWS); }
@@ -1215,6 +1358,29 @@ int key_info_launch(const char* what, FaArgs& a, int64_t batch, const uint8_t* p
   TraceScope trace("flash_attn_key_info", st);
   hipLaunchKernelGGL(flash_key_info_kernel, dim3(static_cast<unsigned>(batch)), dim3(256), 0, st, pad, a.max_k,
                      static_cast<int32_t*>(key_info), a.kinfo_pitch);
+  return 0;
+}
+
+// the time mask of a batch-strided call: fills time_info (the two summaries, one behind the other) ahead of every kernel
+int64_t time_info_words(int64_t len_q, int64_t len_k) {
+  return (len_q + 31) / 32 * (1 + (len_k + FA_TILE - 1) / FA_TILE) + (len_k + 31) / 32 * (2 + (len_q + FA_TILE - 1) / FA_TILE);
+}
+int time_info_launch(const char* what, FaArgs& a, const uint8_t* time_mask, void* time_info, hipStream_t st) {
+  if (time_mask == nullptr) return 0;
+  NMTG_REQUIRE(a.pad == nullptr, "%s: a key padding mask or a time mask, not both", what);
+  NMTG_REQUIRE(time_info != nullptr && reinterpret_cast<uintptr_t>(time_info) % 4 == 0,
+               "%s: a time mask needs the time_info workspace (nmtg_flash_attn_time_info_bytes)", what);
+  if (a.max_q == 0 || a.max_k == 0) return 0;
+  const int qgroups = (a.max_q + 31) / 32, kgroups = (a.max_k + 31) / 32;
+  a.tmask = time_mask;
+  a.qinfo_pitch = 1 + (a.max_k + FA_TILE - 1) / FA_TILE;
+  a.kqinfo_pitch = 2 + (a.max_q + FA_TILE - 1) / FA_TILE;
+  int32_t* base = static_cast<int32_t*>(time_info);
+  a.qinfo = base;
+  a.kqinfo = base + static_cast<int64_t>(qgroups) * a.qinfo_pitch;
+  TraceScope trace("flash_attn_time_info", st);
+  hipLaunchKernelGGL(flash_time_info_kernel, dim3(static_cast<unsigned>(qgroups + kgroups)), dim3(256), 0, st, time_mask, a.max_q,
+                     a.max_k, base, a.qinfo_pitch, base + static_cast<int64_t>(qgroups) * a.qinfo_pitch, a.kqinfo_pitch);
   return 0;
 }
 
@@ -1349,8 +1515,13 @@ extern "C" int64_t nmtg_flash_attn_key_info_bytes(int64_t batch, int64_t len_k) 
   return batch * (1 + (len_k + FA_TILE - 1) / FA_TILE) * 4;
 }
 
+extern "C" int64_t nmtg_flash_attn_time_info_bytes(int64_t len_q, int64_t len_k) {
+  if (len_q <= 0 || len_k <= 0) return 0;
+  return time_info_words(len_q, len_k) * 4;
+}
+
 extern "C" int nmtg_flash_attn_batched_fwd(const void* q, const void* k, const void* v, void* out, const uint8_t* key_padding_mask,
-                                           void* key_info, float* softmax_lse, int64_t batch, int64_t heads, int64_t head_dim,
+                                           void* key_info, const uint8_t* time_mask, void* time_info, float* softmax_lse, int64_t batch, int64_t heads, int64_t head_dim,
                                            int64_t len_q, int64_t len_k, int64_t q_stride_t, int64_t q_stride_b, int64_t q_stride_h,
                                            int64_t k_stride_t, int64_t k_stride_b, int64_t k_stride_h, int64_t v_stride_t,
                                            int64_t v_stride_b, int64_t v_stride_h, int64_t out_stride_t, int64_t out_stride_b,
@@ -1378,12 +1549,14 @@ extern "C" int nmtg_flash_attn_batched_fwd(const void* q, const void* k, const v
   set_dropout(a, dropout_mode, dropout_p, seed, offset);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (int rc = key_info_launch(what, a, batch, key_padding_mask, key_info, st)) return rc;
+  if (int rc = time_info_launch(what, a, time_mask, time_info, st)) return rc;
   return fwd_run(what, a, batch, head_dim, dropout_mode, dropout_bits, dtype, st);
 }
 
 extern "C" int nmtg_flash_attn_batched_bwd(const void* dout, const void* q, const void* k, const void* v, const void* out,
                                            const float* softmax_lse, void* dq, void* dk, void* dv, float* softmax_d,
-                                           const uint8_t* key_padding_mask, void* key_info, int64_t batch, int64_t heads,
+                                           const uint8_t* key_padding_mask, void* key_info, const uint8_t* time_mask,
+                                           void* time_info, int64_t batch, int64_t heads,
                                            int64_t head_dim, int64_t len_q, int64_t len_k, int64_t q_stride_t, int64_t q_stride_b,
                                            int64_t q_stride_h, int64_t k_stride_t, int64_t k_stride_b, int64_t k_stride_h,
                                            int64_t v_stride_t, int64_t v_stride_b, int64_t v_stride_h, int64_t out_stride_t,
@@ -1415,5 +1588,6 @@ extern "C" int nmtg_flash_attn_batched_bwd(const void* dout, const void* q, cons
   set_dropout(a, dropout_mode, dropout_p, seed, offset);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (int rc = key_info_launch(what, a, batch, key_padding_mask, key_info, st)) return rc;
+  if (int rc = time_info_launch(what, a, time_mask, time_info, st)) return rc;
   return bwd_run(what, a, batch, head_dim, dropout_mode, dropout_bits, dropout_bits_ready != 0, dtype, st);
 }

@@ -84,7 +84,7 @@ def encdec_attn_func(*args):
         if len(args) >= 17 and not args[15]:          # training call whose coverage nobody reads: no [B*H, Tq, Tk] tensor
             from . import flash_core
             (recompute, is_training, heads, inputs_q, inputs_kv, w_q, w_kv, w_out, mask, p) = args[:10]
-            if flash_core.eligible(is_training, args[16], False, recompute, inputs_q, heads) and inputs_kv.dtype == inputs_q.dtype:
+            if flash_core.eligible(is_training, args[16], recompute, inputs_q, heads) and inputs_kv.dtype == inputs_q.dtype:
                 return (flash_core.EncdecAttnFlashFunc.apply(heads, inputs_q, inputs_kv, w_q, w_kv, w_out, None, None, None, mask, p,
                                                              args[17] if len(args) > 17 else None),)
         return EncdecAttnFunc.apply(*args)

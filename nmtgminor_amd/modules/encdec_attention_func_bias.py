@@ -83,7 +83,7 @@ def encdec_attn_bias_func(*args):
         if len(args) >= 20:                           # training call whose coverage nobody reads: no [B*H, Tq, Tk] tensor
             from . import flash_core
             (recompute, is_training, heads, inputs_q, inputs_kv, w_q, w_kv, w_out, b_q, b_kv, b_out, mask, p) = args[:13]
-            if flash_core.eligible(is_training, args[19], False, recompute, inputs_q, heads) and inputs_kv.dtype == inputs_q.dtype:
+            if flash_core.eligible(is_training, args[19], recompute, inputs_q, heads) and inputs_kv.dtype == inputs_q.dtype:
                 return (flash_core.EncdecAttnFlashFunc.apply(heads, inputs_q, inputs_kv, w_q, w_kv, w_out, b_q, b_kv, b_out, mask,
                                                              p, args[20] if len(args) > 20 else None),)
         return EncdecAttnBiasFunc.apply(*args)

@@ -8,9 +8,10 @@ nmtg_flash_attn_batched_fwd / _bwd on the slots of the projections (queries, key
 projection GEMM left them, and their gradients are written into the slots of one gradient buffer): per call the forward
 keeps the projections, the context, one fp32 per (sequence, head, query) and one bit per element of the dropout mask.
 
-Taken when: training mode, return_coverage false, no time mask, no recompute, 16-bit tensors, head dimension 64 or 128.
-The mask is the reference's key padding mask ([B, len_k] or [B, 1, 1, len_k], 1 = masked) or None. A query whose keys
-are all masked gets a zero context here (the reference's softmax gives NaN). NMTG_ATTN_FLASH_TRAIN=0 keeps such calls on
+Taken when: training mode, return_coverage false, no recompute, 16-bit tensors, head dimension 64 or 128.
+The mask is the reference's key padding mask ([B, len_k] or [B, 1, 1, len_k], 1 = masked), its time mask ([len_q, len_k]
+with use_time_mask, any pattern) or None. A query whose keys are all masked gets a zero context here (the reference's
+softmax gives NaN). NMTG_ATTN_FLASH_TRAIN=0 keeps such calls on
 the extension's path."""
 import os
 
@@ -20,8 +21,8 @@ from ..native import flash_attn_cuda as fa
 from .rotary import _linear, _linear_bwd
 
 
-def eligible(is_training, return_coverage, use_time_mask, recompute, x, heads):
-    if not is_training or return_coverage or use_time_mask or recompute:
+def eligible(is_training, return_coverage, recompute, x, heads):
+    if not is_training or return_coverage or recompute:
         return False
     if os.environ.get("NMTG_ATTN_FLASH_TRAIN", "1") == "0":
         return False
@@ -38,29 +39,38 @@ def _pad(mask, batch, len_k):
     return mask.view(torch.uint8) if mask.dtype == torch.bool else mask.to(torch.uint8)     # a bool mask is its bytes
 
 
+def _time(mask, len_q, len_k):
+    if mask is None or mask.numel() == 0:
+        return None
+    if mask.numel() != len_q * len_k:
+        raise RuntimeError("time mask must be [len_q, len_k]")
+    return _pad(mask, len_q, len_k)
+
+
 class SelfAttnFlashFunc(torch.autograd.Function):
-    """apply(heads, inputs, input_weights, output_weights, input_biases, output_biases, mask, dropout_prob,
-    dropout_mask=None) -> outputs [T, B, E]"""
+    """apply(use_time_mask, heads, inputs, input_weights, output_weights, input_biases, output_biases, mask, dropout_prob,
+    dropout_mask=None) -> outputs [T, B, E]; mask: key padding [B, T], or with use_time_mask a time mask [T, T]"""
 
     @staticmethod
-    def forward(ctx, heads, inputs, w_in, w_out, b_in, b_out, mask, p, dropout_mask=None):
+    def forward(ctx, use_time_mask, heads, inputs, w_in, w_out, b_in, b_out, mask, p, dropout_mask=None):
         inputs = inputs.contiguous()
         t, bsz, e = inputs.shape
         d = e // heads
         lin = _linear(inputs, w_in, b_in)                               # [T, B, H, 3, D]
         slots = lin.view(t, bsz, heads, 3, d)
-        pad = _pad(mask, bsz, t)
+        pad = None if use_time_mask else _pad(mask, bsz, t)
+        tm = _time(mask, t, t) if use_time_mask else None
         ctx_t, lse, state = fa.fwd_batched(slots[:, :, :, 0], slots[:, :, :, 1], slots[:, :, :, 2], pad, p, d ** -0.5, False,
-                                           dropout_mask=dropout_mask)
+                                           dropout_mask=dropout_mask, time_mask=tm)
         outputs = _linear(ctx_t.view(t, bsz, e), w_out, b_out)
         ctx.heads, ctx.p, ctx.state = heads, p, state
         ctx.has_bias = (b_in is not None, b_out is not None)
-        ctx.save_for_backward(inputs, w_in, w_out, lin, ctx_t, lse, pad)
+        ctx.save_for_backward(inputs, w_in, w_out, lin, ctx_t, lse, pad, tm)
         return outputs
 
     @staticmethod
     def backward(ctx, output_grads):
-        inputs, w_in, w_out, lin, ctx_t, lse, pad = ctx.saved_tensors
+        inputs, w_in, w_out, lin, ctx_t, lse, pad, tm = ctx.saved_tensors
         t, bsz, e = inputs.shape
         heads = ctx.heads
         d = e // heads
@@ -71,9 +81,10 @@ class SelfAttnFlashFunc(torch.autograd.Function):
         dlin = torch.empty_like(lin)
         dslots = dlin.view(t, bsz, heads, 3, d)
         fa.bwd_batched(dctx.view(t, bsz, heads, d), slots[:, :, :, 0], slots[:, :, :, 1], slots[:, :, :, 2], ctx_t, lse,
-                       dslots[:, :, :, 0], dslots[:, :, :, 1], dslots[:, :, :, 2], pad, ctx.p, d ** -0.5, False, ctx.state)
+                       dslots[:, :, :, 0], dslots[:, :, :, 1], dslots[:, :, :, 2], pad, ctx.p, d ** -0.5, False, ctx.state,
+                       time_mask=tm)
         dx, dw_in, db_in = _linear_bwd(dlin, inputs, w_in, want_w, want_w and ctx.has_bias[0])
-        return (None, dx, dw_in, dw_out, db_in, db_out, None, None, None)
+        return (None, None, dx, dw_in, dw_out, db_in, db_out, None, None, None)
 
 
 class EncdecAttnFlashFunc(torch.autograd.Function):

@@ -7,7 +7,7 @@ optional, T <= 4096). Rotary position encodings take the composed path of nmtgmi
 GEMM, rotation kernel, compact core); rotary together with incremental decoding raises. Incremental decoding (inference, `incremental=True` with a cache dict) runs in
 nmtgminor_amd/modules/incremental.py. As in the reference's fused branch the result is always
 the pair (outputs, dropout_results). An 18th optional argument replays an explicit dropout
-keep-mask. A training call with return_coverage false and a key padding mask (or none) runs the tiled attention core
+keep-mask. A training call with return_coverage false (key padding mask, time mask or none) runs the tiled attention core
 of nmtgminor_amd/modules/flash_core.py instead and returns an empty tensor as dropout_results."""
 import torch
 
@@ -94,8 +94,8 @@ def self_attn_func(*args):
         if len(args) >= 17:                           # training call whose coverage nobody reads: no [B*H, T, T] tensor
             from . import flash_core
             (use_time_mask, is_training, heads, inputs, w_in, w_out, b_in, b_out, mask, p) = args[:10]
-            if flash_core.eligible(is_training, args[15], use_time_mask, args[16], inputs, heads):
-                outputs = flash_core.SelfAttnFlashFunc.apply(heads, inputs, w_in, w_out, b_in, b_out, mask, p,
+            if flash_core.eligible(is_training, args[15], args[16], inputs, heads):
+                outputs = flash_core.SelfAttnFlashFunc.apply(bool(use_time_mask), heads, inputs, w_in, w_out, b_in, b_out, mask, p,
                                                              args[17] if len(args) > 17 else None)
                 return outputs, outputs.new_empty(0)
         return SelfAttnFunc.apply(*args)

@@ -149,7 +149,7 @@ class DecoderLayer(_Layer):
             input = self._macaron_step(input)
             query = self.preprocess_attn(input)
             out, _ = self.multihead_tgt(query, None, None, mask_tgt, incremental=incremental,
-                                        incremental_cache=incremental_cache)
+                                        incremental_cache=incremental_cache, return_coverage=False)   # dropped here
             input = self.postprocess_attn(self._survivor_scale(out), input)
             if not self.ignore_source:
                 query = self.preprocess_src_attn(input)

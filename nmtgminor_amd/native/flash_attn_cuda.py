@@ -161,8 +161,21 @@ def _pad_mask(mask, batch, len_k):
     return mask
 
 
-def fwd_batched(q, k, v, key_padding_mask, dropout_p, softmax_scale, causal, *, dropout_mask=None, rng=None, want_mask=False):
-    """q [len_q, B, H, D], k / v [len_k, B, H, D] (views with a contiguous D), key_padding_mask uint8 [B, len_k] or None
+def _time_mask(mask, len_q, len_k, device):
+    """-> (mask, workspace) of a time mask uint8 [len_q, len_k] shared by every sequence and head, or (None, None)"""
+    if mask is None:
+        return None, None
+    _check(mask.dtype == torch.uint8 and tuple(mask.shape) == (len_q, len_k) and mask.is_contiguous(),
+           "flash_attn: time_mask must be contiguous uint8 [len_q, len_k]")
+    L.require_cuda(mask)
+    n = L.load().nmtg_flash_attn_time_info_bytes(L.i64(len_q), L.i64(len_k))
+    return mask, torch.empty(max(int(n), 4) // 4, dtype=torch.int32, device=device)
+
+
+def fwd_batched(q, k, v, key_padding_mask, dropout_p, softmax_scale, causal, *, dropout_mask=None, rng=None, want_mask=False,
+                time_mask=None):
+    """q [len_q, B, H, D], k / v [len_k, B, H, D] (views with a contiguous D), key_padding_mask uint8 [B, len_k] or None,
+    time_mask uint8 [len_q, len_k] or None (one of the two at most)
     -> (out [len_q, B, H, D] contiguous, softmax_lse [B, H, len_q], state); `state` goes to bwd_batched as it is (dropout
     mode, Philox pair, explicit mask, keep bits, drawn mask when want_mask)."""
     L.require_cuda(q, k, v)
@@ -174,6 +187,7 @@ def fwd_batched(q, k, v, key_padding_mask, dropout_p, softmax_scale, causal, *, 
     _check(tuple(k.shape[1:]) == (batch, heads, d), "flash_attn: k and v must have q's batch, heads and head_dim")
     pad = _pad_mask(key_padding_mask, batch, len_k)
     kinfo = _key_info(batch, len_k, q.device) if pad is not None else None
+    tmask, tinfo = _time_mask(time_mask, len_q, len_k, q.device)
     out = torch.empty(len_q, batch, heads, d, dtype=q.dtype, device=q.device)
     lse = torch.empty(batch, heads, len_q, dtype=torch.float32, device=q.device)
     mode, seed, offset, mask_out, bits = 0, 0, 0, None, None
@@ -190,7 +204,8 @@ def fwd_batched(q, k, v, key_padding_mask, dropout_p, softmax_scale, causal, *, 
             seed, offset = rng if rng is not None else philox_seed_offset(q.device, 4 * blocks)
             if want_mask:
                 mask_out = torch.zeros(batch, heads, len_q, len_k, dtype=torch.uint8, device=q.device)
-    L.call("nmtg_flash_attn_batched_fwd", L.ptr(q), L.ptr(k), L.ptr(v), L.ptr(out), L.ptr(pad), L.ptr(kinfo), L.ptr(lse),
+    L.call("nmtg_flash_attn_batched_fwd", L.ptr(q), L.ptr(k), L.ptr(v), L.ptr(out), L.ptr(pad), L.ptr(kinfo), L.ptr(tmask),
+           L.ptr(tinfo), L.ptr(lse),
            L.i64(batch), L.i64(heads), L.i64(d), L.i64(len_q), L.i64(len_k), *_view4(q, "q", heads, d), *_view4(k, "k", heads, d),
            *_view4(v, "v", heads, d), *_view4(out, "out", heads, d), L.f32(softmax_scale), L.i32(int(bool(causal))), L.i32(mode),
            L.f32(dropout_p), L.ptr(dropout_mask if mode == 1 else None), L.ptr(mask_out), L.ptr(bits), ctypes.c_uint64(seed),
@@ -198,7 +213,8 @@ def fwd_batched(q, k, v, key_padding_mask, dropout_p, softmax_scale, causal, *, 
     return out, lse, (mode, seed, offset, dropout_mask if mode == 1 else None, bits, mask_out)
 
 
-def bwd_batched(dout, q, k, v, out, softmax_lse, dq, dk, dv, key_padding_mask, dropout_p, softmax_scale, causal, state):
+def bwd_batched(dout, q, k, v, out, softmax_lse, dq, dk, dv, key_padding_mask, dropout_p, softmax_scale, causal, state, *,
+                time_mask=None):
     """Writes dq, dk, dv (views with the strides of q, k, v: the slots of one projection-gradient buffer) -> softmax_d."""
     L.require_cuda(dout, q, k, v, out, softmax_lse, dq, dk, dv)
     len_q, batch, heads, d = q.shape
@@ -212,6 +228,7 @@ def bwd_batched(dout, q, k, v, out, softmax_lse, dq, dk, dv, key_padding_mask, d
            "flash_attn: softmax_lse must be contiguous fp32 [B, H, len_q]")
     pad = _pad_mask(key_padding_mask, batch, len_k)
     kinfo = _key_info(batch, len_k, q.device) if pad is not None else None
+    tmask, tinfo = _time_mask(time_mask, len_q, len_k, q.device)
     mode, seed, offset, mask, bits = state[:5]
     if dropout_p <= 0.0:
         mode, bits = 0, None
@@ -220,7 +237,8 @@ def bwd_batched(dout, q, k, v, out, softmax_lse, dq, dk, dv, key_padding_mask, d
         bits = _bits(batch, heads, len_q, len_k, q.device)
     softmax_d = torch.empty(batch, heads, len_q, dtype=torch.float32, device=q.device)
     L.call("nmtg_flash_attn_batched_bwd", L.ptr(dout), L.ptr(q), L.ptr(k), L.ptr(v), L.ptr(out), L.ptr(softmax_lse), L.ptr(dq),
-           L.ptr(dk), L.ptr(dv), L.ptr(softmax_d), L.ptr(pad), L.ptr(kinfo), L.i64(batch), L.i64(heads), L.i64(d), L.i64(len_q),
+           L.ptr(dk), L.ptr(dv), L.ptr(softmax_d), L.ptr(pad), L.ptr(kinfo), L.ptr(tmask), L.ptr(tinfo), L.i64(batch), L.i64(heads),
+           L.i64(d), L.i64(len_q),
            L.i64(len_k), *_view4(q, "q", heads, d), *_view4(k, "k", heads, d), *_view4(v, "v", heads, d),
            *_view4(out, "out", heads, d), L.f32(softmax_scale), L.i32(int(bool(causal))), L.i32(mode), L.f32(dropout_p),
            L.ptr(mask if mode == 1 else None), L.ptr(bits), L.i32(ready), ctypes.c_uint64(seed), ctypes.c_uint64(offset),

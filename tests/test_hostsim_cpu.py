@@ -412,6 +412,17 @@ def test_encoder_layer_on_the_tiled_attention_core(mi355x, monkeypatch):
     tla.test_encoder_layer_with_head_dimension_64_drops_the_coverage_and_runs_the_tiled_core(CPU, BF16, monkeypatch)
 
 
+def test_decoder_layer_on_the_tiled_attention_core(mi355x, monkeypatch):
+    tla.test_decoder_layer_with_head_dimension_64_runs_its_self_attention_on_the_tiled_core(CPU, F16, monkeypatch)
+
+
+@pytest.mark.parametrize("dtype", HALVES)
+def test_training_attention_with_time_masks_without_coverage(mi355x, dtype):
+    tnc.test_self_attention_training_with_a_causal_time_mask(CPU, dtype, 200, 2, 256, 4, 0.25)
+    tnc.test_self_attention_training_with_time_masks_of_other_shapes(CPU, dtype)
+    tnc.test_a_causal_time_mask_equals_the_causal_flag_bit_for_bit(CPU, 64, 0.2)
+
+
 @pytest.mark.parametrize("dtype", HALVES)
 @pytest.mark.parametrize("ignore_source", [False, pytest.param(True, marks=long_case)])
 def test_decoder_layer(mi355x, dtype, ignore_source):

@@ -155,7 +155,23 @@ def test_encoder_layer_stochastic_depth(dev):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("ignore_source", [False, True])
 def test_decoder_layer_matches_the_oracle(dev, dtype, ignore_source):
-    opt = options(ignore_source=ignore_source)
+    _decoder_case(dev, dtype, ignore_source)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_decoder_layer_with_head_dimension_64_runs_its_self_attention_on_the_tiled_core(dev, dtype, monkeypatch):
+    """The layer drops the coverage of its self-attention (the cross-attention's is returned), so in training the time-masked
+    self-attention writes no [B*H, T, T] tensor where the tiled core takes the shape. Same oracle, same tolerance."""
+    from nmtgminor_amd.native import flash_attn_cuda
+    calls = []
+    real = flash_attn_cuda.fwd_batched
+    monkeypatch.setattr(flash_attn_cuda, "fwd_batched", lambda *a, **k: (calls.append(k.get("time_mask") is not None), real(*a, **k))[1])
+    _decoder_case(dev, dtype, False, model_size=256, inner_size=512)
+    assert calls == [True]
+
+
+def _decoder_case(dev, dtype, ignore_source, **more):
+    opt = options(ignore_source=ignore_source, **more)
     tq, tk, b = 24, 50, 2
     g = torch.Generator().manual_seed(86)
     layer = randomise(DecoderLayer(opt), 87)
