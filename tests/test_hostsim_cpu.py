@@ -412,13 +412,15 @@ def test_encoder_layer_on_the_tiled_attention_core(mi355x, monkeypatch):
     tla.test_encoder_layer_with_head_dimension_64_drops_the_coverage_and_runs_the_tiled_core(CPU, BF16, monkeypatch)
 
 
+@long_case
 def test_decoder_layer_on_the_tiled_attention_core(mi355x, monkeypatch):
     tla.test_decoder_layer_with_head_dimension_64_runs_its_self_attention_on_the_tiled_core(CPU, F16, monkeypatch)
 
 
 @pytest.mark.parametrize("dtype", HALVES)
 def test_training_attention_with_time_masks_without_coverage(mi355x, dtype):
-    tnc.test_self_attention_training_with_a_causal_time_mask(CPU, dtype, 200, 2, 256, 4, 0.25)
+    if not SANITIZER_RUN:
+        tnc.test_self_attention_training_with_a_causal_time_mask(CPU, dtype, 200, 2, 256, 4, 0.25)
     tnc.test_self_attention_training_with_time_masks_of_other_shapes(CPU, dtype)
     tnc.test_a_causal_time_mask_equals_the_causal_flag_bit_for_bit(CPU, 64, 0.2)
 
@@ -666,17 +668,19 @@ def test_packed_attention_dropout_philox_and_autograd_functions():
 
 # ----------------------------------------------------------------------------- the same kernels over a padded batch
 def test_training_attention_without_coverage(mi355x, monkeypatch):
-    tnc.test_self_attention_training_without_coverage(CPU, BF16, 128, 3, 512, 8, 0.1)
-    tnc.test_self_attention_training_without_coverage(CPU, F16, 33, 2, 128, 2, 0.1)
     tnc.test_self_attention_with_masked_keys_anywhere(CPU, BF16)
     tnc.test_encdec_attention_training_without_coverage(CPU, F16, 17, 100, 3, 128, 2, 0.2)
-    tnc.test_encdec_attention_training_without_coverage(CPU, BF16, 40, 130, 2, 256, 2, 0.1)
     tnc.test_a_sequence_with_every_key_masked(CPU)
-    tnc.test_bias_free_encdec_function_without_coverage(CPU, F16)
+    if not SANITIZER_RUN:
+        tnc.test_self_attention_training_without_coverage(CPU, BF16, 128, 3, 512, 8, 0.1)
+        tnc.test_self_attention_training_without_coverage(CPU, F16, 33, 2, 128, 2, 0.1)
+        tnc.test_encdec_attention_training_without_coverage(CPU, BF16, 40, 130, 2, 256, 2, 0.1)
+        tnc.test_bias_free_encdec_function_without_coverage(CPU, F16)
     tnc.test_the_switch_keeps_the_extension_path(CPU, monkeypatch)   # sets a switch: last
 
 
-@pytest.mark.parametrize("d,causal,p", [(64, True, 0.2), pytest.param(128, False, 0.2, marks=long_case), (64, False, 0.0)])
+@pytest.mark.parametrize("d,causal,p", [(64, True, 0.2), pytest.param(128, False, 0.2, marks=long_case),
+                                        pytest.param(64, False, 0.0, marks=long_case)])
 def test_batch_strided_attention_equals_packed_attention_bit_for_bit(d, causal, p):
     tnc.test_batch_strided_call_equals_packed_call_bit_for_bit(CPU, d, causal, p)
 
