@@ -671,6 +671,7 @@ def test_training_attention_without_coverage(mi355x, monkeypatch):
     tnc.test_self_attention_with_masked_keys_anywhere(CPU, BF16)
     tnc.test_encdec_attention_training_without_coverage(CPU, F16, 17, 100, 3, 128, 2, 0.2)
     tnc.test_a_sequence_with_every_key_masked(CPU)
+    tnc.test_dropout_drawn_on_the_device_is_replayed_by_its_own_mask(CPU)
     if not SANITIZER_RUN:
         tnc.test_self_attention_training_without_coverage(CPU, BF16, 128, 3, 512, 8, 0.1)
         tnc.test_self_attention_training_without_coverage(CPU, F16, 33, 2, 128, 2, 0.1)

@@ -210,6 +210,43 @@ def test_a_sequence_with_every_key_masked(dev):
     assert (dqkv[:, 1] == 0).all() and (dqkv[60:, 2, :, 1:] == 0).all()
 
 
+def test_dropout_drawn_on_the_device_is_replayed_by_its_own_mask(dev):
+    """A call without an explicit dropout mask draws one from the device generator (what training does). The keep flags it
+    hands back, replayed as an explicit mask, must give the same output and gradients bit for bit; their density is
+    1 - p on the live keys; and the module-level call draws a fresh mask per call."""
+    t, b, h, d, p, dtype = 100, 2, 2, 64, 0.25, torch.float16
+    g = torch.Generator().manual_seed(41)
+    qkv = torch.randn(t, b, h, 3, d, generator=g).to(dtype).to(dev)
+    do = torch.randn(t, b, h, d, generator=g).to(dtype).to(dev)
+    pad = torch.zeros(b, t, dtype=torch.uint8)
+    pad[1, 70:] = 1
+    pad = pad.to(dev)
+    q, k, v = qkv[:, :, :, 0], qkv[:, :, :, 1], qkv[:, :, :, 2]
+    torch.manual_seed(7)
+    res = []
+    out, lse, state = fa.fwd_batched(q, k, v, pad, p, d ** -0.5, False, want_mask=True)
+    drawn = state[5]
+    for st, kw in ((state, {}), (None, dict(dropout_mask=drawn))):
+        if st is None:
+            out2, lse2, st = fa.fwd_batched(q, k, v, pad, p, d ** -0.5, False, **kw)
+            assert torch.equal(lse2, lse)
+            # the drawn mask's scale is 256 / round(256 (1 - p)), the replayed one's 1 / (1 - p): the same number for p = 0.25
+            assert torch.equal(out2, out)
+        dqkv = torch.full_like(qkv, float("nan"))
+        fa.bwd_batched(do, q, k, v, out, lse, dqkv[:, :, :, 0], dqkv[:, :, :, 1], dqkv[:, :, :, 2], pad, p, d ** -0.5, False, st)
+        res.append(dqkv)
+    assert torch.equal(res[0], res[1])
+    live = drawn[0].float()                                   # sequence 0 has no masked key
+    assert abs(live.mean().item() - (1 - p)) < 0.02
+    x = torch.randn(t, b, h * d, generator=g).to(dtype).to(dev)
+    w_in = (torch.randn(3 * h * d, h * d, generator=g) * 0.05).to(dtype).to(dev)
+    w_out = (torch.randn(h * d, h * d, generator=g) * 0.05).to(dtype).to(dev)
+    call = lambda: self_attn_func(False, True, h, x, w_in, w_out, None, None, pad.bool(), p, False, None, False, None, True, False,
+                                  False)[0]
+    a1, a2 = call(), call()
+    assert torch.isfinite(a1).all() and not torch.equal(a1, a2)
+
+
 @pytest.mark.parametrize("d", [64, 128])
 @pytest.mark.parametrize("causal,p", [(False, 0.0), (True, 0.0), (False, 0.2), (True, 0.2)])
 def test_batch_strided_call_equals_packed_call_bit_for_bit(dev, d, causal, p):
