@@ -26,7 +26,8 @@ class EncdecAttnBiasFunc(torch.autograd.Function):
         ctx.has_bias = (input_bias_q is not None, input_bias_kv is not None, output_bias is not None)
         q_lin, kv_lin, scores, dropped, dmask, ctx_t, outputs = native.forward(
             is_training, heads, inputs_q, inputs_kv, input_weights_q, input_weights_kv, output_weights, input_bias_q,
-            input_bias_kv, output_bias, mask, dropout_prob, dropout_mask=dropout_mask, want_probs=bool(return_coverage))
+            input_bias_kv, output_bias, mask, dropout_prob, dropout_mask=dropout_mask, want_probs=bool(return_coverage),
+            need_backward=any(ctx.needs_input_grad))
         if recompute:
             ctx.save_for_backward(inputs_q, inputs_kv, input_weights_q, input_weights_kv, output_weights, input_bias_q,
                                   input_bias_kv, mask, dmask)
@@ -101,7 +102,8 @@ class EncdecAttnBiasCompactFunc(torch.autograd.Function):
             raise NotImplementedError("encdec_attn_bias_compact_func: rotary / incremental modes have no HIP kernel")
         q_lin, kv_lin = q_lin.contiguous(), kv_lin.contiguous()
         scores, dropped, dmask, ctx_t = native.forward_compact(is_training, heads, q_lin, kv_lin, mask, dropout_prob,
-                                                               dropout_mask=dropout_mask)
+                                                               dropout_mask=dropout_mask,
+                                                               need_backward=any(ctx.needs_input_grad))
         ctx.heads, ctx.p, ctx.return_coverage = heads, dropout_prob, return_coverage
         ctx.save_for_backward(q_lin, kv_lin, scores, dropped, dmask)
         ctx.mark_non_differentiable(dropped)

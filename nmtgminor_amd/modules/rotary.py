@@ -79,7 +79,8 @@ class EncdecAttnRotaryFunc(torch.autograd.Function):
         rot.rotate_q_(q_lin, cos_q, sin_q, bsz * heads, d)
         rot.rotate_k_(kv_lin, cos_k, sin_k, bsz * heads, d)
         scores, dropped, dmask, ctx_t = ed_native.forward_compact(is_training, heads, q_lin, kv_lin, mask, p,
-                                                                  dropout_mask=dropout_mask)
+                                                                  dropout_mask=dropout_mask,
+                                                                  need_backward=any(ctx.needs_input_grad))
         outputs = _linear(ctx_t, w_out, b_out)
         ctx.heads, ctx.p = heads, p
         ctx.has_bias = (b_q is not None, b_kv is not None, b_out is not None)

@@ -38,7 +38,8 @@ class SelfAttnFunc(torch.autograd.Function):
         ctx.has_out_bias = output_biases is not None
         lin, scores, dropped, dmask, ctx_t, outputs = native.forward(
             use_time_mask, is_training, heads, inputs, input_weights, output_weights, input_biases, output_biases, mask,
-            dropout_prob, dropout_mask=dropout_mask, want_probs=bool(return_coverage))
+            dropout_prob, dropout_mask=dropout_mask, want_probs=bool(return_coverage),
+            need_backward=any(ctx.needs_input_grad))
         if recompute:
             ctx.save_for_backward(inputs, input_weights, output_weights, input_biases, output_biases, mask, dmask)
         else:

@@ -54,12 +54,17 @@ def dropout_args(is_training, p, shape, device, dropout_mask):
     return torch.empty(0, dtype=torch.uint8, device=device), 0, 0, 0
 
 
-def scores_needed(is_training, dtype, head_dim, tk):
+def scores_needed(is_training, dtype, head_dim, tk, need_backward=None):
     """Whether a forward call has to keep the pre-softmax scores. They exist for the backward; a call that is neither in
-    training mode nor recorded by autograd (inference under torch.no_grad()) leaves them out where the one-kernel
+    training mode nor followed by a backward (inference under torch.no_grad()) leaves them out where the one-kernel
     inference path takes the shape (16-bit tensors, head dimension 64 or 128, a key count that is a multiple of 4), and
-    the stand-in then returns an empty tensor in their place. NMTG_ATTN_PROBS=0 keeps them always."""
-    if is_training or torch.is_grad_enabled() or os.environ.get("NMTG_ATTN_PROBS", "1") == "0":
+    the stand-in then returns an empty tensor in their place. NMTG_ATTN_PROBS=0 keeps them always.
+    `need_backward`: what the caller knows about a backward to come. An autograd function passes
+    any(ctx.needs_input_grad) (inside its forward the grad mode is always off, whatever the caller's was); None asks
+    the grad mode, which is right for a direct call of the stand-in module."""
+    if need_backward is None:
+        need_backward = torch.is_grad_enabled()
+    if is_training or need_backward or os.environ.get("NMTG_ATTN_PROBS", "1") == "0":
         return True
     return not (dtype in (torch.float16, torch.bfloat16) and head_dim in (64, 128) and tk >= 1 and tk % 4 == 0)
 

@@ -25,14 +25,14 @@ def _shapes(q3, kv3, heads, kv_last):
 
 
 def _fwd(is_training, heads, x_q, x_kv, w_q, w_kv, w_out, b_q, b_kv, b_out, q_lin, kv_lin, pad_mask, p, dropout_mask,
-         tq, tk, b, e, dev, dt, softmax_out=None, want_probs=True):
+         tq, tk, b, e, dev, dt, softmax_out=None, want_probs=True, need_backward=None):
     km, kind = A.mask_arg(pad_mask, False, b, tq, tk)
     bh = b * heads
     if q_lin is None:
         q_lin = torch.empty(tq, b, e, dtype=dt, device=dev)
     if kv_lin is None:
         kv_lin = torch.empty(tk, b, 2 * e, dtype=dt, device=dev)
-    keep_scores = softmax_out is not None or A.scores_needed(is_training, dt, e // heads, tk)
+    keep_scores = softmax_out is not None or A.scores_needed(is_training, dt, e // heads, tk, need_backward)
     scores = torch.empty((bh, tq, tk) if keep_scores else (0,), dtype=dt, device=dev)
     keep_probs = want_probs or keep_scores
     dropped = torch.empty((bh, tq, tk) if keep_probs else (0,), dtype=dt, device=dev)
@@ -75,7 +75,8 @@ def _fwd_padded_keys(heads, x_q, x_kv, w_q, w_kv, w_out, b_q, b_kv, b_out, pad_m
 
 
 def forward(is_training, heads, inputs_q, inputs_kv, input_weights_q, input_weights_kv, output_weights, input_biases_q,
-            input_biases_kv, output_biases, pad_mask, dropout_prob, *, dropout_mask=None, want_probs=True):
+            input_biases_kv, output_biases, pad_mask, dropout_prob, *, dropout_mask=None, want_probs=True,
+            need_backward=None):
     """-> [input_lin_q_results, input_lin_kv_results, attn_scores, dropout_results, dropout_mask,
     matmul2_results, outputs]; attn_scores is empty for an inference call under torch.no_grad() (see
     _attn_common.scores_needed), and so is dropout_results when such a call says want_probs=False."""
@@ -90,23 +91,24 @@ def forward(is_training, heads, inputs_q, inputs_kv, input_weights_q, input_weig
     # inference with a key length that is not a multiple of 64: keys / values padded with masked zero rows, so that every
     # tensor of the middle section is 16-byte aligned (NMTG_ATTN_PAD_KEYS=0 keeps the exact-length buffers)
     if (not is_training and tk % KEY_BLOCK != 0 and os.environ.get("NMTG_ATTN_PAD_KEYS") != "0"
-            and A.scores_needed(False, inputs_q.dtype, e // heads, tk)):
+            and A.scores_needed(False, inputs_q.dtype, e // heads, tk, need_backward)):
         return _fwd_padded_keys(heads, c(inputs_q), c(inputs_kv), c(input_weights_q), c(input_weights_kv), c(output_weights),
                                 c(input_biases_q), c(input_biases_kv), c(output_biases), pad_mask, tq, tk, b, e)
     return list(_fwd(is_training, heads, c(inputs_q), c(inputs_kv), c(input_weights_q), c(input_weights_kv),
                      c(output_weights), c(input_biases_q), c(input_biases_kv), c(output_biases), None, None, pad_mask,
-                     dropout_prob, dropout_mask, tq, tk, b, e, inputs_q.device, inputs_q.dtype, want_probs=want_probs))
+                     dropout_prob, dropout_mask, tq, tk, b, e, inputs_q.device, inputs_q.dtype, want_probs=want_probs,
+                     need_backward=need_backward))
 
 
 def forward_compact(is_training, heads, input_lin_q_results, input_lin_kv_results, pad_mask, dropout_prob, *,
-                    dropout_mask=None):
+                    dropout_mask=None, need_backward=None):
     """-> [attn_scores, dropout_results, dropout_mask, matmul2_results]"""
     L.require_cuda(input_lin_q_results, input_lin_kv_results, pad_mask, dropout_mask)
     A.check_half(input_lin_q_results, input_lin_kv_results)
     tq, tk, b, e = _shapes(input_lin_q_results, input_lin_kv_results, heads, 2)
     r = _fwd(is_training, heads, None, None, None, None, None, None, None, None, input_lin_q_results.contiguous(),
              input_lin_kv_results.contiguous(), pad_mask, dropout_prob, dropout_mask, tq, tk, b, e,
-             input_lin_q_results.device, input_lin_q_results.dtype)
+             input_lin_q_results.device, input_lin_q_results.dtype, need_backward=need_backward)
     return [r[2], r[3], r[4], r[5]]
 
 
@@ -200,6 +202,7 @@ def backward_recompute(heads, output_grads, inputs_q, inputs_kv, input_weights_q
     q_lin, kv_lin, scores, dropped, dmask, ctx, _ = forward(training, heads, inputs_q, inputs_kv, input_weights_q,
                                                             input_weights_kv, output_weights, input_biases_q,
                                                             input_biases_kv, None, pad_mask, dropout_prob,
-                                                            dropout_mask=dropout_mask if training else None)
+                                                            dropout_mask=dropout_mask if training else None,
+                                                            need_backward=True)
     return backward(heads, output_grads, ctx, dropped, scores, q_lin, kv_lin, inputs_q, inputs_kv, input_weights_q,
                     input_weights_kv, output_weights, dmask, dropout_prob)

@@ -19,7 +19,7 @@ def _dims(inputs, heads, last):
 
 
 def forward(use_time_mask, is_training, heads, inputs, input_weights, output_weights, input_biases, output_biases,
-            pad_mask, dropout_prob, *, dropout_mask=None, want_probs=True):
+            pad_mask, dropout_prob, *, dropout_mask=None, want_probs=True, need_backward=None):
     """-> [input_lin_results, attn_scores, dropout_results, dropout_mask, matmul2_results, outputs]; attn_scores is empty
     for an inference call under torch.no_grad() (see _attn_common.scores_needed); such a call with want_probs=False
     (the caller does not return the coverage) leaves dropout_results empty too: no [B*H, T, T] tensor exists then."""
@@ -36,7 +36,7 @@ def forward(use_time_mask, is_training, heads, inputs, input_weights, output_wei
     km, kind = A.mask_arg(pad_mask, use_time_mask, b, t, t)
     bh = b * heads
     lin = torch.empty(t, b, 3 * e, dtype=dt, device=dev)
-    keep_scores = A.scores_needed(is_training, dt, e // heads, t)
+    keep_scores = A.scores_needed(is_training, dt, e // heads, t, need_backward)
     scores = torch.empty((bh, t, t) if keep_scores else (0,), dtype=dt, device=dev)
     keep_probs = want_probs or keep_scores
     dropped = torch.empty((bh, t, t) if keep_probs else (0,), dtype=dt, device=dev)
@@ -145,6 +145,6 @@ def backward_recompute(use_time_mask, heads, output_grads, inputs, input_weights
     training = dropout_mask is not None and dropout_mask.numel() > 0 and dropout_prob > 0.0
     lin, scores, dropped, dmask, ctx, _ = forward(use_time_mask, training, heads, inputs, input_weights, output_weights,
                                                   input_biases, output_biases, pad_mask, dropout_prob,
-                                                  dropout_mask=dropout_mask if training else None)
+                                                  dropout_mask=dropout_mask if training else None, need_backward=True)
     return backward(use_time_mask, heads, output_grads, ctx, dropped, scores, lin, inputs, input_weights, output_weights,
                     dmask, dropout_prob)

@@ -110,6 +110,73 @@ def test_self_attention_rng_dropout_eval_and_no_bias(dev):
         sa_native.forward(False, False, h, g("x").float(), g("w_in").float(), g("w_out").float(), None, None, None, 0.0)
 
 
+@pytest.mark.parametrize("mode", ["eval", "eval_no_coverage", "recompute_p0"])
+def test_self_attention_backward_without_dropout_state(dev, mode):
+    # A backward through a call that is not in training mode (grad mode on, is_training False), and through a
+    # recomputing call with p = 0: inside an autograd function the grad mode is off, so the decision to keep the
+    # scores for the backward must come from the inputs' requires_grad (head dimension 64 and a key count that is a
+    # multiple of 4: the shape the score-free inference kernel would otherwise take).
+    dtype = torch.bfloat16
+    t, b, e, h = 64, 2, 256, 4
+    d = inputs.self_attn_inputs(t, b, e, h, dtype, p=0.0, seed=75, zero_bias=False)
+    fwd = oat.self_attn_fwd(d["x"], d["w_in"], d["w_out"], d["b_in"], d["b_out"], h, d["pad_mask"], None, 0.0, None, D,
+                            round_to=dtype)
+    bwd = oat.self_attn_bwd(d["dout"], d["x"], d["w_in"], d["w_out"], h, fwd, 0.0, None, D, round_to=dtype)
+    leaves = [d[k].to(dev).requires_grad_() for k in ("x", "w_in", "w_out", "b_in", "b_out")]
+    training, p, cover, recompute = {"eval": (False, 0.3, True, False), "eval_no_coverage": (False, 0.3, False, False),
+                                     "recompute_p0": (True, 0.0, True, True)}[mode]
+    out, cov = self_attn_func(False, training, h, *leaves, d["pad_mask"].to(dev), p, False, None, False, None, True, cover,
+                              recompute)
+    out.backward(d["dout"].to(dev))
+    assert_close(out, fwd["outputs"], dtype, "outputs")
+    if cover:
+        assert_close(cov, fwd["dropout_results"], dtype, "coverage")
+    for leaf, key in zip(leaves, ("dx", "dw_in", "dw_out", "db_in", "db_out")):
+        assert_close(leaf.grad, bwd[key], dtype, key, scale_atol=True)
+    # the same call under no_grad still leaves the score tensor out
+    with torch.no_grad():
+        r = sa_native.forward(False, False, h, *[z.detach() for z in leaves], d["pad_mask"].to(dev), 0.0)
+    assert r[1].numel() == 0
+
+
+@pytest.mark.parametrize("mode", ["eval", "eval_compact", "recompute_p0"])
+def test_encdec_attention_backward_without_dropout_state(dev, mode):
+    dtype = torch.bfloat16
+    tq, tk, b, e, h = 32, 128, 2, 256, 4
+    d = inputs.encdec_attn_inputs(tq, tk, b, e, h, dtype, p=0.0, seed=76, zero_bias=False)
+    fwd = oat.encdec_attn_fwd(d["x_q"], d["x_kv"], d["w_q"], d["w_kv"], d["w_out"], d["b_q"], d["b_kv"], d["b_out"], h,
+                              d["pad_mask"], 0.0, None, D, round_to=dtype)
+    bwd = oat.encdec_attn_bwd(d["dout"], d["x_q"], d["x_kv"], d["w_q"], d["w_kv"], d["w_out"], h, fwd, 0.0, None, D,
+                              round_to=dtype)
+    names = ("x_q", "x_kv", "w_q", "w_kv", "w_out", "b_q", "b_kv", "b_out")
+    leaf = {k: d[k].to(dev).requires_grad_() for k in names}
+    pad = d["pad_mask"].to(dev)
+    if mode == "eval_compact":
+        q_lin = fwd["input_lin_q_results"].to(dtype).to(dev).requires_grad_()
+        kv_lin = fwd["input_lin_kv_results"].to(dtype).to(dev).requires_grad_()
+        (ctx_t,) = encdec_attn_bias_compact_func(False, False, h, q_lin, kv_lin, pad, 0.3, False, None, False, None, None, True,
+                                                 False)
+        dctx = torch.randn(tq, b, e, generator=torch.Generator().manual_seed(2)).to(dtype)
+        ctx_t.backward(dctx.to(dev))
+        assert_close(ctx_t, fwd["matmul2_results"], dtype, "context")
+        k, v = [fwd["input_lin_kv_results"].to(D).view(tk, b * h, 2, e // h)[:, :, i] for i in range(2)]
+        q = fwd["input_lin_q_results"].to(D).view(tq, b * h, e // h)
+        dq, dk, dv = oat._core_bwd(dctx.to(D).view(tq, b * h, e // h), q, k, v, fwd["softmax_results"], fwd["dropout_results"],
+                                   0.0, None, D, round_to=dtype)
+        assert_close(q_lin.grad, dq.reshape(tq, b, e), dtype, "dq", scale_atol=True)
+        assert_close(kv_lin.grad, torch.stack([dk, dv], 2).reshape(tk, b, 2 * e), dtype, "dkv", scale_atol=True)
+        return
+    recompute, training, p = (True, True, 0.0) if mode == "recompute_p0" else (False, False, 0.3)
+    out, cov = encdec_attn_bias_func(recompute, training, h, leaf["x_q"], leaf["x_kv"], leaf["w_q"], leaf["w_kv"], leaf["w_out"],
+                                     leaf["b_q"], leaf["b_kv"], leaf["b_out"], pad, p, False, None, False, None, None, True, True)
+    out.backward(d["dout"].to(dev))
+    assert_close(out, fwd["outputs"], dtype, "outputs")
+    assert_close(cov, fwd["dropout_results"], dtype, "coverage")
+    for key, n in (("dx_q", "x_q"), ("dx_kv", "x_kv"), ("dw_q", "w_q"), ("dw_kv", "w_kv"), ("dw_out", "w_out"),
+                   ("db_q", "b_q"), ("db_kv", "b_kv"), ("db_out", "b_out")):
+        assert_close(leaf[n].grad, bwd[key], dtype, key, scale_atol=True)
+
+
 def _encdec_case(dev, tq, tk, b, e, h, dtype, p, zero_bias=False, biases=True, seed=74):
     d = inputs.encdec_attn_inputs(tq, tk, b, e, h, dtype, p=p, seed=seed, zero_bias=zero_bias)
     if not biases:

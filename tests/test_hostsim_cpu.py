@@ -389,6 +389,16 @@ def test_attention_inference_random_shapes(mi355x, monkeypatch, seed):
     tat.test_inference_kernel_on_randomly_drawn_shapes(CPU, monkeypatch, seed)
 
 
+@pytest.mark.parametrize("mode", ["eval", "eval_no_coverage", "recompute_p0"])
+def test_self_attention_backward_without_dropout_state(mi355x, mode):
+    tat.test_self_attention_backward_without_dropout_state(CPU, mode)
+
+
+@pytest.mark.parametrize("mode", ["eval", "eval_compact", "recompute_p0"])
+def test_encdec_attention_backward_without_dropout_state(mi355x, mode):
+    tat.test_encdec_attention_backward_without_dropout_state(CPU, mode)
+
+
 def test_encdec_attention_without_biases_compact_and_modules(mi355x):
     tat.test_encdec_attention_without_biases_and_compact(CPU)
     tat.test_modules_state_dict_names_and_forward(CPU)
