@@ -83,6 +83,7 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
     a.splits = 1;
     a.defer_reduce = 0;
     a.tile_used = -1;
+    a.riders_taken = 0;
     if (planned_out) *planned_out = a;
     return gemm_skinny_run(dtype, a, st);
   }
@@ -173,6 +174,10 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
     return fail(NMTG_ERR_INVALID, "gemm: the split-K epilogue needs a workspace");
   a.tile_used = tile;
   if (epi != EPI_SPLITK) a.defer_reduce = 0;
+  // riders travel with the kernels that ring_rider<> (gemm_inst.hip.h) names, and only in an unbatched launch
+  const bool can_ride = tile == TILE_M && a.vec == 8 && a.ring && a.batch == 1 && layout == LAYOUT_NN && epi == EPI_PLAIN;
+  a.riders_taken = (a.riders != nullptr && a.rider_blocks > 0 && can_ride) ? 1 : 0;
+  if (!a.riders_taken) { a.riders = nullptr; a.rider_blocks = 0; }
   if (planned_out) *planned_out = a;
   int rc;
   if (layout == LAYOUT_NT) rc = gemm_launch_nt(dtype, tile, epi, a, st);

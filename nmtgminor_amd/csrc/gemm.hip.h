@@ -77,6 +77,12 @@ struct GemmArgs {
   int act_lut;              // gelu / gelu' through the LDS table (ring kernels only; set by the host on request)
   int defer_reduce;         // host only: a split-K call leaves its reduction to the caller (who queues it in a ReduceTail)
   int tile_used;            // host only, filled by gemm_run: the tile the call ran with
+  // host only: a list of small reduction jobs (TailArgs, reduce.hip.h) that `rider_blocks` extra blocks of this launch
+  // run beside the GEMM's own blocks (they have no part in the product; what they read must be complete before the
+  // launch). Kernels that cannot carry them leave riders_taken at 0 and the caller launches the list itself.
+  const void* riders;
+  int rider_blocks;
+  int riders_taken;
   float* colsum_part;
   const uint8_t* kmask;
   int kmask_kind, heads;

@@ -49,12 +49,24 @@ int gemm_launch_vec(const GemmArgs& a, hipStream_t st) {
 // tile takes 5 slots so that two blocks share a CU and one block's epilogue overlaps the other's
 // main loop.
 template <int TILE> struct ring_slots { static constexpr int value = TILE == TILE_M ? 5 : 10; };
+// The 128x128 tile runs one wavefront per SIMD: its main loop keeps a whole stage's fragments in registers (STEPBUF).
+template <int TILE> struct ring_stepbuf { static constexpr bool value = TILE == TILE_M; };
+
+// Which kernels carry riders (GemmArgs::riders): the plain 128x128 data-gradient product, the last kernel of a backward
+// pass, which leaves one block on a CU at the shapes of a feed-forward block.
+template <int TILE, bool A_KC, bool B_KC, int EPI> struct ring_rider {
+  static constexpr bool value = TILE == TILE_M && A_KC && !B_KC && EPI == EPI_PLAIN;
+};
 
 template <typename T, int TILE, bool A_KC, bool B_KC, int EPI>
 int gemm_launch_ring(const GemmArgs& a, hipStream_t st) {
   using C = tile_cfg<TILE>;
   constexpr int RING = ring_slots<TILE>::value;
-  auto kern = gemm_ring_kernel<T, C::BM, C::BN, C::WM, C::WN, A_KC, B_KC, EPI, RING>;
+  constexpr bool RIDER = ring_rider<TILE, A_KC, B_KC, EPI>::value;
+  auto kern = [] {
+    if constexpr (RIDER) return gemm_ring_rider_kernel<T, C::BM, C::BN, C::WM, C::WN, A_KC, B_KC, EPI, RING, ring_stepbuf<TILE>::value>;
+    else return gemm_ring_kernel<T, C::BM, C::BN, C::WM, C::WN, A_KC, B_KC, EPI, RING, ring_stepbuf<TILE>::value>;
+  }();
   constexpr int lds = gemm_ring_lds_bytes<C::BM, C::BN, RING>();
   static bool attr_done = false;
   if (!attr_done) {
@@ -68,7 +80,17 @@ int gemm_launch_ring(const GemmArgs& a, hipStream_t st) {
                                   (EPI == EPI_PLAIN ? "plain" : EPI == EPI_ACT_FWD ? "actfwd" : EPI == EPI_ACT_BWD ? "actbwd"
                                    : EPI == EPI_SCORES ? "scores" : "splitk") + "_ring";
   TraceScope trace(name.c_str(), st);
-  hipLaunchKernelGGL(kern, grid, dim3(64 * C::WM * C::WN), lds, st, a);
+  if constexpr (RIDER) {
+    const bool ride = a.riders != nullptr && a.rider_blocks > 0;
+    TailArgs riders{};
+    if (ride) {
+      riders = *static_cast<const TailArgs*>(a.riders);
+      grid.x += static_cast<unsigned>(a.rider_blocks);
+    }
+    hipLaunchKernelGGL(kern, grid, dim3(64 * C::WM * C::WN), lds, st, a, riders);
+  } else {
+    hipLaunchKernelGGL(kern, grid, dim3(64 * C::WM * C::WN), lds, st, a);
+  }
   return 0;
 }
 

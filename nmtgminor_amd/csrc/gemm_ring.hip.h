@@ -86,8 +86,18 @@ constexpr int gemm_ring_lds_bytes() {
   return main_loop > c_tile ? main_loop : c_tile;
 }
 
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC, int EPI, int RING>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_ring_kernel(const GemmArgs g) {
+// STEPBUF = false: a step reads its operand fragments from LDS k-group by k-group, one k-group ahead of the MFMAs
+// that use them, and ends with the wait for the next stage and the barrier: the matrix pipe drains there, which two
+// wavefronts per SIMD (the 256x256 tile) cover in part and a single one (the 128x128 tile) does not.
+// STEPBUF = true (one wavefront per SIMD): "phase p" reads the fragments of the whole stage p into one of two register
+// sets while it multiplies stage p - 1 out of the other. The phase starts with the MFMAs of the first k-group, then
+// waits for stage p's transfers, passes the barrier (the reads of phase p - 1 have had those MFMAs to land; behind the
+// barrier every wavefront is done with stage p - 1's slots, which are refilled right there) and deals stage p's reads
+// out between the MFMAs of the remaining k-groups. The matrix pipe has work on both sides of the barrier. Phase 0
+// only reads, one more phase without reads follows the last stage; the ring positions and the vmcnt bookkeeping are
+// those of the plain loop.
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC, int EPI, int RING, bool STEPBUF = false>
+__device__ __forceinline__ void gemm_ring_body(const GemmArgs& g, int block_x) {
   constexpr int NT = 64 * WAVES_M * WAVES_N, NW = NT / 64;
   constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
   constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -107,7 +117,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_ring_kernel(const
   const int wm0 = (wave / WAVES_N) * WTM, wn0 = (wave % WAVES_N) * WTN;
 
   // tile order: see gemm_kernel
-  int bid = blockIdx.x;
+  int bid = block_x;
   const int ntile = g.m_tiles * g.n_tiles;
   if ((ntile & 7) == 0) bid = (bid & 7) * (ntile >> 3) + (bid >> 3);
   constexpr int GM = 4;
@@ -154,10 +164,12 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_ring_kernel(const
 #pragma unroll
     for (int i = 0; i < IPS; ++i) dB[j][i] = lane_offsets(std::integral_constant<bool, B_KC>{}, g.N, n0, ldb_b, j, i);
 
+  // LDS address of the ring (the transfers name their destination by address, not through a pointer)
+  const uint32_t lds_base = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds_raw)));
   // Issues slot j of a stage whose k = 0 is at (a_stage, b_stage) into ring position pos.
   auto issue = [&](auto jtag, const char* a_stage, const char* b_stage, int pos) {
     constexpr int j = decltype(jtag)::value;
-    const uint32_t dst = static_cast<uint32_t>(pos * RING_SLOT_BYTES + wave * 1024);
+    const uint32_t dst = lds_base + static_cast<uint32_t>(pos * RING_SLOT_BYTES + wave * 1024);
 #pragma unroll
     for (int i = 0; i < IPS; ++i) {
       if constexpr (j < SA) dma16(dA[j][i], a_stage, dst + i * NW * 1024);
@@ -207,103 +219,219 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_ring_kernel(const
   ring_barrier();
 
   NMTG_PROF_MARK(1);
+  constexpr int KG = GEMM_BK / 16;                                        // k-groups (MFMA depths) per stage
+  constexpr int READS = (A_KC ? TM : 2 * TM) + (B_KC ? TN : 2 * TN);     // LDS read instructions per k-group
+  constexpr int MFMAS = TM * TN;
+  auto load_frags = [&](auto kk_tag, const uint8_t* sa, const uint8_t* sb, uint4 (&fm_)[TM], uint4 (&fn_)[TN]) {
+    constexpr int kk = decltype(kk_tag)::value;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      if constexpr (A_KC) {
+        fm_[i] = *reinterpret_cast<const uint4*>(sa + fa[i][kk]);
+      } else {
+        const uint8_t* p = sa + fa[i][0] + kk * 16 * 256;
+        const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(p));
+        const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(p + 4 * 256));
+        union { short4_t s[2]; uint4 u; } cv;
+        cv.s[0] = lo;
+        cv.s[1] = hi;
+        fm_[i] = cv.u;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      if constexpr (B_KC) {
+        fn_[j] = *reinterpret_cast<const uint4*>(sb + fb[j][kk]);
+      } else {
+        const uint8_t* p = sb + fb[j][0] + kk * 16 * 256;
+        const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(p));
+        const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(p + 4 * 256));
+        union { short4_t s[2]; uint4 u; } cv;
+        cv.s[0] = lo;
+        cv.s[1] = hi;
+        fn_[j] = cv.u;
+      }
+    }
+  };
   int pos_r = 0, pos_w = 0;
-  const char* a_cur = a_base - step_a;  // stage s - 1 at the top of iteration s
+  const char* a_cur = a_base - step_a;  // stage p - 1 at the top of phase p
   const char* b_cur = b_base - step_b;
-  for (int s = 0; s < nk; ++s) {
-    if (s >= 1) {
-      // the slots of stage s - 1 are free: issue the next SPS slots of the sequence
+  // Top of phase p >= 1: the slots of stage p - 1 are free (every wavefront has passed the barrier behind its reads):
+  // issue the next SPS slots of the sequence.
+  auto refill = [&](int p) {
+    if (p >= 1) {
       static_for<0, SPS>([&](auto tt) {
         constexpr int t = decltype(tt)::value;
         constexpr int j = (RING + t) % SPS, d = (RING + t) / SPS;
-        if (s - 1 + d < nk) issue(std::integral_constant<int, j>{}, a_cur + d * step_a, b_cur + d * step_b, pos_w);
+        if (p - 1 + d < nk) issue(std::integral_constant<int, j>{}, a_cur + d * step_a, b_cur + d * step_b, pos_w);
         pos_w = (pos_w + 1 == RING) ? 0 : pos_w + 1;
       });
     }
     a_cur += step_a;
     b_cur += step_b;
+  };
+  // End of phase p: stage p + 1 must have landed for every wavefront before anyone reads it.
+  auto certify_next = [&](int p) {
+    if (p + 1 < nk) {
+      const int issued = min(RING + p * SPS, total);
+      wait_vmcnt_upto<(RING - 2 * SPS) * IPS, IPS>((issued - (p + 2) * SPS) * IPS);
+    }
+    ring_barrier();
+  };
 
-    int pa = pos_r + ja, pb = pos_r + SA + jb;
-    if (pa >= RING) pa -= RING;
-    if (pb >= RING) pb -= RING;
-    const uint8_t* sa = lds_raw + pa * RING_SLOT_BYTES;
-    const uint8_t* sb = lds_raw + pb * RING_SLOT_BYTES;
-    // Fragments are double-buffered in registers: the LDS reads of k-group kk + 1 are issued ahead of the MFMAs of
-    // k-group kk, so the matrix pipe does not wait for the LDS latency (with the 128x128 tile there is one wavefront
-    // per SIMD and nothing else to hide it).
-    uint4 fm[2][TM], fn[2][TN];
-    auto load_frags = [&](auto kk_tag, uint4 (&fm_)[TM], uint4 (&fn_)[TN]) {
-      constexpr int kk = decltype(kk_tag)::value;
+  if constexpr (!STEPBUF) {
+    for (int s = 0; s < nk; ++s) {
+      refill(s);
+      int pa = pos_r + ja, pb = pos_r + SA + jb;
+      if (pa >= RING) pa -= RING;
+      if (pb >= RING) pb -= RING;
+      const uint8_t* sa = lds_raw + pa * RING_SLOT_BYTES;
+      const uint8_t* sb = lds_raw + pb * RING_SLOT_BYTES;
+      {
+        // Fragments are double-buffered in registers: the LDS reads of k-group kk + 1 are issued ahead of the MFMAs of
+        // k-group kk.
+        uint4 fm[2][TM], fn[2][TN];
+        load_frags(std::integral_constant<int, 0>{}, sa, sb, fm[0], fn[0]);
+        static_for<0, KG>([&](auto kk_tag) {
+          constexpr int kk = decltype(kk_tag)::value;
+          if constexpr (kk + 1 < KG) load_frags(std::integral_constant<int, kk + 1>{}, sa, sb, fm[(kk + 1) & 1], fn[(kk + 1) & 1]);
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        if constexpr (A_KC) {
-          fm_[i] = *reinterpret_cast<const uint4*>(sa + fa[i][kk]);
-        } else {
-          const uint8_t* p = sa + fa[i][0] + kk * 16 * 256;
-          const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(p));
-          const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(p + 4 * 256));
-          union { short4_t s[2]; uint4 u; } cv;
-          cv.s[0] = lo;
-          cv.s[1] = hi;
-          fm_[i] = cv.u;
-        }
-      }
+          for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        if constexpr (B_KC) {
-          fn_[j] = *reinterpret_cast<const uint4*>(sb + fb[j][kk]);
-        } else {
-          const uint8_t* p = sb + fb[j][0] + kk * 16 * 256;
-          const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(p));
-          const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(p + 4 * 256));
-          union { short4_t s[2]; uint4 u; } cv;
-          cv.s[0] = lo;
-          cv.s[1] = hi;
-          fn_[j] = cv.u;
-        }
+            for (int j = 0; j < TN; ++j) mfma<T>::run(fn[kk & 1][j], fm[kk & 1][i], acc[i][j]);
+        });
+        // Pin that order (the scheduler otherwise sinks the reads back down to save registers): the first k-group's
+        // reads, then for every k-group its MFMAs with the next group's reads dealt out one per MFMA from the start.
+        __builtin_amdgcn_sched_group_barrier(0x100, READS, 0);
+        static_for<0, KG>([&](auto kk_tag) {
+          constexpr int kk = decltype(kk_tag)::value;
+          if constexpr (kk + 1 < KG) {
+            constexpr int PAIRS = READS < MFMAS ? READS : MFMAS;
+            static_for<0, PAIRS>([&](auto) {
+              __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+              __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            });
+            if constexpr (READS > PAIRS) __builtin_amdgcn_sched_group_barrier(0x100, READS - PAIRS, 0);
+            if constexpr (MFMAS > PAIRS) __builtin_amdgcn_sched_group_barrier(0x008, MFMAS - PAIRS, 0);
+          } else {
+            __builtin_amdgcn_sched_group_barrier(0x008, MFMAS, 0);
+          }
+        });
       }
+      pos_r += SPS;
+      if (pos_r >= RING) pos_r -= RING;
+      certify_next(s);
+    }
+  } else {
+    // Two register sets of a whole stage's fragments; phases alternate between them. Phase 0 only reads, the phase
+    // behind the last stage only multiplies; they are peeled off so that the loop body is two straight middle phases
+    // (with the MFMAs in branches the accumulators end up in different registers on different paths and are copied
+    // at every join).
+    uint4 fmS[2][KG][TM], fnS[2][KG][TN];
+    auto stage_slots = [&](const uint8_t*& sa, const uint8_t*& sb) {
+      int pa = pos_r + ja, pb = pos_r + SA + jb;
+      if (pa >= RING) pa -= RING;
+      if (pb >= RING) pb -= RING;
+      sa = lds_raw + pa * RING_SLOT_BYTES;
+      sb = lds_raw + pb * RING_SLOT_BYTES;
+      pos_r += SPS;
+      if (pos_r >= RING) pos_r -= RING;
     };
-    load_frags(std::integral_constant<int, 0>{}, fm[0], fn[0]);
-    static_for<0, GEMM_BK / 16>([&](auto kk_tag) {
-      constexpr int kk = decltype(kk_tag)::value;
-      if constexpr (kk + 1 < GEMM_BK / 16) load_frags(std::integral_constant<int, kk + 1>{}, fm[(kk + 1) & 1], fn[(kk + 1) & 1]);
+    auto multiply = [&](auto set_tag) {
+      constexpr int Q = decltype(set_tag)::value;
+      static_for<0, KG>([&](auto kk_tag) {
+        constexpr int kk = decltype(kk_tag)::value;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j) mfma<T>::run(fnS[Q][kk][j], fmS[Q][kk][i], acc[i][j]);
+      });
+    };
+    // End of the first k-group of phase p >= 1: stage p must have landed for every wavefront, and every wavefront must be
+    // done with its reads of stage p - 1 (issued in phase p - 1; their last ones land under this phase's first MFMAs).
+    auto certify_cur = [&](int p) {
+      const int issued = min(RING + (p - 1) * SPS, total);
+      wait_vmcnt_upto<(RING - 2 * SPS) * IPS, IPS>((issued - (p + 1) * SPS) * IPS);
+      ring_barrier();
+    };
+    auto middle = [&](auto par_tag, int p) {
+      constexpr int P = decltype(par_tag)::value;   // set written in this phase; the MFMAs read set P ^ 1
+      const uint8_t *sa, *sb;
+      stage_slots(sa, sb);
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j) mfma<T>::run(fn[kk & 1][j], fm[kk & 1][i], acc[i][j]);
-    });
-    // Pin that order (the scheduler otherwise sinks the reads back down to save registers): the first k-group's reads,
-    // then for every k-group its MFMAs with the next group's reads dealt out one per MFMA from the start.
-    constexpr int READS = (A_KC ? TM : 2 * TM) + (B_KC ? TN : 2 * TN);   // LDS read instructions per k-group
-    constexpr int MFMAS = TM * TN;
-    __builtin_amdgcn_sched_group_barrier(0x100, READS, 0);
-    static_for<0, GEMM_BK / 16>([&](auto kk_tag) {
-      constexpr int kk = decltype(kk_tag)::value;
-      if constexpr (kk + 1 < GEMM_BK / 16) {
-        constexpr int PAIRS = READS < MFMAS ? READS : MFMAS;
-        static_for<0, PAIRS>([&](auto) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        for (int j = 0; j < TN; ++j) mfma<T>::run(fnS[P ^ 1][0][j], fmS[P ^ 1][0][i], acc[i][j]);
+      certify_cur(p);
+      refill(p);
+      // the other k-groups of stage p - 1, with all of stage p's reads dealt out between them
+      static_for<0, KG>([&](auto kk_tag) {
+        constexpr int kk = decltype(kk_tag)::value;
+        load_frags(kk_tag, sa, sb, fmS[P][kk], fnS[P][kk]);
+        if constexpr (kk >= 1) {
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) mfma<T>::run(fnS[P ^ 1][kk][j], fmS[P ^ 1][kk][i], acc[i][j]);
+        }
+      });
+      constexpr int NM = (KG - 1) * MFMAS, NR = KG * READS;
+      static_for<0, NM>([&](auto it) {
+        constexpr int i = decltype(it)::value;
+        constexpr int r = (i + 1) * NR / NM - i * NR / NM;
+        if constexpr (r > 0) __builtin_amdgcn_sched_group_barrier(0x100, r, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      });
+    };
+    if (nk > 0) {
+      {
+        refill(0);
+        const uint8_t *sa, *sb;
+        stage_slots(sa, sb);
+        static_for<0, KG>([&](auto kk_tag) {
+          constexpr int kk = decltype(kk_tag)::value;
+          load_frags(kk_tag, sa, sb, fmS[0][kk], fnS[0][kk]);
         });
-        if constexpr (READS > PAIRS) __builtin_amdgcn_sched_group_barrier(0x100, READS - PAIRS, 0);
-        if constexpr (MFMAS > PAIRS) __builtin_amdgcn_sched_group_barrier(0x008, MFMAS - PAIRS, 0);
-      } else {
-        __builtin_amdgcn_sched_group_barrier(0x008, MFMAS, 0);
       }
-    });
-    pos_r += SPS;
-    if (pos_r >= RING) pos_r -= RING;
-
-    // stage s + 1 must have landed for every wavefront before anyone reads it
-    if (s + 1 < nk) {
-      const int issued = min(RING + s * SPS, total);
-      wait_vmcnt_upto<(RING - 2 * SPS) * IPS, IPS>((issued - (s + 2) * SPS) * IPS);
+      int p = 1;
+      for (; p + 1 < nk; p += 2) {
+        middle(std::integral_constant<int, 1>{}, p);
+        middle(std::integral_constant<int, 0>{}, p + 1);
+      }
+      if (p < nk) {
+        middle(std::integral_constant<int, 1>{}, p);
+        multiply(std::integral_constant<int, 1>{});
+      } else {
+        multiply(std::integral_constant<int, 0>{});
+      }
+      ring_barrier();   // every wavefront is done reading the ring: the epilogue stages the output tile there
     }
-    ring_barrier();
   }
 
   NMTG_PROF_MARK(2);
   gemm_epilogue<T, BM, BN, WAVES_M, WAVES_N, EPI, 8, true>(g, acc, lds_raw, tile_m, tile_n, bz, split);
+}
+
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC, int EPI, int RING, bool STEPBUF = false>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_ring_kernel(const GemmArgs g) {
+  gemm_ring_body<T, BM, BN, WAVES_M, WAVES_N, A_KC, B_KC, EPI, RING, STEPBUF>(g, static_cast<int>(blockIdx.x));
+}
+
+// The same kernel with riders: the first g.rider_blocks blocks of the grid's x extent (first batch and split only) run
+// a list of small reduction jobs instead of a tile (reduce.hip.h). A product that leaves one block on a CU has room
+// for a second one there; the riders' loads and adds fill the memory pipes that the main loop leaves idle, and the
+// launches those jobs would otherwise need fall away. The jobs are independent of this product. The riders come
+// first, one per CU, so that the tiles that follow spread over the CUs as they would without them.
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC, int EPI, int RING, bool STEPBUF = false>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_ring_rider_kernel(const GemmArgs g, const TailArgs riders) {
+  static_assert(64 * WAVES_M * WAVES_N == 256, "the reduction jobs are written for blocks of 256 threads");
+  if (static_cast<int>(blockIdx.x) < g.rider_blocks) {
+    extern __shared__ __align__(16) uint8_t lds_raw[];   // the launch's ring memory: far more than a rider needs
+    if (blockIdx.y == 0 && blockIdx.z == 0)
+      tail_ride<T>(riders, static_cast<int>(blockIdx.x), g.rider_blocks, reinterpret_cast<float*>(lds_raw));
+    return;
+  }
+  gemm_ring_body<T, BM, BN, WAVES_M, WAVES_N, A_KC, B_KC, EPI, RING, STEPBUF>(g, static_cast<int>(blockIdx.x) - g.rider_blocks);
 }
 
 }  // namespace nmtg

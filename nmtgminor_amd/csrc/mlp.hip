@@ -176,6 +176,17 @@ extern "C" int nmtg_mlp_bwd(int num_layers, const void* x, const void* const* we
   const void* g_cur = grad_out;      // gradient wrt layer i's linear output
   bool bias_from_parts = false;      // colsum_ws holds the partial column sums of g_cur
   int parts_rows = 0;
+  // The final reductions (split-K sums, bias-gradient sums) ride along with the last data-gradient product, which
+  // leaves room on the CUs (GemmArgs::riders); where there is no such product they are one launch at the end. The
+  // partial column sums of the output gradient, which those read, are a launch of their own ahead of the GEMMs.
+  const int max_riders = num_cus();   // one rider per CU, whatever the number of jobs' blocks
+  ReduceTail head;                   // partial column sums of grad_out, owed before the tail's final sums
+  bool head_pending = false;
+  auto flush_head = [&]() -> int {
+    if (!head_pending) return 0;
+    head_pending = false;
+    return tail_launch(head, dtype, st);
+  };
   for (int i = num_layers - 1; i >= 0; --i) {
     const int64_t out_i = out_features[i];
     const int64_t in_i = i == 0 ? in_features : out_features[i - 1];
@@ -189,7 +200,8 @@ extern "C" int nmtg_mlp_bwd(int num_layers, const void* x, const void* const* we
         rc = 0;
         if (!bias_from_parts) {
           parts = colsum_parts(static_cast<int>(batch));
-          rc = colsum_partial_run(dtype, g_cur, out_i, static_cast<int>(batch), static_cast<int>(out_i), colsum_ws, st);
+          rc = tail_add_colsum_partial(head, dtype, g_cur, out_i, static_cast<int>(batch), static_cast<int>(out_i), colsum_ws);
+          head_pending = !rc;
         }
         if (!rc) rc = tail_add_colsum(tail, colsum_ws, parts, static_cast<int>(out_i), grad_biases[i]);
       } else if (bias_from_parts) {
@@ -208,6 +220,9 @@ extern "C" int nmtg_mlp_bwd(int num_layers, const void* x, const void* const* we
       g.M = static_cast<int>(out_i); g.N = static_cast<int>(in_i); g.K = static_cast<int>(batch);
       g.batch = 1; g.alpha = 1.f;
       g.defer_reduce = (tail_mode && !tail.full()) ? 1 : 0;
+      // (the partial column sums do not ride with this product: a split-K launch repeats the rider blocks in every
+      // split, and the tiles then share CUs unevenly; measured slower than the launch of their own)
+      if (int rc2 = flush_head()) return rc2;
       GemmArgs planned{};
       rc = gemm_run(dtype, LAYOUT_TN, EPI_PLAIN, g, splitk_region(i), plan.splitk_bytes, st, nullptr, &planned);
       if (!rc && planned.defer_reduce && planned.splits > 1)
@@ -241,15 +256,20 @@ extern "C" int nmtg_mlp_bwd(int num_layers, const void* x, const void* const* we
       bias_from_parts = g.colsum_part != nullptr;
       g_cur = dh[i & 1];
     } else if (grad_x != nullptr) {
+      if (int rc2 = flush_head()) return rc2;     // the tail's final sums read what the head writes
       GemmArgs g{};
       g.A = g_cur; g.lda = out_i;
       g.B = weights[0]; g.ldb = in_i;
       g.C = grad_x; g.ldc = in_i;
       g.M = static_cast<int>(batch); g.N = static_cast<int>(in_i); g.K = static_cast<int>(out_i);
       g.batch = 1; g.alpha = 1.f;
-      rc = gemm_run(dtype, LAYOUT_NN, EPI_PLAIN, g, nullptr, 0, st);
+      if (!tail.empty()) { g.riders = &tail.args; g.rider_blocks = max_riders; }
+      GemmArgs planned{};
+      rc = gemm_run(dtype, LAYOUT_NN, EPI_PLAIN, g, nullptr, 0, st, nullptr, &planned);
       if (rc) return rc;
+      if (planned.riders_taken) return 0;        // every reduction has run beside this product
     }
   }
+  if (int rc = flush_head()) return rc;
   return tail_launch(tail, dtype, st);
 }

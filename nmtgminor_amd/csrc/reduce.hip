@@ -7,7 +7,8 @@ namespace {
 int ceil_div(int a, int b) { return (a + b - 1) / b; }
 }  // namespace
 
-int colsum_parts(int M) { return std::max(1, std::min(64, ceil_div(M, 128))); }
+// row blocks of 64 rows (eight rows per row lane), at most 256 of them: a [8192 x 512] gradient is 256 blocks
+int colsum_parts(int M) { return std::max(1, std::min(256, ceil_div(M, 64))); }
 
 int colsum_finish(int dtype, const float* part, int parts, int N, void* out, hipStream_t st) {
   TraceScope trace("colsum_final", st);
@@ -73,11 +74,28 @@ int tail_add_colsum(ReduceTail& t, const float* part, int parts, int N, void* ou
   return 0;
 }
 
+int tail_add_colsum_partial(ReduceTail& t, int dtype, const void* X, int64_t ld, int M, int N, float* part) {
+  if (t.full()) return fail(NMTG_ERR_UNSUPPORTED, "reduce tail: too many jobs");
+  const int parts = colsum_parts(M);
+  const bool vec = dtype != NMTG_F32 && aligned16(X) && ld % 8 == 0 && N % 8 == 0;
+  TailJob& j = t.args.job[t.args.njobs++];
+  j = TailJob{};
+  j.kind = vec ? TAIL_COLSUM_PARTIAL_VEC : TAIL_COLSUM_PARTIAL;
+  j.first_block = t.blocks;
+  j.x = X; j.ldc = ld; j.M = M; j.N = N; j.dst = part;
+  j.rows_per_block = ceil_div(M, parts);
+  j.col_blocks = ceil_div(N, vec ? 256 : 32);
+  t.blocks += j.col_blocks * parts;
+  return 0;
+}
+
 int tail_launch(const ReduceTail& t, int dtype, hipStream_t st) {
   if (t.args.njobs == 0 || t.blocks == 0) return 0;
   TraceScope trace("reduce_tail", st);
+  const TailArgs args = t.args;
+  const unsigned blocks = static_cast<unsigned>(args.blocks);
   NMTG_DISPATCH_DTYPE(dtype, T,
-                      hipLaunchKernelGGL((reduce_tail_kernel<T>), dim3(static_cast<unsigned>(t.blocks)), dim3(256), 0, st, t.args));
+                      hipLaunchKernelGGL((reduce_tail_kernel<T>), dim3(blocks), dim3(256), 0, st, args));
   NMTG_CHECK_LAUNCH("reduce_tail");
   return 0;
 }

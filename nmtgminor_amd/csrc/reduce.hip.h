@@ -3,6 +3,7 @@
 // in flight before the first add. Hosts: reduce.hip (column sums), gemm_inst.hip.h (split-K).
 #pragma once
 #include "common.hip.h"
+#include <type_traits>
 
 namespace nmtg {
 
@@ -62,47 +63,51 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
 // Column sums of a row-major [M, N] matrix: partial[mb][n] over row blocks (fp32), fixed order.
 // Block = 32 column lanes (8 columns each = one 16-byte load for 16-bit T) x 8 row lanes.
 template <typename T, bool VEC>
-__global__ __launch_bounds__(256) void colsum_partial_kernel(const T* __restrict__ X, int64_t ld, int M, int N,
-                                                             int rows_per_block, float* __restrict__ part) {
+__device__ __forceinline__ void colsum_partial_block(int bx, int by, const T* __restrict__ X, int64_t ld, int M, int N,
+                                                     int rows_per_block, float* __restrict__ part, float* red_lds) {
   constexpr int CPT = VEC ? 8 : 1;
-  __shared__ float red[8][32 * CPT + 1];
+  float (*red)[32 * CPT + 1] = reinterpret_cast<float (*)[32 * CPT + 1]>(red_lds);   // [8][32 * CPT + 1] floats of LDS
   const int cl = threadIdx.x & 31, rl = threadIdx.x >> 5;
-  const int n = (blockIdx.x * 32 + cl) * CPT;
-  const int r0 = blockIdx.y * rows_per_block;
+  const int n = (bx * 32 + cl) * CPT;
+  const int r0 = by * rows_per_block;
   const int r1 = min(M, r0 + rows_per_block);
   float s[CPT];
 #pragma unroll
   for (int j = 0; j < CPT; ++j) s[j] = 0.f;
   if (n < N) {
-    // Latency-bound (few blocks, short rows): 16 rows are loaded before any is added (two loops on
-    // purpose, see ln_bwd_finalize_kernel); the sum order is unchanged.
-    constexpr int BATCH = 16;
+    // Latency-bound (few blocks, short rows): 16 (then 8) rows are loaded before any is added (two loops on
+    // purpose, see ln_bwd_finalize_kernel); the sum order is that of the rows.
     int r = r0 + rl;
-    for (; r + (BATCH - 1) * 8 < r1; r += BATCH * 8) {
-      // raw words first, conversion only in the adding loop (a conversion is a use of the load)
-      constexpr int NV = (CPT * sizeof(T)) / 16;   // 16-byte vectors per access; 0 in the scalar form
-      if constexpr (NV > 0) {
-        uint4 raw[BATCH][NV];
+    auto batched = [&](auto batch_tag) {
+      constexpr int BATCH = decltype(batch_tag)::value;
+      for (; r + (BATCH - 1) * 8 < r1; r += BATCH * 8) {
+        // raw words first, conversion only in the adding loop (a conversion is a use of the load)
+        constexpr int NV = (CPT * sizeof(T)) / 16;   // 16-byte vectors per access; 0 in the scalar form
+        if constexpr (NV > 0) {
+          uint4 raw[BATCH][NV];
 #pragma unroll
-        for (int u = 0; u < BATCH; ++u)
+          for (int u = 0; u < BATCH; ++u)
 #pragma unroll
-          for (int i = 0; i < NV; ++i)
-            raw[u][i] = reinterpret_cast<const uint4*>(X + static_cast<int64_t>(r + u * 8) * ld + n)[i];
-        __builtin_amdgcn_sched_barrier(0);   // keep every load ahead of the first add
+            for (int i = 0; i < NV; ++i)
+              raw[u][i] = reinterpret_cast<const uint4*>(X + static_cast<int64_t>(r + u * 8) * ld + n)[i];
+          __builtin_amdgcn_sched_barrier(0);   // keep every load ahead of the first add
 #pragma unroll
-        for (int u = 0; u < BATCH; ++u) {
-          const T* e = reinterpret_cast<const T*>(raw[u]);
+          for (int u = 0; u < BATCH; ++u) {
+            const T* e = reinterpret_cast<const T*>(raw[u]);
 #pragma unroll
-          for (int j = 0; j < CPT; ++j) s[j] += elem<T>::to_float(e[j]);
+            for (int j = 0; j < CPT; ++j) s[j] += elem<T>::to_float(e[j]);
+          }
+        } else {
+          T raw[BATCH];
+#pragma unroll
+          for (int u = 0; u < BATCH; ++u) raw[u] = X[static_cast<int64_t>(r + u * 8) * ld + n];
+#pragma unroll
+          for (int u = 0; u < BATCH; ++u) s[0] += elem<T>::to_float(raw[u]);
         }
-      } else {
-        T raw[BATCH];
-#pragma unroll
-        for (int u = 0; u < BATCH; ++u) raw[u] = X[static_cast<int64_t>(r + u * 8) * ld + n];
-#pragma unroll
-        for (int u = 0; u < BATCH; ++u) s[0] += elem<T>::to_float(raw[u]);
       }
-    }
+    };
+    batched(std::integral_constant<int, 16>{});
+    batched(std::integral_constant<int, 8>{});
     for (; r < r1; r += 8) {
       float v[CPT];
       load_pack<T, CPT>(X + static_cast<int64_t>(r) * ld + n, v);
@@ -114,14 +119,22 @@ __global__ __launch_bounds__(256) void colsum_partial_kernel(const T* __restrict
   for (int j = 0; j < CPT; ++j) red[rl][cl * CPT + j] = s[j];
   __syncthreads();
   for (int c = threadIdx.x; c < 32 * CPT; c += 256) {
-    const int col = blockIdx.x * 32 * CPT + c;
+    const int col = bx * 32 * CPT + c;
     if (col < N) {
       float t = 0.f;
 #pragma unroll
       for (int k = 0; k < 8; ++k) t += red[k][c];
-      part[static_cast<int64_t>(blockIdx.y) * N + col] = t;
+      part[static_cast<int64_t>(by) * N + col] = t;
     }
   }
+  __syncthreads();   // a caller that runs several of these blocks one after the other reuses `red`
+}
+
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void colsum_partial_kernel(const T* __restrict__ X, int64_t ld, int M, int N,
+                                                             int rows_per_block, float* __restrict__ part) {
+  __shared__ float red[8 * (32 * (VEC ? 8 : 1) + 1)];
+  colsum_partial_block<T, VEC>(blockIdx.x, blockIdx.y, X, ld, M, N, rows_per_block, part, red);
 }
 
 // out[n] = T(sum_p part[p][n]) in order p = 0..parts-1; 8 partial rows in flight per thread.
@@ -169,29 +182,43 @@ template <> struct tile_cfg<TILE_M> { static constexpr int BM = 128, BN = 128, W
 template <> struct tile_cfg<TILE_S> { static constexpr int BM = 256, BN = 64, WM = 4, WN = 1; };
 template <> struct tile_cfg<TILE_R> { static constexpr int BM = 128, BN = 512, WM = 4, WN = 2; };
 
-enum TailKind { TAIL_SPLITK_M = 1, TAIL_SPLITK_L = 2, TAIL_COLSUM = 3 };
+enum TailKind { TAIL_SPLITK_M = 1, TAIL_SPLITK_L = 2, TAIL_COLSUM = 3, TAIL_COLSUM_PARTIAL = 4, TAIL_COLSUM_PARTIAL_VEC = 5 };
 struct TailJob {
   int kind;
   int first_block;       // the job's blocks are [first_block, next job's first_block)
   const float* src;      // split-K partials / column-sum partial rows
   void* dst;
-  int64_t ldc, sC;
+  int64_t ldc, sC;       // TAIL_COLSUM_PARTIAL*: ldc = row pitch of x
   int M, N, m_tiles, n_tiles, batch, splits, c_vec, parts;
   float alpha;
+  const void* x;         // TAIL_COLSUM_PARTIAL*: the matrix whose columns are summed (dst: fp32 partial rows)
+  int rows_per_block, col_blocks;
 };
 constexpr int TAIL_MAX_JOBS = 8;
 struct TailArgs {
   int njobs;
+  int blocks;            // all jobs together
   TailJob job[TAIL_MAX_JOBS];
 };
 
+constexpr int TAIL_LDS_FLOATS = 8 * (32 * 8 + 1);   // what a partial column sum needs
+
+// One block of 256 threads runs block `vb` of the job list: exactly what the stand-alone kernel's block does.
+// lds: TAIL_LDS_FLOATS floats of LDS for the block's use.
 template <typename T>
-__global__ __launch_bounds__(256) void reduce_tail_kernel(const TailArgs a) {
+__device__ __forceinline__ void tail_block(const TailArgs& a, int vb, float* lds) {
   int j = 0;
-  while (j + 1 < a.njobs && static_cast<int>(blockIdx.x) >= a.job[j + 1].first_block) ++j;
+  while (j + 1 < a.njobs && vb >= a.job[j + 1].first_block) ++j;
   const TailJob& t = a.job[j];
-  const int64_t local = static_cast<int64_t>(blockIdx.x - t.first_block) * 256 + threadIdx.x;
-  if (t.kind == TAIL_SPLITK_M) {
+  const int64_t local = static_cast<int64_t>(vb - t.first_block) * 256 + threadIdx.x;
+  if (t.kind == TAIL_COLSUM_PARTIAL || t.kind == TAIL_COLSUM_PARTIAL_VEC) {
+    const int lb = vb - t.first_block, bx = lb % t.col_blocks, by = lb / t.col_blocks;
+    if (t.kind == TAIL_COLSUM_PARTIAL_VEC) {
+      if constexpr (sizeof(T) == 2) colsum_partial_block<T, true>(bx, by, static_cast<const T*>(t.x), t.ldc, t.M, t.N, t.rows_per_block, static_cast<float*>(t.dst), lds);
+    } else {
+      colsum_partial_block<T, false>(bx, by, static_cast<const T*>(t.x), t.ldc, t.M, t.N, t.rows_per_block, static_cast<float*>(t.dst), lds);
+    }
+  } else if (t.kind == TAIL_SPLITK_M) {
     using C = tile_cfg<TILE_M>;
     splitk_reduce_slot<T, C::BM, C::BN, C::WM, C::WN>(local, t.src, static_cast<T*>(t.dst), t.ldc, t.M, t.N, t.m_tiles, t.n_tiles,
                                                       t.batch, t.sC, t.splits, t.alpha, t.c_vec);
@@ -204,16 +231,33 @@ __global__ __launch_bounds__(256) void reduce_tail_kernel(const TailArgs a) {
   }
 }
 
+template <typename T>
+__global__ __launch_bounds__(256) void reduce_tail_kernel(const TailArgs a) {
+  __shared__ float lds[TAIL_LDS_FLOATS];
+  tail_block<T>(a, static_cast<int>(blockIdx.x), lds);
+}
+
+// The same job list run by `nriders` blocks that ride along in another kernel's launch (gemm_ring.hip.h): the blocks
+// of the list are dealt out round-robin.
+template <typename T>
+__device__ __forceinline__ void tail_ride(const TailArgs& a, int rider, int nriders, float* lds) {
+  for (int vb = rider; vb < a.blocks; vb += nriders) tail_block<T>(a, vb, lds);
+}
+
 // Host side (reduce.hip): a list of jobs of one dtype, launched once.
 struct ReduceTail {
   TailArgs args;
-  int blocks;
-  ReduceTail() : blocks(0) { args.njobs = 0; }
+  int& blocks;
+  ReduceTail() : blocks(args.blocks) { args.njobs = 0; args.blocks = 0; }
+  ReduceTail(const ReduceTail&) = delete;
   bool full() const { return args.njobs >= TAIL_MAX_JOBS; }
+  bool empty() const { return args.njobs == 0 || args.blocks == 0; }
 };
 int tail_add_splitk(ReduceTail& t, int tile, const float* ws, void* C, int64_t ldc, int M, int N, int m_tiles, int n_tiles,
                     int batch, int64_t sC, int splits, float alpha, int c_vec);
 int tail_add_colsum(ReduceTail& t, const float* part, int parts, int N, void* out);
+// the partial phase of a column sum as a job (what colsum_partial_run launches on its own)
+int tail_add_colsum_partial(ReduceTail& t, int dtype, const void* X, int64_t ld, int M, int N, float* part);
 int tail_launch(const ReduceTail& t, int dtype, hipStream_t st);
 // the partial phase of colsum_run alone (its final sum is then queued with tail_add_colsum)
 int colsum_partial_run(int dtype, const void* X, int64_t ld, int M, int N, float* part, hipStream_t st);

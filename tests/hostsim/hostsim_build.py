@@ -42,7 +42,7 @@ ASM_REWRITES = [
     # one 1 KB global -> LDS transfer: lane l copies 16 bytes from sbase + voff to LDS address lds_addr + 16 l
     (r'asm volatile\("s_mov_b32 m0, %2\\n\\ts_nop 0\\n\\tglobal_load_lds_dwordx4 %0, %1"\s*:\s*:\s*"v"\(voff\), "s"\(sbase\), '
      r'"s"\(lds_addr\)\s*:\s*"memory", "m0"\);',
-     "::hostsim::dma_issue(static_cast<const char*>(sbase) + voff, lds_addr + 16 * ::hostsim::lane_id(), 16);"),
+     "::hostsim::dma_issue(static_cast<const char*>(sbase) + voff, ::hostsim::lds_offset_of(lds_addr) + 16 * ::hostsim::lane_id(), 16);"),
     # LDS reads done, then the workgroup barrier
     (r'asm volatile\("s_waitcnt lgkmcnt\(0\)\\n\\ts_barrier" ::: "memory"\);', "::hostsim::sync_block();"),
 ]

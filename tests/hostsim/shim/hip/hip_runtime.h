@@ -63,6 +63,9 @@ extern unsigned char* dynamic_lds;   // at least dynamic_lds_bytes of the curren
 extern hostsim::Index threadIdx, blockIdx;
 extern dim3 blockDim, gridDim;
 
+// cycle counters (tuning aids of the kernels): no clock on the host
+static inline long long clock64() { return 0; }
+static inline long long wall_clock64() { return 0; }
 static inline hipError_t hipGetLastError() { return hipSuccess; }
 static inline const char* hipGetErrorString(hipError_t) { return "host simulation"; }
 static inline hipError_t hipGetDevice(int* dev) { *dev = 0; return hipSuccess; }

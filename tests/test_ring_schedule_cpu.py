@@ -80,6 +80,65 @@ def simulate(ring, sa, sb, ips, nk):
     return len(issued)
 
 
+def simulate_stepbuf(ring, sa, sb, ips, nk):
+    """The loop form that keeps a whole stage's fragments in registers: phase p reads stage p (phase 0 ahead of the loop);
+    a phase p >= 1 first multiplies, then waits for stage p, passes the barrier, refills the slots of stage p - 1 and
+    reads stage p. Same three properties as simulate()."""
+    sps = sa + sb
+    assert ring >= 2 * sps
+    total = nk * sps
+    issued, content, covered, visible = [], [None] * ring, set(), set()
+    done_reading = -1      # newest stage whose reads a barrier has closed
+
+    def issue(q, pos):
+        old = content[pos]
+        if old is not None:
+            assert old // sps <= done_reading, (ring, sps, nk, q, pos, old, done_reading)   # property 2
+        content[pos] = q
+        issued.extend((q, i) for i in range(ips))
+
+    def wait(n, max_n):
+        k = min(n, max_n)
+        assert k >= 0 and k % ips == 0
+        for q, _ in (issued if k == 0 else issued[:-k]):
+            covered.add(q)
+
+    def read_stage(st, pos):
+        for j in range(sps):
+            p = pos + j - (ring if pos + j >= ring else 0)
+            q = st * sps + j
+            assert content[p] == q, (ring, sps, nk, st, j, p, content[p])     # property 3
+            assert q in visible, (ring, sps, nk, st, j)                        # property 1
+
+    for t in range(ring):
+        if t // sps < nk:
+            issue(t, t)
+    if nk > 0:
+        wait((min(ring, total) - sps) * ips, (ring - sps) * ips)
+    visible.update(covered)                                                   # barrier
+    if nk == 0:
+        return 0
+    pos_r = pos_w = 0
+    read_stage(0, pos_r)
+    pos_r = (pos_r + sps) % ring
+    for p in range(1, nk):
+        n_issued = min(ring + (p - 1) * sps, total)
+        assert n_issued * ips == len(issued)
+        wait((n_issued - (p + 1) * sps) * ips, (ring - 2 * sps) * ips)
+        visible.update(covered)                                               # barrier: also closes the reads of stage p - 1
+        done_reading = p - 1
+        for t in range(sps):
+            d = (ring + t) // sps
+            q = ring + (p - 1) * sps + t
+            assert q // sps == p - 1 + d and q % sps == (ring + t) % sps
+            if p - 1 + d < nk:
+                issue(q, pos_w)
+            pos_w = 0 if pos_w + 1 == ring else pos_w + 1
+        read_stage(p, pos_r)
+        pos_r = (pos_r + sps) % ring
+    return len(issued)
+
+
 CONFIGS = [(ring, sa, sb, ips) for ring, (sa, sb), ips in itertools.product((4, 5, 6, 8, 10), ((1, 1), (2, 1), (2, 2)), (2, 4))
            if ring >= 2 * (sa + sb)]
 
@@ -89,6 +148,13 @@ def test_ring_schedule_has_no_hazard(ring, sa, sb, ips):
     for nk in range(0, 70):
         n = simulate(ring, sa, sb, ips, nk)
         assert n == nk * (sa + sb) * ips          # every slot of every stage is issued exactly once
+
+
+@pytest.mark.parametrize("ring,sa,sb,ips", CONFIGS)
+def test_ring_schedule_with_a_stage_of_fragments_in_registers_has_no_hazard(ring, sa, sb, ips):
+    for nk in range(0, 70):
+        n = simulate_stepbuf(ring, sa, sb, ips, nk)
+        assert n == nk * (sa + sb) * ips
 
 
 def test_shipped_configurations_are_covered():
