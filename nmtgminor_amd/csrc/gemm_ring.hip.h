@@ -270,57 +270,72 @@ __device__ __forceinline__ void gemm_ring_body(const GemmArgs& g, int block_x) {
     a_cur += step_a;
     b_cur += step_b;
   };
-  // End of phase p: stage p + 1 must have landed for every wavefront before anyone reads it.
-  auto certify_next = [&](int p) {
-    if (p + 1 < nk) {
-      const int issued = min(RING + p * SPS, total);
-      wait_vmcnt_upto<(RING - 2 * SPS) * IPS, IPS>((issued - (p + 2) * SPS) * IPS);
-    }
-    ring_barrier();
-  };
-
   if constexpr (!STEPBUF) {
-    for (int s = 0; s < nk; ++s) {
-      refill(s);
-      int pa = pos_r + ja, pb = pos_r + SA + jb;
+    // Fragments are double-buffered in registers by k-group: the LDS reads of a k-group are issued under the MFMAs of
+    // the one before. The wait for the next stage and the barrier sit in front of the LAST k-group's MFMAs, not behind
+    // them: by then every read of the stage has been issued (and has had a k-group's MFMAs to land), so the slots can be
+    // handed back, and the last k-group multiplies out of registers while the first reads of the next stage go out. The
+    // matrix pipe has work on both sides of the barrier.
+    uint4 fm[2][TM], fn[2][TN];
+    auto mfmas = [&](auto buf_tag) {
+      constexpr int Bf = decltype(buf_tag)::value;
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) mfma<T>::run(fn[Bf][j], fm[Bf][i], acc[i][j]);
+    };
+    auto pin_pairs = [&]() {   // the MFMAs of one k-group with the reads of another dealt out one per MFMA from the start
+      constexpr int PAIRS = READS < MFMAS ? READS : MFMAS;
+      static_for<0, PAIRS>([&](auto) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      });
+      if constexpr (READS > PAIRS) __builtin_amdgcn_sched_group_barrier(0x100, READS - PAIRS, 0);
+      if constexpr (MFMAS > PAIRS) __builtin_amdgcn_sched_group_barrier(0x008, MFMAS - PAIRS, 0);
+    };
+    static_assert(KG % 2 == 0, "the fragment buffers alternate by k-group and the loop carries buffer 0 across steps");
+    auto slots_of = [&](int pos, const uint8_t*& sa, const uint8_t*& sb) {
+      int pa = pos + ja, pb = pos + SA + jb;
       if (pa >= RING) pa -= RING;
       if (pb >= RING) pb -= RING;
-      const uint8_t* sa = lds_raw + pa * RING_SLOT_BYTES;
-      const uint8_t* sb = lds_raw + pb * RING_SLOT_BYTES;
-      {
-        // Fragments are double-buffered in registers: the LDS reads of k-group kk + 1 are issued ahead of the MFMAs of
-        // k-group kk.
-        uint4 fm[2][TM], fn[2][TN];
-        load_frags(std::integral_constant<int, 0>{}, sa, sb, fm[0], fn[0]);
-        static_for<0, KG>([&](auto kk_tag) {
-          constexpr int kk = decltype(kk_tag)::value;
-          if constexpr (kk + 1 < KG) load_frags(std::integral_constant<int, kk + 1>{}, sa, sb, fm[(kk + 1) & 1], fn[(kk + 1) & 1]);
-#pragma unroll
-          for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j) mfma<T>::run(fn[kk & 1][j], fm[kk & 1][i], acc[i][j]);
-        });
-        // Pin that order (the scheduler otherwise sinks the reads back down to save registers): the first k-group's
-        // reads, then for every k-group its MFMAs with the next group's reads dealt out one per MFMA from the start.
-        __builtin_amdgcn_sched_group_barrier(0x100, READS, 0);
-        static_for<0, KG>([&](auto kk_tag) {
-          constexpr int kk = decltype(kk_tag)::value;
-          if constexpr (kk + 1 < KG) {
-            constexpr int PAIRS = READS < MFMAS ? READS : MFMAS;
-            static_for<0, PAIRS>([&](auto) {
-              __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-              __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            });
-            if constexpr (READS > PAIRS) __builtin_amdgcn_sched_group_barrier(0x100, READS - PAIRS, 0);
-            if constexpr (MFMAS > PAIRS) __builtin_amdgcn_sched_group_barrier(0x008, MFMAS - PAIRS, 0);
-          } else {
-            __builtin_amdgcn_sched_group_barrier(0x008, MFMAS, 0);
-          }
-        });
-      }
+      sa = lds_raw + pa * RING_SLOT_BYTES;
+      sb = lds_raw + pb * RING_SLOT_BYTES;
+    };
+    const uint8_t *sa, *sb;
+    if (nk > 0) {
+      refill(0);   // nothing to issue yet: moves the operand cursors onto stage 0
+      slots_of(0, sa, sb);
+      load_frags(std::integral_constant<int, 0>{}, sa, sb, fm[0], fn[0]);
+    }
+    // k-groups 0 .. KG - 2 of a stage, each under the reads of the next one
+    auto leading_groups = [&]() {
+      static_for<0, KG - 1>([&](auto kk_tag) {
+        constexpr int kk = decltype(kk_tag)::value;
+        load_frags(std::integral_constant<int, kk + 1>{}, sa, sb, fm[(kk + 1) & 1], fn[(kk + 1) & 1]);
+        mfmas(std::integral_constant<int, kk & 1>{});
+      });
+      static_for<0, KG - 1>([&](auto) { pin_pairs(); });
+    };
+    // every stage but the last (the last one is peeled off: with the MFMAs of a step in two branches the accumulators
+    // are copied where the branches join)
+    for (int s = 0; s + 1 < nk; ++s) {
+      leading_groups();
       pos_r += SPS;
       if (pos_r >= RING) pos_r -= RING;
-      certify_next(s);
+      // stage s + 1 must have landed for every wavefront, and every wavefront must be done reading stage s
+      const int issued = min(RING + s * SPS, total);
+      wait_vmcnt_upto<(RING - 2 * SPS) * IPS, IPS>((issued - (s + 2) * SPS) * IPS);
+      ring_barrier();
+      slots_of(pos_r, sa, sb);
+      load_frags(std::integral_constant<int, 0>{}, sa, sb, fm[0], fn[0]);
+      mfmas(std::integral_constant<int, (KG - 1) & 1>{});
+      pin_pairs();
+      refill(s + 1);   // into the slots of stage s, behind the MFMAs that keep the pipe busy right after the barrier
+    }
+    if (nk > 0) {
+      leading_groups();
+      mfmas(std::integral_constant<int, (KG - 1) & 1>{});
+      ring_barrier();   // every wavefront is done reading the ring: the epilogue stages the output tile there
     }
   } else {
     // Two register sets of a whole stage's fragments; phases alternate between them. Phase 0 only reads, the phase
@@ -363,25 +378,44 @@ __device__ __forceinline__ void gemm_ring_body(const GemmArgs& g, int block_x) {
 #pragma unroll
         for (int j = 0; j < TN; ++j) mfma<T>::run(fnS[P ^ 1][0][j], fmS[P ^ 1][0][i], acc[i][j]);
       certify_cur(p);
+      // the other k-groups of stage p - 1, with all of stage p's reads dealt out between them; the refill of the freed
+      // slots goes out behind the first of them, so that MFMAs follow the barrier at once
+      constexpr int NM = (KG - 1) * MFMAS, NR = KG * READS;
+      load_frags(std::integral_constant<int, 0>{}, sa, sb, fmS[P][0], fnS[P][0]);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) mfma<T>::run(fnS[P ^ 1][1][j], fmS[P ^ 1][1][i], acc[i][j]);
+      {
+        constexpr int PAIRS = READS < MFMAS ? READS : MFMAS;
+        static_for<0, PAIRS>([&](auto) {
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        });
+        if constexpr (READS > PAIRS) __builtin_amdgcn_sched_group_barrier(0x100, READS - PAIRS, 0);
+        if constexpr (MFMAS > PAIRS) __builtin_amdgcn_sched_group_barrier(0x008, MFMAS - PAIRS, 0);
+      }
       refill(p);
-      // the other k-groups of stage p - 1, with all of stage p's reads dealt out between them
-      static_for<0, KG>([&](auto kk_tag) {
+      static_for<1, KG>([&](auto kk_tag) {
         constexpr int kk = decltype(kk_tag)::value;
         load_frags(kk_tag, sa, sb, fmS[P][kk], fnS[P][kk]);
-        if constexpr (kk >= 1) {
+        if constexpr (kk >= 2) {
 #pragma unroll
           for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j) mfma<T>::run(fnS[P ^ 1][kk][j], fmS[P ^ 1][kk][i], acc[i][j]);
         }
       });
-      constexpr int NM = (KG - 1) * MFMAS, NR = KG * READS;
-      static_for<0, NM>([&](auto it) {
-        constexpr int i = decltype(it)::value;
-        constexpr int r = (i + 1) * NR / NM - i * NR / NM;
-        if constexpr (r > 0) __builtin_amdgcn_sched_group_barrier(0x100, r, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      });
+      {
+        constexpr int NM2 = (KG - 2) * MFMAS, NR2 = (KG - 1) * READS;
+        static_for<0, NM2>([&](auto it) {
+          constexpr int i = decltype(it)::value;
+          constexpr int r = (i + 1) * NR2 / NM2 - i * NR2 / NM2;
+          if constexpr (r > 0) __builtin_amdgcn_sched_group_barrier(0x100, r, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        });
+      }
+      (void)NM; (void)NR;
     };
     if (nk > 0) {
       {

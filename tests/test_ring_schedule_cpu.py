@@ -45,6 +45,15 @@ def simulate(ring, sa, sb, ips, nk):
     def barrier():
         visible.update(covered)
 
+    def read_stage(st, pos):
+        for j in range(sps):           # every operand slot of the stage is read by some wavefront
+            p = pos + j
+            if p >= ring:
+                p -= ring
+            q = st * sps + j
+            assert content[p] == q, (ring, sps, nk, st, j, p, content[p])          # property 3
+            assert q in visible, (ring, sps, nk, st, j)                             # property 1
+
     # prologue
     for t in range(ring):
         if t // sps < nk:
@@ -54,29 +63,25 @@ def simulate(ring, sa, sb, ips, nk):
     barrier()
     pos_r = pos_w = 0
     for s in range(nk):
-        if s >= 1:
-            for t in range(sps):
-                d = (ring + t) // sps
-                q = ring + (s - 1) * sps + t
-                assert q // sps == s - 1 + d and q % sps == (ring + t) % sps     # the kernel's compile-time (j, d)
-                if s - 1 + d < nk:
-                    issue(q, pos_w, reading_stage=s)
-                pos_w = 0 if pos_w + 1 == ring else pos_w + 1
-        for j in range(sps):           # every operand slot of stage s is read by some wavefront
-            p = pos_r + j
-            if p >= ring:
-                p -= ring
-            q = s * sps + j
-            assert content[p] == q, (ring, sps, nk, s, j, p, content[p])          # property 3
-            assert q in visible, (ring, sps, nk, s, j)                             # property 1
+        read_stage(s, pos_r)           # the first k-group's reads were issued behind the barrier of the step before
         pos_r += sps
         if pos_r >= ring:
             pos_r -= ring
         if s + 1 < nk:
+            # in front of the last k-group's MFMAs: wait for stage s + 1, barrier, first reads of stage s + 1, and the
+            # slots of stage s (all of its reads issued and landed before the barrier) are refilled
             n_issued = min(ring + s * sps, total)
             assert n_issued * ips == len(issued)
             wait((n_issued - (s + 2) * sps) * ips, (ring - 2 * sps) * ips)
-        barrier()
+            barrier()
+            read_stage(s + 1, pos_r)
+            for t in range(sps):
+                d = (ring + t) // sps
+                q = ring + s * sps + t
+                assert q // sps == s + d and q % sps == (ring + t) % sps     # the kernel's compile-time (j, d)
+                if s + d < nk:
+                    issue(q, pos_w, reading_stage=s + 1)
+                pos_w = 0 if pos_w + 1 == ring else pos_w + 1
     return len(issued)
 
 
