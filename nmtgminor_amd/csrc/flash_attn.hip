@@ -851,9 +851,8 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dkv_ker
     // s[n][r]: query 32 n + 8 (r / 4) + 4 half + r % 4 of the tile, key krow. P (dropped, scaled) stays in dp's place
     // for dV, dS goes to s for dK.
     // time mask: bit 16 n + r of tdead = the mask hides query (n, r) of the tile from this lane's key; the 32 bytes are
-    // requested together, ahead of the masking. (Here and in the other two kernels a form with each byte load inside
-    // the masking condition of its element passed on the CPU and gave wrong gradients on the GPU in some of the
-    // head-dimension-64 variants; with the loads gathered first every variant agrees bit for bit with the causal flag.)
+    // requested together, ahead of the masking, so that one wait covers them all (a byte load inside each element's
+    // masking condition compiles to 32 load-wait-branch rounds in a row).
     bool tmt = false;
     if constexpr (TM != 0) tmt = a.kqinfo[static_cast<int64_t>(kgroup) * a.kqinfo_pitch + 2 + t] != 0;
     uint32_t tdead = 0;

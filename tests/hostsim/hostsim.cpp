@@ -9,8 +9,15 @@
 //   late  (default)  a transfer lands only when its lane executes the vmcnt wait that covers it: a missing or too
 //                    weak wait leaves stale (poisoned) LDS behind the reads that needed it;
 //   early            a transfer lands the moment it is issued: a slot that is refilled before every wavefront has
-//                    finished reading it corrupts those reads (the scheduler runs wavefront 0 as far as it can go,
-//                    then wavefront 1, ..., so later wavefronts are the slow readers).
+//                    finished reading it corrupts those reads.
+// Between two block barriers the wavefronts of a block run in an order HOSTSIM_ORDER picks; a kernel whose wavefronts
+// exchange data through LDS or global memory without a barrier gives different results under different orders:
+//   forward (default)   wavefront 0 as far as it can go, then wavefront 1, ... (later wavefronts are the slow ones)
+//   reverse             the last wavefront first
+//   random              a new random order after every barrier (HOSTSIM_SEED)
+//   interleave          the wavefronts advance side by side, one wavefront-wide operation (MFMA, shuffle, LDS transpose
+//                       read) at a time
+//   interleave_random   the same, in a new random order every turn
 // Dynamic LDS is filled with 0xFF bytes (NaN in every float format used) at the start of every block.
 // Test infrastructure only.
 #include <hip/hip_runtime.h>
@@ -86,6 +93,15 @@ struct Fiber {
 
 bool dma_early = false;
 size_t lds_in_use = 0;
+enum WaveOrder { ORDER_FORWARD, ORDER_REVERSE, ORDER_RANDOM, ORDER_INTERLEAVE, ORDER_INTERLEAVE_RANDOM };
+WaveOrder wave_order = ORDER_FORWARD;
+uint64_t random_state = 1;
+uint32_t next_random() {   // xorshift64*
+  random_state ^= random_state >> 12;
+  random_state ^= random_state << 25;
+  random_state ^= random_state >> 27;
+  return static_cast<uint32_t>((random_state * 0x2545F4914F6CDD1DULL) >> 33);
+}
 
 Fiber fibers[MAX_THREADS];
 unsigned char* stacks = nullptr;
@@ -151,25 +167,47 @@ void run_block(int nthreads) {
   }
   std::memset(dynamic_lds, 0xff, lds_in_use);
   const int waves = (nthreads + WAVE - 1) / WAVE;
-  for (;;) {
-    for (int w = 0; w < waves; ++w) {
-      const int lo = w * WAVE, hi = std::min(nthreads, lo + WAVE);
-      for (;;) {
-        for (int t = lo; t < hi; ++t)
-          if (fibers[t].state == RUNNABLE) resume(t);
-        int arrived = 0;
-        for (int t = lo; t < hi; ++t) arrived += fibers[t].state == AT_COLLECTIVE;
-        if (arrived == 0) break;                // wavefront finished or waits at the block barrier
-        current = lo;
-        if (arrived != hi - lo) die("wavefront-wide operation reached by only some of the lanes");
-        void* payloads[WAVE];
-        for (int t = lo; t < hi; ++t) {
-          if (fibers[t].resolver != fibers[lo].resolver) die("lanes of one wavefront are at different wavefront-wide operations");
-          payloads[t - lo] = fibers[t].payload;
-        }
-        fibers[lo].resolver(payloads, hi - lo);
-        for (int t = lo; t < hi; ++t) fibers[t].state = RUNNABLE;
+  // Runs wavefront w until it has no runnable lane and no pending wavefront-wide operation (it is done or waits at
+  // the block barrier), or, with `one_step`, until it has resolved one wavefront-wide operation. Returns whether it
+  // made progress.
+  auto run_wave = [&](int w, bool one_step) -> bool {
+    const int lo = w * WAVE, hi = std::min(nthreads, lo + WAVE);
+    bool progressed = false;
+    for (;;) {
+      for (int t = lo; t < hi; ++t)
+        if (fibers[t].state == RUNNABLE) { resume(t); progressed = true; }
+      int arrived = 0;
+      for (int t = lo; t < hi; ++t) arrived += fibers[t].state == AT_COLLECTIVE;
+      if (arrived == 0) return progressed;      // wavefront finished or waits at the block barrier
+      current = lo;
+      if (arrived != hi - lo) die("wavefront-wide operation reached by only some of the lanes");
+      void* payloads[WAVE];
+      for (int t = lo; t < hi; ++t) {
+        if (fibers[t].resolver != fibers[lo].resolver) die("lanes of one wavefront are at different wavefront-wide operations");
+        payloads[t - lo] = fibers[t].payload;
       }
+      fibers[lo].resolver(payloads, hi - lo);
+      for (int t = lo; t < hi; ++t) fibers[t].state = RUNNABLE;
+      progressed = true;
+      if (one_step) return true;
+    }
+  };
+  int order[MAX_THREADS / WAVE];
+  for (;;) {
+    // the order in which the wavefronts run between two block barriers (see the header comment)
+    for (int w = 0; w < waves; ++w) order[w] = wave_order == ORDER_REVERSE ? waves - 1 - w : w;
+    if (wave_order == ORDER_RANDOM || wave_order == ORDER_INTERLEAVE_RANDOM)
+      for (int w = waves - 1; w > 0; --w) std::swap(order[w], order[next_random() % (w + 1)]);
+    if (wave_order == ORDER_INTERLEAVE || wave_order == ORDER_INTERLEAVE_RANDOM) {
+      // one wavefront-wide operation per wavefront and turn: the wavefronts advance side by side
+      for (bool any = true; any;) {
+        any = false;
+        for (int i = 0; i < waves; ++i) any |= run_wave(order[i], true);
+        if (wave_order == ORDER_INTERLEAVE_RANDOM)
+          for (int w = waves - 1; w > 0; --w) std::swap(order[w], order[next_random() % (w + 1)]);
+      }
+    } else {
+      for (int i = 0; i < waves; ++i) run_wave(order[i], false);
     }
     int done = 0, waiting = 0;
     for (int t = 0; t < nthreads; ++t) {
@@ -343,6 +381,13 @@ void launch(dim3 grid, dim3 block, size_t dynamic_lds_bytes, const std::function
   }
   const char* mode = std::getenv("HOSTSIM_DMA");
   dma_early = mode != nullptr && std::strcmp(mode, "early") == 0;
+  const char* ord = std::getenv("HOSTSIM_ORDER");
+  wave_order = ord == nullptr ? ORDER_FORWARD
+               : std::strcmp(ord, "reverse") == 0 ? ORDER_REVERSE
+               : std::strcmp(ord, "random") == 0 ? ORDER_RANDOM
+               : std::strcmp(ord, "interleave") == 0 ? ORDER_INTERLEAVE
+               : std::strcmp(ord, "interleave_random") == 0 ? ORDER_INTERLEAVE_RANDOM : ORDER_FORWARD;
+  if (const char* seed = std::getenv("HOSTSIM_SEED")) random_state = std::strtoull(seed, nullptr, 10) * 2654435761ULL + 1;
   lds_in_use = dynamic_lds_bytes;
   kernel_body = &body;
   cur_block_dim = block;

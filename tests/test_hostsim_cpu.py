@@ -435,6 +435,18 @@ def test_training_attention_with_time_masks_without_coverage(mi355x, dtype):
     tnc.test_a_causal_time_mask_equals_the_causal_flag_bit_for_bit(CPU, 64, 0.2)
 
 
+@pytest.mark.parametrize("order", ["reverse", "interleave_random"])
+def test_tiled_kernels_do_not_depend_on_the_order_of_their_wavefronts(mi355x, monkeypatch, order):
+    """Between two block barriers the wavefronts of a block may run in any order and interleaving: the tiled attention
+    kernels with a time mask (bit for bit against the causal flag) and the ring GEMM give the same results when the
+    CPU build runs them last-to-first, or one wavefront-wide operation at a time in a random order."""
+    monkeypatch.setenv("HOSTSIM_ORDER", order)
+    monkeypatch.setenv("HOSTSIM_SEED", "11")
+    tnc.test_a_causal_time_mask_equals_the_causal_flag_bit_for_bit(CPU, 64, 0.2)
+    tnc.test_self_attention_training_with_time_masks_of_other_shapes(CPU, BF16)
+    tg.test_gemm_layouts(CPU, F16, 300, 520, 448, "nn")
+
+
 @pytest.mark.parametrize("dtype", HALVES)
 @pytest.mark.parametrize("ignore_source", [False, pytest.param(True, marks=long_case)])
 def test_decoder_layer(mi355x, dtype, ignore_source):
