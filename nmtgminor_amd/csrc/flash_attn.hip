@@ -535,9 +535,11 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
         s[n][r] = pr;
         lsum += pr;
       }
-    if constexpr (PAD != 0) if (padt) {
+    if constexpr (PAD != 0) if (edge) {
       // A row that has met no live key yet still has the initial m, against which a dead score is not small: such
-      // probabilities are set to 0 by hand. (Without masked keys inside the sequence, key 0 is live for every row.)
+      // probabilities are set to 0 by hand, in every tile that holds a dead key of any kind (a row whose keys up to the
+      // causal diagonal are all masked meets the diagonal's dead keys in tiles without a masked key). Without a mask,
+      // key 0 is live for every row.
       lsum = 0.f;
 #pragma unroll
       for (int n = 0; n < 2; ++n)

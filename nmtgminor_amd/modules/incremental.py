@@ -4,7 +4,8 @@ What the reference does in the `incremental` branches of its attention functions
 (onmt/modules/optimized/self_attention_func.py:162-174, encdec_attention_func_bias.py:181-213), with the same
 cache entries so that the reference's beam search can reorder them (every entry is time-first [T, B, E] and is
 re-indexed along dimension 1):
-    self-attention     cache['k'], cache['v']      keys / values of all positions decoded so far (grow by one row)
+    self-attention     cache['k'], cache['v']      keys / values of all positions decoded so far (grow by one row,
+                                                   inside a buffer with room to grow: see _append)
     cross-attention    cache['c_k'], cache['c_v']  keys / values of the encoder states (computed at the first step)
 Inference only (no autograd graph, no dropout). The projections are GEMM calls of the library, the attention core is
 the compact cross-attention entry point (queries and a [Tk, B*H, 2, D] key/value block come in, the context goes
@@ -76,14 +77,36 @@ def _key_mask(mask, use_time_mask, b, tk, device):
     if use_time_mask:
         if mask.dim() == 1:
             mask = mask.unsqueeze(0)
-        if mask.dim() != 2 or mask.size(-1) != tk:
-            raise RuntimeError(f"incremental self-attention: time mask of shape {tuple(mask.shape)} does not cover {tk} keys")
+        if mask.dim() != 2 or mask.size(-1) != tk or mask.size(0) not in (1, tk):
+            raise RuntimeError(f"incremental self-attention: time mask of shape {tuple(mask.shape)}, expected [1, {tk}] (the new "
+                               f"position's row) or [{tk}, {tk}] (whose last row it is)")
         return mask[-1:].expand(b, tk).contiguous()
     if mask.dim() == 3:
         mask = mask.squeeze(1)
     if mask.shape != (b, tk):
         raise RuntimeError(f"incremental self-attention: key-padding mask of shape {tuple(mask.shape)}, expected {(b, tk)}")
     return mask.contiguous()
+
+
+def _append(cache, name, row):
+    """cache[name] [T, B, E] with `row` [1, B, E] behind it. The reference concatenates (a copy of the whole cache per
+    step, self_attention_func.py:165-169). Here the rows live in a buffer with room to grow and cache[name] is its
+    leading slice, which carries the buffer as an attribute (the dict keeps exactly the reference's entries): while the
+    caller leaves that tensor in place, a step writes one row. A caller that replaces cache[name] (beam search re-indexes
+    every entry along dimension 1, which yields new tensors) gets a fresh buffer filled from it: the reference's copy,
+    with room for the steps that follow."""
+    old = cache[name]
+    n = old.shape[0]
+    buf = getattr(old, "_nmtg_buffer", None)
+    in_place = (buf is not None and buf.shape[0] > n and buf.shape[1:] == old.shape[1:] and buf.dtype == old.dtype
+                and buf.device == old.device and old.is_contiguous() and old.data_ptr() == buf.data_ptr())
+    if not in_place:
+        buf = old.new_empty((max(2 * n, n + 64),) + tuple(old.shape[1:]))
+        buf[:n].copy_(old)
+    buf[n:n + 1].copy_(row)
+    grown = buf[:n + 1]
+    grown._nmtg_buffer = buf
+    return grown
 
 
 @torch.no_grad()
@@ -102,8 +125,8 @@ def self_attn_step(heads, inputs, input_weights, output_weights, input_biases, o
     if not first:
         if t_new != 1:
             raise NotImplementedError("incremental self-attention: one new position per step once the cache is filled")
-        keys = torch.cat([cache["k"], keys], dim=0)
-        values = torch.cat([cache["v"], values], dim=0)
+        keys = _append(cache, "k", keys)
+        values = _append(cache, "v", values)
     cache["k"], cache["v"] = keys, values
     if first and t_new > 1:
         # a prefix of several positions: the full-sequence kernel with its mask, fed with the same projection

@@ -2,7 +2,8 @@
 
 Mirrors onmt/modules/layer_norm.py:37-168 (FastLayerNormFN, fast_layer_norm_affine,
 layer_norm_func, LayerNorm) and the in-sync variant with `memory_efficient`
-(whisper/memory_efficient_whisper.py:73-140). The reference only routes hidden sizes
+(whisper/memory_efficient_whisper.py:73-140), and MultilingualLayerNorm (:175-227: one affine pair per language, the
+pair of the call picked by `factor`). The reference only routes hidden sizes
 768/1024/2048/3072/4096 to its native kernels; here every hidden size takes the native path.
 """
 import numbers
@@ -104,3 +105,45 @@ class LayerNorm(torch.nn.Module):
 
     def extra_repr(self):
         return "{normalized_shape}, eps={eps}, elementwise_affine={elementwise_affine}".format(**self.__dict__)
+
+
+class MultilingualLayerNorm(torch.nn.Module):
+    """One (weight, bias) pair per language, [n_languages, hidden] each; `forward(input, factor)` normalises with the pair
+    that `factor` (an index tensor with one element) selects (onmt/modules/layer_norm.py:175-227). The selection is an
+    index_select, so the gradient lands in the selected rows and the others get zeros, as in the reference."""
+
+    def __init__(self, normalized_shape, eps=1e-5, elementwise_affine=True, n_languages=1):
+        super().__init__()
+        if isinstance(normalized_shape, numbers.Integral):
+            normalized_shape = (normalized_shape,)
+        if len(normalized_shape) != 1:
+            raise ValueError("MultilingualLayerNorm normalises over the last dimension only")
+        self.n_languages = n_languages
+        self.normalized_shape = torch.Size(normalized_shape)
+        self.eps = eps
+        self.elementwise_affine = elementwise_affine
+        if elementwise_affine:
+            self.weight = Parameter(torch.empty(n_languages, *normalized_shape))
+            self.bias = Parameter(torch.empty(n_languages, *normalized_shape))
+        else:
+            self.register_parameter("weight", None)
+            self.register_parameter("bias", None)
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        if self.elementwise_affine:
+            init.ones_(self.weight)
+            init.zeros_(self.bias)
+
+    def forward(self, input, factor):
+        weight = bias = None
+        if self.elementwise_affine:
+            if factor is None or factor.numel() != 1:
+                raise RuntimeError("MultilingualLayerNorm: `factor` must be an index tensor with one element (the language)")
+            weight = torch.index_select(self.weight, 0, factor.view(1)).squeeze(0)
+            bias = torch.index_select(self.bias, 0, factor.view(1)).squeeze(0)
+        weight, bias = _affine_or_identity(input, weight, bias, self.normalized_shape[0])
+        return fast_layer_norm_affine(input, weight, bias, self.normalized_shape, self.eps)
+
+    def extra_repr(self):
+        return "{normalized_shape}, eps={eps}, elementwise_affine={elementwise_affine}, n_languages={n_languages}".format(**self.__dict__)

@@ -6,13 +6,14 @@ Constructor arguments, attribute names and state_dict keys (`layer_norm.function
 reference's. On the HIP path "n" is the LayerNorm kernel and an adjacent "d", "a" pair with plain (element-wise)
 dropout is the fused dropout + residual-add kernel, in place on the sub-layer's output; the variational dropout
 (one mask per sequence position-independent [1, B, H] slice) keeps the reference's tensor expression.
-Multilingual LayerNorm has no kernel here and raises.
+With multilingual=True "n" is the MultilingualLayerNorm (one affine pair per language; `forward(..., factor=)` picks it; state_dict
+keys `layer_norm.weight`, `.bias` as in the reference, which does not wrap that module in Bottle).
 """
 import torch
 from torch import nn
 
 from .dropout_add import fused_dropout_add
-from .layer_norm import LayerNorm
+from .layer_norm import LayerNorm, MultilingualLayerNorm
 
 
 class Bottle(nn.Module):
@@ -47,15 +48,16 @@ class PrePostProcessing(nn.Module):
     def __init__(self, d_model, dropout_p, sequence="nda", variational=False, elementwise_affine=True,
                  multilingual=False, n_languages=1):
         super().__init__()
-        if multilingual:
-            raise NotImplementedError("PrePostProcessing: the multilingual LayerNorm has no HIP kernel")
         self.d_model = d_model
         self.dropout_p = dropout_p
         self.multilingual = multilingual
         self.variational = variational
         self.steps = list(sequence)
         if "n" in self.steps:
-            self.layer_norm = Bottle(LayerNorm((d_model,), elementwise_affine=elementwise_affine))
+            if multilingual:      # one affine pair per language, picked by forward's `factor` (pre_post_processing.py:40-42)
+                self.layer_norm = MultilingualLayerNorm((d_model,), eps=1e-5, elementwise_affine=True, n_languages=n_languages)
+            else:
+                self.layer_norm = Bottle(LayerNorm((d_model,), elementwise_affine=elementwise_affine))
         if "d" in self.steps:
             self.dropout = VariationalDropout(dropout_p, batch_first=False) if variational \
                 else nn.Dropout(dropout_p, inplace=False)
@@ -81,7 +83,7 @@ class PrePostProcessing(nn.Module):
         while i < len(self.steps):
             step = self.steps[i]
             if step == "n":
-                output = self.layer_norm(output)
+                output = self.layer_norm(output, factor) if self.multilingual else self.layer_norm(output)
             elif step == "d":
                 if self._fusable(i, output, input_tensor):
                     # dropout and the residual add in one pass over the tensor

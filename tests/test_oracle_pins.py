@@ -337,6 +337,53 @@ def test_encdec_attention_matches_library_and_autograd():
     torch.testing.assert_close(fwd0["outputs"], ref.detach(), rtol=1e-10, atol=1e-11)
 
 
+@pytest.mark.parametrize("causal,p", [(False, 0.0), (False, 0.25), (True, 0.25)])
+def test_tiled_core_restatement_matches_autograd_when_nothing_is_rounded(causal, p):
+    """core="tiled" regroups the same mathematics (unnormalised exponentials times V, divided by the row sum afterwards;
+    dS from D = rowsum(dctx * ctx)): with round_to=None it has to equal autograd through the library's ops, for self- and
+    encoder-decoder attention, with a fully masked row among the cases (encoder-decoder inputs mask whole tails)."""
+    t, b, e, h = 9, 3, 12, 3
+    d = inputs.self_attn_inputs(t, b, e, h, torch.float64, p=p, seed=13, min_len=4, causal=causal, zero_bias=False)
+    fwd = attention.self_attn_fwd(d["x"], d["w_in"], d["w_out"], d["b_in"], d["b_out"], h, d["pad_mask"], d["time_mask"],
+                                  p, d["dropout_mask"], D, core="tiled")
+    bwd = attention.self_attn_bwd(d["dout"], d["x"], d["w_in"], d["w_out"], h, fwd, p, d["dropout_mask"], D, core="tiled")
+    out, dx, (dwi, dwo, dbi, dbo) = _self_attn_autograd(d, h, d["pad_mask"], d["time_mask"], p, d["dropout_mask"])
+    torch.testing.assert_close(fwd["outputs"], out, rtol=1e-10, atol=1e-11)
+    for name, got, want in (("dx", bwd["dx"], dx), ("dw_in", bwd["dw_in"], dwi), ("dw_out", bwd["dw_out"], dwo),
+                            ("db_in", bwd["db_in"], dbi), ("db_out", bwd["db_out"], dbo)):
+        torch.testing.assert_close(got, want, rtol=1e-8, atol=1e-10, msg=lambda m, n=name: f"{n}: {m}")
+    tq, tk = 5, 11
+    d = inputs.encdec_attn_inputs(tq, tk, b, e, h, torch.float64, p=p, seed=14, zero_bias=False)
+    args = (d["x_q"], d["x_kv"], d["w_q"], d["w_kv"], d["w_out"])
+    res = {}
+    for core in ("stored", "tiled"):
+        f = attention.encdec_attn_fwd(*args, d["b_q"], d["b_kv"], d["b_out"], h, d["pad_mask"], p, d["dropout_mask"], D, core=core)
+        res[core] = (f, attention.encdec_attn_bwd(d["dout"], *args, h, f, p, d["dropout_mask"], D, core=core))
+    torch.testing.assert_close(res["tiled"][0]["outputs"], res["stored"][0]["outputs"], rtol=1e-10, atol=1e-11)
+    for key, want in res["stored"][1].items():
+        torch.testing.assert_close(res["tiled"][1][key], want, rtol=1e-8, atol=1e-10, msg=lambda m, n=key: f"{n}: {m}")
+
+
+def test_tiled_core_restatement_rounds_only_operands_and_results():
+    """With round_to=bf16 the two restatements differ by roundings only: the tiled one keeps scores and statistics exact,
+    so its context is the closer of the two to the unrounded one, and a single key (probability exactly 1, dropout scale
+    1 / (1 - p) applied in full precision at the end) gives round(v / (1 - p)) rather than round(round(1 / (1 - p)) v)."""
+    t, b, e, h, p = 40, 2, 64, 2, 0.25
+    d = inputs.self_attn_inputs(t, b, e, h, torch.bfloat16, p=p, seed=21, zero_bias=False)
+    kw = dict(pad_mask=d["pad_mask"], p=p, dropout_mask=d["dropout_mask"], ctype=D)
+    a = (d["x"], d["w_in"], d["w_out"], d["b_in"], d["b_out"], h)
+    exact = attention.self_attn_fwd(*a, **kw)["matmul2_results"]
+    err = {c: (attention.self_attn_fwd(*a, **kw, round_to=torch.bfloat16, core=c)["matmul2_results"] - exact).abs().mean()
+           for c in ("stored", "tiled")}
+    assert err["tiled"] < err["stored"]
+    q = torch.randn(1, 1, 8, dtype=D)
+    v = torch.randn(1, 1, 8, dtype=D).to(torch.bfloat16).to(D)
+    keep = torch.ones(1, 1, 1, dtype=torch.bool)
+    _, prob, _, ctx = attention._core_fwd_tiled(q, q, v, 1, None, None, p, keep, D, torch.bfloat16)
+    assert prob.item() == 1.0
+    assert torch.equal(ctx, (v / (1 - p)).to(torch.bfloat16).to(D))
+
+
 def test_attention_finite_differences():
     # the reference validates its hand-written backward with fp64 gradcheck on tiny shapes
     t, b, e, h = 4, 2, 8, 2
@@ -587,6 +634,30 @@ def test_layer_oracle_matches_torch_modules():
     torch.testing.assert_close(got, half(half(x)), rtol=1e-10, atol=1e-12)
 
 
+def test_layer_oracle_with_the_tiled_core_differentiates_to_the_same_gradients():
+    """attn_core="tiled" routes the self-attention through an autograd node whose backward is written out (the kernels'
+    formulation); nothing rounded, a whole layer's gradients have to equal those of plain autograd."""
+    t, b, e, h, inner = 9, 3, 16, 4, 40
+    g = torch.Generator().manual_seed(73)
+    torch.manual_seed(74)
+    dec = torch.nn.TransformerDecoderLayer(e, h, inner, dropout=0.0, activation="gelu", norm_first=True, dtype=D)
+    params = _layer_params_from_torch(dec, h, True)
+    x0 = torch.randn(t, b, e, generator=g, dtype=D)
+    c0 = torch.randn(11, b, e, generator=g, dtype=D)
+    dy = torch.randn(t, b, e, generator=g, dtype=D)
+    causal = torch.triu(torch.ones(t, t), 1).bool()
+    src_pad, _ = inputs.lengths_mask(b, 11, 5, 11, g)
+    grads = {}
+    for core in ("stored", "tiled"):
+        x, c = x0.clone().requires_grad_(), c0.clone().requires_grad_()
+        prm = {k: v.detach().clone().requires_grad_() for k, v in params.items()}
+        y, _ = transformer_layers.decoder_layer(x, c, prm, h, causal, src_pad, act="gelu", attn_core=core)
+        y.backward(dy)
+        grads[core] = [y.detach(), x.grad, c.grad] + [prm[k].grad for k in sorted(prm)]
+    for a, bb in zip(grads["stored"], grads["tiled"]):
+        torch.testing.assert_close(a, bb, rtol=1e-9, atol=1e-11)
+
+
 def test_zipf_targets_and_masks_are_seeded():
     a = inputs.xentropy_inputs(2000, 1000, with_logits=False, seed=1)
     b = inputs.xentropy_inputs(2000, 1000, with_logits=False, seed=1)
@@ -700,6 +771,50 @@ def test_packed_attention_is_library_attention_on_every_sequence_by_itself(causa
         # D = rowsum(dO * O) = rowsum(P * dP): the identity the backward kernels rest on
         dp = torch.einsum("hid,hjd->hij", do[sq].transpose(0, 1), vb.detach())
         assert torch.allclose(delta[b, :, :lq[b]], (torch.softmax(s, -1) * dp).sum(-1), atol=1e-12)
+
+
+@pytest.mark.parametrize("causal,p", [(False, 0.0), (True, 0.25)])
+def test_packed_attention_written_out_backward_equals_autograd(causal, p):
+    """The backward as the kernels compute it (dS = P (keep dP / (1 - p) - D) with D = rowsum(dO O)) against autograd of
+    the forward, nothing rounded; an empty sequence and unequal lengths among the cases."""
+    from oracle import flash_attention as ofa
+    lq, lk = ([3, 6, 4], [5, 0, 7]) if not causal else ([3, 6, 4], [3, 6, 4])
+    q, k, v, do, cu_q, cu_k = _packed_case(503, lq, lk)
+    keep = (torch.rand(3, 2, max(lq), max(lk), generator=torch.Generator().manual_seed(8)) < 0.75).to(torch.uint8)
+    a = ofa.flash_attn_bwd(do, q, k, v, cu_q, cu_k, max(lq), 0.3, causal, p, keep, explicit=False)
+    b = ofa.flash_attn_bwd(do, q, k, v, cu_q, cu_k, max(lq), 0.3, causal, p, keep, explicit=True)
+    for x, y in zip(a, b):
+        assert torch.allclose(x, y, atol=1e-12)
+
+
+def test_tiled_operand_is_the_softmax_numerator_under_a_moving_reference_point():
+    """Unrounded, operand / l is the softmax whatever the reference points were (rows whose maximum sits in a late tile
+    and exceeds the first tile's by more than 2^8, rows that start with masked tiles, a row without a live key); rounded,
+    every entry is a 16-bit value times the reference shift, i.e. the rounding was applied to exp2(s2 - m_tile): dividing
+    the shift back out leaves exactly representable numbers."""
+    g = torch.Generator().manual_seed(9)
+    s = torch.randn(2, 5, 200, generator=g, dtype=D)
+    s[0, 0, 150] += 12.0                    # a late maximum beyond the lazy threshold: the reference point moves at tile 2
+    s[0, 1, 70] += 3.0                      # a late maximum below it: the reference point stays
+    s[1, 2, :130] = -math.inf               # the first two tiles masked: the reference point is set in the third
+    s[1, 3, :] = -math.inf                  # no live key at all
+    keep = torch.ones_like(s)
+    op, l = attention.tiled_operand(s, keep, None)
+    want = torch.softmax(s, -1)
+    want[1, 3] = 0
+    got = torch.where(l > 0, op / l, torch.zeros_like(op))
+    assert torch.allclose(got, want, atol=1e-14)
+    assert l[1, 3].item() == 0 and bool((op[1, 3] == 0).all())
+    opr, lr = attention.tiled_operand(s, keep, torch.bfloat16)
+    assert torch.equal(lr, l)                                                  # the row sum is formed before the rounding
+    rel = ((opr - op).abs() / op.clamp_min(1e-300))[op > 0]
+    assert rel.max() <= 2.0 ** -8 + 1e-12 and rel.mean() > 2.0 ** -12           # half a unit of an 8-bit significand at most, and really rounded
+    # row (0, 0): keys of tiles 0 and 1 were rounded against the first tile's maximum, then rescaled by 2^(m0 - m2)
+    s2 = s[0, 0] * 1.4426950408889634
+    m0, m2 = s2[:64].max(), s2[128:192].max()
+    first = opr[0, 0, :128] * torch.exp2(m2 - m0)
+    assert torch.allclose(first, first.to(torch.bfloat16).to(D), rtol=1e-12, atol=0)
+    assert torch.allclose(opr[0, 0, 128:], opr[0, 0, 128:].to(torch.bfloat16).to(D), rtol=1e-12, atol=0)
 
 
 def test_packed_attention_with_unequal_lengths_dropout_and_an_empty_sequence_by_loops():

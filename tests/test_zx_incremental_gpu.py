@@ -57,12 +57,15 @@ def test_self_attention_step_by_step(dev, dtype, prefix):
         out, cov = attn(x[:prefix], None, None, causal[:prefix, :prefix], incremental=True, incremental_cache=cache)
         rows.append(out)
         assert cov.shape == (b * h, prefix, prefix)
+        homes = set()
         for i in range(prefix, t):
             out, cov = attn(x[i:i + 1], None, None, causal[i:i + 1, :i + 1], incremental=True, incremental_cache=cache)
             rows.append(out)
             assert cache["k"].shape == (i + 1, b, e) and cache["v"].shape == (i + 1, b, e)
+            homes.add((cache["k"].data_ptr(), cache["v"].data_ptr()))
             assert cov.shape == (b * h, 1, i + 1)
             assert_close(cov.float().sum(-1), torch.ones(b * h, 1), dtype, "probabilities sum to one", atol=2e-2)
+        assert len(homes) == 1                 # the cache grows inside one buffer: a step writes a row, it copies nothing
     w_in, w_out, b_in, b_out = _cpu(attn, "in_proj_weight", "out_proj_weight", "in_proj_bias", "out_proj_bias")
     want = oat.self_attn_fwd(x.cpu(), w_in, w_out, b_in, b_out, h, None, causal.cpu(), 0.0, None, D, round_to=dtype)
     assert_close(torch.cat(rows), want["outputs"], dtype, "stepwise self-attention vs oracle")
@@ -72,6 +75,11 @@ def test_self_attention_step_by_step(dev, dtype, prefix):
         attn(x[:2], None, None, None, incremental=True, incremental_cache=cache)       # two positions onto a filled cache
     with pytest.raises(RuntimeError):
         attn(x[:1], None, None, None, incremental=True, incremental_cache=None)
+    # a time mask for a step is the new position's row, or the square mask whose last row that is: other row counts are
+    # refused (filled caches are copied: the refused call must not have grown them)
+    keys = cache["k"].shape[0]
+    with pytest.raises(RuntimeError, match="time mask"):
+        attn(x[:1], None, None, causal[:3, :keys + 1], incremental=True, incremental_cache=dict(cache))
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
@@ -96,6 +104,31 @@ def test_self_attention_steps_honour_a_key_padding_mask(dev, dtype):
             # exact zeros on the padded keys
             for bi in range(b):
                 assert (cov[bi * h:(bi + 1) * h, :, :pads[bi]] == 0).all()
+
+
+def test_one_position_against_the_longest_cache_at_head_dimension_128(dev):
+    """16384 cached keys of head dimension 128: the score row plus the partial contexts take more than 64 KB of LDS, the
+    launch that has to ask for the larger allocation. One query position, a key mask on the second sequence; probabilities
+    and context against the softmax of the same row in fp64 (scores rounded to the tensors' type, as the kernel stores them)."""
+    from nmtgminor_amd.modules import incremental
+    tk, b, h, d, dtype = 16384, 2, 2, 128, torch.bfloat16
+    e = h * d
+    g = torch.Generator().manual_seed(97)
+    q = torch.randn(1, b, e, generator=g).to(dtype)
+    keys = torch.randn(tk, b, e, generator=g).to(dtype)
+    values = torch.randn(tk, b, e, generator=g).to(dtype)
+    pad = torch.zeros(b, tk, dtype=torch.bool)
+    pad[1, 16000:] = True
+    pad[1, 5] = True
+    assert incremental._decode_ok(q.to(dev), keys.to(dev), values.to(dev), h)
+    ctx, probs = incremental._decode_core(h, q.to(dev), keys.to(dev), values.to(dev), pad.to(dev))
+    q4, k4, v4 = q.view(b, h, d).to(D), keys.view(tk, b, h, d).to(D), values.view(tk, b, h, d).to(D)
+    s = (torch.einsum("bhd,tbhd->bht", q4, k4) * d ** -0.5).to(dtype).to(D)
+    s = s.masked_fill(pad.view(b, 1, tk), float("-inf"))
+    pr = torch.softmax(s, -1)
+    assert_close(probs.view(b, h, tk), pr, dtype, "probabilities", atol=1e-5)
+    assert (probs.view(b, h, tk).cpu()[1, :, 16000:] == 0).all() and (probs.view(b, h, tk).cpu()[1, :, 5] == 0).all()
+    assert_close(ctx.view(b, h, d), torch.einsum("bht,tbhd->bhd", pr.to(dtype).to(D), v4), dtype, "context")
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])

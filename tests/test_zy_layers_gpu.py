@@ -39,10 +39,26 @@ def randomise(module, seed):
     return module
 
 
-def layer_close(actual, expected, dtype, what):
-    # a whole layer rounds to `dtype` at every operator boundary, the oracle nowhere
-    tol = {torch.bfloat16: 2.5e-2, torch.float16: 4e-3}[dtype]
-    assert_close(actual, expected, dtype, what, rtol=3e-2, atol=tol * max(1.0, float(expected.detach().abs().max())))
+def layer_close(actual, expected, dtype, what, summed=False):
+    """The oracle rounds to `dtype` where the layer does (every operator boundary, the operators' stored tensors, the
+    stored gradients), so nearly every element meets the comparison every 16-bit result gets: 2e-2 relative, 1e-3 of the
+    largest magnitude absolute. What remains are last-place flips: where the fp32-accumulating kernel and the fp64 oracle
+    land on opposite sides of a rounding boundary of an intermediate of magnitude M, a residual sum that cancels to a
+    small value inherits one unit in the last place of M. Such elements are few (under 1 %) and bounded by one unit in
+    the last place of the largest magnitude (eps * max); a wrong term or a missing rounding point shows as many elements,
+    or as a larger error. summed: a parameter gradient, a sum over all tokens of such elements, so that a flip in any one
+    of its hundred-odd terms shows in it: the bound alone."""
+    a, e = actual.detach().to("cpu", D), expected.detach().to("cpu", D)
+    peak = max(1.0, float(e.abs().max()))
+    outside = ((a - e).abs() > 1e-3 * peak + 2e-2 * e.abs()).double().mean().item()
+    assert summed or outside < 0.01, f"{what}: {100 * outside:.2f} % of the elements beyond the 16-bit tolerance"
+    assert_close(actual, expected, dtype, what, atol=torch.finfo(dtype).eps * peak)
+
+
+def attn_core(opt, training):
+    """Which attention kernels the layer's self-attention runs, hence which rounding points the oracle models: the tiled
+    core in training where it takes the head dimension, the extension's stored-tensor chain otherwise."""
+    return "tiled" if training and opt.model_size // opt.n_heads in (64, 128) else "stored"
 
 
 def params64(module):
@@ -81,15 +97,32 @@ def test_pre_post_processing_sequences(dev, dtype):
     if dtype == torch.float32:
         assert_close(got, want + r.to(D).view(t * b, e), dtype, "nda")
     else:
-        layer_close(got, want + r.to(D).view(t * b, e), dtype, "nda")      # rounded after "n" and again after "a"
+        layer_close(got, want.to(dtype).to(D) + r.to(D).view(t * b, e), dtype, "nda")      # "n" stores its result in `dtype`
     z = PrePostProcessing(e, 0.0, sequence="z").to(dev)
     assert_close(z(x.to(dev), r.to(dev)), r.to(D), dtype, "z")
     # variational dropout: one mask per (batch, feature), shared over time
     v = PrePostProcessing(e, 0.5, sequence="d", variational=True).to(dev).train()
     y = v(torch.ones(t, b, e, device=dev))
     assert torch.equal(y[0], y[-1]) and set(y.unique().tolist()) <= {0.0, 2.0}
-    with pytest.raises(NotImplementedError):
-        PrePostProcessing(e, 0.1, multilingual=True, n_languages=3)
+    # multilingual: the affine pair of language `factor`; the gradient lands in that row only
+    ml = PrePostProcessing(e, 0.0, sequence="n", multilingual=True, n_languages=3)
+    assert sorted(ml.state_dict()) == ["layer_norm.bias", "layer_norm.weight"] and ml.layer_norm.weight.shape == (3, e)
+    ml = randomise(ml, 85).to(dev).to(dtype)
+    factor = torch.tensor([2], device=dev)
+    xin = x.to(dev).requires_grad_()
+    out = ml(xin, factor=factor)
+    dy = torch.randn(t, b, e, generator=g).to(dtype)
+    out.backward(dy.to(dev))
+    w, bb = ml.layer_norm.weight.detach().cpu(), ml.layer_norm.bias.detach().cpu()
+    want, mu, rs = oln.ln_fwd(x.view(t * b, e), w[2], bb[2], 1e-5, D)
+    dxo, dgo, dbo = oln.ln_bwd(dy.view(t * b, e), x.view(t * b, e), mu, rs, w[2], D)
+    assert_close(out.view(t * b, e), want, dtype, "multilingual n")
+    assert_close(xin.grad.view(t * b, e), dxo, dtype, "multilingual dx", atol=1e-5 if dtype == torch.float32 else None)
+    assert_close(ml.layer_norm.weight.grad[2], dgo, dtype, "multilingual dgamma", scale_atol=True, atol=1e-5 if dtype == torch.float32 else None)
+    assert_close(ml.layer_norm.bias.grad[2], dbo, dtype, "multilingual dbeta", scale_atol=True, atol=1e-5 if dtype == torch.float32 else None)
+    assert (ml.layer_norm.weight.grad[:2] == 0).all() and (ml.layer_norm.bias.grad[:2] == 0).all()
+    with pytest.raises(RuntimeError, match="factor"):
+        ml(x.to(dev))
 
 
 def _encoder_case(dev, dtype, macaron, training, death_rate=0.0, seed=84, **more):
@@ -108,12 +141,13 @@ def _encoder_case(dev, dtype, macaron, training, death_rate=0.0, seed=84, **more
     y.backward(dy.to(dev))
     x64 = x.to(D).requires_grad_()
     p64r = {k: v.detach().to(dtype).to(D).requires_grad_() for k, v in p64.items()}     # the weights the kernels saw
-    want = otl.encoder_layer(x64, p64r, opt.n_heads, pad, act="gelu", macaron=macaron, death_rate=death_rate, training=training)
+    want = otl.encoder_layer(x64, p64r, opt.n_heads, pad, act="gelu", macaron=macaron, death_rate=death_rate, training=training,
+                             round_to=dtype, attn_core=attn_core(opt, training))
     want.backward(dy.to(D))
     layer_close(y, want.detach(), dtype, "encoder output")
     layer_close(xin.grad, x64.grad, dtype, "encoder dx")
     for name, prm in layer.named_parameters():
-        layer_close(prm.grad, p64r[name].grad, dtype, "d " + name)
+        layer_close(prm.grad, p64r[name].grad, dtype, "d " + name, summed=True)
     return layer
 
 
@@ -187,7 +221,8 @@ def _decoder_case(dev, dtype, ignore_source, **more):
     y.backward(dy.to(dev))
     x64, c64 = x.to(D).requires_grad_(), ctxt.to(D).requires_grad_()
     p64r = {k: v.detach().to(dtype).to(D).requires_grad_() for k, v in p64.items()}
-    want, cov = otl.decoder_layer(x64, c64, p64r, opt.n_heads, causal, src_pad, act="gelu", ignore_source=ignore_source, training=True)
+    want, cov = otl.decoder_layer(x64, c64, p64r, opt.n_heads, causal, src_pad, act="gelu", ignore_source=ignore_source, training=True,
+                                  round_to=dtype, attn_core=attn_core(opt, True))
     want.backward(dy.to(D))
     layer_close(y, want.detach(), dtype, "decoder output")
     layer_close(xin.grad, x64.grad, dtype, "decoder dx")
@@ -197,9 +232,9 @@ def _decoder_case(dev, dtype, ignore_source, **more):
         assert not any(n.startswith("multihead_src") or n.startswith("preprocess_src_attn") for n in layer.state_dict())
     else:
         layer_close(cin.grad, c64.grad, dtype, "decoder dcontext")
-        assert_close(coverage, cov.detach(), dtype, "coverage", atol=4e-3)   # probabilities behind three rounded operators
+        assert_close(coverage, cov.detach(), dtype, "coverage")
     for name, prm in layer.named_parameters():
-        layer_close(prm.grad, p64r[name].grad, dtype, "d " + name)
+        layer_close(prm.grad, p64r[name].grad, dtype, "d " + name, summed=True)
 
 
 def test_layers_with_dropout_and_unsupported_options(dev):

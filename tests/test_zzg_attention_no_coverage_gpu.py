@@ -3,12 +3,12 @@ tiled kernels over the padded batch (nmtg_flash_attn_batched_fwd / _bwd) and no 
 
 What the reference computes: onmt/modules/optimized/self_attention_func.py:50-520 and encdec_attention_func_bias.py:41-668
 with return_coverage false; checked against the same oracle as the calls that return the coverage (oracle/attention.py),
-to the same relative tolerance (util.assert_close: 2e-2, gradients' absolute part scaled by their magnitude). The absolute
-part is 4e-3 for bf16 instead of 1e-3: the oracle rounds the scores to the 16-bit type, as the extension's stored score
-tensor does, while the tiled core keeps them in fp32. A bf16 score of magnitude 4 moves by up to 2^-7 in that rounding and
-its probability by 0.8 %, which the signed sums of the context and of the output projection (values of order 0.1 to 1)
-turn into a few 1e-3 of absolute difference between two equally accurate results; fp16 rounds eight times finer.
-The batch-strided entry points are also held bit for bit against the packed ones on the sequences that both can express.
+in its core="tiled" mode, which rounds to 16 bits where these kernels do (scores and softmax statistics stay in fp32, the
+operands of the second product and of the gradient products are rounded, the dropout scale is applied in fp32 at the end)
+instead of where the extension's stored tensors do. Tolerance: the one every 16-bit comparison here uses
+(util.assert_close: 2e-2 relative, 1e-3 absolute, gradients' absolute part scaled by their magnitude), both types, all
+masks. The batch-strided entry points are also held bit for bit against the packed ones on the sequences that both can
+express.
 """
 import pytest
 import torch
@@ -22,7 +22,6 @@ from util import assert_close
 
 pytestmark = pytest.mark.gpu
 D = torch.float64
-ATOL = {torch.bfloat16: 4e-3, torch.float16: None}
 
 
 def _self_case(dev, t, b, e, h, dtype, p, pad_mask=None, seed=171, biases=True, time_mask=None):
@@ -34,8 +33,8 @@ def _self_case(dev, t, b, e, h, dtype, p, pad_mask=None, seed=171, biases=True, 
     if not biases:
         d["b_in"] = d["b_out"] = None
     fwd = oat.self_attn_fwd(d["x"], d["w_in"], d["w_out"], d["b_in"], d["b_out"], h, d["pad_mask"], time_mask, p, d["dropout_mask"], D,
-                            round_to=dtype)
-    bwd = oat.self_attn_bwd(d["dout"], d["x"], d["w_in"], d["w_out"], h, fwd, p, d["dropout_mask"], D, round_to=dtype)
+                            round_to=dtype, core="tiled")
+    bwd = oat.self_attn_bwd(d["dout"], d["x"], d["w_in"], d["w_out"], h, fwd, p, d["dropout_mask"], D, round_to=dtype, core="tiled")
     names = ("x", "w_in", "w_out", "b_in", "b_out")
     leaves = [d[k].to(dev).requires_grad_() if d[k] is not None else None for k in names]
     dm = d["dropout_mask"].to(dev) if p > 0 else None
@@ -44,20 +43,10 @@ def _self_case(dev, t, b, e, h, dtype, p, pad_mask=None, seed=171, biases=True, 
                               False, None, False, None, True, False, False, dm)
     assert cov.numel() == 0                               # the tiled core: no probability tensor exists
     out.backward(d["dout"].to(dev))
-    # Time masks: early rows attend a handful of keys, so their context is not an average but close to single value rows
-    # (magnitude 1 to 3 instead of 0.1), and the bf16 rounding of that context, summed over the model width by the output
-    # projection, doubles the absolute part. With dropout a lone kept probability is 1 / (1 - p): the oracle rounds it to
-    # bf16 as the extension's stored tensor does (1.3359 for p = 0.25), the tiled core multiplies by the fp32 scale at the
-    # end, and the two contexts then round to different bf16 neighbours where the values are past 2 (rounding unit 2^-6):
-    # the factor 2 / (1 - p) that tests/test_zze_flash_attention_gpu.py uses for the same effect. What pins the masking
-    # itself is test_a_causal_time_mask_equals_the_causal_flag_bit_for_bit below.
-    atol = ATOL[dtype]
-    if time_mask is not None and dtype == torch.bfloat16:
-        atol = 2 * ATOL[dtype] * (2 / (1 - p) if p > 0 else 1)
-    assert_close(out, fwd["outputs"], dtype, "outputs", atol=atol)
+    assert_close(out, fwd["outputs"], dtype, "outputs")
     for leaf, key in zip(leaves, ("dx", "dw_in", "dw_out", "db_in", "db_out")):
         if leaf is not None:
-            assert_close(leaf.grad, bwd[key], dtype, key, atol=atol, scale_atol=True)
+            assert_close(leaf.grad, bwd[key], dtype, key, scale_atol=True)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
@@ -130,9 +119,9 @@ def _encdec_case(dev, tq, tk, b, e, h, dtype, p, seed=174, biases=True):
     if not biases:
         d["b_q"] = d["b_kv"] = d["b_out"] = None
     fwd = oat.encdec_attn_fwd(d["x_q"], d["x_kv"], d["w_q"], d["w_kv"], d["w_out"], d["b_q"], d["b_kv"], d["b_out"], h,
-                              d["pad_mask"], p, d["dropout_mask"], D, round_to=dtype)
+                              d["pad_mask"], p, d["dropout_mask"], D, round_to=dtype, core="tiled")
     bwd = oat.encdec_attn_bwd(d["dout"], d["x_q"], d["x_kv"], d["w_q"], d["w_kv"], d["w_out"], h, fwd, p, d["dropout_mask"], D,
-                              round_to=dtype)
+                              round_to=dtype, core="tiled")
     names = ("x_q", "x_kv", "w_q", "w_kv", "w_out", "b_q", "b_kv", "b_out")
     leaf = {k: (d[k].to(dev).requires_grad_() if d[k] is not None else None) for k in names}
     dm = d["dropout_mask"].to(dev) if p > 0 else None
@@ -141,11 +130,11 @@ def _encdec_case(dev, tq, tk, b, e, h, dtype, p, seed=174, biases=True):
                                 dm)
     assert len(res) == 1
     res[0].backward(d["dout"].to(dev))
-    assert_close(res[0], fwd["outputs"], dtype, "outputs", atol=ATOL[dtype])
+    assert_close(res[0], fwd["outputs"], dtype, "outputs")
     for key, n in (("dx_q", "x_q"), ("dx_kv", "x_kv"), ("dw_q", "w_q"), ("dw_kv", "w_kv"), ("dw_out", "w_out"), ("db_q", "b_q"),
                    ("db_kv", "b_kv"), ("db_out", "b_out")):
         if leaf[n] is not None:
-            assert_close(leaf[n].grad, bwd[key], dtype, key, atol=ATOL[dtype], scale_atol=True)
+            assert_close(leaf[n].grad, bwd[key], dtype, key, scale_atol=True)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
@@ -161,9 +150,9 @@ def test_bias_free_encdec_function_without_coverage(dev, dtype):
     tq, tk, b, e, h, p = 24, 200, 3, 256, 4, 0.1
     d = inputs.encdec_attn_inputs(tq, tk, b, e, h, dtype, p=p, seed=175)
     fwd = oat.encdec_attn_fwd(d["x_q"], d["x_kv"], d["w_q"], d["w_kv"], d["w_out"], None, None, None, h, d["pad_mask"], p,
-                              d["dropout_mask"], D, round_to=dtype)
+                              d["dropout_mask"], D, round_to=dtype, core="tiled")
     bwd = oat.encdec_attn_bwd(d["dout"], d["x_q"], d["x_kv"], d["w_q"], d["w_kv"], d["w_out"], h, fwd, p, d["dropout_mask"], D,
-                              round_to=dtype)
+                              round_to=dtype, core="tiled")
     names = ("x_q", "x_kv", "w_q", "w_kv", "w_out")
     leaf = {k: d[k].to(dev).requires_grad_() for k in names}
     res = encdec_attn_func(False, True, h, leaf["x_q"], leaf["x_kv"], leaf["w_q"], leaf["w_kv"], leaf["w_out"],
@@ -171,9 +160,9 @@ def test_bias_free_encdec_function_without_coverage(dev, dtype):
                            d["dropout_mask"].to(dev))
     assert len(res) == 1
     res[0].backward(d["dout"].to(dev))
-    assert_close(res[0], fwd["outputs"], dtype, "outputs", atol=ATOL[dtype])
+    assert_close(res[0], fwd["outputs"], dtype, "outputs")
     for key, n in (("dx_q", "x_q"), ("dx_kv", "x_kv"), ("dw_q", "w_q"), ("dw_kv", "w_kv"), ("dw_out", "w_out")):
-        assert_close(leaf[n].grad, bwd[key], dtype, key, atol=ATOL[dtype], scale_atol=True)
+        assert_close(leaf[n].grad, bwd[key], dtype, key, scale_atol=True)
 
 
 def test_the_switch_keeps_the_extension_path(dev, monkeypatch):
@@ -208,6 +197,38 @@ def test_a_sequence_with_every_key_masked(dev):
     fa.bwd_batched(do, q, k, v, out, lse, dqkv[:, :, :, 0], dqkv[:, :, :, 1], dqkv[:, :, :, 2], pad, 0.0, d ** -0.5, False, state)
     assert torch.isfinite(dqkv).all()
     assert (dqkv[:, 1] == 0).all() and (dqkv[60:, 2, :, 1:] == 0).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_the_causal_flag_together_with_masked_leading_keys(dev, dtype):
+    """Sequence 1 masks its first 10 keys: queries 0..9 see no live key under the causal flag (all their keys up to the
+    diagonal are masked), also in key tiles that hold no masked key but lie across the diagonal. Such rows give out = 0,
+    lse = -inf and no gradient; every other row follows the oracle with both masks (scale 0.3, not the default)."""
+    t, b, h, d, scale = 150, 3, 2, 64, 0.3
+    g = torch.Generator().manual_seed(57)
+    qkv = (0.5 * torch.randn(t, b, h, 3, d, generator=g)).to(dtype)
+    do = torch.randn(t, b, h, d, generator=g).to(dtype)
+    pad = torch.zeros(b, t, dtype=torch.bool)
+    pad[1, :10] = True
+    pad[2, 140:] = True
+    pad[2, 3] = True
+    qkv_d = qkv.to(dev)
+    q, k, v = (qkv_d[:, :, :, i] for i in range(3))
+    out, lse, state = fa.fwd_batched(q, k, v, pad.to(torch.uint8).to(dev), 0.0, scale, True)
+    dqkv = torch.full_like(qkv_d, float("nan"))
+    fa.bwd_batched(do.to(dev), q, k, v, out, lse, dqkv[:, :, :, 0], dqkv[:, :, :, 1], dqkv[:, :, :, 2], pad.to(torch.uint8).to(dev),
+                   0.0, scale, True, state)
+    assert (out[:10, 1] == 0).all() and torch.isinf(lse[1, :, :10]).all() and (dqkv[:10, 1, :, 0] == 0).all()
+    assert torch.isfinite(out).all() and torch.isfinite(dqkv).all() and torch.isfinite(lse[1, :, 10:]).all()
+    causal = torch.triu(torch.ones(t, t), 1).bool()
+    r = d ** 0.5 * scale                                  # the oracle's core scales by 1 / sqrt(d): fold the rest into q
+    q3, k3, v3, do3 = (x.reshape(t, b * h, d).to(D) for x in (qkv[:, :, :, 0], qkv[:, :, :, 1], qkv[:, :, :, 2], do))
+    _, prob, keep, ctx = oat._core_fwd_tiled(q3 * r, k3, v3, h, pad, causal, 0.0, None, D, dtype)
+    dq, dk, dv = oat._core_bwd_tiled(do3, out.cpu().reshape(t, b * h, d).to(D), q3 * r, k3, v3, prob, keep, 0.0, D, dtype)
+    assert_close(out.reshape(t, b * h, d), ctx, dtype, "out")
+    assert_close(dqkv[:, :, :, 0].reshape(t, b * h, d), dq * r, dtype, "dq", scale_atol=True)
+    assert_close(dqkv[:, :, :, 1].reshape(t, b * h, d), dk, dtype, "dk", scale_atol=True)
+    assert_close(dqkv[:, :, :, 2].reshape(t, b * h, d), dv, dtype, "dv", scale_atol=True)
 
 
 def test_dropout_drawn_on_the_device_is_replayed_by_its_own_mask(dev):

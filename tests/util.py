@@ -15,12 +15,23 @@ TOL = {
 }
 
 
-def assert_close(actual, expected, dtype, what="", rtol=None, atol=None, scale_atol=False):
+def assert_close(actual, expected, dtype, what="", rtol=None, atol=None, scale_atol=False, flips=None):
     """actual: tensor from the HIP path (any device / dtype); expected: oracle (CPU, fp32/fp64).
 
     scale_atol: multiply the absolute tolerance by max|expected| — for reductions over thousands
     of terms (weight / bias gradients) whose magnitude is far above 1.
+    flips: an absolute tolerance that at most one element in a thousand may use instead of `atol`. Two chains of the same
+    16-bit roundings, one accumulating in fp32 and one in fp64, now and then land on opposite sides of a rounding boundary
+    of an intermediate; a result that cancels to a small value then inherits that intermediate's unit in the last place.
     """
+    if flips is not None:
+        a = actual.detach().to("cpu", torch.float64)
+        e = expected.detach().to("cpu", torch.float64)
+        tol = dict(TOL[dtype])
+        at = (tol["atol"] if atol is None else atol) * (max(1.0, float(e.abs().max())) if scale_atol else 1.0)
+        outside = (a - e).abs() > at + (tol["rtol"] if rtol is None else rtol) * e.abs()
+        assert outside.double().mean().item() <= 1e-3, f"{what}: {int(outside.sum())}/{outside.numel()} elements beyond atol={at}"
+        atol = flips
     tol = dict(TOL[dtype])
     if rtol is not None:
         tol["rtol"] = rtol
