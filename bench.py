@@ -797,11 +797,56 @@ class CopyWL(Workload):
         return 2 * self.src.numel() * 4
 
 
+class StreamProbeWL(Workload):
+    """One launch of the library's streaming probe (nmtg_stream_probe): the simplest kernel with the access mix of the
+    bandwidth-bound kernels (16 bytes per lane and access, four in flight, the grid covers the buffer once). Its rate is
+    the practical ceiling of this HBM for that mix, the figure the roofline fractions of the streaming workloads are read
+    against. Not part of `--workload all`; `--workload streams` runs the six of them."""
+    bound = "hbm"
+    dtype = "f32"
+    MODE, STREAMS, BYTES = 0, 2, 1 << 30
+
+    def setup(self, dev):
+        from nmtgminor_amd import _lib as L
+        self.L = L
+        n = self.BYTES // 4
+        self.a = torch.ones(n, dtype=torch.float32, device=dev)
+        self.b = torch.ones(n, dtype=torch.float32, device=dev) if self.MODE == 1 else None
+        blocks = L.load().nmtg_stream_probe_blocks(L.i64(self.BYTES))
+        self.out = torch.empty(blocks if self.MODE == 2 else n, dtype=torch.float32, device=dev)
+
+    def step(self):
+        L = self.L
+        L.call("nmtg_stream_probe", L.ptr(self.a), L.ptr(self.b), L.ptr(self.out), L.i64(self.BYTES), L.i32(self.MODE),
+               L.stream_of(self.a))
+        return self.out
+
+    def work_per_step(self):
+        return self.STREAMS * self.BYTES + (self.out.numel() * 4 if self.MODE == 2 else 0)
+
+    def kernel_work(self):
+        return {"stream_probe": self.work_per_step()}
+
+
+def _stream_probe(name, mode, streams, nbytes, what):
+    size = f"{nbytes >> 20} MiB"
+    return type("StreamProbe_" + name, (StreamProbeWL,), dict(
+        name=name, MODE=mode, STREAMS=streams, BYTES=nbytes,
+        description=f"streaming probe, {what}, {size} per buffer (fp32 lanes, 16 B per lane and access)"))
+
+
+STREAM_PROBES = [_stream_probe(n + suffix, mode, streams, nbytes, what)
+                 for suffix, nbytes in (("", 1 << 30), ("_64m", 1 << 26))
+                 for n, mode, streams, what in (("stream_copy", 0, 2, "one stream read and one written"),
+                                                ("stream_add", 1, 3, "two streams read and one written"),
+                                                ("stream_read", 2, 1, "one stream read, one float per block written"))]
+
+
 # the five benchmark configurations first, then the workloads added beside them
 WORKLOADS = {w.name: w for w in (LayerNormWL, MlpWL, SelfAttnWL, EncdecAttnWL, XentropyWL, SoftmaxDropoutWL, DropoutAddWL,
                                     GeneratorLossWL, RelSelfAttnWL, FusedAdamWL, LayerNormLargeWL, FlashAttnWL, DecodeStepWL,
                                     SelfAttnNoCoverageWL)}
-EXTRA_WORKLOADS = {CopyWL.name: CopyWL}
+EXTRA_WORKLOADS = {CopyWL.name: CopyWL, **{w.name: w for w in STREAM_PROBES}}
 PRIMARY = "mlp"
 
 
@@ -1006,7 +1051,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="all", help="one or more (comma-separated) of %s, or all" % ", ".join(WORKLOADS))
+    ap.add_argument("--workload", default="all", help="one or more (comma-separated) of %s, or all; beside them: copy (counter calibration) and streams (the six "
+                    "streaming probes %s)" % (", ".join(WORKLOADS), ", ".join(w.name for w in STREAM_PROBES)))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--trace-steps", type=int, default=10)
     ap.add_argument("--cpu-time-allowance", type=float, default=240.0,
@@ -1029,6 +1075,8 @@ def main():
         sys.exit(2)
     table = dict(WORKLOADS, **EXTRA_WORKLOADS)
     names = list(WORKLOADS) if args.workload == "all" else [n.strip() for n in args.workload.split(",") if n.strip()]
+    if names == ["streams"]:
+        names = [w.name for w in STREAM_PROBES]
     unknown = [n for n in names if n not in table]
     if unknown or not names:
         sys.stderr.write("bench.py: unknown workload %s; choose from %s\n" % (", ".join(unknown) or "''", ", ".join(table)))

@@ -632,6 +632,19 @@ int nmtg_multi_tensor_l2norm_scale(int n_tensors, const void* const* in, void* c
 int nmtg_trace_begin(void);
 int64_t nmtg_trace_end(char* out, int64_t capacity);
 
+/* ------------------------------------------------------------------------------------------
+ * Streaming probes (no counterpart in the reference; a measurement aid like the tracing above).
+ * One launch of the simplest kernel with the access mix of the library's bandwidth-bound
+ * kernels, to be timed: what this HBM gives such a mix is the practical ceiling their roofline
+ * fractions are read against. `bytes` (a multiple of 16) is the size of each buffer.
+ *   mode 0  out[i] = a[i]                         one stream read, one written
+ *   mode 1  out[i] = a[i] + b[i] (fp32 lanes)     two streams read, one written
+ *   mode 2  out[block] = sum of the block's chunk of a (fp32)   read only; `out` holds
+ *           nmtg_stream_probe_blocks(bytes) floats
+ * ------------------------------------------------------------------------------------------ */
+int64_t nmtg_stream_probe_blocks(int64_t bytes);
+int nmtg_stream_probe(const void* a, const void* b, void* out, int64_t bytes, int mode, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -54,7 +54,7 @@ def load():
         lib.nmtg_version.restype = ctypes.c_int
         for name in header_functions():
             fn = getattr(lib, name)  # AttributeError here = header / library mismatch
-            if name.endswith("_parts") or name.endswith("_bytes") or name == "nmtg_trace_end":
+            if name.endswith(("_parts", "_bytes", "_blocks")) or name == "nmtg_trace_end":
                 fn.restype = ctypes.c_int64
         _lib = lib
     return _lib

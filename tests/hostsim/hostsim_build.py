@@ -31,7 +31,7 @@ OPT = os.environ.get("HOSTSIM_OPT", "-O0")
 LIB = os.path.join(BUILD, "libnmtg_hostsim_asan.so" if SANITIZE else "libnmtg_hostsim.so")
 
 KERNEL_SOURCES = ["api.hip", "layer_norm.hip", "softmax_dropout.hip", "dropout_add.hip", "xentropy.hip", "reduce.hip",
-                  "gemm.hip", "gemm_nt.hip", "gemm_nn.hip", "gemm_tn.hip", "mlp.hip", "attention.hip", "rel_position.hip", "multi_tensor.hip", "rotary.hip", "flash_attn.hip", "gemm_f32.hip", "glu.hip", "attn_decode.hip", "gemm_skinny.hip"]
+                  "gemm.hip", "gemm_nt.hip", "gemm_nn.hip", "gemm_tn.hip", "mlp.hip", "attention.hip", "rel_position.hip", "multi_tensor.hip", "rotary.hip", "flash_attn.hip", "gemm_f32.hip", "glu.hip", "attn_decode.hip", "gemm_skinny.hip", "stream_probe.hip"]
 HEADERS = ["common.hip.h", "trace.hip.h", "reduce.hip.h", "gemm.hip.h", "gemm_ring.hip.h", "gemm_inst.hip.h"]
 OWN_SOURCES = ["hostsim.cpp", "stubs.cpp"]
 

@@ -291,3 +291,28 @@ def test_xentropy_errors(dev):
         xentropy_cuda.forward(x, torch.zeros(5, device=dev, dtype=torch.long), 0.1, False)
     with pytest.raises(RuntimeError):
         xentropy_cuda.forward(x, torch.zeros(4, device=dev, dtype=torch.long), 0.1, True)     # half_to_float on fp32
+
+
+@pytest.mark.parametrize("nbytes", [16, 4096 * 16 + 48, 1 << 20])
+def test_streaming_probes_move_what_they_say(dev, nbytes):
+    """The bench's streaming probes (nmtg_stream_probe) are kernels like any other: copy, fp32 add and per-block sums of a
+    buffer whose size is not a multiple of a block's chunk (16 KiB) are exact (sums: small integers, exact in fp32)."""
+    from nmtgminor_amd import _lib as L
+    n = nbytes // 4
+    g = torch.Generator().manual_seed(nbytes)
+    a = torch.randint(-8, 9, (n,), generator=g).float().to(dev)
+    b = torch.randint(-8, 9, (n,), generator=g).float().to(dev)
+    out = torch.full((n + 4,), 7.0, device=dev)
+    for mode, want in ((0, a), (1, a + b)):
+        out.fill_(7.0)
+        L.call("nmtg_stream_probe", L.ptr(a), L.ptr(b), L.ptr(out), L.i64(nbytes), L.i32(mode), L.stream_of(a))
+        assert torch.equal(out[:n], want) and (out[n:] == 7.0).all()
+    blocks = L.load().nmtg_stream_probe_blocks(L.i64(nbytes))
+    assert blocks == (nbytes + 16383) // 16384
+    sums = torch.full((blocks + 1,), 7.0, device=dev)
+    L.call("nmtg_stream_probe", L.ptr(a), L.ptr(None), L.ptr(sums), L.i64(nbytes), L.i32(2), L.stream_of(a))
+    pad = torch.zeros(blocks * 4096, device=dev)
+    pad[:n] = a
+    assert torch.equal(sums[:blocks], pad.view(blocks, 4096).sum(1)) and sums[blocks] == 7.0
+    with pytest.raises(RuntimeError, match="multiple of 16"):
+        L.call("nmtg_stream_probe", L.ptr(a), L.ptr(b), L.ptr(out), L.i64(24), L.i32(0), L.stream_of(a))

@@ -229,6 +229,11 @@ def test_xentropy_no_smoothing_module_and_autograd():
 CODE = {F32: 0, F16: 1, BF16: 2}
 
 
+@pytest.mark.parametrize("nbytes", [16, 4096 * 16 + 48])
+def test_streaming_probes(nbytes):
+    tel.test_streaming_probes_move_what_they_say(CPU, nbytes)
+
+
 @pytest.mark.parametrize("dtype", tel.DTYPES)
 @pytest.mark.parametrize("m,n,pad", [(1, 8, 0), (7, 40, 0), (128, 256, 8), (129, 24, 0), (1000, 264, 0), (8195, 64, 8),
                                      (2100, 37, 3), (16, 1, 0), (4099, 520, 0)])
