@@ -1065,7 +1065,7 @@ def main():
     ap.add_argument("--emit-results", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--variants", default="",
                     help="semicolon-separated sets of per-call library switches to time after the default configuration, "
-                         "e.g. 'NMTG_GELU_LUT=0;NMTG_GELU_LUT=0+NMTG_MLP_TAIL=0'. Each set is exported (NAME=VALUE, or NAME=1 "
+                         "e.g. 'NMTG_GEMM_TILE=1;NMTG_ATTN_FUSED=0+NMTG_GEMM_SKINNY=0'. Each set is exported (NAME=VALUE, or NAME=1 "
                          "when no value is given) for one extra measurement of every selected workload (no CPU baseline); "
                          "results go to 'variants'.")
     args = ap.parse_args()

@@ -149,20 +149,13 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
   }
   if (!gemm_has(layout, tile, epi))
     return fail(NMTG_ERR_UNSUPPORTED, "gemm: layout %d has no kernel for epilogue %d", layout, epi);
-  // direct-to-LDS operand loads need whole 64-k steps (k_per_split is a multiple of 64 already)
-  static const bool dma_off = getenv("NMTG_GEMM_NO_DMA") != nullptr;
-  a.dma = (!dma_off && a.K > 0 && a.K % GEMM_BK == 0) ? 1 : 0;
-  // the slot-ring kernel addresses each operand with 32-bit lane offsets
-  static const bool ring_off = getenv("NMTG_GEMM_NO_RING") != nullptr;
+  // The slot-ring kernel (direct global -> LDS loads) needs whole 64-k steps (k_per_split is a multiple of 64 already),
+  // 16-byte accesses, and addresses each operand with 32-bit lane offsets; every other call takes the two-buffer loop.
   const int64_t a_bytes = static_cast<int64_t>(a_kc ? a.M : a.K) * a.lda * 2;
   const int64_t b_bytes = static_cast<int64_t>(b_kc ? a.N : a.K) * a.ldb * 2;
-  // NMTG_GEMM_RING_S=0 keeps the 256x64 tile (the per-head attention products) on the two-buffer loop.
-  const bool ring_s = !switched_off("NMTG_GEMM_RING_S");
-  a.ring = (!ring_off && a.dma && vec == 8 && (tile != TILE_S || ring_s) && a_bytes < (int64_t{1} << 32) &&
-            b_bytes < (int64_t{1} << 32)) ? 1 : 0;
-  // gelu and gelu' of the activation epilogues come from a table in LDS (ring kernels only, they have the LDS room);
-  // NMTG_GELU_LUT=0 evaluates the formula instead.
-  a.act_lut = (a.ring && (epi == EPI_ACT_FWD || epi == EPI_ACT_BWD) && !switched_off("NMTG_GELU_LUT")) ? 1 : 0;
+  a.ring = (a.K > 0 && a.K % GEMM_BK == 0 && vec == 8 && a_bytes < (int64_t{1} << 32) && b_bytes < (int64_t{1} << 32)) ? 1 : 0;
+  // gelu and gelu' of the activation epilogues come from a table in LDS in the ring kernels (they have the LDS room)
+  a.act_lut = (a.ring && (epi == EPI_ACT_FWD || epi == EPI_ACT_BWD)) ? 1 : 0;
   int bm, bn;
   tile_dims(tile, bm, bn);
   a.m_tiles = ceil_div(a.M, bm);
@@ -202,7 +195,6 @@ int row_tile_try(int dtype, int epi, GemmArgs a, const void* extra_like_c, hipSt
   auto ok8 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 8 == 0; };
   if ((a.dmask && !ok8(a.dmask)) || (a.kmask && a.kmask_kind != 0 && !ok8(a.kmask))) return 0;
   a.vec = 8;
-  a.dma = 0;
   a.ring = 0;
   a.splits = 1;
   a.k_per_split = ceil_div(a.K, GEMM_BK) * GEMM_BK;

@@ -62,7 +62,6 @@ struct GemmArgs {
   int splits, k_per_split;
   float alpha;
   int vec;                  // widest access (elements: 8, 4 or 1) every operand and extent allows
-  int dma;                  // every 64-k step of every split is full: direct-to-LDS loads allowed
   int ring;                 // the call meets the requirements of the slot-ring kernel (gemm_ring.hip.h)
   const void* bias;
   void* aux_out;
@@ -454,34 +453,6 @@ struct TileStage {
     }
   }
 };
-
-// Direct global -> LDS load of a reduction-contiguous tile [ROWS][64 k] (gfx950
-// global_load_lds_dwordx4): no staging registers and no ds_write instructions. Wave w's i-th
-// instruction fills the 64 consecutive 16-byte chunks p = (i * NW + w) * 64 + lane of the tile, so
-// the swizzle is applied on the global side: chunk p holds row p / 8, k-chunk (p % 8) ^ swz(row).
-// Rows past the end are clamped to the last row (their products land in rows that are never
-// stored); the caller guarantees that the 64 k of the step are all valid.
-template <typename T, int ROWS, int NT>
-__device__ __forceinline__ void dma_tile(const T* __restrict__ base, int64_t ld, int rows_total, int row0, int k0,
-                                         T* lds_tile, int tid) {
-  constexpr int NW = NT / 64;
-  constexpr int INSTR = ROWS * 8 / NT;
-  static_assert(ROWS * 8 % NT == 0, "tile must be a whole number of wave instructions");
-  const int lane = tid & 63, wave = tid >> 6;
-#pragma unroll
-  for (int i = 0; i < INSTR; ++i) {
-    const int p = (i * NW + wave) * 64 + lane;
-    const int row = p >> 3, c = (p & 7) ^ lds_swz(row);
-    const int grow = min(row0 + row, rows_total - 1);
-    const T* src = base + static_cast<int64_t>(grow) * ld + k0 + c * 8;
-    const uint32_t dst = __builtin_amdgcn_readfirstlane(
-        static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds_tile)) + static_cast<uint32_t>((i * NW + wave) * 1024));
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                     (__attribute__((address_space(3))) void*)static_cast<uintptr_t>(dst), 16, 0, 0);
-  }
-}
-
-__device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0f70); }  // vmcnt(0)
 
 // ---------------------------------------------------------------------------------------------
 // Epilogue shared by the GEMM kernels: accumulators -> (bias, activation, masks, ...) -> global.
@@ -883,7 +854,7 @@ constexpr int gemm_lds_bytes() {
   return main_loop > c_tile ? main_loop : c_tile;
 }
 
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC, int EPI, int VEC, bool DMA = false>
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool A_KC, bool B_KC, int EPI, int VEC>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const GemmArgs g) {
   constexpr int NT = 64 * WAVES_M * WAVES_N;
   constexpr int BK = GEMM_BK;
@@ -929,18 +900,12 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const Gemm
   TileStage<T, BM, NT, A_KC, VEC> stA;
   TileStage<T, BN, NT, B_KC, VEC> stB;
 
-  // DMA: reduction-contiguous operands go global -> LDS directly (whole 64-k steps only; the host
-  // selects this variant when every step of every split is full).
-  constexpr bool DMA_A = DMA && A_KC && VEC == 8, DMA_B = DMA && B_KC && VEC == 8;
   NMTG_PROF_MARK(0);
   if (nk > 0) {
-    if constexpr (DMA_A) dma_tile<T, BM, NT>(A, g.lda, g.M, m0, kbeg, sA, tid);
-    else stA.load(A, g.lda, g.M, m0, kbeg, kend, tid);
-    if constexpr (DMA_B) dma_tile<T, BN, NT>(B, g.ldb, g.N, n0, kbeg, sB, tid);
-    else stB.load(B, g.ldb, g.N, n0, kbeg, kend, tid);
-    if constexpr (!DMA_A) stA.store(sA, tid);
-    if constexpr (!DMA_B) stB.store(sB, tid);
-    if constexpr (DMA_A || DMA_B) wait_vmem_all();
+    stA.load(A, g.lda, g.M, m0, kbeg, kend, tid);
+    stB.load(B, g.ldb, g.N, n0, kbeg, kend, tid);
+    stA.store(sA, tid);
+    stB.store(sB, tid);
   }
   __syncthreads();
 
@@ -963,10 +928,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const Gemm
   for (int kt = 0; kt < nk; ++kt) {
     const int cur = kt & 1;
     if (kt + 1 < nk) {
-      if constexpr (DMA_A) dma_tile<T, BM, NT>(A, g.lda, g.M, m0, kbeg + (kt + 1) * BK, sA + (cur ^ 1) * BM * BK, tid);
-      else stA.load(A, g.lda, g.M, m0, kbeg + (kt + 1) * BK, kend, tid);
-      if constexpr (DMA_B) dma_tile<T, BN, NT>(B, g.ldb, g.N, n0, kbeg + (kt + 1) * BK, sB + (cur ^ 1) * BN * BK, tid);
-      else stB.load(B, g.ldb, g.N, n0, kbeg + (kt + 1) * BK, kend, tid);
+      stA.load(A, g.lda, g.M, m0, kbeg + (kt + 1) * BK, kend, tid);
+      stB.load(B, g.ldb, g.N, n0, kbeg + (kt + 1) * BK, kend, tid);
     }
     const T* cA = sA + cur * BM * BK;
     const T* cB = sB + cur * BN * BK;
@@ -984,9 +947,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const Gemm
         for (int j = 0; j < TN; ++j) mfma<T>::run(fn[j], fm[i], acc[i][j]);
     }
     if (kt + 1 < nk) {
-      if constexpr (!DMA_A) stA.store(sA + (cur ^ 1) * BM * BK, tid);
-      if constexpr (!DMA_B) stB.store(sB + (cur ^ 1) * BN * BK, tid);
-      if constexpr (DMA_A || DMA_B) wait_vmem_all();
+      stA.store(sA + (cur ^ 1) * BM * BK, tid);
+      stB.store(sB + (cur ^ 1) * BN * BK, tid);
     }
     __syncthreads();
   }

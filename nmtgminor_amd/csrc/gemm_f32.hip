@@ -258,7 +258,7 @@ int gemm_f32_run(int layout, int epi, GemmArgs a, hipStream_t st, int* m_tiles_o
   a.vec = wide ? 4 : 1;
   a.splits = 1;
   a.k_per_split = a.K;
-  a.dma = a.ring = a.act_lut = a.defer_reduce = a.riders_taken = 0;
+  a.ring = a.act_lut = a.defer_reduce = a.riders_taken = 0;
   a.m_tiles = (a.M + F32_BM - 1) / F32_BM;
   a.n_tiles = (a.N + F32_BN - 1) / F32_BN;
   a.tile_used = -1;

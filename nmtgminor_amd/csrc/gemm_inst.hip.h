@@ -20,10 +20,10 @@ inline void tile_dims(int tile, int& bm, int& bn) {
   else { bm = 256; bn = 64; }
 }
 
-template <typename T, int TILE, bool A_KC, bool B_KC, int EPI, int VEC, bool DMA = false>
+template <typename T, int TILE, bool A_KC, bool B_KC, int EPI, int VEC>
 int gemm_launch_vec(const GemmArgs& a, hipStream_t st) {
   using C = tile_cfg<TILE>;
-  auto kern = gemm_kernel<T, C::BM, C::BN, C::WM, C::WN, A_KC, B_KC, EPI, VEC, DMA>;
+  auto kern = gemm_kernel<T, C::BM, C::BN, C::WM, C::WN, A_KC, B_KC, EPI, VEC>;
   constexpr int lds = gemm_lds_bytes<C::BM, C::BN>();
   static bool attr_done = false;
   if (!attr_done) {
@@ -37,8 +37,7 @@ int gemm_launch_vec(const GemmArgs& a, hipStream_t st) {
                                   (EPI == EPI_PLAIN ? "plain" : EPI == EPI_ACT_FWD ? "actfwd" : EPI == EPI_ACT_BWD ? "actbwd"
                                    : EPI == EPI_SCORES ? "scores" : (EPI == EPI_SCORES_SOFTMAX || EPI == EPI_SCORES_SOFTMAX_RNG) ? "scores_softmax" : EPI == EPI_DSOFTMAX ? "dsoftmax"
                                    : "splitk") +
-                                  (VEC == 8 ? "" : VEC == 4 ? "_v4" : "_v1") +
-                                  (DMA ? "_dma" : "");
+                                  (VEC == 8 ? "" : VEC == 4 ? "_v4" : "_v1");
   TraceScope trace(name.c_str(), st);
   hipLaunchKernelGGL(kern, grid, dim3(64 * C::WM * C::WN), lds, st, a);
   return 0;
@@ -98,9 +97,6 @@ int gemm_launch_ring(const GemmArgs& a, hipStream_t st) {
 template <typename T, int TILE, bool A_KC, bool B_KC, int EPI>
 int gemm_launch_one(const GemmArgs& a, hipStream_t st) {
   if (a.vec == 8 && a.ring) return gemm_launch_ring<T, TILE, A_KC, B_KC, EPI>(a, st);
-  if constexpr (TILE == TILE_S && (A_KC || B_KC)) {
-    if (a.vec == 8 && a.dma) return gemm_launch_vec<T, TILE, A_KC, B_KC, EPI, 8, true>(a, st);
-  }
   if (a.vec == 8) return gemm_launch_vec<T, TILE, A_KC, B_KC, EPI, 8>(a, st);
   if constexpr (TILE != TILE_L) {
     if (a.vec == 4) return gemm_launch_vec<T, TILE, A_KC, B_KC, EPI, 4>(a, st);

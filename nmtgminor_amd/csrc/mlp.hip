@@ -158,15 +158,14 @@ extern "C" int nmtg_mlp_bwd(int num_layers, const void* x, const void* const* we
   NMTG_REQUIRE(batch == 0 || (x && grad_out), "mlp_bwd: null pointer argument");
   uint8_t* wsb = static_cast<uint8_t*>(workspace);
   void* dh[2] = {wsb, wsb + plan.dh_bytes};
-  // The split-K reductions and the final bias-gradient sums of all layers run as one launch at the end;
-  // NMTG_MLP_TAIL=0 gives each its own launch (two per layer). Results are bit-identical.
-  const bool tail_mode = !switched_off("NMTG_MLP_TAIL");
+  // The split-K reductions and the final bias-gradient sums of all layers are collected as jobs of one reduction
+  // (ReduceTail, up to its capacity; layers beyond that get launches of their own, with bit-identical results).
   ReduceTail tail;
   auto colsum_region = [&](int layer) {
-    return reinterpret_cast<float*>(wsb + 2 * plan.dh_bytes + (tail_mode ? layer : 0) * plan.colsum_bytes);
+    return reinterpret_cast<float*>(wsb + 2 * plan.dh_bytes + layer * plan.colsum_bytes);
   };
   auto splitk_region = [&](int layer) {
-    return static_cast<void*>(wsb + 2 * plan.dh_bytes + plan.layers * plan.colsum_bytes + (tail_mode ? layer : 0) * plan.splitk_bytes);
+    return static_cast<void*>(wsb + 2 * plan.dh_bytes + plan.layers * plan.colsum_bytes + layer * plan.splitk_bytes);
   };
 
   // element offsets of each hidden layer inside the concatenated buffers
@@ -195,7 +194,7 @@ extern "C" int nmtg_mlp_bwd(int num_layers, const void* x, const void* const* we
     // bias gradient (its partial rows: written by the data-gradient GEMM of the layer above, or by a kernel of its own)
     float* colsum_ws = colsum_region(i);
     if (grad_biases && grad_biases[i]) {
-      if (tail_mode && !tail.full()) {
+      if (!tail.full()) {
         int parts = parts_rows;
         rc = 0;
         if (!bias_from_parts) {
@@ -219,7 +218,7 @@ extern "C" int nmtg_mlp_bwd(int num_layers, const void* x, const void* const* we
       g.C = grad_weights[i]; g.ldc = in_i;
       g.M = static_cast<int>(out_i); g.N = static_cast<int>(in_i); g.K = static_cast<int>(batch);
       g.batch = 1; g.alpha = 1.f;
-      g.defer_reduce = (tail_mode && !tail.full()) ? 1 : 0;
+      g.defer_reduce = !tail.full() ? 1 : 0;
       // (the partial column sums do not ride with this product: a split-K launch repeats the rider blocks in every
       // split, and the tiles then share CUs unevenly; measured slower than the launch of their own)
       if (int rc2 = flush_head()) return rc2;

@@ -89,8 +89,8 @@ def forward(is_training, heads, inputs_q, inputs_kv, input_weights_q, input_weig
             "weight shapes do not match the inputs")
     c = lambda z: z.contiguous() if z is not None else None
     # inference with a key length that is not a multiple of 64: keys / values padded with masked zero rows, so that every
-    # tensor of the middle section is 16-byte aligned (NMTG_ATTN_PAD_KEYS=0 keeps the exact-length buffers)
-    if (not is_training and tk % KEY_BLOCK != 0 and os.environ.get("NMTG_ATTN_PAD_KEYS") != "0"
+    # tensor of the middle section is 16-byte aligned
+    if (not is_training and tk % KEY_BLOCK != 0
             and A.scores_needed(False, inputs_q.dtype, e // heads, tk, need_backward)):
         return _fwd_padded_keys(heads, c(inputs_q), c(inputs_kv), c(input_weights_q), c(input_weights_kv), c(output_weights),
                                 c(input_biases_q), c(input_biases_kv), c(output_biases), pad_mask, tq, tk, b, e)

@@ -624,7 +624,7 @@ def test_fused_adam_optimizer(dtype, adam_w):
 @pytest.mark.parametrize("dtype", HALVES)
 @pytest.mark.parametrize("batch,m,n,k", [(3, 300, 64, 192), (2, 256, 64, 64), (5, 77, 64, 128)])
 def test_ring_loop_of_the_256x64_tile(mi355x, dma, dtype, batch, m, n, k):
-    tst.test_ring_256x64_matches_two_buffer_loop(CPU, dtype, batch, m, n, k)
+    tst.test_ring_256x64_products(CPU, dtype, batch, m, n, k)
 
 
 @pytest.mark.parametrize("dtype", HALVES)
