@@ -140,7 +140,9 @@ int nmtg_softmax_dropout_bwd(const void* grad_dropped, const void* saved, int sa
  * The backward is elementwise once lse is known, so it also works on a slice of the classes:
  * the `vocab` columns handed in are classes [class_offset, class_offset + vocab) of
  * total_classes (labels stay global; smoothing spreads over total_classes). The whole row:
- * class_offset = 0, total_classes = vocab.
+ * class_offset = 0, total_classes = vocab. grad_logits may be the logits buffer itself (same
+ * pitch): every element is read before it is overwritten. (The reference allocates a second
+ * tensor of the logits' size, xentropy_kernel.cu:636-645.)
  * ------------------------------------------------------------------------------------------ */
 int nmtg_xentropy_fwd(const void* logits, const int64_t* labels, float* losses, float* lse,
                       int64_t rows, int64_t vocab, int64_t ld_logits, float smoothing,

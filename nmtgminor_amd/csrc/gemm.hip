@@ -150,10 +150,11 @@ int gemm_run(int dtype, int layout, int epi, GemmArgs a, void* workspace, size_t
   if (!gemm_has(layout, tile, epi))
     return fail(NMTG_ERR_UNSUPPORTED, "gemm: layout %d has no kernel for epilogue %d", layout, epi);
   // The slot-ring kernel (direct global -> LDS loads) needs whole 64-k steps (k_per_split is a multiple of 64 already),
-  // 16-byte accesses, and addresses each operand with 32-bit lane offsets; every other call takes the two-buffer loop.
-  const int64_t a_bytes = static_cast<int64_t>(a_kc ? a.M : a.K) * a.lda * 2;
-  const int64_t b_bytes = static_cast<int64_t>(b_kc ? a.N : a.K) * a.ldb * 2;
-  a.ring = (a.K > 0 && a.K % GEMM_BK == 0 && vec == 8 && a_bytes < (int64_t{1} << 32) && b_bytes < (int64_t{1} << 32)) ? 1 : 0;
+  // 16-byte accesses, and 32-bit lane offsets inside one tile of an operand: 256 rows of a reduction-contiguous one, 64
+  // k-rows plus a row of the other kind. Every other call takes the two-buffer loop.
+  const int64_t a_span = a_kc ? 256 * a.lda * 2 : 64 * a.lda * 2 + static_cast<int64_t>(a.M) * 2;
+  const int64_t b_span = b_kc ? 256 * a.ldb * 2 : 64 * a.ldb * 2 + static_cast<int64_t>(a.N) * 2;
+  a.ring = (a.K > 0 && a.K % GEMM_BK == 0 && vec == 8 && a_span < (int64_t{1} << 32) && b_span < (int64_t{1} << 32)) ? 1 : 0;
   // gelu and gelu' of the activation epilogues come from a table in LDS in the ring kernels (they have the LDS room)
   a.act_lut = (a.ring && (epi == EPI_ACT_FWD || epi == EPI_ACT_BWD)) ? 1 : 0;
   int bm, bn;

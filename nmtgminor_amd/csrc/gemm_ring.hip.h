@@ -134,8 +134,12 @@ __device__ __forceinline__ void gemm_ring_body(const GemmArgs& g, int block_x) {
   const int total = nk * SPS;
 
   const int64_t lda_b = g.lda * 2, ldb_b = g.ldb * 2;  // bytes
-  const char* a_base = static_cast<const char*>(g.A) + static_cast<int64_t>(bz) * g.sA * 2 + static_cast<int64_t>(kbeg) * (A_KC ? 2 : lda_b);
-  const char* b_base = static_cast<const char*>(g.B) + static_cast<int64_t>(bz) * g.sB * 2 + static_cast<int64_t>(kbeg) * (B_KC ? 2 : ldb_b);
+  // A reduction-contiguous operand is addressed from the first row of this block's tile (64-bit, scalar), so that the
+  // per-lane offsets span one tile's rows and fit 32 bits whatever the size of the operand.
+  const char* a_base = static_cast<const char*>(g.A) + static_cast<int64_t>(bz) * g.sA * 2 + static_cast<int64_t>(kbeg) * (A_KC ? 2 : lda_b) +
+                       (A_KC ? static_cast<int64_t>(m0) * lda_b : 0);
+  const char* b_base = static_cast<const char*>(g.B) + static_cast<int64_t>(bz) * g.sB * 2 + static_cast<int64_t>(kbeg) * (B_KC ? 2 : ldb_b) +
+                       (B_KC ? static_cast<int64_t>(n0) * ldb_b : 0);
   const int64_t step_a = A_KC ? GEMM_BK * 2 : GEMM_BK * lda_b;
   const int64_t step_b = B_KC ? GEMM_BK * 2 : GEMM_BK * ldb_b;
 
@@ -146,7 +150,7 @@ __device__ __forceinline__ void gemm_ring_body(const GemmArgs& g, int block_x) {
     if constexpr (decltype(kc_tag)::value) {
       const int r = 8 * ii + (lane >> 3);
       const int c = (lane & 7) ^ lds_swz(r);
-      const int row = min(row0 + 128 * j + r, rows_total - 1);
+      const int row = min(row0 + 128 * j + r, rows_total - 1) - row0;      // from the tile's first row (see a_base)
       return static_cast<uint32_t>(static_cast<int64_t>(row) * ld_b + c * 16);
     } else {
       const int k = 4 * ii + (lane >> 4);

@@ -191,8 +191,8 @@ __global__ __launch_bounds__(XE_THREADS) void xentropy_fwd_kernel(
 
 template <typename T, bool VEC>
 __global__ __launch_bounds__(XE_THREADS) void xentropy_bwd_kernel(
-    const float* __restrict__ grad_loss, const T* __restrict__ logits, const float* __restrict__ lse_in,
-    const int64_t* __restrict__ labels, T* __restrict__ grad_logits, int64_t vocab, int64_t ld, int64_t ld_grad,
+    const float* __restrict__ grad_loss, const T* logits, const float* __restrict__ lse_in,
+    const int64_t* __restrict__ labels, T* grad_logits, int64_t vocab, int64_t ld, int64_t ld_grad,
     int64_t class_offset, int64_t total_classes, float smoothing, int64_t padding_idx) {
   constexpr int EPV = 16 / sizeof(T);
   const int64_t row = blockIdx.x;

@@ -1,4 +1,5 @@
-"""Output projection + label-smoothed cross-entropy without the [N, V] logits tensor.
+"""Output projection + label-smoothed cross-entropy: the logits are kept once, in the working dtype, when they fit a
+stated budget of device memory, and never materialised otherwise.
 
 The reference projects the decoder states to the vocabulary (Generator.forward,
 onmt/modules/base_seq2seq.py:26-47) and hands the whole logits tensor to the loss
@@ -13,6 +14,13 @@ with the slice's weights (gradient of the states, [N, E], summed over the slices
 the unchunked pair of operators to rounding; arbitrary per-row upstream gradients (loss weights) are supported because
 nothing of the backward is precomputed in the forward.
 
+Kept logits (`keep_logits_bytes`, default 16 GiB): a training call whose [N, V] logits fit the budget (8.2 GB for the
+case above; this GPU has 288 GB) projects once over all rows, keeps the logits for the backward and turns them into their
+gradient in place there, which is then contracted once with the states (the weight gradient) and once with the weights
+(the gradient of the states): three products of N x E x V per step instead of four, and one tensor of the logits' size
+where the reference holds two (the logits saved by autograd and their gradient, xentropy_kernel.cu:636-645). A second
+backward over the same graph finds the logits consumed and takes the recomputing path.
+
 The chunk buffers have a row pitch of the vocabulary rounded up to 64 elements, so that the projection's stores and the
 two contractions that read the logits gradient move 16 bytes per access whatever the vocabulary size (250 054 is not a
 multiple of 4); the cross-entropy kernels read and write the first V elements of each pitched row in place.
@@ -26,6 +34,7 @@ import torch.nn as nn
 from ..native import linear_gemm, xentropy_cuda
 
 DEFAULT_CHUNK_ROWS = 4096
+DEFAULT_KEEP_LOGITS_BYTES = 16 << 30
 
 
 def _check(cond, msg):
@@ -67,28 +76,66 @@ def _logits(hidden, weight, bias, r0, r1, buf):
 
 class LinearSoftmaxCrossEntropy(torch.autograd.Function):
     """apply(hidden [N, E], weight [V, E], bias [V] | None, labels [N], smoothing=0.0, padding_idx=-100,
-    chunk_rows=4096) -> losses fp32 [N] (zeros where labels == padding_idx): what
+    chunk_rows=4096, keep_logits_bytes=16 GiB) -> losses fp32 [N] (zeros where labels == padding_idx): what
     SoftmaxCrossEntropyLoss.apply(F.linear(hidden, weight, bias), labels, smoothing, padding_idx, True) returns."""
 
     @staticmethod
-    def forward(ctx, hidden, weight, bias, labels, smoothing=0.0, padding_idx=-100, chunk_rows=DEFAULT_CHUNK_ROWS):
+    def forward(ctx, hidden, weight, bias, labels, smoothing=0.0, padding_idx=-100, chunk_rows=DEFAULT_CHUNK_ROWS,
+                keep_logits_bytes=DEFAULT_KEEP_LOGITS_BYTES):
         _check_inputs(hidden, weight, bias, labels, chunk_rows)
         hidden, weight, labels = hidden.contiguous(), weight.contiguous(), labels.contiguous()
         bias = bias.contiguous() if bias is not None else None
         n, v = hidden.size(0), weight.size(0)
         losses = torch.empty(n, dtype=torch.float32, device=hidden.device)
         lse = torch.empty(n, dtype=torch.float32, device=hidden.device)
+        ctx.kept = None
         if n > 0:
             _check(v > 0, "Number of classes in input should not be 0")
-            buf = _chunk_buffer(min(n, chunk_rows), v, hidden)
-            for r0, r1 in _chunks(n, chunk_rows):
-                z = _logits(hidden, weight, bias, r0, r1, buf)
-                part, m = xentropy_cuda.forward(z, labels[r0:r1], smoothing, True, padding_idx=padding_idx)
-                losses[r0:r1] = part
-                lse[r0:r1] = m
+            pitch = (v + 63) // 64 * 64
+            keep = any(ctx.needs_input_grad[:3]) and n * pitch * hidden.element_size() <= int(keep_logits_bytes)
+            if keep:
+                # the columns between V and the pitch are multiplied by nothing, but the contraction over the classes
+                # reads whole 16-byte groups: keep them finite
+                full = torch.empty(n, pitch, dtype=hidden.dtype, device=hidden.device)
+                full[:, v:].zero_()
+                z = linear_gemm.gemm(hidden, weight, trans_b=True, bias=bias, out=full[:, :v])
+                part, m = xentropy_cuda.forward(z, labels, smoothing, True, padding_idx=padding_idx)
+                losses.copy_(part)
+                lse.copy_(m)
+                ctx.kept = full
+            else:
+                buf = _chunk_buffer(min(n, chunk_rows), v, hidden)
+                for r0, r1 in _chunks(n, chunk_rows):
+                    z = _logits(hidden, weight, bias, r0, r1, buf)
+                    part, m = xentropy_cuda.forward(z, labels[r0:r1], smoothing, True, padding_idx=padding_idx)
+                    losses[r0:r1] = part
+                    lse[r0:r1] = m
         ctx.save_for_backward(hidden, weight, bias, labels, lse)
         ctx.smoothing, ctx.padding_idx, ctx.chunk_rows = smoothing, padding_idx, chunk_rows
         return losses
+
+    @staticmethod
+    def _backward_from_kept(ctx, full, grad_loss, hidden, weight, bias, labels, lse, need_h, need_w, need_b):
+        """The kept logits become their gradient in place; one contraction with the states, one with the weights."""
+        n, v = hidden.size(0), weight.size(0)
+        z = full[:, :v]
+        dz = xentropy_cuda.backward(grad_loss, z, lse, labels, ctx.smoothing, padding_idx=ctx.padding_idx, out=z)
+        dh = dw = db = None
+        if need_w:
+            dw = linear_gemm.gemm(dz, hidden, trans_a=True)                          # [V, N] x [N, E]
+        if need_b:
+            db = linear_gemm.colsum(dz)                                              # fixed-order fp32 column sums
+        if need_h:
+            # the contraction over the classes in whole 64-class steps (the matrix-core loop fed from LDS directly), and
+            # the last V % 64 classes as a product of their own; summed in fp32
+            v0 = v // 64 * 64
+            if v0 == v or v0 == 0:
+                dh = linear_gemm.gemm(dz, weight)
+            else:
+                dh32 = linear_gemm.gemm(full[:, :v0], weight[:v0]).float()
+                dh32.add_(linear_gemm.gemm(full[:, v0:v], weight[v0:]))
+                dh = dh32.to(hidden.dtype)
+        return dh, dw, db
 
     @staticmethod
     def backward(ctx, grad_loss):
@@ -104,6 +151,11 @@ class LinearSoftmaxCrossEntropy(torch.autograd.Function):
             db = torch.empty_like(bias) if n > 0 else torch.zeros_like(bias)
         if need_h:
             dh = torch.empty_like(hidden)
+        full, ctx.kept = ctx.kept, None              # consumed below: a second backward recomputes
+        if full is not None and n > 0 and (need_h or need_w or need_b):
+            dh, dw, db = LinearSoftmaxCrossEntropy._backward_from_kept(ctx, full, grad_loss, hidden, weight, bias, labels, lse,
+                                                                       need_h, need_w, need_b)
+            return dh, dw, db, None, None, None, None, None
         if n > 0 and (need_h or need_w or need_b):
             # Given the log-sum-exp of each row the logits gradient is elementwise, so the backward walks the
             # vocabulary in slices of whole columns: a slice's weight and bias gradients are complete (contracted over
@@ -136,7 +188,7 @@ class LinearSoftmaxCrossEntropy(torch.autograd.Function):
                         dh32.add_(part)
             if need_h and dh32 is not None:
                 dh.copy_(dh32)
-        return dh, dw, db, None, None, None, None
+        return dh, dw, db, None, None, None, None, None
 
 
 def linear_cross_entropy_eval(hidden, weight, bias, labels, padding_idx=-100, chunk_rows=DEFAULT_CHUNK_ROWS):

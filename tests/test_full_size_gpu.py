@@ -298,3 +298,28 @@ def test_relative_attention_workload(dev, monkeypatch):
         assert_close(out[:, col:col + 1], f["outputs"], BF, f"outputs[{col}]", flips=2e-3)
         assert_close(cov[col], f["dropout_results"], BF, f"dropout_results[{col}]")
         assert_close(grads[0][:, col:col + 1], g["dx"], BF, f"dx[{col}]", scale_atol=True)
+
+
+def test_products_with_operands_beyond_four_gib(dev):
+    """Operands of 4.6 and 4.9 GB through the GEMM entry point: the matrix-core loop fed from LDS directly addresses an
+    operand from its tile's first row, so its 32-bit lane offsets hold whatever the operand's size. Row blocks from the
+    start, the 4 GiB boundary and the end of each result against fp64 on those rows."""
+    from nmtgminor_amd.native import linear_gemm
+    g = torch.Generator(device=dev)
+    g.manual_seed(77)
+    m, k, n = 70000, 32768, 128
+    a = torch.randn(m, k, generator=g, device=dev, dtype=torch.bfloat16)           # rows of 64 KiB: 4 GiB ends at row 65536
+    b = (torch.randn(n, k, generator=g, device=dev) / k ** 0.5).to(torch.bfloat16)
+    c = linear_gemm.gemm(a, b, trans_b=True)
+    for r0 in (0, 65400, m - 256):
+        want = a[r0:r0 + 256].double() @ b.double().t()
+        assert_close(c[r0:r0 + 256], want.cpu(), torch.bfloat16, f"C = A B^T, rows from {r0}", scale_atol=True)
+    del a, c
+    kk, mm = 8192, 300000                                                          # A^T B with A [K, M]: rows of 600 KB
+    at = torch.randn(kk, mm, generator=g, device=dev, dtype=torch.bfloat16)
+    bt = (torch.randn(kk, n, generator=g, device=dev) / kk ** 0.5).to(torch.bfloat16)
+    ct = linear_gemm.gemm(at, bt, trans_a=True)
+    assert ct.shape == (mm, n)
+    for c0 in (0, 150000, mm - 256):
+        want = at[:, c0:c0 + 256].double().t() @ bt.double()
+        assert_close(ct[c0:c0 + 256], want.cpu(), torch.bfloat16, f"C = A^T B, rows from {c0}", scale_atol=True)

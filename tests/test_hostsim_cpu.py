@@ -510,15 +510,15 @@ def test_incremental_decoder_layer_with_beam_reordering(mi355x):
 # ----------------------------------------------------------------------------- projection + loss in row chunks
 @pytest.mark.parametrize("dtype", HALVES)
 def test_chunked_projection_loss(mi355x, dtype):
-    tgen.test_chunked_projection_loss_matches_oracle_and_unchunked_operators(CPU, dtype, 40, 64, 250, 16, True, 0.1)
+    tgen.test_chunked_projection_loss_matches_oracle_and_unchunked_operators(CPU, dtype, 40, 64, 250, 16, True, 0.1, True)
     if not SANITIZER_RUN:
-        tgen.test_chunked_projection_loss_matches_oracle_and_unchunked_operators(CPU, dtype, 80, 64, 1000, 32, True, 0.1)
-        tgen.test_chunked_projection_loss_matches_oracle_and_unchunked_operators(CPU, dtype, 33, 64, 2048, 8, True, 0.3)
+        tgen.test_chunked_projection_loss_matches_oracle_and_unchunked_operators(CPU, dtype, 80, 64, 1000, 32, True, 0.1, False)
+        tgen.test_chunked_projection_loss_matches_oracle_and_unchunked_operators(CPU, dtype, 33, 64, 2048, 8, True, 0.3, True)
 
 
 @long_case
 def test_chunked_projection_loss_module_and_validation(mi355x):
-    tgen.test_chunked_projection_loss_matches_oracle_and_unchunked_operators(CPU, F16, 64, 128, 517, 64, False, 0.0)
+    tgen.test_chunked_projection_loss_matches_oracle_and_unchunked_operators(CPU, F16, 64, 128, 517, 64, False, 0.0, False)
     tgen.test_per_row_weights_and_no_gradient_for_frozen_weights(CPU)
     tgen.test_validation_pass_counts_correct_predictions(CPU)
     tgen.test_module_matches_the_reference_loss_assembly(CPU)

@@ -33,12 +33,15 @@ def _case(n, e, v, dtype, bias, seed):
 @pytest.mark.parametrize("n,e,v,chunk,bias,eps", [(80, 64, 1000, 32, True, 0.1),      # 32 + 32 + 16 rows
                                                   (64, 128, 517, 64, False, 0.0),     # one chunk, odd vocabulary
                                                   (33, 64, 2048, 8, True, 0.3)])      # ragged last chunk of one row
-def test_chunked_projection_loss_matches_oracle_and_unchunked_operators(dev, dtype, n, e, v, chunk, bias, eps):
+@pytest.mark.parametrize("kept", [True, False])
+def test_chunked_projection_loss_matches_oracle_and_unchunked_operators(dev, dtype, n, e, v, chunk, bias, eps, kept):
+    """kept: the logits fit the memory budget and stay for the backward (one projection, the gradient written over them);
+    otherwise they are never whole (rows in chunks forward, class slices recomputed backward). Same oracle, same tolerance."""
     h, w, b, y, gl = _case(n, e, v, dtype, bias, 100 + n)
     hd, wd, yd, gd = h.to(dev).requires_grad_(), w.to(dev).requires_grad_(), y.to(dev), gl.to(dev)
     bd = b.to(dev).requires_grad_() if bias else None
-    loss = LinearSoftmaxCrossEntropy.apply(hd, wd, bd, yd, eps, PAD, chunk)
-    loss.backward(gd)
+    loss = LinearSoftmaxCrossEntropy.apply(hd, wd, bd, yd, eps, PAD, chunk, (16 << 30) if kept else 0)
+    loss.backward(gd, retain_graph=kept)
     # the fp32 oracle with the logits rounded where the reference stores them
     want, _, _ = og.generator_loss_fwd(h, w, b, y, eps, PAD, dtype)
     dh, dw, db = og.generator_loss_bwd(gl, h, w, b, y, eps, PAD, dtype)
@@ -50,6 +53,13 @@ def test_chunked_projection_loss_matches_oracle_and_unchunked_operators(dev, dty
         assert_close(bd.grad, db, dtype, "grad of the bias", scale_atol=True)
     pad = y == PAD
     assert pad.any() and (loss.cpu()[pad] == 0).all() and (hd.grad.cpu()[pad] == 0).all()     # exact zeros on padding
+    if kept:
+        # the first backward turned the kept logits into their gradient: a second one over the same graph recomputes
+        first = [t.grad.clone() for t in (hd, wd)]
+        hd.grad = wd.grad = None
+        loss.backward(gd)
+        assert_close(hd.grad, first[0].float().cpu(), dtype, "second backward, states")
+        assert_close(wd.grad, first[1].float().cpu(), dtype, "second backward, weight", scale_atol=True)
     # the unchunked operators on the same device (the GEMM may pick another main loop for the dense, odd-pitched logits
     # tensor than for the 64-element-pitched chunk, so the two agree to rounding, not bit for bit)
     z = linear_gemm.gemm(h.to(dev), w.to(dev), trans_b=True, bias=None if b is None else b.to(dev))
