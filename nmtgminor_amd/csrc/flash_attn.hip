@@ -474,7 +474,10 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
     bool padt = false;
     [[maybe_unused]] uint32_t mdead = 0;
     if constexpr (PAD != 0) {
-      padt = masked_tile<PAD>(a, b, min(group, (a.max_q + 31) / 32 - 1), t);
+      // With the causal flag on top of a mask, a row whose keys up to the diagonal are all masked meets the diagonal's
+      // dead keys in tiles without a masked key and still has the initial m there: every tile takes the masked-tile route
+      // then (the combination is rare; the reference's decoder passes its causal mask as a time mask).
+      padt = masked_tile<PAD>(a, b, min(group, (a.max_q + 31) / 32 - 1), t) || a.causal != 0;
       if (padt) {
 #pragma unroll
         for (int n = 0; n < 2; ++n)
@@ -535,11 +538,10 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
         s[n][r] = pr;
         lsum += pr;
       }
-    if constexpr (PAD != 0) if (edge) {
+    if constexpr (PAD != 0) if (padt) {
       // A row that has met no live key yet still has the initial m, against which a dead score is not small: such
-      // probabilities are set to 0 by hand, in every tile that holds a dead key of any kind (a row whose keys up to the
-      // causal diagonal are all masked meets the diagonal's dead keys in tiles without a masked key). Without a mask,
-      // key 0 is live for every row.
+      // probabilities are set to 0 by hand. (Without masked keys inside the sequence, key 0 is live for every row. Under
+      // the causal flag every tile counts as one with masked keys, see padt above.)
       lsum = 0.f;
 #pragma unroll
       for (int n = 0; n < 2; ++n)
