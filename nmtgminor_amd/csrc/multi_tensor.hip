@@ -6,7 +6,7 @@
 // multi_tensor_scale_kernel.cu:29-113, multi_tensor_axpby_kernel.cu:27-126, multi_tensor_l2norm_kernel.cu:27-232,
 // multi_tensor_l2norm_scale_kernel.cu:28-125; launch machinery multi_tensor_apply.cuh).
 // A model has hundreds of parameter tensors, most of them small: one launch per tensor would be launch-bound, so the
-// tensors' addresses and sizes travel in the kernel arguments (a table of up to MT_MAX tensors, 2 KB) and block b finds
+// tensors' addresses and sizes travel in the kernel arguments (a table of as many tensors as fit the 4 KB of kernel arguments: 84 for the four lists of an Adam step) and block b finds
 // its tensor and its 32768-element chunk from the table's prefix of block counts. All three passes are bandwidth bound:
 // Adam reads g, p, m, v and writes p, m, v (28 B per fp32 element), scale reads and writes once, the norm reads once.
 // 16-byte accesses whenever a tensor's pointers are 16-byte aligned (chunks start on multiples of 32768 elements), with
@@ -20,16 +20,18 @@
 namespace nmtg {
 namespace {
 
-constexpr int MT_MAX = 48;          // tensors per launch
-constexpr int MT_CHUNK = 32768;     // elements per block: a transformer-base parameter list then gives ~7 blocks per CU, all resident at once
+// tensors per launch for a table of L pointer lists: 8 L + 12 bytes per tensor inside the 4 KB of kernel arguments,
+// beside the kernel's scalars
+template <int L> constexpr int mt_max() { return L >= 4 ? 84 : L == 3 ? 100 : L == 2 ? 128 : 160; }
+constexpr int MT_CHUNK = 8192;      // elements per block
 constexpr int MT_THREADS = 256;
 constexpr int MT_WAVES = MT_THREADS / kWave;
 
 template <int L>
 struct MtTable {
-  void* addr[L][MT_MAX];
-  int64_t size[MT_MAX];
-  int first_block[MT_MAX + 1];      // prefix sums of the tensors' chunk counts
+  void* addr[L][mt_max<L>()];
+  int64_t size[mt_max<L>()];
+  int first_block[mt_max<L>() + 1];   // prefix sums of the tensors' chunk counts
   int count;
 };
 
@@ -75,11 +77,7 @@ __global__ __launch_bounds__(MT_THREADS) void mt_adam_kernel(const MtTable<4> ta
   const bool vec = ((reinterpret_cast<uintptr_t>(g) | reinterpret_cast<uintptr_t>(p) | reinterpret_cast<uintptr_t>(m) |
                      reinterpret_cast<uintptr_t>(v)) & 15u) == 0;
   const int nvec = vec ? n / EPV : 0;
-  for (int i = threadIdx.x; i < nvec; i += MT_THREADS) {
-    // four loads in flight before the first conversion
-    pack<T, EPV> rg = load_raw<T, EPV>(g + i * EPV), rp = load_raw<T, EPV>(p + i * EPV), rm = load_raw<T, EPV>(m + i * EPV),
-                 rv = load_raw<T, EPV>(v + i * EPV);
-    pin_raw(rg); pin_raw(rp); pin_raw(rm); pin_raw(rv);
+  auto update = [&](int i, const pack<T, EPV>& rg, const pack<T, EPV>& rp, const pack<T, EPV>& rm, const pack<T, EPV>& rv) {
     float gv[EPV], pv[EPV], mv[EPV], vv[EPV];
     unpack_raw<T, EPV>(rg, gv); unpack_raw<T, EPV>(rp, pv); unpack_raw<T, EPV>(rm, mv); unpack_raw<T, EPV>(rv, vv);
 #pragma unroll
@@ -87,6 +85,25 @@ __global__ __launch_bounds__(MT_THREADS) void mt_adam_kernel(const MtTable<4> ta
     store_pack<T, EPV>(p + i * EPV, pv);
     store_pack<T, EPV>(m + i * EPV, mv);
     store_pack<T, EPV>(v + i * EPV, vv);
+  };
+  int i = threadIdx.x;
+  for (; i + MT_THREADS < nvec; i += 2 * MT_THREADS) {
+    // two vectors of each of the four streams in flight before the first conversion
+    const int k = i + MT_THREADS;
+    pack<T, EPV> rg = load_raw<T, EPV>(g + i * EPV), rp = load_raw<T, EPV>(p + i * EPV), rm = load_raw<T, EPV>(m + i * EPV),
+                 rv = load_raw<T, EPV>(v + i * EPV);
+    pack<T, EPV> sg = load_raw<T, EPV>(g + k * EPV), sp = load_raw<T, EPV>(p + k * EPV), sm = load_raw<T, EPV>(m + k * EPV),
+                 sv = load_raw<T, EPV>(v + k * EPV);
+    pin_raw(rg); pin_raw(rp); pin_raw(rm); pin_raw(rv);
+    pin_raw(sg); pin_raw(sp); pin_raw(sm); pin_raw(sv);
+    update(i, rg, rp, rm, rv);
+    update(k, sg, sp, sm, sv);
+  }
+  for (; i < nvec; i += MT_THREADS) {
+    pack<T, EPV> rg = load_raw<T, EPV>(g + i * EPV), rp = load_raw<T, EPV>(p + i * EPV), rm = load_raw<T, EPV>(m + i * EPV),
+                 rv = load_raw<T, EPV>(v + i * EPV);
+    pin_raw(rg); pin_raw(rp); pin_raw(rm); pin_raw(rv);
+    update(i, rg, rp, rm, rv);
   }
   for (int i = nvec * EPV + threadIdx.x; i < n; i += MT_THREADS) {
     float pv = elem<T>::to_float(p[i]), mv = elem<T>::to_float(m[i]), vv = elem<T>::to_float(v[i]);
@@ -259,7 +276,7 @@ __global__ __launch_bounds__(MT_THREADS) void mt_norm_final_kernel(const float* 
 
 int64_t chunks_of(int64_t n) { return (n + MT_CHUNK - 1) / MT_CHUNK; }
 
-// Walks the tensor list in groups that fit one table (at most MT_MAX tensors, at most 2^30 blocks); empty tensors take
+// Walks the tensor list in groups that fit one table (at most mt_max<L>() tensors, at most 2^30 blocks); empty tensors take
 // no blocks. launch(table, blocks, first tensor of the group, first block of the group).
 template <int L, typename F>
 int mt_for_groups(int n_tensors, const void* const* const (&lists)[L], const int64_t* sizes, F launch) {
@@ -269,7 +286,7 @@ int mt_for_groups(int n_tensors, const void* const* const (&lists)[L], const int
     MtTable<L> tab{};
     int64_t blocks = 0;
     int cnt = 0;
-    while (t0 + cnt < n_tensors && cnt < MT_MAX && blocks + chunks_of(sizes[t0 + cnt]) <= (int64_t(1) << 30)) {
+    while (t0 + cnt < n_tensors && cnt < mt_max<L>() && blocks + chunks_of(sizes[t0 + cnt]) <= (int64_t(1) << 30)) {
       for (int l = 0; l < L; ++l) tab.addr[l][cnt] = const_cast<void*>(lists[l][t0 + cnt]);
       tab.size[cnt] = sizes[t0 + cnt];
       tab.first_block[cnt] = static_cast<int>(blocks);
@@ -278,7 +295,7 @@ int mt_for_groups(int n_tensors, const void* const* const (&lists)[L], const int
     }
     if (cnt == 0) return fail(NMTG_ERR_INVALID, "multi_tensor: tensor %d has too many elements for one launch", t0);
     tab.first_block[cnt] = static_cast<int>(blocks);
-    for (int i = cnt + 1; i <= MT_MAX; ++i) tab.first_block[i] = static_cast<int>(blocks);
+    for (int i = cnt + 1; i <= mt_max<L>(); ++i) tab.first_block[i] = static_cast<int>(blocks);
     tab.count = cnt;
     if (int rc = launch(tab, static_cast<int>(blocks), t0, block_base)) return rc;
     block_base += blocks;

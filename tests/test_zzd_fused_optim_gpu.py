@@ -20,8 +20,9 @@ from util import assert_close, load_golden
 
 pytestmark = pytest.mark.gpu
 D = torch.float64
-# sizes around the 16-byte vector width, around one 65536-element chunk, an empty tensor, and more than 48 tensors
-SIZES = [1, 7, 64, 1000, 65536, 65537, 0, 200003] + [33 + i for i in range(50)]
+# sizes around the 16-byte vector width, around one 8192-element chunk, an empty tensor, and more tensors than any
+# launch's table holds (84 to 160, by the number of lists)
+SIZES = [1, 7, 64, 1000, 65536, 65537, 0, 200003, 8191, 8192, 8193] + [33 + i for i in range(170)]
 
 
 def _tensors(sizes, dtype, seed, scale=1.0, positive=False):
@@ -222,7 +223,7 @@ def test_fused_optim_golden_fixture(dev, name, adam_w):
 def test_randomly_drawn_tensor_lists(dev, seed):
     rnd = random.Random(seed)
     dtype = rnd.choice([torch.float32, torch.bfloat16, torch.float16])
-    sizes = [rnd.choice([0, 1, 3, 8, 100, 4097, 32767, 32768, 32769, 70001]) for _ in range(rnd.choice([1, 2, 47, 48, 49, 97]))]
+    sizes = [rnd.choice([0, 1, 3, 8, 100, 4097, 8191, 8192, 8193, 70001]) for _ in range(rnd.choice([1, 2, 84, 85, 129, 161, 170]))]
     case = f"seed {seed}: {dtype}, {len(sizes)} tensors, {sum(sizes)} elements"
     g, p = _tensors(sizes, dtype, seed), _tensors(sizes, dtype, seed + 1)
     m, v = _tensors(sizes, dtype, seed + 2, 0.1), _tensors(sizes, dtype, seed + 3, 0.01, positive=True)
