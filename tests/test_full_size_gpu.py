@@ -323,3 +323,58 @@ def test_products_with_operands_beyond_four_gib(dev):
     for c0 in (0, 150000, mm - 256):
         want = at[:, c0:c0 + 256].double().t() @ bt.double()
         assert_close(ct[c0:c0 + 256], want.cpu(), torch.bfloat16, f"C = A^T B, rows from {c0}", scale_atol=True)
+
+
+def test_projection_and_loss_workload(dev):
+    """The benchmark's projection + loss (16384 positions x 1024 -> 250054 classes, eps 0.1, padding index 1) with the
+    logits kept once (8.2 GB) and without them (rows in chunks forward, class slices recomputed backward). Losses and the
+    gradient of the states on sampled rows (rows are independent given the weights), the weight gradient on sampled
+    classes (a class's row of it is a sum over all positions of that class's logit gradients, which the oracle forms
+    from the fp64 logits of that class and the log-sum-exp checked on the sampled rows), zeros on padding, and the two
+    memory policies against each other."""
+    from nmtgminor_amd.modules.generator_loss import LinearSoftmaxCrossEntropy
+    N, E, V, eps, pad_idx = 16384, 1024, 250054, 0.1, 1
+    d = inputs.xentropy_inputs(N, V, with_logits=False)
+    labels, gl = d["labels"], d["grad_loss"]
+    g = torch.Generator(device=dev)
+    g.manual_seed(1006)
+    h = torch.randn(N, E, generator=g, device=dev).to(BF)
+    w = (torch.randn(V, E, generator=g, device=dev) / E ** 0.5).to(BF)
+
+    def run(budget):
+        hd, wd = h.clone().requires_grad_(), w.clone().requires_grad_()
+        losses = LinearSoftmaxCrossEntropy.apply(hd, wd, None, labels.to(dev), eps, pad_idx, 4096, budget)
+        losses.backward(gl.to(dev))
+        return losses.detach(), hd.grad, wd.grad
+
+    kept = run(16 << 30)
+    rows = torch.tensor([0, 1, 4097, 12345, N - 1])
+    rows = rows[labels[rows] != pad_idx] if (labels[rows] != pad_idx).any() else rows
+    hc, wc = h.cpu(), w.cpu()
+    z = (hc[rows].to(D) @ wc.to(D).t()).to(BF)                                   # the logits as stored
+    lo, lseo = oxe.xentropy_fwd(z, labels[rows], eps, pad_idx, D)
+    assert_close(kept[0][rows.to(dev)], lo, BF, "losses", atol=2e-3)
+    dz = oxe.xentropy_bwd(gl[rows], z, lseo, labels[rows], eps, pad_idx, D).to(BF).to(D)
+    assert_close(kept[1][rows.to(dev)], dz @ wc.to(D), BF, "gradient of the states, sampled rows")
+    # sampled classes: the most frequent target, a rare one, the last class
+    classes = torch.tensor([int(labels[labels != pad_idx].mode().values), 7, V - 1])
+    zc = (hc.to(D) @ wc[classes].to(D).t()).to(BF).to(D)                         # [N, 3]
+    # per-row log-sum-exp over all classes, from the device's logits of the kept run's twin: recompute it in slices
+    lse = torch.empty(N, dtype=torch.float64)
+    for r0 in range(0, N, 2048):
+        zz = (h[r0:r0 + 2048].float() @ w.float().t()).to(BF).float()
+        lse[r0:r0 + 2048] = torch.logsumexp(zz, 1).double().cpu()
+    assert (lse[rows] - lseo).abs().max() < 2e-3
+    real = (labels != pad_idx).to(D)
+    p = torch.exp(zc - lse[:, None])
+    target = (labels[:, None] == classes[None, :]).to(D)
+    dzc = ((p - eps / V - (1 - eps) * target) * (gl.to(D) * real)[:, None]).to(BF).to(D)
+    assert_close(kept[2][classes.to(dev)], dzc.t() @ hc.to(D), BF, "weight gradient, sampled classes", scale_atol=True)
+    pad = (labels == pad_idx).to(dev)
+    assert (kept[0][pad] == 0).all() and int(kept[1][pad].ne(0).sum()) == 0
+    assert torch.isfinite(kept[2]).all()
+    lean = run(0)
+    assert_close(lean[0], kept[0].cpu(), BF, "losses, the two memory policies", atol=2e-3)
+    assert_close(lean[1], kept[1].float().cpu(), BF, "gradient of the states, the two memory policies")
+    from util import rel_err
+    assert rel_err(lean[2], kept[2].float().cpu()) < 5e-3
