@@ -505,7 +505,7 @@ class DecodeStepWL(Workload):
     dtype = "bf16"
     description = ("one incremental decoding step of the decoder's attention, bf16: cross-attention of 1 new position over "
                    "1500 cached encoder keys / values (B=32 hypotheses, E=1024, 16 heads, key-padding lengths U[750,1500]) + "
-                   "self-attention of the new position over 127 cached positions (cache grown by concatenation, as the reference does)")
+                   "self-attention of the new position over 127 cached positions (the step starts from a cache tensor without room to grow, so it copies the cache once, as the reference's concatenation does)")
     TK, TPREV, B, E, H = 1500, 127, 32, 1024, 16
 
     def setup(self, dev):

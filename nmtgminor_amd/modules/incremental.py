@@ -89,7 +89,7 @@ def _key_mask(mask, use_time_mask, b, tk, device):
 
 
 def _append(cache, name, row):
-    """cache[name] [T, B, E] with `row` [1, B, E] behind it. The reference concatenates (a copy of the whole cache per
+    """cache[name] [T, B, E] with `row` (the B * E values of one position) behind it. The reference concatenates (a copy of the whole cache per
     step, self_attention_func.py:165-169). Here the rows live in a buffer with room to grow and cache[name] is its
     leading slice, which carries the buffer as an attribute (the dict keeps exactly the reference's entries): while the
     caller leaves that tensor in place, a step writes one row. A caller that replaces cache[name] (beam search re-indexes
@@ -103,7 +103,7 @@ def _append(cache, name, row):
     if not in_place:
         buf = old.new_empty((max(2 * n, n + 64),) + tuple(old.shape[1:]))
         buf[:n].copy_(old)
-    buf[n:n + 1].copy_(row)
+    buf[n:n + 1].view(row.shape).copy_(row)       # `row` may be the strided [1, B*H, D] slice of the projection
     grown = buf[:n + 1]
     grown._nmtg_buffer = buf
     return grown
@@ -119,14 +119,16 @@ def self_attn_step(heads, inputs, input_weights, output_weights, input_biases, o
     d = e // heads
     lin = _project(inputs, input_weights, input_biases).view(t_new, b * heads, 3, d)
     queries = lin[:, :, 0, :].reshape(t_new, b, e)
-    keys = lin[:, :, 1, :].reshape(t_new, b, e)
-    values = lin[:, :, 2, :].reshape(t_new, b, e)
     first = not ("k" in cache and "v" in cache)
     if not first:
         if t_new != 1:
             raise NotImplementedError("incremental self-attention: one new position per step once the cache is filled")
-        keys = _append(cache, "k", keys)
-        values = _append(cache, "v", values)
+        # the new row goes from the interleaved projection straight into the cache (one copy each)
+        keys = _append(cache, "k", lin[:, :, 1, :])
+        values = _append(cache, "v", lin[:, :, 2, :])
+    else:
+        keys = lin[:, :, 1, :].reshape(t_new, b, e)
+        values = lin[:, :, 2, :].reshape(t_new, b, e)
     cache["k"], cache["v"] = keys, values
     if first and t_new > 1:
         # a prefix of several positions: the full-sequence kernel with its mask, fed with the same projection
