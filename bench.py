@@ -504,7 +504,7 @@ class DecodeStepWL(Workload):
     bound = "hbm"
     dtype = "bf16"
     description = ("one incremental decoding step of the decoder's attention, bf16: cross-attention of 1 new position over "
-                   "1500 cached encoder keys / values (B=32 hypotheses, E=1024, 16 heads, key-padding lengths U[750,1500]) + "
+                   "1500 cached encoder keys / values (B=32 hypotheses, E=1024, 16 heads, key-padding lengths U[750,1500]: bytes counted over the live keys) + "
                    "self-attention of the new position over 127 cached positions (the step starts from a cache tensor without room to grow, so it copies the cache once, as the reference's concatenation does)")
     TK, TPREV, B, E, H = 1500, 127, 32, 1024, 16
 
@@ -523,6 +523,8 @@ class DecodeStepWL(Workload):
                              a["pad_mask"], self.cross_cache)                       # fills c_k / c_v: not part of a step
         inc.self_attn_step(self.H, sa["x"][:self.TPREV], sa["w_in"], sa["w_out"], sa["b_in"], sa["b_out"], None, self_cache, False)
         self.prev_k, self.prev_v = self_cache["k"], self_cache["v"]
+        # the cache rows a step has to read: the live keys of every sentence (the kernel does not read a sentence's padding)
+        self.live_keys = int((~d["pad_mask"].bool()).sum())
 
     def step(self):
         a, sa = self.a, self.s
@@ -535,7 +537,7 @@ class DecodeStepWL(Workload):
 
     def _bytes(self):
         tk, tp, b, e, h = self.TK, self.TPREV, self.B, self.E, self.H
-        cross = 2 * tk * b * e * 2 + 2 * e * e * 2 + b * h * tk * 2 + 4 * b * e * 2         # K, V cache; W_q, W_out; probabilities; rows
+        cross = 2 * self.live_keys * e * 2 + 2 * e * e * 2 + b * h * tk * 2 + 4 * b * e * 2  # live K, V rows; W_q, W_out; probabilities; rows
         self_ = 2 * (tp + tp + 1) * b * e * 2 + 4 * e * e * 2 + b * h * (tp + 1) * 2 + 5 * b * e * 2   # cache read + rewritten
         return cross + self_
 
@@ -545,7 +547,7 @@ class DecodeStepWL(Workload):
     def kernel_work(self):
         tk, tp, b, e, h = self.TK, self.TPREV, self.B, self.E, self.H
         # the two launches of the cache-streaming kernel: keys and values read once, probabilities written, a row in and out
-        return {"attn_decode": 2 * (tk + tp + 1) * b * e * 2 + b * h * (tk + tp + 1) * 2 + 4 * b * e * 2}
+        return {"attn_decode": 2 * (self.live_keys + (tp + 1) * b) * e * 2 + b * h * (tk + tp + 1) * 2 + 4 * b * e * 2}
 
     def cpu_baseline(self):
         from oracle import attention as o

@@ -468,6 +468,8 @@ int nmtg_flash_attn_batched_bwd(const void* dout, const void* q, const void* k, 
  * stride_t = B * E, stride_b = E); key_mask [batch, tk] (1 = masked key) or NULL.
  * probs [batch * heads, tk] = softmax(round(scale * q . k)) in the tensors' 16-bit type (rows without
  * a live key: zeros), context [batch, heads * head_dim] (row stride ctx_stride_b) = probs x values.
+ * Keys and values behind a sentence's last unmasked key are not read (what the cache holds there,
+ * NaN included, does not reach the results; the reference's 0 x NaN would).
  * head_dim 32, 64 or 128; tk <= 16384; fp16 / bf16; strides multiples of 8 elements.
  * ------------------------------------------------------------------------------------------ */
 int nmtg_attn_decode(const void* q, int64_t q_stride_b, const void* keys, int64_t k_stride_t,

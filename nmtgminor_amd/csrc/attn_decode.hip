@@ -60,13 +60,24 @@ __global__ __launch_bounds__(DEC_THREADS) void attn_decode_kernel(DecArgs a) {
   const T* vb = static_cast<const T*>(a.values) + b * a.v_sb + head_off;
   const uint8_t* km = a.kmask ? a.kmask + static_cast<int64_t>(b) * a.tk : nullptr;
 
+  // Keys behind the sentence's last live one (the padding of a shorter sentence) have probability zero whatever the
+  // cache holds there: their keys and values are not read.
+  int live = a.tk;
+  if (km != nullptr) {
+    int last = 0;
+    for (int j = tid; j < a.tk; j += DEC_THREADS)
+      if (!km[j]) last = j + 1;
+    live = static_cast<int>(block_reduce(static_cast<float>(last), true, red));   // <= 16384: exact in fp32
+    for (int j = live + tid; j < a.tk; j += DEC_THREADS) sc[j] = -INFINITY;
+  }
+
   // ---- scores ----
-  for (int j0 = 0; j0 < a.tk; j0 += RPS * U) {
+  for (int j0 = 0; j0 < live; j0 += RPS * U) {
     pack<T, 8> raw[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int j = j0 + u * RPS + slot;
-      raw[u] = load_raw<T, 8>(kb + static_cast<int64_t>(j < a.tk ? j : 0) * a.k_st);
+      raw[u] = load_raw<T, 8>(kb + static_cast<int64_t>(j < live ? j : 0) * a.k_st);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -78,7 +89,7 @@ __global__ __launch_bounds__(DEC_THREADS) void attn_decode_kernel(DecArgs a) {
       for (int e = 0; e < 4; ++e) dot = dot2<T>(qw[e], kw[e], dot);
 #pragma unroll
       for (int d = 1; d < LPR; d <<= 1) dot += __shfl_xor(dot, d);
-      if (c == 0 && j < a.tk) sc[j] = (km != nullptr && km[j]) ? -INFINITY : round_to<T>(dot * a.scale);
+      if (c == 0 && j < live) sc[j] = (km != nullptr && km[j]) ? -INFINITY : round_to<T>(dot * a.scale);
     }
   }
   __syncthreads();
@@ -107,17 +118,17 @@ __global__ __launch_bounds__(DEC_THREADS) void attn_decode_kernel(DecArgs a) {
 
   // ---- context = probabilities x values ----
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  for (int j0 = 0; j0 < a.tk; j0 += RPS * U) {
+  for (int j0 = 0; j0 < live; j0 += RPS * U) {
     pack<T, 8> raw[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int j = j0 + u * RPS + slot;
-      raw[u] = load_raw<T, 8>(vb + static_cast<int64_t>(j < a.tk ? j : 0) * a.v_st);
+      raw[u] = load_raw<T, 8>(vb + static_cast<int64_t>(j < live ? j : 0) * a.v_st);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int j = j0 + u * RPS + slot;
-      const float p = j < a.tk ? sc[j] : 0.f;
+      const float p = j < live ? sc[j] : 0.f;
       float vv[8];
       unpack_raw<T, 8>(raw[u], vv);
 #pragma unroll

@@ -501,6 +501,11 @@ def test_incremental_decoding(mi355x, dtype):
     tinc.test_cross_attention_with_cached_encoder_states(CPU, dtype)
 
 
+@pytest.mark.parametrize("d", [32, 64, 128])
+def test_decoding_kernel_skips_the_padded_tail_of_the_cache(d):
+    tinc.test_one_position_does_not_read_the_cache_behind_a_sentences_last_live_key(CPU, d)
+
+
 @long_case
 def test_incremental_decoder_layer_with_beam_reordering(mi355x):
     tinc.test_self_attention_step_by_step(CPU, F16, 1)

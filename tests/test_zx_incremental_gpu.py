@@ -131,6 +131,41 @@ def test_one_position_against_the_longest_cache_at_head_dimension_128(dev):
     assert_close(ctx.view(b, h, d), torch.einsum("bht,tbhd->bhd", pr.to(dtype).to(D), v4), dtype, "context")
 
 
+@pytest.mark.parametrize("d", [32, 64, 128])
+def test_one_position_does_not_read_the_cache_behind_a_sentences_last_live_key(dev, d):
+    """Key masks of every kind in one batch: padding at the end, a hole in the middle, both, a sentence without any live
+    key, a sentence with every key live. The cache rows behind each sentence's last live key hold NaN: the kernel must
+    not read them (their probability is zero whatever they hold), and the row still equals the masked softmax in fp64."""
+    from nmtgminor_amd.modules import incremental
+    tk, b, h, dtype = 700, 5, 2, torch.bfloat16
+    e = h * d
+    g = torch.Generator().manual_seed(98)
+    q = torch.randn(1, b, e, generator=g).to(dtype)
+    keys = torch.randn(tk, b, e, generator=g).to(dtype)
+    values = torch.randn(tk, b, e, generator=g).to(dtype)
+    pad = torch.zeros(b, tk, dtype=torch.bool)
+    pad[0, 333:] = True
+    pad[1, 100:164] = True
+    pad[2, 7] = True
+    pad[2, 699] = True
+    pad[3, :] = True
+    live = [333, tk, 699, 0, tk]
+    kd, vd = keys.clone(), values.clone()
+    for bi, n in enumerate(live):
+        kd[n:, bi] = float("nan")
+        vd[n:, bi] = float("nan")
+    assert incremental._decode_ok(q.to(dev), kd.to(dev), vd.to(dev), h)
+    ctx, probs = incremental._decode_core(h, q.to(dev), kd.to(dev), vd.to(dev), pad.to(dev))
+    q4, k4, v4 = q.view(b, h, d).to(D), keys.view(tk, b, h, d).to(D), values.view(tk, b, h, d).to(D)
+    s = (torch.einsum("bhd,tbhd->bht", q4, k4) * d ** -0.5).to(dtype).to(D)
+    s = s.masked_fill(pad.view(b, 1, tk), float("-inf"))
+    pr = torch.softmax(s, -1)
+    pr[3] = 0.0                                     # no live key: zeros, not the NaN of an empty softmax
+    assert_close(probs.view(b, h, tk), pr, dtype, "probabilities", atol=1e-5)
+    assert (probs.view(b, h, tk).cpu()[pad.view(b, 1, tk).expand(b, h, tk)] == 0).all()
+    assert_close(ctx.view(b, h, d), torch.einsum("bht,tbhd->bhd", pr.to(dtype).to(D), v4), dtype, "context")
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_cross_attention_with_cached_encoder_states(dev, dtype):
     tq, tk, b, e, h = 7, 37, 3, 128, 4
