@@ -64,9 +64,15 @@ build, test_file, runtime, log = sys.argv[1:5]
 env = dict(os.environ, HOSTSIM_SANITIZE="1")
 rc = subprocess.run([sys.executable, build, "--if-stale"], env=env, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL).returncode
 if rc == 0:
-    env.update(LD_PRELOAD=runtime, ASAN_OPTIONS="detect_leaks=0:detect_stack_use_after_return=0")
+    env.update(LD_PRELOAD=runtime, ASAN_OPTIONS="detect_leaks=0:detect_stack_use_after_return=0", OMP_NUM_THREADS="2")
+    spread = []          # the checks are independent of each other: four worker processes where pytest-xdist is there
+    try:
+        import xdist
+        spread = ["-n", "4"]
+    except ImportError:
+        pass
     with open(log, "w") as out:
-        rc = subprocess.run([sys.executable, "-m", "pytest", test_file, "-x", "-q", "-p", "no:cacheprovider"], env=env,
+        rc = subprocess.run([sys.executable, "-m", "pytest", test_file, "-x", "-q", "-p", "no:cacheprovider"] + spread, env=env,
                             stdout=out, stderr=subprocess.STDOUT, cwd=os.path.dirname(os.path.dirname(test_file))).returncode
 sys.exit(rc)
 """
