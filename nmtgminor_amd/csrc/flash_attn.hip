@@ -178,6 +178,18 @@ __device__ __forceinline__ void load_resident(uint4 (&f)[D / 16], const T* base,
   for (int s = 0; s < D / 16; ++s) f[s] = row < len ? *reinterpret_cast<const uint4*>(p + 16 * s) : make_uint4(0, 0, 0, 0);
 }
 
+// Touches the rows that stay in registers for a whole tile loop (the queries of the inference kernel), in front of the
+// loop and outside any branch. They are loaded under conditions, and without a use that the compiler sees on every path
+// it repeats the wait for them inside the loop, behind the loads of the next tile: every tile then waits for its own
+// prefetch. Not for the training kernels: behind a statement like this one (or a wait instruction of our own) the
+// compiler no longer reads wave-uniform values (tile classes, dropout bits) through the scalar cache but with vector
+// loads, each waited for on the spot.
+template <int N>
+__device__ __forceinline__ void registers_landed(const uint4 (&f)[N]) {
+#pragma unroll
+  for (int i = 0; i < N; ++i) asm volatile("" ::"v"(f[i].x), "v"(f[i].y), "v"(f[i].z), "v"(f[i].w));
+}
+
 // Where sequence b lies and how long it is. Packed calls read the cumulative lengths. Batch-strided calls (no cumulative
 // lengths) give every sequence max_q queries and max_k keys, b * *_sb elements into each tensor; a key padding mask cuts
 // the keys at the last live one, and masked keys below that are handled tile by tile (pad_tile()).
@@ -444,12 +456,13 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
   [[maybe_unused]] const int qr = min(qrow, lq - 1);   // the row whose time-mask bytes this lane reads
 
   Staged<D> sk, sv;
-  if (ntiles > 0) {
-    sk.load(kb, a.k_st, 0, lk);
-    sv.load(vb, a.v_st, 0, lk);
-    sk.store_rows(lds_raw);
-    sv.store_transposed(lds_raw + IMG);
-  }
+  // (not under `ntiles > 0`: rows past the end load nothing and store zeros, and a wait that lies on every path into
+  // the loop lets the compiler know there that the resident rows above have landed; behind a branch it would repeat
+  // their wait inside the loop, after the next tile's loads, and every tile would wait for its own prefetch)
+  sk.load(kb, a.k_st, 0, lk);
+  sv.load(vb, a.v_st, 0, lk);
+  sk.store_rows(lds_raw);
+  sv.store_transposed(lds_raw + IMG);
   __syncthreads();
   for (int t = 0; t < ntiles; ++t) {
     const uint8_t* kimg = lds_raw + (t & 1) * 2 * IMG;
@@ -643,13 +656,11 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dq_kern
 
   // per buffer: K row image, K transposed image, V row image
   Staged<D> sk, sv;
-  if (ntiles > 0) {
-    sk.load(kb, a.k_st, 0, lk);
-    sv.load(vb, a.v_st, 0, lk);
-    sk.store_rows(lds_raw);
-    sk.store_transposed(lds_raw + IMG);
-    sv.store_rows(lds_raw + 2 * IMG);
-  }
+  sk.load(kb, a.k_st, 0, lk);          // on every path, as in the forward kernel
+  sv.load(vb, a.v_st, 0, lk);
+  sk.store_rows(lds_raw);
+  sk.store_transposed(lds_raw + IMG);
+  sv.store_rows(lds_raw + 2 * IMG);
   __syncthreads();
   for (int t = 0; t < ntiles; ++t) {
     const uint8_t* kimg = lds_raw + (t & 1) * 3 * IMG;
@@ -822,12 +833,10 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dkv_ker
     sg.store_transposed(buf + 3 * IMG);
     if (threadIdx.x < 2 * FA_TILE) reinterpret_cast<float*>(buf + 4 * IMG)[threadIdx.x] = st_val;
   };
-  if (t0 < ntiles) {
-    sq.load(qb, a.q_st, t0 * FA_TILE, lq);
-    sg.load(gb, a.do_st, t0 * FA_TILE, lq);
-    load_stats(t0);
-    store_tile(lds_raw + (t0 & 1) * BUF);
-  }
+  sq.load(qb, a.q_st, t0 * FA_TILE, lq);          // on every path, as in the forward kernel
+  sg.load(gb, a.do_st, t0 * FA_TILE, lq);
+  load_stats(t0);
+  store_tile(lds_raw + (t0 & 1) * BUF);
   __syncthreads();
   for (int t = t0; t < ntiles; ++t) {
     const uint8_t* qimg = lds_raw + (t & 1) * BUF;
@@ -957,22 +966,28 @@ template <> __device__ __forceinline__ float unpack_hi<f16_t>(uint32_t w) {
 }
 
 // mask bytes (1 = masked) of the four keys key0 .. key0 + 3 for this lane's query, keys past the end count as masked.
-// The load is unconditional (from a clamped address) and the eight words of a tile are requested together, ahead of
-// the products: as loads inside branches they were waited for one by one.
+// The load is unconditional (from a clamped address) and the eight words of a tile are requested together. Two steps,
+// so that a caller can ask for a tile's words early and touch them (which is where the wait for the load lands) late:
+// the load from the clamped address, then the words of keys past the end.
 template <int MASK>
-__device__ __forceinline__ uint32_t mask_word(const AttnProbsCall& a, int b, int qrow, int key0) {
-  if constexpr (MASK == 0) return key0 < a.tk ? 0u : 0x01010101u;
+__device__ __forceinline__ uint32_t mask_word_load(const AttnProbsCall& a, int b, int qrow, int key0) {
+  if constexpr (MASK == 0) return 0u;
   const int kc = min(key0, a.tk - 4);                 // tk is a positive multiple of 4
   const int64_t row = MASK == 1 ? b : min(qrow, a.tq - 1);
-  const uint32_t w = *reinterpret_cast<const uint32_t*>(a.mask + row * a.tk + kc);
-  return key0 < a.tk ? w : 0x01010101u;
+  return *reinterpret_cast<const uint32_t*>(a.mask + row * a.tk + kc);
 }
 template <int MASK>
-__device__ __forceinline__ void tile_mask_words(const AttnProbsCall& a, int b, int qrow, int t, int half, uint32_t (&mw)[2][4]) {
+__device__ __forceinline__ void tile_mask_load(const AttnProbsCall& a, int b, int qrow, int t, int half, uint32_t (&mw)[2][4]) {
 #pragma unroll
   for (int n = 0; n < 2; ++n)
 #pragma unroll
-    for (int g = 0; g < 4; ++g) mw[n][g] = mask_word<MASK>(a, b, qrow, t * FA_TILE + 32 * n + 8 * g + 4 * half);
+    for (int g = 0; g < 4; ++g) mw[n][g] = mask_word_load<MASK>(a, b, qrow, t * FA_TILE + 32 * n + 8 * g + 4 * half);
+}
+__device__ __forceinline__ void tile_mask_finish(const AttnProbsCall& a, int t, int half, const uint32_t (&raw)[2][4], uint32_t (&mw)[2][4]) {
+#pragma unroll
+  for (int n = 0; n < 2; ++n)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) mw[n][g] = t * FA_TILE + 32 * n + 8 * g + 4 * half < a.tk ? raw[n][g] : 0x01010101u;
 }
 
 // G groups of four wavefronts share the block's 128 queries and take the key tiles in turn (tile t goes to group
@@ -1019,10 +1034,10 @@ __global__ __launch_bounds__(FA_THREADS * G, (D == 64 && G == 1) ? 2 : 1) void a
     __syncthreads();                                        // stats is written again after pass 1
   }
 
-  // the tile's 32 scores of this lane, rounded and masked
-  auto tile_scores = [&](const uint8_t* kimg, int t, acc16_t (&s)[2]) {
-    uint32_t mw[2][4];
-    tile_mask_words<MASK>(a, b, qrow, t, half, mw);
+  // the tile's 32 scores of this lane, rounded and masked. The mask words of a tile are requested one round ahead, behind
+  // the loads of that tile's keys (values): vector loads return in order, so a mask word asked for at its tile would be
+  // waited for together with the next tile's keys, and every round would last a whole memory latency.
+  auto tile_scores = [&](const uint8_t* kimg, const uint32_t (&mw)[2][4], acc16_t (&s)[2]) {
 #pragma unroll
     for (int n = 0; n < 2; ++n)
 #pragma unroll
@@ -1050,18 +1065,33 @@ __global__ __launch_bounds__(FA_THREADS * G, (D == 64 && G == 1) ? 2 : 1) void a
   float m = PA_DEAD, l = 0.f;
   Staged<D> sk, sv;
   const int live_rounds = (live_tiles + G - 1) / G;
+  uint32_t mw[2][4], mw_next[2][4];
+  // (the empty statement keeps the compiler from working on the words, and so from waiting for them, any earlier)
+  auto take_next_mask = [&](int t) {
+#pragma unroll
+    for (int n = 0; n < 2; ++n)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) asm volatile("" : "+v"(mw_next[n][g]));
+    tile_mask_finish(a, t, half, mw_next, mw);
+  };
+  tile_mask_load<MASK>(a, b, qrow, group, half, mw_next);   // clamped addresses: any tile index may be asked for
+  tile_mask_finish(a, group, half, mw_next, mw);
   if (group < live_tiles) {
     sk.load(kb, a.k_st, group * FA_TILE, a.tk);
     sk.store_rows(tiles);
   }
+  registers_landed(qf);
   __syncthreads();
   for (int it = 0; it < live_rounds; ++it) {
     const int t = it * G + group;
     const uint8_t* kimg = tiles + (it & 1) * 2 * IMG;
-    if (t + G < live_tiles) sk.load(kb, a.k_st, (t + G) * FA_TILE, a.tk);
+    if (t + G < live_tiles) {
+      sk.load(kb, a.k_st, (t + G) * FA_TILE, a.tk);
+      tile_mask_load<MASK>(a, b, qrow, t + G, half, mw_next);
+    }
     if (t < live_tiles) {
       acc16_t s[2];
-      tile_scores(kimg, t, s);
+      tile_scores(kimg, mw, s);
       float mx = s[0][0];
 #pragma unroll
       for (int n = 0; n < 2; ++n)
@@ -1077,7 +1107,10 @@ __global__ __launch_bounds__(FA_THREADS * G, (D == 64 && G == 1) ? 2 : 1) void a
       l = l * fast_exp2((m - m_new) * FA_LOG2E) + sum;
       m = m_new;
     }
-    if (t + G < live_tiles) sk.store_rows(tiles + ((it + 1) & 1) * 2 * IMG);
+    if (t + G < live_tiles) {
+      sk.store_rows(tiles + ((it + 1) & 1) * 2 * IMG);
+      take_next_mask(t + G);
+    }
     __syncthreads();
   }
   l = pair_sum(l);
@@ -1108,12 +1141,15 @@ __global__ __launch_bounds__(FA_THREADS * G, (D == 64 && G == 1) ? 2 : 1) void a
   for (int i = 0; i < D / 32; ++i)
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
+  tile_mask_load<MASK>(a, b, qrow, group, half, mw_next);
+  tile_mask_finish(a, group, half, mw_next, mw);
   if (group < live_tiles) {
     sk.load(kb, a.k_st, group * FA_TILE, a.tk);
     sv.load(vb, a.v_st, group * FA_TILE, a.tk);
     sk.store_rows(tiles);
     sv.store_transposed(tiles + IMG);
   }
+  registers_landed(qf);
   __syncthreads();
   T* prow = static_cast<T*>(a.probs) + (static_cast<int64_t>(b) * a.heads + h) * a.tq * a.tk;
   // the tiles behind the last live key: zeros, no arithmetic (every wavefront of the block takes its share of them)
@@ -1131,10 +1167,11 @@ __global__ __launch_bounds__(FA_THREADS * G, (D == 64 && G == 1) ? 2 : 1) void a
     if (t + G < live_tiles) {
       sk.load(kb, a.k_st, (t + G) * FA_TILE, a.tk);
       sv.load(vb, a.v_st, (t + G) * FA_TILE, a.tk);
+      tile_mask_load<MASK>(a, b, qrow, t + G, half, mw_next);
     }
     if (t < live_tiles) {
       acc16_t s[2];
-      tile_scores(kimg, t, s);
+      tile_scores(kimg, mw, s);
 #pragma unroll
       for (int n = 0; n < 2; ++n)
 #pragma unroll
@@ -1179,6 +1216,7 @@ __global__ __launch_bounds__(FA_THREADS * G, (D == 64 && G == 1) ? 2 : 1) void a
       uint8_t* nk = tiles + ((it + 1) & 1) * 2 * IMG;
       sk.store_rows(nk);
       sv.store_transposed(nk + IMG);
+      take_next_mask(t + G);
     }
     __syncthreads();
   }
