@@ -412,15 +412,17 @@ int nmtg_flash_attn_bwd(const void* dout, const void* q, const void* k, const vo
  * key_padding_mask: NULL, or uint8 [batch, len_k], 1 = masked, any pattern. A query whose keys are
  * all masked has out = 0 and softmax_lse = -inf (the reference's softmax yields NaN there).
  * key_info: with a mask, device workspace of nmtg_flash_attn_key_info_bytes(batch, len_k) bytes,
- * 4-byte aligned; a small kernel ahead of the others writes each sequence's last live key and
- * which 64-key tiles hold masked keys in front of it (only those tiles read the mask again).
+ * 4-byte aligned; a small kernel ahead of the others writes each sequence's last live key,
+ * which 64-key tiles hold masked keys in front of it, and the mask of those tiles packed to bits
+ * (the attention kernels read the packed words, not the mask).
  * time_mask: NULL, or uint8 [len_q, len_k], 1 = masked, shared by every sequence and head (the
  * reference's use_time_mask form; any pattern, a causal one included); not together with
  * key_padding_mask. time_info: with it, device workspace of
  * nmtg_flash_attn_time_info_bytes(len_q, len_k) bytes, 4-byte aligned: a small kernel classifies
  * the mask by patches of 32 x 64 (no masked element / some / all) for both kernel orientations, the
- * attention kernels stop at the last key tile (start at the first query tile) with a live element
- * and read mask bytes only in patches that hold masked ones.
+ * attention kernels stop at the last key tile (start at the first query tile) with a live element;
+ * the same kernel packs the mask to bits in both orientations (len_q * len_k / 4 bytes), and the
+ * attention kernels read one packed word per lane in patches that hold masked elements.
  * causal, dropout_*, seed, offset, softmax_lse [batch, heads, len_q], softmax_d: as above, with
  * max_seqlen_* = len_*.
  * nmtg_flash_attn_batched_bwd: dout has the strides of out; dq, dk, dv have the strides of q, k, v

@@ -50,6 +50,11 @@ struct FaArgs {
   const uint8_t* tmask;  // batch-strided calls: time mask [max_q, max_k] shared by every sequence and head, 1 = masked, or null
   const int32_t *qinfo, *kqinfo;   // with tmask: summaries by 32 queries x 64 keys and by 32 keys x 64 queries (flash_time_info_kernel)
   int qinfo_pitch, kqinfo_pitch;   // 1 + ceil(max_k / 64) and 2 + ceil(max_q / 64)
+  // The mask itself, one bit per element in the order of a lane's 32 accumulator registers (tile_bit()): a lane reads ONE
+  // word per masked tile. pad_bits [B][key tiles][2], tq_bits [max_q][key tiles][2] (a query's keys), tk_bits
+  // [max_k][query tiles][2] (a key's queries); the last index is the lane's half of the wavefront.
+  const uint32_t *pad_bits, *tq_bits, *tk_bits;
+  int key_tiles, query_tiles;
   int heads, max_q, max_k;
   float scale, scale_log2;
   int causal;
@@ -218,11 +223,11 @@ __device__ __forceinline__ bool masked_tile(const FaArgs& a, int b, int group, i
   if constexpr (MODE == 1) return a.kinfo[static_cast<int64_t>(b) * a.kinfo_pitch + 1 + t] != 0;
   else return a.qinfo[static_cast<int64_t>(group) * a.qinfo_pitch + 1 + t] != 0;
 }
-// the mask byte of (query qr, key): both inside the tensors
+// the packed mask of tile t for this lane's query qr (inside the mask): one load
 template <int MODE>
-__device__ __forceinline__ bool masked_key(const FaArgs& a, const uint8_t* padrow, int qr, int key) {
-  if constexpr (MODE == 1) return padrow[key] != 0;
-  else return a.tmask[static_cast<int64_t>(qr) * a.max_k + key] != 0;
+__device__ __forceinline__ uint32_t tile_mask_bits(const FaArgs& a, int b, int qr, int t, int half) {
+  if constexpr (MODE == 1) return a.pad_bits[(static_cast<int64_t>(b) * a.key_tiles + t) * 2 + half];
+  else return a.tq_bits[(static_cast<int64_t>(qr) * a.key_tiles + t) * 2 + half];
 }
 // time mask: the number of key tiles that a block of 128 queries has to visit (behind it every key is masked for all of them)
 __device__ __forceinline__ int tile_bound(const FaArgs& a, int block) {
@@ -232,15 +237,44 @@ __device__ __forceinline__ int tile_bound(const FaArgs& a, int block) {
   return n;
 }
 
+// Bit i = 16 n + r of a packed mask word stands for element (n, r) of a lane's 32 accumulator registers of a tile:
+// index 64 t + 32 n + 8 (r / 4) + 4 half + r % 4 along the tile's 64 keys (queries, in the key-major kernel).
+__device__ __forceinline__ int tile_bit_index(int t, int i, int half) {
+  const int n = i >> 4, r = i & 15;
+  return FA_TILE * t + 32 * n + 8 * (r / 4) + 4 * half + r % 4;
+}
+
 // Time mask [max_q, max_k] -> the two summaries. Blocks 0 .. ceil(max_q / 32) - 1 write qinfo: per group of 32 queries,
 // word 0 = 1 + the last key tile with a live key (0: none), word 1 + t = class of tile t (0 no masked key, 1 some, 2 all).
 // The other blocks write kqinfo: per group of 32 keys, word 0 = the first tile of 64 queries with a live element (the tile
 // count if none), word 1 = 1 + the last one, word 2 + t = class of query tile t. Elements outside the mask do not count.
 __global__ __launch_bounds__(256) void flash_time_info_kernel(const uint8_t* tmask, int max_q, int max_k, int32_t* qinfo,
-                                                              int qpitch, int32_t* kqinfo, int kpitch) {
+                                                              int qpitch, int32_t* kqinfo, int kpitch, uint32_t* tq_bits,
+                                                              uint32_t* tk_bits) {
   __shared__ int first[4], last[4];
   const int tid = static_cast<int>(threadIdx.x), wave = tid >> 6, lane = tid & 63;
-  const int qgroups = (max_q + 31) / 32;
+  const int qgroups = (max_q + 31) / 32, kgroups = (max_k + 31) / 32;
+  if (static_cast<int>(blockIdx.x) >= qgroups + kgroups) {
+    // the blocks behind the summaries pack the mask: one thread per word, first the words by query, then those by key
+    const int nkt = qpitch - 1, nqt = kpitch - 2;
+    const int64_t by_q = static_cast<int64_t>(max_q) * nkt * 2, by_k = static_cast<int64_t>(max_k) * nqt * 2;
+    const int64_t w = (static_cast<int64_t>(blockIdx.x) - qgroups - kgroups) * 256 + tid;
+    if (w < by_q) {
+      const int half = static_cast<int>(w & 1), t = static_cast<int>((w >> 1) % nkt), q = static_cast<int>((w >> 1) / nkt);
+      const uint8_t* row = tmask + static_cast<int64_t>(q) * max_k;
+      uint32_t word = 0;
+      for (int i = 0; i < 32; ++i) word |= (row[min(tile_bit_index(t, i, half), max_k - 1)] != 0 ? 1u : 0u) << i;
+      tq_bits[w] = word;
+    } else if (w < by_q + by_k) {
+      const int64_t u = w - by_q;
+      const int half = static_cast<int>(u & 1), t = static_cast<int>((u >> 1) % nqt), k = static_cast<int>((u >> 1) / nqt);
+      uint32_t word = 0;
+      for (int i = 0; i < 32; ++i)
+        word |= (tmask[static_cast<int64_t>(min(tile_bit_index(t, i, half), max_q - 1)) * max_k + k] != 0 ? 1u : 0u) << i;
+      tk_bits[u] = word;
+    }
+    return;
+  }
   const bool by_query = static_cast<int>(blockIdx.x) < qgroups;
   const int g = by_query ? static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x) - qgroups;
   const int ntiles = by_query ? qpitch - 1 : kpitch - 2;
@@ -277,7 +311,8 @@ __global__ __launch_bounds__(256) void flash_time_info_kernel(const uint8_t* tma
 
 // Key padding mask [B, max_k] -> key_info [B, 1 + ceil(max_k / 64)]: word 0 = 1 + the index of the last live key (0 when
 // every key is masked), word 1 + t = whether tile t has a masked key below that. One block per sequence.
-__global__ __launch_bounds__(256) void flash_key_info_kernel(const uint8_t* pad, int max_k, int32_t* kinfo, int pitch) {
+__global__ __launch_bounds__(256) void flash_key_info_kernel(const uint8_t* pad, int max_k, int32_t* kinfo, int pitch,
+                                                             uint32_t* pad_bits) {
   __shared__ int part[4];
   const int b = blockIdx.x, tid = static_cast<int>(threadIdx.x);
   const uint8_t* row = pad + static_cast<int64_t>(b) * max_k;
@@ -296,6 +331,16 @@ __global__ __launch_bounds__(256) void flash_key_info_kernel(const uint8_t* pad,
     const bool masked = key < lk && row[key] != 0;
     const bool any = __builtin_amdgcn_ballot_w64(masked) != 0;
     if ((tid & 63) == 0) out[1 + t] = any ? 1 : 0;
+  }
+  // the mask below the last live key, packed: one thread per word [tile][half]
+  for (int w = tid; w < 2 * (pitch - 1); w += 256) {
+    const int t = w >> 1, half = w & 1;
+    uint32_t word = 0;
+    for (int i = 0; i < 32; ++i) {
+      const int key = tile_bit_index(t, i, half);
+      word |= (key < lk && row[key] != 0 ? 1u : 0u) << i;
+    }
+    pad_bits[static_cast<int64_t>(b) * 2 * (pitch - 1) + w] = word;
   }
 }
 
@@ -452,8 +497,7 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
     for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
   float m = FA_NEG, l = 0.f;
   const float dead_raw = FA_NEG / a.scale_log2;   // the raw score that the scale turns into -1e30
-  [[maybe_unused]] const uint8_t* padrow = PAD == 1 ? a.pad + static_cast<int64_t>(b) * a.max_k : nullptr;   // read below lk only
-  [[maybe_unused]] const int qr = min(qrow, lq - 1);   // the row whose time-mask bytes this lane reads
+  [[maybe_unused]] const int qr = min(qrow, lq - 1);   // the row whose time-mask words this lane reads
 
   Staged<D> sk, sv;
   // (not under `ntiles > 0`: rows past the end load nothing and store zeros, and a wait that lies on every path into
@@ -482,8 +526,8 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
       for (int n = 0; n < 2; ++n) mfma<T>::run(read_rows<D>(kimg, n, ss, lane), qf[ss], s[n]);
     // Masking only where the tile crosses the end of the keys or the causal diagonal (the same for the whole wavefront).
     // A masked raw score is the value that the scale turns into -1e30 or beyond: its probability is exp2 of that, 0.
-    // bit 16 n + r of mdead: the mask hides key (n, r) of the tile from this lane's query. The 32 bytes are requested
-    // together, ahead of the masking.
+    // bit 16 n + r of mdead: the mask hides key (n, r) of the tile from this lane's query. One word, packed by the mask's
+    // summary kernel (as byte loads, 32 per tile, the compiler waited for each in turn).
     bool padt = false;
     [[maybe_unused]] uint32_t mdead = 0;
     if constexpr (PAD != 0) {
@@ -492,13 +536,7 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
       // then (the combination is rare; the reference's decoder passes its causal mask as a time mask).
       padt = masked_tile<PAD>(a, b, min(group, (a.max_q + 31) / 32 - 1), t) || a.causal != 0;
       if (padt) {
-#pragma unroll
-        for (int n = 0; n < 2; ++n)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int key = t * FA_TILE + 32 * n + 8 * (r / 4) + 4 * half + r % 4;
-            mdead |= (masked_key<PAD>(a, padrow, qr, min(key, lk - 1)) ? 1u : 0u) << (16 * n + r);
-          }
+        mdead = tile_mask_bits<PAD>(a, b, qr, t, half);
       }
     }
     const bool edge = (t + 1) * FA_TILE > lk || (a.causal && t * FA_TILE + FA_TILE - 1 > q0 + 32 * wave) || padt;
@@ -646,8 +684,7 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dq_kern
   if constexpr (PAD == 2) ntiles = min(ntiles, tile_bound(a, static_cast<int>(blockIdx.x)));
   const int group = static_cast<int>(blockIdx.x) * (FA_ROWS / 32) + __builtin_amdgcn_readfirstlane(wave);   // of 32 queries
   const float dead_raw = FA_NEG / a.scale_log2;   // the raw score that the scale turns into -1e30
-  [[maybe_unused]] const uint8_t* padrow = PAD == 1 ? a.pad + static_cast<int64_t>(b) * a.max_k : nullptr;   // read below lk only
-  [[maybe_unused]] const int qr = min(qrow, lq - 1);   // the row whose time-mask bytes this lane reads
+  [[maybe_unused]] const int qr = min(qrow, lq - 1);   // the row whose time-mask words this lane reads
   acc16_t dq[D / 32];
 #pragma unroll
   for (int i = 0; i < D / 32; ++i)
@@ -683,20 +720,14 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dq_kern
         mfma<T>::run(read_rows<D>(vimg, n, ss, lane), gf[ss], dp[n]);
       }
     // masking as in the forward: only where the tile crosses the end of the keys or the causal diagonal
-    // bit 16 n + r of mdead: the mask hides key (n, r) of the tile from this lane's query. The 32 bytes are requested
-    // together, ahead of the masking.
+    // bit 16 n + r of mdead: the mask hides key (n, r) of the tile from this lane's query. One word, packed by the mask's
+    // summary kernel (as byte loads, 32 per tile, the compiler waited for each in turn).
     bool padt = false;
     [[maybe_unused]] uint32_t mdead = 0;
     if constexpr (PAD != 0) {
       padt = masked_tile<PAD>(a, b, min(group, (a.max_q + 31) / 32 - 1), t);
       if (padt) {
-#pragma unroll
-        for (int n = 0; n < 2; ++n)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int key = t * FA_TILE + 32 * n + 8 * (r / 4) + 4 * half + r % 4;
-            mdead |= (masked_key<PAD>(a, padrow, qr, min(key, lk - 1)) ? 1u : 0u) << (16 * n + r);
-          }
+        mdead = tile_mask_bits<PAD>(a, b, qr, t, half);
       }
     }
     if ((t + 1) * FA_TILE > lk || (a.causal && t * FA_TILE + FA_TILE - 1 > q0 + 32 * wave) || padt) {
@@ -801,7 +832,7 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dkv_ker
     t0 = max(t0, lo);
     ntiles = min(ntiles, hi);
   }
-  const int krow_c = min(krow, a.max_k - 1);   // the column whose time-mask bytes this lane reads
+  const int krow_c = min(krow, a.max_k - 1);   // the column whose time-mask words this lane reads
   const float dead_raw = FA_NEG / a.scale_log2;   // the raw score that the scale turns into -1e30
   acc16_t dk[D / 32], dv[D / 32];
 #pragma unroll
@@ -863,22 +894,12 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dkv_ker
       }
     // s[n][r]: query 32 n + 8 (r / 4) + 4 half + r % 4 of the tile, key krow. P (dropped, scaled) stays in dp's place
     // for dV, dS goes to s for dK.
-    // time mask: bit 16 n + r of tdead = the mask hides query (n, r) of the tile from this lane's key; the 32 bytes are
-    // requested together, ahead of the masking, so that one wait covers them all (a byte load inside each element's
-    // masking condition compiles to 32 load-wait-branch rounds in a row).
+    // time mask: bit 16 n + r of tdead = the mask hides query (n, r) of the tile from this lane's key; one word, packed
+    // by the mask's summary kernel.
     bool tmt = false;
     if constexpr (TM != 0) tmt = a.kqinfo[static_cast<int64_t>(kgroup) * a.kqinfo_pitch + 2 + t] != 0;
     uint32_t tdead = 0;
-    if (TM != 0 && tmt) {
-      const uint8_t* col = a.tmask + krow_c;
-#pragma unroll
-      for (int n = 0; n < 2; ++n)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int qi = t * FA_TILE + 32 * n + 8 * (r / 4) + 4 * half + r % 4;
-          tdead |= (col[static_cast<int64_t>(min(qi, lq - 1)) * a.max_k] != 0 ? 1u : 0u) << (16 * n + r);
-        }
-    }
+    if (TM != 0 && tmt) tdead = a.tk_bits[(static_cast<int64_t>(krow_c) * a.query_tiles + t) * 2 + half];
     if (wave_dead || (a.causal && t * FA_TILE < k0 + 32 * wave + 31) || tmt) {
 #pragma unroll
       for (int n = 0; n < 2; ++n)
@@ -1395,16 +1416,22 @@ int key_info_launch(const char* what, FaArgs& a, int64_t batch, const uint8_t* p
   a.pad = pad;
   a.kinfo = static_cast<const int32_t*>(key_info);
   a.kinfo_pitch = 1 + (a.max_k + FA_TILE - 1) / FA_TILE;
+  a.key_tiles = a.kinfo_pitch - 1;
+  uint32_t* bits = static_cast<uint32_t*>(key_info) + batch * a.kinfo_pitch;      // behind the summaries
+  a.pad_bits = bits;
   if (a.max_k == 0) return 0;
   TraceScope trace("flash_attn_key_info", st);
   hipLaunchKernelGGL(flash_key_info_kernel, dim3(static_cast<unsigned>(batch)), dim3(256), 0, st, pad, a.max_k,
-                     static_cast<int32_t*>(key_info), a.kinfo_pitch);
+                     static_cast<int32_t*>(key_info), a.kinfo_pitch, bits);
   return 0;
 }
 
 // the time mask of a batch-strided call: fills time_info (the two summaries, one behind the other) ahead of every kernel
-int64_t time_info_words(int64_t len_q, int64_t len_k) {
+int64_t time_summary_words(int64_t len_q, int64_t len_k) {
   return (len_q + 31) / 32 * (1 + (len_k + FA_TILE - 1) / FA_TILE) + (len_k + 31) / 32 * (2 + (len_q + FA_TILE - 1) / FA_TILE);
+}
+int64_t time_info_words(int64_t len_q, int64_t len_k) {   // + the packed mask, by query and by key
+  return time_summary_words(len_q, len_k) + 2 * len_q * ((len_k + FA_TILE - 1) / FA_TILE) + 2 * len_k * ((len_q + FA_TILE - 1) / FA_TILE);
 }
 int time_info_launch(const char* what, FaArgs& a, const uint8_t* time_mask, void* time_info, hipStream_t st) {
   if (time_mask == nullptr) return 0;
@@ -1419,9 +1446,18 @@ int time_info_launch(const char* what, FaArgs& a, const uint8_t* time_mask, void
   int32_t* base = static_cast<int32_t*>(time_info);
   a.qinfo = base;
   a.kqinfo = base + static_cast<int64_t>(qgroups) * a.qinfo_pitch;
+  a.key_tiles = a.qinfo_pitch - 1;
+  a.query_tiles = a.kqinfo_pitch - 2;
+  uint32_t* tq = reinterpret_cast<uint32_t*>(base + time_summary_words(a.max_q, a.max_k));
+  uint32_t* tk = tq + static_cast<int64_t>(a.max_q) * a.key_tiles * 2;
+  a.tq_bits = tq;
+  a.tk_bits = tk;
+  const int64_t words = 2 * (static_cast<int64_t>(a.max_q) * a.key_tiles + static_cast<int64_t>(a.max_k) * a.query_tiles);
+  const int64_t blocks = qgroups + kgroups + (words + 255) / 256;
+  NMTG_REQUIRE(blocks <= 0x7fffffff, "%s: time mask too large", what);
   TraceScope trace("flash_attn_time_info", st);
-  hipLaunchKernelGGL(flash_time_info_kernel, dim3(static_cast<unsigned>(qgroups + kgroups)), dim3(256), 0, st, time_mask, a.max_q,
-                     a.max_k, base, a.qinfo_pitch, base + static_cast<int64_t>(qgroups) * a.qinfo_pitch, a.kqinfo_pitch);
+  hipLaunchKernelGGL(flash_time_info_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st, time_mask, a.max_q,
+                     a.max_k, base, a.qinfo_pitch, base + static_cast<int64_t>(qgroups) * a.qinfo_pitch, a.kqinfo_pitch, tq, tk);
   return 0;
 }
 
@@ -1553,7 +1589,7 @@ extern "C" int nmtg_flash_attn_bwd(const void* dout, const void* q, const void* 
 
 extern "C" int64_t nmtg_flash_attn_key_info_bytes(int64_t batch, int64_t len_k) {
   if (batch <= 0 || len_k < 0) return 0;
-  return batch * (1 + (len_k + FA_TILE - 1) / FA_TILE) * 4;
+  return batch * (1 + 3 * ((len_k + FA_TILE - 1) / FA_TILE)) * 4;      // summaries + two packed words per tile
 }
 
 extern "C" int64_t nmtg_flash_attn_time_info_bytes(int64_t len_q, int64_t len_k) {
