@@ -499,6 +499,12 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
   const float dead_raw = FA_NEG / a.scale_log2;   // the raw score that the scale turns into -1e30
   [[maybe_unused]] const int qr = min(qrow, lq - 1);   // the row whose time-mask words this lane reads
 
+  // The packed mask word of a tile is asked for one tile ahead, behind that tile's keys and values, and is there when the
+  // wait for those ends the iteration; asked for at its own tile it would be waited for together with the next tile's loads.
+  [[maybe_unused]] uint32_t mdead_next = 0;
+  if constexpr (PAD != 0) {
+    if (ntiles > 0) mdead_next = tile_mask_bits<PAD>(a, b, qr, 0, half);
+  }
   Staged<D> sk, sv;
   // (not under `ntiles > 0`: rows past the end load nothing and store zeros, and a wait that lies on every path into
   // the loop lets the compiler know there that the resident rows above have landed; behind a branch it would repeat
@@ -511,9 +517,11 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
   for (int t = 0; t < ntiles; ++t) {
     const uint8_t* kimg = lds_raw + (t & 1) * 2 * IMG;
     const uint8_t* vimg = kimg + IMG;
+    [[maybe_unused]] const uint32_t mdead = mdead_next;
     if (t + 1 < ntiles) {
       sk.load(kb, a.k_st, (t + 1) * FA_TILE, lk);
       sv.load(vb, a.v_st, (t + 1) * FA_TILE, lk);
+      if constexpr (PAD != 0) mdead_next = tile_mask_bits<PAD>(a, b, qr, t + 1, half);
     }
     acc16_t s[2];
 #pragma unroll
@@ -529,15 +537,11 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 3 : 1) void flash_fwd_kernel(
     // bit 16 n + r of mdead: the mask hides key (n, r) of the tile from this lane's query. One word, packed by the mask's
     // summary kernel (as byte loads, 32 per tile, the compiler waited for each in turn).
     bool padt = false;
-    [[maybe_unused]] uint32_t mdead = 0;
     if constexpr (PAD != 0) {
       // With the causal flag on top of a mask, a row whose keys up to the diagonal are all masked meets the diagonal's
       // dead keys in tiles without a masked key and still has the initial m there: every tile takes the masked-tile route
       // then (the combination is rare; the reference's decoder passes its causal mask as a time mask).
       padt = masked_tile<PAD>(a, b, min(group, (a.max_q + 31) / 32 - 1), t) || a.causal != 0;
-      if (padt) {
-        mdead = tile_mask_bits<PAD>(a, b, qr, t, half);
-      }
     }
     const bool edge = (t + 1) * FA_TILE > lk || (a.causal && t * FA_TILE + FA_TILE - 1 > q0 + 32 * wave) || padt;
     if (edge) {
@@ -691,6 +695,10 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dq_kern
 #pragma unroll
     for (int r = 0; r < 16; ++r) dq[i][r] = 0.f;
 
+  [[maybe_unused]] uint32_t mdead_next = 0;      // the packed mask word, one tile ahead, as in the forward kernel
+  if constexpr (PAD != 0) {
+    if (ntiles > 0) mdead_next = tile_mask_bits<PAD>(a, b, qr, 0, half);
+  }
   // per buffer: K row image, K transposed image, V row image
   Staged<D> sk, sv;
   sk.load(kb, a.k_st, 0, lk);          // on every path, as in the forward kernel
@@ -703,9 +711,11 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dq_kern
     const uint8_t* kimg = lds_raw + (t & 1) * 3 * IMG;
     const uint8_t* ktimg = kimg + IMG;
     const uint8_t* vimg = kimg + 2 * IMG;
+    [[maybe_unused]] const uint32_t mdead = mdead_next;
     if (t + 1 < ntiles) {
       sk.load(kb, a.k_st, (t + 1) * FA_TILE, lk);
       sv.load(vb, a.v_st, (t + 1) * FA_TILE, lk);
+      if constexpr (PAD != 0) mdead_next = tile_mask_bits<PAD>(a, b, qr, t + 1, half);
     }
     acc16_t s[2], dp[2];
 #pragma unroll
@@ -723,13 +733,7 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dq_kern
     // bit 16 n + r of mdead: the mask hides key (n, r) of the tile from this lane's query. One word, packed by the mask's
     // summary kernel (as byte loads, 32 per tile, the compiler waited for each in turn).
     bool padt = false;
-    [[maybe_unused]] uint32_t mdead = 0;
-    if constexpr (PAD != 0) {
-      padt = masked_tile<PAD>(a, b, min(group, (a.max_q + 31) / 32 - 1), t);
-      if (padt) {
-        mdead = tile_mask_bits<PAD>(a, b, qr, t, half);
-      }
-    }
+    if constexpr (PAD != 0) padt = masked_tile<PAD>(a, b, min(group, (a.max_q + 31) / 32 - 1), t);
     if ((t + 1) * FA_TILE > lk || (a.causal && t * FA_TILE + FA_TILE - 1 > q0 + 32 * wave) || padt) {
 #pragma unroll
       for (int n = 0; n < 2; ++n)
@@ -864,6 +868,8 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dkv_ker
     sg.store_transposed(buf + 3 * IMG);
     if (threadIdx.x < 2 * FA_TILE) reinterpret_cast<float*>(buf + 4 * IMG)[threadIdx.x] = st_val;
   };
+  uint32_t tdead_next = 0;                        // the packed time-mask word, one tile ahead, as in the forward kernel
+  if (TM != 0 && t0 < ntiles) tdead_next = a.tk_bits[(static_cast<int64_t>(krow_c) * a.query_tiles + t0) * 2 + half];
   sq.load(qb, a.q_st, t0 * FA_TILE, lq);          // on every path, as in the forward kernel
   sg.load(gb, a.do_st, t0 * FA_TILE, lq);
   load_stats(t0);
@@ -875,10 +881,12 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dkv_ker
     const uint8_t* gimg = qimg + 2 * IMG;
     const uint8_t* gtimg = qimg + 3 * IMG;
     const float* stats = reinterpret_cast<const float*>(qimg + 4 * IMG);
+    const uint32_t tdead = tdead_next;
     if (t + 1 < ntiles) {
       sq.load(qb, a.q_st, (t + 1) * FA_TILE, lq);
       sg.load(gb, a.do_st, (t + 1) * FA_TILE, lq);
       load_stats(t + 1);
+      if (TM != 0) tdead_next = a.tk_bits[(static_cast<int64_t>(krow_c) * a.query_tiles + t + 1) * 2 + half];
     }
     acc16_t s[2], dp[2];
 #pragma unroll
@@ -898,8 +906,6 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dkv_ker
     // by the mask's summary kernel.
     bool tmt = false;
     if constexpr (TM != 0) tmt = a.kqinfo[static_cast<int64_t>(kgroup) * a.kqinfo_pitch + 2 + t] != 0;
-    uint32_t tdead = 0;
-    if (TM != 0 && tmt) tdead = a.tk_bits[(static_cast<int64_t>(krow_c) * a.query_tiles + t) * 2 + half];
     if (wave_dead || (a.causal && t * FA_TILE < k0 + 32 * wave + 31) || tmt) {
 #pragma unroll
       for (int n = 0; n < 2; ++n)
