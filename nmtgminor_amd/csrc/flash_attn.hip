@@ -243,6 +243,16 @@ __device__ __forceinline__ int tile_bit_index(int t, int i, int half) {
   const int n = i >> 4, r = i & 15;
   return FA_TILE * t + 32 * n + 8 * (r / 4) + 4 * half + r % 4;
 }
+// The packed word of one half from the tile's 64 bits in index order (a wavefront's ballot, lane = index within the tile).
+__device__ __forceinline__ uint32_t tile_word_of(uint64_t in_order, int half) {
+  uint32_t word = 0;
+#pragma unroll
+  for (int n = 0; n < 2; ++n)
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+      word |= static_cast<uint32_t>((in_order >> (32 * n + 8 * g + 4 * half)) & 0xfu) << (16 * n + 4 * g);
+  return word;
+}
 
 // Time mask [max_q, max_k] -> the two summaries. Blocks 0 .. ceil(max_q / 32) - 1 write qinfo: per group of 32 queries,
 // word 0 = 1 + the last key tile with a live key (0: none), word 1 + t = class of tile t (0 no masked key, 1 some, 2 all).
@@ -256,6 +266,7 @@ __global__ __launch_bounds__(256) void flash_time_info_kernel(const uint8_t* tma
   const int qgroups = (max_q + 31) / 32, kgroups = (max_k + 31) / 32;
   if (static_cast<int>(blockIdx.x) >= qgroups + kgroups) {
     // the blocks behind the summaries pack the mask: one thread per word, first the words by query, then those by key
+    // (a wavefront per 64 x 64 patch with ballots was measured too: 22 us against 16 for the whole kernel at T = 512)
     const int nkt = qpitch - 1, nqt = kpitch - 2;
     const int64_t by_q = static_cast<int64_t>(max_q) * nkt * 2, by_k = static_cast<int64_t>(max_k) * nqt * 2;
     const int64_t w = (static_cast<int64_t>(blockIdx.x) - qgroups - kgroups) * 256 + tid;
@@ -329,18 +340,10 @@ __global__ __launch_bounds__(256) void flash_key_info_kernel(const uint8_t* pad,
   for (int t = tid >> 6; t < pitch - 1; t += 4) {
     const int key = FA_TILE * t + (tid & 63);
     const bool masked = key < lk && row[key] != 0;
-    const bool any = __builtin_amdgcn_ballot_w64(masked) != 0;
-    if ((tid & 63) == 0) out[1 + t] = any ? 1 : 0;
-  }
-  // the mask below the last live key, packed: one thread per word [tile][half]
-  for (int w = tid; w < 2 * (pitch - 1); w += 256) {
-    const int t = w >> 1, half = w & 1;
-    uint32_t word = 0;
-    for (int i = 0; i < 32; ++i) {
-      const int key = tile_bit_index(t, i, half);
-      word |= (key < lk && row[key] != 0 ? 1u : 0u) << i;
-    }
-    pad_bits[static_cast<int64_t>(b) * 2 * (pitch - 1) + w] = word;
+    const uint64_t keys = __builtin_amdgcn_ballot_w64(masked);
+    if ((tid & 63) == 0) out[1 + t] = keys != 0 ? 1 : 0;
+    // the mask below the last live key, packed: the tile's two words [tile][half]
+    if ((tid & 63) < 2) pad_bits[(static_cast<int64_t>(b) * (pitch - 1) + t) * 2 + (tid & 63)] = tile_word_of(keys, tid & 63);
   }
 }
 
