@@ -848,20 +848,17 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dkv_ker
     for (int r = 0; r < 16; ++r) { dk[i][r] = 0.f; dv[i][r] = 0.f; }
 
   Staged<D> sq, sg;
-  float st_val = 0.f;   // threads 0..63: lse2 of the tile's query, 64..127: its D
+  // threads 0..63: the log-sum-exp of the tile's query (-inf past the end), 64..127: its D. As loaded: the value is only
+  // looked at when the tile is stored (a comparison or a product right behind the load would be a wait right behind the
+  // tile loads issued before it, every tile).
+  float st_raw = 0.f;
   auto load_stats = [&](int t) {
     const int tid = static_cast<int>(threadIdx.x);
     if (tid < 2 * FA_TILE) {
       const int qi = t * FA_TILE + (tid & (FA_TILE - 1));
-      if (tid < FA_TILE) {
-        st_val = -FA_NEG;
-        if (qi < lq) {
-          const float v = a.lse[static_cast<int64_t>(bh) * a.max_q + qi];
-          st_val = v == -INFINITY ? -FA_NEG : v * FA_LOG2E;
-        }
-      } else {
-        st_val = qi < lq ? a.delta[static_cast<int64_t>(bh) * a.max_q + qi] : 0.f;
-      }
+      const float* src = tid < FA_TILE ? a.lse : a.delta;
+      st_raw = tid < FA_TILE ? -INFINITY : 0.f;
+      if (qi < lq) st_raw = src[static_cast<int64_t>(bh) * a.max_q + qi];
     }
   };
   auto store_tile = [&](uint8_t* buf) {
@@ -869,13 +866,30 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dkv_ker
     sq.store_transposed(buf + IMG);
     sg.store_rows(buf + 2 * IMG);
     sg.store_transposed(buf + 3 * IMG);
-    if (threadIdx.x < 2 * FA_TILE) reinterpret_cast<float*>(buf + 4 * IMG)[threadIdx.x] = st_val;
+    if (threadIdx.x < 2 * FA_TILE) {
+      // lse in units of log2; a row without a live key (or past the end) gets the large positive value that turns its
+      // probabilities into zeros
+      const float lse2 = st_raw == -INFINITY ? -FA_NEG : st_raw * FA_LOG2E;
+      reinterpret_cast<float*>(buf + 4 * IMG)[threadIdx.x] = threadIdx.x < FA_TILE ? lse2 : st_raw;
+    }
+  };
+  // keep bits of this lane's key for a tile's two groups of 32 queries, requested one tile ahead like the tile itself
+  [[maybe_unused]] uint32_t kraw_next[2] = {0, 0};
+  auto load_keep_bits = [&](int t) {
+    if constexpr (DROP != 0) {
+      if (krow < lk) {
+        const uint32_t* w = a.bits + (static_cast<int64_t>(bh) * a.q32 + 2 * t) * a.kp + bit_slot(krow);
+        kraw_next[0] = w[0];
+        kraw_next[1] = w[a.kp];
+      }
+    }
   };
   uint32_t tdead_next = 0;                        // the packed time-mask word, one tile ahead, as in the forward kernel
   if (TM != 0 && t0 < ntiles) tdead_next = a.tk_bits[(static_cast<int64_t>(krow_c) * a.query_tiles + t0) * 2 + half];
   sq.load(qb, a.q_st, t0 * FA_TILE, lq);          // on every path, as in the forward kernel
   sg.load(gb, a.do_st, t0 * FA_TILE, lq);
   load_stats(t0);
+  if (t0 < ntiles) load_keep_bits(t0);
   store_tile(lds_raw + (t0 & 1) * BUF);
   __syncthreads();
   for (int t = t0; t < ntiles; ++t) {
@@ -885,10 +899,12 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dkv_ker
     const uint8_t* gtimg = qimg + 3 * IMG;
     const float* stats = reinterpret_cast<const float*>(qimg + 4 * IMG);
     const uint32_t tdead = tdead_next;
+    [[maybe_unused]] const uint32_t kraw[2] = {kraw_next[0], kraw_next[1]};
     if (t + 1 < ntiles) {
       sq.load(qb, a.q_st, (t + 1) * FA_TILE, lq);
       sg.load(gb, a.do_st, (t + 1) * FA_TILE, lq);
       load_stats(t + 1);
+      load_keep_bits(t + 1);
       if (TM != 0) tdead_next = a.tk_bits[(static_cast<int64_t>(krow_c) * a.query_tiles + t + 1) * 2 + half];
     }
     acc16_t s[2], dp[2];
@@ -921,11 +937,8 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dkv_ker
     // keep bits of this lane's key for the tile's two groups of 32 queries, shifted so that bit 8 g + c is register 4 g + c
     uint32_t kbits[2] = {0, 0};
     if constexpr (DROP != 0) {
-      if (krow < lk) {
-        const uint32_t* w = a.bits + (static_cast<int64_t>(bh) * a.q32 + 2 * t) * a.kp + bit_slot(krow);
-        kbits[0] = w[0] >> (4 * half);
-        kbits[1] = w[a.kp] >> (4 * half);
-      }
+      kbits[0] = kraw[0] >> (4 * half);
+      kbits[1] = kraw[1] >> (4 * half);
     }
 #pragma unroll
     for (int n = 0; n < 2; ++n)
