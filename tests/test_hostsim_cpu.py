@@ -80,7 +80,7 @@ sys.exit(rc)
 
 def _start_sanitizer_run():
     """Starts, beside this process, the child that builds the AddressSanitizer variant of the kernels and repeats this
-    file against it (the last test of the file collects its verdict). -> reason for not running it, or None."""
+    file against it (the last test of the file collects its result). -> reason for not running it, or None."""
     preloaded = os.environ.get("LD_PRELOAD", "").strip()
     if os.path.exists("/etc/ld.so.preload"):
         with open("/etc/ld.so.preload") as f:
