@@ -273,15 +273,23 @@ __global__ __launch_bounds__(256) void flash_time_info_kernel(const uint8_t* tma
     if (w < by_q) {
       const int half = static_cast<int>(w & 1), t = static_cast<int>((w >> 1) % nkt), q = static_cast<int>((w >> 1) / nkt);
       const uint8_t* row = tmask + static_cast<int64_t>(q) * max_k;
+      // the 32 bytes first (independent loads, out together), then the word
+      uint8_t byte[32];
+#pragma unroll
+      for (int i = 0; i < 32; ++i) byte[i] = row[min(tile_bit_index(t, i, half), max_k - 1)];
       uint32_t word = 0;
-      for (int i = 0; i < 32; ++i) word |= (row[min(tile_bit_index(t, i, half), max_k - 1)] != 0 ? 1u : 0u) << i;
+#pragma unroll
+      for (int i = 0; i < 32; ++i) word |= (byte[i] != 0 ? 1u : 0u) << i;
       tq_bits[w] = word;
     } else if (w < by_q + by_k) {
       const int64_t u = w - by_q;
       const int half = static_cast<int>(u & 1), t = static_cast<int>((u >> 1) % nqt), k = static_cast<int>((u >> 1) / nqt);
+      uint8_t byte[32];
+#pragma unroll
+      for (int i = 0; i < 32; ++i) byte[i] = tmask[static_cast<int64_t>(min(tile_bit_index(t, i, half), max_q - 1)) * max_k + k];
       uint32_t word = 0;
-      for (int i = 0; i < 32; ++i)
-        word |= (tmask[static_cast<int64_t>(min(tile_bit_index(t, i, half), max_q - 1)) * max_k + k] != 0 ? 1u : 0u) << i;
+#pragma unroll
+      for (int i = 0; i < 32; ++i) word |= (byte[i] != 0 ? 1u : 0u) << i;
       tk_bits[u] = word;
     }
     return;
@@ -295,16 +303,18 @@ __global__ __launch_bounds__(256) void flash_time_info_kernel(const uint8_t* tma
     // by_query: this lane's key against the group's 32 queries; otherwise this lane's query against the group's 32 keys
     const int mine = FA_TILE * t + lane;
     const bool valid = mine < (by_query ? max_k : max_q);
+    // (no early exit and clamped addresses: the 32 loads are independent and go out together)
     bool any = false, all = true;
-    if (valid)
-      for (int r = 0; r < 32; ++r) {
-        const int other = 32 * g + r;
-        if (other >= (by_query ? max_q : max_k)) break;
-        const int q = by_query ? other : mine, k = by_query ? mine : other;
-        const bool m = tmask[static_cast<int64_t>(q) * max_k + k] != 0;
-        any |= m;
-        all &= m;
-      }
+    const int mine_c = min(mine, (by_query ? max_k : max_q) - 1), others = by_query ? max_q : max_k;
+#pragma unroll
+    for (int r = 0; r < 32; ++r) {
+      const int other = 32 * g + r, other_c = min(other, others - 1);
+      const int q = by_query ? other_c : mine_c, k = by_query ? mine_c : other_c;
+      const bool m = tmask[static_cast<int64_t>(q) * max_k + k] != 0;
+      any |= m && other < others;
+      all &= m || other >= others;
+    }
+    any = any && valid;
     const bool none_live = __builtin_amdgcn_ballot_w64(valid && !all) == 0;
     const bool some_masked = __builtin_amdgcn_ballot_w64(valid && any) != 0;
     const int cls = none_live ? 2 : some_masked ? 1 : 0;
