@@ -336,6 +336,40 @@ class SelfAttnNoCoverageWL(SelfAttnWL):
         return {"gemm_": 3 * (self._flops_fwd() - core), "flash_attn_bwd": 2 * core}
 
 
+class SelfAttnTimeMaskWL(SelfAttnNoCoverageWL):
+    """Not part of the default run (`--workload self_attn_time_mask`): the decoder's self-attention in training."""
+    name = "self_attn_time_mask"
+    description = ("decoder self-attention in training, return_coverage=False: the self_attn shapes (T=512, B=32, E=1024, 16 heads) "
+                   "under a causal time mask [T, T] instead of the key-padding mask, explicit dropout mask; tiled kernels that read "
+                   "the mask as packed words; FLOPs counted dense, as the reference computes them under a mask")
+
+    def setup(self, dev):
+        super().setup(dev)
+        self.tmask = torch.triu(torch.ones(self.T, self.T, dtype=torch.bool), 1).to(dev)
+
+    def step(self):
+        with torch.no_grad():
+            c = _PlainCtx()
+            self.fn.forward(c, True, self.H, self.x, self.w_in, self.w_out, self.b_in, self.b_out, self.tmask, 0.1, self.dm)
+            return self.fn.backward(c, self.dout)
+
+    def cpu_baseline(self):
+        from oracle import attention as o
+        d = self.cpu
+        nb = 2
+        sl = lambda z: z[:, :nb].float()
+        x, dout = sl(d["x"]), sl(d["dout"])
+        w_in, w_out, b_in, b_out = (d[k].float() for k in ("w_in", "w_out", "b_in", "b_out"))
+        tm, dm = torch.triu(torch.ones(self.T, self.T, dtype=torch.bool), 1), d["dropout_mask"][:nb * self.H]
+
+        def run():
+            f = o.self_attn_fwd(x, w_in, w_out, b_in, b_out, self.H, None, tm, 0.1, dm)
+            o.self_attn_bwd(dout, x, w_in, w_out, self.H, f, 0.1, dm)
+        t = _time_cpu(run, 3)
+        return dict(value=self.work_per_step() * nb / self.B / t / 1e12, unit="TFLOP/s", cores=torch.get_num_threads(),
+                    kind="port", sample=f"{nb} of {self.B} batch columns (independent), fp32 on the bf16-rounded values, median of 3")
+
+
 class FlashAttnWL(Workload):
     name = "flash_attn"
     bound = "mfma"
@@ -848,7 +882,7 @@ STREAM_PROBES = [_stream_probe(n + suffix, mode, streams, nbytes, what)
 WORKLOADS = {w.name: w for w in (LayerNormWL, MlpWL, SelfAttnWL, EncdecAttnWL, XentropyWL, SoftmaxDropoutWL, DropoutAddWL,
                                     GeneratorLossWL, RelSelfAttnWL, FusedAdamWL, LayerNormLargeWL, FlashAttnWL, DecodeStepWL,
                                     SelfAttnNoCoverageWL)}
-EXTRA_WORKLOADS = {CopyWL.name: CopyWL, **{w.name: w for w in STREAM_PROBES}}
+EXTRA_WORKLOADS = {CopyWL.name: CopyWL, SelfAttnTimeMaskWL.name: SelfAttnTimeMaskWL, **{w.name: w for w in STREAM_PROBES}}
 PRIMARY = "mlp"
 
 
