@@ -730,6 +730,13 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dq_kern
       sv.load(vb, a.v_st, (t + 1) * FA_TILE, lk);
       if constexpr (PAD != 0) mdead_next = tile_mask_bits<PAD>(a, b, qr, t + 1, half);
     }
+    // the lane masks of the tile's first 32 keys: asked for ahead of the products, which cover the scalar cache's latency
+    [[maybe_unused]] uint64_t first_masks[16];
+    if constexpr (DROP != 0) {
+      const uint64_t* lm = tile_lane_masks(a, bh, group, t);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) first_masks[r] = lm[r];
+    }
     acc16_t s[2], dp[2];
 #pragma unroll
     for (int n = 0; n < 2; ++n)
@@ -765,7 +772,8 @@ __global__ __launch_bounds__(FA_THREADS, D == 64 ? 2 : 1) void flash_bwd_dq_kern
       for (int r = 0; r < 16; ++r) {
         const float pr = fast_exp2(__builtin_fmaf(s[n][r], a.scale_log2, -lse2));
         float kscale = 1.f;
-        if constexpr (DROP != 0) kscale = __builtin_amdgcn_inverse_ballot_w64(lane_mask[16 * n + r]) ? a.drop_scale : 0.f;
+        if constexpr (DROP != 0)
+          kscale = __builtin_amdgcn_inverse_ballot_w64(n == 0 ? first_masks[r] : lane_mask[16 + r]) ? a.drop_scale : 0.f;
         s[n][r] = pr * __builtin_fmaf(dp[n][r], kscale, -delta);     // dS
       }
 #pragma unroll
